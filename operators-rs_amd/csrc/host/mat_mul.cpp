@@ -1,0 +1,275 @@
+// mat_mul on the HIP backend.  Layout normalisation is Args::layout
+// (mat_mul/args.rs:64-192); scalars follow the CPU backend
+// (mat_mul/common_cpu/mod.rs:60-105): for f16 data alpha and beta are rounded
+// to f16 first and C is read only when the f32 beta is non-zero.
+#include <algorithm>
+#include <cstdlib>
+
+#include "../kernels/params.h"
+#include "handle.hpp"
+
+using namespace ophip;
+
+namespace {
+
+struct Matrix {  // mat_mul/args.rs:124-192, strides in elements
+    size_t batch;
+    ptrdiff_t stride;
+    size_t r, c;
+    ptrdiff_t rs, cs;
+
+    static Matrix from(const ophip_tensor_layout &t) {
+        for (size_t i = 0; i < t.ndim; ++i)
+            if (is_dyn(t.shape[i]) || is_dyn(t.strides[i])) throw dyn_not_support("");
+        if (t.ndim < 2) throw rank_not_support("Matrix must have rank 2 or more");
+        if (t.ndim > 3) throw shape_not_support("Higher-rank tensors not supported");
+        const ptrdiff_t unit = (ptrdiff_t)ophip_dtype_nbytes(t.dt);
+        if (unit == 0) throw type_not_support("unknown data type");
+        Matrix m;
+        if (t.ndim == 2 || t.shape[0] == 1) {
+            m.batch = 1;
+            m.stride = 0;
+        } else {
+            m.batch = t.shape[0];
+            m.stride = t.strides[0] / unit;
+        }
+        m.r = t.shape[t.ndim - 2];
+        m.c = t.shape[t.ndim - 1];
+        m.rs = t.strides[t.ndim - 2] / unit;
+        m.cs = t.strides[t.ndim - 1] / unit;
+        return m;
+    }
+    bool match_batch(size_t b) const { return batch == 1 || batch == b; }
+    void transpose() {
+        std::swap(r, c);
+        std::swap(rs, cs);
+    }
+    void ld_trans(ptrdiff_t &ld, int32_t &trans) const {
+        if (rs == 1) {
+            ld = cs;
+            trans = 0;
+        } else if (cs == 1) {
+            ld = rs;
+            trans = 1;
+        } else {
+            throw strides_not_support("Matrix is not contiguous");
+        }
+    }
+};
+
+ophip_mat_mul_layout mat_mul_layout(const ophip_mat_mul_args &args) {
+    Matrix c = Matrix::from(args.c_layout), a = Matrix::from(args.a_layout), b = Matrix::from(args.b_layout);
+    if (c.r != a.r || c.c != b.c || a.c != b.r) throw shape_mismatch("Inconsistent matrix shapes");
+    const size_t batch = c.batch;
+    if (!a.match_batch(batch) || !b.match_batch(batch)) throw shape_mismatch("Inconsistent batch sizes");
+    ophip_mat_mul_layout L{};
+    if (c.rs == 1 && c.cs != 1) {
+        L.ab_swap = 0;
+    } else if (c.cs == 1) {  // C is row-major: C^T = B^T A^T
+        c.transpose();
+        a.transpose();
+        b.transpose();
+        std::swap(a, b);
+        L.ab_swap = 1;
+    } else {
+        throw strides_not_support("Matrix is not contiguous");
+    }
+    a.ld_trans(L.a_ld, L.a_trans);
+    b.ld_trans(L.b_ld, L.b_trans);
+    L.dt = type_distinct({args.c_layout.dt, args.a_layout.dt, args.b_layout.dt});
+    L.batch = batch;
+    L.m = c.r;
+    L.n = c.c;
+    L.k = a.c;
+    L.c_stride = c.stride;
+    L.c_ld = c.cs;
+    L.a_stride = a.stride;
+    L.b_stride = b.stride;
+    return L;
+}
+
+// The canonical problem handed to the kernels plus the kernel choice.
+struct GemmPlan {
+    GemmParams p{};
+    enum Kind { Generic, Skinny } kind = Generic;
+    int mt = 1, qmode = 0;
+    size_t workspace = 0;
+};
+
+bool mult8(int64_t v) { return (v & 7) == 0; }
+
+GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L, unsigned cus) {
+    const void *a = L.ab_swap ? args.b_base : args.a_base;
+    const void *b = L.ab_swap ? args.a_base : args.b_base;
+    const int64_t a_si = L.a_trans ? L.a_ld : 1, a_sl = L.a_trans ? 1 : L.a_ld;
+    const int64_t b_sl = L.b_trans ? L.b_ld : 1, b_sj = L.b_trans ? 1 : L.b_ld;
+
+    GemmPlan g;
+    GemmParams &p = g.p;
+    p.batch = (uint32_t)L.batch;
+    p.K = (uint32_t)L.k;
+    p.d = args.c_base;
+    p.d_sb = L.c_stride;
+    const bool f16 = L.dt == OPHIP_DT_F16;
+    p.alpha = f16 ? round_to_f16(args.alpha) : args.alpha;
+    p.beta = f16 ? round_to_f16(args.beta) : args.beta;
+    p.read_dst = args.beta != 0.f;
+    p.split_k = 1;
+    p.k_per_split = (uint32_t)((L.k + 31) / 32 * 32);
+
+    auto orient = [&](bool transposed) {
+        if (!transposed) {  // D = C, P = A, Q = B
+            p.M = (uint32_t)L.m;
+            p.N = (uint32_t)L.n;
+            p.d_si = 1;
+            p.d_sj = L.c_ld;
+            p.p = a;
+            p.p_si = a_si;
+            p.p_sl = a_sl;
+            p.p_sb = L.a_stride;
+            p.q = b;
+            p.q_sl = b_sl;
+            p.q_sj = b_sj;
+            p.q_sb = L.b_stride;
+        } else {  // D = C^T, P = B^T, Q = A^T
+            p.M = (uint32_t)L.n;
+            p.N = (uint32_t)L.m;
+            p.d_si = L.c_ld;
+            p.d_sj = 1;
+            p.p = b;
+            p.p_si = b_sj;
+            p.p_sl = b_sl;
+            p.p_sb = L.b_stride;
+            p.q = a;
+            p.q_sl = a_sl;
+            p.q_sj = a_si;
+            p.q_sb = L.a_stride;
+        }
+    };
+    auto skinny_ok = [&]() {
+        if (!f16 || p.M == 0 || p.M > 64 || p.K == 0) return false;
+        if (p.p_sl != 1 || !mult8(p.p_si) || !mult8(p.p_sb) || !aligned16(p.p)) return false;
+        if (p.K % 8 != 0 || p.N % 8 != 0) return false;
+        if (!aligned16(p.q) || !mult8(p.q_sb)) return false;
+        if (p.q_sj == 1) {
+            if (!mult8(p.q_sl)) return false;
+        } else if (p.q_sl == 1) {
+            if (!mult8(p.q_sj)) return false;
+        } else {
+            return false;
+        }
+        if (p.d_sj == 1 && (!aligned16(p.d) || !mult8(p.d_si) || !mult8(p.d_sb))) return false;
+        return true;
+    };
+
+    // prefer the orientation whose row count is the small dimension
+    const bool first_transposed = L.n <= L.m;
+    for (int attempt = 0; attempt < 2; ++attempt) {
+        orient(attempt == 0 ? first_transposed : !first_transposed);
+        if (skinny_ok()) {
+            g.kind = GemmPlan::Skinny;
+            g.mt = p.M <= 16 ? 1 : p.M <= 32 ? 2 : 4;
+            g.qmode = p.q_sj == 1 ? 0 : 1;
+            // split K until there are a few workgroups per CU, keeping >= 8 K-steps per workgroup
+            const size_t ntiles = (p.N + 127) / 128, slabs = (p.K + 31) / 32;
+            const size_t base = ntiles * p.batch;
+            size_t split = std::max<size_t>(1, (4 * (size_t)cus + base / 2) / base);
+            split = std::min(split, std::max<size_t>(1, slabs / 8));
+            if (const char *e = std::getenv("OPHIP_GEMM_SPLITK")) split = std::max(1, std::atoi(e));
+            size_t sps = (slabs + split - 1) / split;  // K-steps per split
+            split = (slabs + sps - 1) / sps;
+            p.k_per_split = (uint32_t)(sps * 32);
+            p.split_k = (uint32_t)split;
+            g.workspace = split > 1 ? split * p.batch * (size_t)p.M * p.N * sizeof(float) : 0;
+            return g;
+        }
+    }
+    orient(false);
+    g.kind = GemmPlan::Generic;
+    return g;
+}
+
+}  // namespace
+
+struct ophip_mat_mul {
+    ophip_device *dev;
+    hipFunction_t skinny[3][2];  // [mt index 1,2,4][qmode]
+    hipFunction_t reduce, generic_f16, generic_f32;
+    explicit ophip_mat_mul(ophip_device *d) : dev(d) {
+        ophip_device_retain(d);
+        static const int mts[3] = {1, 2, 4};
+        for (int i = 0; i < 3; ++i)
+            for (int q = 0; q < 2; ++q)
+                skinny[i][q] =
+                    d->kernel("gemm", ("gemm_skinny_m" + std::to_string(mts[i]) + "_q" + std::to_string(q)).c_str());
+        reduce = d->kernel("gemm", "gemm_splitk_reduce");
+        generic_f16 = d->kernel("gemm", "gemm_generic_f16");
+        generic_f32 = d->kernel("gemm", "gemm_generic_f32");
+    }
+    ~ophip_mat_mul() { ophip_device_release(dev); }
+};
+
+extern "C" {
+
+int ophip_mat_mul_plan(const ophip_mat_mul_args *args, ophip_mat_mul_layout *out) {
+    return guard([&] { *out = mat_mul_layout(*args); });
+}
+
+int ophip_mat_mul_create(ophip_device *dev, ophip_mat_mul **out) {
+    return guard([&] {
+        if (!dev || !out) throw args_not_support("null argument");
+        *out = new ophip_mat_mul(dev);
+    });
+}
+void ophip_mat_mul_destroy(ophip_mat_mul *op) { delete op; }
+
+// The reference's scheme() prepares nothing (mat_mul/cuda/mod.rs:30-37).  Here it
+// also reports the split-K workspace when every shape is already known.
+int ophip_mat_mul_scheme(ophip_mat_mul *op, const ophip_mat_mul_args *args, size_t max_ws, size_t *ws) {
+    return guard([&] {
+        if (ws) *ws = 0;
+        ophip_mat_mul_layout L;
+        try {
+            L = mat_mul_layout(*args);
+        } catch (const Error &e) {
+            if (e.kind == OPHIP_DYNAMIC_NOT_SUPPORT) return;  // decide at launch
+            throw;
+        }
+        if (L.dt != OPHIP_DT_F16 && L.dt != OPHIP_DT_F32) throw type_not_support("mat_mul supports f16 and f32");
+        const GemmPlan g = make_plan(*args, L, (unsigned)op->dev->props.multiProcessorCount);
+        if (ws && g.workspace <= max_ws) *ws = g.workspace;
+    });
+}
+
+int ophip_mat_mul_launch(const ophip_mat_mul *op, const ophip_mat_mul_args *args, void *workspace,
+                         size_t workspace_len, const ophip_queue_alloc *qa) {
+    return guard([&] {
+        const ophip_mat_mul_layout L = mat_mul_layout(*args);
+        if (L.dt != OPHIP_DT_F16 && L.dt != OPHIP_DT_F32) throw type_not_support("mat_mul supports f16 and f32");
+        if (is_dyn(args->alpha) || is_dyn(args->beta)) throw dyn_not_support("");
+        if (L.m == 0 || L.n == 0 || L.batch == 0) return;
+        if (L.m > 0x7fffffffu || L.n > 0x7fffffffu || L.k > 0x7fffffffu || L.batch > 65535)
+            throw shape_not_support("mat_mul dimension too large");
+        GemmPlan g = make_plan(*args, L, (unsigned)op->dev->props.multiProcessorCount);
+        const GemmParams &p = g.p;
+        hipStream_t stream = stream_of(qa);
+        op->dev->make_current();
+        if (g.kind == GemmPlan::Skinny) {
+            Workspace ws(qa, workspace, workspace_len, g.workspace);
+            g.p.partial = ws.ptr();
+            const int mi = g.mt == 1 ? 0 : g.mt == 2 ? 1 : 2;
+            launch(op->skinny[mi][g.qmode], Dim3{(p.N + 127) / 128, p.split_k, p.batch}, Dim3{256}, 0, stream, g.p);
+            if (p.split_k > 1) {
+                const size_t total = (size_t)p.batch * p.M * (p.N / 8);
+                launch(op->reduce, Dim3{(unsigned)((total + 255) / 256)}, Dim3{256}, 0, stream, g.p);
+            }
+            return;
+        }
+        const unsigned gx = (p.N + 63) / 64, gy = (p.M + 63) / 64;
+        if (gy > 65535) throw shape_not_support("mat_mul dimension too large for the generic kernel");
+        launch(L.dt == OPHIP_DT_F16 ? op->generic_f16 : op->generic_f32, Dim3{gx, gy, p.batch}, Dim3{256}, 0, stream,
+               g.p);
+    });
+}
+
+}  // extern "C"

@@ -1,0 +1,618 @@
+// rms_norm, rope, fuesd_softmax, rearrange and swiglu on the HIP backend:
+// argument validation as in the reference's Args::meta / Scheme::new, kernel
+// selection, and asynchronous launch on the caller's queue.
+#include <algorithm>
+#include <cstring>
+
+#include "../kernels/params.h"
+#include "handle.hpp"
+
+using namespace ophip;
+
+namespace {
+
+FastDivU32 make_fastdiv(uint32_t d) {
+    // q = (t + ((n - t) >> s1)) >> s2 with t = mulhi(m, n); exact for every 32-bit n, d >= 1
+    FastDivU32 f{};
+    f.d = d;
+    uint32_t l = 0;
+    while ((1ull << l) < d) ++l;
+    f.m = (uint32_t)(((1ull << 32) * ((1ull << l) - d)) / d + 1);
+    f.s1 = l < 1 ? l : 1;
+    f.s2 = l == 0 ? 0 : l - 1;
+    return f;
+}
+
+unsigned ceil_div(size_t a, size_t b) { return (unsigned)((a + b - 1) / b); }
+
+struct OpBase {
+    ophip_device *dev;
+    explicit OpBase(ophip_device *d) : dev(d) { ophip_device_retain(d); }
+    ~OpBase() { ophip_device_release(dev); }
+};
+
+const char *dt_tag(uint64_t dt) { return dt == OPHIP_DT_F16 ? "f16" : dt == OPHIP_DT_F32 ? "f32" : "?"; }
+
+}  // namespace
+
+// =============================================================== rms_norm ===
+// Args::meta: rms_norm/args.rs:25-49.  Launch-time checks follow
+// rms_norm/cuda/mod.rs:49-114 (static shapes, contiguous inner dims).
+
+struct RmsNormMeta {
+    uint64_t dt_a, dt_w;
+    size_t n, d;
+};
+
+static RmsNormMeta rms_norm_meta(const ophip_rms_norm_args &a) {
+    expect_rank(a.y_layout, "y", 2);
+    expect_rank(a.x_layout, "x", 2);
+    expect_rank(a.w_layout, "w", 1);
+    RmsNormMeta m;
+    m.dt_a = type_distinct({a.y_layout.dt, a.x_layout.dt});
+    m.dt_w = a.w_layout.dt;
+    m.n = dim_distinct({a.y_layout.shape[0], a.x_layout.shape[0]});
+    m.d = dim_distinct({a.y_layout.shape[1], a.x_layout.shape[1], a.w_layout.shape[0]});
+    return m;
+}
+
+static void rms_norm_check_types(uint64_t dt_a, uint64_t dt_w) {
+    const bool ok = (dt_a == OPHIP_DT_F16 && (dt_w == OPHIP_DT_F16 || dt_w == OPHIP_DT_F32)) ||
+                    (dt_a == OPHIP_DT_F32 && dt_w == OPHIP_DT_F32);
+    if (!ok) throw type_not_support("rms_norm supports (a, w) in {(f16, f16), (f16, f32), (f32, f32)}");
+}
+
+struct RmsKey {
+    uint64_t dt_a, dt_w;
+    size_t d;
+    bool operator==(const RmsKey &o) const { return dt_a == o.dt_a && dt_w == o.dt_w && d == o.d; }
+};
+struct RmsKeyHash {
+    size_t operator()(const RmsKey &k) const { return k.d * 1315423911u ^ (k.dt_a << 8) ^ k.dt_w; }
+};
+struct RmsScheme {  // kernels for one (dt_a, dt_w, d): a vector variant per group width plus the scalar one
+    hipFunction_t g64, g256, g1024, scalar;
+};
+
+struct ophip_rms_norm : OpBase {
+    mutable LruCache<RmsKey, RmsScheme, RmsKeyHash> schemes;
+    explicit ophip_rms_norm(ophip_device *d) : OpBase(d), schemes(d->config.low_diversity_cache) {}
+
+    RmsScheme scheme_for(const RmsKey &key) const {
+        return schemes.get_or_insert(key, [&] {
+            const std::string base = std::string("rms_norm_") + dt_tag(key.dt_a) + "_" + dt_tag(key.dt_w);
+            RmsScheme s;
+            s.g64 = dev->kernel("rms_norm", (base + "_g64").c_str());
+            s.g256 = dev->kernel("rms_norm", (base + "_g256").c_str());
+            s.g1024 = dev->kernel("rms_norm", (base + "_g1024").c_str());
+            s.scalar = dev->kernel("rms_norm", (base + "_scalar").c_str());
+            return s;
+        });
+    }
+};
+
+extern "C" int ophip_rms_norm_create(ophip_device *dev, ophip_rms_norm **out) {
+    return guard([&] {
+        if (!dev || !out) throw args_not_support("null argument");
+        *out = new ophip_rms_norm(dev);
+    });
+}
+extern "C" void ophip_rms_norm_destroy(ophip_rms_norm *op) { delete op; }
+
+extern "C" int ophip_rms_norm_scheme(ophip_rms_norm *op, const ophip_rms_norm_args *args, size_t, size_t *ws) {
+    return guard([&] {
+        if (ws) *ws = 0;
+        const RmsNormMeta m = rms_norm_meta(*args);
+        const size_t d = static_of(m.d);  // rms_norm/cuda/mod.rs:38-39
+        rms_norm_check_types(m.dt_a, m.dt_w);
+        op->scheme_for(RmsKey{m.dt_a, m.dt_w, d});
+    });
+}
+
+extern "C" int ophip_rms_norm_launch(const ophip_rms_norm *op, const ophip_rms_norm_args *args, void *, size_t,
+                                     const ophip_queue_alloc *qa) {
+    return guard([&] {
+        const RmsNormMeta m = rms_norm_meta(*args);
+        const size_t n = static_of(m.n), d = static_of(m.d);
+        const ptrdiff_t nsy = static_of(args->y_layout.strides[0]), dsy = static_of(args->y_layout.strides[1]);
+        const ptrdiff_t nsx = static_of(args->x_layout.strides[0]), dsx = static_of(args->x_layout.strides[1]);
+        const ptrdiff_t dsw = static_of(args->w_layout.strides[0]);
+        rms_norm_check_types(m.dt_a, m.dt_w);
+        const ptrdiff_t unit = (ptrdiff_t)ophip_dtype_nbytes(m.dt_a);
+        if (dsy != unit || dsx != unit || dsw != (ptrdiff_t)ophip_dtype_nbytes(m.dt_w))
+            throw strides_not_support("rms_norm needs contiguous inner dimensions");
+        if (n == 0 || d == 0) return;
+        if (n > 0x7fffffffu || d > 0x7fffffffu) throw shape_not_support("rms_norm dimension too large");
+
+        const RmsScheme s = op->scheme_for(RmsKey{m.dt_a, m.dt_w, d});
+        RmsNormParams p{};
+        p.y = args->y_base;
+        p.x = args->x_base;
+        p.w = args->w_base;
+        p.nsy = nsy;
+        p.nsx = nsx;
+        p.n = (uint32_t)n;
+        p.d = (uint32_t)d;
+        p.epsilon = args->epsilon;
+
+        const size_t vec_elems = 16 / (size_t)unit;
+        const bool vec = d % vec_elems == 0 && aligned16(p.y) && aligned16(p.x) && aligned16(p.w) && mult16(nsy) &&
+                         mult16(nsx);
+        op->dev->make_current();
+        if (!vec) {
+            launch(s.scalar, Dim3{(unsigned)n}, Dim3{256}, 0, stream_of(qa), p);
+            return;
+        }
+        // group width: 8 vectors per thread fit in registers; widen the group when
+        // there are too few rows to occupy the machine with one wave per row
+        const size_t nvec = d / vec_elems;
+        unsigned G = nvec <= 64 * 8 ? 64 : nvec <= 256 * 8 ? 256 : 1024;
+        while (G < 1024 && n * (G / 64) < 2048 && nvec >= 4 * (size_t)G) G *= 4;
+        const unsigned block = G < 256 ? 256 : G, rpb = block / G;
+        hipFunction_t fn = G == 64 ? s.g64 : G == 256 ? s.g256 : s.g1024;
+        launch(fn, Dim3{ceil_div(n, rpb)}, Dim3{block}, 0, stream_of(qa), p);
+    });
+}
+
+// =================================================================== rope ===
+// Args::meta: rope/args.rs:29-72.  Launch checks: rope/cuda/mod.rs:82-160 and
+// rope/common_cpu/mod.rs:98-100.
+
+struct RopeMeta {
+    uint64_t dt_t, dt_p;
+    size_t nt, dh;
+};
+
+static RopeMeta rope_meta(const ophip_rope_args &a) {
+    expect_rank(a.t_layout, "t", 3);
+    expect_rank(a.p_layout, "p", 1);
+    expect_rank(a.sin_layout, "sin", 2);
+    expect_rank(a.cos_layout, "cos", 2);
+    RopeMeta m;
+    m.dt_t = a.t_layout.dt;
+    m.dt_p = a.p_layout.dt;
+    if (!is_float_dtype(m.dt_t)) throw type_not_support("t must be floating-point numbers");
+    if (!is_unsigned_dtype(m.dt_p)) throw type_not_support("p must be unsigned integers");
+    m.nt = dim_distinct({a.t_layout.shape[0], a.p_layout.shape[0]});
+    m.dh = dim_distinct({a.t_layout.shape[2], a.sin_layout.shape[1], a.cos_layout.shape[1]});
+    return m;
+}
+
+struct ophip_rope : OpBase {
+    hipFunction_t f16_vec, f16_pairs, f32_pairs;
+    explicit ophip_rope(ophip_device *d) : OpBase(d) {
+        f16_vec = d->kernel("rope", "rope_f16_vec");
+        f16_pairs = d->kernel("rope", "rope_f16_pairs");
+        f32_pairs = d->kernel("rope", "rope_f32_pairs");
+    }
+};
+
+extern "C" int ophip_rope_create(ophip_device *dev, ophip_rope **out) {
+    return guard([&] {
+        if (!dev || !out) throw args_not_support("null argument");
+        *out = new ophip_rope(dev);
+    });
+}
+extern "C" void ophip_rope_destroy(ophip_rope *op) { delete op; }
+
+extern "C" int ophip_rope_scheme(ophip_rope *, const ophip_rope_args *args, size_t, size_t *ws) {
+    return guard([&] {
+        if (ws) *ws = 0;
+        (void)rope_meta(*args);
+    });
+}
+
+extern "C" int ophip_rope_launch(const ophip_rope *op, const ophip_rope_args *args, void *, size_t,
+                                 const ophip_queue_alloc *qa) {
+    return guard([&] {
+        const RopeMeta m = rope_meta(*args);
+        if (m.dt_t != OPHIP_DT_F16 && m.dt_t != OPHIP_DT_F32) throw type_not_support("rope supports f16 and f32 tokens");
+        if (m.dt_p != OPHIP_DT_U32 && m.dt_p != OPHIP_DT_U64) throw type_not_support("rope supports u32 and u64 positions");
+        const size_t nt = static_of(m.nt), nh = static_of(args->t_layout.shape[1]), dh = static_of(m.dh);
+        const ptrdiff_t st = static_of(args->t_layout.strides[0]), sh = static_of(args->t_layout.strides[1]),
+                        sd = static_of(args->t_layout.strides[2]), sp = static_of(args->p_layout.strides[0]);
+        const ptrdiff_t unit = (ptrdiff_t)ophip_dtype_nbytes(m.dt_t), punit = (ptrdiff_t)ophip_dtype_nbytes(m.dt_p);
+        if (sd != unit) throw strides_not_support("rope needs a contiguous head dimension");
+        if (sp % punit != 0 || st % unit != 0 || sh % unit != 0) throw strides_not_support("misaligned strides");
+        if (nt == 0 || nh == 0 || dh < 2) return;
+        if (nt > 0x7fffffffu || nh > 0xffffffu || dh > 0xffffffu) throw shape_not_support("rope dimension too large");
+        const size_t smem = (dh / 2) * 8;
+        if (smem > 64 * 1024) throw shape_not_support("rope head dimension too large");
+
+        RopeParams p{};
+        p.t = args->t_base;
+        p.pos = args->p_base;
+        p.st = st;
+        p.sh = sh;
+        p.sp = sp;
+        p.nt = (uint32_t)nt;
+        p.nh = (uint32_t)nh;
+        p.dh = (uint32_t)dh;
+        p.theta = args->theta;
+        p.pos_is_u64 = m.dt_p == OPHIP_DT_U64;
+
+        const bool vec = m.dt_t == OPHIP_DT_F16 && dh % 8 == 0 && aligned16(p.t) && mult16(st) && mult16(sh);
+        // split a token's heads over blockIdx.y when there are few tokens, keeping >= 256 items per block
+        const size_t per_head = vec ? dh / 8 : dh / 2;
+        size_t max_by = std::max<size_t>(1, nh * per_head / 256);
+        size_t want_by = (2048 + nt - 1) / nt;
+        size_t by = std::min(std::min(max_by, want_by), nh);
+        size_t hpb = (nh + by - 1) / by;
+        by = (nh + hpb - 1) / hpb;
+        if (by > 65535) throw shape_not_support("too many heads");
+        p.heads_per_block = (uint32_t)hpb;
+        hipFunction_t fn = vec ? op->f16_vec : (m.dt_t == OPHIP_DT_F16 ? op->f16_pairs : op->f32_pairs);
+        op->dev->make_current();
+        launch(fn, Dim3{(unsigned)nt, (unsigned)by}, Dim3{256}, smem, stream_of(qa), p);
+    });
+}
+
+// fill_pos (rope/mod.rs:46-58) + upload (rope/cuda/mod.rs:36-56)
+extern "C" int ophip_rope_build_pos(uint64_t dt, size_t nt, const ophip_rope_seq *seqs, size_t nseq,
+                                    const ophip_queue_alloc *qa, void **out) {
+    return guard([&] {
+        if (!qa || !qa->alloc || !out) throw args_not_support("null argument");
+        if (dt != OPHIP_DT_U32 && dt != OPHIP_DT_U64) throw type_not_support("positions must be u32 or u64");
+        const size_t unit = ophip_dtype_nbytes(dt);
+        std::vector<unsigned char> host(unit * nt, 0);
+        size_t o = 0;
+        for (size_t s = 0; s < nseq && o < nt; ++s)
+            for (size_t q = seqs[s].pos; q < seqs[s].pos + seqs[s].len && o < nt; ++q, ++o) {
+                if (dt == OPHIP_DT_U32) {
+                    const uint32_t v = (uint32_t)q;
+                    std::memcpy(&host[o * 4], &v, 4);
+                } else {
+                    const uint64_t v = (uint64_t)q;
+                    std::memcpy(&host[o * 8], &v, 8);
+                }
+            }
+        void *mem = qa->alloc(qa->ctx, host.size());
+        if (!mem && !host.empty()) throw execution_failed("queue allocator returned null");
+        if (!host.empty()) {
+            check_hip(hipMemcpyAsync(mem, host.data(), host.size(), hipMemcpyHostToDevice, stream_of(qa)),
+                      "hipMemcpyAsync");
+            // the staging buffer dies with this call, so the copy must have left it
+            check_hip(hipStreamSynchronize(stream_of(qa)), "hipStreamSynchronize");
+        }
+        *out = mem;
+    });
+}
+
+extern "C" int ophip_rope_build_sincos(uint64_t, size_t, size_t, const ophip_queue_alloc *qa, size_t *nctx_out,
+                                       void **out) {
+    return guard([&] {
+        if (!qa || !qa->alloc || !out) throw args_not_support("null argument");
+        if (nctx_out) *nctx_out = 0;
+        *out = qa->alloc(qa->ctx, 0);
+    });
+}
+
+// ========================================================== fuesd_softmax ===
+// Args::meta: fuesd_softmax/args.rs:31-37; launch checks: fuesd_softmax/cuda/mod.rs:52-119.
+
+struct SoftmaxVariant {
+    int vec, pt, g;
+    hipFunction_t fn;
+};
+
+struct ophip_fused_softmax : OpBase {
+    std::vector<SoftmaxVariant> variants;
+    hipFunction_t stream_fn;
+    explicit ophip_fused_softmax(ophip_device *d) : OpBase(d) {
+        static const int table[][3] = {{8, 1, 64},  {8, 2, 64},   {8, 4, 64},   {8, 1, 256},  {8, 2, 256},
+                                       {8, 4, 256}, {8, 8, 256},  {8, 4, 1024}, {8, 8, 1024}, {1, 8, 64},
+                                       {1, 16, 64}, {1, 8, 256},  {1, 16, 256}, {1, 32, 256}, {1, 16, 1024}};
+        for (auto &t : table) {
+            const std::string name = "softmax_f16_v" + std::to_string(t[0]) + "_p" + std::to_string(t[1]) + "_g" +
+                                     std::to_string(t[2]);
+            variants.push_back({t[0], t[1], t[2], d->kernel("fused_softmax", name.c_str())});
+        }
+        stream_fn = d->kernel("fused_softmax", "softmax_f16_stream");
+    }
+};
+
+extern "C" int ophip_fused_softmax_create(ophip_device *dev, ophip_fused_softmax **out) {
+    return guard([&] {
+        if (!dev || !out) throw args_not_support("null argument");
+        *out = new ophip_fused_softmax(dev);
+    });
+}
+extern "C" void ophip_fused_softmax_destroy(ophip_fused_softmax *op) { delete op; }
+
+extern "C" int ophip_fused_softmax_scheme(ophip_fused_softmax *, const ophip_fused_softmax_args *args, size_t,
+                                          size_t *ws) {
+    return guard([&] {
+        if (ws) *ws = 0;
+        if (args->att_layout.ndim != 3) throw rank_not_support("");
+        if (args->att_layout.dt != OPHIP_DT_F16) throw type_not_support("fused softmax supports f16");
+    });
+}
+
+extern "C" int ophip_fused_softmax_launch(const ophip_fused_softmax *op, const ophip_fused_softmax_args *args, void *,
+                                          size_t, const ophip_queue_alloc *qa) {
+    return guard([&] {
+        const ophip_tensor_layout &l = args->att_layout;
+        if (l.ndim != 3) throw rank_not_support("");
+        if (l.dt != OPHIP_DT_F16) throw type_not_support("fused softmax supports f16");
+        if (args->att_mask != OPHIP_MASK_NONE && args->att_mask != OPHIP_MASK_CAUSAL)
+            throw args_not_support("unknown attention mask");
+        const size_t nh = static_of(l.shape[0]), seq = static_of(l.shape[1]), att = static_of(l.shape[2]);
+        const ptrdiff_t sh = static_of(l.strides[0]), ss = static_of(l.strides[1]), sa = static_of(l.strides[2]);
+        if (sa != 2) throw strides_not_support("fused softmax needs a contiguous last dimension");
+        if (sh % 2 != 0 || ss % 2 != 0) throw strides_not_support("misaligned strides");
+        const size_t rows = nh * seq;
+        if (rows == 0) return;
+        const bool causal = args->att_mask == OPHIP_MASK_CAUSAL;
+        // a row that keeps no column has no maximum: the reference panics there
+        if (att == 0 || (causal && att < seq)) throw shape_not_support("a softmax row keeps no column");
+        if (rows > 0x7fffffffu || att > 0x7fffffffu) throw shape_not_support("softmax dimension too large");
+
+        SoftmaxParams p{};
+        p.att = args->att_base;
+        p.sh = sh;
+        p.ss = ss;
+        p.nh = (uint32_t)nh;
+        p.seq = (uint32_t)seq;
+        p.att_len = (uint32_t)att;
+        p.causal = causal;
+
+        const bool vec = att % 8 == 0 && aligned16(p.att) && mult16(sh) && mult16(ss);
+        const int want_vec = vec ? 8 : 1;
+        // narrowest group that holds the row in registers; with few rows prefer a
+        // whole workgroup per row so more lanes pull on memory
+        const SoftmaxVariant *pick = nullptr;
+        for (const auto &v : op->variants) {
+            if (v.vec != want_vec) continue;
+            if ((size_t)v.vec * v.pt * v.g < att) continue;
+            if (rows < 2048 && v.g < 256 && att >= (size_t)256 * v.vec) continue;
+            if (!pick || v.g < pick->g || (v.g == pick->g && v.pt < pick->pt)) pick = &v;
+        }
+        op->dev->make_current();
+        if (!pick) {
+            launch(op->stream_fn, Dim3{(unsigned)rows}, Dim3{1024}, 0, stream_of(qa), p);
+            return;
+        }
+        const unsigned block = pick->g < 256 ? 256 : pick->g, rpb = block / pick->g;
+        launch(pick->fn, Dim3{ceil_div(rows, rpb)}, Dim3{block}, 0, stream_of(qa), p);
+    });
+}
+
+// ============================================================== rearrange ===
+// Scheme::new: rearrange/args.rs:35-153.
+
+namespace {
+struct RDim {
+    size_t len;
+    ptrdiff_t dst, src;
+};
+struct RScheme {
+    size_t unit = 0;
+    std::vector<size_t> idx;  // ndim + 1 entries: count ... 1
+    std::vector<ptrdiff_t> dst, src;
+    size_t ndim() const { return dst.size(); }
+    size_t count() const { return idx.empty() ? 1 : idx[0]; }
+};
+
+ptrdiff_t iabs(ptrdiff_t v) { return v < 0 ? -v : v; }
+
+RScheme rearrange_scheme(const ophip_rearrange_args &a) {
+    const ophip_tensor_layout &D = a.dst_layout, &S = a.src_layout;
+    (void)type_distinct({D.dt, S.dt});
+    if (D.ndim != S.ndim)
+        throw rank_mismatch("dst.ndim = " + std::to_string(D.ndim) + ", src.ndim = " + std::to_string(S.ndim));
+    std::vector<RDim> dims;
+    for (size_t i = 0; i < D.ndim; ++i) {
+        const size_t dd = static_of(D.shape[i]), ds = static_of(S.shape[i]);
+        if (dd != ds)
+            throw shape_mismatch("dst[" + std::to_string(i) + "] = " + std::to_string(dd) + ", src[" +
+                                 std::to_string(i) + "] = " + std::to_string(ds));
+        RDim dim{dd, static_of(D.strides[i]), static_of(S.strides[i])};
+        if (dim.len != 1) {
+            if (dim.dst == 0) throw shape_not_support("Reducing is not allowed for rearrangement.");
+            dims.push_back(dim);
+        }
+    }
+    // |dst| descending, |src| descending, len ascending
+    std::sort(dims.begin(), dims.end(), [](const RDim &x, const RDim &y) {
+        if (iabs(x.dst) != iabs(y.dst)) return iabs(x.dst) > iabs(y.dst);
+        if (iabs(x.src) != iabs(y.src)) return iabs(x.src) > iabs(y.src);
+        return x.len < y.len;
+    });
+    ptrdiff_t unit = (ptrdiff_t)ophip_dtype_nbytes(D.dt);
+    if (unit == 0) throw type_not_support("unknown data type");
+    size_t ndim = dims.size();
+    for (size_t r = dims.size(); r-- > 0;) {  // trailing contiguous dims fold into the unit
+        if (dims[r].dst == unit && dims[r].src == unit) {
+            unit *= (ptrdiff_t)dims[r].len;
+            --ndim;
+        } else {
+            break;
+        }
+    }
+    dims.resize(ndim);
+    for (size_t i = dims.size(); i-- > 1;) {  // neighbours with proportional strides merge
+        RDim &f = dims[i - 1], &b = dims[i];
+        const ptrdiff_t len = (ptrdiff_t)b.len;
+        if (b.dst * len == f.dst && b.src * len == f.src) {
+            f = RDim{b.len * f.len, b.dst, b.src};
+            b = RDim{1, 0, 0};
+            --ndim;
+        }
+    }
+    RScheme s;
+    s.unit = (size_t)unit;
+    std::vector<size_t> lens;
+    for (const RDim &d : dims)
+        if (d.len != 1) {
+            lens.push_back(d.len);
+            s.dst.push_back(d.dst);
+            s.src.push_back(d.src);
+        }
+    s.idx.assign(ndim + 1, 1);
+    for (size_t i = ndim; i-- > 0;) s.idx[i] = lens[i] * s.idx[i + 1];
+    return s;
+}
+}  // namespace
+
+extern "C" int ophip_rearrange_plan(const ophip_rearrange_args *args, ptrdiff_t *out, size_t *ndim_out) {
+    return guard([&] {
+        const RScheme s = rearrange_scheme(*args);
+        const size_t nd = s.ndim();
+        out[0] = (ptrdiff_t)s.unit;
+        for (size_t i = 0; i <= nd; ++i) out[1 + i] = (ptrdiff_t)s.idx[i];
+        for (size_t i = 0; i < nd; ++i) {
+            out[2 + nd + i] = s.dst[i];
+            out[2 + 2 * nd + i] = s.src[i];
+        }
+        if (ndim_out) *ndim_out = nd;
+    });
+}
+
+struct ophip_rearrange : OpBase {
+    hipFunction_t k32[5], k64[5];  // chunk sizes 16, 8, 4, 2, 1
+    explicit ophip_rearrange(ophip_device *d) : OpBase(d) {
+        static const int sizes[5] = {16, 8, 4, 2, 1};
+        for (int i = 0; i < 5; ++i) {
+            k32[i] = d->kernel("rearrange", ("rearrange_b" + std::to_string(sizes[i])).c_str());
+            k64[i] = d->kernel("rearrange", ("rearrange64_b" + std::to_string(sizes[i])).c_str());
+        }
+    }
+};
+
+extern "C" int ophip_rearrange_create(ophip_device *dev, ophip_rearrange **out) {
+    return guard([&] {
+        if (!dev || !out) throw args_not_support("null argument");
+        *out = new ophip_rearrange(dev);
+    });
+}
+extern "C" void ophip_rearrange_destroy(ophip_rearrange *op) { delete op; }
+
+// The reference's scheme() does no work at all (rearrange/cuda/mod.rs:45-52).
+extern "C" int ophip_rearrange_scheme(ophip_rearrange *, const ophip_rearrange_args *, size_t, size_t *ws) {
+    return guard([&] {
+        if (ws) *ws = 0;
+    });
+}
+
+extern "C" int ophip_rearrange_launch(const ophip_rearrange *op, const ophip_rearrange_args *args, void *, size_t,
+                                      const ophip_queue_alloc *qa) {
+    return guard([&] {
+        const RScheme s = rearrange_scheme(*args);
+        if (s.unit == 0 || s.count() == 0) return;
+        op->dev->make_current();
+        if (s.ndim() == 0) {  // one contiguous run: a device-to-device copy (rearrange/cuda/mod.rs:64-70)
+            check_hip(hipMemcpyAsync(args->dst_base, args->src_base, s.unit, hipMemcpyDeviceToDevice, stream_of(qa)),
+                      "hipMemcpyAsync");
+            return;
+        }
+        if (s.ndim() > OPHIP_REARRANGE_MAXD)
+            throw rank_not_support("rearrange supports at most " + std::to_string(OPHIP_REARRANGE_MAXD) +
+                                   " non-mergeable dimensions");
+        // widest chunk that divides the unit and keeps every access aligned
+        uintptr_t bits = (uintptr_t)s.unit | reinterpret_cast<uintptr_t>(args->dst_base) |
+                         reinterpret_cast<uintptr_t>(args->src_base);
+        for (size_t i = 0; i < s.ndim(); ++i) bits |= (uintptr_t)iabs(s.dst[i]) | (uintptr_t)iabs(s.src[i]);
+        int ci = 0;
+        size_t B = 16;
+        while (bits & (B - 1)) {
+            B >>= 1;
+            ++ci;
+        }
+        RearrangeParams p{};
+        p.dst = args->dst_base;
+        p.src = args->src_base;
+        p.ndim = (uint32_t)s.ndim();
+        const size_t cpu = s.unit / B;
+        p.total = (uint64_t)s.count() * cpu;
+        bool small = p.total <= 0x7fffffffu && cpu <= 0x7fffffffu;
+        for (size_t i = 0; i < s.ndim(); ++i) {
+            p.idx[i] = s.idx[i + 1];
+            p.dst_s[i] = s.dst[i];
+            p.src_s[i] = s.src[i];
+            if (s.idx[i + 1] > 0x7fffffffu) small = false;
+        }
+        p.chunks_per_unit = (uint32_t)cpu;
+        if (small) {
+            p.cpu_div = make_fastdiv((uint32_t)cpu);
+            for (size_t i = 0; i < s.ndim(); ++i) p.idx_div[i] = make_fastdiv((uint32_t)s.idx[i + 1]);
+            const unsigned per_block = 256 * 4;  // RE_ITEMS chunks per thread
+            launch(op->k32[ci], Dim3{ceil_div(p.total, per_block)}, Dim3{256}, 0, stream_of(qa), p);
+        } else {
+            if (cpu > 0xffffffffu) throw shape_not_support("rearrange unit too large");
+            const uint64_t blocks = std::min<uint64_t>((p.total + 255) / 256, 1u << 20);
+            launch(op->k64[ci], Dim3{(unsigned)blocks}, Dim3{256}, 0, stream_of(qa), p);
+        }
+    });
+}
+
+// ================================================================= swiglu ===
+// Args::meta: swiglu/args.rs:31-50; launch checks: swiglu/cuda/mod.rs:53-98.
+
+struct ophip_swiglu : OpBase {
+    hipFunction_t f16_vec, f16_scalar, f32_scalar;
+    explicit ophip_swiglu(ophip_device *d) : OpBase(d) {
+        f16_vec = d->kernel("swiglu", "swiglu_f16_vec");
+        f16_scalar = d->kernel("swiglu", "swiglu_f16_scalar");
+        f32_scalar = d->kernel("swiglu", "swiglu_f32_scalar");
+    }
+};
+
+struct SwigluMeta {
+    uint64_t dt;
+    size_t n, d;
+};
+static SwigluMeta swiglu_meta(const ophip_swiglu_args &a) {
+    expect_rank(a.gate_layout, "gate", 2);
+    expect_rank(a.up_layout, "up", 2);
+    SwigluMeta m;
+    m.dt = type_distinct({a.gate_layout.dt, a.up_layout.dt});
+    m.n = dim_distinct({a.gate_layout.shape[0], a.up_layout.shape[0]});
+    m.d = dim_distinct({a.gate_layout.shape[1], a.up_layout.shape[1]});
+    return m;
+}
+
+extern "C" int ophip_swiglu_create(ophip_device *dev, ophip_swiglu **out) {
+    return guard([&] {
+        if (!dev || !out) throw args_not_support("null argument");
+        *out = new ophip_swiglu(dev);
+    });
+}
+extern "C" void ophip_swiglu_destroy(ophip_swiglu *op) { delete op; }
+
+extern "C" int ophip_swiglu_scheme(ophip_swiglu *, const ophip_swiglu_args *args, size_t, size_t *ws) {
+    return guard([&] {
+        if (ws) *ws = 0;
+        (void)swiglu_meta(*args);
+    });
+}
+
+extern "C" int ophip_swiglu_launch(const ophip_swiglu *op, const ophip_swiglu_args *args, void *, size_t,
+                                   const ophip_queue_alloc *qa) {
+    return guard([&] {
+        const SwigluMeta m = swiglu_meta(*args);
+        if (m.dt != OPHIP_DT_F16 && m.dt != OPHIP_DT_F32) throw type_not_support("swiglu supports f16 and f32");
+        const size_t n = static_of(m.n), d = static_of(m.d);
+        const ptrdiff_t sgn = static_of(args->gate_layout.strides[0]), sgd = static_of(args->gate_layout.strides[1]);
+        const ptrdiff_t sun = static_of(args->up_layout.strides[0]), sud = static_of(args->up_layout.strides[1]);
+        const ptrdiff_t unit = (ptrdiff_t)ophip_dtype_nbytes(m.dt);
+        if (sgd != unit || sud != unit) throw strides_not_support("swiglu needs contiguous inner dimensions");
+        if (sgn % unit != 0 || sun % unit != 0) throw strides_not_support("misaligned strides");
+        if (n == 0 || d == 0) return;
+        if (n > 0x7fffffffu || d > 0x7fffffffu) throw shape_not_support("swiglu dimension too large");
+        SwigluParams p{};
+        p.gate = args->gate_base;
+        p.up = args->up_base;
+        p.sgn = sgn;
+        p.sun = sun;
+        p.n = (uint32_t)n;
+        p.d = (uint32_t)d;
+        const bool vec = m.dt == OPHIP_DT_F16 && d % 8 == 0 && aligned16(p.gate) && aligned16(p.up) && mult16(sgn) &&
+                         mult16(sun);
+        const size_t items = vec ? d / 8 : d;
+        const unsigned gx = std::min<unsigned>(ceil_div(items, 256), 65535u);
+        const unsigned gy = (unsigned)std::min<size_t>(n, 65535);
+        hipFunction_t fn = vec ? op->f16_vec : (m.dt == OPHIP_DT_F16 ? op->f16_scalar : op->f32_scalar);
+        op->dev->make_current();
+        launch(fn, Dim3{gx, gy}, Dim3{256}, 0, stream_of(qa), p);
+    });
+}

@@ -1,0 +1,153 @@
+// random_sample on the HIP backend.  Validation: random_sample/args.rs:93-120 and
+// random_sample/cuda/mod.rs:84-150; mode selection: SampleArgs::is_argmax
+// (args.rs:80-84).
+#include <cstring>
+
+#include "../kernels/params.h"
+#include "handle.hpp"
+
+using namespace ophip;
+
+namespace {
+
+constexpr size_t TOPK_FAST_MAX = 1024;  // candidates the single-workgroup top-k kernel sorts in LDS
+
+struct SampleMeta {
+    uint64_t dt;
+    size_t n;
+};
+
+SampleMeta sample_meta(const ophip_random_sample_args &a) {
+    if (a.kv_pair.dt != OPHIP_DT_KVPAIR) throw type_not_support("output must be KVpair");
+    const uint64_t dt = a.logits.dt;
+    const size_t nb = ophip_dtype_nbytes(dt);
+    if (nb == 0 || nb > sizeof(uint32_t)) throw type_not_support("element too large");
+    if (a.indices.dt != OPHIP_DT_U32) throw type_not_support("indices must be u32");
+    expect_rank(a.logits, "logits", 1);
+    expect_rank(a.indices, "indices", 1);
+    return {dt, a.logits.shape[0]};
+}
+
+size_t next_pow2(size_t n) {
+    size_t p = 1;
+    while (p < n) p <<= 1;
+    return p;
+}
+
+// bytes of workspace the full-sort kernel needs for one row
+size_t full_sort_workspace(size_t n) { return next_pow2(n) * 8 + ((n * 4 + 15) & ~(size_t)15); }
+
+}  // namespace
+
+struct ophip_random_sample {
+    ophip_device *dev;
+    hipFunction_t argmax[2], topk[2], full[2];  // [0] f16, [1] f32
+    explicit ophip_random_sample(ophip_device *d) : dev(d) {
+        ophip_device_retain(d);
+        argmax[0] = d->kernel("random_sample", "argmax_f16");
+        argmax[1] = d->kernel("random_sample", "argmax_f32");
+        topk[0] = d->kernel("random_sample", "sample_topk_f16");
+        topk[1] = d->kernel("random_sample", "sample_topk_f32");
+        full[0] = d->kernel("random_sample", "sample_full_f16");
+        full[1] = d->kernel("random_sample", "sample_full_f32");
+    }
+    ~ophip_random_sample() { ophip_device_release(dev); }
+};
+
+extern "C" {
+
+int ophip_sample_args_new(float temperature, float top_p, size_t top_k, ophip_sample_args *out) {
+    if (temperature < 0.f) return 1;           // NegativeTemperature
+    if (top_k == 0 || top_p <= 0.f) return 2;  // NonPositiveTop
+    out->temperature = temperature;
+    out->top_p = top_p < 1.f ? top_p : 1.f;
+    out->top_k = top_k;
+    return 0;
+}
+
+ophip_sample_args ophip_sample_args_argmax(void) { return ophip_sample_args{0.f, 1.f, SIZE_MAX}; }
+
+int ophip_random_sample_create(ophip_device *dev, ophip_random_sample **out) {
+    return guard([&] {
+        if (!dev || !out) throw args_not_support("null argument");
+        *out = new ophip_random_sample(dev);
+    });
+}
+void ophip_random_sample_destroy(ophip_random_sample *op) { delete op; }
+
+// The workspace answer follows random_sample/cuda/mod.rs:55-82: the larger of the
+// two modes' needs if it fits, else the smaller, else 0; 0 for a dynamic n.
+int ophip_random_sample_scheme(ophip_random_sample *, const ophip_random_sample_args *args, size_t max_ws,
+                               size_t *ws) {
+    return guard([&] {
+        if (ws) *ws = 0;
+        const SampleMeta m = sample_meta(*args);
+        if (m.dt != OPHIP_DT_F16 && m.dt != OPHIP_DT_F32) throw type_not_support("logits must be f16 or f32");
+        if (is_dyn(m.n)) return;
+        const size_t argmax_size = 0, sample_size = full_sort_workspace(m.n);
+        if (ws) *ws = sample_size <= max_ws ? sample_size : argmax_size;
+    });
+}
+
+int ophip_random_sample_launch(const ophip_random_sample *op, const ophip_random_sample_args *args, void *workspace,
+                               size_t workspace_len, const ophip_queue_alloc *qa) {
+    return guard([&] {
+        const SampleMeta m = sample_meta(*args);
+        if (args->kv_pair.ndim != 0) throw rank_error("kv_pair", 0, args->kv_pair.ndim);
+        const size_t n = static_of(m.n);
+        const ptrdiff_t sp = static_of(args->logits.strides[0]);
+        const ptrdiff_t si = static_of(args->indices.strides[0]);
+        if (m.dt != OPHIP_DT_F16 && m.dt != OPHIP_DT_F32) throw type_not_support("logits must be f16 or f32");
+        if (sp != (ptrdiff_t)ophip_dtype_nbytes(m.dt)) throw strides_not_support("logits must be contiguous");
+        if (si != (ptrdiff_t)sizeof(uint32_t)) throw strides_not_support("indices must be contiguous");
+        if (n == 0) throw shape_not_support("empty logits");  // the reference unwraps an empty maximum
+        if (n > 0x7fffffffu) throw shape_not_support("too many logits");
+
+        const int ti = m.dt == OPHIP_DT_F16 ? 0 : 1;
+        const ophip_sample_args &cfg = args->config;
+        SampleParams p{};
+        p.kv = args->kv_pair_base;
+        p.logits = args->logits_base;
+        p.row_stride = 0;
+        p.n = (uint32_t)n;
+        op->dev->make_current();
+        if (cfg.temperature == 0.f || cfg.top_k == 1) {
+            launch(op->argmax[ti], Dim3{1}, Dim3{1024}, 0, stream_of(qa), p);
+            return;
+        }
+        if (is_dyn(cfg.temperature) || is_dyn(cfg.top_p) || is_dyn(args->seed)) throw dyn_not_support("");
+        if (!(cfg.temperature > 0.f) || cfg.top_k == 0 || !(cfg.top_p > 0.f))
+            throw args_not_support("sampling needs temperature > 0, top_k >= 1, top_p > 0");
+        const size_t k_eff = cfg.top_k < n ? cfg.top_k : n;
+        p.k_eff = (uint32_t)k_eff;
+        p.temperature = cfg.temperature;
+        p.top_p = cfg.top_p;
+        p.seed = args->seed;
+        if (k_eff <= TOPK_FAST_MAX) {
+            launch(op->topk[ti], Dim3{1}, Dim3{1024}, 0, stream_of(qa), p);
+            return;
+        }
+        p.npow2 = (uint32_t)next_pow2(n);
+        Workspace ws(qa, workspace, workspace_len, full_sort_workspace(n));
+        p.workspace = ws.ptr();
+        launch(op->full[ti], Dim3{1}, Dim3{1024}, 0, stream_of(qa), p);
+    });
+}
+
+int ophip_random_sample_build_indices(size_t n, const ophip_queue_alloc *qa, void **out) {
+    return guard([&] {
+        if (!qa || !qa->alloc || !out) throw args_not_support("null argument");
+        std::vector<uint32_t> host(n);
+        for (size_t i = 0; i < n; ++i) host[i] = (uint32_t)i;
+        void *mem = qa->alloc(qa->ctx, n * sizeof(uint32_t));
+        if (!mem && n) throw execution_failed("queue allocator returned null");
+        if (n) {
+            check_hip(hipMemcpyAsync(mem, host.data(), n * sizeof(uint32_t), hipMemcpyHostToDevice, stream_of(qa)),
+                      "hipMemcpyAsync");
+            check_hip(hipStreamSynchronize(stream_of(qa)), "hipStreamSynchronize");
+        }
+        *out = mem;
+    });
+}
+
+}  // extern "C"

@@ -1,0 +1,89 @@
+// Device-side helpers for the gfx950 kernels: 128-bit vector types, wave64 and
+// workgroup reductions, f16 conversions.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "params.h"
+
+typedef _Float16 f16;
+typedef f16 f16x2 __attribute__((ext_vector_type(2)));
+typedef f16 f16x4 __attribute__((ext_vector_type(4)));
+typedef f16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+#define WAVE 64
+
+__device__ __forceinline__ u32x4 ld128(const void *p) { return *reinterpret_cast<const u32x4 *>(p); }
+__device__ __forceinline__ void st128(void *p, u32x4 v) { *reinterpret_cast<u32x4 *>(p) = v; }
+
+__device__ __forceinline__ float h2f(f16 h) { return (float)h; }
+// round-to-nearest-even, subnormals kept (v_cvt_f16_f32)
+__device__ __forceinline__ f16 f2h(float f) { return (f16)f; }
+
+union Pack8 {
+    u32x4 u;
+    f16x8 h;
+    f16 e[8];
+};
+union Pack4f {
+    u32x4 u;
+    f32x4 f;
+    float e[4];
+};
+
+template <typename T>
+__device__ __forceinline__ T wave_sum(T v) {
+#pragma unroll
+    for (int o = WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = WAVE / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));
+    return v;
+}
+
+// Sum over a group of G consecutive threads (G = 64 * 2^k, G <= blockDim).
+// Groups wider than a wave combine their per-wave partials through `smem`
+// (one float per wave of the block) in a fixed order; all threads must call.
+template <int G>
+__device__ __forceinline__ float group_sum(float v, float *smem) {
+    v = wave_sum(v);
+    if constexpr (G > WAVE) {
+        const int wave = threadIdx.x / WAVE;
+        __syncthreads();
+        if ((threadIdx.x & (WAVE - 1)) == 0) smem[wave] = v;
+        __syncthreads();
+        const int first = (threadIdx.x / G) * (G / WAVE);
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < G / WAVE; ++i) s += smem[first + i];
+        v = s;
+    }
+    return v;
+}
+template <int G>
+__device__ __forceinline__ float group_max(float v, float *smem) {
+    v = wave_max(v);
+    if constexpr (G > WAVE) {
+        const int wave = threadIdx.x / WAVE;
+        __syncthreads();
+        if ((threadIdx.x & (WAVE - 1)) == 0) smem[wave] = v;
+        __syncthreads();
+        const int first = (threadIdx.x / G) * (G / WAVE);
+        float s = smem[first];
+#pragma unroll
+        for (int i = 1; i < G / WAVE; ++i) s = fmaxf(s, smem[first + i]);
+        v = s;
+    }
+    return v;
+}
+
+__device__ __forceinline__ uint32_t fastdiv(uint32_t n, const FastDivU32 &d) {
+    uint32_t t = __umulhi(d.m, n);
+    return (t + ((n - t) >> d.s1)) >> d.s2;
+}

@@ -1,0 +1,284 @@
+// mat_mul kernels for gfx950 (f16 storage, f32 accumulation).
+//
+// Canonical problem (the host maps the reference's column-major descriptor onto it):
+//     D[i, j] = alpha * sum_l P[i, l] * Q[l, j] + (read_dst ? beta * D[i, j] : 0)
+//
+//  gemm_skinny_*  : M <= 64 rows (decode: a handful of tokens against a weight
+//                   matrix).  HBM-bound: Q is streamed exactly once with 16-byte
+//                   loads straight into MFMA operand registers, P (tiny) comes
+//                   from L2, the product runs on v_mfma_f32_16x16x32_f16.
+//  gemm_generic_* : any strides / alignment, LDS-tiled FMA; the safety net.
+//  gemm_splitk_reduce : sums the f32 partials of a split-K skinny launch in a
+//                   fixed order and applies alpha / beta.
+#include "device_util.h"
+
+// ----------------------------------------------------------- skinny (MFMA) --
+//
+// Wave tile: 16*MT rows x 128 columns x 32 of K per step.  Lane (j, g) with
+// j = lane % 16, g = lane / 16 owns columns n0 + 8j .. 8j+7 and the K-slots
+// 8g .. 8g+7 of the step.
+//   QMODE 0 (Q is j-contiguous, e.g. W[K, N]): the lane loads 8 rows x 16 bytes,
+//     i.e. an 8(k) x 8(j) block, and transposes it inside its own registers
+//     (byte-permutes, no LDS, no cross-lane traffic) into eight B operands, one
+//     per column offset t.
+//   QMODE 1 (Q is l-contiguous, e.g. K-cache used as K^T): one 16-byte load per
+//     column offset t already is the B operand.
+// MFMA number t multiplies the 16 rows of P with the 16 columns {n0 + 8j + t};
+// after the eight of them a lane holds, for 4 rows, 8 consecutive columns: one
+// 16-byte store per row.
+// The block's 4 waves take interleaved K-steps and are summed through LDS; with
+// split_k > 1 the block writes f32 partials instead of the final tile.
+
+constexpr int SK_WAVES = 4;
+
+template <int QMODE>
+__device__ __forceinline__ void skinny_load_q(const GemmParams &p, const f16 *qb, uint32_t kb,
+                                              uint32_t kend, uint32_t col0, uint32_t g, u32x4 (&w)[8]) {
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+        w[r] = u32x4{0, 0, 0, 0};
+        if constexpr (QMODE == 0) {
+            const uint32_t k = kb + 8 * g + r;
+            if (k < kend && col0 < p.N) w[r] = ld128(qb + (int64_t)k * p.q_sl + col0);
+        } else {
+            const uint32_t k = kb + 8 * g, col = col0 + r;
+            if (k < kend && col < p.N) w[r] = ld128(qb + (int64_t)col * p.q_sj + k);
+        }
+    }
+}
+
+// b[t] = column t of the lane's 8x8 block: (w[0][t], ..., w[7][t])
+__device__ __forceinline__ void transpose8x8(const u32x4 (&w)[8], u32x4 (&b)[8]) {
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            const uint32_t lo = w[2 * d][t / 2], hi = w[2 * d + 1][t / 2];
+            b[t][d] = (t & 1) ? ((lo >> 16) | (hi & 0xffff0000u)) : ((lo & 0xffffu) | (hi << 16));
+        }
+    }
+}
+
+template <int MT, int QMODE>
+__device__ __forceinline__ void gemm_skinny(const GemmParams &p) {
+    __shared__ float red[SK_WAVES][32][WAVE];
+
+    const uint32_t wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    const uint32_t j16 = lane % 16, g = lane / 16;
+    const uint32_t n0 = blockIdx.x * 128;
+    const uint32_t split = blockIdx.y, bat = blockIdx.z;
+    const uint32_t kbeg = split * p.k_per_split;
+    const uint32_t kend = min(p.K, kbeg + p.k_per_split);
+    const uint32_t col0 = n0 + 8 * j16;
+
+    const f16 *qb = reinterpret_cast<const f16 *>(p.q) + (int64_t)bat * p.q_sb;
+    const f16 *pb = reinterpret_cast<const f16 *>(p.p) + (int64_t)bat * p.p_sb;
+
+    f32x4 acc[MT][8];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int t = 0; t < 8; ++t) acc[mt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    u32x4 wcur[8], wnext[8];
+    uint32_t kb = kbeg + 32 * wave;
+    if (kb < kend) skinny_load_q<QMODE>(p, qb, kb, kend, col0, g, wcur);
+    for (; kb < kend; kb += 32 * SK_WAVES) {
+        const uint32_t kn = kb + 32 * SK_WAVES;
+        if (kn < kend) skinny_load_q<QMODE>(p, qb, kn, kend, col0, g, wnext);
+
+        Pack8 a[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const uint32_t i = mt * 16 + j16, k = kb + 8 * g;
+            a[mt].u = u32x4{0, 0, 0, 0};
+            if (i < p.M && k < kend) a[mt].u = ld128(pb + (int64_t)i * p.p_si + k);
+        }
+        u32x4 b[8];
+        if constexpr (QMODE == 0) {
+            transpose8x8(wcur, b);
+        } else {
+#pragma unroll
+            for (int t = 0; t < 8; ++t) b[t] = wcur[t];
+        }
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            Pack8 bt;
+            bt.u = b[t];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+                acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[mt].h, bt.h, acc[mt][t], 0, 0, 0);
+        }
+#pragma unroll
+        for (int r = 0; r < 8; ++r) wcur[r] = wnext[r];
+    }
+
+    // combine the 4 waves, then row = mt*16 + 4g + wave, columns col0 .. col0+7
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        __syncthreads();
+#pragma unroll
+        for (int t = 0; t < 8; ++t)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) red[wave][t * 4 + q][lane] = acc[mt][t][q];
+        __syncthreads();
+        float sum[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            float s = 0.f;
+#pragma unroll
+            for (int w = 0; w < SK_WAVES; ++w) s += red[w][t * 4 + wave][lane];
+            sum[t] = s;
+        }
+        const uint32_t i = mt * 16 + 4 * g + wave;
+        if (i < p.M && col0 < p.N) {
+            if (p.split_k > 1) {
+                float *dst = reinterpret_cast<float *>(p.partial) +
+                             (((size_t)split * p.batch + bat) * p.M + i) * p.N + col0;
+                *reinterpret_cast<f32x4 *>(dst) = f32x4{sum[0], sum[1], sum[2], sum[3]};
+                *reinterpret_cast<f32x4 *>(dst + 4) = f32x4{sum[4], sum[5], sum[6], sum[7]};
+            } else {
+                f16 *dst = reinterpret_cast<f16 *>(p.d) + (int64_t)bat * p.d_sb + (int64_t)i * p.d_si;
+                if (p.d_sj == 1) {
+                    Pack8 o;
+                    if (p.read_dst) {
+                        Pack8 c;
+                        c.u = ld128(dst + col0);
+#pragma unroll
+                        for (int t = 0; t < 8; ++t) o.e[t] = f2h(p.beta * h2f(c.e[t]) + p.alpha * sum[t]);
+                    } else {
+#pragma unroll
+                        for (int t = 0; t < 8; ++t) o.e[t] = f2h(p.alpha * sum[t]);
+                    }
+                    st128(dst + col0, o.u);
+                } else {
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) {
+                        f16 *e = dst + (int64_t)(col0 + t) * p.d_sj;
+                        float r = p.alpha * sum[t];
+                        if (p.read_dst) r = p.beta * h2f(*e) + r;
+                        *e = f2h(r);
+                    }
+                }
+            }
+        }
+    }
+}
+
+#define GEMM_SKINNY(MT, QMODE)                                                                   \
+    extern "C" __global__ void __launch_bounds__(256) gemm_skinny_m##MT##_q##QMODE(GemmParams p) { \
+        gemm_skinny<MT, QMODE>(p);                                                               \
+    }
+GEMM_SKINNY(1, 0)
+GEMM_SKINNY(2, 0)
+GEMM_SKINNY(4, 0)
+GEMM_SKINNY(1, 1)
+GEMM_SKINNY(2, 1)
+GEMM_SKINNY(4, 1)
+
+// One thread per (batch, row, 8 columns): partial sums in ascending split order.
+extern "C" __global__ void __launch_bounds__(256) gemm_splitk_reduce(GemmParams p) {
+    const uint32_t nvec = p.N / 8;
+    const size_t total = (size_t)p.batch * p.M * nvec;
+    const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= total) return;
+    const uint32_t v = gid % nvec;
+    const uint32_t i = (gid / nvec) % p.M;
+    const uint32_t bat = gid / ((size_t)nvec * p.M);
+    const uint32_t col0 = v * 8;
+    float sum[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (uint32_t s = 0; s < p.split_k; ++s) {
+        const float *src = reinterpret_cast<const float *>(p.partial) +
+                           (((size_t)s * p.batch + bat) * p.M + i) * p.N + col0;
+        const f32x4 lo = *reinterpret_cast<const f32x4 *>(src);
+        const f32x4 hi = *reinterpret_cast<const f32x4 *>(src + 4);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            sum[t] += lo[t];
+            sum[4 + t] += hi[t];
+        }
+    }
+    f16 *dst = reinterpret_cast<f16 *>(p.d) + (int64_t)bat * p.d_sb + (int64_t)i * p.d_si;
+    if (p.d_sj == 1) {
+        Pack8 o;
+        if (p.read_dst) {
+            Pack8 c;
+            c.u = ld128(dst + col0);
+#pragma unroll
+            for (int t = 0; t < 8; ++t) o.e[t] = f2h(p.beta * h2f(c.e[t]) + p.alpha * sum[t]);
+        } else {
+#pragma unroll
+            for (int t = 0; t < 8; ++t) o.e[t] = f2h(p.alpha * sum[t]);
+        }
+        st128(dst + col0, o.u);
+    } else {
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            f16 *e = dst + (int64_t)(col0 + t) * p.d_sj;
+            float r = p.alpha * sum[t];
+            if (p.read_dst) r = p.beta * h2f(*e) + r;
+            *e = f2h(r);
+        }
+    }
+}
+
+// ------------------------------------------------------------ generic (FMA) --
+// 64 x 64 tile per 256-thread block, 4 x 4 outputs per thread, K-step 16.
+// Element-wise loads with arbitrary strides; used when the fast kernels'
+// alignment or contiguity requirements are not met.
+template <typename T>
+__device__ __forceinline__ void gemm_generic(const GemmParams &p) {
+    constexpr int BM = 64, BN = 64, BK = 16;
+    __shared__ float Ps[BK][BM + 4];
+    __shared__ float Qs[BK][BN + 4];
+    const uint32_t bat = blockIdx.z;
+    const uint32_t i0 = blockIdx.y * BM, j0 = blockIdx.x * BN;
+    const T *pb = reinterpret_cast<const T *>(p.p) + (int64_t)bat * p.p_sb;
+    const T *qb = reinterpret_cast<const T *>(p.q) + (int64_t)bat * p.q_sb;
+    T *db = reinterpret_cast<T *>(p.d) + (int64_t)bat * p.d_sb;
+    const uint32_t tx = threadIdx.x % 16, ty = threadIdx.x / 16;
+    float acc[4][4] = {};
+    for (uint32_t k0 = 0; k0 < p.K; k0 += BK) {
+        for (uint32_t e = threadIdx.x; e < BM * BK; e += 256) {
+            uint32_t li, ll;
+            if (p.p_sl == 1) { ll = e % BK; li = e / BK; } else { li = e % BM; ll = e / BM; }
+            const uint32_t i = i0 + li, l = k0 + ll;
+            Ps[ll][li] = (i < p.M && l < p.K) ? (float)pb[(int64_t)i * p.p_si + (int64_t)l * p.p_sl] : 0.f;
+        }
+        for (uint32_t e = threadIdx.x; e < BN * BK; e += 256) {
+            uint32_t lj, ll;
+            if (p.q_sl == 1) { ll = e % BK; lj = e / BK; } else { lj = e % BN; ll = e / BN; }
+            const uint32_t j = j0 + lj, l = k0 + ll;
+            Qs[ll][lj] = (j < p.N && l < p.K) ? (float)qb[(int64_t)l * p.q_sl + (int64_t)j * p.q_sj] : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int l = 0; l < BK; ++l) {
+            float a[4], b[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) a[r] = Ps[l][ty * 4 + r];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) b[c] = Qs[l][tx * 4 + c];
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int c = 0; c < 4; ++c) acc[r][c] += a[r] * b[c];
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint32_t i = i0 + ty * 4 + r, j = j0 + tx * 4 + c;
+            if (i < p.M && j < p.N) {
+                T *e = db + (int64_t)i * p.d_si + (int64_t)j * p.d_sj;
+                float v = p.alpha * acc[r][c];
+                if (p.read_dst) v = p.beta * (float)*e + v;
+                *e = (T)v;
+            }
+        }
+}
+
+extern "C" __global__ void __launch_bounds__(256) gemm_generic_f16(GemmParams p) { gemm_generic<f16>(p); }
+extern "C" __global__ void __launch_bounds__(256) gemm_generic_f32(GemmParams p) { gemm_generic<float>(p); }

@@ -1,0 +1,89 @@
+// Kernel parameter blocks shared by the host library and the gfx950 kernels.
+// Every kernel takes exactly one of these structs by value; the host fills it
+// and hands it to hipModuleLaunchKernel as the raw argument buffer.
+// Plain C layout only: this header is compiled by g++ (host) and hipcc (device).
+#pragma once
+#include <stdint.h>
+
+// Unsigned 32-bit division by a launch-time constant: q = n / d for any n.
+//   t = mulhi(m, n);  q = (t + ((n - t) >> s1)) >> s2
+struct FastDivU32 {
+    uint32_t m, s1, s2, d;
+};
+
+struct RmsNormParams {
+    void *y;
+    const void *x;
+    const void *w;
+    int64_t nsy, nsx;  // row strides in bytes
+    uint32_t n, d;
+    float epsilon;
+    uint32_t _pad;
+};
+
+struct SwigluParams {
+    void *gate;
+    const void *up;
+    int64_t sgn, sun;  // row strides in bytes
+    uint32_t n, d;
+};
+
+struct RopeParams {
+    void *t;
+    const void *pos;
+    int64_t st, sh, sp;  // token / head / position strides in bytes
+    uint32_t nt, nh, dh;
+    float theta;
+    uint32_t pos_is_u64;
+    uint32_t heads_per_block;
+};
+
+struct SoftmaxParams {
+    void *att;
+    int64_t sh, ss;  // head / row strides in bytes
+    uint32_t nh, seq, att_len;
+    uint32_t causal;
+};
+
+#define OPHIP_REARRANGE_MAXD 8
+struct RearrangeParams {
+    void *dst;
+    const void *src;
+    uint64_t total;  // number of chunks = count * chunks_per_unit
+    uint32_t ndim;
+    uint32_t chunks_per_unit;
+    FastDivU32 cpu_div;
+    FastDivU32 idx_div[OPHIP_REARRANGE_MAXD];
+    uint64_t idx[OPHIP_REARRANGE_MAXD];      // idx_strides (units per step of dim q)
+    int64_t dst_s[OPHIP_REARRANGE_MAXD];     // bytes
+    int64_t src_s[OPHIP_REARRANGE_MAXD];     // bytes
+};
+
+struct SampleParams {
+    void *kv;            // ophip_kv_pair*, one per row
+    const void *logits;  // rows x n
+    void *workspace;     // general path only
+    int64_t row_stride;  // bytes between rows of logits
+    uint32_t n;
+    uint32_t k_eff;      // min(top_k, n)
+    float temperature, top_p, seed;
+    uint32_t npow2;      // general path: n rounded up to a power of two
+};
+
+// Canonical GEMM seen by the kernels:
+//   D[i, j] = alpha * sum_l P[i, l] * Q[l, j] + beta * D[i, j]
+// element strides; exactly one of each operand's two strides is 1.
+struct GemmParams {
+    void *d;
+    const void *p;
+    const void *q;
+    void *partial;  // f32 [split_k][batch][M][N] when split_k > 1
+    int64_t d_si, d_sj, d_sb;
+    int64_t p_si, p_sl, p_sb;
+    int64_t q_sl, q_sj, q_sb;
+    uint32_t M, N, K, batch;
+    float alpha, beta;
+    uint32_t read_dst;  // the reference reads C only when beta != 0
+    uint32_t split_k;
+    uint32_t k_per_split;  // multiple of 32
+};

@@ -1,0 +1,95 @@
+// rearrange (N-d strided copy) for gfx950.
+//
+// The host normalises the two layouts into `count` units of `unit` contiguous
+// bytes plus per-dimension index/dst/src strides.  A unit is cut into chunks of
+// B bytes (the largest of 16/8/4/2/1 that divides the unit and keeps every
+// address aligned); chunk g belongs to unit g / chunks_per_unit.  Consecutive
+// threads take consecutive chunks, and since dimensions are ordered by
+// descending destination stride, consecutive chunks land on ascending
+// destination addresses: the stores coalesce into full lines while the loads
+// gather `unit`-byte runs.  Divisions by the launch-time constants use
+// multiply-high, so the index decode costs a few integer ops per chunk.
+// Byte-exact for any element type, negative strides and zero source strides.
+#include "device_util.h"
+
+template <int B>
+struct Chunk;
+template <>
+struct Chunk<16> { typedef u32x4 T; };
+template <>
+struct Chunk<8> { typedef u32x2 T; };
+template <>
+struct Chunk<4> { typedef uint32_t T; };
+template <>
+struct Chunk<2> { typedef uint16_t T; };
+template <>
+struct Chunk<1> { typedef uint8_t T; };
+
+constexpr int RE_ITEMS = 4;  // chunks per thread, loads issued before stores
+
+template <int B>
+__device__ __forceinline__ void rearrange32(const RearrangeParams &p) {
+    typedef typename Chunk<B>::T T;
+    const uint32_t total = (uint32_t)p.total;
+    T val[RE_ITEMS];
+    int64_t doff[RE_ITEMS];
+    bool ok[RE_ITEMS];
+#pragma unroll
+    for (int it = 0; it < RE_ITEMS; ++it) {
+        const uint32_t g = (blockIdx.x * RE_ITEMS + it) * blockDim.x + threadIdx.x;
+        ok[it] = g < total;
+        doff[it] = 0;
+        if (ok[it]) {
+            const uint32_t u = fastdiv(g, p.cpu_div);
+            const uint32_t c = g - u * p.chunks_per_unit;
+            uint32_t rem = u;
+            int64_t d = (int64_t)c * B, s = (int64_t)c * B;
+            for (uint32_t q = 0; q < p.ndim; ++q) {
+                const uint32_t k = fastdiv(rem, p.idx_div[q]);
+                rem -= k * p.idx_div[q].d;
+                d += (int64_t)k * p.dst_s[q];
+                s += (int64_t)k * p.src_s[q];
+            }
+            doff[it] = d;
+            val[it] = *reinterpret_cast<const T *>(reinterpret_cast<const char *>(p.src) + s);
+        }
+    }
+#pragma unroll
+    for (int it = 0; it < RE_ITEMS; ++it)
+        if (ok[it]) *reinterpret_cast<T *>(reinterpret_cast<char *>(p.dst) + doff[it]) = val[it];
+}
+
+// 64-bit indices: more than 2^32 chunks or an index stride beyond 32 bits.
+template <int B>
+__device__ __forceinline__ void rearrange64(const RearrangeParams &p) {
+    typedef typename Chunk<B>::T T;
+    for (uint64_t g = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; g < p.total;
+         g += (uint64_t)gridDim.x * blockDim.x) {
+        const uint64_t u = g / p.chunks_per_unit;
+        const uint64_t c = g % p.chunks_per_unit;
+        uint64_t rem = u;
+        int64_t d = (int64_t)c * B, s = (int64_t)c * B;
+        for (uint32_t q = 0; q < p.ndim; ++q) {
+            const uint64_t k = rem / p.idx[q];
+            rem %= p.idx[q];
+            d += (int64_t)k * p.dst_s[q];
+            s += (int64_t)k * p.src_s[q];
+        }
+        *reinterpret_cast<T *>(reinterpret_cast<char *>(p.dst) + d) =
+            *reinterpret_cast<const T *>(reinterpret_cast<const char *>(p.src) + s);
+    }
+}
+
+#define REARRANGE(B)                                                                             \
+    extern "C" __global__ void __launch_bounds__(256) rearrange_b##B(RearrangeParams p) {       \
+        rearrange32<B>(p);                                                                       \
+    }                                                                                            \
+    extern "C" __global__ void __launch_bounds__(256) rearrange64_b##B(RearrangeParams p) {     \
+        rearrange64<B>(p);                                                                       \
+    }
+
+REARRANGE(16)
+REARRANGE(8)
+REARRANGE(4)
+REARRANGE(2)
+REARRANGE(1)

@@ -1,0 +1,157 @@
+// rms_norm for gfx950:  y = (k * w) * x,  k = 1 / sqrt(mean(x^2) + eps).
+//
+// A row of d elements is owned by a group of G threads (one wave, or a whole
+// 256/1024-thread workgroup for few or long rows).  Each thread pulls 16-byte
+// vectors of x, keeps up to CACHE of them in registers, and the row is read
+// from HBM exactly once; w is shared by all rows and stays in L2.
+// Sum of squares: per-thread f32 partials, wave butterfly, then one LDS slot per
+// wave combined in fixed order.  The product keeps the reference's (k*w)*x
+// order and 1/sqrt is the IEEE divide and square root.
+#include "device_util.h"
+
+template <typename TA>
+struct Vec;  // 16 bytes of TA
+template <>
+struct Vec<f16> {
+    static constexpr int N = 8;
+    Pack8 v;
+    __device__ __forceinline__ float get(int i) const { return h2f(v.e[i]); }
+    __device__ __forceinline__ void set(int i, float f) { v.e[i] = f2h(f); }
+};
+template <>
+struct Vec<float> {
+    static constexpr int N = 4;
+    Pack4f v;
+    __device__ __forceinline__ float get(int i) const { return v.e[i]; }
+    __device__ __forceinline__ void set(int i, float f) { v.e[i] = f; }
+};
+
+template <typename TW>
+__device__ __forceinline__ float load_w(const void *w, uint32_t j) {
+    return (float)reinterpret_cast<const TW *>(w)[j];
+}
+
+// N consecutive weights starting at element j (j multiple of N, base 16-byte aligned)
+template <typename TW, int N>
+__device__ __forceinline__ void load_w_vec(const void *w, uint32_t j, float (&out)[N]) {
+    if constexpr (sizeof(TW) == 2) {
+        static_assert(N == 8, "");
+        Pack8 p;
+        p.u = ld128(reinterpret_cast<const f16 *>(w) + j);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) out[i] = h2f(p.e[i]);
+    } else {
+#pragma unroll
+        for (int c = 0; c < N / 4; ++c) {
+            Pack4f p;
+            p.u = ld128(reinterpret_cast<const float *>(w) + j + 4 * c);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) out[4 * c + i] = p.e[i];
+        }
+    }
+}
+
+template <typename TA, typename TW, int G>
+__device__ __forceinline__ void rms_norm_vec(const RmsNormParams &p) {
+    constexpr int N = Vec<TA>::N;
+    constexpr int CACHE = 8;
+    constexpr int BLOCK = G < 256 ? 256 : G;
+    constexpr int RPB = BLOCK / G;
+    __shared__ float smem[BLOCK / WAVE];
+
+    const uint32_t lane = threadIdx.x % G;
+    uint32_t row = blockIdx.x * RPB + threadIdx.x / G;
+    const bool live = row < p.n;
+    if (!live) row = p.n - 1;  // keep every thread on the barriers; stores are suppressed
+
+    const char *xr = reinterpret_cast<const char *>(p.x) + (int64_t)row * p.nsx;
+    char *yr = reinterpret_cast<char *>(p.y) + (int64_t)row * p.nsy;
+    const uint32_t nvec = p.d / N;
+
+    Vec<TA> cache[CACHE];
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < CACHE; ++c) {
+        const uint32_t v = lane + c * G;
+        if (v < nvec) {
+            cache[c].v.u = ld128(xr + (size_t)v * 16);
+#pragma unroll
+            for (int i = 0; i < N; ++i) {
+                const float f = cache[c].get(i);
+                ss += f * f;
+            }
+        }
+    }
+    for (uint32_t v = lane + CACHE * G; v < nvec; v += G) {
+        Vec<TA> t;
+        t.v.u = ld128(xr + (size_t)v * 16);
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            const float f = t.get(i);
+            ss += f * f;
+        }
+    }
+    ss = group_sum<G>(ss, smem);
+    const float k = 1.0f / sqrtf(ss / (float)p.d + p.epsilon);
+
+#pragma unroll
+    for (int c = 0; c < CACHE; ++c) {
+        const uint32_t v = lane + c * G;
+        if (v < nvec) {
+            float w[N];
+            load_w_vec<TW, N>(p.w, v * N, w);
+            Vec<TA> o;
+#pragma unroll
+            for (int i = 0; i < N; ++i) o.set(i, (k * w[i]) * cache[c].get(i));
+            if (live) st128(yr + (size_t)v * 16, o.v.u);
+        }
+    }
+    for (uint32_t v = lane + CACHE * G; v < nvec; v += G) {
+        Vec<TA> t, o;
+        t.v.u = ld128(xr + (size_t)v * 16);
+        float w[N];
+        load_w_vec<TW, N>(p.w, v * N, w);
+#pragma unroll
+        for (int i = 0; i < N; ++i) o.set(i, (k * w[i]) * t.get(i));
+        if (live) st128(yr + (size_t)v * 16, o.v.u);
+    }
+}
+
+// Element-wise variant for rows that are not 16-byte friendly (odd d, odd strides).
+template <typename TA, typename TW>
+__device__ __forceinline__ void rms_norm_scalar(const RmsNormParams &p) {
+    constexpr int G = 256;
+    __shared__ float smem[G / WAVE];
+    const uint32_t row = blockIdx.x;
+    const TA *xr = reinterpret_cast<const TA *>(reinterpret_cast<const char *>(p.x) + (int64_t)row * p.nsx);
+    TA *yr = reinterpret_cast<TA *>(reinterpret_cast<char *>(p.y) + (int64_t)row * p.nsy);
+    float ss = 0.f;
+    for (uint32_t j = threadIdx.x; j < p.d; j += G) {
+        const float f = (float)xr[j];
+        ss += f * f;
+    }
+    ss = group_sum<G>(ss, smem);
+    const float k = 1.0f / sqrtf(ss / (float)p.d + p.epsilon);
+    for (uint32_t j = threadIdx.x; j < p.d; j += G)
+        yr[j] = (TA)((k * load_w<TW>(p.w, j)) * (float)xr[j]);
+}
+
+#define RMS_VEC(NAME, TA, TW, G)                                                        \
+    extern "C" __global__ void __launch_bounds__((G) < 256 ? 256 : (G)) NAME(RmsNormParams p) { \
+        rms_norm_vec<TA, TW, G>(p);                                                     \
+    }
+#define RMS_SCALAR(NAME, TA, TW) \
+    extern "C" __global__ void __launch_bounds__(256) NAME(RmsNormParams p) { rms_norm_scalar<TA, TW>(p); }
+
+RMS_VEC(rms_norm_f16_f16_g64, f16, f16, 64)
+RMS_VEC(rms_norm_f16_f16_g256, f16, f16, 256)
+RMS_VEC(rms_norm_f16_f16_g1024, f16, f16, 1024)
+RMS_VEC(rms_norm_f16_f32_g64, f16, float, 64)
+RMS_VEC(rms_norm_f16_f32_g256, f16, float, 256)
+RMS_VEC(rms_norm_f16_f32_g1024, f16, float, 1024)
+RMS_VEC(rms_norm_f32_f32_g64, float, float, 64)
+RMS_VEC(rms_norm_f32_f32_g256, float, float, 256)
+RMS_VEC(rms_norm_f32_f32_g1024, float, float, 1024)
+RMS_SCALAR(rms_norm_f16_f16_scalar, f16, f16)
+RMS_SCALAR(rms_norm_f16_f32_scalar, f16, float)
+RMS_SCALAR(rms_norm_f32_f32_scalar, float, float)

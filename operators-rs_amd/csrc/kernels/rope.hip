@@ -1,0 +1,75 @@
+// rope for gfx950: in-place rotary embedding on adjacent pairs (2k, 2k+1).
+//
+// One workgroup serves one token (optionally one slice of its heads).  The dh/2
+// (sin, cos) pairs of the token depend only on its position, so they are
+// evaluated once per workgroup into LDS with the accurate powf / sinf / cosf
+// (angles reach hundreds of radians, so the range reduction matters) and then
+// shared by every head: nh times fewer transcendentals than one evaluation per
+// element.  Each thread then rotates 16 bytes (4 pairs) per step in registers;
+// every byte of t is read once and written once.
+//   ang = f32(pos) / powf(theta, f32(k) / f32(dh/2));  [a, b] <- [a c - b s, a s + b c]
+#include "device_util.h"
+
+extern __shared__ float2 rope_sc[];  // dh/2 entries of (sin, cos)
+
+__device__ __forceinline__ float rope_pos(const RopeParams &p, uint32_t token) {
+    const char *pp = reinterpret_cast<const char *>(p.pos) + (int64_t)token * p.sp;
+    if (p.pos_is_u64) return (float)*reinterpret_cast<const uint64_t *>(pp);
+    return (float)*reinterpret_cast<const uint32_t *>(pp);
+}
+
+__device__ __forceinline__ void rope_fill_table(const RopeParams &p, uint32_t token) {
+    const uint32_t H = p.dh / 2;
+    const float pos = rope_pos(p, token);
+    for (uint32_t k = threadIdx.x; k < H; k += blockDim.x) {
+        const float ang = pos / powf(p.theta, (float)k / (float)H);
+        rope_sc[k] = make_float2(sinf(ang), cosf(ang));
+    }
+    __syncthreads();
+}
+
+extern "C" __global__ void __launch_bounds__(256) rope_f16_vec(RopeParams p) {
+    const uint32_t token = blockIdx.x;
+    rope_fill_table(p, token);
+    const uint32_t cpv = p.dh / 8;  // 16-byte chunks per head
+    const uint32_t h0 = blockIdx.y * p.heads_per_block;
+    const uint32_t h1 = min(h0 + p.heads_per_block, p.nh);
+    const uint32_t total = (h1 - h0) * cpv;
+    char *base = reinterpret_cast<char *>(p.t) + (int64_t)token * p.st;
+    for (uint32_t v = threadIdx.x; v < total; v += blockDim.x) {
+        const uint32_t h = h0 + v / cpv, c = v % cpv;
+        char *ptr = base + (int64_t)h * p.sh + (size_t)c * 16;
+        Pack8 x, o;
+        x.u = ld128(ptr);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float2 sc = rope_sc[4 * c + i];
+            const float a = h2f(x.e[2 * i]), b = h2f(x.e[2 * i + 1]);
+            o.e[2 * i] = f2h(a * sc.y - b * sc.x);
+            o.e[2 * i + 1] = f2h(a * sc.x + b * sc.y);
+        }
+        st128(ptr, o.u);
+    }
+}
+
+template <typename T>
+__device__ __forceinline__ void rope_pairs(const RopeParams &p) {
+    const uint32_t token = blockIdx.x;
+    rope_fill_table(p, token);
+    const uint32_t H = p.dh / 2;
+    const uint32_t h0 = blockIdx.y * p.heads_per_block;
+    const uint32_t h1 = min(h0 + p.heads_per_block, p.nh);
+    const uint32_t total = (h1 - h0) * H;
+    char *base = reinterpret_cast<char *>(p.t) + (int64_t)token * p.st;
+    for (uint32_t v = threadIdx.x; v < total; v += blockDim.x) {
+        const uint32_t h = h0 + v / H, k = v % H;
+        T *ptr = reinterpret_cast<T *>(base + (int64_t)h * p.sh) + 2 * k;
+        const float2 sc = rope_sc[k];
+        const float a = (float)ptr[0], b = (float)ptr[1];
+        ptr[0] = (T)(a * sc.y - b * sc.x);
+        ptr[1] = (T)(a * sc.x + b * sc.y);
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(256) rope_f16_pairs(RopeParams p) { rope_pairs<f16>(p); }
+extern "C" __global__ void __launch_bounds__(256) rope_f32_pairs(RopeParams p) { rope_pairs<float>(p); }

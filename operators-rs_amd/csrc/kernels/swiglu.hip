@@ -1,0 +1,41 @@
+// swiglu for gfx950:  gate <- (a * sigmoid(a)) * b,  a = gate, b = up, f32 inside.
+//
+// Pure streaming: every thread moves one 16-byte vector of gate and one of up
+// per step; gate and up rows carry independent byte strides because they are
+// normally the two halves of one [n, 2*di] GEMM output.
+#include "device_util.h"
+
+__device__ __forceinline__ float swiglu_f32(float a, float b) {
+    // same evaluation order as the reference: a * (1 / (1 + exp(-a))) * b
+    const float sig = 1.0f / (1.0f + expf(-a));
+    return (a * sig) * b;
+}
+
+extern "C" __global__ void __launch_bounds__(256) swiglu_f16_vec(SwigluParams p) {
+    const uint32_t nvec = p.d / 8;
+    for (uint32_t row = blockIdx.y; row < p.n; row += gridDim.y) {
+        char *g = reinterpret_cast<char *>(p.gate) + (int64_t)row * p.sgn;
+        const char *u = reinterpret_cast<const char *>(p.up) + (int64_t)row * p.sun;
+        for (uint32_t v = blockIdx.x * blockDim.x + threadIdx.x; v < nvec; v += gridDim.x * blockDim.x) {
+            Pack8 a, b, o;
+            a.u = ld128(g + (size_t)v * 16);
+            b.u = ld128(u + (size_t)v * 16);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) o.e[i] = f2h(swiglu_f32(h2f(a.e[i]), h2f(b.e[i])));
+            st128(g + (size_t)v * 16, o.u);
+        }
+    }
+}
+
+template <typename T>
+__device__ __forceinline__ void swiglu_scalar(const SwigluParams &p) {
+    for (uint32_t row = blockIdx.y; row < p.n; row += gridDim.y) {
+        T *g = reinterpret_cast<T *>(reinterpret_cast<char *>(p.gate) + (int64_t)row * p.sgn);
+        const T *u = reinterpret_cast<const T *>(reinterpret_cast<const char *>(p.up) + (int64_t)row * p.sun);
+        for (uint32_t j = blockIdx.x * blockDim.x + threadIdx.x; j < p.d; j += gridDim.x * blockDim.x)
+            g[j] = (T)swiglu_f32((float)g[j], (float)u[j]);
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(256) swiglu_f16_scalar(SwigluParams p) { swiglu_scalar<f16>(p); }
+extern "C" __global__ void __launch_bounds__(256) swiglu_f32_scalar(SwigluParams p) { swiglu_scalar<float>(p); }
