@@ -1,0 +1,385 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X backend on the operators-rs hot path.
+
+One "step" is one pass of the Llama-7B-shape decode layer (16 tokens, d = 4096,
+32 heads x 128, KV length 2048, FFN 11008) through the operator API: rms_norm,
+QKV mat_mul, rope(q), rope(k), QK^T mat_mul, causal softmax, PV mat_mul, O-proj
+mat_mul, rms_norm, gate/up mat_mul, swiglu, down mat_mul - twelve launches on one
+stream, inputs resident in HBM, synthetic data.  `value` is the layer's
+algorithmic bytes divided by the measured time per step.
+
+Beside it the script reports, in the same JSON line:
+  per_op       every operator at its benchmark shape (and a scaled shape large
+               enough to leave the 256 MiB Infinity Cache): us/op, GB/s or
+               TFLOP/s, fraction of the roofline;
+  roofline     the dominant kernel of the step (the gate/up weight-streaming
+               mat_mul), timed with HIP events inside the timed region;
+  cpu_baseline the CPU oracle (a port of the crate's CPU backend) timed on the
+               same layer on the host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "operators-rs_amd"))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12        # B/s, MI355X HBM3E
+MFMA_F16_PEAK = 2.5e15   # flop/s, MI355X dense f16 MFMA
+
+NT, D, NH, DH, KV, DI = 16, 4096, 32, 128, 2048, 11008
+f16 = np.float16
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def normal_f16(rng, shape, std):
+    return (rng.standard_normal(shape, dtype=np.float32) * np.float32(std)).astype(f16)
+
+
+class Layer:
+    """Device buffers, Args and operators of one decode layer."""
+
+    def __init__(self, ophip, gpu, rng, host=False):
+        L, F16 = ophip.TensorLayout, ophip.dt.F16
+        self.ophip, self.gpu = ophip, gpu
+        h = self.h = {}
+        h["x"] = normal_f16(rng, (NT, D), 1.0)
+        h["w_norm1"] = rng.uniform(0.5, 1.5, D).astype(np.float32).astype(f16)
+        h["w_norm2"] = rng.uniform(0.5, 1.5, D).astype(np.float32).astype(f16)
+        h["w_qkv"] = normal_f16(rng, (D, 3 * D), 0.02)
+        h["w_o"] = normal_f16(rng, (D, D), 0.02)
+        h["w_gu"] = normal_f16(rng, (D, 2 * DI), 0.02)
+        h["w_d"] = normal_f16(rng, (DI, D), 0.02)
+        h["k_cache"] = normal_f16(rng, (NH, KV, DH), 1.0)
+        h["v_cache"] = normal_f16(rng, (NH, KV, DH), 1.0)
+        h["pos"] = (np.arange(NT) + KV - NT).astype(np.uint32)
+        d = self.d = {k: gpu.from_host(v) for k, v in h.items()}
+        for name, nbytes in [("xn", NT * D * 2), ("qkv", NT * 3 * D * 2), ("att", NH * NT * KV * 2),
+                             ("o", NT * D * 2), ("y", NT * D * 2), ("yn", NT * D * 2), ("gu", NT * 2 * DI * 2),
+                             ("out", NT * D * 2), ("ws", 64 << 20)]:
+            d[name] = gpu.malloc(nbytes)
+        if not host:
+            self.h = {k: v for k, v in h.items() if k in ("x",)}  # drop host weights
+
+        c = lambda *s: L.new_contiguous(F16, list(s))
+        q_lay = L(F16, [NT, NH, DH], [3 * D * 2, DH * 2, 2])          # q / k views inside qkv
+        qb_lay = L(F16, [NH, NT, DH], [DH * 2, 3 * D * 2, 2])         # q as [head, token, dh]
+        kt_lay = L(F16, [NH, DH, KV], [KV * DH * 2, 2, DH * 2])       # K-cache as K^T
+        ob_lay = L(F16, [NH, NT, DH], [DH * 2, D * 2, 2])             # attention output as [token, head*dh]
+        half = L(F16, [NT, DI], [2 * DI * 2, 2])                      # gate / up halves of gu
+        empty = L(F16, [0, DH], [2 * DH, 2])
+        o = ophip
+        self.ops = dict(rms=o.RmsNorm(gpu), mm=o.MatMul(gpu), rope=o.Rope(gpu), sm=o.FusedSoftmax(gpu),
+                        sw=o.Swiglu(gpu))
+        A = self.args = {}
+        A["rms_norm_1"] = ("rms", o.RmsNormArgs(c(NT, D), d["xn"], c(NT, D), d["x"], c(D), d["w_norm1"], 1e-5))
+        A["qkv"] = ("mm", o.MatMulArgs(c(NT, 3 * D), d["qkv"], 0.0, c(NT, D), d["xn"], c(D, 3 * D), d["w_qkv"], 1.0))
+        A["rope_q"] = ("rope", o.RopeArgs(q_lay, d["qkv"].ptr, c(NT), d["pos"], empty, None, empty, None, 1e4))
+        A["rope_k"] = ("rope", o.RopeArgs(q_lay, d["qkv"].ptr + D * 2, c(NT), d["pos"], empty, None, empty, None, 1e4))
+        A["rope_q"][1].p_layout = A["rope_k"][1].p_layout = L(o.dt.U32, [NT], [4])
+        A["qk_t"] = ("mm", o.MatMulArgs(c(NH, NT, KV), d["att"], 0.0, qb_lay, d["qkv"].ptr, kt_lay, d["k_cache"],
+                                        float(1.0 / np.sqrt(DH))))
+        A["softmax"] = ("sm", o.FusedSoftmaxArgs(o.AttnMask.CAUSAL, c(NH, NT, KV), d["att"]))
+        A["pv"] = ("mm", o.MatMulArgs(ob_lay, d["o"], 0.0, c(NH, NT, KV), d["att"], c(NH, KV, DH), d["v_cache"], 1.0))
+        A["o_proj"] = ("mm", o.MatMulArgs(c(NT, D), d["y"], 0.0, c(NT, D), d["o"], c(D, D), d["w_o"], 1.0))
+        A["rms_norm_2"] = ("rms", o.RmsNormArgs(c(NT, D), d["yn"], c(NT, D), d["y"], c(D), d["w_norm2"], 1e-5))
+        A["gate_up"] = ("mm", o.MatMulArgs(c(NT, 2 * DI), d["gu"], 0.0, c(NT, D), d["yn"], c(D, 2 * DI), d["w_gu"], 1.0))
+        A["swiglu"] = ("sw", o.SwigluArgs(half, d["gu"].ptr, half, d["gu"].ptr + DI * 2))
+        A["down"] = ("mm", o.MatMulArgs(c(NT, D), d["out"], 0.0, half, d["gu"].ptr, c(DI, D), d["w_d"], 1.0))
+        self.order = ["rms_norm_1", "qkv", "rope_q", "rope_k", "qk_t", "softmax", "pv", "o_proj", "rms_norm_2",
+                      "gate_up", "swiglu", "down"]
+        for name in self.order:
+            kind, a = A[name]
+            self.ops[kind].scheme(a, 64 << 20)
+
+    def launch(self, name, stream):
+        kind, a = self.args[name]
+        self.ops[kind].launch(a, self.d["ws"], stream)
+
+    def step(self, stream, around=None):
+        for name in self.order:
+            if around and name in around:
+                around[name][0].record(stream)
+                self.launch(name, stream)
+                around[name][1].record(stream)
+            else:
+                self.launch(name, stream)
+
+
+# algorithmic bytes (f16 operands read once, outputs written once) and flops per op of the layer
+def layer_work():
+    gemm = lambda m, n, k, b=1: (2 * b * (m * k + k * n + m * n), 2 * b * m * n * k)
+    w = {
+        "rms_norm_1": (2 * NT * D * 2 + D * 2, 0),
+        "qkv": gemm(NT, 3 * D, D),
+        "rope_q": (2 * NT * NH * DH * 2 + NT * 4, 0),
+        "rope_k": (2 * NT * NH * DH * 2 + NT * 4, 0),
+        "qk_t": gemm(NT, KV, DH, NH),
+        "softmax": (2 * NH * NT * KV * 2, 0),
+        "pv": gemm(NT, DH, KV, NH),
+        "o_proj": gemm(NT, D, D),
+        "rms_norm_2": (2 * NT * D * 2 + D * 2, 0),
+        "gate_up": gemm(NT, 2 * DI, D),
+        "swiglu": (3 * NT * DI * 2, 0),
+        "down": gemm(NT, D, DI),
+    }
+    return w
+
+
+def time_launches(gpu, stream, fn, reps, warm=5):
+    for _ in range(warm):
+        fn()
+    e0, e1 = gpu.event(), gpu.event()
+    stream.synchronize()
+    e0.record(stream)
+    for _ in range(reps):
+        fn()
+    e1.record(stream)
+    e1.synchronize()
+    return e0.elapsed_ms(e1) * 1e3 / reps  # us per launch
+
+
+def standalone_ops(ophip, gpu, stream, rng, reps):
+    """Every operator at its benchmark shape plus a scaled shape that does not fit the Infinity Cache."""
+    o, L, F16 = ophip, ophip.TensorLayout, ophip.dt.F16
+    c = lambda *s: L.new_contiguous(F16, list(s))
+    out = []
+
+    def add(name, shape, nbytes, us, flops=0, note=None):
+        rec = {"op": name, "shape": shape, "us": round(us, 3), "bytes": nbytes,
+               "GBps": round(nbytes / us / 1e3, 1), "hbm_frac": round(nbytes / (us * 1e-6) / HBM_PEAK, 4)}
+        if flops:
+            rec["TFLOPs"] = round(flops / us / 1e6, 2)
+            rec["mfma_frac"] = round(flops / (us * 1e-6) / MFMA_F16_PEAK, 4)
+        if nbytes < (256 << 20):
+            rec["cache_resident"] = True
+        if note:
+            rec["note"] = note
+        out.append(rec)
+        log("  %-28s %-22s %10.2f us %9.1f GB/s  %5.1f%% HBM%s" % (
+            name, shape, us, rec["GBps"], 100 * rec["hbm_frac"],
+            ("  %.1f TFLOP/s %.1f%% MFMA" % (rec["TFLOPs"], 100 * rec["mfma_frac"])) if flops else ""))
+
+    # rms_norm: [64, 4096] and [65536, 4096]
+    rms = o.RmsNorm(gpu)
+    for n in (64, 65536):
+        x = gpu.malloc(n * D * 2)
+        y = gpu.malloc(n * D * 2)
+        gpu.memset(x, 0x3C)
+        w = gpu.from_host(np.ones(D, f16))
+        a = o.RmsNormArgs(c(n, D), y, c(n, D), x, c(D), w, 1e-5)
+        rms.scheme(a, 0)
+        us = time_launches(gpu, stream, lambda: rms.launch(a, None, stream), reps)
+        add("rms_norm", "[%d,%d]" % (n, D), 2 * n * D * 2 + D * 2, us)
+        x.free(); y.free()
+    # rope: [512, 32, 128] and [32768, 32, 128]
+    rope = o.Rope(gpu)
+    empty = L(F16, [0, DH], [2 * DH, 2])
+    for nt in (512, 32768):
+        t = gpu.malloc(nt * NH * DH * 2)
+        gpu.memset(t, 0x3C)
+        pos = gpu.from_host((np.arange(nt) % 4096).astype(np.uint32))
+        a = o.RopeArgs(c(nt, NH, DH), t, L(o.dt.U32, [nt], [4]), pos, empty, None, empty, None, 1e4)
+        us = time_launches(gpu, stream, lambda: rope.launch(a, None, stream), reps)
+        add("rope", "[%d,%d,%d]" % (nt, NH, DH), 2 * nt * NH * DH * 2 + nt * 4, us)
+        t.free()
+    # rearrange: [32, 512, 128] -> [512, 32, 128] and a 64x larger one
+    rea = o.Rearrange(gpu)
+    for s0, s1 in ((32, 512), (32, 32768)):
+        src = gpu.malloc(s0 * s1 * DH * 2)
+        dst = gpu.malloc(s0 * s1 * DH * 2)
+        gpu.memset(src, 0x3C)
+        a = o.RearrangeArgs(L(F16, [s0, s1, DH], [DH * 2, s0 * DH * 2, 2]), dst, c(s0, s1, DH), src)
+        us = time_launches(gpu, stream, lambda: rea.launch(a, None, stream), reps)
+        add("rearrange", "[%d,%d,%d]->T" % (s0, s1, DH), 2 * s0 * s1 * DH * 2, us)
+        src.free(); dst.free()
+    # fused softmax: prefill [32, 512, 512], decode [32, 1, 2048], scaled [32, 8192, 2048] (no mask to keep all columns)
+    sm = o.FusedSoftmax(gpu)
+    for nh, seq, al, mask in ((32, 512, 512, 1), (32, 1, 2048, 1), (32, 8192, 2048, 0)):
+        att_host = None
+        att = gpu.malloc(nh * seq * al * 2)
+        gpu.memset(att, 0x3C)
+        a = o.FusedSoftmaxArgs(mask, c(nh, seq, al), att)
+        us = time_launches(gpu, stream, lambda: sm.launch(a, None, stream), reps)
+        add("fused_softmax", "[%d,%d,%d]%s" % (nh, seq, al, "" if mask else " nomask"), 2 * nh * seq * al * 2, us)
+        att.free()
+    # swiglu: [16, 11008] halves and [8192, 11008]
+    sw = o.Swiglu(gpu)
+    for n in (16, 8192):
+        gu = gpu.malloc(n * 2 * DI * 2)
+        gpu.memset(gu, 0x3C)
+        half = L(F16, [n, DI], [2 * DI * 2, 2])
+        a = o.SwigluArgs(half, gu.ptr, half, gu.ptr + DI * 2)
+        us = time_launches(gpu, stream, lambda: sw.launch(a, None, stream), reps)
+        add("swiglu", "[%d,%d]" % (n, DI), 3 * n * DI * 2, us)
+        gu.free()
+    # random_sample: 16 rows x [32000], one launch per row as the API prescribes
+    rs = o.RandomSample(gpu)
+    logits = gpu.from_host(normal_f16(rng, (16, 32000), np.sqrt(3.0)))
+    kv = gpu.malloc(16 * 8)
+    for mode, cfg, seed in (("argmax", o.SampleArgs.argmax(), 0.0), ("top-k 50 / top-p 0.9", o.SampleArgs(0.8, 0.9, 50), 0.37)):
+        arg_rows = []
+        for r in range(16):
+            a = o.RandomSampleArgs.layout(F16, 32000)
+            a.kv_pair_base, a.logits_base, a.config, a.seed = kv.ptr + 8 * r, logits.ptr + r * 64000, cfg, seed
+            arg_rows.append(a)
+
+        def run16():
+            for a in arg_rows:
+                rs.launch(a, None, stream)
+        us = time_launches(gpu, stream, run16, max(reps // 4, 5))
+        add("random_sample " + mode, "16 x [32000]", 16 * (32000 * 2 + 8), us, note="16 launches")
+    # compute-bound mat_mul: 4096^3 and 8192^3
+    mm = o.MatMul(gpu)
+    for n in (4096, 8192):
+        A_, B_, C_ = gpu.malloc(n * n * 2), gpu.malloc(n * n * 2), gpu.malloc(n * n * 2)
+        gpu.memset(A_, 0x3C); gpu.memset(B_, 0x3C)
+        a = o.MatMulArgs(c(n, n), C_, 0.0, c(n, n), A_, c(n, n), B_, 1.0)
+        mm.scheme(a, 0)
+        us = time_launches(gpu, stream, lambda: mm.launch(a, None, stream), 3, warm=1)
+        add("mat_mul", "%d^3" % n, 3 * n * n * 2, us, flops=2 * n ** 3)
+        A_.free(); B_.free(); C_.free()
+    return out
+
+
+def cpu_layer_step(oracle, h, threads):
+    """The same twelve operations through the CPU oracle (threads on the axes the reference hands to rayon)."""
+    oracle.set_threads(threads)
+    xn = oracle.rms_norm(np.empty_like(h["x"]), h["x"], h["w_norm1"], 1e-5)
+    qkv = oracle.mat_mul(np.zeros((NT, 3 * D), f16), 0.0, xn, h["w_qkv"], 1.0)
+    oracle.set_threads(1)  # rope is single-threaded in the reference
+    oracle.rope(qkv[:, :D].reshape(NT, NH, DH), h["pos"], 1e4)
+    oracle.rope(qkv[:, D:2 * D].reshape(NT, NH, DH), h["pos"], 1e4)
+    oracle.set_threads(threads)
+    q = qkv[:, :D].reshape(NT, NH, DH).transpose(1, 0, 2)
+    att = oracle.mat_mul(np.zeros((NH, NT, KV), f16), 0.0, q, h["k_cache"].transpose(0, 2, 1), float(1 / np.sqrt(DH)))
+    oracle.fused_softmax(att, causal=True)
+    o = np.zeros((NT, D), f16)
+    oracle.mat_mul(o.reshape(NT, NH, DH).transpose(1, 0, 2), 0.0, att, h["v_cache"], 1.0)
+    y = oracle.mat_mul(np.zeros((NT, D), f16), 0.0, o, h["w_o"], 1.0)
+    yn = oracle.rms_norm(np.empty_like(y), y, h["w_norm2"], 1e-5)
+    gu = oracle.mat_mul(np.zeros((NT, 2 * DI), f16), 0.0, yn, h["w_gu"], 1.0)
+    oracle.set_threads(1)  # swiglu is single-threaded in the reference
+    oracle.swiglu(gu[:, :DI], gu[:, DI:])
+    oracle.set_threads(threads)
+    out = oracle.mat_mul(np.zeros((NT, D), f16), 0.0, gu[:, :DI], h["w_d"], 1.0)
+    oracle.set_threads(1)
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--reps", type=int, default=100, help="launches per standalone-operator timing")
+    ap.add_argument("--no-per-op", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+
+    import ophip
+    if not os.path.exists(ophip.LIB_PATH):
+        import __graft_entry__
+        __graft_entry__.build()
+    gpu = ophip.Gpu(0)
+    info = gpu.info()
+    log("device: %s (%s), %d CUs" % (info.name.decode(), info.arch.decode(), info.compute_units))
+    stream = gpu.stream()
+    rng = np.random.default_rng(0)
+
+    # two layers' worth of distinct weights (2 x 404 MB), alternated per step, so no
+    # step finds its weights in the 256 MiB Infinity Cache
+    layers = [Layer(ophip, gpu, rng, host=(i == 0)) for i in range(2)]
+    work = layer_work()
+    layer_bytes = sum(b for b, _ in work.values())
+    layer_flops = sum(f for _, f in work.values())
+
+    for i in range(args.warmup):
+        layers[i % 2].step(stream)
+    stream.synchronize()
+
+    DOM = "gate_up"
+    pairs = [(gpu.event(), gpu.event()) for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        layers[i % 2].step(stream, around={DOM: pairs[i]})
+    stream.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    dom_us = float(np.mean([a.elapsed_ms(b) for a, b in pairs])) * 1e3
+    dom_bytes = work[DOM][0]
+
+    # per-op times inside the layer (back-to-back launches of one op; small ops are cache-resident)
+    per_layer = []
+    log("decode layer, per op:")
+    for name in layers[0].order:
+        us = time_launches(gpu, stream, lambda: layers[0].launch(name, stream), args.reps)
+        b, f = work[name]
+        rec = {"op": name, "us": round(us, 3), "bytes": b, "GBps": round(b / us / 1e3, 1),
+               "hbm_frac": round(b / (us * 1e-6) / HBM_PEAK, 4)}
+        if f:
+            rec["TFLOPs"] = round(f / us / 1e6, 2)
+        if b < (256 << 20):
+            rec["cache_resident"] = True
+        per_layer.append(rec)
+        log("  %-12s %9.2f us %9.1f GB/s %5.1f%% HBM" % (name, us, rec["GBps"], 100 * rec["hbm_frac"]))
+
+    per_op = []
+    if not args.no_per_op:
+        log("standalone operators:")
+        per_op = standalone_ops(ophip, gpu, stream, rng, args.reps)
+
+    cpu = None
+    if not args.no_cpu:
+        import oracle
+        threads = min(oracle.max_threads(), 16)
+        h = layers[0].h
+        t_cpu, n_cpu = 0.0, 0
+        while n_cpu < 2 or (t_cpu < 10.0 and n_cpu < 20):
+            c0 = time.perf_counter()
+            cpu_layer_step(oracle, h, threads)
+            t_cpu += time.perf_counter() - c0
+            n_cpu += 1
+        cpu = {"value": round(layer_bytes / (t_cpu / n_cpu) / 1e9, 3), "unit": "GB/s", "cores": threads,
+               "kind": "port", "ms_per_step": round(t_cpu / n_cpu * 1e3, 2),
+               "sample": "%d full decode-layer steps of the same workload through the CPU oracle" % n_cpu}
+
+    result = {
+        "metric": "per-op HBM GB/s (% of 8 TB/s) + us/op at Llama-7B shapes; mat_mul MFMA %",
+        "value": round(layer_bytes / (ms_per_step * 1e-3) / 1e9, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "llama7b_decode_layer_16tok_kv2048 (BASELINE.json configs[4])",
+                   "launches_per_step": len(layers[0].order), "algorithmic_bytes_per_step": layer_bytes,
+                   "flops_per_step": layer_flops, "hbm_frac_of_step": round(layer_bytes / (ms_per_step * 1e-3) / HBM_PEAK, 4)},
+        "roofline": {"bound": "hbm", "kernel": "gemm_skinny (gate/up mat_mul 16x4096 . 4096x22016)",
+                     "achieved": round(dom_bytes / (dom_us * 1e-6) / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": round(dom_bytes / (dom_us * 1e-6) / HBM_PEAK, 4), "traffic": None,
+                     "us": round(dom_us, 3), "algorithmic_bytes": dom_bytes},
+        "cpu_baseline": cpu,
+        "per_op_layer": per_layer,
+        "per_op": per_op,
+    }
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

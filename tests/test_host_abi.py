@@ -1,0 +1,194 @@
+"""CPU-only checks of the C ABI: the library loads, exports every declared symbol,
+and its host-side logic (layout normalisers, validators, allocator bookkeeping)
+agrees with the reference's known answers and with the oracle.  No compute call
+is made here, so no GPU is needed."""
+import os
+import re
+
+import numpy as np
+import pytest
+
+import ophip
+import oracle
+from ophip import TensorLayout, dt
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+F16 = dt.F16
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "ophip.h")).read()
+    declared = set(re.findall(r"OPHIP_API[^;(]*?\b(ophip_[a-z0-9_]+)\s*\(", header))
+    assert len(declared) >= 60
+    L = ophip.lib()
+    missing = sorted(s for s in declared if not hasattr(L, s))
+    assert not missing, missing
+    assert declared == set(ophip.EXPORTS)
+
+
+def test_status_names_and_dtype_sizes():
+    L = ophip.lib()
+    names = ["Ok", "TypeNotSupport", "TypeMismatch", "RankNotSupport", "RankMismatch", "ShapeNotSupport",
+             "ShapeMismatch", "StridesNotSupport", "ArgsNotSupport", "DynamicNotSupport"]
+    assert [L.ophip_status_name(i).decode() for i in range(10)] == names
+    assert L.ophip_status_name(100).decode() == "ExecutionFailed"
+    for d in range(1, 15):
+        assert L.ophip_dtype_nbytes(d) == ophip.dtype_nbytes(d)
+    assert L.ophip_dtype_nbytes(99) == 0
+
+
+def test_no_device_means_no_backend():
+    if ophip.device_count() > 0:
+        pytest.skip("a GPU is present")
+    assert ophip.Gpu.init() is None
+    with pytest.raises(ophip.SchemeError) as e:
+        ophip.Gpu(0)
+    assert e.value.kind == "ExecutionFailed"
+
+
+def rearr_args(shape, dst_strides, src_strides, dtype=F16, src_shape=None):
+    return ophip.RearrangeArgs(TensorLayout(dtype, shape, dst_strides), None,
+                               TensorLayout(dtype, src_shape or shape, src_strides), None)
+
+
+def test_rearrange_plan_reference_known_answers():
+    """rearrange/args.rs:242-304"""
+    s = ophip.Rearrange.plan(rearr_args([4, 3, 2, 1, 2, 3, 4], [288, 96, 48, 48, 24, 8, 2],
+                                        [576, 192, 96, 48, 8, 16, 2]))
+    assert s == [8, 144, 6, 3, 1, 48, 24, 8, 96, 8, 16]
+    st = [33554432 * 2, 16777216 * 2, 524288 * 2, 128 * 2, 2]
+    assert ophip.Rearrange.plan(rearr_args([32, 2, 32, 456, 128], st, st)) == [116736, 2048, 1, 1048576, 1048576]
+    assert ophip.Rearrange.plan(rearr_args([32, 512, 128], [256, 8192, 2], [131072, 256, 2])) == \
+        [256, 16384, 32, 1, 8192, 256, 256, 131072]
+
+
+def test_rearrange_plan_matches_oracle_on_random_layouts():
+    rng = np.random.default_rng(0)
+    for _ in range(300):
+        nd = int(rng.integers(0, 6))
+        shape = [int(rng.integers(1, 6)) for _ in range(nd)]
+        es = int(rng.choice([1, 2, 4, 8]))
+        dtype = {1: dt.U8, 2: dt.F16, 4: dt.F32, 8: dt.F64}[es]
+
+        def strides():
+            perm = rng.permutation(nd)
+            st, mul = [0] * nd, es
+            for ax in perm:
+                st[ax] = mul * int(rng.choice([1, 1, 1, 2])) * int(rng.choice([1, 1, -1]))
+                mul = abs(st[ax]) * shape[ax]
+            return st
+
+        ds, ss = strides(), strides()
+        want = oracle.rearrange_scheme(shape, ds, ss, es)
+        got = ophip.Rearrange.plan(rearr_args(shape, ds, ss, dtype))
+        nd_o = (len(want) - 2) // 3
+        assert got[: 2 + nd_o] == want[: 2 + nd_o]
+        # dims equal under the sort key may come out in either order; the strides are the same multiset
+        assert sorted(zip(got[2 + nd_o: 2 + 2 * nd_o], got[2 + 2 * nd_o:])) == \
+            sorted(zip(want[2 + nd_o: 2 + 2 * nd_o], want[2 + 2 * nd_o:]))
+
+
+def test_rearrange_plan_errors():
+    cases = [
+        (rearr_args([2, 3], [0, 4], [12, 4], dt.F32), "ShapeNotSupport"),
+        (rearr_args([2, 3], [12, 4], [12, 4], dt.F32, src_shape=[2, 4]), "ShapeMismatch"),
+        (rearr_args([None, 3], [12, 4], [12, 4], dt.F32, src_shape=[None, 3]), "DynamicNotSupport"),
+        (ophip.RearrangeArgs(TensorLayout(dt.F32, [2, 3], [12, 4]), None, TensorLayout(dt.F32, [6], [4]), None),
+         "RankMismatch"),
+        (ophip.RearrangeArgs(TensorLayout(dt.F32, [6], [4]), None, TensorLayout(dt.U32, [6], [4]), None),
+         "TypeMismatch"),
+    ]
+    for args, kind in cases:
+        with pytest.raises(ophip.SchemeError) as e:
+            ophip.Rearrange.plan(args)
+        assert e.value.kind == kind
+
+
+def mm_args(c, a, b, dtype=F16):
+    mk = lambda arr: TensorLayout(dtype, arr.shape, arr.strides)
+    return ophip.MatMulArgs(mk(c), None, 1.0, mk(a), None, mk(b), None, 1.0)
+
+
+def test_mat_mul_plan_matches_oracle_layout():
+    f16 = np.float16
+    z = lambda *s: np.zeros(s, f16)
+    cases = [
+        (z(5, 7), z(5, 3), z(3, 7)),
+        (z(7, 5).T, z(5, 3), z(3, 7)),
+        (z(5, 7), z(3, 5).T, z(7, 3).T),
+        (z(7, 5).T, z(3, 5).T, z(3, 7)),
+        (z(4, 5, 7), z(4, 5, 3), z(1, 3, 7)),
+        (z(4, 5, 7), z(5, 3), z(4, 7, 3).transpose(0, 2, 1)),
+        (z(16, 12288), z(16, 4096), z(4096, 12288)),
+        (z(32, 16, 2048), z(32, 16, 128), z(32, 2048, 128).transpose(0, 2, 1)),
+    ]
+    for c, a, b in cases:
+        got = mm_args(c, a, b).layout().as_dict()
+        want = oracle.mat_mul_layout(2, (c.shape, c.strides), (a.shape, a.strides), (b.shape, b.strides)).as_dict()
+        assert got == want, (got, want)
+    assert mm_args(*cases[0]).layout().as_dict() == dict(
+        ab_swap=1, a_trans=0, b_trans=0, batch=1, m=7, n=5, k=3, c_stride=0, c_ld=7, a_stride=0, a_ld=7,
+        b_stride=0, b_ld=3)
+
+
+def test_mat_mul_plan_errors():
+    f16 = np.float16
+    z = lambda *s: np.zeros(s, f16)
+    cases = [
+        ((z(5, 7), z(5, 4), z(3, 7)), "ShapeMismatch"),
+        ((z(10, 14)[::2, ::2], z(5, 3), z(3, 7)), "StridesNotSupport"),
+        ((z(5, 7), z(10, 6)[::2, ::2], z(3, 7)), "StridesNotSupport"),
+        ((z(7), z(5, 3), z(3, 7)), "RankNotSupport"),
+        ((z(1, 1, 5, 7), z(5, 3), z(3, 7)), "ShapeNotSupport"),
+        ((z(2, 5, 7), z(3, 5, 3), z(3, 7)), "ShapeMismatch"),
+    ]
+    for (c, a, b), kind in cases:
+        with pytest.raises(ophip.SchemeError) as e:
+            mm_args(c, a, b).layout()
+        assert e.value.kind == kind, kind
+    args = mm_args(z(5, 7), z(5, 3), z(3, 7))
+    args.a_layout = TensorLayout(F16, [5, None], [6, 2])
+    with pytest.raises(ophip.SchemeError) as e:
+        args.layout()
+    assert e.value.kind == "DynamicNotSupport"
+    args = mm_args(z(5, 7), z(5, 3), z(3, 7))
+    args.b_layout = TensorLayout(dt.F32, [3, 7], [28, 4])
+    with pytest.raises(ophip.SchemeError) as e:
+        args.layout()
+    assert e.value.kind == "TypeMismatch"
+
+
+def test_sample_args_constructor_rules():
+    """random_sample/args.rs:66-84"""
+    with pytest.raises(ophip.SampleArgsError, match="NegativeTemperature"):
+        ophip.SampleArgs(-0.1, 0.9, 50)
+    with pytest.raises(ophip.SampleArgsError, match="NonPositiveTop"):
+        ophip.SampleArgs(0.8, 0.9, 0)
+    with pytest.raises(ophip.SampleArgsError, match="NonPositiveTop"):
+        ophip.SampleArgs(0.8, 0.0, 50)
+    s = ophip.SampleArgs(0.8, 1.7, 50)
+    assert s.struct.top_p == 1.0 and not s.is_argmax()
+    assert ophip.SampleArgs(0.0, 0.9, 50).is_argmax() and ophip.SampleArgs(0.8, 0.9, 1).is_argmax()
+    am = ophip.SampleArgs.argmax()
+    assert (am.struct.temperature, am.struct.top_p, am.struct.top_k) == (0.0, 1.0, ophip.DYN_USIZE)
+
+
+def test_offset_calculator_best_fit_and_coalescing():
+    """common/calculator.rs:25-79"""
+    c = ophip.OffsetCalculator(256)
+    assert c.take(0) == (ophip.DYN_USIZE, ophip.DYN_USIZE)  # zero size: sentinel
+    assert c.take(1) is None
+    c.put(0x10000, 0x10000 + 4096)
+    c.put(0x40000, 0x40000 + 1024)
+    a = c.take(1000)  # best fit: the 1 KiB area, not the 4 KiB one
+    assert a == (0x40000, 0x40000 + 1000)
+    b = c.take(300)  # rounded to 512, carved from the 4 KiB area
+    assert b == (0x10000, 0x10000 + 300)
+    d = c.take(3584)
+    assert d == (0x10000 + 512, 0x10000 + 512 + 3584)
+    assert c.take(1) is None
+    c.put(*b)
+    c.put(*d)  # coalesces with the neighbour to its left
+    assert c.take(4096) == (0x10000, 0x10000 + 4096)
+    c.put(*a)
+    assert c.take(1024) == (0x40000, 0x40000 + 1024)
