@@ -4,6 +4,8 @@
 // to f16 first and C is read only when the f32 beta is non-zero.
 #include <algorithm>
 #include <cstdlib>
+#include <mutex>
+#include <unordered_map>
 
 #include "../kernels/params.h"
 #include "handle.hpp"
@@ -170,10 +172,12 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
             g.kind = GemmPlan::Skinny;
             g.mt = p.M <= 16 ? 1 : p.M <= 32 ? 2 : 4;
             g.qmode = p.q_sj == 1 ? 0 : 1;
-            // split K until there are a few workgroups per CU, keeping >= 8 K-steps per workgroup
+            // The kernel is latency-bound per CU, so a CU that holds two workgroups takes
+            // twice as long as one that holds one: split K only as far as one workgroup
+            // per CU (rounding down), keeping at least 8 K-steps per workgroup.
             const size_t ntiles = (p.N + 127) / 128, slabs = (p.K + 31) / 32;
             const size_t base = ntiles * p.batch;
-            size_t split = std::max<size_t>(1, (4 * (size_t)cus + base / 2) / base);
+            size_t split = std::max<size_t>(1, (size_t)cus / base);
             split = std::min(split, std::max<size_t>(1, slabs / 8));
             if (const char *e = std::getenv("OPHIP_GEMM_SPLITK")) split = std::max(1, std::atoi(e));
             size_t sps = (slabs + split - 1) / split;  // K-steps per split
@@ -191,10 +195,29 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
 
 }  // namespace
 
+// u32 split-K arrival counters per (batch, column tile) of one launch
+constexpr size_t SPLITK_COUNTERS = 1 << 16;
+
 struct ophip_mat_mul {
     ophip_device *dev;
     hipFunction_t skinny[3][2];  // [mt index 1,2,4][qmode]
     hipFunction_t reduce, generic_f16, generic_f32;
+    // Arrival counters live in a buffer owned by the operator, one per stream:
+    // launches on one stream run in order and every kernel leaves its counters at
+    // zero, so the buffer is zeroed once, when a stream is first seen.
+    mutable std::mutex mu;
+    mutable std::unordered_map<hipStream_t, void *> counters;
+
+    void *counters_for(hipStream_t stream) const {
+        std::lock_guard<std::mutex> lock(mu);
+        auto it = counters.find(stream);
+        if (it != counters.end()) return it->second;
+        void *buf = nullptr;
+        check_hip(hipMalloc(&buf, SPLITK_COUNTERS * sizeof(uint32_t)), "hipMalloc");
+        check_hip(hipMemsetAsync(buf, 0, SPLITK_COUNTERS * sizeof(uint32_t), stream), "hipMemsetAsync");
+        counters[stream] = buf;
+        return buf;
+    }
     explicit ophip_mat_mul(ophip_device *d) : dev(d) {
         ophip_device_retain(d);
         static const int mts[3] = {1, 2, 4};
@@ -206,7 +229,10 @@ struct ophip_mat_mul {
         generic_f16 = d->kernel("gemm", "gemm_generic_f16");
         generic_f32 = d->kernel("gemm", "gemm_generic_f32");
     }
-    ~ophip_mat_mul() { ophip_device_release(dev); }
+    ~ophip_mat_mul() {
+        for (auto &c : counters) (void)hipFree(c.second);
+        ophip_device_release(dev);
+    }
 };
 
 extern "C" {
@@ -257,9 +283,11 @@ int ophip_mat_mul_launch(const ophip_mat_mul *op, const ophip_mat_mul_args *args
         if (g.kind == GemmPlan::Skinny) {
             Workspace ws(qa, workspace, workspace_len, g.workspace);
             g.p.partial = ws.ptr();
+            const size_t tiles = (size_t)((p.N + 127) / 128) * p.batch;
+            g.p.counters = (p.split_k > 1 && tiles <= SPLITK_COUNTERS) ? op->counters_for(stream) : nullptr;
             const int mi = g.mt == 1 ? 0 : g.mt == 2 ? 1 : 2;
             launch(op->skinny[mi][g.qmode], Dim3{(p.N + 127) / 128, p.split_k, p.batch}, Dim3{256}, 0, stream, g.p);
-            if (p.split_k > 1) {
+            if (p.split_k > 1 && !g.p.counters) {
                 const size_t total = (size_t)p.batch * p.M * (p.N / 8);
                 launch(op->reduce, Dim3{(unsigned)((total + 255) / 256)}, Dim3{256}, 0, stream, g.p);
             }

@@ -10,6 +10,8 @@
 //  gemm_generic_* : any strides / alignment, LDS-tiled FMA; the safety net.
 //  gemm_splitk_reduce : sums the f32 partials of a split-K skinny launch in a
 //                   fixed order and applies alpha / beta.
+#include <type_traits>
+
 #include "device_util.h"
 
 // ----------------------------------------------------------- skinny (MFMA) --
@@ -31,18 +33,35 @@
 
 constexpr int SK_WAVES = 4;
 
+// Loads the lane's 8 x 16 bytes of one K-step.  `colc` is the lane's first column
+// clamped into the matrix (lanes past N load valid memory and their results are
+// dropped at the store), so the steady-state loop carries no branches.
 template <int QMODE>
-__device__ __forceinline__ void skinny_load_q(const GemmParams &p, const f16 *qb, uint32_t kb,
-                                              uint32_t kend, uint32_t col0, uint32_t g, u32x4 (&w)[8]) {
+__device__ __forceinline__ void skinny_load_q(const GemmParams &p, const f16 *qb, uint32_t kb, uint32_t colc,
+                                              uint32_t g, u32x4 (&w)[8]) {
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+        if constexpr (QMODE == 0) {
+            w[r] = ld128(qb + (int64_t)(kb + 8 * g + r) * p.q_sl + colc);
+        } else {
+            const uint32_t col = min(colc + r, p.N - 1);
+            w[r] = ld128(qb + (int64_t)col * p.q_sj + (kb + 8 * g));
+        }
+    }
+}
+// Same, for a final K-step that reaches past kend: rows beyond it read as zero.
+template <int QMODE>
+__device__ __forceinline__ void skinny_load_q_tail(const GemmParams &p, const f16 *qb, uint32_t kb, uint32_t kend,
+                                                   uint32_t colc, uint32_t g, u32x4 (&w)[8]) {
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
         w[r] = u32x4{0, 0, 0, 0};
         if constexpr (QMODE == 0) {
             const uint32_t k = kb + 8 * g + r;
-            if (k < kend && col0 < p.N) w[r] = ld128(qb + (int64_t)k * p.q_sl + col0);
+            if (k < kend) w[r] = ld128(qb + (int64_t)k * p.q_sl + colc);
         } else {
-            const uint32_t k = kb + 8 * g, col = col0 + r;
-            if (k < kend && col < p.N) w[r] = ld128(qb + (int64_t)col * p.q_sj + k);
+            const uint32_t k = kb + 8 * g, col = min(colc + r, p.N - 1);
+            if (k < kend) w[r] = ld128(qb + (int64_t)col * p.q_sj + k);
         }
     }
 }
@@ -55,6 +74,49 @@ __device__ __forceinline__ void transpose8x8(const u32x4 (&w)[8], u32x4 (&b)[8])
         for (int d = 0; d < 4; ++d) {
             const uint32_t lo = w[2 * d][t / 2], hi = w[2 * d + 1][t / 2];
             b[t][d] = (t & 1) ? ((lo >> 16) | (hi & 0xffff0000u)) : ((lo & 0xffffu) | (hi << 16));
+        }
+    }
+}
+
+// Split-K partials cross workgroups that may sit on different XCDs (each with its
+// own L2), inside one kernel.  They are moved with device-scope relaxed atomics
+// (64-bit, write-through / L2-bypassing accesses) instead of plain accesses plus
+// device-scope fences: a device-scope fence writes back and invalidates the whole
+// L2, which is ruinous while the same L2 is streaming weights.
+__device__ __forceinline__ void partial_store(float *dst, float a, float b) {
+    const unsigned long long v = (unsigned long long)__float_as_uint(a) | ((unsigned long long)__float_as_uint(b) << 32);
+    __hip_atomic_store(reinterpret_cast<unsigned long long *>(dst), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void partial_load(const float *src, float &a, float &b) {
+    const unsigned long long v = __hip_atomic_load(reinterpret_cast<const unsigned long long *>(src), __ATOMIC_RELAXED,
+                                                   __HIP_MEMORY_SCOPE_AGENT);
+    a = __uint_as_float((uint32_t)v);
+    b = __uint_as_float((uint32_t)(v >> 32));
+}
+
+// D[i, col0 .. col0+7] = alpha * sum + beta * D, rounded once to f16
+__device__ __forceinline__ void skinny_store(const GemmParams &p, uint32_t bat, uint32_t i, uint32_t col0,
+                                             const float (&sum)[8]) {
+    f16 *dst = reinterpret_cast<f16 *>(p.d) + (int64_t)bat * p.d_sb + (int64_t)i * p.d_si;
+    if (p.d_sj == 1) {
+        Pack8 o;
+        if (p.read_dst) {
+            Pack8 c;
+            c.u = ld128(dst + col0);
+#pragma unroll
+            for (int t = 0; t < 8; ++t) o.e[t] = f2h(p.beta * h2f(c.e[t]) + p.alpha * sum[t]);
+        } else {
+#pragma unroll
+            for (int t = 0; t < 8; ++t) o.e[t] = f2h(p.alpha * sum[t]);
+        }
+        st128(dst + col0, o.u);
+    } else {
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            f16 *e = dst + (int64_t)(col0 + t) * p.d_sj;
+            float r = p.alpha * sum[t];
+            if (p.read_dst) r = p.beta * h2f(*e) + r;
+            *e = f2h(r);
         }
     }
 }
@@ -80,40 +142,88 @@ __device__ __forceinline__ void gemm_skinny(const GemmParams &p) {
 #pragma unroll
         for (int t = 0; t < 8; ++t) acc[mt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    u32x4 wcur[8], wnext[8];
-    uint32_t kb = kbeg + 32 * wave;
-    if (kb < kend) skinny_load_q<QMODE>(p, qb, kb, kend, col0, g, wcur);
-    for (; kb < kend; kb += 32 * SK_WAVES) {
-        const uint32_t kn = kb + 32 * SK_WAVES;
-        if (kn < kend) skinny_load_q<QMODE>(p, qb, kn, kend, col0, g, wnext);
-
-        Pack8 a[MT];
+    // rows of P this lane feeds (clamped: rows past M only produce output rows that are never stored)
+    const f16 *prow[MT];
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            const uint32_t i = mt * 16 + j16, k = kb + 8 * g;
-            a[mt].u = u32x4{0, 0, 0, 0};
-            if (i < p.M && k < kend) a[mt].u = ld128(pb + (int64_t)i * p.p_si + k);
-        }
+    for (int mt = 0; mt < MT; ++mt) prow[mt] = pb + (int64_t)min(mt * 16 + j16, p.M - 1) * p.p_si + 8 * g;
+    const uint32_t colc = min(col0, p.N - 8);
+
+    auto step = [&](const u32x4(&w)[8], const u32x4(&a)[MT]) {
         u32x4 b[8];
         if constexpr (QMODE == 0) {
-            transpose8x8(wcur, b);
+            transpose8x8(w, b);
         } else {
 #pragma unroll
-            for (int t = 0; t < 8; ++t) b[t] = wcur[t];
+            for (int t = 0; t < 8; ++t) b[t] = w[t];
         }
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
             Pack8 bt;
             bt.u = b[t];
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
-                acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[mt].h, bt.h, acc[mt][t], 0, 0, 0);
+            for (int mt = 0; mt < MT; ++mt) {
+                Pack8 at;
+                at.u = a[mt];
+                acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(at.h, bt.h, acc[mt][t], 0, 0, 0);
+            }
         }
+    };
+
+    // Full K-steps run through a ring of three register buffers: while one step is
+    // being multiplied, the loads of the next two are in flight (16 KB per wave).
+    const uint32_t kfull = kbeg + (kend - kbeg) / 32 * 32;  // end of the full steps
+    constexpr uint32_t STRIDE = 32 * SK_WAVES;
+    const uint32_t kb0 = kbeg + 32 * wave;
+    const uint32_t cnt = kfull > kb0 ? (kfull - kb0 + STRIDE - 1) / STRIDE : 0;  // full steps of this wave
+    u32x4 wbuf[3][8], abuf[3][MT];
+    auto issue = [&](auto U, uint32_t idx) {
+        constexpr int u = decltype(U)::value;
+        const uint32_t kb = kb0 + idx * STRIDE;
 #pragma unroll
-        for (int r = 0; r < 8; ++r) wcur[r] = wnext[r];
+        for (int mt = 0; mt < MT; ++mt) abuf[u][mt] = ld128(prow[mt] + kb);
+        skinny_load_q<QMODE>(p, qb, kb, colc, g, wbuf[u]);
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    uint32_t issued = 0, done = 0;
+    if (cnt > 0) { issue(I0{}, 0); issued = 1; }
+    if (cnt > 1) { issue(I1{}, 1); issued = 2; }
+    while (issued + 3 <= cnt) {
+        issue(I2{}, issued);
+        step(wbuf[0], abuf[0]);
+        issue(I0{}, issued + 1);
+        step(wbuf[1], abuf[1]);
+        issue(I1{}, issued + 2);
+        step(wbuf[2], abuf[2]);
+        issued += 3;
+        done += 3;
+    }
+    const uint32_t rem = cnt - issued;  // 0, 1 or 2 steps still to load
+    if (done < cnt) {
+        if (rem >= 1) issue(I2{}, issued);
+        step(wbuf[0], abuf[0]);
+    }
+    if (done + 1 < cnt) {
+        if (rem >= 2) issue(I0{}, issued + 1);
+        step(wbuf[1], abuf[1]);
+    }
+    if (rem >= 1) step(wbuf[2], abuf[2]);
+    if (rem >= 2) step(wbuf[0], abuf[0]);
+
+    if (kfull < kend && kb0 + cnt * STRIDE == kfull) {  // the ragged last step belongs to exactly one wave
+        const uint32_t kb = kfull;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            abuf[0][mt] = u32x4{0, 0, 0, 0};
+            if (kb + 8 * g < kend) abuf[0][mt] = ld128(prow[mt] + kb);
+        }
+        skinny_load_q_tail<QMODE>(p, qb, kb, kend, colc, g, wbuf[0]);
+        step(wbuf[0], abuf[0]);
     }
 
     // combine the 4 waves, then row = mt*16 + 4g + wave, columns col0 .. col0+7
+    __shared__ uint32_t s_last;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         __syncthreads();
@@ -135,32 +245,58 @@ __device__ __forceinline__ void gemm_skinny(const GemmParams &p) {
             if (p.split_k > 1) {
                 float *dst = reinterpret_cast<float *>(p.partial) +
                              (((size_t)split * p.batch + bat) * p.M + i) * p.N + col0;
-                *reinterpret_cast<f32x4 *>(dst) = f32x4{sum[0], sum[1], sum[2], sum[3]};
-                *reinterpret_cast<f32x4 *>(dst + 4) = f32x4{sum[4], sum[5], sum[6], sum[7]};
-            } else {
-                f16 *dst = reinterpret_cast<f16 *>(p.d) + (int64_t)bat * p.d_sb + (int64_t)i * p.d_si;
-                if (p.d_sj == 1) {
-                    Pack8 o;
-                    if (p.read_dst) {
-                        Pack8 c;
-                        c.u = ld128(dst + col0);
+                if (p.counters) {
 #pragma unroll
-                        for (int t = 0; t < 8; ++t) o.e[t] = f2h(p.beta * h2f(c.e[t]) + p.alpha * sum[t]);
-                    } else {
-#pragma unroll
-                        for (int t = 0; t < 8; ++t) o.e[t] = f2h(p.alpha * sum[t]);
-                    }
-                    st128(dst + col0, o.u);
+                    for (int t = 0; t < 8; t += 2) partial_store(dst + t, sum[t], sum[t + 1]);
                 } else {
+                    *reinterpret_cast<f32x4 *>(dst) = f32x4{sum[0], sum[1], sum[2], sum[3]};
+                    *reinterpret_cast<f32x4 *>(dst + 4) = f32x4{sum[4], sum[5], sum[6], sum[7]};
+                }
+            } else {
+                skinny_store(p, bat, i, col0, sum);
+            }
+        }
+    }
+    if (p.split_k > 1 && p.counters) {
+        // Split-K without a second kernel: every workgroup publishes its partial tile,
+        // then bumps the tile's counter; the workgroup that arrives last sums all
+        // partials in ascending split order (so the result does not depend on
+        // arrival order) and resets the counter for the next launch.
+        // The partials were written with device-scope (write-through) stores; once
+        // every thread has seen its stores acknowledged the count may be published.
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __syncthreads();
+        uint32_t *counter = reinterpret_cast<uint32_t *>(p.counters) + (size_t)bat * gridDim.x + blockIdx.x;
+        if (threadIdx.x == 0) s_last = atomicAdd(counter, 1u) == p.split_k - 1 ? 1u : 0u;
+        __syncthreads();
+        if (s_last) {
 #pragma unroll
-                    for (int t = 0; t < 8; ++t) {
-                        f16 *e = dst + (int64_t)(col0 + t) * p.d_sj;
-                        float r = p.alpha * sum[t];
-                        if (p.read_dst) r = p.beta * h2f(*e) + r;
-                        *e = f2h(r);
+            for (int mt = 0; mt < MT; ++mt) {
+                const uint32_t i = mt * 16 + 4 * g + wave;
+                if (i < p.M && col0 < p.N) {
+                    float sum[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+                    const size_t sstride = (size_t)p.batch * p.M * p.N;  // floats between splits
+                    const float *src0 = reinterpret_cast<const float *>(p.partial) + ((size_t)bat * p.M + i) * p.N + col0;
+                    for (uint32_t s0 = 0; s0 < p.split_k; s0 += 4) {  // four splits' loads in flight, summed in order
+                        float v[4][8];
+#pragma unroll
+                        for (int u = 0; u < 4; ++u)
+#pragma unroll
+                            for (int t = 0; t < 8; t += 2) {
+                                v[u][t] = v[u][t + 1] = 0.f;
+                                if (s0 + u < p.split_k) partial_load(src0 + (s0 + u) * sstride + t, v[u][t], v[u][t + 1]);
+                            }
+#pragma unroll
+                        for (int u = 0; u < 4; ++u)
+                            if (s0 + u < p.split_k) {
+#pragma unroll
+                                for (int t = 0; t < 8; ++t) sum[t] += v[u][t];
+                            }
                     }
+                    skinny_store(p, bat, i, col0, sum);
                 }
             }
+            if (threadIdx.x == 0) *counter = 0;
         }
     }
 }
@@ -198,28 +334,7 @@ extern "C" __global__ void __launch_bounds__(256) gemm_splitk_reduce(GemmParams 
             sum[4 + t] += hi[t];
         }
     }
-    f16 *dst = reinterpret_cast<f16 *>(p.d) + (int64_t)bat * p.d_sb + (int64_t)i * p.d_si;
-    if (p.d_sj == 1) {
-        Pack8 o;
-        if (p.read_dst) {
-            Pack8 c;
-            c.u = ld128(dst + col0);
-#pragma unroll
-            for (int t = 0; t < 8; ++t) o.e[t] = f2h(p.beta * h2f(c.e[t]) + p.alpha * sum[t]);
-        } else {
-#pragma unroll
-            for (int t = 0; t < 8; ++t) o.e[t] = f2h(p.alpha * sum[t]);
-        }
-        st128(dst + col0, o.u);
-    } else {
-#pragma unroll
-        for (int t = 0; t < 8; ++t) {
-            f16 *e = dst + (int64_t)(col0 + t) * p.d_sj;
-            float r = p.alpha * sum[t];
-            if (p.read_dst) r = p.beta * h2f(*e) + r;
-            *e = f2h(r);
-        }
-    }
+    skinny_store(p, bat, i, col0, sum);
 }
 
 // ------------------------------------------------------------ generic (FMA) --

@@ -77,7 +77,8 @@ struct GemmParams {
     void *d;
     const void *p;
     const void *q;
-    void *partial;  // f32 [split_k][batch][M][N] when split_k > 1
+    void *partial;   // f32 [split_k][batch][M][N] when split_k > 1
+    void *counters;  // u32 per (batch, column tile), zero between launches; null = separate reduce kernel
     int64_t d_si, d_sj, d_sb;
     int64_t p_si, p_sl, p_sb;
     int64_t q_sl, q_sj, q_sb;
