@@ -93,8 +93,9 @@ ophip_mat_mul_layout mat_mul_layout(const ophip_mat_mul_args &args) {
 // The canonical problem handed to the kernels plus the kernel choice.
 struct GemmPlan {
     GemmParams p{};
-    enum Kind { Generic, Skinny } kind = Generic;
+    enum Kind { Generic, Skinny, Tile } kind = Generic;
     int mt = 1, qmode = 0;
+    int tile = 256, pk = 1, qk = 1;  // Tile: block size and whether P / Q are K-contiguous
     size_t workspace = 0;
 };
 
@@ -188,6 +189,37 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
             return g;
         }
     }
+    // Compute-bound shapes: the LDS-tiled MFMA kernel.  Of the two orientations take
+    // the one whose epilogue can store several adjacent outputs per lane.
+    auto tile_ok = [&](uint32_t b) {
+        if (!f16 || p.K == 0 || p.K % 32 != 0 || p.M % b != 0 || p.N % b != 0) return false;
+        if (!aligned16(p.p) || !aligned16(p.q) || !aligned16(p.d)) return false;
+        if (!mult8(p.p_sb) || !mult8(p.q_sb) || !mult8(p.d_sb)) return false;
+        if (!(p.p_sl == 1 ? mult8(p.p_si) : mult8(p.p_sl))) return false;
+        if (!(p.q_sl == 1 ? mult8(p.q_sj) : mult8(p.q_sl))) return false;
+        if (!(p.d_sj == 1 ? mult8(p.d_si) : mult8(p.d_sj))) return false;
+        return true;
+    };
+    for (uint32_t b : {256u, 128u}) {
+        int best = -1;
+        for (int attempt = 0; attempt < 2; ++attempt) {
+            orient(attempt == 1);
+            if (!tile_ok(b)) continue;
+            if (b == 256 && (size_t)(p.M / b) * (p.N / b) * p.batch < cus / 2 && p.M % 128 == 0 && p.N % 128 == 0)
+                continue;  // too few 256-tiles to fill the machine: let the 128 pass take it
+            const bool wide = (p.q_sl != 1 && p.d_sj == 1) || (p.p_sl == 1 && p.d_si == 1);
+            if (best < 0 || wide) best = attempt;
+            if (wide) break;
+        }
+        if (best >= 0) {
+            orient(best == 1);
+            g.kind = GemmPlan::Tile;
+            g.tile = (int)b;
+            g.pk = p.p_sl == 1;
+            g.qk = p.q_sl == 1;
+            return g;
+        }
+    }
     orient(false);
     g.kind = GemmPlan::Generic;
     return g;
@@ -202,6 +234,7 @@ struct ophip_mat_mul {
     ophip_device *dev;
     hipFunction_t skinny[3][2];  // [mt index 1,2,4][qmode]
     hipFunction_t reduce, generic_f16, generic_f32;
+    hipFunction_t tile[2][2][2];  // [256 / 128][P K-contiguous][Q K-contiguous]
     // Arrival counters live in a buffer owned by the operator, one per stream:
     // launches on one stream run in order and every kernel leaves its counters at
     // zero, so the buffer is zeroed once, when a stream is first seen.
@@ -225,6 +258,13 @@ struct ophip_mat_mul {
             for (int q = 0; q < 2; ++q)
                 skinny[i][q] =
                     d->kernel("gemm", ("gemm_skinny_m" + std::to_string(mts[i]) + "_q" + std::to_string(q)).c_str());
+        for (int b = 0; b < 2; ++b)
+            for (int pk = 0; pk < 2; ++pk)
+                for (int qk = 0; qk < 2; ++qk) {
+                    const std::string sz = b == 0 ? "256x256" : "128x128";
+                    tile[b][pk][qk] = d->kernel(
+                        "gemm_tile", ("gemm_tile_" + sz + "_p" + std::to_string(pk) + "_q" + std::to_string(qk)).c_str());
+                }
         reduce = d->kernel("gemm", "gemm_splitk_reduce");
         generic_f16 = d->kernel("gemm", "gemm_generic_f16");
         generic_f32 = d->kernel("gemm", "gemm_generic_f32");
@@ -291,6 +331,11 @@ int ophip_mat_mul_launch(const ophip_mat_mul *op, const ophip_mat_mul_args *args
                 const size_t total = (size_t)p.batch * p.M * (p.N / 8);
                 launch(op->reduce, Dim3{(unsigned)((total + 255) / 256)}, Dim3{256}, 0, stream, g.p);
             }
+            return;
+        }
+        if (g.kind == GemmPlan::Tile) {
+            const unsigned tiles = (p.M / g.tile) * (p.N / g.tile);
+            launch(op->tile[g.tile == 256 ? 0 : 1][g.pk][g.qk], Dim3{tiles, 1, p.batch}, Dim3{256}, 0, stream, g.p);
             return;
         }
         const unsigned gx = (p.N + 63) / 64, gy = (p.M + 63) / 64;

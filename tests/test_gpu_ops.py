@@ -795,6 +795,47 @@ def test_mat_mul_all_layouts(gpu, stream, ta, tb, tc, m, n, k):
     check_mat_mul(out, cv, av, bv, 0.75, 0.5, "mat_mul layouts")
 
 
+@pytest.mark.parametrize("ta", [False, True])
+@pytest.mark.parametrize("tb", [False, True])
+@pytest.mark.parametrize("tc", [False, True])
+@pytest.mark.parametrize("m,n,k,bt", [(256, 512, 96, 2), (128, 384, 64, 1), (512, 256, 32, 1)])
+def test_mat_mul_mfma_tile_kernel_layouts(gpu, stream, ta, tb, tc, m, n, k, bt):
+    """Shapes that divide into 128 / 256 tiles run on the LDS-tiled MFMA kernel, in every operand layout."""
+    rng = np.random.default_rng(m + n + k + 4 * ta + 2 * tb + tc)
+    a = rng.standard_normal((bt, k, m) if ta else (bt, m, k)).astype(f32).astype(f16)
+    b = rng.standard_normal((bt, n, k) if tb else (bt, k, n)).astype(f32).astype(f16)
+    c = rng.standard_normal((bt, n, m) if tc else (bt, m, n)).astype(f32).astype(f16)
+    av = a.transpose(0, 2, 1) if ta else a
+    bv = b.transpose(0, 2, 1) if tb else b
+    cv = c.transpose(0, 2, 1) if tc else c
+    say("mat_mul tile ta=%s tb=%s tc=%s %dx%dx%d" % (ta, tb, tc, m, n, k))
+    out = run_mat_mul(gpu, stream, cv, av, bv, 0.75, 0.5)
+    check_mat_mul(out, cv, av, bv, 0.75, 0.5, "mat_mul tile layouts")
+    cn = np.full(c.shape, np.nan, f16)
+    cnv = cn.transpose(0, 2, 1) if tc else cn
+    out0 = run_mat_mul(gpu, stream, cnv, av, bv, 1.0, 0.0)
+    check_mat_mul(out0, np.zeros(cv.shape, f16), av, bv, 1.0, 0.0, "mat_mul tile beta 0")
+
+
+def test_mat_mul_compute_bound_shape(gpu, stream):
+    rng = np.random.default_rng(12)
+    n = 2048
+    a = normal_f16(rng, (n, n), std=1.0)
+    b = normal_f16(rng, (n, n), std=0.05)
+    c = np.zeros((n, n), f16)
+    say("mat_mul 2048^3")
+    out = run_mat_mul(gpu, stream, c, a, b, 1.0, 0.0)
+    ref = (a.astype(np.float32) @ b.astype(np.float32)).astype(np.float64)
+    err = np.abs(out.astype(np.float64) - ref)
+    assert (err <= 2e-3 + 1e-2 * np.abs(ref)).all(), err.max()
+    oracle.set_threads(8)
+    try:
+        sub = oracle.mat_mul(np.zeros((64, n), f16), 0.0, a[:64], b, 1.0)  # oracle on a slice of rows
+    finally:
+        oracle.set_threads(1)
+    assert_close_f16(out[:64], sub, "2048^3 rows 0..63", abs_tol=2e-3 + 4e-3 * float(np.abs(sub).max()))
+
+
 def test_mat_mul_beta_zero_never_reads_c_and_scalars_round_to_f16(gpu, stream):
     a = np.ones((16, 2048), f16)
     a[:, 2047] = 0  # 2047 ones per row
