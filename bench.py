@@ -237,6 +237,9 @@ def standalone_ops(ophip, gpu, stream, rng, reps):
                 rs.launch(a, None, stream)
         us = time_launches(gpu, stream, run16, max(reps // 4, 5))
         add("random_sample " + mode, "16 x [32000]", 16 * (32000 * 2 + 8), us, note="16 launches")
+        b = arg_rows[0]
+        us = time_launches(gpu, stream, lambda: rs.launch_batch(b, 16, 64000, None, None, stream), reps)
+        add("random_sample " + mode, "16 x [32000]", 16 * (32000 * 2 + 8), us, note="1 batched launch (extension)")
     # compute-bound mat_mul: 4096^3 and 8192^3
     mm = o.MatMul(gpu)
     for n in (4096, 8192):

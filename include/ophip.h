@@ -334,6 +334,18 @@ OPHIP_API int ophip_random_sample_launch(const ophip_random_sample *op,
                                          size_t workspace_len,
                                          const ophip_queue_alloc *queue_alloc);
 OPHIP_API void ophip_random_sample_destroy(ophip_random_sample *op);
+/* Batched launch: no counterpart in the reference, whose operator samples one
+ * row per launch (random_sample/args.rs:9-18).  `rows` independent logit rows,
+ * row r starting `row_stride` bytes after row r-1, are sampled by one launch
+ * with the shared config; results go to `rows` consecutive ophip_kv_pair at
+ * kv_pair_base.  `seeds` is either NULL (args->seed is used for every row) or a
+ * DEVICE array of `rows` draws.  Each row's result is what ophip_random_sample_launch
+ * returns for that row.  The workspace need is rows times the single-row need. */
+OPHIP_API int ophip_random_sample_launch_batch(const ophip_random_sample *op,
+                                               const ophip_random_sample_args *args, size_t rows,
+                                               ptrdiff_t row_stride, const float *seeds,
+                                               void *workspace, size_t workspace_len,
+                                               const ophip_queue_alloc *queue_alloc);
 /* RandomSample::build_indices (random_sample/cuda/mod.rs:29-38): uploads 0..n as
  * u32.  *out is owned by the caller. */
 OPHIP_API int ophip_random_sample_build_indices(size_t n, const ophip_queue_alloc *queue_alloc,

@@ -72,6 +72,7 @@ struct RmsKeyHash {
 };
 struct RmsScheme {  // kernels for one (dt_a, dt_w, d): a vector variant per group width plus the scalar one
     hipFunction_t g64, g256, g1024, scalar;
+    hipFunction_t rows;  // f16 activations only: one wave per row over many rows
 };
 
 struct ophip_rms_norm : OpBase {
@@ -86,6 +87,7 @@ struct ophip_rms_norm : OpBase {
             s.g256 = dev->kernel("rms_norm", (base + "_g256").c_str());
             s.g1024 = dev->kernel("rms_norm", (base + "_g1024").c_str());
             s.scalar = dev->kernel("rms_norm", (base + "_scalar").c_str());
+            s.rows = key.dt_a == OPHIP_DT_F16 ? dev->kernel("rms_norm", (base + "_rows").c_str()) : nullptr;
             return s;
         });
     }
@@ -148,6 +150,14 @@ extern "C" int ophip_rms_norm_launch(const ophip_rms_norm *op, const ophip_rms_n
         const size_t nvec = d / vec_elems;
         unsigned G = nvec <= 64 * 8 ? 64 : nvec <= 256 * 8 ? 256 : 1024;
         while (G < 1024 && n * (G / 64) < 2048 && nvec >= 4 * (size_t)G) G *= 4;
+        const unsigned cus = (unsigned)op->dev->props.multiProcessorCount;
+        if (G == 64 && s.rows && n >= (size_t)cus * 64) {
+            // enough rows for several per wave: as many waves as stay resident (registers allow
+            // 16 per CU with f16 weights, 12 with f32), each streaming rows with w held in registers
+            const unsigned per_cu = m.dt_w == OPHIP_DT_F16 ? 4 : 3;
+            launch(s.rows, Dim3{cus * per_cu}, Dim3{256}, 0, stream_of(qa), p);
+            return;
+        }
         const unsigned block = G < 256 ? 256 : G, rpb = block / G;
         hipFunction_t fn = G == 64 ? s.g64 : G == 256 ? s.g256 : s.g1024;
         launch(fn, Dim3{ceil_div(n, rpb)}, Dim3{block}, 0, stream_of(qa), p);
@@ -521,20 +531,70 @@ extern "C" int ophip_rearrange_launch(const ophip_rearrange *op, const ophip_rea
         RearrangeParams p{};
         p.dst = args->dst_base;
         p.src = args->src_base;
-        p.ndim = (uint32_t)s.ndim();
         const size_t cpu = s.unit / B;
+
+        // Visiting order of the units.  The scheme's order walks the destination
+        // linearly, so the source is gathered in `unit`-byte runs that may sit far
+        // apart.  When another dimension is (nearly) contiguous in the source, walk
+        // small 2-D tiles instead - A = innermost destination dimension, B = the
+        // source-contiguous one - so that a workgroup's 16 KB touches runs of a few KB
+        // on both sides.  Any visiting order copies every unit exactly once.
+        std::vector<size_t> lens(s.ndim());
+        for (size_t i = 0; i < s.ndim(); ++i) lens[i] = s.idx[i] / s.idx[i + 1];
+        std::vector<size_t> o_len(lens);
+        std::vector<ptrdiff_t> o_dst(s.dst), o_src(s.src);
+        if (s.ndim() >= 2 && s.unit <= 2048) {
+            const size_t A = s.ndim() - 1;
+            size_t Bd = A;
+            for (size_t i = 0; i < A; ++i)
+                if (iabs(s.src[i]) < iabs(s.src[Bd])) Bd = i;
+            if (Bd != A && iabs(s.src[A]) > 4096 && iabs(s.src[Bd]) <= 4096) {
+                auto divisor_at_most = [](size_t len, size_t cap) {
+                    size_t best = 1;
+                    for (size_t t = 1; t <= cap && t <= len; ++t)
+                        if (len % t == 0) best = t;
+                    return best;
+                };
+                const size_t per_tile = std::max<size_t>(1, 16384 / s.unit);  // units in one workgroup's share
+                const size_t tA = divisor_at_most(lens[A], std::max<size_t>(1, std::min<size_t>(per_tile, 2048 / s.unit)));
+                const size_t tB = divisor_at_most(lens[Bd], std::max<size_t>(1, per_tile / tA));
+                if (tA * tB > 1) {
+                    o_len.clear(); o_dst.clear(); o_src.clear();
+                    auto push = [&](size_t len, ptrdiff_t d, ptrdiff_t sr) {
+                        if (len == 1) return;
+                        o_len.push_back(len); o_dst.push_back(d); o_src.push_back(sr);
+                    };
+                    for (size_t i = 0; i < s.ndim(); ++i)
+                        if (i != A && i != Bd) push(lens[i], s.dst[i], s.src[i]);
+                    // B's outer part goes outside A's: consecutive workgroups then finish one
+                    // destination region after another instead of revisiting each several times
+                    push(lens[Bd] / tB, s.dst[Bd] * (ptrdiff_t)tB, s.src[Bd] * (ptrdiff_t)tB);
+                    push(lens[A] / tA, s.dst[A] * (ptrdiff_t)tA, s.src[A] * (ptrdiff_t)tA);
+                    push(tB, s.dst[Bd], s.src[Bd]);
+                    push(tA, s.dst[A], s.src[A]);
+                    if (o_len.size() > OPHIP_REARRANGE_MAXD) {  // keep the plain order
+                        o_len = lens; o_dst = s.dst; o_src = s.src;
+                    }
+                }
+            }
+        }
+        const size_t nd = o_len.size();
+        std::vector<size_t> o_idx(nd + 1, 1);
+        for (size_t i = nd; i-- > 0;) o_idx[i] = o_len[i] * o_idx[i + 1];
+
+        p.ndim = (uint32_t)nd;
         p.total = (uint64_t)s.count() * cpu;
         bool small = p.total <= 0x7fffffffu && cpu <= 0x7fffffffu;
-        for (size_t i = 0; i < s.ndim(); ++i) {
-            p.idx[i] = s.idx[i + 1];
-            p.dst_s[i] = s.dst[i];
-            p.src_s[i] = s.src[i];
-            if (s.idx[i + 1] > 0x7fffffffu) small = false;
+        for (size_t i = 0; i < nd; ++i) {
+            p.idx[i] = o_idx[i + 1];
+            p.dst_s[i] = o_dst[i];
+            p.src_s[i] = o_src[i];
+            if (o_idx[i + 1] > 0x7fffffffu) small = false;
         }
         p.chunks_per_unit = (uint32_t)cpu;
         if (small) {
             p.cpu_div = make_fastdiv((uint32_t)cpu);
-            for (size_t i = 0; i < s.ndim(); ++i) p.idx_div[i] = make_fastdiv((uint32_t)s.idx[i + 1]);
+            for (size_t i = 0; i < nd; ++i) p.idx_div[i] = make_fastdiv((uint32_t)o_idx[i + 1]);
             const unsigned per_block = 256 * 4;  // RE_ITEMS chunks per thread
             launch(op->k32[ci], Dim3{ceil_div(p.total, per_block)}, Dim3{256}, 0, stream_of(qa), p);
         } else {

@@ -89,49 +89,64 @@ int ophip_random_sample_scheme(ophip_random_sample *, const ophip_random_sample_
     });
 }
 
+static void sample_launch(const ophip_random_sample *op, const ophip_random_sample_args *args, size_t rows,
+                          ptrdiff_t row_stride, const float *seeds, void *workspace, size_t workspace_len,
+                          const ophip_queue_alloc *qa) {
+    const SampleMeta m = sample_meta(*args);
+    if (args->kv_pair.ndim != 0) throw rank_error("kv_pair", 0, args->kv_pair.ndim);
+    const size_t n = static_of(m.n);
+    const ptrdiff_t sp = static_of(args->logits.strides[0]);
+    const ptrdiff_t si = static_of(args->indices.strides[0]);
+    if (m.dt != OPHIP_DT_F16 && m.dt != OPHIP_DT_F32) throw type_not_support("logits must be f16 or f32");
+    if (sp != (ptrdiff_t)ophip_dtype_nbytes(m.dt)) throw strides_not_support("logits must be contiguous");
+    if (si != (ptrdiff_t)sizeof(uint32_t)) throw strides_not_support("indices must be contiguous");
+    if (n == 0) throw shape_not_support("empty logits");  // the reference unwraps an empty maximum
+    if (n > 0x7fffffffu) throw shape_not_support("too many logits");
+    if (rows == 0) return;
+    if (rows > 0x7fffffffu) throw shape_not_support("too many rows");
+    if (row_stride % sp != 0) throw strides_not_support("row stride must be a multiple of the element size");
+
+    const int ti = m.dt == OPHIP_DT_F16 ? 0 : 1;
+    const ophip_sample_args &cfg = args->config;
+    SampleParams p{};
+    p.kv = args->kv_pair_base;
+    p.logits = args->logits_base;
+    p.row_stride = row_stride;
+    p.n = (uint32_t)n;
+    p.seeds = seeds;
+    const Dim3 grid{(unsigned)rows};
+    op->dev->make_current();
+    if (cfg.temperature == 0.f || cfg.top_k == 1) {
+        launch(op->argmax[ti], grid, Dim3{1024}, 0, stream_of(qa), p);
+        return;
+    }
+    if (is_dyn(cfg.temperature) || is_dyn(cfg.top_p) || is_dyn(args->seed)) throw dyn_not_support("");
+    if (!(cfg.temperature > 0.f) || cfg.top_k == 0 || !(cfg.top_p > 0.f))
+        throw args_not_support("sampling needs temperature > 0, top_k >= 1, top_p > 0");
+    const size_t k_eff = cfg.top_k < n ? cfg.top_k : n;
+    p.k_eff = (uint32_t)k_eff;
+    p.temperature = cfg.temperature;
+    p.top_p = cfg.top_p;
+    p.seed = args->seed;
+    if (k_eff <= TOPK_FAST_MAX) {
+        launch(op->topk[ti], grid, Dim3{1024}, 0, stream_of(qa), p);
+        return;
+    }
+    p.npow2 = (uint32_t)next_pow2(n);
+    Workspace ws(qa, workspace, workspace_len, rows * full_sort_workspace(n));
+    p.workspace = ws.ptr();
+    launch(op->full[ti], grid, Dim3{1024}, 0, stream_of(qa), p);
+}
+
 int ophip_random_sample_launch(const ophip_random_sample *op, const ophip_random_sample_args *args, void *workspace,
                                size_t workspace_len, const ophip_queue_alloc *qa) {
-    return guard([&] {
-        const SampleMeta m = sample_meta(*args);
-        if (args->kv_pair.ndim != 0) throw rank_error("kv_pair", 0, args->kv_pair.ndim);
-        const size_t n = static_of(m.n);
-        const ptrdiff_t sp = static_of(args->logits.strides[0]);
-        const ptrdiff_t si = static_of(args->indices.strides[0]);
-        if (m.dt != OPHIP_DT_F16 && m.dt != OPHIP_DT_F32) throw type_not_support("logits must be f16 or f32");
-        if (sp != (ptrdiff_t)ophip_dtype_nbytes(m.dt)) throw strides_not_support("logits must be contiguous");
-        if (si != (ptrdiff_t)sizeof(uint32_t)) throw strides_not_support("indices must be contiguous");
-        if (n == 0) throw shape_not_support("empty logits");  // the reference unwraps an empty maximum
-        if (n > 0x7fffffffu) throw shape_not_support("too many logits");
+    return guard([&] { sample_launch(op, args, 1, 0, nullptr, workspace, workspace_len, qa); });
+}
 
-        const int ti = m.dt == OPHIP_DT_F16 ? 0 : 1;
-        const ophip_sample_args &cfg = args->config;
-        SampleParams p{};
-        p.kv = args->kv_pair_base;
-        p.logits = args->logits_base;
-        p.row_stride = 0;
-        p.n = (uint32_t)n;
-        op->dev->make_current();
-        if (cfg.temperature == 0.f || cfg.top_k == 1) {
-            launch(op->argmax[ti], Dim3{1}, Dim3{1024}, 0, stream_of(qa), p);
-            return;
-        }
-        if (is_dyn(cfg.temperature) || is_dyn(cfg.top_p) || is_dyn(args->seed)) throw dyn_not_support("");
-        if (!(cfg.temperature > 0.f) || cfg.top_k == 0 || !(cfg.top_p > 0.f))
-            throw args_not_support("sampling needs temperature > 0, top_k >= 1, top_p > 0");
-        const size_t k_eff = cfg.top_k < n ? cfg.top_k : n;
-        p.k_eff = (uint32_t)k_eff;
-        p.temperature = cfg.temperature;
-        p.top_p = cfg.top_p;
-        p.seed = args->seed;
-        if (k_eff <= TOPK_FAST_MAX) {
-            launch(op->topk[ti], Dim3{1}, Dim3{1024}, 0, stream_of(qa), p);
-            return;
-        }
-        p.npow2 = (uint32_t)next_pow2(n);
-        Workspace ws(qa, workspace, workspace_len, full_sort_workspace(n));
-        p.workspace = ws.ptr();
-        launch(op->full[ti], Dim3{1}, Dim3{1024}, 0, stream_of(qa), p);
-    });
+int ophip_random_sample_launch_batch(const ophip_random_sample *op, const ophip_random_sample_args *args, size_t rows,
+                                     ptrdiff_t row_stride, const float *seeds, void *workspace,
+                                     size_t workspace_len, const ophip_queue_alloc *qa) {
+    return guard([&] { sample_launch(op, args, rows, row_stride, seeds, workspace, workspace_len, qa); });
 }
 
 int ophip_random_sample_build_indices(size_t n, const ophip_queue_alloc *qa, void **out) {

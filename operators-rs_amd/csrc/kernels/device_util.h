@@ -83,6 +83,12 @@ __device__ __forceinline__ float group_max(float v, float *smem) {
     return v;
 }
 
+// exp(x) through the hardware base-2 exponential (about 1 ulp plus |x| * 2^-24 from the
+// scaling by log2(e)): two instructions instead of libm's range reduction.  The
+// streaming kernels whose result is rounded to f16 use it; at 8 TB/s the accurate
+// expf alone would exceed their per-element instruction budget.
+__device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f); }
+
 __device__ __forceinline__ uint32_t fastdiv(uint32_t n, const FastDivU32 &d) {
     uint32_t t = __umulhi(d.m, n);
     return (t + ((n - t) >> d.s1)) >> d.s2;

@@ -61,7 +61,7 @@ __device__ __forceinline__ void softmax_reg(const SoftmaxParams &p) {
         for (int e = 0; e < VEC; ++e) {
             const uint32_t col = (lane + i * G) * VEC + e;
             if (col < kept) {
-                const float ex = expf(x[i][e] - mx);
+                const float ex = fast_exp(x[i][e] - mx);
                 sum += ex;
                 x[i][e] = h2f(f2h(ex));  // the reference stores f16(e) and re-reads it
             } else {
@@ -101,7 +101,7 @@ extern "C" __global__ void __launch_bounds__(1024) softmax_f16_stream(SoftmaxPar
     mx = group_max<G>(mx, smem);
     float sum = 0.f;
     for (uint32_t c = threadIdx.x; c < kept; c += G) {
-        const float ex = expf(h2f(row[c]) - mx);
+        const float ex = fast_exp(h2f(row[c]) - mx);
         sum += ex;
         row[c] = f2h(ex);
     }

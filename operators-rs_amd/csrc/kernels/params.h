@@ -63,6 +63,7 @@ struct SampleParams {
     void *kv;            // ophip_kv_pair*, one per row
     const void *logits;  // rows x n
     void *workspace;     // general path only
+    const float *seeds;  // optional per-row draws (device memory); null = `seed` for every row
     int64_t row_stride;  // bytes between rows of logits
     uint32_t n;
     uint32_t k_eff;      // min(top_k, n)

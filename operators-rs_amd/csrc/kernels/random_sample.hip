@@ -74,6 +74,75 @@ struct Logit<float> {
 
 constexpr int SB = 1024;  // workgroup size of every kernel in this file
 
+// Calls f(index, raw bits) for every element of the row, 16 bytes per load when the
+// row is 16-byte aligned (8 f16 or 4 f32 per thread and step), else element-wise.
+template <typename T, typename F>
+__device__ __forceinline__ void for_each_logit(const char *row, uint32_t n, F &&f) {
+    constexpr uint32_t PER = 16 / sizeof(T);
+    if ((reinterpret_cast<uintptr_t>(row) & 15u) == 0) {
+        const uint32_t nvec = n / PER;
+        for (uint32_t v = threadIdx.x; v < nvec; v += SB) {
+            const u32x4 raw = ld128(row + (size_t)v * 16);
+#pragma unroll
+            for (uint32_t e = 0; e < PER; ++e) {
+                uint32_t b;
+                if constexpr (sizeof(T) == 2) b = (raw[e / 2] >> (16 * (e & 1))) & 0xffffu;
+                else b = raw[e];
+                f(v * PER + e, b);
+            }
+        }
+        for (uint32_t i = nvec * PER + threadIdx.x; i < n; i += SB) f(i, Logit<T>::bits(row, i));
+    } else {
+        for (uint32_t i = threadIdx.x; i < n; i += SB) f(i, Logit<T>::bits(row, i));
+    }
+}
+
+// A row that fits (n <= 32768) is pulled into registers once, with every load in
+// flight at the same time, and all later sweeps of the workgroup run from there;
+// longer or misaligned rows are swept from memory (L2) each time.
+template <typename T>
+struct RowCache {
+    static constexpr uint32_t PER = 16 / sizeof(T);
+    static constexpr int NV = 32768 / (SB * PER);  // vectors per thread: 4 for f16, 8 for f32
+    u32x4 v[NV];
+    bool cached;
+
+    __device__ __forceinline__ void load(const char *row, uint32_t n) {
+        cached = (reinterpret_cast<uintptr_t>(row) & 15u) == 0 && n <= (uint32_t)NV * SB * PER;
+        if (!cached) return;
+        const uint32_t nvec = n / PER;
+#pragma unroll
+        for (int c = 0; c < NV; ++c) {
+            const uint32_t idx = threadIdx.x + c * SB;
+            v[c] = u32x4{0, 0, 0, 0};
+            if (idx < nvec) v[c] = ld128(row + (size_t)idx * 16);
+        }
+    }
+
+    template <typename F>
+    __device__ __forceinline__ void for_each(const char *row, uint32_t n, F &&f) const {
+        if (!cached) {
+            for_each_logit<T>(row, n, f);
+            return;
+        }
+        const uint32_t nvec = n / PER;
+#pragma unroll
+        for (int c = 0; c < NV; ++c) {
+            const uint32_t idx = threadIdx.x + c * SB;
+            if (idx < nvec) {
+#pragma unroll
+                for (uint32_t e = 0; e < PER; ++e) {
+                    uint32_t b;
+                    if constexpr (sizeof(T) == 2) b = (v[c][e / 2] >> (16 * (e & 1))) & 0xffffu;
+                    else b = v[c][e];
+                    f(idx * PER + e, b);
+                }
+            }
+        }
+        for (uint32_t i = nvec * PER + threadIdx.x; i < n; i += SB) f(i, Logit<T>::bits(row, i));
+    }
+};
+
 // ---------------------------------------------------------------- argmax ----
 
 struct Best {
@@ -121,11 +190,12 @@ __device__ __forceinline__ void argmax_impl(const SampleParams &p) {
 
     Best b{-INFINITY, -1};
     int last_nan = -1;
-    for (int i = threadIdx.x; i < n; i += SB) {
-        const float v = Logit<T>::value(Logit<T>::bits(row, i));
-        if (v != v) last_nan = i;
-        else if (!(b.v > v)) b = Best{v, i};
-    }
+    // within a thread indices ascend, so "replace unless strictly greater" keeps the last maximum
+    for_each_logit<T>(row, (uint32_t)n, [&](uint32_t i, uint32_t bits) {
+        const float v = Logit<T>::value(bits);
+        if (v != v) last_nan = (int)i;
+        else if (!(b.v > v)) b = Best{v, (int)i};
+    });
     last_nan = block_max_int(last_nan, sint);
     b = block_best(b, sbest);
     if (last_nan >= 0) {  // uniform branch
@@ -157,6 +227,8 @@ __device__ __forceinline__ uint64_t composite(uint32_t key, uint32_t idx) {
 }
 __device__ __forceinline__ uint32_t comp_key(uint64_t c) { return (uint32_t)(c >> 32); }
 __device__ __forceinline__ uint32_t comp_idx(uint64_t c) { return 0xffffffffu - (uint32_t)c; }
+
+__device__ __forceinline__ float row_seed(const SampleParams &p) { return p.seeds ? p.seeds[blockIdx.x] : p.seed; }
 
 // exp() the way a correctly rounded expf would return it
 __device__ __forceinline__ float exp_cr(float x) { return (float)exp((double)x); }
@@ -195,46 +267,83 @@ __device__ __forceinline__ void bitonic_lds(uint64_t *a, uint32_t cnt, uint32_t 
     }
 }
 
+// Finds, among 256 histogram bins scanned from the top (descending) or from the
+// bottom, the bin in which the running count reaches `want`; writes the bin and the
+// count still wanted inside it to out[0..1].  All threads call; out is valid after return.
+__device__ __forceinline__ void pick_bucket(const uint32_t *hist, uint32_t want, bool descending, uint32_t *wave_tot,
+                                            uint32_t *out) {
+    const uint32_t lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+    uint32_t bin = 0, c = 0, incl = 0;
+    if (threadIdx.x < 256) {
+        bin = descending ? 255u - threadIdx.x : threadIdx.x;
+        c = hist[bin];
+        incl = c;
+#pragma unroll
+        for (int o = 1; o < WAVE; o <<= 1) {
+            const uint32_t t = __shfl_up(incl, o, WAVE);
+            if (lane >= (uint32_t)o) incl += t;
+        }
+        if (lane == WAVE - 1) wave_tot[wave] = incl;
+    }
+    __syncthreads();
+    if (threadIdx.x < 256) {
+        for (uint32_t w = 0; w < wave; ++w) incl += wave_tot[w];
+        const uint32_t excl = incl - c;
+        if (excl < want && want <= incl) {
+            out[0] = bin;
+            out[1] = want - excl;
+        }
+    }
+    __syncthreads();
+}
+
+__device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t v, int m) {
+    const uint32_t lo = __shfl_xor((uint32_t)v, m, WAVE), hi = __shfl_xor((uint32_t)(v >> 32), m, WAVE);
+    return ((uint64_t)hi << 32) | lo;
+}
+
 template <typename T>
 __device__ __forceinline__ void sample_topk_impl(const SampleParams &p) {
     typedef Logit<T> L;
     __shared__ uint32_t hist[256];
+    __shared__ uint32_t hist_w[SB / WAVE][256];  // one histogram per wave: 16x less contention on hot bins
+    __shared__ uint32_t s_wtot[4];
     __shared__ uint32_t s_sel[2];
     __shared__ uint32_t s_cnt;
     __shared__ uint64_t cand[SB];
     __shared__ float s_cum[SB];
     __shared__ float s_red[SB / WAVE];
+    __shared__ float s_mx;
 
     const char *row = reinterpret_cast<const char *>(p.logits) + (int64_t)blockIdx.x * p.row_stride;
     const uint32_t n = p.n, k = p.k_eff;
+    RowCache<T> rc;
+    rc.load(row, n);
 
-    // 1a. k-th largest key
+    // 1a. k-th largest key, one 8-bit digit per sweep
     uint32_t prefix = 0, krem = k, eq_count = 0;
     for (int shift = L::KEY_BITS - 8; shift >= 0; shift -= 8) {
-        if (threadIdx.x < 256) hist[threadIdx.x] = 0;
+        for (uint32_t i = threadIdx.x; i < (SB / WAVE) * 256; i += SB) (&hist_w[0][0])[i] = 0;
         __syncthreads();
         const bool first = shift == L::KEY_BITS - 8;
-        for (uint32_t i = threadIdx.x; i < n; i += SB) {
-            const uint32_t key = L::key(L::bits(row, i));
-            if (first || (key >> (shift + 8)) == (prefix >> (shift + 8)))
-                atomicAdd(&hist[(key >> shift) & 255u], 1u);
+        const uint32_t hi_mask = first ? 0u : (0xffffffffu << (shift + 8));
+        uint32_t *my_hist = hist_w[threadIdx.x / WAVE];
+        rc.for_each(row, n, [&](uint32_t, uint32_t bits) {
+            const uint32_t key = L::key(bits);
+            if (((key ^ prefix) & hi_mask) == 0) atomicAdd(&my_hist[(key >> shift) & 255u], 1u);
+        });
+        __syncthreads();
+        if (threadIdx.x < 256) {
+            uint32_t c = 0;
+#pragma unroll
+            for (int w = 0; w < SB / WAVE; ++w) c += hist_w[w][threadIdx.x];
+            hist[threadIdx.x] = c;
         }
         __syncthreads();
-        if (threadIdx.x == 0) {
-            uint32_t acc = 0;
-            int b = 255;
-            for (; b > 0; --b) {
-                const uint32_t c = hist[b];
-                if (acc + c >= krem) break;
-                acc += c;
-            }
-            s_sel[0] = prefix | ((uint32_t)b << shift);
-            s_sel[1] = krem - acc;
-        }
-        __syncthreads();
-        prefix = s_sel[0];
+        pick_bucket(hist, krem, true, s_wtot, s_sel);
+        prefix |= s_sel[0] << shift;
         krem = s_sel[1];
-        eq_count = hist[(prefix >> shift) & 255u];
+        eq_count = hist[s_sel[0]];
         __syncthreads();
     }
     const uint32_t kstar = prefix;  // k-th largest key; `krem` of the `eq_count` ties are wanted
@@ -246,77 +355,122 @@ __device__ __forceinline__ void sample_topk_impl(const SampleParams &p) {
         for (int shift = 24; shift >= 0; shift -= 8) {
             if (threadIdx.x < 256) hist[threadIdx.x] = 0;
             __syncthreads();
-            for (uint32_t i = threadIdx.x; i < n; i += SB) {
-                if (L::key(L::bits(row, i)) != kstar) continue;
-                if (shift == 24 || (i >> (shift + 8)) == (ipre >> (shift + 8)))
-                    atomicAdd(&hist[(i >> shift) & 255u], 1u);
-            }
+            const uint32_t hi_mask = shift == 24 ? 0u : (0xffffffffu << (shift + 8));
+            rc.for_each(row, n, [&](uint32_t i, uint32_t bits) {
+                if (L::key(bits) == kstar && ((i ^ ipre) & hi_mask) == 0) atomicAdd(&hist[(i >> shift) & 255u], 1u);
+            });
             __syncthreads();
-            if (threadIdx.x == 0) {
-                uint32_t acc = 0;
-                int b = 0;
-                for (; b < 255; ++b) {
-                    const uint32_t c = hist[b];
-                    if (acc + c >= irem) break;
-                    acc += c;
-                }
-                s_sel[0] = ipre | ((uint32_t)b << shift);
-                s_sel[1] = irem - acc;
-            }
-            __syncthreads();
-            ipre = s_sel[0];
+            pick_bucket(hist, irem, false, s_wtot, s_sel);
+            ipre |= s_sel[0] << shift;
             irem = s_sel[1];
             __syncthreads();
         }
         istar = ipre;
     }
 
-    // 2. gather exactly k candidates, pad to a power of two, sort
+    // 2. gather exactly k candidates, pad to a power of two
     uint32_t P = 64;
     while (P < k) P <<= 1;
     if (threadIdx.x == 0) s_cnt = 0;
     for (uint32_t i = threadIdx.x; i < P; i += SB) cand[i] = 0;
     __syncthreads();
-    for (uint32_t i = threadIdx.x; i < n; i += SB) {
-        const uint32_t key = L::key(L::bits(row, i));
+    rc.for_each(row, n, [&](uint32_t i, uint32_t bits) {
+        const uint32_t key = L::key(bits);
         if (key > kstar || (key == kstar && i <= istar)) {
             const uint32_t slot = atomicAdd(&s_cnt, 1u);
             if (slot < SB) cand[slot] = composite(key, i);
         }
-    }
+    });
     __syncthreads();
-    bitonic_lds(cand, P, 2, P, P, 0);
 
+    const float t = p.temperature;
+    if (P == 64) {
+        // k <= 64: sort, prefix and search live in the registers of wave 0
+        const uint32_t lane = threadIdx.x % WAVE;
+        uint64_t x = 0;
+        if (threadIdx.x < WAVE) {
+            x = cand[lane];
+#pragma unroll
+            for (int k2 = 2; k2 <= WAVE; k2 <<= 1)
+#pragma unroll
+                for (int j = k2 >> 1; j > 0; j >>= 1) {
+                    const uint64_t y = shfl_xor_u64(x, j);
+                    const bool desc = (lane & k2) == 0, lower = (lane & j) == 0;
+                    x = (lower == desc) ? (x > y ? x : y) : (x < y ? x : y);
+                }
+            if (lane == 0) s_mx = L::value(L::unkey(comp_key(x)));
+        }
+        __syncthreads();
+        const float mx = s_mx;
+        float part = 0.f;
+        // the total only feeds the top_p bound: hardware exp2 and a reciprocal keep this sweep cheap
+        const float inv_t = 1.0f / t;
+        rc.for_each(row, n, [&](uint32_t, uint32_t bits) { part += fast_exp((L::value(bits) - mx) * inv_t); });
+        const float total = block_sum_f32(part, s_red);
+        if (threadIdx.x < WAVE) {
+            float e = 0.f;
+            if (lane > 0 && lane < k) e = exp_cr((L::value(L::unkey(comp_key(x))) - mx) / t);
+            // cum[i] = cum[i-1] + e[i], strictly in order, every lane replaying the same chain
+            float c = 1.0f, mine = 1.0f;
+#pragma unroll
+            for (int i = 1; i < WAVE; ++i) {
+                c = c + __shfl(e, i, WAVE);
+                if (lane == (uint32_t)i) mine = c;
+            }
+            const float pk = c;  // terms past k are zero, so the chain ends at cum[k-1]
+            const float plimit = row_seed(p) * fminf(pk, total * p.top_p);
+            const uint64_t hit = __ballot(lane < k && mine >= plimit);
+            const uint32_t ans = hit ? (uint32_t)__ffsll((long long)hit) - 1 : k - 1;
+            if (lane == ans) {
+                KvPair *out = reinterpret_cast<KvPair *>(p.kv) + blockIdx.x;
+                out->idx = comp_idx(x);
+                out->val = L::from_f32(mine);
+            }
+        }
+        return;
+    }
+
+    bitonic_lds(cand, P, 2, P, P, 0);
     // 3. running sums
     const float mx = L::value(L::unkey(comp_key(cand[0])));
-    const float t = p.temperature;
     float part = 0.f;
-    for (uint32_t i = threadIdx.x; i < n; i += SB)
-        part += expf((L::value(L::bits(row, i)) - mx) / t);
+    const float inv_t = 1.0f / t;
+    rc.for_each(row, n, [&](uint32_t, uint32_t bits) { part += fast_exp((L::value(bits) - mx) * inv_t); });
     const float total = block_sum_f32(part, s_red);
-    if (threadIdx.x < k)
-        s_cum[threadIdx.x] = threadIdx.x == 0
-                                 ? 1.0f
-                                 : exp_cr((L::value(L::unkey(comp_key(cand[threadIdx.x]))) - mx) / t);
+    if (threadIdx.x < P)
+        s_cum[threadIdx.x] = threadIdx.x == 0   ? 1.0f
+                             : threadIdx.x < k ? exp_cr((L::value(L::unkey(comp_key(cand[threadIdx.x]))) - mx) / t)
+                                               : 0.f;
     __syncthreads();
-    if (threadIdx.x == 0) {
-        float cum = 1.0f;
-        for (uint32_t i = 1; i < k; ++i) {
-            cum = cum + s_cum[i];
-            s_cum[i] = cum;
+    if (threadIdx.x < WAVE) {
+        // wave 0 replays the sequential sum 64 entries at a time, carrying the running value
+        const uint32_t lane = threadIdx.x;
+        float c = 0.f;
+        for (uint32_t base = 0; base < P; base += WAVE) {
+            const float e = s_cum[base + lane];
+            float mine = 0.f;
+#pragma unroll
+            for (int i = 0; i < WAVE; ++i) {
+                c = c + __shfl(e, i, WAVE);
+                if (lane == (uint32_t)i) mine = c;
+            }
+            s_cum[base + lane] = mine;
         }
-        const float pk = cum;
-        const float pp = total * p.top_p;
-        const float plimit = p.seed * fminf(pk, pp);
+        const float pk = c;  // entries past k add zero
+        const float plimit = row_seed(p) * fminf(pk, total * p.top_p);
         uint32_t ans = k - 1;
-        for (uint32_t i = 0; i < k; ++i)
-            if (s_cum[i] >= plimit) {
-                ans = i;
+        for (uint32_t base = 0; base < P; base += WAVE) {
+            const uint64_t hit = __ballot(base + lane < k && s_cum[base + lane] >= plimit);
+            if (hit) {
+                ans = base + (uint32_t)__ffsll((long long)hit) - 1;
                 break;
             }
-        KvPair *out = reinterpret_cast<KvPair *>(p.kv) + blockIdx.x;
-        out->idx = comp_idx(cand[ans]);
-        out->val = L::from_f32(s_cum[ans]);
+        }
+        if (lane == 0) {
+            KvPair *out = reinterpret_cast<KvPair *>(p.kv) + blockIdx.x;
+            out->idx = comp_idx(cand[ans]);
+            out->val = L::from_f32(s_cum[ans]);
+        }
     }
 }
 
@@ -391,7 +545,7 @@ __device__ __forceinline__ void sample_full_impl(const SampleParams &p) {
     __syncthreads();
     const float pk = cum[p.k_eff - 1];
     const float pp = cum[n - 1] * p.top_p;
-    const float plimit = p.seed * fminf(pk, pp);
+    const float plimit = row_seed(p) * fminf(pk, pp);
     uint32_t mine = 0xffffffffu;
     for (uint32_t i = threadIdx.x; i < n; i += SB)
         if (cum[i] >= plimit) {

@@ -136,6 +136,94 @@ __device__ __forceinline__ void rms_norm_scalar(const RmsNormParams &p) {
         yr[j] = (TA)((k * load_w<TW>(p.w, j)) * (float)xr[j]);
 }
 
+
+// Many short rows (d <= 4096 halves): one wave per row, rows dealt round-robin to a
+// fixed number of waves.  w is converted once and stays in registers for all rows
+// of the wave; the next row's x is already in flight while the current one is reduced
+// and written, so each wave keeps reads and writes streaming.
+template <typename TW>
+__device__ __forceinline__ void rms_norm_rows(const RmsNormParams &p) {
+    constexpr int CACHE = 8;
+    const uint32_t lane = threadIdx.x % WAVE;
+    const uint32_t waves = gridDim.x * (blockDim.x / WAVE);
+    uint32_t row = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+    const uint32_t nvec = p.d / 8;
+    if (row >= p.n) return;
+
+    // w stays in its storage type (f16 weights: 4 registers per vector) and is widened on use
+    struct WVec {
+        u32x4 raw[sizeof(TW) / 2];
+        __device__ __forceinline__ float get(int i) const {
+            if constexpr (sizeof(TW) == 2) {
+                Pack8 t;
+                t.u = raw[0];
+                return h2f(t.e[i]);
+            } else {
+                return __uint_as_float(raw[i / 4][i % 4]);
+            }
+        }
+    } w[CACHE];
+#pragma unroll
+    for (int c = 0; c < CACHE; ++c) {
+        const uint32_t v = lane + c * WAVE;
+        if (v < nvec) {
+#pragma unroll
+            for (int q = 0; q < (int)(sizeof(TW) / 2); ++q)
+                w[c].raw[q] = ld128(reinterpret_cast<const char *>(p.w) + ((size_t)v * 8 * sizeof(TW)) + 16 * q);
+        }
+    }
+    Pack8 cur[CACHE], nxt[CACHE];
+    {
+        const char *xr = reinterpret_cast<const char *>(p.x) + (int64_t)row * p.nsx;
+#pragma unroll
+        for (int c = 0; c < CACHE; ++c) {
+            const uint32_t v = lane + c * WAVE;
+            if (v < nvec) cur[c].u = ld128(xr + (size_t)v * 16);
+        }
+    }
+    for (; row < p.n; row += waves) {
+        const uint32_t next = row + waves;
+        if (next < p.n) {
+            const char *xn = reinterpret_cast<const char *>(p.x) + (int64_t)next * p.nsx;
+#pragma unroll
+            for (int c = 0; c < CACHE; ++c) {
+                const uint32_t v = lane + c * WAVE;
+                if (v < nvec) nxt[c].u = ld128(xn + (size_t)v * 16);
+            }
+        }
+        float ss = 0.f;
+#pragma unroll
+        for (int c = 0; c < CACHE; ++c) {
+            const uint32_t v = lane + c * WAVE;
+            if (v < nvec) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const float f = h2f(cur[c].e[i]);
+                    ss += f * f;
+                }
+            }
+        }
+        ss = wave_sum(ss);
+        const float k = 1.0f / sqrtf(ss / (float)p.d + p.epsilon);
+        char *yr = reinterpret_cast<char *>(p.y) + (int64_t)row * p.nsy;
+#pragma unroll
+        for (int c = 0; c < CACHE; ++c) {
+            const uint32_t v = lane + c * WAVE;
+            if (v < nvec) {
+                Pack8 o;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) o.e[i] = f2h((k * w[c].get(i)) * h2f(cur[c].e[i]));
+                st128(yr + (size_t)v * 16, o.u);
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < CACHE; ++c) cur[c] = nxt[c];
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(256) rms_norm_f16_f16_rows(RmsNormParams p) { rms_norm_rows<f16>(p); }
+extern "C" __global__ void __launch_bounds__(256) rms_norm_f16_f32_rows(RmsNormParams p) { rms_norm_rows<float>(p); }
+
 #define RMS_VEC(NAME, TA, TW, G)                                                        \
     extern "C" __global__ void __launch_bounds__((G) < 256 ? 256 : (G)) NAME(RmsNormParams p) { \
         rms_norm_vec<TA, TW, G>(p);                                                     \

@@ -179,7 +179,7 @@ EXPORTS = [
     "ophip_swiglu_create", "ophip_swiglu_scheme", "ophip_swiglu_launch", "ophip_swiglu_destroy",
     "ophip_sample_args_new", "ophip_sample_args_argmax",
     "ophip_random_sample_create", "ophip_random_sample_scheme", "ophip_random_sample_launch",
-    "ophip_random_sample_destroy", "ophip_random_sample_build_indices",
+    "ophip_random_sample_destroy", "ophip_random_sample_build_indices", "ophip_random_sample_launch_batch",
     "ophip_mat_mul_plan", "ophip_mat_mul_create", "ophip_mat_mul_scheme", "ophip_mat_mul_launch",
     "ophip_mat_mul_destroy",
 ]
@@ -625,6 +625,19 @@ class Swiglu(_Operator):
 
 class RandomSample(_Operator):
     NAME = "random_sample"
+
+    def launch_batch(self, args, rows, row_stride, seeds, workspace, queue_alloc):
+        """Extension: `rows` rows in one launch (seeds: None or a device pointer to `rows` f32 draws)."""
+        if workspace is None:
+            wp, wl = None, 0
+        elif isinstance(workspace, DevMem):
+            wp, wl = ctypes.c_void_p(workspace.ptr), workspace.size
+        else:
+            wp, wl = ctypes.c_void_p(workspace[0]), workspace[1]
+        _check(lib().ophip_random_sample_launch_batch(self.handle, ctypes.byref(args.c()), ctypes.c_size_t(rows),
+                                                      ctypes.c_ssize_t(row_stride),
+                                                      ctypes.c_void_p(_p(seeds)) if seeds is not None else None,
+                                                      wp, ctypes.c_size_t(wl), _qa(queue_alloc)), launch=True)
 
     @staticmethod
     def build_indices(n, queue_alloc):

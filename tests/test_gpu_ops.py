@@ -556,6 +556,36 @@ def test_random_sample_benchmark_config(gpu, stream):
         assert abs(val_of(val, f16) - val_of(rval, f16)) <= 2e-3 + 1e-2 * abs(val_of(rval, f16))
 
 
+def test_random_sample_batched_rows_match_single_launches(gpu, stream):
+    """The batched entry point (an extension) returns, per row, what the per-row launch returns."""
+    rng = np.random.default_rng(1)
+    rows = normal_f16(rng, (16, 32000), std=np.sqrt(3.0))
+    ld = gpu.from_host(rows)
+    kvd = gpu.from_host(np.full(32, 0xFFFFFFFF, np.uint32))
+    seeds = rng.random(16).astype(f32)
+    sd = gpu.from_host(seeds)
+    op = ophip.RandomSample(gpu)
+    args = ophip.RandomSampleArgs.layout(dt.F16, 32000)
+    args.kv_pair_base, args.logits_base = kvd, ld
+    say("random_sample batch argmax")
+    op.launch_batch(args, 16, 64000, None, None, stream)
+    kv = gpu.to_host(kvd, np.uint32, 32, stream=stream).reshape(16, 2)
+    for r in range(16):
+        assert (int(kv[r, 0]), int(kv[r, 1])) == oracle.argmax(rows[r])
+    args.config, args.seed = ophip.SampleArgs(0.8, 0.9, 50), 0.37
+    say("random_sample batch sample, shared draw")
+    op.launch_batch(args, 16, 64000, None, None, stream)
+    kv = gpu.to_host(kvd, np.uint32, 32, stream=stream).reshape(16, 2)
+    for r in range(16):
+        assert int(kv[r, 0]) == oracle.random_sample(rows[r], 0.8, 0.9, 50, 0.37)[0]
+    say("random_sample batch sample, per-row draws")
+    op.launch_batch(args, 16, 64000, sd, None, stream)
+    kv = gpu.to_host(kvd, np.uint32, 32, stream=stream).reshape(16, 2)
+    for r in range(16):
+        want = {oracle.random_sample(rows[r], 0.8, 0.9, 50, float(seeds[r]) * f)[0] for f in (1 - 1e-5, 1.0, 1 + 1e-5)}
+        assert int(kv[r, 0]) in want
+
+
 def test_random_sample_reference_config_f32(gpu, stream):
     """random_sample/cuda/mod.rs:240-370: n = 32000 f32 logits U[0,1); argmax; T 0.9, top_p 0.9, top_k 200, draw 0.75."""
     rng = np.random.default_rng(0)
