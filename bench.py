@@ -18,6 +18,7 @@ Beside it the script reports, in the same JSON line:
                same layer on the host cores.
 """
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -147,6 +148,33 @@ def time_launches(gpu, stream, fn, reps, warm=5):
     return e0.elapsed_ms(e1) * 1e3 / reps  # us per launch
 
 
+def profiled_traffic():
+    """HBM bytes per launch of the dominant kernel, measured with FETCH_SIZE / WRITE_SIZE in separate
+    counter runs and kept as text under profiles/ (a counter run cannot share a process with the timing)."""
+    path = os.path.join(ROOT, "profiles", "gemm_skinny_gate_up_pmc.txt")
+    try:
+        for line in open(path):
+            if line.startswith("traffic_bytes"):
+                return int(line.split("=")[1].split()[0])
+    except OSError:
+        pass
+    return None
+
+
+def copy_ceiling(ophip, gpu, stream):
+    """What a plain device-to-device copy of 1 GiB reaches (read + write counted): the practical
+    ceiling for streaming kernels on this machine, and the known-size kernel that calibrates
+    the FETCH_SIZE / WRITE_SIZE counters."""
+    a_, b_ = gpu.malloc(1 << 30), gpu.malloc(1 << 30)
+    gpu.memset(a_, 0x3C)
+    us = time_launches(gpu, stream, lambda: ophip._check(ophip.lib().ophip_memcpy_d2d(
+        gpu.handle, ctypes.c_void_p(b_.ptr), ctypes.c_void_p(a_.ptr), ctypes.c_size_t(1 << 30), stream.handle)), 10, warm=2)
+    a_.free(); b_.free()
+    log("  copy 1 GiB d2d (hipMemcpyAsync): %.1f us, %.1f GB/s read+write" % (us, (2 << 30) / us / 1e3))
+    return {"bytes": 2 << 30, "us": round(us, 2), "GBps": round((2 << 30) / us / 1e3, 1),
+            "hbm_frac": round((2 << 30) / (us * 1e-6) / HBM_PEAK, 4)}
+
+
 def standalone_ops(ophip, gpu, stream, rng, reps):
     """Every operator at its benchmark shape plus a scaled shape that does not fit the Infinity Cache."""
     o, L, F16 = ophip, ophip.TensorLayout, ophip.dt.F16
@@ -183,7 +211,7 @@ def standalone_ops(ophip, gpu, stream, rng, reps):
     # rope: [512, 32, 128] and [32768, 32, 128]
     rope = o.Rope(gpu)
     empty = L(F16, [0, DH], [2 * DH, 2])
-    for nt in (512, 32768):
+    for nt in (512, 65536):
         t = gpu.malloc(nt * NH * DH * 2)
         gpu.memset(t, 0x3C)
         pos = gpu.from_host((np.arange(nt) % 4096).astype(np.uint32))
@@ -193,7 +221,7 @@ def standalone_ops(ophip, gpu, stream, rng, reps):
         t.free()
     # rearrange: [32, 512, 128] -> [512, 32, 128] and a 64x larger one
     rea = o.Rearrange(gpu)
-    for s0, s1 in ((32, 512), (32, 32768)):
+    for s0, s1 in ((32, 512), (32, 65536)):
         src = gpu.malloc(s0 * s1 * DH * 2)
         dst = gpu.malloc(s0 * s1 * DH * 2)
         gpu.memset(src, 0x3C)
@@ -213,7 +241,7 @@ def standalone_ops(ophip, gpu, stream, rng, reps):
         att.free()
     # swiglu: [16, 11008] halves and [8192, 11008]
     sw = o.Swiglu(gpu)
-    for n in (16, 8192):
+    for n in (16, 16384):
         gu = gpu.malloc(n * 2 * DI * 2)
         gpu.memset(gu, 0x3C)
         half = L(F16, [n, DI], [2 * DI * 2, 2])
@@ -243,11 +271,11 @@ def standalone_ops(ophip, gpu, stream, rng, reps):
     # compute-bound mat_mul: 4096^3 and 8192^3
     mm = o.MatMul(gpu)
     for n in (4096, 8192):
-        A_, B_, C_ = gpu.malloc(n * n * 2), gpu.malloc(n * n * 2), gpu.malloc(n * n * 2)
-        gpu.memset(A_, 0x3C); gpu.memset(B_, 0x3C)
+        A_, B_, C_ = gpu.from_host(normal_f16(rng, (n, n), 1.0)), gpu.from_host(normal_f16(rng, (n, n), 0.02)), \
+            gpu.malloc(n * n * 2)
         a = o.MatMulArgs(c(n, n), C_, 0.0, c(n, n), A_, c(n, n), B_, 1.0)
         mm.scheme(a, 0)
-        us = time_launches(gpu, stream, lambda: mm.launch(a, None, stream), 3, warm=1)
+        us = time_launches(gpu, stream, lambda: mm.launch(a, None, stream), 10, warm=2)
         add("mat_mul", "%d^3" % n, 3 * n * n * 2, us, flops=2 * n ** 3)
         A_.free(); B_.free(); C_.free()
     return out
@@ -337,6 +365,7 @@ def main():
         per_layer.append(rec)
         log("  %-12s %9.2f us %9.1f GB/s %5.1f%% HBM" % (name, us, rec["GBps"], 100 * rec["hbm_frac"]))
 
+    ceiling = copy_ceiling(ophip, gpu, stream)
     per_op = []
     if not args.no_per_op:
         log("standalone operators:")
@@ -375,9 +404,10 @@ def main():
                    "flops_per_step": layer_flops, "hbm_frac_of_step": round(layer_bytes / (ms_per_step * 1e-3) / HBM_PEAK, 4)},
         "roofline": {"bound": "hbm", "kernel": "gemm_skinny (gate/up mat_mul 16x4096 . 4096x22016)",
                      "achieved": round(dom_bytes / (dom_us * 1e-6) / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": round(dom_bytes / (dom_us * 1e-6) / HBM_PEAK, 4), "traffic": None,
+                     "frac": round(dom_bytes / (dom_us * 1e-6) / HBM_PEAK, 4), "traffic": profiled_traffic(),
                      "us": round(dom_us, 3), "algorithmic_bytes": dom_bytes},
         "cpu_baseline": cpu,
+        "copy_ceiling": ceiling,
         "per_op_layer": per_layer,
         "per_op": per_op,
     }
