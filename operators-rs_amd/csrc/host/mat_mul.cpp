@@ -3,6 +3,7 @@
 // (mat_mul/common_cpu/mod.rs:60-105): for f16 data alpha and beta are rounded
 // to f16 first and C is read only when the f32 beta is non-zero.
 #include <algorithm>
+#include <cstdio>
 #include <cstdlib>
 #include <mutex>
 #include <unordered_map>
@@ -175,11 +176,12 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
             g.qmode = p.q_sj == 1 ? 0 : 1;
             // The kernel is latency-bound per CU, so a CU that holds two workgroups takes
             // twice as long as one that holds one: split K only as far as one workgroup
-            // per CU (rounding down), keeping at least 8 K-steps per workgroup.
+            // per CU (rounding down), keeping at least 16 K-steps per workgroup (the in-kernel
+            // reduction of a split costs a few microseconds of tail).
             const size_t ntiles = (p.N + 127) / 128, slabs = (p.K + 31) / 32;
             const size_t base = ntiles * p.batch;
             size_t split = std::max<size_t>(1, (size_t)cus / base);
-            split = std::min(split, std::max<size_t>(1, slabs / 8));
+            split = std::min(split, std::max<size_t>(1, slabs / 16));
             if (const char *e = std::getenv("OPHIP_GEMM_SPLITK")) split = std::max(1, std::atoi(e));
             size_t sps = (slabs + split - 1) / split;  // K-steps per split
             split = (slabs + sps - 1) / sps;
@@ -192,12 +194,16 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
     // Compute-bound shapes: the LDS-tiled MFMA kernel.  Of the two orientations take
     // the one whose epilogue can store several adjacent outputs per lane.
     auto tile_ok = [&](uint32_t b) {
-        if (!f16 || p.K == 0 || p.K % 32 != 0 || p.M % b != 0 || p.N % b != 0) return false;
+        if (!f16 || p.K == 0 || p.K % (b == 256 ? 64 : 32) != 0 || p.M % b != 0 || p.N % b != 0) return false;
         if (!aligned16(p.p) || !aligned16(p.q) || !aligned16(p.d)) return false;
         if (!mult8(p.p_sb) || !mult8(p.q_sb) || !mult8(p.d_sb)) return false;
         if (!(p.p_sl == 1 ? mult8(p.p_si) : mult8(p.p_sl))) return false;
         if (!(p.q_sl == 1 ? mult8(p.q_sj) : mult8(p.q_sl))) return false;
         if (!(p.d_sj == 1 ? mult8(p.d_si) : mult8(p.d_sj))) return false;
+        // the kernel addresses inside an operand tile with 32-bit byte offsets
+        const int64_t lim = (int64_t)1 << 22;
+        for (int64_t st : {p.p_si, p.p_sl, p.q_sj, p.q_sl})
+            if (st <= 0 || st >= lim) return false;
         return true;
     };
     for (uint32_t b : {256u, 128u}) {
@@ -205,8 +211,12 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
         for (int attempt = 0; attempt < 2; ++attempt) {
             orient(attempt == 1);
             if (!tile_ok(b)) continue;
-            if (b == 256 && (size_t)(p.M / b) * (p.N / b) * p.batch < cus / 2 && p.M % 128 == 0 && p.N % 128 == 0)
-                continue;  // too few 256-tiles to fill the machine: let the 128 pass take it
+            // too few 256-tiles to fill the machine: let the 128 pass take it
+            // (OPHIP_GEMM_TILE=256 keeps the large tile, for tests of that kernel on small shapes)
+            const char *force = std::getenv("OPHIP_GEMM_TILE");
+            if (b == 256 && !(force && std::atoi(force) == 256) &&
+                (size_t)(p.M / b) * (p.N / b) * p.batch < cus / 2 && p.M % 128 == 0 && p.N % 128 == 0)
+                continue;
             const bool wide = (p.q_sl != 1 && p.d_sj == 1) || (p.p_sl == 1 && p.d_si == 1);
             if (best < 0 || wide) best = attempt;
             if (wide) break;
@@ -304,6 +314,21 @@ int ophip_mat_mul_scheme(ophip_mat_mul *op, const ophip_mat_mul_args *args, size
         if (L.dt != OPHIP_DT_F16 && L.dt != OPHIP_DT_F32) throw type_not_support("mat_mul supports f16 and f32");
         const GemmPlan g = make_plan(*args, L, (unsigned)op->dev->props.multiProcessorCount);
         if (ws && g.workspace <= max_ws) *ws = g.workspace;
+    });
+}
+
+int ophip_mat_mul_describe(const ophip_mat_mul *op, const ophip_mat_mul_args *args, char *out, size_t len) {
+    return guard([&] {
+        if (!op || !args || !out || len == 0) throw args_not_support("null argument");
+        const ophip_mat_mul_layout L = mat_mul_layout(*args);
+        if (L.dt != OPHIP_DT_F16 && L.dt != OPHIP_DT_F32) throw type_not_support("mat_mul supports f16 and f32");
+        const GemmPlan g = make_plan(*args, L, (unsigned)op->dev->props.multiProcessorCount);
+        if (g.kind == GemmPlan::Skinny)
+            std::snprintf(out, len, "skinny rows<=%d q%s split_k=%u", 16 * g.mt, g.qmode ? "K" : "N", g.p.split_k);
+        else if (g.kind == GemmPlan::Tile)
+            std::snprintf(out, len, "tile%d p%s q%s", g.tile, g.pk ? "K" : "M", g.qk ? "K" : "N");
+        else
+            std::snprintf(out, len, "generic");
     });
 }
 

@@ -3,8 +3,8 @@
 //     D[i, j] = alpha * sum_l P[i, l] * Q[l, j] + (read_dst ? beta * D[i, j] : 0)
 //
 // A 256-thread workgroup (4 waves, 2 x 2) owns a BM x BN tile of D and walks K in
-// steps of 32.  Both operands are staged in LDS as K-contiguous rows (one row per
-// i for P, one per j for Q, padded to 40 halves so that 16-byte reads of 32
+// steps of TK (64 for 256 x 256 tiles, 32 for 128 x 128).  Both operands are staged in LDS as K-contiguous rows (one row per
+// i for P, one per j for Q, padded by 8 halves so that 16-byte reads of 32
 // consecutive rows hit distinct banks), which is the layout MFMA wants: every
 // lane reads its 8 consecutive k with one ds_read_b128.  An operand that is
 // K-contiguous in memory is copied 16 bytes at a time; one that is contiguous
@@ -16,14 +16,17 @@
 // them) each work on a compact block of tiles and share operand panels in
 // their own L2.
 //
-// Requirements checked by the host: M % BM == 0, N % BN == 0, K % 32 == 0,
+// Requirements checked by the host: M % BM == 0, N % BN == 0, K % TK == 0 (TK = 64 for the
+// 256 tiles, 32 for the 128 tiles),
 // 16-byte aligned bases and strides.  Everything else runs on the generic kernel.
+#include <type_traits>
+
 #include "device_util.h"
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int TK = 32;       // K per step
-constexpr int LDK = TK + 8;  // LDS row pitch in halves (80 bytes)
+// TK = K per step (32 or 64); LDS row pitch = TK + 8 halves (80 or 144 bytes: an odd
+// multiple of 16, so 16-byte reads of consecutive rows spread over all banks).
 
 // Copies one R x 32 operand tile from global memory to registers (`fetch`) and
 // from registers to LDS (`commit`).  KCONTIG: rows are K-contiguous in memory.
@@ -36,8 +39,9 @@ constexpr int LDK = TK + 8;  // LDS row pitch in halves (80 bytes)
 // consecutive slots.  MFMA does not care which rows a tile holds, so the readers
 // simply take 32 consecutive slots and the epilogue maps slots back to rows with
 // row(s) = (s % (R / 8)) * 8 + s / (R / 8).
-template <int R, bool KCONTIG>
+template <int R, bool KCONTIG, int TK>
 struct TileLoader {
+    static constexpr int LDK = TK + 8;
     static constexpr bool PERMUTED = !KCONTIG;
     __device__ static __forceinline__ uint32_t row_of_slot(uint32_t s) {
         return PERMUTED ? (s % (R / 8)) * 8 + s / (R / 8) : s;
@@ -48,65 +52,74 @@ struct TileLoader {
         if constexpr (PERMUTED && R == 128) return (w * 4 + 2 * (r / 16) + t) * 16 + r % 16;
         return w * (R / 2) + t * 32 + r;
     }
-    // K-contiguous: R * 4 vectors of 8 halves, R / 64 per thread.
-    // Row-contiguous: thread (cb, kb) takes KR = R / 64 k-rows x 8 columns.
-    static constexpr int NV = R / 64;
+    // K-contiguous: R * TK/8 vectors of 8 halves, NV per thread.
+    // Row-contiguous: thread (cb, kb) takes NV k-rows x 8 columns.
+    static constexpr int KV = TK / 8;
+    static constexpr int NV = R * KV / 256;
     u32x4 reg[NV];
+    uint32_t voff[NV];  // byte offset of each of the thread's vectors from the tile's first element
 
-    __device__ __forceinline__ void fetch(const f16 *base, int64_t s_row, int64_t s_k, uint32_t row0, uint32_t k0) {
+    // s_row: stride between rows (i or j), s_k: stride along K, in elements; one of them is 1.
+    // The host guarantees that offsets inside a tile fit 32 bits.
+    __device__ __forceinline__ void init(int64_t s_row, int64_t s_k) {
         const uint32_t t = threadIdx.x;
-        if constexpr (KCONTIG) {
 #pragma unroll
-            for (int v = 0; v < NV; ++v) {
-                const uint32_t idx = t + v * 256, row = idx / 4, kv = idx % 4;
-                reg[v] = ld128(base + (int64_t)(row0 + row) * s_row + (k0 + kv * 8));
+        for (int v = 0; v < NV; ++v) {
+            if constexpr (KCONTIG) {
+                const uint32_t idx = t + v * 256, row = idx / KV, kv = idx % KV;
+                voff[v] = (row * (uint32_t)s_row + kv * 8) * 2;
+            } else {
+                const uint32_t cb = t % (R / 8), kb = t / (R / 8);
+                voff[v] = ((kb * NV + v) * (uint32_t)s_k + cb * 8) * 2;
             }
-        } else {
-            const uint32_t cb = t % (R / 8), kb = t / (R / 8);
-#pragma unroll
-            for (int v = 0; v < NV; ++v)
-                reg[v] = ld128(base + (int64_t)(k0 + kb * NV + v) * s_k + (row0 + cb * 8));
         }
     }
 
-    __device__ __forceinline__ void commit(f16 *lds) const {
+    // `tile` (wave-uniform) points at element (row0, k0) of the operand.  The copy is cut
+    // into NV pieces so that the main loop can place them one by one between MFMAs.
+    __device__ __forceinline__ void fetch_piece(const f16 *tile, int v) {
+        reg[v] = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(tile) + voff[v]);
+    }
+    __device__ __forceinline__ void fetch(const f16 *tile) {
+#pragma unroll
+        for (int v = 0; v < NV; ++v) fetch_piece(tile, v);
+    }
+
+    // Piece v of the register -> LDS copy.  K-contiguous: vector v.  Row-contiguous: reg[v]
+    // holds k-row (kb*NV + v), columns cb*8 .. +8, and piece v writes columns
+    // v*8/NV .. (v+1)*8/NV, each as the NV halves the thread holds of it (so every piece
+    // reads all NV registers: refill them only after the last piece).
+    __device__ __forceinline__ void commit_piece(f16 *lds, int v) const {
         const uint32_t t = threadIdx.x;
         if constexpr (KCONTIG) {
-#pragma unroll
-            for (int v = 0; v < NV; ++v) {
-                const uint32_t idx = t + v * 256, row = idx / 4, kv = idx % 4;
-                st128(lds + row * LDK + kv * 8, reg[v]);
-            }
+            const uint32_t idx = t + v * 256, row = idx / KV, kv = idx % KV;
+            st128(lds + row * LDK + kv * 8, reg[v]);
         } else {
             const uint32_t cb = t % (R / 8), kb = t / (R / 8);
-            // reg[v] holds k-row (kb*NV + v), columns cb*8 .. +8: write column c's NV halves together
 #pragma unroll
-            for (int c = 0; c < 8; ++c) {
+            for (int c = v * 8 / NV; c < (v + 1) * 8 / NV; ++c) {
                 f16 *dst = lds + (c * (R / 8) + cb) * LDK + kb * NV;
-                if constexpr (NV == 4) {
-                    uint32_t lo, hi;
-                    const uint32_t a0 = reg[0][c / 2], a1 = reg[1][c / 2], a2 = reg[2][c / 2], a3 = reg[3][c / 2];
-                    if (c & 1) {
-                        lo = (a0 >> 16) | (a1 & 0xffff0000u);
-                        hi = (a2 >> 16) | (a3 & 0xffff0000u);
-                    } else {
-                        lo = (a0 & 0xffffu) | (a1 << 16);
-                        hi = (a2 & 0xffffu) | (a3 << 16);
-                    }
-                    *reinterpret_cast<u32x2 *>(dst) = u32x2{lo, hi};
-                } else {
-                    static_assert(NV == 2, "");
-                    const uint32_t a0 = reg[0][c / 2], a1 = reg[1][c / 2];
-                    *reinterpret_cast<uint32_t *>(dst) =
-                        (c & 1) ? ((a0 >> 16) | (a1 & 0xffff0000u)) : ((a0 & 0xffffu) | (a1 << 16));
+                uint32_t w[NV / 2];
+#pragma unroll
+                for (int d = 0; d < NV / 2; ++d) {
+                    const uint32_t a0 = reg[2 * d][c / 2], a1 = reg[2 * d + 1][c / 2];
+                    w[d] = (c & 1) ? ((a0 >> 16) | (a1 & 0xffff0000u)) : ((a0 & 0xffffu) | (a1 << 16));
                 }
+                if constexpr (NV == 8) *reinterpret_cast<u32x4 *>(dst) = u32x4{w[0], w[1], w[2], w[3]};
+                else if constexpr (NV == 4) *reinterpret_cast<u32x2 *>(dst) = u32x2{w[0], w[1]};
+                else *reinterpret_cast<uint32_t *>(dst) = w[0];
             }
         }
+    }
+    __device__ __forceinline__ void commit(f16 *lds) const {
+#pragma unroll
+        for (int v = 0; v < NV; ++v) commit_piece(lds, v);
     }
 };
 
-template <int BM, int BN, bool PK, bool QK>
+template <int BM, int BN, bool PK, bool QK, int TK>
 __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
+    constexpr int LDK = TK + 8;
     constexpr int WM = BM / 2, WN = BN / 2;  // wave tile
     constexpr int TM = WM / 32, TN = WN / 32;
     __shared__ f16 lds[2][(BM + BN) * LDK];
@@ -146,42 +159,96 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
 
-    typedef TileLoader<BM, PK> LP;
-    typedef TileLoader<BN, QK> LQ;
+    typedef TileLoader<BM, PK, TK> LP;
+    typedef TileLoader<BN, QK, TK> LQ;
     LP lp;
     LQ lq;
     const uint32_t ksteps = p.K / TK;
-    lp.fetch(pb, p.p_si, p.p_sl, i0, 0);
-    lq.fetch(qb, p.q_sj, p.q_sl, j0, 0);
+    constexpr int KK = TK / 16;  // MFMA k-steps per LDS tile
+    lp.init(p.p_si, p.p_sl);
+    lq.init(p.q_sj, p.q_sl);
+    const f16 *ptile = pb + (int64_t)i0 * p.p_si, *qtile = qb + (int64_t)j0 * p.q_sj;
+    const int64_t pstep = (int64_t)TK * p.p_sl, qstep = (int64_t)TK * p.q_sl;
+    // One wave per SIMD: nothing hides a stall, so the loop is software-pipelined by hand.
+    //   registers  : tile s+1 waits in `reg` while tile s is multiplied; MFMA fragments are
+    //                double-buffered, the LDS reads of k-step kk+1 run under the MFMAs of kk
+    //   k-step 0   : tile s+1 goes from registers to the other LDS buffer
+    //   k-step 1   : the global loads of tile s+2 refill the registers
+    //   barrier    : before the last k-step (whose fragments are already in registers), so
+    //                that step's MFMAs cover the first fragment reads of tile s+1
+    // The code below is written in exactly that order, one memory operation of each kind
+    // after each MFMA, and sched_barrier(0) after every such group keeps the compiler from
+    // regrouping them.
+    lp.fetch(ptile);
+    lq.fetch(qtile);
     lp.commit(lds[0]);
     lq.commit(lds[0] + BM * LDK);
+    if (ksteps > 1) {
+        lp.fetch(ptile + pstep);
+        lq.fetch(qtile + qstep);
+    }
     __syncthreads();
 
-    for (uint32_t ks = 0; ks < ksteps; ++ks) {
-        const f16 *Ps = lds[ks & 1], *Qs = lds[ks & 1] + BM * LDK;
-        if (ks + 1 < ksteps) {
-            lp.fetch(pb, p.p_si, p.p_sl, i0, (ks + 1) * TK);
-            lq.fetch(qb, p.q_sj, p.q_sl, j0, (ks + 1) * TK);
-        }
+    Pack8 a[2][TM], b[2][TN];
+    const uint32_t a_off = LP::reader_slot(wm, 0, l32) * LDK + lk * 8;
+    const uint32_t b_off = BM * LDK + LQ::reader_slot(wn, 0, l32) * LDK + lk * 8;
+    // fragment r of k-step kk of the tile at `tile`: r < TM is a P fragment, the rest are Q's
+    auto read_one = [&](int buf, const f16 *tile, int kk, int r) {
+        if (r < TM)
+            a[buf][r].u = ld128(tile + a_off + (LP::reader_slot(wm, r, l32) - LP::reader_slot(wm, 0, l32)) * LDK + kk * 16);
+        else
+            b[buf][r - TM].u = ld128(tile + b_off + (LQ::reader_slot(wn, r - TM, l32) - LQ::reader_slot(wn, 0, l32)) * LDK + kk * 16);
+    };
+    auto mfma_one = [&](int buf, int m) {
+        const int tm = m / TN, tn = m % TN;
+        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[buf][tm].h, b[buf][tn].h, acc[tm][tn], 0, 0, 0);
+    };
+    constexpr int NMFMA = TM * TN, NREAD = TM + TN, NLOAD = LP::NV + LQ::NV;
+    static_assert(NREAD <= NMFMA && NLOAD <= NMFMA, "one memory operation of a kind per MFMA at most");
+    static_assert(KK >= 2 && KK % 2 == 0, "fragment buffers alternate per k-step");
+    constexpr int LOAD_KK = KK > 2 ? 1 : 0;  // the k-step that carries the global loads
+    // STORE: tile ks+1 exists (it is in `reg`); LOAD: tile ks+2 exists.
+    auto step = [&](uint32_t ks, auto store, auto load) {
+        constexpr bool STORE = decltype(store)::value, LOAD = decltype(load)::value;
+        f16 *cur = lds[ks & 1], *nxt = lds[(ks + 1) & 1];
+        const f16 *pnext = ptile + (ks + 2) * pstep, *qnext = qtile + (ks + 2) * qstep;
 #pragma unroll
-        for (int kk = 0; kk < TK / 16; ++kk) {
-            Pack8 a[TM], b[TN];
+        for (int kk = 0; kk < KK - 1; ++kk) {
 #pragma unroll
-            for (int t = 0; t < TM; ++t) a[t].u = ld128(Ps + LP::reader_slot(wm, t, l32) * LDK + kk * 16 + lk * 8);
-#pragma unroll
-            for (int t = 0; t < TN; ++t) b[t].u = ld128(Qs + LQ::reader_slot(wn, t, l32) * LDK + kk * 16 + lk * 8);
-#pragma unroll
-            for (int tm = 0; tm < TM; ++tm)
-#pragma unroll
-                for (int tn = 0; tn < TN; ++tn)
-                    acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[tm].h, b[tn].h, acc[tm][tn], 0, 0, 0);
-        }
-        if (ks + 1 < ksteps) {
-            lp.commit(lds[(ks + 1) & 1]);
-            lq.commit(lds[(ks + 1) & 1] + BM * LDK);
+            for (int m = 0; m < NMFMA; ++m) {
+                mfma_one(kk & 1, m);
+                if (m < NREAD) read_one((kk + 1) & 1, cur, kk + 1, m);
+                if (STORE && kk == 0 && m < NLOAD) {
+                    if (m < LP::NV) lp.commit_piece(nxt, m);
+                    else lq.commit_piece(nxt + BM * LDK, m - LP::NV);
+                }
+                if (LOAD && KK > 2 && kk == LOAD_KK && m < NLOAD) {
+                    if (m < LP::NV) lp.fetch_piece(pnext, m);
+                    else lq.fetch_piece(qnext, m - LP::NV);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (LOAD && KK == 2 && kk == 0) {
+                lp.fetch(pnext);
+                lq.fetch(qnext);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
         __syncthreads();
-    }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int m = 0; m < NMFMA; ++m) {
+            mfma_one((KK - 1) & 1, m);
+            if (STORE && m < NREAD) read_one(0, nxt, 0, m);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+#pragma unroll
+    for (int r = 0; r < NREAD; ++r) read_one(0, lds[0], 0, r);
+    uint32_t ks = 0;
+    for (; ks + 2 < ksteps; ++ks) step(ks, std::true_type{}, std::true_type{});
+    if (ks + 1 < ksteps) step(ks++, std::true_type{}, std::false_type{});
+    step(ks, std::false_type{}, std::false_type{});
 
     // 32x32 accumulator tile: lane holds slot-column l32 and slot-rows 8*(e/4) + 4*lk + e%4.
     f16 *db = reinterpret_cast<f16 *>(p.d) + (int64_t)bat * p.d_sb;
@@ -248,16 +315,16 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
     }
 }
 
-#define GEMM_TILE(BM, BN, PK, QK)                                                                        \
+#define GEMM_TILE(BM, BN, PK, QK, TK)                                                                    \
     extern "C" __global__ void __launch_bounds__(256) gemm_tile_##BM##x##BN##_p##PK##_q##QK(GemmParams p) { \
-        gemm_tile<BM, BN, PK, QK>(p);                                                                    \
+        gemm_tile<BM, BN, PK, QK, TK>(p);                                                                \
     }
 
-GEMM_TILE(256, 256, 1, 1)
-GEMM_TILE(256, 256, 1, 0)
-GEMM_TILE(256, 256, 0, 1)
-GEMM_TILE(256, 256, 0, 0)
-GEMM_TILE(128, 128, 1, 1)
-GEMM_TILE(128, 128, 1, 0)
-GEMM_TILE(128, 128, 0, 1)
-GEMM_TILE(128, 128, 0, 0)
+GEMM_TILE(256, 256, 1, 1, 64)
+GEMM_TILE(256, 256, 1, 0, 64)
+GEMM_TILE(256, 256, 0, 1, 64)
+GEMM_TILE(256, 256, 0, 0, 64)
+GEMM_TILE(128, 128, 1, 1, 32)
+GEMM_TILE(128, 128, 1, 0, 32)
+GEMM_TILE(128, 128, 0, 1, 32)
+GEMM_TILE(128, 128, 0, 0, 32)

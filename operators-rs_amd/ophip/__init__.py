@@ -181,7 +181,7 @@ EXPORTS = [
     "ophip_random_sample_create", "ophip_random_sample_scheme", "ophip_random_sample_launch",
     "ophip_random_sample_destroy", "ophip_random_sample_build_indices", "ophip_random_sample_launch_batch",
     "ophip_mat_mul_plan", "ophip_mat_mul_create", "ophip_mat_mul_scheme", "ophip_mat_mul_launch",
-    "ophip_mat_mul_destroy",
+    "ophip_mat_mul_destroy", "ophip_mat_mul_describe",
 ]
 
 _lib = None
@@ -648,3 +648,9 @@ class RandomSample(_Operator):
 
 class MatMul(_Operator):
     NAME = "mat_mul"
+
+    def describe(self, args):
+        """Name of the kernel family launch() would pick for these arguments (diagnostics)."""
+        buf = ctypes.create_string_buffer(96)
+        _check(lib().ophip_mat_mul_describe(self.handle, ctypes.byref(args.c()), buf, ctypes.c_size_t(96)))
+        return buf.value.decode()

@@ -847,6 +847,28 @@ def test_mat_mul_mfma_tile_kernel_layouts(gpu, stream, ta, tb, tc, m, n, k, bt):
     check_mat_mul(out0, np.zeros(cv.shape, f16), av, bv, 1.0, 0.0, "mat_mul tile beta 0")
 
 
+@pytest.mark.parametrize("ta", [False, True])
+@pytest.mark.parametrize("tb", [False, True])
+@pytest.mark.parametrize("tc", [False, True])
+@pytest.mark.parametrize("m,n,k,bt", [(512, 768, 192, 2), (256, 256, 64, 1), (256, 512, 128, 1)])
+def test_mat_mul_mfma_256_tile_kernel_layouts(gpu, stream, monkeypatch, ta, tb, tc, m, n, k, bt):
+    """The 256 x 256 tile kernel (normally kept for shapes with at least 128 tiles) on one, two and
+    three K-steps - the pipeline's last, second-last and steady-state iterations - in every layout."""
+    monkeypatch.setenv("OPHIP_GEMM_TILE", "256")
+    rng = np.random.default_rng(m + n + k + 4 * ta + 2 * tb + tc)
+    a = rng.standard_normal((bt, k, m) if ta else (bt, m, k)).astype(f32).astype(f16)
+    b = rng.standard_normal((bt, n, k) if tb else (bt, k, n)).astype(f32).astype(f16)
+    c = rng.standard_normal((bt, n, m) if tc else (bt, m, n)).astype(f32).astype(f16)
+    av = a.transpose(0, 2, 1) if ta else a
+    bv = b.transpose(0, 2, 1) if tb else b
+    cv = c.transpose(0, 2, 1) if tc else c
+    say("mat_mul 256-tile ta=%s tb=%s tc=%s %dx%dx%d" % (ta, tb, tc, m, n, k))
+    args = ophip.MatMulArgs(TensorLayout.of(cv), None, 0.5, TensorLayout.of(av), None, TensorLayout.of(bv), None, 0.75)
+    assert ophip.MatMul(gpu).describe(args).startswith("tile256"), ophip.MatMul(gpu).describe(args)
+    out = run_mat_mul(gpu, stream, cv, av, bv, 0.75, 0.5)
+    check_mat_mul(out, cv, av, bv, 0.75, 0.5, "mat_mul 256-tile layouts")
+
+
 def test_mat_mul_compute_bound_shape(gpu, stream):
     rng = np.random.default_rng(12)
     n = 2048
