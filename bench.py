@@ -280,6 +280,21 @@ def standalone_ops(ophip, gpu, stream, rng, reps):
         b = arg_rows[0]
         us = time_launches(gpu, stream, lambda: rs.launch_batch(b, 16, 64000, None, None, stream), reps)
         add("random_sample " + mode, "16 x [32000]", 16 * (32000 * 2 + 8), us, note="1 batched launch (extension)")
+    # attention_kv_cached, the crate's composite, at the decode-layer shape: two cache appends, a staging copy
+    # of the strided q, QK^T, causal softmax, PV and the copy into o - seven launches
+    nt, pos = NT, KV - NT
+    qkv = gpu.from_host(normal_f16(rng, (nt, 3 * D), 1.0))
+    kc, vc = gpu.from_host(normal_f16(rng, (NH, KV, DH), 1.0)), gpu.from_host(normal_f16(rng, (NH, KV, DH), 1.0))
+    obuf = gpu.malloc(nt * D * 2)
+    head_major = lambda row_bytes: L(F16, [NH, nt, DH], [DH * 2, row_bytes, 2])
+    akv = o.AttnKVCached(gpu)
+    a = o.AttnKVCachedArgs(head_major(3 * D * 2), qkv.ptr, head_major(3 * D * 2), qkv.ptr + D * 2,
+                           head_major(3 * D * 2), qkv.ptr + 2 * D * 2, head_major(D * 2), obuf,
+                           c(NH, KV, DH), kc, c(NH, KV, DH), vc, o.AttnMask.CAUSAL, pos)
+    ws = gpu.malloc(max(akv.scheme(a, 1 << 30), 1))
+    us = time_launches(gpu, stream, lambda: akv.launch(a, ws, stream), reps)
+    add("attention_kv_cached", "nh32 seq16 pos2032 dh128", 2 * NH * KV * DH * 2 + 8 * nt * D * 2, us,
+        note="composite of 7 launches; bytes = both caches read once + q, k, v, o and the appended rows")
     # compute-bound mat_mul: 4096^3 and 8192^3
     mm = o.MatMul(gpu)
     for n in (4096, 8192):

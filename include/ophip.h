@@ -384,6 +384,67 @@ OPHIP_API void ophip_mat_mul_destroy(ophip_mat_mul *op);
  * "generic") into out[0..len). */
 OPHIP_API int ophip_mat_mul_describe(const ophip_mat_mul *op, const ophip_mat_mul_args *args, char *out, size_t len);
 
+/* ---- attention: attention/args.rs:10-24, attention/operator.rs:31-277 ------ */
+/* The composite the crate builds from mat_mul, fuesd_softmax and rearrange
+ * (attention/mod.rs:8-17): att = softmax(q . k^T / sqrt(dh)) per kv-head group,
+ * o = att . v.  q [nh, seq, dh], k and v [nkvh, att, dh], o [nh, seq, dh];
+ * nh must be a multiple of nkvh.  As in the reference, q is overwritten (it
+ * receives att . v before the copy into o) unless its layout forces a staging
+ * copy, and launch() needs nh*seq*(dh + att) elements of workspace, taken from
+ * the queue allocator when the caller's slice is smaller. */
+typedef struct ophip_attention_args {
+    ophip_tensor_layout q_layout;
+    void *q_base;
+    ophip_tensor_layout k_layout;
+    const void *k_base;
+    ophip_tensor_layout v_layout;
+    const void *v_base;
+    ophip_tensor_layout o_layout;
+    void *o_base;
+    uint8_t mask; /* ophip_attn_mask */
+} ophip_attention_args;
+typedef struct ophip_attention ophip_attention;
+OPHIP_API int ophip_attention_create(ophip_device *dev, ophip_attention **out);
+OPHIP_API int ophip_attention_scheme(ophip_attention *op, const ophip_attention_args *args,
+                                     size_t max_workspace_size, size_t *workspace_size);
+OPHIP_API int ophip_attention_launch(const ophip_attention *op, const ophip_attention_args *args,
+                                     void *workspace, size_t workspace_len,
+                                     const ophip_queue_alloc *queue_alloc);
+OPHIP_API void ophip_attention_destroy(ophip_attention *op);
+
+/* ---- attention_kv_cached: attention_kv_cached/args.rs:8-30, operator.rs:29-183 */
+/* Appends k, v [nkvh, seq, dh] to the caches [nkvh, buf, dh] at row `pos`
+ * (two rearranges), then runs attention over cache rows [0, pos + seq).
+ * pos + seq beyond either cache's buf is ShapeMismatch ("Out of cache
+ * buffer").  As in the reference, the v-cache is addressed with the k-cache's
+ * strides (operator.rs:114,156): give both caches the same layout. */
+typedef struct ophip_attention_kv_cached_args {
+    ophip_tensor_layout q_layout;
+    void *q_base;
+    ophip_tensor_layout k_layout;
+    const void *k_base;
+    ophip_tensor_layout v_layout;
+    const void *v_base;
+    ophip_tensor_layout o_layout;
+    void *o_base;
+    ophip_tensor_layout k_cache_layout;
+    void *k_cache_base;
+    ophip_tensor_layout v_cache_layout;
+    void *v_cache_base;
+    uint8_t mask; /* ophip_attn_mask */
+    size_t pos;   /* OPHIP_DYN_USIZE = dynamic (scheme only) */
+} ophip_attention_kv_cached_args;
+typedef struct ophip_attention_kv_cached ophip_attention_kv_cached;
+OPHIP_API int ophip_attention_kv_cached_create(ophip_device *dev, ophip_attention_kv_cached **out);
+OPHIP_API int ophip_attention_kv_cached_scheme(ophip_attention_kv_cached *op,
+                                               const ophip_attention_kv_cached_args *args,
+                                               size_t max_workspace_size, size_t *workspace_size);
+OPHIP_API int ophip_attention_kv_cached_launch(const ophip_attention_kv_cached *op,
+                                               const ophip_attention_kv_cached_args *args,
+                                               void *workspace, size_t workspace_len,
+                                               const ophip_queue_alloc *queue_alloc);
+OPHIP_API void ophip_attention_kv_cached_destroy(ophip_attention_kv_cached *op);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,391 @@
+// attention and attention_kv_cached on the HIP backend: the two composites that sit
+// directly on top of mat_mul, fuesd_softmax and rearrange in the reference
+// (attention/operator.rs:1-278, attention_kv_cached/operator.rs:1-184).  They own no
+// kernels: they plan workspace, build views and launch the three operators in the
+// reference's order, so the work lands on the queue exactly as the crate would put it.
+#include <cmath>
+
+#include "handle.hpp"
+
+using namespace ophip;
+
+namespace {
+
+// a sub-operator's status code back into an Error, keeping its message
+void sub(int code) {
+    if (code != OPHIP_OK) throw Error{code, ophip_last_error()};
+}
+
+// rank-3 layout with owned shape / strides (bytes), viewable as ophip_tensor_layout
+struct Lay3 {
+    size_t shape[3];
+    ptrdiff_t strides[3];
+    ophip_tensor_layout tl(uint64_t dt) const { return ophip_tensor_layout{dt, 3, shape, strides}; }
+    static Lay3 contiguous(uint64_t dt, size_t a, size_t b, size_t c) {  // TensorLayout::new_contiguous
+        const ptrdiff_t e = (ptrdiff_t)ophip_dtype_nbytes(dt);
+        return Lay3{{a, b, c}, {(ptrdiff_t)(b * c) * e, (ptrdiff_t)c * e, e}};
+    }
+    static Lay3 dyn(size_t a, size_t b, size_t c) {  // TensorLayout::new_dyn with dynamic strides
+        return Lay3{{a, b, c}, {OPHIP_DYN_ISIZE, OPHIP_DYN_ISIZE, OPHIP_DYN_ISIZE}};
+    }
+    static Lay3 of(const ophip_tensor_layout &l) {
+        return Lay3{{l.shape[0], l.shape[1], l.shape[2]}, {l.strides[0], l.strides[1], l.strides[2]}};
+    }
+};
+
+// WorkspaceCollector (common/workspace.rs:54-90): bases first, then the largest sub-operator
+// need, each taken only while the running total still fits.
+struct WorkspaceCollector {
+    std::vector<size_t> base;
+    size_t sub_need = 0;
+    void push_base(size_t b) { base.push_back(b); }
+    void push_sub(size_t s) { sub_need = std::max(sub_need, s); }
+    size_t calculate(size_t max_ws) {
+        base.push_back(sub_need);
+        size_t ans = 0;
+        for (size_t s : base) {
+            if (s <= max_ws && ans <= max_ws - s) ans += s;
+            else return ans;
+        }
+        return ans;
+    }
+};
+
+struct AttentionMeta {
+    uint64_t dt;
+    size_t nh, nkvh, seq, att, dh;
+};
+
+// attention/args.rs:60-90
+AttentionMeta attention_meta(const ophip_attention_args &a) {
+    expect_rank(a.q_layout, "q", 3);
+    expect_rank(a.k_layout, "k", 3);
+    expect_rank(a.v_layout, "v", 3);
+    expect_rank(a.o_layout, "o", 3);
+    AttentionMeta m;
+    m.dt = type_distinct({a.q_layout.dt, a.k_layout.dt, a.v_layout.dt, a.o_layout.dt});
+    m.nh = dim_distinct({a.q_layout.shape[0], a.o_layout.shape[0]});
+    m.nkvh = dim_distinct({a.k_layout.shape[0], a.v_layout.shape[0]});
+    m.seq = dim_distinct({a.q_layout.shape[1], a.o_layout.shape[1]});
+    m.att = dim_distinct({a.k_layout.shape[1], a.v_layout.shape[1]});
+    m.dh = dim_distinct({a.q_layout.shape[2], a.k_layout.shape[2], a.v_layout.shape[2], a.o_layout.shape[2]});
+    return m;
+}
+
+}  // namespace
+
+struct ophip_attention {
+    ophip_device *dev;
+    ophip_mat_mul *mat_mul = nullptr;
+    ophip_fused_softmax *softmax = nullptr;
+    ophip_rearrange *rearrange = nullptr;
+    explicit ophip_attention(ophip_device *d) : dev(d) {
+        ophip_device_retain(d);
+        try {
+            sub(ophip_mat_mul_create(d, &mat_mul));
+            sub(ophip_fused_softmax_create(d, &softmax));
+            sub(ophip_rearrange_create(d, &rearrange));
+        } catch (...) {
+            release();
+            throw;
+        }
+    }
+    void release() {
+        ophip_mat_mul_destroy(mat_mul);
+        ophip_fused_softmax_destroy(softmax);
+        ophip_rearrange_destroy(rearrange);
+        ophip_device_release(dev);
+    }
+    ~ophip_attention() { release(); }
+    ophip_attention(const ophip_attention &) = delete;
+    ophip_attention &operator=(const ophip_attention &) = delete;
+};
+
+namespace {
+
+// Operator::scheme (attention/operator.rs:46-141)
+size_t attention_scheme(ophip_attention *op, const ophip_attention_args &args, size_t max_ws) {
+    const AttentionMeta m = attention_meta(args);
+    size_t need = 0;
+    WorkspaceCollector wc;
+    if (is_dyn(m.nh) || is_dyn(m.seq) || is_dyn(m.att) || is_dyn(m.dh)) {
+        // not all of nh, seq, att, dh known: initialise the operators with placeholders
+        const Lay3 any = Lay3::dyn(OPHIP_DYN_USIZE, OPHIP_DYN_USIZE, OPHIP_DYN_USIZE);
+        const ophip_mat_mul_args mm{any.tl(m.dt), nullptr, 1.f, any.tl(m.dt), nullptr, any.tl(m.dt), nullptr, 1.f};
+        sub(ophip_mat_mul_scheme(op->mat_mul, &mm, max_ws, &need));
+        wc.push_sub(need);
+        const Lay3 att = Lay3::dyn(m.nh, m.seq, m.att);
+        const ophip_fused_softmax_args sm{args.mask, att.tl(m.dt), nullptr};
+        sub(ophip_fused_softmax_scheme(op->softmax, &sm, max_ws, &need));
+        wc.push_sub(need);
+        const ophip_rearrange_args re{any.tl(m.dt), nullptr, any.tl(m.dt), nullptr};
+        sub(ophip_rearrange_scheme(op->rearrange, &re, max_ws, &need));
+        wc.push_sub(need);
+        return wc.calculate(max_ws);
+    }
+    const size_t ele = ophip_dtype_nbytes(m.dt);
+    const Lay3 att = Lay3::contiguous(m.dt, m.nh, m.seq, m.att);
+    const size_t q_size = m.nh * m.seq * m.dh * ele, att_size = m.nh * m.seq * m.att * ele;
+    const size_t rest = max_ws > q_size + att_size ? max_ws - (q_size + att_size) : 0;  // saturating_sub
+    wc.push_base(q_size);
+    wc.push_base(att_size);
+    // att = q . k^T
+    const ophip_mat_mul_args qk{att.tl(m.dt), nullptr, 0.f, args.q_layout, nullptr, args.k_layout, nullptr, 1.f};
+    sub(ophip_mat_mul_scheme(op->mat_mul, &qk, rest, &need));
+    wc.push_sub(need);
+    // att = softmax(att)
+    const ophip_fused_softmax_args sm{args.mask, att.tl(m.dt), nullptr};
+    sub(ophip_fused_softmax_scheme(op->softmax, &sm, rest, &need));
+    wc.push_sub(need);
+    // q = att . v
+    const ophip_mat_mul_args pv{args.q_layout, nullptr, 0.f, att.tl(m.dt), nullptr, args.v_layout, nullptr, 1.f};
+    sub(ophip_mat_mul_scheme(op->mat_mul, &pv, rest, &need));
+    wc.push_sub(need);
+    // o = rearrange(q)
+    const ophip_rearrange_args re{args.o_layout, nullptr, args.q_layout, nullptr};
+    sub(ophip_rearrange_scheme(op->rearrange, &re, rest, &need));
+    wc.push_sub(need);
+    return wc.calculate(max_ws);
+}
+
+// Operator::launch (attention/operator.rs:143-277).  q is overwritten with att . v, as in
+// the reference, unless it had to be copied into the workspace first.
+void attention_launch(const ophip_attention *op, const ophip_attention_args &args, void *workspace,
+                      size_t workspace_len, const ophip_queue_alloc *qa) {
+    const AttentionMeta m = attention_meta(args);
+    const uint64_t dt = m.dt;
+    const size_t ele = ophip_dtype_nbytes(dt);
+    const size_t nh = static_of(m.nh), seq = static_of(m.seq), dh = static_of(m.dh);
+    const ptrdiff_t nh_sq = static_of(args.q_layout.strides[0]), seq_sq = static_of(args.q_layout.strides[1]),
+                    dh_sq = static_of(args.q_layout.strides[2]);
+    const size_t nkvh = static_of(m.nkvh), att = static_of(m.att);
+    const ptrdiff_t nkvh_sk = static_of(args.k_layout.strides[0]), att_sk = static_of(args.k_layout.strides[1]),
+                    dh_sk = static_of(args.k_layout.strides[2]);
+    if (nkvh == 0 || nh % nkvh != 0) throw shape_mismatch("nh must be a multiple of nkvh");
+
+    // ArrayLayout::merge_be(0, 2) of ndarray-layout: heads and tokens fold into one dimension
+    // when the head stride is seq * token stride (a dimension of length 1 folds with anything)
+    const bool merged = nh == 1 || seq == 1 || nh_sq == (ptrdiff_t)seq * seq_sq;
+    const ptrdiff_t row_sq = seq == 1 ? nh_sq : seq_sq;  // stride of the merged [nh * seq] dimension
+    // k^T: ArrayLayout::transpose(&[2, 1])
+    const Lay3 kt{{nkvh, dh, att}, {nkvh_sk, dh_sk, att_sk}};
+
+    const size_t q_size = merged ? 0 : nh * seq * dh * ele;
+    const size_t att_size = nh * seq * att * ele;
+    Workspace ws(qa, workspace, workspace_len, q_size + att_size);
+    char *q_buf = static_cast<char *>(ws.ptr());
+    char *att_buf = q_buf + q_size;
+    // what is left of a caller-provided workspace goes to the sub-operators
+    const bool ext = ws.ptr() == workspace && workspace_len >= q_size + att_size;
+    void *rest = ext ? att_buf + att_size : nullptr;
+    const size_t rest_len = ext ? workspace_len - (q_size + att_size) : 0;
+
+    const size_t head_group = nh / nkvh;
+    Lay3 q_lay, qx_lay;
+    void *q_base;
+    if (!merged) {
+        q_lay = Lay3::contiguous(dt, nh, seq, dh);
+        qx_lay = Lay3::contiguous(dt, nkvh, head_group * seq, dh);
+        q_base = q_buf;
+        const ophip_rearrange_args re{q_lay.tl(dt), q_base, args.q_layout, args.q_base};
+        sub(ophip_rearrange_launch(op->rearrange, &re, rest, rest_len, qa));
+    } else {
+        // tile_be(0, &[nkvh, head_group * seq]) of the merged dimension
+        q_lay = Lay3::of(args.q_layout);
+        qx_lay = Lay3{{nkvh, head_group * seq, dh}, {(ptrdiff_t)(head_group * seq) * row_sq, row_sq, dh_sq}};
+        q_base = args.q_base;
+    }
+    const Lay3 att_mm = Lay3::contiguous(dt, nkvh, head_group * seq, att);
+    const Lay3 att_sm = Lay3::contiguous(dt, nh, seq, att);
+
+    // att = q . k^T
+    const ophip_mat_mul_args qk{att_mm.tl(dt), att_buf, 0.f, qx_lay.tl(dt), q_base, kt.tl(dt), args.k_base,
+                                1.0f / std::sqrt((float)dh)};
+    sub(ophip_mat_mul_launch(op->mat_mul, &qk, rest, rest_len, qa));
+    // att = softmax(att)
+    const ophip_fused_softmax_args sm{args.mask, att_sm.tl(dt), att_buf};
+    sub(ophip_fused_softmax_launch(op->softmax, &sm, rest, rest_len, qa));
+    // q = att . v
+    const ophip_mat_mul_args pv{qx_lay.tl(dt), q_base, 0.f, att_mm.tl(dt), att_buf, args.v_layout, args.v_base, 1.f};
+    sub(ophip_mat_mul_launch(op->mat_mul, &pv, rest, rest_len, qa));
+    // o = rearrange(q)
+    if (q_base != args.o_base) {
+        const ophip_rearrange_args re{args.o_layout, args.o_base, q_lay.tl(dt), q_base};
+        sub(ophip_rearrange_launch(op->rearrange, &re, rest, rest_len, qa));
+    }
+}
+
+}  // namespace
+
+struct ophip_attention_kv_cached {
+    ophip_device *dev;
+    ophip_rearrange *rearrange = nullptr;
+    ophip_attention *attention = nullptr;
+    explicit ophip_attention_kv_cached(ophip_device *d) : dev(d) {
+        ophip_device_retain(d);
+        try {
+            sub(ophip_rearrange_create(d, &rearrange));
+            sub(ophip_attention_create(d, &attention));
+        } catch (...) {
+            release();
+            throw;
+        }
+    }
+    void release() {
+        ophip_rearrange_destroy(rearrange);
+        ophip_attention_destroy(attention);
+        ophip_device_release(dev);
+    }
+    ~ophip_attention_kv_cached() { release(); }
+    ophip_attention_kv_cached(const ophip_attention_kv_cached &) = delete;
+    ophip_attention_kv_cached &operator=(const ophip_attention_kv_cached &) = delete;
+};
+
+namespace {
+
+struct KvCachedMeta {
+    uint64_t dt;
+    size_t nh, nkvh, dh, seq;
+};
+
+// attention_kv_cached/args.rs:72-115
+KvCachedMeta kv_cached_meta(const ophip_attention_kv_cached_args &a) {
+    expect_rank(a.q_layout, "q", 3);
+    expect_rank(a.k_layout, "k", 3);
+    expect_rank(a.v_layout, "v", 3);
+    expect_rank(a.o_layout, "o", 3);
+    expect_rank(a.k_cache_layout, "k_cache", 3);
+    expect_rank(a.v_cache_layout, "v_cache", 3);
+    KvCachedMeta m;
+    m.dt = type_distinct({a.q_layout.dt, a.k_layout.dt, a.v_layout.dt, a.o_layout.dt, a.k_cache_layout.dt,
+                          a.v_cache_layout.dt});
+    m.nh = dim_distinct({a.q_layout.shape[0], a.o_layout.shape[0]});
+    m.nkvh = dim_distinct({a.k_layout.shape[0], a.v_layout.shape[0], a.k_cache_layout.shape[0],
+                           a.v_cache_layout.shape[0]});
+    m.dh = dim_distinct({a.q_layout.shape[2], a.k_layout.shape[2], a.v_layout.shape[2], a.o_layout.shape[2],
+                         a.k_cache_layout.shape[2], a.v_cache_layout.shape[2]});
+    m.seq = dim_distinct({a.q_layout.shape[1], a.k_layout.shape[1], a.v_layout.shape[1], a.o_layout.shape[1]});
+    return m;
+}
+
+// Operator::scheme (attention_kv_cached/operator.rs:42-77)
+size_t kv_cached_scheme(ophip_attention_kv_cached *op, const ophip_attention_kv_cached_args &args, size_t max_ws) {
+    const KvCachedMeta m = kv_cached_meta(args);
+    WorkspaceCollector wc;
+    size_t need = 0;
+    const Lay3 any = Lay3::dyn(OPHIP_DYN_USIZE, OPHIP_DYN_USIZE, OPHIP_DYN_USIZE);
+    const ophip_rearrange_args re{any.tl(m.dt), nullptr, any.tl(m.dt), nullptr};
+    sub(ophip_rearrange_scheme(op->rearrange, &re, max_ws, &need));
+    wc.push_sub(need);
+    const size_t att = (!is_dyn(m.seq) && !is_dyn(args.pos)) ? args.pos + m.seq : OPHIP_DYN_USIZE;
+    // attention::Args::new_null(mask, dt, nh, nkvh, seq, att, dh): every stride dynamic
+    const Lay3 qo = Lay3::dyn(m.nh, m.seq, m.dh), kv = Lay3::dyn(m.nkvh, att, m.dh);
+    ophip_attention_args at{};
+    at.q_layout = at.o_layout = qo.tl(m.dt);
+    at.k_layout = at.v_layout = kv.tl(m.dt);
+    at.mask = args.mask;
+    need = attention_scheme(op->attention, at, max_ws);
+    wc.push_sub(need);
+    return wc.calculate(max_ws);
+}
+
+// Operator::launch (attention_kv_cached/operator.rs:79-183).  As in the reference, the
+// v-cache view takes its strides from k_cache_layout (operator.rs:114) and the appended v
+// rows land at the k-cache's byte offset (operator.rs:156): the two caches are expected to
+// share one layout.
+void kv_cached_launch(const ophip_attention_kv_cached *op, const ophip_attention_kv_cached_args &args,
+                      void *workspace, size_t workspace_len, const ophip_queue_alloc *qa) {
+    const KvCachedMeta m = kv_cached_meta(args);
+    const size_t pos = static_of(args.pos), seq = static_of(m.seq);
+    const size_t buf_k = static_of(args.k_cache_layout.shape[1]);
+    const size_t nkvh = static_of(m.nkvh), buf_v = static_of(args.v_cache_layout.shape[1]), dh = static_of(m.dh);
+    const ptrdiff_t nkvh_skc = static_of(args.k_cache_layout.strides[0]),
+                    buf_skc = static_of(args.k_cache_layout.strides[1]),
+                    dh_skc = static_of(args.k_cache_layout.strides[2]);
+    const ptrdiff_t nkvh_svc = nkvh_skc, buf_svc = buf_skc, dh_svc = dh_skc;
+
+    // cache capacity
+    const size_t att = pos + seq;
+    if (buf_k < att || buf_v < att) throw shape_mismatch("Out of cache buffer");
+    // concatenate the new rows onto the caches: slice(1, pos, 1, seq)
+    const Lay3 k_cat{{nkvh, seq, dh}, {nkvh_skc, buf_skc, dh_skc}};
+    const Lay3 v_cat{{nkvh, seq, dh}, {nkvh_svc, buf_svc, dh_svc}};
+    const ptrdiff_t cat_offset = (ptrdiff_t)pos * buf_skc;
+    const ophip_rearrange_args rk{k_cat.tl(m.dt), static_cast<char *>(args.k_cache_base) + cat_offset, args.k_layout,
+                                  args.k_base};
+    sub(ophip_rearrange_launch(op->rearrange, &rk, workspace, workspace_len, qa));
+    const ophip_rearrange_args rv{v_cat.tl(m.dt), static_cast<char *>(args.v_cache_base) + cat_offset, args.v_layout,
+                                  args.v_base};
+    sub(ophip_rearrange_launch(op->rearrange, &rv, workspace, workspace_len, qa));
+    // attention over rows [0, att) of the caches
+    const Lay3 k_all{{nkvh, att, dh}, {nkvh_skc, buf_skc, dh_skc}};
+    const Lay3 v_all{{nkvh, att, dh}, {nkvh_svc, buf_svc, dh_svc}};
+    ophip_attention_args at{};
+    at.q_layout = args.q_layout;
+    at.q_base = args.q_base;
+    at.k_layout = k_all.tl(m.dt);
+    at.k_base = args.k_cache_base;
+    at.v_layout = v_all.tl(m.dt);
+    at.v_base = args.v_cache_base;
+    at.o_layout = args.o_layout;
+    at.o_base = args.o_base;
+    at.mask = args.mask;
+    attention_launch(op->attention, at, workspace, workspace_len, qa);
+}
+
+}  // namespace
+
+extern "C" {
+
+int ophip_attention_create(ophip_device *dev, ophip_attention **out) {
+    return guard([&] {
+        if (!dev || !out) throw args_not_support("null argument");
+        *out = new ophip_attention(dev);
+    });
+}
+void ophip_attention_destroy(ophip_attention *op) { delete op; }
+
+int ophip_attention_scheme(ophip_attention *op, const ophip_attention_args *args, size_t max_ws, size_t *ws) {
+    return guard([&] {
+        if (ws) *ws = 0;
+        if (!op || !args) throw args_not_support("null argument");
+        const size_t need = attention_scheme(op, *args, max_ws);
+        if (ws) *ws = need;
+    });
+}
+
+int ophip_attention_launch(const ophip_attention *op, const ophip_attention_args *args, void *workspace,
+                           size_t workspace_len, const ophip_queue_alloc *qa) {
+    return guard([&] {
+        if (!op || !args) throw args_not_support("null argument");
+        attention_launch(op, *args, workspace, workspace_len, qa);
+    });
+}
+
+int ophip_attention_kv_cached_create(ophip_device *dev, ophip_attention_kv_cached **out) {
+    return guard([&] {
+        if (!dev || !out) throw args_not_support("null argument");
+        *out = new ophip_attention_kv_cached(dev);
+    });
+}
+void ophip_attention_kv_cached_destroy(ophip_attention_kv_cached *op) { delete op; }
+
+int ophip_attention_kv_cached_scheme(ophip_attention_kv_cached *op, const ophip_attention_kv_cached_args *args,
+                                     size_t max_ws, size_t *ws) {
+    return guard([&] {
+        if (ws) *ws = 0;
+        if (!op || !args) throw args_not_support("null argument");
+        const size_t need = kv_cached_scheme(op, *args, max_ws);
+        if (ws) *ws = need;
+    });
+}
+
+int ophip_attention_kv_cached_launch(const ophip_attention_kv_cached *op, const ophip_attention_kv_cached_args *args,
+                                     void *workspace, size_t workspace_len, const ophip_queue_alloc *qa) {
+    return guard([&] {
+        if (!op || !args) throw args_not_support("null argument");
+        kv_cached_launch(op, *args, workspace, workspace_len, qa);
+    });
+}
+
+}  // extern "C"

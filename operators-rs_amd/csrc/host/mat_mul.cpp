@@ -299,21 +299,22 @@ int ophip_mat_mul_create(ophip_device *dev, ophip_mat_mul **out) {
 }
 void ophip_mat_mul_destroy(ophip_mat_mul *op) { delete op; }
 
-// The reference's scheme() prepares nothing (mat_mul/cuda/mod.rs:30-37).  Here it
-// also reports the split-K workspace when every shape is already known.
+// The reference's scheme() prepares nothing and never fails (mat_mul/cuda/mod.rs:30-37): the
+// composites rely on that and hand it layouts that are not even a valid product
+// (attention/operator.rs:104-128 passes q and the untransposed k).  Here it additionally
+// reports the split-K workspace when the arguments already describe a launchable product;
+// anything else is left for launch() to judge.
 int ophip_mat_mul_scheme(ophip_mat_mul *op, const ophip_mat_mul_args *args, size_t max_ws, size_t *ws) {
     return guard([&] {
         if (ws) *ws = 0;
-        ophip_mat_mul_layout L;
+        if (!op || !args) return;
         try {
-            L = mat_mul_layout(*args);
-        } catch (const Error &e) {
-            if (e.kind == OPHIP_DYNAMIC_NOT_SUPPORT) return;  // decide at launch
-            throw;
+            const ophip_mat_mul_layout L = mat_mul_layout(*args);
+            if (L.dt != OPHIP_DT_F16 && L.dt != OPHIP_DT_F32) return;
+            const GemmPlan g = make_plan(*args, L, (unsigned)op->dev->props.multiProcessorCount);
+            if (ws && g.workspace <= max_ws) *ws = g.workspace;
+        } catch (const Error &) {
         }
-        if (L.dt != OPHIP_DT_F16 && L.dt != OPHIP_DT_F32) throw type_not_support("mat_mul supports f16 and f32");
-        const GemmPlan g = make_plan(*args, L, (unsigned)op->dev->props.multiProcessorCount);
-        if (ws && g.workspace <= max_ws) *ws = g.workspace;
     });
 }
 

@@ -42,10 +42,10 @@ __device__ __forceinline__ void skinny_load_q(const GemmParams &p, const f16 *qb
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
         if constexpr (QMODE == 0) {
-            w[r] = ld128(qb + (int64_t)(kb + 8 * g + r) * p.q_sl + colc);
+            w[r] = ld128_nt(qb + (int64_t)(kb + 8 * g + r) * p.q_sl + colc);
         } else {
             const uint32_t col = min(colc + r, p.N - 1);
-            w[r] = ld128(qb + (int64_t)col * p.q_sj + (kb + 8 * g));
+            w[r] = ld128_nt(qb + (int64_t)col * p.q_sj + (kb + 8 * g));
         }
     }
 }
@@ -58,10 +58,10 @@ __device__ __forceinline__ void skinny_load_q_tail(const GemmParams &p, const f1
         w[r] = u32x4{0, 0, 0, 0};
         if constexpr (QMODE == 0) {
             const uint32_t k = kb + 8 * g + r;
-            if (k < kend) w[r] = ld128(qb + (int64_t)k * p.q_sl + colc);
+            if (k < kend) w[r] = ld128_nt(qb + (int64_t)k * p.q_sl + colc);
         } else {
             const uint32_t k = kb + 8 * g, col = min(colc + r, p.N - 1);
-            if (k < kend) w[r] = ld128(qb + (int64_t)col * p.q_sj + k);
+            if (k < kend) w[r] = ld128_nt(qb + (int64_t)col * p.q_sj + k);
         }
     }
 }

@@ -154,6 +154,19 @@ class DeviceInfo(ctypes.Structure):
 
 class KVPair(ctypes.Structure):
     _fields_ = [("idx", ctypes.c_uint32), ("val", ctypes.c_uint32)]
+class _AttentionArgs(ctypes.Structure):
+    _fields_ = [("q_layout", _Layout), ("q_base", ctypes.c_void_p), ("k_layout", _Layout),
+                ("k_base", ctypes.c_void_p), ("v_layout", _Layout), ("v_base", ctypes.c_void_p),
+                ("o_layout", _Layout), ("o_base", ctypes.c_void_p), ("mask", ctypes.c_uint8)]
+
+
+class _AttnKVCachedArgs(ctypes.Structure):
+    _fields_ = [("q_layout", _Layout), ("q_base", ctypes.c_void_p), ("k_layout", _Layout),
+                ("k_base", ctypes.c_void_p), ("v_layout", _Layout), ("v_base", ctypes.c_void_p),
+                ("o_layout", _Layout), ("o_base", ctypes.c_void_p),
+                ("k_cache_layout", _Layout), ("k_cache_base", ctypes.c_void_p),
+                ("v_cache_layout", _Layout), ("v_cache_base", ctypes.c_void_p),
+                ("mask", ctypes.c_uint8), ("pos", ctypes.c_size_t)]
 
 
 # every symbol include/ophip.h declares
@@ -182,6 +195,9 @@ EXPORTS = [
     "ophip_random_sample_destroy", "ophip_random_sample_build_indices", "ophip_random_sample_launch_batch",
     "ophip_mat_mul_plan", "ophip_mat_mul_create", "ophip_mat_mul_scheme", "ophip_mat_mul_launch",
     "ophip_mat_mul_destroy", "ophip_mat_mul_describe",
+    "ophip_attention_create", "ophip_attention_scheme", "ophip_attention_launch", "ophip_attention_destroy",
+    "ophip_attention_kv_cached_create", "ophip_attention_kv_cached_scheme", "ophip_attention_kv_cached_launch",
+    "ophip_attention_kv_cached_destroy",
 ]
 
 _lib = None
@@ -577,6 +593,39 @@ class MatMulArgs:
         return out
 
 
+class AttentionArgs:
+    """attention/args.rs:10-24"""
+
+    def __init__(self, q_layout, q_base, k_layout, k_base, v_layout, v_base, o_layout, o_base, mask):
+        self.__dict__.update(locals())
+
+    def c(self):
+        return _AttentionArgs(self.q_layout.c(), _p(self.q_base), self.k_layout.c(), _p(self.k_base),
+                              self.v_layout.c(), _p(self.v_base), self.o_layout.c(), _p(self.o_base), self.mask)
+
+    @classmethod
+    def new_null(cls, mask, dtype, nh, nkvh, seq, att, dh):
+        """Args::new_null (attention/args.rs:36-58): shapes only, every stride dynamic."""
+        qo = TensorLayout(dtype, [nh, seq, dh], [None] * 3)
+        kv = TensorLayout(dtype, [nkvh, att, dh], [None] * 3)
+        return cls(qo, None, kv, None, kv, None, qo, None, mask)
+
+
+class AttnKVCachedArgs:
+    """attention_kv_cached/args.rs:8-30; pos = None is dynamic."""
+
+    def __init__(self, q_layout, q_base, k_layout, k_base, v_layout, v_base, o_layout, o_base,
+                 k_cache_layout, k_cache_base, v_cache_layout, v_cache_base, mask, pos):
+        self.__dict__.update(locals())
+
+    def c(self):
+        return _AttnKVCachedArgs(self.q_layout.c(), _p(self.q_base), self.k_layout.c(), _p(self.k_base),
+                                 self.v_layout.c(), _p(self.v_base), self.o_layout.c(), _p(self.o_base),
+                                 self.k_cache_layout.c(), _p(self.k_cache_base),
+                                 self.v_cache_layout.c(), _p(self.v_cache_base), self.mask,
+                                 DYN_USIZE if self.pos is None else self.pos)
+
+
 class RmsNorm(_Operator):
     NAME = "rms_norm"
 
@@ -621,6 +670,14 @@ class Rearrange(_Operator):
 
 class Swiglu(_Operator):
     NAME = "swiglu"
+
+
+class Attention(_Operator):
+    NAME = "attention"
+
+
+class AttnKVCached(_Operator):
+    NAME = "attention_kv_cached"
 
 
 class RandomSample(_Operator):

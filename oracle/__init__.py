@@ -225,3 +225,56 @@ def mat_mul(c, beta, a, b, alpha):
     L = mat_mul_layout(c.dtype.itemsize, (c.shape, c.strides), (a.shape, a.strides), (b.shape, b.strides))
     _check(lib().oracle_mat_mul(_ptr(c), beta, _ptr(a), _ptr(b), alpha, ctypes.byref(L), _DT[c.dtype]))
     return c
+
+
+def _heads_and_tokens_merge(q):
+    """ArrayLayout::merge_be(0, 2) as attention/operator.rs:186 uses it: can q[nh, seq, dh] be
+    viewed as [nh * seq, dh]?  (The layout crate, ndarray-layout, is not part of the reference
+    tree; a dimension of length 1 is taken to merge with anything.  The choice only decides
+    whether q is staged in workspace - the outputs are the same either way.)"""
+    nh, seq, _ = q.shape
+    return nh == 1 or seq == 1 or q.strides[0] == seq * q.strides[1]
+
+
+def attention(q, k, v, o, causal=True):
+    """The attention composite (attention/operator.rs:143-277) over the CPU restatements:
+    q, o [nh, seq, dh]; k, v [nkvh, att, dh] as numpy views.  att = q . k^T / sqrt(dh) per
+    kv-head group, masked softmax, q <- att . v, o <- q.  Like the reference, q itself is
+    overwritten when its heads and tokens merge into one dimension."""
+    nh, seq, dh = q.shape
+    nkvh, att, _ = k.shape
+    assert nh % nkvh == 0
+    group = nh // nkvh
+    if _heads_and_tokens_merge(q):
+        rows = np.lib.stride_tricks.as_strided(
+            q, (nh * seq, dh), (q.strides[0] if seq == 1 else q.strides[1], q.strides[2]))
+        qx = np.lib.stride_tricks.as_strided(
+            rows, (nkvh, group * seq, dh), (group * seq * rows.strides[0], rows.strides[0], rows.strides[1]))
+        q_work = q
+    else:
+        q_work = np.empty((nh, seq, dh), q.dtype)
+        rearrange(q_work, q)
+        qx = q_work.reshape(nkvh, group * seq, dh)
+    att_buf = np.zeros((nkvh, group * seq, att), q.dtype)
+    alpha = float(np.float32(1.0) / np.sqrt(np.float32(dh)))
+    mat_mul(att_buf, 0.0, qx, k.transpose(0, 2, 1), alpha)
+    fused_softmax(att_buf.reshape(nh, seq, att), causal=causal)
+    mat_mul(qx, 0.0, att_buf, v, 1.0)
+    if q_work is not o:
+        rearrange(o, q_work)
+    return o
+
+
+def attention_kv_cached(q, k, v, o, k_cache, v_cache, pos, causal=True):
+    """attention_kv_cached/operator.rs:79-183: k, v [nkvh, seq, dh] are copied into rows
+    [pos, pos + seq) of the caches [nkvh, buf, dh], then attention runs over rows
+    [0, pos + seq).  Both caches must share one layout (the reference addresses the v-cache
+    with the k-cache's strides)."""
+    seq = q.shape[1]
+    att = pos + seq
+    if k_cache.shape[1] < att or v_cache.shape[1] < att:
+        raise OracleError(6)  # ShapeMismatch: "Out of cache buffer"
+    assert k_cache.strides == v_cache.strides
+    rearrange(k_cache[:, pos:att], k)
+    rearrange(v_cache[:, pos:att], v)
+    return attention(q, k_cache[:, :att], v_cache[:, :att], o, causal=causal)

@@ -1,0 +1,174 @@
+"""attention and attention_kv_cached on the HIP backend against the oracle's composites,
+through the C ABI.  Shapes: the reference's device test (attention/cuda.rs:97-160:
+nh 32, nkvh 4, seq 7, att 127, dh 64), its kv-cached counterpart, and the Llama-7B decode
+layer (q and o as strided views of the fused QKV / token-major buffers)."""
+import numpy as np
+import pytest
+
+import ophip
+import oracle
+from helpers import assert_close_f16, normal_f16
+from ophip import TensorLayout, dt
+
+pytestmark = pytest.mark.gpu
+
+f16 = np.float16
+CAUSAL, NONE = ophip.AttnMask.CAUSAL, ophip.AttnMask.NONE
+
+
+def say(msg):
+    print(msg, flush=True)
+
+
+def attention_f64(q, k, v, causal):
+    nh, seq, dh = q.shape
+    nkvh, att, _ = k.shape
+    g = nh // nkvh
+    kk, vv = np.repeat(k.astype(np.float64), g, axis=0), np.repeat(v.astype(np.float64), g, axis=0)
+    s = np.einsum("hsd,had->hsa", q.astype(np.float64), kk) / np.sqrt(dh)
+    if causal:
+        keep = np.arange(att)[None, :] <= (att - seq + np.arange(seq))[:, None]
+        s = np.where(keep[None], s, -np.inf)
+    p = np.exp(s - s.max(-1, keepdims=True))
+    p /= p.sum(-1, keepdims=True)
+    return np.einsum("hsa,had->hsd", p, vv)
+
+
+def upload(gpu, a):
+    return gpu.from_host(np.ascontiguousarray(a))
+
+
+def download(gpu, stream, mem, like):
+    return gpu.to_host(mem, like.dtype, like.size, stream=stream).reshape(like.shape)
+
+
+@pytest.mark.parametrize("nh,nkvh,seq,att,dh,mask", [(32, 4, 7, 127, 64, CAUSAL), (8, 8, 33, 33, 128, CAUSAL),
+                                                     (6, 2, 3, 40, 16, NONE), (4, 1, 1, 300, 64, CAUSAL)])
+def test_attention_contiguous(gpu, stream, nh, nkvh, seq, att, dh, mask):
+    rng = np.random.default_rng(nh * 1000 + att)
+    q, k, v = (rng.random(s).astype(f16) for s in ((nh, seq, dh), (nkvh, att, dh), (nkvh, att, dh)))
+    qd, kd, vd = upload(gpu, q), upload(gpu, k), upload(gpu, v)
+    od = gpu.malloc(q.nbytes)
+    op = ophip.Attention(gpu)
+    lay = TensorLayout.of
+    args = ophip.AttentionArgs(lay(q), qd, lay(k), kd, lay(v), vd, lay(q), od, mask)
+    need = op.scheme(args, 2 ** 40)
+    assert need >= (nh * seq * dh + nh * seq * att) * 2
+    say("attention nh=%d nkvh=%d seq=%d att=%d dh=%d" % (nh, nkvh, seq, att, dh))
+    op.launch(args, None, stream)
+    out = download(gpu, stream, od, q)
+    q_after = download(gpu, stream, qd, q)
+    ref = oracle.attention(q.copy(), k, v, np.zeros_like(q), causal=(mask == CAUSAL))
+    assert_close_f16(out, ref, "attention vs oracle")
+    assert_close_f16(out, attention_f64(q, k, v, mask == CAUSAL), "attention vs f64")
+    assert np.array_equal(q_after, out)  # q receives att . v, as in the reference
+
+
+def test_attention_decode_layer_views(gpu, stream):
+    """Llama-7B decode: q is the [token, head, dh] slice of the [16, 12288] QKV buffer viewed head-major,
+    o the same view of a [16, 4096] buffer, k / v the first 2048 rows of [32, 2048, 128] caches."""
+    rng = np.random.default_rng(16)
+    nt, nh, dh, att = 16, 32, 128, 2048
+    qkv = normal_f16(rng, (nt, 3 * nh * dh))
+    k, v = normal_f16(rng, (nh, att, dh)), normal_f16(rng, (nh, att, dh))
+    qkv_d, kd, vd = upload(gpu, qkv), upload(gpu, k), upload(gpu, v)
+    obuf = np.zeros((nt, nh * dh), f16)
+    od = upload(gpu, obuf)
+    q_lay = TensorLayout(dt.F16, [nh, nt, dh], [dh * 2, 3 * nh * dh * 2, 2])
+    o_lay = TensorLayout(dt.F16, [nh, nt, dh], [dh * 2, nh * dh * 2, 2])
+    op = ophip.Attention(gpu)
+    args = ophip.AttentionArgs(q_lay, qkv_d, TensorLayout.of(k), kd, TensorLayout.of(v), vd, o_lay, od, CAUSAL)
+    need = op.scheme(args, 2 ** 40)
+    ws = gpu.malloc(need)
+    pool = ophip.StreamMemPool(gpu, stream)
+    pool.put(need + (1 << 20))
+    q_view = qkv[:, :nh * dh].reshape(nt, nh, dh).transpose(1, 0, 2)
+    ref = oracle.attention(q_view, k, v, np.zeros((nt, nh * dh), f16).reshape(nt, nh, dh).transpose(1, 0, 2))
+    for label, w, qa in (("own workspace", ws, stream), ("stream allocator", None, stream), ("pool", None, pool)):
+        say("attention decode views, %s" % label)
+        gpu.memset(od, 0)
+        op.launch(args, w, qa)
+        out = download(gpu, stream, od, obuf).reshape(nt, nh, dh).transpose(1, 0, 2)
+        assert_close_f16(out, ref, "attention decode " + label)
+    assert np.array_equal(download(gpu, stream, qkv_d, qkv), qkv)  # a staged q is left alone
+
+
+def test_attention_scheme_workspace_rules(gpu):
+    """WorkspaceCollector (common/workspace.rs:54-90): q, att, then the largest sub-operator need,
+    each added only while the total still fits; unknown shapes plan nothing."""
+    op = ophip.Attention(gpu)
+    nh, nkvh, seq, att, dh = 32, 4, 7, 127, 64
+    c = lambda *s: TensorLayout.new_contiguous(dt.F16, list(s))
+    args = ophip.AttentionArgs(c(nh, seq, dh), None, c(nkvh, att, dh), None, c(nkvh, att, dh), None, c(nh, seq, dh),
+                               None, CAUSAL)
+    q_size, att_size = nh * seq * dh * 2, nh * seq * att * 2
+    assert op.scheme(args, 2 ** 40) >= q_size + att_size
+    assert op.scheme(args, q_size + att_size) == q_size + att_size
+    assert op.scheme(args, q_size + att_size - 1) == q_size
+    assert op.scheme(args, q_size - 1) == 0
+    dyn = ophip.AttentionArgs.new_null(CAUSAL, dt.F16, 32, None, 7, 127, None)  # attention/cuda.rs:10-21
+    assert op.scheme(dyn, 2 ** 40) == 0
+
+
+def test_attention_errors(gpu, stream):
+    op = ophip.Attention(gpu)
+    c = lambda d, *s: TensorLayout.new_contiguous(d, list(s))
+    F = dt.F16
+    with pytest.raises(ophip.SchemeError) as e:
+        op.scheme(ophip.AttentionArgs(c(F, 4, 8), None, c(F, 4, 3, 8), None, c(F, 4, 3, 8), None, c(F, 4, 2, 8), None,
+                                      CAUSAL), 0)
+    assert e.value.kind == "RankNotSupport"
+    with pytest.raises(ophip.SchemeError) as e:
+        op.scheme(ophip.AttentionArgs(c(F, 4, 2, 8), None, c(F, 4, 3, 8), None, c(dt.F32, 4, 3, 8), None,
+                                      c(F, 4, 2, 8), None, CAUSAL), 0)
+    assert e.value.kind == "TypeMismatch"
+    with pytest.raises(ophip.SchemeError) as e:
+        op.scheme(ophip.AttentionArgs(c(F, 4, 2, 8), None, c(F, 4, 3, 8), None, c(F, 4, 3, 16), None, c(F, 4, 2, 8),
+                                      None, CAUSAL), 0)
+    assert e.value.kind == "ShapeMismatch"
+    with pytest.raises(ophip.LaunchError) as e:
+        op.launch(ophip.AttentionArgs.new_null(CAUSAL, F, 32, 4, None, 127, 64), None, stream)
+    assert e.value.kind == "DynamicNotSupport"
+
+
+@pytest.mark.parametrize("nh,nkvh,seq,dh,buf,pos", [(32, 4, 7, 64, 160, 120), (32, 32, 16, 128, 2048, 2032),
+                                                    (8, 2, 1, 32, 50, 0)])
+def test_attention_kv_cached(gpu, stream, nh, nkvh, seq, dh, buf, pos):
+    rng = np.random.default_rng(nh + buf + pos)
+    q, k, v = normal_f16(rng, (nh, seq, dh)), normal_f16(rng, (nkvh, seq, dh)), normal_f16(rng, (nkvh, seq, dh))
+    kc, vc = normal_f16(rng, (nkvh, buf, dh)), normal_f16(rng, (nkvh, buf, dh))
+    qd, kd, vd, kcd, vcd = (upload(gpu, a) for a in (q, k, v, kc, vc))
+    od = gpu.malloc(q.nbytes)
+    lay = TensorLayout.of
+    op = ophip.AttnKVCached(gpu)
+    args = ophip.AttnKVCachedArgs(lay(q), qd, lay(k), kd, lay(v), vd, lay(q), od, lay(kc), kcd, lay(vc), vcd, CAUSAL, pos)
+    op.scheme(args, 2 ** 40)
+    say("attention_kv_cached nh=%d nkvh=%d seq=%d dh=%d buf=%d pos=%d" % (nh, nkvh, seq, dh, buf, pos))
+    op.launch(args, None, stream)
+    out = download(gpu, stream, od, q)
+    kc_ref, vc_ref = kc.copy(), vc.copy()
+    ref = oracle.attention_kv_cached(q.copy(), k, v, np.zeros_like(q), kc_ref, vc_ref, pos)
+    assert np.array_equal(download(gpu, stream, kcd, kc), kc_ref)  # caches: appended rows exact, rest untouched
+    assert np.array_equal(download(gpu, stream, vcd, vc), vc_ref)
+    assert_close_f16(out, ref, "attention_kv_cached vs oracle")
+    assert_close_f16(out, attention_f64(q, kc_ref[:, :pos + seq], vc_ref[:, :pos + seq], True), "kv cached vs f64")
+
+
+def test_attention_kv_cached_errors_and_scheme(gpu, stream):
+    op = ophip.AttnKVCached(gpu)
+    c = lambda *s: TensorLayout.new_contiguous(dt.F16, list(s))
+    mk = lambda pos, buf=16: ophip.AttnKVCachedArgs(c(8, 3, 32), None, c(2, 3, 32), None, c(2, 3, 32), None, c(8, 3, 32),
+                                                    None, c(2, buf, 32), None, c(2, buf, 32), None, CAUSAL, pos)
+    assert op.scheme(mk(None), 2 ** 40) == 0   # position unknown: nothing planned (attention/… new_null, att dynamic)
+    assert op.scheme(mk(5), 2 ** 40) >= (8 * 3 * 32 + 8 * 3 * 8) * 2
+    with pytest.raises(ophip.LaunchError) as e:
+        op.launch(mk(14), None, stream)   # 14 + 3 > 16
+    assert e.value.kind == "ShapeMismatch"
+    with pytest.raises(ophip.LaunchError) as e:
+        op.launch(mk(None), None, stream)
+    assert e.value.kind == "DynamicNotSupport"
+    bad = mk(0)
+    bad.v_cache_layout = c(3, 16, 32)
+    with pytest.raises(ophip.SchemeError) as e:
+        op.scheme(bad, 0)
+    assert e.value.kind == "ShapeMismatch"

@@ -83,7 +83,8 @@ def test_rms_norm_reference_sweep_f32_weights(gpu, stream, k):
 
 @pytest.mark.parametrize("n,d,dta,dtw", [(4096, 4096, f16, f16), (3, 16384, f16, f16), (5, 80000, f16, f32),
                                           (7, 1000, f16, f16), (9, 4095, f16, f32), (300, 4096, f32, f32),
-                                          (2, 130, f32, f32), (1, 8, f16, f16), (33, 2048, f16, f16)])
+                                          (2, 130, f32, f32), (1, 8, f16, f16), (33, 2048, f16, f16),
+                                          (20001, 1024, f16, f16), (17000, 1024, f16, f32)])  # the last two: one wave streaming many rows
 def test_rms_norm_shapes_and_types(gpu, stream, n, d, dta, dtw):
     rng = np.random.default_rng(n * 131 + d)
     x = rng.standard_normal((n, d)).astype(f32).astype(dta)
@@ -443,7 +444,8 @@ def test_rearrange_random_layouts_bit_exact(gpu, stream):
 
 @pytest.mark.parametrize("shape,perm,dtype", [((1000, 37), (1, 0), np.uint16), ((64, 64, 64), (2, 1, 0), np.uint8),
                                               ((7, 2048, 128), (1, 0, 2), np.uint16), ((5, 3, 7, 11, 13), (4, 2, 0, 3, 1), np.uint32),
-                                              ((4096, 4096), (0, 1), np.uint16), ((3,), (0,), np.uint64)])
+                                              ((4096, 4096), (0, 1), np.uint16), ((3,), (0,), np.uint64),
+                                              ((64, 8200, 64), (1, 0, 2), np.uint16)])  # the last: > 64 MiB
 def test_rearrange_permutations(gpu, stream, shape, perm, dtype):
     rng = np.random.default_rng(7)
     src = rng.integers(0, 256, int(np.prod(shape)) * np.dtype(dtype).itemsize).astype(np.uint8).view(dtype).reshape(shape)
@@ -488,7 +490,8 @@ def test_swiglu_reference_shape(gpu, stream):
     assert_close_f16(out, oracle.swiglu(g.copy(), u), "swiglu ref shape")
 
 
-@pytest.mark.parametrize("n,d,ld", [(16, 11008, 22016), (3, 1001, 2002), (1, 8, 16), (70000, 16, 40)])
+@pytest.mark.parametrize("n,d,ld", [(16, 11008, 22016), (3, 1001, 2002), (1, 8, 16), (70000, 16, 40), (8195, 512, 1032),
+                                     (16400, 2048, 4096)])  # the last: > 64 MiB
 def test_swiglu_gate_up_halves(gpu, stream, n, d, ld):
     """gate and up are the two halves of one [n, 2*d] GEMM output (independent row strides)."""
     rng = np.random.default_rng(n + d)
