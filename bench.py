@@ -280,6 +280,42 @@ def standalone_ops(ophip, gpu, stream, rng, reps):
         b = arg_rows[0]
         us = time_launches(gpu, stream, lambda: rs.launch_batch(b, 16, 64000, None, None, stream), reps)
         add("random_sample " + mode, "16 x [32000]", 16 * (32000 * 2 + 8), us, note="1 batched launch (extension)")
+    # the remaining single-device operators, small and out-of-cache
+    ln = o.LayerNorm(gpu)
+    for n in (64, 65536):
+        x, y = gpu.malloc(n * D * 2), gpu.malloc(n * D * 2)
+        gpu.memset(x, 0x3C)
+        sc, bi = gpu.from_host(np.ones(D, np.float32)), gpu.from_host(np.zeros(D, np.float32))
+        a = o.LayerNormArgs(c(n, D), y, c(n, D), x, L.new_contiguous(o.dt.F32, [D]), sc,
+                            L.new_contiguous(o.dt.F32, [D]), bi, 1e-5)
+        us = time_launches(gpu, stream, lambda: ln.launch(a, None, stream), reps)
+        add("layer_norm", "[%d,%d]" % (n, D), 2 * n * D * 2 + 2 * D * 4, us)
+        x.free(); y.free()
+    ge = o.Gelu(gpu)
+    for n in (16, 16384):
+        t = gpu.malloc(n * DI * 2)
+        gpu.memset(t, 0x3C)
+        a = o.GeluArgs(c(n, DI), t)
+        us = time_launches(gpu, stream, lambda: ge.launch(a, None, stream), reps)
+        add("gelu", "[%d,%d]" % (n, DI), 2 * n * DI * 2, us)
+        t.free()
+    ad = o.Add(gpu)
+    for n in (16, 65536):
+        x, y, z = gpu.malloc(n * D * 2), gpu.malloc(n * D * 2), gpu.malloc(n * D * 2)
+        gpu.memset(x, 0x3C); gpu.memset(y, 0x3C)
+        a = o.AddArgs(c(n, D), z, c(n, D), x, c(n, D), y)
+        us = time_launches(gpu, stream, lambda: ad.launch(a, None, stream), reps)
+        add("add", "[%d,%d]" % (n, D), 3 * n * D * 2, us)
+        x.free(); y.free(); z.free()
+    ar = o.AddRows(gpu)
+    for m in (16, 32768):   # position-embedding style: dst[1, m, 4096] += table[idx[m], :], table 32000 rows
+        dst, table = gpu.malloc(m * D * 2), gpu.malloc(32000 * D * 2)
+        gpu.memset(dst, 0x3C); gpu.memset(table, 0x3C)
+        idx = gpu.from_host(rng.integers(0, 32000, (1, m)).astype(np.uint32))
+        a = o.AddRowsArgs(c(1, m, D), dst, c(32000, D), table, L.new_contiguous(o.dt.U32, [1, m]), idx)
+        us = time_launches(gpu, stream, lambda: ar.launch(a, None, stream), reps)
+        add("add_rows", "[1,%d,%d] from 32000 rows" % (m, D), 3 * m * D * 2 + m * 4, us)
+        dst.free(); table.free()
     # attention_kv_cached, the crate's composite, at the decode-layer shape: two cache appends, a staging copy
     # of the strided q, QK^T, causal softmax, PV and the copy into o - seven launches
     nt, pos = NT, KV - NT

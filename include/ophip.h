@@ -445,6 +445,81 @@ OPHIP_API int ophip_attention_kv_cached_launch(const ophip_attention_kv_cached *
                                                const ophip_queue_alloc *queue_alloc);
 OPHIP_API void ophip_attention_kv_cached_destroy(ophip_attention_kv_cached *op);
 
+/* ---- layer_norm: layer_norm/args.rs:7-55 ----------------------------------- */
+/* y[n,d] = (x - mean) * scale / (std + epsilon) + bias, std = sqrt(mean(x^2) - mean^2)
+ * (layer_norm/common_cpu/mod.rs:127-147).  (scale/bias, x/y) in {(f16,f16), (f32,f16), (f32,f32)}. */
+typedef struct ophip_layer_norm_args {
+    ophip_tensor_layout y_layout;
+    void *y_base;
+    ophip_tensor_layout x_layout;
+    const void *x_base;
+    ophip_tensor_layout scale_layout;
+    const void *scale_base;
+    ophip_tensor_layout bias_layout;
+    const void *bias_base;
+    float epsilon;
+} ophip_layer_norm_args;
+typedef struct ophip_layer_norm ophip_layer_norm;
+OPHIP_API int ophip_layer_norm_create(ophip_device *dev, ophip_layer_norm **out);
+OPHIP_API int ophip_layer_norm_scheme(ophip_layer_norm *op, const ophip_layer_norm_args *args,
+                                      size_t max_workspace_size, size_t *workspace_size);
+OPHIP_API int ophip_layer_norm_launch(const ophip_layer_norm *op, const ophip_layer_norm_args *args,
+                                      void *workspace, size_t workspace_len,
+                                      const ophip_queue_alloc *queue_alloc);
+OPHIP_API void ophip_layer_norm_destroy(ophip_layer_norm *op);
+
+/* ---- gelu: gelu/args.rs:4-36 (in place, tanh form, gelu/common_cpu/mod.rs:112-116) */
+typedef struct ophip_gelu_args {
+    ophip_tensor_layout layout; /* [n, d] */
+    void *base;
+} ophip_gelu_args;
+typedef struct ophip_gelu ophip_gelu;
+OPHIP_API int ophip_gelu_create(ophip_device *dev, ophip_gelu **out);
+OPHIP_API int ophip_gelu_scheme(ophip_gelu *op, const ophip_gelu_args *args, size_t max_workspace_size,
+                                size_t *workspace_size);
+OPHIP_API int ophip_gelu_launch(const ophip_gelu *op, const ophip_gelu_args *args, void *workspace,
+                                size_t workspace_len, const ophip_queue_alloc *queue_alloc);
+OPHIP_API void ophip_gelu_destroy(ophip_gelu *op);
+
+/* ---- add: add/args.rs:12-19; c = a + b, equal shapes, any strides (0 = broadcast in a, b) */
+typedef struct ophip_add_args {
+    ophip_tensor_layout c_layout;
+    void *c_base;
+    ophip_tensor_layout a_layout;
+    const void *a_base;
+    ophip_tensor_layout b_layout;
+    const void *b_base;
+} ophip_add_args;
+typedef struct ophip_add ophip_add;
+OPHIP_API int ophip_add_create(ophip_device *dev, ophip_add **out);
+OPHIP_API int ophip_add_scheme(ophip_add *op, const ophip_add_args *args, size_t max_workspace_size,
+                               size_t *workspace_size);
+OPHIP_API int ophip_add_launch(const ophip_add *op, const ophip_add_args *args, void *workspace,
+                               size_t workspace_len, const ophip_queue_alloc *queue_alloc);
+OPHIP_API void ophip_add_destroy(ophip_add *op);
+/* The layout normaliser Scheme::new (add/args.rs:42-167), host-only.  out receives
+ * [idx_strides (ndim+1 values: count ... 1), c_strides, a_strides, b_strides (ndim each)]
+ * and must hold 1 + 4*args->c_layout.ndim values; *ndim_out is the merged rank. */
+OPHIP_API int ophip_add_plan(const ophip_add_args *args, ptrdiff_t *out, size_t *ndim_out);
+
+/* ---- add_rows: add_rows/args.rs:10-17; dst[b, m, :] += src[idx[b, m], :], idx u32 or u64 */
+typedef struct ophip_add_rows_args {
+    ophip_tensor_layout dst_layout; /* [batch, m, n] */
+    void *dst_base;
+    ophip_tensor_layout src_layout; /* [k, n] */
+    const void *src_base;
+    ophip_tensor_layout idx_layout; /* [batch, m] */
+    const void *idx_base;
+} ophip_add_rows_args;
+typedef struct ophip_add_rows ophip_add_rows;
+OPHIP_API int ophip_add_rows_create(ophip_device *dev, ophip_add_rows **out);
+OPHIP_API int ophip_add_rows_scheme(ophip_add_rows *op, const ophip_add_rows_args *args,
+                                    size_t max_workspace_size, size_t *workspace_size);
+OPHIP_API int ophip_add_rows_launch(const ophip_add_rows *op, const ophip_add_rows_args *args,
+                                    void *workspace, size_t workspace_len,
+                                    const ophip_queue_alloc *queue_alloc);
+OPHIP_API void ophip_add_rows_destroy(ophip_add_rows *op);
+
 #ifdef __cplusplus
 }
 #endif

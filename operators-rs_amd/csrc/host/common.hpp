@@ -13,6 +13,7 @@
 #include <utility>
 #include <vector>
 
+#include "../kernels/params.h"
 #include "ophip.h"
 
 namespace ophip {
@@ -103,6 +104,19 @@ inline bool is_float_dtype(uint64_t dt) {
 }
 inline bool is_unsigned_dtype(uint64_t dt) {
     return dt == OPHIP_DT_U8 || dt == OPHIP_DT_U16 || dt == OPHIP_DT_U32 || dt == OPHIP_DT_U64;
+}
+
+// Division of any 32-bit n by a launch-time constant d >= 1 (the kernels' `fastdiv`):
+// q = (t + ((n - t) >> s1)) >> s2 with t = mulhi(m, n).
+inline FastDivU32 make_fastdiv(uint32_t d) {
+    FastDivU32 f{};
+    f.d = d;
+    uint32_t l = 0;
+    while ((1ull << l) < d) ++l;
+    f.m = (uint32_t)(((1ull << 32) * ((1ull << l) - d)) / d + 1);
+    f.s1 = l < 1 ? l : 1;
+    f.s2 = l == 0 ? 0 : l - 1;
+    return f;
 }
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

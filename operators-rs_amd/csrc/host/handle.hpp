@@ -50,6 +50,17 @@ inline void launch(hipFunction_t fn, Dim3 grid, Dim3 block, size_t smem, hipStre
 
 void check_hip(hipError_t e, const char *what);
 
+// every operator object keeps its device alive
+struct OpBase {
+    ophip_device *dev;
+    explicit OpBase(ophip_device *d) : dev(d) { ophip_device_retain(d); }
+    ~OpBase() { ophip_device_release(dev); }
+    OpBase(const OpBase &) = delete;
+    OpBase &operator=(const OpBase &) = delete;
+};
+
+inline unsigned ceil_div(size_t a, size_t b) { return (unsigned)((a + b - 1) / b); }
+
 inline hipStream_t stream_of(const ophip_queue_alloc *qa) {
     return qa ? reinterpret_cast<hipStream_t>(qa->stream) : nullptr;
 }

@@ -11,26 +11,6 @@ using namespace ophip;
 
 namespace {
 
-FastDivU32 make_fastdiv(uint32_t d) {
-    // q = (t + ((n - t) >> s1)) >> s2 with t = mulhi(m, n); exact for every 32-bit n, d >= 1
-    FastDivU32 f{};
-    f.d = d;
-    uint32_t l = 0;
-    while ((1ull << l) < d) ++l;
-    f.m = (uint32_t)(((1ull << 32) * ((1ull << l) - d)) / d + 1);
-    f.s1 = l < 1 ? l : 1;
-    f.s2 = l == 0 ? 0 : l - 1;
-    return f;
-}
-
-unsigned ceil_div(size_t a, size_t b) { return (unsigned)((a + b - 1) / b); }
-
-struct OpBase {
-    ophip_device *dev;
-    explicit OpBase(ophip_device *d) : dev(d) { ophip_device_retain(d); }
-    ~OpBase() { ophip_device_release(dev); }
-};
-
 const char *dt_tag(uint64_t dt) { return dt == OPHIP_DT_F16 ? "f16" : dt == OPHIP_DT_F32 ? "f32" : "?"; }
 
 }  // namespace

@@ -1,0 +1,62 @@
+// add for gfx950:  c = a + b, element-wise over N-d strided tensors (broadcast = stride 0 in a or b).
+//
+// The host merges the three layouts into at most 8 dimensions (add/args.rs:42-167) and counts
+// items in the innermost one: single elements, or 16-byte vectors when that dimension is
+// contiguous in all three tensors.  Item g is decoded into per-dimension indices with
+// multiply-high divisions; dimensions are ordered by descending c stride, so consecutive
+// threads write ascending addresses.  f16 sums are formed in f32 and rounded once, as
+// half's `f16 + f16` does.
+#include "device_util.h"
+
+struct AddOffsets {
+    int64_t c, a, b;
+};
+
+__device__ __forceinline__ AddOffsets add_decode(const AddParams &p, uint32_t g) {
+    AddOffsets o{0, 0, 0};
+    uint32_t rem = g;
+    for (uint32_t q = 0; q < p.ndim; ++q) {
+        const uint32_t k = fastdiv(rem, p.idx_div[q]);
+        rem -= k * p.idx_div[q].d;
+        o.c += (int64_t)k * p.c_s[q];
+        o.a += (int64_t)k * p.a_s[q];
+        o.b += (int64_t)k * p.b_s[q];
+    }
+    return o;
+}
+
+extern "C" __global__ void __launch_bounds__(256) add_f16_vec(AddParams p) {
+    for (uint32_t g = blockIdx.x * blockDim.x + threadIdx.x; g < p.total; g += gridDim.x * blockDim.x) {
+        const AddOffsets o = add_decode(p, g);
+        Pack8 a, b, c;
+        a.u = ld128(reinterpret_cast<const char *>(p.a) + o.a);
+        b.u = ld128(reinterpret_cast<const char *>(p.b) + o.b);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) c.e[i] = f2h(h2f(a.e[i]) + h2f(b.e[i]));
+        st128(reinterpret_cast<char *>(p.c) + o.c, c.u);
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(256) add_f32_vec(AddParams p) {
+    for (uint32_t g = blockIdx.x * blockDim.x + threadIdx.x; g < p.total; g += gridDim.x * blockDim.x) {
+        const AddOffsets o = add_decode(p, g);
+        Pack4f a, b, c;
+        a.u = ld128(reinterpret_cast<const char *>(p.a) + o.a);
+        b.u = ld128(reinterpret_cast<const char *>(p.b) + o.b);
+        c.f = a.f + b.f;
+        st128(reinterpret_cast<char *>(p.c) + o.c, c.u);
+    }
+}
+
+template <typename T>
+__device__ __forceinline__ void add_scalar(const AddParams &p) {
+    for (uint32_t g = blockIdx.x * blockDim.x + threadIdx.x; g < p.total; g += gridDim.x * blockDim.x) {
+        const AddOffsets o = add_decode(p, g);
+        const float a = (float)*reinterpret_cast<const T *>(reinterpret_cast<const char *>(p.a) + o.a);
+        const float b = (float)*reinterpret_cast<const T *>(reinterpret_cast<const char *>(p.b) + o.b);
+        *reinterpret_cast<T *>(reinterpret_cast<char *>(p.c) + o.c) = (T)(a + b);
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(256) add_f16_scalar(AddParams p) { add_scalar<f16>(p); }
+extern "C" __global__ void __launch_bounds__(256) add_f32_scalar(AddParams p) { add_scalar<float>(p); }

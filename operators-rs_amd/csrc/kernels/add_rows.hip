@@ -1,0 +1,59 @@
+// add_rows for gfx950:  dst[b, m, :] += src[idx[b, m], :]   (add_rows/common_cpu/mod.rs:131-147)
+//
+// blockIdx.y walks the b * m destination rows, blockIdx.x the row in 16-byte vectors (or single
+// elements when the row is not 16-byte friendly).  The row index is read once per workgroup.
+// An index >= k (the reference asserts) leaves the destination row unchanged.
+#include "device_util.h"
+
+__device__ __forceinline__ bool add_rows_locate(const AddRowsParams &p, uint32_t bm, char *&dst, const char *&src) {
+    const uint32_t b = bm / p.m, m = bm % p.m;
+    const char *ip = reinterpret_cast<const char *>(p.idx) + (int64_t)b * p.bsi + (int64_t)m * p.msi;
+    const uint64_t idx = p.idx_is_u64 ? *reinterpret_cast<const uint64_t *>(ip) : *reinterpret_cast<const uint32_t *>(ip);
+    if (idx >= p.k) return false;
+    dst = reinterpret_cast<char *>(p.dst) + (int64_t)b * p.bsd + (int64_t)m * p.msd;
+    src = reinterpret_cast<const char *>(p.src) + (int64_t)idx * p.kss;
+    return true;
+}
+
+extern "C" __global__ void __launch_bounds__(256) add_rows_f16_vec(AddRowsParams p) {
+    const uint32_t nvec = p.n / 8;
+    for (uint32_t bm = blockIdx.y; bm < p.batch * p.m; bm += gridDim.y) {
+        char *dst;
+        const char *src;
+        if (!add_rows_locate(p, bm, dst, src)) continue;
+        for (uint32_t v = blockIdx.x * blockDim.x + threadIdx.x; v < nvec; v += gridDim.x * blockDim.x) {
+            Pack8 d, s;
+            d.u = ld128(dst + (size_t)v * 16);
+            s.u = ld128(src + (size_t)v * 16);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) d.e[i] = f2h(h2f(d.e[i]) + h2f(s.e[i]));
+            st128(dst + (size_t)v * 16, d.u);
+        }
+    }
+}
+
+// element-wise; nsd / nss are the element strides of dst and src rows in bytes
+template <typename T>
+__device__ __forceinline__ void add_rows_scalar(const AddRowsParams &p, int64_t nsd, int64_t nss) {
+    for (uint32_t bm = blockIdx.y; bm < p.batch * p.m; bm += gridDim.y) {
+        char *dst;
+        const char *src;
+        if (!add_rows_locate(p, bm, dst, src)) continue;
+        for (uint32_t j = blockIdx.x * blockDim.x + threadIdx.x; j < p.n; j += gridDim.x * blockDim.x) {
+            T *d = reinterpret_cast<T *>(dst + (int64_t)j * nsd);
+            const T *s = reinterpret_cast<const T *>(src + (int64_t)j * nss);
+            *d = (T)((float)*d + (float)*s);
+        }
+    }
+}
+
+struct AddRowsScalarParams {
+    AddRowsParams p;
+    int64_t nsd, nss;
+};
+extern "C" __global__ void __launch_bounds__(256) add_rows_f16_scalar(AddRowsScalarParams q) {
+    add_rows_scalar<f16>(q.p, q.nsd, q.nss);
+}
+extern "C" __global__ void __launch_bounds__(256) add_rows_f32_scalar(AddRowsScalarParams q) {
+    add_rows_scalar<float>(q.p, q.nsd, q.nss);
+}

@@ -1,0 +1,161 @@
+// layer_norm for gfx950:  y = (x - e) * (scale * k) + bias,  e = mean(x),
+// k = 1 / (sqrt(mean(x^2) - e^2) + eps)  -- epsilon is added to the standard deviation,
+// as the reference does (layer_norm/common_cpu/mod.rs:127-147).
+//
+// Same shape as rms_norm: a row is owned by a group of G threads (a wave, or a whole
+// workgroup for few / long rows), up to 8 vectors per thread stay in registers so the row
+// is read once, the two sums go through wave butterflies and one LDS slot per wave.  The
+// output uses one fused multiply-add per element, like the reference's mul_add.
+#include "device_util.h"
+
+template <typename TA>
+struct Vec;  // 16 bytes of TA
+template <>
+struct Vec<f16> {
+    static constexpr int N = 8;
+    Pack8 v;
+    __device__ __forceinline__ float get(int i) const { return h2f(v.e[i]); }
+    __device__ __forceinline__ void set(int i, float f) { v.e[i] = f2h(f); }
+};
+template <>
+struct Vec<float> {
+    static constexpr int N = 4;
+    Pack4f v;
+    __device__ __forceinline__ float get(int i) const { return v.e[i]; }
+    __device__ __forceinline__ void set(int i, float f) { v.e[i] = f; }
+};
+
+// N consecutive parameters starting at element j (j multiple of N, base 16-byte aligned)
+template <typename TW, int N>
+__device__ __forceinline__ void load_param_vec(const void *w, uint32_t j, float (&out)[N]) {
+    if constexpr (sizeof(TW) == 2) {
+        static_assert(N == 8, "");
+        Pack8 p;
+        p.u = ld128(reinterpret_cast<const f16 *>(w) + j);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) out[i] = h2f(p.e[i]);
+    } else {
+#pragma unroll
+        for (int c = 0; c < N / 4; ++c) {
+            Pack4f p;
+            p.u = ld128(reinterpret_cast<const float *>(w) + j + 4 * c);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) out[4 * c + i] = p.e[i];
+        }
+    }
+}
+
+__device__ __forceinline__ void mean_and_scale(float sum, float sum2, uint32_t d, float eps, float &e, float &k) {
+    const float n = (float)d;
+    e = sum / n;
+    const float e2 = sum2 / n;
+    k = 1.0f / (sqrtf(e2 - e * e) + eps);
+}
+
+template <typename TA, typename TW, int G>
+__device__ __forceinline__ void layer_norm_vec(const LayerNormParams &p) {
+    constexpr int N = Vec<TA>::N;
+    constexpr int CACHE = 8;
+    constexpr int BLOCK = G < 256 ? 256 : G;
+    constexpr int RPB = BLOCK / G;
+    __shared__ float smem[BLOCK / WAVE];
+
+    const uint32_t lane = threadIdx.x % G;
+    uint32_t row = blockIdx.x * RPB + threadIdx.x / G;
+    const bool live = row < p.n;
+    if (!live) row = p.n - 1;  // keep every thread on the barriers; stores are suppressed
+
+    const char *xr = reinterpret_cast<const char *>(p.x) + (int64_t)row * p.nsx;
+    char *yr = reinterpret_cast<char *>(p.y) + (int64_t)row * p.nsy;
+    const uint32_t nvec = p.d / N;
+
+    Vec<TA> cache[CACHE];
+    float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+    for (int c = 0; c < CACHE; ++c) {
+        const uint32_t v = lane + c * G;
+        if (v < nvec) {
+            cache[c].v.u = ld128(xr + (size_t)v * 16);
+#pragma unroll
+            for (int i = 0; i < N; ++i) {
+                const float f = cache[c].get(i);
+                s1 += f;
+                s2 += f * f;
+            }
+        }
+    }
+    for (uint32_t v = lane + CACHE * G; v < nvec; v += G) {
+        Vec<TA> t;
+        t.v.u = ld128(xr + (size_t)v * 16);
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            const float f = t.get(i);
+            s1 += f;
+            s2 += f * f;
+        }
+    }
+    s1 = group_sum<G>(s1, smem);
+    s2 = group_sum<G>(s2, smem);
+    float e, k;
+    mean_and_scale(s1, s2, p.d, p.epsilon, e, k);
+
+    auto emit = [&](const Vec<TA> &x, uint32_t v) {
+        float s[N], b[N];
+        load_param_vec<TW, N>(p.scale, v * N, s);
+        load_param_vec<TW, N>(p.bias, v * N, b);
+        Vec<TA> o;
+#pragma unroll
+        for (int i = 0; i < N; ++i) o.set(i, __builtin_fmaf(x.get(i) - e, s[i] * k, b[i]));
+        if (live) st128(yr + (size_t)v * 16, o.v.u);
+    };
+#pragma unroll
+    for (int c = 0; c < CACHE; ++c) {
+        const uint32_t v = lane + c * G;
+        if (v < nvec) emit(cache[c], v);
+    }
+    for (uint32_t v = lane + CACHE * G; v < nvec; v += G) {
+        Vec<TA> t;
+        t.v.u = ld128(xr + (size_t)v * 16);
+        emit(t, v);
+    }
+}
+
+// Element-wise variant for rows that are not 16-byte friendly (odd d, odd strides).
+template <typename TA, typename TW>
+__device__ __forceinline__ void layer_norm_scalar(const LayerNormParams &p) {
+    constexpr int G = 256;
+    __shared__ float smem[G / WAVE];
+    const uint32_t row = blockIdx.x;
+    const TA *xr = reinterpret_cast<const TA *>(reinterpret_cast<const char *>(p.x) + (int64_t)row * p.nsx);
+    TA *yr = reinterpret_cast<TA *>(reinterpret_cast<char *>(p.y) + (int64_t)row * p.nsy);
+    float s1 = 0.f, s2 = 0.f;
+    for (uint32_t j = threadIdx.x; j < p.d; j += G) {
+        const float f = (float)xr[j];
+        s1 += f;
+        s2 += f * f;
+    }
+    s1 = group_sum<G>(s1, smem);
+    s2 = group_sum<G>(s2, smem);
+    float e, k;
+    mean_and_scale(s1, s2, p.d, p.epsilon, e, k);
+    const TW *sc = reinterpret_cast<const TW *>(p.scale), *bi = reinterpret_cast<const TW *>(p.bias);
+    for (uint32_t j = threadIdx.x; j < p.d; j += G)
+        yr[j] = (TA)__builtin_fmaf((float)xr[j] - e, (float)sc[j] * k, (float)bi[j]);
+}
+
+#define LAYER_NORM(NAME, TA, TW)                                                                                  \
+    extern "C" __global__ void __launch_bounds__(256) layer_norm_##NAME##_g64(LayerNormParams p) {                \
+        layer_norm_vec<TA, TW, 64>(p);                                                                            \
+    }                                                                                                             \
+    extern "C" __global__ void __launch_bounds__(256) layer_norm_##NAME##_g256(LayerNormParams p) {               \
+        layer_norm_vec<TA, TW, 256>(p);                                                                           \
+    }                                                                                                             \
+    extern "C" __global__ void __launch_bounds__(1024) layer_norm_##NAME##_g1024(LayerNormParams p) {             \
+        layer_norm_vec<TA, TW, 1024>(p);                                                                          \
+    }                                                                                                             \
+    extern "C" __global__ void __launch_bounds__(256) layer_norm_##NAME##_scalar(LayerNormParams p) {             \
+        layer_norm_scalar<TA, TW>(p);                                                                             \
+    }
+LAYER_NORM(f16_f16, f16, f16)
+LAYER_NORM(f16_f32, f16, float)
+LAYER_NORM(f32_f32, float, float)

@@ -89,3 +89,45 @@ struct GemmParams {
     uint32_t split_k;
     uint32_t k_per_split;  // multiple of 32
 };
+
+struct LayerNormParams {
+    void *y;
+    const void *x;
+    const void *scale;
+    const void *bias;
+    int64_t nsy, nsx;  // row strides in bytes
+    uint32_t n, d;
+    float epsilon;
+    uint32_t _pad;
+};
+
+struct GeluParams {
+    void *base;
+    int64_t sn;  // row stride in bytes
+    uint32_t n, d;
+};
+
+// c = a + b over up to OPHIP_REARRANGE_MAXD merged dimensions; item g decodes into one index per
+// dimension through idx_div (items per step of that dimension), strides in bytes.
+struct AddParams {
+    void *c;
+    const void *a;
+    const void *b;
+    uint32_t total;  // items: elements, or 16-byte vectors when `vec`
+    uint32_t ndim;
+    FastDivU32 idx_div[OPHIP_REARRANGE_MAXD];
+    int64_t c_s[OPHIP_REARRANGE_MAXD];
+    int64_t a_s[OPHIP_REARRANGE_MAXD];
+    int64_t b_s[OPHIP_REARRANGE_MAXD];
+};
+
+// dst[b, m, :] += src[idx[b, m], :]
+struct AddRowsParams {
+    void *dst;
+    const void *src;
+    const void *idx;
+    int64_t bsd, msd, kss, bsi, msi;  // bytes
+    uint32_t batch, m, n, k;
+    uint32_t idx_is_u64;
+    uint32_t _pad;
+};

@@ -169,6 +169,26 @@ class _AttnKVCachedArgs(ctypes.Structure):
                 ("mask", ctypes.c_uint8), ("pos", ctypes.c_size_t)]
 
 
+class _LayerNormArgs(ctypes.Structure):
+    _fields_ = [("y_layout", _Layout), ("y_base", ctypes.c_void_p), ("x_layout", _Layout),
+                ("x_base", ctypes.c_void_p), ("scale_layout", _Layout), ("scale_base", ctypes.c_void_p),
+                ("bias_layout", _Layout), ("bias_base", ctypes.c_void_p), ("epsilon", ctypes.c_float)]
+
+
+class _GeluArgs(ctypes.Structure):
+    _fields_ = [("layout", _Layout), ("base", ctypes.c_void_p)]
+
+
+class _AddArgs(ctypes.Structure):
+    _fields_ = [("c_layout", _Layout), ("c_base", ctypes.c_void_p), ("a_layout", _Layout),
+                ("a_base", ctypes.c_void_p), ("b_layout", _Layout), ("b_base", ctypes.c_void_p)]
+
+
+class _AddRowsArgs(ctypes.Structure):
+    _fields_ = [("dst_layout", _Layout), ("dst_base", ctypes.c_void_p), ("src_layout", _Layout),
+                ("src_base", ctypes.c_void_p), ("idx_layout", _Layout), ("idx_base", ctypes.c_void_p)]
+
+
 # every symbol include/ophip.h declares
 EXPORTS = [
     "ophip_last_error", "ophip_status_name", "ophip_dtype_nbytes",
@@ -198,6 +218,10 @@ EXPORTS = [
     "ophip_attention_create", "ophip_attention_scheme", "ophip_attention_launch", "ophip_attention_destroy",
     "ophip_attention_kv_cached_create", "ophip_attention_kv_cached_scheme", "ophip_attention_kv_cached_launch",
     "ophip_attention_kv_cached_destroy",
+    "ophip_layer_norm_create", "ophip_layer_norm_scheme", "ophip_layer_norm_launch", "ophip_layer_norm_destroy",
+    "ophip_gelu_create", "ophip_gelu_scheme", "ophip_gelu_launch", "ophip_gelu_destroy",
+    "ophip_add_create", "ophip_add_scheme", "ophip_add_launch", "ophip_add_destroy", "ophip_add_plan",
+    "ophip_add_rows_create", "ophip_add_rows_scheme", "ophip_add_rows_launch", "ophip_add_rows_destroy",
 ]
 
 _lib = None
@@ -626,8 +650,77 @@ class AttnKVCachedArgs:
                                  DYN_USIZE if self.pos is None else self.pos)
 
 
+class LayerNormArgs:
+    """layer_norm/args.rs:7-17"""
+
+    def __init__(self, y_layout, y_base, x_layout, x_base, scale_layout, scale_base, bias_layout, bias_base, epsilon):
+        self.__dict__.update(locals())
+
+    def c(self):
+        return _LayerNormArgs(self.y_layout.c(), _p(self.y_base), self.x_layout.c(), _p(self.x_base),
+                              self.scale_layout.c(), _p(self.scale_base), self.bias_layout.c(), _p(self.bias_base),
+                              self.epsilon)
+
+
+class GeluArgs:
+    """gelu/args.rs:4-7"""
+
+    def __init__(self, layout, base):
+        self.__dict__.update(locals())
+
+    def c(self):
+        return _GeluArgs(self.layout.c(), _p(self.base))
+
+
+class AddArgs:
+    """add/args.rs:12-19"""
+
+    def __init__(self, c_layout, c_base, a_layout, a_base, b_layout, b_base):
+        self.__dict__.update(locals())
+
+    def c(self):
+        return _AddArgs(self.c_layout.c(), _p(self.c_base), self.a_layout.c(), _p(self.a_base),
+                        self.b_layout.c(), _p(self.b_base))
+
+
+class AddRowsArgs:
+    """add_rows/args.rs:10-17"""
+
+    def __init__(self, dst_layout, dst_base, src_layout, src_base, idx_layout, idx_base):
+        self.__dict__.update(locals())
+
+    def c(self):
+        return _AddRowsArgs(self.dst_layout.c(), _p(self.dst_base), self.src_layout.c(), _p(self.src_base),
+                            self.idx_layout.c(), _p(self.idx_base))
+
+
 class RmsNorm(_Operator):
     NAME = "rms_norm"
+
+
+class LayerNorm(_Operator):
+    NAME = "layer_norm"
+
+
+class Gelu(_Operator):
+    NAME = "gelu"
+
+
+class Add(_Operator):
+    NAME = "add"
+
+    @staticmethod
+    def plan(args):
+        """Scheme::new (add/args.rs:42-167) evaluated by the library: [idx strides..., c, a, b strides]."""
+        nd_in = len(args.c_layout.shape)
+        out = (ctypes.c_ssize_t * (1 + 4 * max(nd_in, 1)))()
+        nd = ctypes.c_size_t()
+        _check(lib().ophip_add_plan(ctypes.byref(args.c()), out, ctypes.byref(nd)))
+        return list(out[: 1 + 4 * nd.value])
+
+
+class AddRows(_Operator):
+    NAME = "add_rows"
 
 
 class Rope(_Operator):

@@ -90,6 +90,10 @@ def lib():
         L.oracle_mat_mul_layout.argtypes = [ctypes.POINTER(MMLayout), sz, sz, psz, pss, sz, psz, pss,
                                             sz, psz, pss]
         L.oracle_mat_mul.argtypes = [vp, f, vp, vp, f, ctypes.POINTER(MMLayout), i]
+        L.oracle_layer_norm.argtypes = [vp, ss, ss, vp, ss, ss, vp, ss, vp, ss, sz, sz, f, i, i]
+        L.oracle_gelu.argtypes = [vp, ss, ss, sz, sz, i]
+        L.oracle_add.argtypes = [vp, vp, vp, sz, sz, sz, psz, psz, psz, pss, pss, pss, i, i, i]
+        L.oracle_add_rows.argtypes = [vp, ss, ss, ss, vp, ss, ss, vp, ss, ss, sz, sz, sz, sz, i, i]
         _lib = L
     return _lib
 
@@ -278,3 +282,37 @@ def attention_kv_cached(q, k, v, o, k_cache, v_cache, pos, causal=True):
     rearrange(k_cache[:, pos:att], k)
     rearrange(v_cache[:, pos:att], v)
     return attention(q, k_cache[:, :att], v_cache[:, :att], o, causal=causal)
+
+
+def layer_norm(y, x, scale, bias, epsilon):
+    """y[n,d] <- layer_norm(x[n,d]; scale[d], bias[d]); epsilon is added to the standard deviation."""
+    n, d = x.shape
+    _check(lib().oracle_layer_norm(_ptr(y), y.strides[0], y.strides[1], _ptr(x), x.strides[0], x.strides[1],
+                                   _ptr(scale), scale.strides[0], _ptr(bias), bias.strides[0], n, d,
+                                   float(epsilon), _DT[x.dtype], _DT[scale.dtype]))
+    return y
+
+
+def gelu(t):
+    """In-place tanh-form gelu on t[n,d]."""
+    n, d = t.shape
+    _check(lib().oracle_gelu(_ptr(t), t.strides[0], t.strides[1], n, d, _DT[t.dtype]))
+    return t
+
+
+def add(c, a, b):
+    """c <- a + b on numpy views of equal shape (any strides; stride 0 in a or b broadcasts)."""
+    _check(lib().oracle_add(_ptr(c), _ptr(a), _ptr(b), c.ndim, a.ndim, b.ndim, _usz(c.shape), _usz(a.shape),
+                            _usz(b.shape), _isz(c.strides), _isz(a.strides), _isz(b.strides),
+                            _DT[c.dtype], _DT[a.dtype], _DT[b.dtype]))
+    return c
+
+
+def add_rows(dst, src, idx):
+    """dst[b,m,:] += src[idx[b,m],:]; idx is uint32 or uint64."""
+    batch, m, n = dst.shape
+    k = src.shape[0]
+    _check(lib().oracle_add_rows(_ptr(dst), dst.strides[0], dst.strides[1], dst.strides[2], _ptr(src),
+                                 src.strides[0], src.strides[1], _ptr(idx), idx.strides[0], idx.strides[1],
+                                 batch, m, n, k, _DT[dst.dtype], _DT[idx.dtype]))
+    return dst

@@ -882,3 +882,162 @@ ORACLE_API int oracle_mat_mul(void *c_base, float beta, const void *a_base, cons
     }
     return ORACLE_OK;
 }
+
+/* ------------------------------------------------------------ layer_norm -- */
+/* layer_norm/common_cpu/mod.rs:127-147 (Scheme::calculate), X = f32 for f16 / f32 data:
+ *   sum, sum2 sequential in j; e = sum/d; e2 = sum2/d; std = sqrt(e2 - e*e);
+ *   k = 1/(std + eps);  y = fma(x - e, s*k, b)  (mul_add is one fused operation).
+ * (scale/bias, x/y) in {(f16,f16), (f32,f16), (f32,f32), (f64,f64)} (mod.rs:84-90).
+ * Pinned by: f64 closed form, constant row gives bias exactly, scale 1 / bias 0 gives zero
+ * mean, explicit numpy-f32 replay of the rounding points.
+ */
+ORACLE_API int oracle_layer_norm(void *y, ptrdiff_t nsy, ptrdiff_t dsy, const void *x, ptrdiff_t nsx,
+                                 ptrdiff_t dsx, const void *s, ptrdiff_t dss, const void *b, ptrdiff_t dsb,
+                                 size_t n, size_t d, float epsilon, int dt_a, int dt_w) {
+    const int f64 = dt_a == ORACLE_F64 && dt_w == ORACLE_F64;
+    const int ok = (dt_a == ORACLE_F16 && (dt_w == ORACLE_F16 || dt_w == ORACLE_F32)) ||
+                   (dt_a == ORACLE_F32 && dt_w == ORACLE_F32) || f64;
+    if (!ok) return ORACLE_TYPE_NOT_SUPPORT;
+    for (ptrdiff_t i = 0; i < (ptrdiff_t)n; i++) {
+        const char *xr = (const char *)x + i * nsx;
+        char *yr = (char *)y + i * nsy;
+        if (f64) {
+            double sum = 0.0, sum2 = 0.0;
+            for (ptrdiff_t j = 0; j < (ptrdiff_t)d; j++) {
+                double v = ld_f64(xr + j * dsx);
+                sum += v;
+                sum2 += v * v;
+            }
+            double nn = (double)d, e = sum / nn, e2 = sum2 / nn;
+            double k = 1.0 / (sqrt(e2 - e * e) + (double)epsilon);
+            for (ptrdiff_t j = 0; j < (ptrdiff_t)d; j++)
+                st_f64(yr + j * dsy, fma(ld_f64(xr + j * dsx) - e, ld_f64((const char *)s + j * dss) * k,
+                                         ld_f64((const char *)b + j * dsb)));
+        } else {
+            float sum = 0.0f, sum2 = 0.0f;
+            for (ptrdiff_t j = 0; j < (ptrdiff_t)d; j++) {
+                float v = dt_a == ORACLE_F16 ? ld_f16(xr + j * dsx) : ld_f32(xr + j * dsx);
+                sum += v;
+                sum2 += v * v;
+            }
+            float nn = (float)d, e = sum / nn, e2 = sum2 / nn;
+            float k = 1.0f / (sqrtf(e2 - e * e) + epsilon);
+            for (ptrdiff_t j = 0; j < (ptrdiff_t)d; j++) {
+                float v = dt_a == ORACLE_F16 ? ld_f16(xr + j * dsx) : ld_f32(xr + j * dsx);
+                float sc = dt_w == ORACLE_F16 ? ld_f16((const char *)s + j * dss) : ld_f32((const char *)s + j * dss);
+                float bi = dt_w == ORACLE_F16 ? ld_f16((const char *)b + j * dsb) : ld_f32((const char *)b + j * dsb);
+                float r = fmaf(v - e, sc * k, bi);
+                if (dt_a == ORACLE_F16) st_f16(yr + j * dsy, r);
+                else st_f32(yr + j * dsy, r);
+            }
+        }
+    }
+    return ORACLE_OK;
+}
+
+/* ------------------------------------------------------------------ gelu -- */
+/* gelu/common_cpu/mod.rs:112-123:  0.5 * x * (1 + tanh(sqrt(2/pi) * (x + 0.044715 * x^3))),
+ * evaluated left to right in the element's arithmetic type (f32 for f16 data); powi(3) is
+ * x * x * x; FRAC_2_PI.sqrt() is the correctly rounded square root of the f32 constant.
+ * Pinned by: f64 closed form, gelu(0) = 0, large |x| saturates to x and -0, odd part identity
+ * gelu(x) - gelu(-x) = x.
+ */
+ORACLE_API int oracle_gelu(void *base, ptrdiff_t sn, ptrdiff_t sd, size_t n, size_t d, int dt) {
+    if (dt != ORACLE_F16 && dt != ORACLE_F32 && dt != ORACLE_F64) return ORACLE_TYPE_NOT_SUPPORT;
+    const float c32 = sqrtf(0.636619772367581343076f);
+    const double c64 = sqrt(0.636619772367581343076);
+    for (ptrdiff_t i = 0; i < (ptrdiff_t)n; i++)
+        for (ptrdiff_t j = 0; j < (ptrdiff_t)d; j++) {
+            char *p = (char *)base + i * sn + j * sd;
+            if (dt == ORACLE_F64) {
+                double v = ld_f64(p);
+                st_f64(p, 0.5 * v * (1.0 + tanh(c64 * (v + 0.044715 * (v * v * v)))));
+            } else {
+                float v = dt == ORACLE_F16 ? ld_f16(p) : ld_f32(p);
+                float r = 0.5f * v * (1.0f + tanhf(c32 * (v + 0.044715f * (v * v * v))));
+                if (dt == ORACLE_F16) st_f16(p, r);
+                else st_f32(p, r);
+            }
+        }
+    return ORACLE_OK;
+}
+
+/* ------------------------------------------------------------------- add -- */
+/* add/args.rs:42-167 (validation) + add/common_cpu/mod.rs:29-75: c = a + b element-wise.
+ * The reference's Scheme only chooses the visiting order (merged dimensions); the sum of two
+ * f16 is formed in f32 and rounded once (half's Add).  Checks in the reference's order:
+ * types, ranks, per-dimension shapes, zero c stride on a dimension longer than 1.
+ * Pinned by: numpy on random strided / broadcast layouts (f16 sums of f16 are exact in f32,
+ * so numpy's float16 add rounds identically).
+ */
+ORACLE_API int oracle_add(void *c, const void *a, const void *b, size_t ndim_c, size_t ndim_a, size_t ndim_b,
+                          const size_t *shape_c, const size_t *shape_a, const size_t *shape_b,
+                          const ptrdiff_t *sc, const ptrdiff_t *sa, const ptrdiff_t *sb, int dt_c, int dt_a,
+                          int dt_b) {
+    if (dt_c != dt_a || dt_c != dt_b) return ORACLE_TYPE_MISMATCH;
+    if (ndim_a != ndim_c || ndim_b != ndim_c) return ORACLE_RANK_MISMATCH;
+    size_t total = 1;
+    for (size_t i = 0; i < ndim_c; i++) {
+        if (shape_c[i] == SIZE_MAX || shape_a[i] == SIZE_MAX || shape_b[i] == SIZE_MAX ||
+            sc[i] == PTRDIFF_MAX || sa[i] == PTRDIFF_MAX || sb[i] == PTRDIFF_MAX)
+            return ORACLE_DYNAMIC_NOT_SUPPORT;
+        if (shape_a[i] != shape_c[i] || shape_b[i] != shape_c[i]) return ORACLE_SHAPE_MISMATCH;
+        if (shape_c[i] != 1 && sc[i] == 0) return ORACLE_SHAPE_NOT_SUPPORT;
+        total *= shape_c[i];
+    }
+    if (dt_c != ORACLE_F16 && dt_c != ORACLE_F32 && dt_c != ORACLE_F64) return ORACLE_TYPE_NOT_SUPPORT;
+    for (size_t f = 0; f < total; f++) {
+        size_t rem = f;
+        ptrdiff_t oc = 0, oa = 0, ob = 0;
+        for (size_t q = ndim_c; q-- > 0;) {
+            ptrdiff_t k = (ptrdiff_t)(rem % shape_c[q]);
+            rem /= shape_c[q];
+            oc += k * sc[q];
+            oa += k * sa[q];
+            ob += k * sb[q];
+        }
+        if (dt_c == ORACLE_F16) st_f16((char *)c + oc, ld_f16((const char *)a + oa) + ld_f16((const char *)b + ob));
+        else if (dt_c == ORACLE_F32) st_f32((char *)c + oc, ld_f32((const char *)a + oa) + ld_f32((const char *)b + ob));
+        else st_f64((char *)c + oc, ld_f64((const char *)a + oa) + ld_f64((const char *)b + ob));
+    }
+    return ORACLE_OK;
+}
+
+/* -------------------------------------------------------------- add_rows -- */
+/* add_rows/common_cpu/mod.rs:131-147: dst[b, m, :] += src[idx[b, m], :]; the reference
+ * asserts idx < k (here: ORACLE_ARGS_NOT_SUPPORT, nothing of that row is written).
+ * Pinned by: numpy fancy indexing with repeated and boundary indices.
+ */
+ORACLE_API int oracle_add_rows(void *dst, ptrdiff_t bsd, ptrdiff_t msd, ptrdiff_t nsd, const void *src,
+                               ptrdiff_t kss, ptrdiff_t nss, const void *idx, ptrdiff_t bsi, ptrdiff_t msi,
+                               size_t batch, size_t m, size_t n, size_t k, int dt, int dt_idx) {
+    if (dt_idx != ORACLE_U32 && dt_idx != ORACLE_U64) return ORACLE_TYPE_NOT_SUPPORT;
+    if (dt != ORACLE_F16 && dt != ORACLE_F32 && dt != ORACLE_F64) return ORACLE_TYPE_NOT_SUPPORT;
+    int bad = 0;
+    for (ptrdiff_t bi = 0; bi < (ptrdiff_t)batch; bi++)
+        for (ptrdiff_t mi = 0; mi < (ptrdiff_t)m; mi++) {
+            const char *ip = (const char *)idx + bi * bsi + mi * msi;
+            uint64_t r;
+            if (dt_idx == ORACLE_U32) {
+                uint32_t t;
+                memcpy(&t, ip, 4);
+                r = t;
+            } else {
+                memcpy(&r, ip, 8);
+            }
+            if (r >= k) {
+                bad = 1;
+                continue;
+            }
+            char *d = (char *)dst + bi * bsd + mi * msd;
+            const char *s = (const char *)src + (ptrdiff_t)r * kss;
+            for (ptrdiff_t j = 0; j < (ptrdiff_t)n; j++) {
+                char *pd = d + j * nsd;
+                const char *ps = s + j * nss;
+                if (dt == ORACLE_F16) st_f16(pd, ld_f16(pd) + ld_f16(ps));
+                else if (dt == ORACLE_F32) st_f32(pd, ld_f32(pd) + ld_f32(ps));
+                else st_f64(pd, ld_f64(pd) + ld_f64(ps));
+            }
+        }
+    return bad ? ORACLE_ARGS_NOT_SUPPORT : ORACLE_OK;
+}
