@@ -146,6 +146,17 @@ OPHIP_API int ophip_event_synchronize(ophip_device *dev, ophip_event ev);
 OPHIP_API int ophip_event_elapsed_ms(ophip_device *dev, ophip_event start, ophip_event stop,
                                      float *ms);
 
+/* Launch graphs (no counterpart in the reference's driver crate): a fixed sequence of launch()
+ * calls on `stream` between begin and end is recorded instead of run, and replayed by
+ * ophip_graph_launch without per-launch host cost.  Give every recorded launch a workspace of
+ * its own (scheme() reports the size) and launch mat_mul once on the stream before recording:
+ * its first launch on a stream allocates. */
+typedef void *ophip_graph; /* hipGraphExec_t */
+OPHIP_API int ophip_stream_begin_capture(ophip_device *dev, ophip_stream stream);
+OPHIP_API int ophip_stream_end_capture(ophip_device *dev, ophip_stream stream, ophip_graph *out);
+OPHIP_API int ophip_graph_launch(ophip_device *dev, ophip_graph graph, ophip_stream stream);
+OPHIP_API int ophip_graph_destroy(ophip_device *dev, ophip_graph graph);
+
 /* ---- QueueAlloc: lib.rs:89-102 -------------------------------------------
  * A queue (stream) plus an allocator bound to it.  `alloc`/`free` are called by
  * launch() only when the caller's workspace is too small (common/workspace.rs:

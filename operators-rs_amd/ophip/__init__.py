@@ -198,6 +198,7 @@ EXPORTS = [
     "ophip_stream_create", "ophip_stream_destroy", "ophip_stream_synchronize",
     "ophip_event_create", "ophip_event_destroy", "ophip_event_record", "ophip_event_synchronize",
     "ophip_event_elapsed_ms",
+    "ophip_stream_begin_capture", "ophip_stream_end_capture", "ophip_graph_launch", "ophip_graph_destroy",
     "ophip_queue_alloc_from_stream", "ophip_mem_pool_create", "ophip_mem_pool_put",
     "ophip_mem_pool_queue_alloc", "ophip_mem_pool_destroy",
     "ophip_offset_calculator_create", "ophip_offset_calculator_destroy", "ophip_offset_calculator_put",
@@ -308,9 +309,33 @@ class Stream:
     def synchronize(self):
         _check(lib().ophip_stream_synchronize(self.gpu.handle, self.handle))
 
+    def begin_capture(self):
+        """Record the launches that follow on this stream instead of running them."""
+        _check(lib().ophip_stream_begin_capture(self.gpu.handle, self.handle))
+
+    def end_capture(self):
+        g = ctypes.c_void_p()
+        _check(lib().ophip_stream_end_capture(self.gpu.handle, self.handle, ctypes.byref(g)))
+        return Graph(self.gpu, g)
+
     def destroy(self):
         if self.handle is not None:
             lib().ophip_stream_destroy(self.gpu.handle, self.handle)
+            self.handle = None
+
+
+class Graph:
+    """A recorded launch sequence (hipGraphExec_t)."""
+
+    def __init__(self, gpu, handle):
+        self.gpu, self.handle = gpu, handle
+
+    def launch(self, stream):
+        _check(lib().ophip_graph_launch(self.gpu.handle, self.handle, stream.handle), launch=True)
+
+    def destroy(self):
+        if self.handle is not None:
+            lib().ophip_graph_destroy(self.gpu.handle, self.handle)
             self.handle = None
 
 

@@ -961,3 +961,45 @@ def test_stream_mem_pool_serves_workspaces(gpu, stream):
     assert p3 == p1
     assert not qa.alloc(qa.ctx, 2 << 20)  # the reference panics "out of memory"; here the launch fails cleanly
     pool.destroy()
+
+
+# ---------------------------------------------------------- launch graphs ----
+
+def test_recorded_launch_sequence_replays_like_eager_launches(gpu, stream):
+    """rms_norm -> split-K mat_mul -> swiglu recorded once and replayed: every replay must give the eager
+    result, with eager work and synchronisations in between."""
+    rng = np.random.default_rng(21)
+    x = normal_f16(rng, (16, 4096))
+    w = rng.uniform(0.5, 1.5, 4096).astype(f32).astype(f16)
+    wgu = normal_f16(rng, (4096, 2048), std=0.02)
+    xd, wd, wgud = gpu.from_host(x), gpu.from_host(w), gpu.from_host(wgu)
+    xn, gu = gpu.malloc(x.nbytes), gpu.malloc(16 * 2048 * 2)
+    L = TensorLayout
+    c = lambda *s: L.new_contiguous(dt.F16, list(s))
+    half = L(dt.F16, [16, 1024], [2048 * 2, 2])
+    rms, mm, sw = ophip.RmsNorm(gpu), ophip.MatMul(gpu), ophip.Swiglu(gpu)
+    a_rms = ophip.RmsNormArgs(c(16, 4096), xn, c(16, 4096), xd, c(4096), wd, 1e-5)
+    a_mm = ophip.MatMulArgs(c(16, 2048), gu, 0.0, c(16, 4096), xn, c(4096, 2048), wgud, 1.0)
+    a_sw = ophip.SwigluArgs(half, gu.ptr, half, gu.ptr + 1024 * 2)
+    ws = gpu.malloc(max(mm.scheme(a_mm, 1 << 30), 1))
+
+    def sequence():
+        rms.launch(a_rms, None, stream)
+        mm.launch(a_mm, ws, stream)
+        sw.launch(a_sw, None, stream)
+
+    say("launch graph: eager reference")
+    sequence()  # also lets mat_mul set up its per-stream counters before recording
+    want = gpu.to_host(gu, f16, 16 * 2048, stream=stream).copy()
+    stream.begin_capture()
+    sequence()
+    graph = stream.end_capture()
+    for rep in range(4):
+        gpu.memset(gu, 0, stream=stream)
+        say("launch graph: replay %d" % rep)
+        graph.launch(stream)
+        got = gpu.to_host(gu, f16, 16 * 2048, stream=stream)
+        assert np.array_equal(got, want), "replay %d differs from the eager result" % rep
+        rms.launch(a_rms, None, stream)  # eager work between replays
+        stream.synchronize()
+    graph.destroy()
