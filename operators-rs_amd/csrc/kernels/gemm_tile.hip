@@ -173,7 +173,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
     //   registers  : tile s+1 waits in `reg` while tile s is multiplied; MFMA fragments are
     //                double-buffered, the LDS reads of k-step kk+1 run under the MFMAs of kk
     //   k-step 0   : tile s+1 goes from registers to the other LDS buffer
-    //   k-step 1   : the global loads of tile s+2 refill the registers
+    //   k-steps 1..: the global loads of tile s+2 refill the registers, spread out evenly
     //   barrier    : before the last k-step (whose fragments are already in registers), so
     //                that step's MFMAs cover the first fragment reads of tile s+1
     // The code below is written in exactly that order, one memory operation of each kind
@@ -206,7 +206,6 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
     constexpr int NMFMA = TM * TN, NREAD = TM + TN, NLOAD = LP::NV + LQ::NV;
     static_assert(NREAD <= NMFMA && NLOAD <= NMFMA, "one memory operation of a kind per MFMA at most");
     static_assert(KK >= 2 && KK % 2 == 0, "fragment buffers alternate per k-step");
-    constexpr int LOAD_KK = KK > 2 ? 1 : 0;  // the k-step that carries the global loads
     // STORE: tile ks+1 exists (it is in `reg`); LOAD: tile ks+2 exists.
     auto step = [&](uint32_t ks, auto store, auto load) {
         constexpr bool STORE = decltype(store)::value, LOAD = decltype(load)::value;
@@ -222,9 +221,19 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
                     if (m < LP::NV) lp.commit_piece(nxt, m);
                     else lq.commit_piece(nxt + BM * LDK, m - LP::NV);
                 }
-                if (LOAD && KK > 2 && kk == LOAD_KK && m < NLOAD) {
-                    if (m < LP::NV) lp.fetch_piece(pnext, m);
-                    else lq.fetch_piece(qnext, m - LP::NV);
+                if constexpr (LOAD && KK > 2) {
+                    // The global loads are spread over k-steps 1 .. KK-2, one every SPREAD MFMAs: a
+                    // 1 KiB load occupies the CU's address path for 16 cycles, and a burst of them
+                    // blocks the issuing wave (and with it the MFMA pipe).  They stay a k-step behind
+                    // the LDS stores of the registers they refill: a load issued right after the
+                    // store of its register has to wait for that store to drain.
+                    constexpr int SLOTS = (KK - 2) * NMFMA, SPREAD = SLOTS / NLOAD;
+                    const int slot = (kk - 1) * NMFMA + m;
+                    if (kk >= 1 && slot % SPREAD == 0 && slot / SPREAD < NLOAD) {
+                        const int piece = slot / SPREAD;
+                        if (piece < LP::NV) lp.fetch_piece(pnext, piece);
+                        else lq.fetch_piece(qnext, piece - LP::NV);
+                    }
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
