@@ -103,6 +103,14 @@ extern "C" int ophip_layer_norm_launch(const ophip_layer_norm *op, const ophip_l
         const size_t nvec = d / vec_elems;
         unsigned G = nvec <= 64 * 8 ? 64 : nvec <= 256 * 8 ? 256 : 1024;
         while (G < 1024 && n * (G / 64) < 2048 && nvec >= 4 * (size_t)G) G *= 4;
+        const unsigned cus = (unsigned)op->dev->props.multiProcessorCount;
+        if (G == 64 && m.dt_a == OPHIP_DT_F16 && d <= 4096 && n >= (size_t)cus * 64 &&
+            n * d * (size_t)unit >= ((size_t)32 << 20)) {
+            // many rows and more bytes than the L2s hold: persistent workgroups (four per CU: 32 KiB
+            // of LDS each for scale and bias) whose waves stream rows
+            launch(op->dev->kernel("layer_norm", (base + "_rows").c_str()), Dim3{cus * 4}, Dim3{256}, 0, stream_of(qa), p);
+            return;
+        }
         const unsigned block = G < 256 ? 256 : G, rpb = block / G;
         const std::string name = base + (G == 64 ? "_g64" : G == 256 ? "_g256" : "_g1024");
         launch(op->dev->kernel("layer_norm", name.c_str()), Dim3{ceil_div(n, rpb)}, Dim3{block}, 0, stream_of(qa), p);

@@ -143,6 +143,82 @@ __device__ __forceinline__ void layer_norm_scalar(const LayerNormParams &p) {
         yr[j] = (TA)__builtin_fmaf((float)xr[j] - e, (float)sc[j] * k, (float)bi[j]);
 }
 
+// Many short rows of f16 (d <= 4096): a persistent workgroup converts scale and bias to f32
+// once into LDS, then each of its waves streams rows (dealt round-robin over all waves of the
+// grid) with the next row's loads in flight while the current one is reduced and written.
+// Per row the only global traffic left is x in and y out.
+template <typename TW>
+__device__ __forceinline__ void layer_norm_rows(const LayerNormParams &p) {
+    constexpr int CACHE = 8, MAXD = 4096;
+    __shared__ float s_scale[MAXD], s_bias[MAXD];
+    for (uint32_t j = threadIdx.x; j < p.d; j += blockDim.x) {
+        s_scale[j] = (float)reinterpret_cast<const TW *>(p.scale)[j];
+        s_bias[j] = (float)reinterpret_cast<const TW *>(p.bias)[j];
+    }
+    __syncthreads();
+
+    const uint32_t lane = threadIdx.x % WAVE;
+    const uint32_t waves = gridDim.x * (blockDim.x / WAVE);
+    uint32_t row = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+    const uint32_t nvec = p.d / 8;
+    if (row >= p.n) return;
+
+    Pack8 cur[CACHE], nxt[CACHE];
+    {
+        const char *xr = reinterpret_cast<const char *>(p.x) + (int64_t)row * p.nsx;
+#pragma unroll
+        for (int c = 0; c < CACHE; ++c) {
+            const uint32_t v = lane + c * WAVE;
+            if (v < nvec) cur[c].u = ld128(xr + (size_t)v * 16);
+        }
+    }
+    for (; row < p.n; row += waves) {
+        const uint32_t next = row + waves;
+        if (next < p.n) {
+            const char *xn = reinterpret_cast<const char *>(p.x) + (int64_t)next * p.nsx;
+#pragma unroll
+            for (int c = 0; c < CACHE; ++c) {
+                const uint32_t v = lane + c * WAVE;
+                if (v < nvec) nxt[c].u = ld128(xn + (size_t)v * 16);
+            }
+        }
+        float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+        for (int c = 0; c < CACHE; ++c) {
+            const uint32_t v = lane + c * WAVE;
+            if (v < nvec) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const float f = h2f(cur[c].e[i]);
+                    s1 += f;
+                    s2 += f * f;
+                }
+            }
+        }
+        s1 = wave_sum(s1);
+        s2 = wave_sum(s2);
+        float e, k;
+        mean_and_scale(s1, s2, p.d, p.epsilon, e, k);
+        char *yr = reinterpret_cast<char *>(p.y) + (int64_t)row * p.nsy;
+#pragma unroll
+        for (int c = 0; c < CACHE; ++c) {
+            const uint32_t v = lane + c * WAVE;
+            if (v < nvec) {
+                Pack8 o;
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    o.e[i] = f2h(__builtin_fmaf(h2f(cur[c].e[i]) - e, s_scale[v * 8 + i] * k, s_bias[v * 8 + i]));
+                st128(yr + (size_t)v * 16, o.u);
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < CACHE; ++c) cur[c] = nxt[c];
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(256) layer_norm_f16_f16_rows(LayerNormParams p) { layer_norm_rows<f16>(p); }
+extern "C" __global__ void __launch_bounds__(256) layer_norm_f16_f32_rows(LayerNormParams p) { layer_norm_rows<float>(p); }
+
 #define LAYER_NORM(NAME, TA, TW)                                                                                  \
     extern "C" __global__ void __launch_bounds__(256) layer_norm_##NAME##_g64(LayerNormParams p) {                \
         layer_norm_vec<TA, TW, 64>(p);                                                                            \
