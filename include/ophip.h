@@ -531,6 +531,31 @@ OPHIP_API int ophip_add_rows_launch(const ophip_add_rows *op, const ophip_add_ro
                                     const ophip_queue_alloc *queue_alloc);
 OPHIP_API void ophip_add_rows_destroy(ophip_add_rows *op);
 
+/* ---- conv: conv/args.rs:7-19, conv/im2col.rs:9-242 ------------------------- */
+/* y[n, m, hy, wy] = w[m, c, hk, wk] (*) x[n, c, h, w] + b[m], the crate's im2col composite:
+ * bias broadcast (rearrange), x unfolded into workspace (rearrange), one batched mat_mul
+ * with beta = 1.  pads must be zero; (h - ((hk-1)*dilation+1)) must divide by the stride. */
+typedef struct ophip_conv_args {
+    ophip_tensor_layout y_layout;
+    void *y_base;
+    ophip_tensor_layout x_layout;
+    const void *x_base;
+    ophip_tensor_layout w_layout;
+    const void *w_base;
+    ophip_tensor_layout b_layout;
+    const void *b_base;
+    size_t strides[2];
+    size_t dilations[2];
+    size_t pads[4];
+} ophip_conv_args;
+typedef struct ophip_conv ophip_conv;
+OPHIP_API int ophip_conv_create(ophip_device *dev, ophip_conv **out);
+OPHIP_API int ophip_conv_scheme(ophip_conv *op, const ophip_conv_args *args, size_t max_workspace_size,
+                                size_t *workspace_size);
+OPHIP_API int ophip_conv_launch(const ophip_conv *op, const ophip_conv_args *args, void *workspace,
+                                size_t workspace_len, const ophip_queue_alloc *queue_alloc);
+OPHIP_API void ophip_conv_destroy(ophip_conv *op);
+
 #ifdef __cplusplus
 }
 #endif

@@ -189,6 +189,13 @@ class _AddRowsArgs(ctypes.Structure):
                 ("src_base", ctypes.c_void_p), ("idx_layout", _Layout), ("idx_base", ctypes.c_void_p)]
 
 
+class _ConvArgs(ctypes.Structure):
+    _fields_ = [("y_layout", _Layout), ("y_base", ctypes.c_void_p), ("x_layout", _Layout),
+                ("x_base", ctypes.c_void_p), ("w_layout", _Layout), ("w_base", ctypes.c_void_p),
+                ("b_layout", _Layout), ("b_base", ctypes.c_void_p), ("strides", ctypes.c_size_t * 2),
+                ("dilations", ctypes.c_size_t * 2), ("pads", ctypes.c_size_t * 4)]
+
+
 # every symbol include/ophip.h declares
 EXPORTS = [
     "ophip_last_error", "ophip_status_name", "ophip_dtype_nbytes",
@@ -223,6 +230,7 @@ EXPORTS = [
     "ophip_gelu_create", "ophip_gelu_scheme", "ophip_gelu_launch", "ophip_gelu_destroy",
     "ophip_add_create", "ophip_add_scheme", "ophip_add_launch", "ophip_add_destroy", "ophip_add_plan",
     "ophip_add_rows_create", "ophip_add_rows_scheme", "ophip_add_rows_launch", "ophip_add_rows_destroy",
+    "ophip_conv_create", "ophip_conv_scheme", "ophip_conv_launch", "ophip_conv_destroy",
 ]
 
 _lib = None
@@ -717,6 +725,24 @@ class AddRowsArgs:
     def c(self):
         return _AddRowsArgs(self.dst_layout.c(), _p(self.dst_base), self.src_layout.c(), _p(self.src_base),
                             self.idx_layout.c(), _p(self.idx_base))
+
+
+class ConvArgs:
+    """conv/args.rs:7-19"""
+
+    def __init__(self, y_layout, y_base, x_layout, x_base, w_layout, w_base, b_layout, b_base,
+                 strides=(1, 1), dilations=(1, 1), pads=(0, 0, 0, 0)):
+        self.__dict__.update(locals())
+
+    def c(self):
+        return _ConvArgs(self.y_layout.c(), _p(self.y_base), self.x_layout.c(), _p(self.x_base),
+                         self.w_layout.c(), _p(self.w_base), self.b_layout.c(), _p(self.b_base),
+                         (ctypes.c_size_t * 2)(*self.strides), (ctypes.c_size_t * 2)(*self.dilations),
+                         (ctypes.c_size_t * 4)(*self.pads))
+
+
+class Conv(_Operator):
+    NAME = "conv"
 
 
 class RmsNorm(_Operator):

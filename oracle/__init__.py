@@ -316,3 +316,29 @@ def add_rows(dst, src, idx):
                                  src.strides[0], src.strides[1], _ptr(idx), idx.strides[0], idx.strides[1],
                                  batch, m, n, k, _DT[dst.dtype], _DT[idx.dtype]))
     return dst
+
+
+def conv(y, x, w, b, strides=(1, 1), dilations=(1, 1), pads=(0, 0, 0, 0)):
+    """The conv composite (conv/im2col.rs:85-242) over the CPU restatements: y[n,m,hy,wy] <- bias,
+    x unfolded to [n, c*hk*wk, hy*wy] by a strided copy, then y += w . unfolded (mat_mul, beta 1)."""
+    if any(pads):
+        raise OracleError(8)  # ArgsNotSupport: non-zero padding for im2col is not supported
+    n, c, h, wd_ = x.shape
+    m, _, hk, wk = w.shape
+    _, _, hy, wy = y.shape
+    (hs, ws), (hd, wd) = strides, dilations
+    hkd, wkd = (hk - 1) * hd + 1, (wk - 1) * wd + 1
+    if (h - hkd) % hs or (wd_ - wkd) % ws:
+        raise OracleError(7)  # StridesNotSupport: output size not divisible by strides
+    as_strided = np.lib.stride_tricks.as_strided
+    if not (hy == 1 or wy == 1 or y.strides[2] == wy * y.strides[3]):
+        raise OracleError(7)
+    c_y = as_strided(y, (n, m, hy * wy), (y.strides[0], y.strides[1], y.strides[2] if wy == 1 else y.strides[3]))
+    rearrange(c_y, as_strided(b, (n, m, hy * wy), (0, b.strides[0], 0)))
+    unfolded = np.empty((n, c, hk, wk, hy, wy), x.dtype)
+    xs = x.strides
+    rearrange(unfolded, as_strided(x, unfolded.shape, (xs[0], xs[1], xs[2] * hd, xs[3] * wd, xs[2] * hs, xs[3] * ws)))
+    w2 = np.ascontiguousarray(w).reshape(m, c * hk * wk) if not w.flags.c_contiguous else w.reshape(m, c * hk * wk)
+    a_w = as_strided(w2, (n, m, c * hk * wk), (0, w2.strides[0], w2.strides[1]))
+    mat_mul(c_y, 1.0, a_w, unfolded.reshape(n, c * hk * wk, hy * wy), 1.0)
+    return y
