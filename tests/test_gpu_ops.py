@@ -1003,3 +1003,44 @@ def test_recorded_launch_sequence_replays_like_eager_launches(gpu, stream):
         rms.launch(a_rms, None, stream)  # eager work between replays
         stream.synchronize()
     graph.destroy()
+
+
+# ------------------------------------------------------------- threading ----
+
+def test_one_operator_instance_launched_from_several_threads(gpu):
+    """launch takes &self in the reference and is internally synchronised (rms_norm/cuda/mod.rs:16,90-96):
+    one mat_mul and one rms_norm instance, four threads, each on its own stream with its own buffers."""
+    import threading
+
+    rms, mm = ophip.RmsNorm(gpu), ophip.MatMul(gpu)
+    L = TensorLayout
+    c = lambda *s: L.new_contiguous(dt.F16, list(s))
+    errors = []
+
+    def worker(seed):
+        try:
+            rng = np.random.default_rng(seed)
+            st = gpu.stream()
+            x = normal_f16(rng, (16, 2048))
+            w = rng.uniform(0.5, 1.5, 2048).astype(f32).astype(f16)
+            b = normal_f16(rng, (2048, 512), std=0.05)
+            xd, wd, bd = gpu.from_host(x), gpu.from_host(w), gpu.from_host(b)
+            xn, out = gpu.malloc(x.nbytes), gpu.malloc(16 * 512 * 2)
+            ref_n = oracle.rms_norm(np.empty_like(x), x, w, 1e-5)
+            ref = oracle.mat_mul(np.zeros((16, 512), f16), 0.0, ref_n, b, 1.0)
+            for _ in range(25):
+                rms.launch(ophip.RmsNormArgs(c(16, 2048), xn, c(16, 2048), xd, c(2048), wd, 1e-5), None, st)
+                mm.launch(ophip.MatMulArgs(c(16, 512), out, 0.0, c(16, 2048), xn, c(2048, 512), bd, 1.0), None, st)
+            got = gpu.to_host(out, f16, 16 * 512, stream=st).reshape(16, 512)
+            assert_close_f16(got, ref, "thread %d" % seed, abs_tol=4e-3)
+            st.synchronize()
+        except Exception as e:  # surfaced in the main thread
+            errors.append(e)
+
+    say("4 threads x 25 launches of shared operator instances")
+    threads = [threading.Thread(target=worker, args=(s,)) for s in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
