@@ -172,3 +172,25 @@ def test_attention_kv_cached_errors_and_scheme(gpu, stream):
     with pytest.raises(ophip.SchemeError) as e:
         op.scheme(bad, 0)
     assert e.value.kind == "ShapeMismatch"
+
+
+def test_decode_layer_chain_matches_the_oracle_end_to_end(gpu, stream):
+    """The benchmark's step - rms_norm, QKV mat_mul, rope (q, k), QK^T, causal softmax, PV, O-proj, rms_norm,
+    gate/up, swiglu, down at Llama-7B decode shapes - run once on the GPU and once through the oracle on
+    the same seeded weights; every intermediate rounding to f16 happens in both."""
+    import bench
+
+    rng = np.random.default_rng(0)
+    layer = bench.Layer(ophip, gpu, rng, host=True)
+    print("decode layer chain, 12 launches", flush=True)
+    layer.step(stream)
+    out = gpu.to_host(layer.d["out"], f16, bench.NT * bench.D, stream=stream).reshape(bench.NT, bench.D)
+    ref = bench.cpu_layer_step(oracle, layer.h, min(oracle.max_threads(), 16))
+    # Twelve chained operators, each rounding to f16: single-ulp differences of an intermediate (summation
+    # order in mat_mul) spread through the later products, so the per-operator outlier rule does not apply.
+    # The bar here: every element within 1e-2 of the output scale, and the typical element much closer.
+    err = np.abs(out.astype(np.float64) - ref.astype(np.float64))
+    scale = float(np.abs(ref.astype(np.float64)).max())
+    print("decode layer: max err %.3g, median err %.3g, output scale %.3g" % (err.max(), np.median(err), scale), flush=True)
+    assert err.max() <= 1e-2 * scale, err.max() / scale
+    assert np.median(err) <= 1e-3 * scale, np.median(err) / scale
