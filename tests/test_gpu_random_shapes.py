@@ -1,0 +1,187 @@
+"""Seeded sweeps over random shapes and row paddings for every operator, against the oracle.
+Each device tensor sits inside a buffer with 4 KiB of guard bytes on both sides and random
+padding between rows; after the launch everything outside the tensor's elements must be
+unchanged, so a stray store is caught as a failed assertion."""
+import numpy as np
+import pytest
+
+import ophip
+import oracle
+from helpers import assert_close_f16
+from ophip import TensorLayout, dt
+
+pytestmark = pytest.mark.gpu
+
+f16, f32 = np.float16, np.float32
+GUARD = 4096
+
+
+def say(msg):
+    print(msg, flush=True)
+
+
+class Guarded:
+    """A [rows.., cols] tensor with row pitch `cols + pad` elements inside guard bytes."""
+
+    def __init__(self, gpu, rng, shape, dtype, pad, fill=None, scale=1.0):
+        self.gpu, self.shape, self.dtype = gpu, tuple(shape), np.dtype(dtype)
+        lead = int(np.prod(shape[:-1])) if len(shape) > 1 else 1
+        pitch = shape[-1] + pad
+        n = lead * pitch
+        body = (rng.standard_normal(n).astype(f32) * f32(scale)).astype(dtype) if fill is None else np.full(n, fill, dtype)
+        raw = np.concatenate([rng.integers(0, 256, GUARD, dtype=np.uint8), body.view(np.uint8),
+                              rng.integers(0, 256, GUARD, dtype=np.uint8)])
+        self.raw = raw
+        it = self.dtype.itemsize
+        strides = [it]
+        mul = pitch * it
+        for d in reversed(shape[:-1]):
+            strides.append(mul)
+            mul *= d
+        self.strides = tuple(reversed(strides))
+        self.mem = gpu.from_host(raw)
+        self.ptr = self.mem.ptr + GUARD
+        self.layout = TensorLayout(ophip.NP_DT[self.dtype], list(shape), list(self.strides))
+
+    def view(self, raw=None):
+        raw = self.raw if raw is None else raw
+        return np.lib.stride_tricks.as_strided(raw[GUARD:].view(self.dtype), self.shape, self.strides, writeable=True)
+
+    def fetch(self, stream):
+        """Device contents; asserts that nothing outside the tensor's elements changed."""
+        got = self.gpu.to_host(self.mem, np.uint8, self.raw.size, stream=stream)
+        mask = np.ones(self.raw.size, bool)
+        inside = np.lib.stride_tricks.as_strided(mask[GUARD:].view(np.uint8), tuple(self.shape) + (self.dtype.itemsize,),
+                                                 self.strides + (1,), writeable=True)
+        inside[...] = 0
+        assert np.array_equal(got[mask.view(bool)], self.raw[mask.view(bool)]), "bytes outside the tensor were written"
+        return self.view(got)
+
+
+def test_random_rms_norm_and_layer_norm(gpu, stream):
+    rng = np.random.default_rng(100)
+    rms, ln = ophip.RmsNorm(gpu), ophip.LayerNorm(gpu)
+    for case in range(30):
+        n = int(rng.integers(1, 70))
+        d = int(rng.choice([8, 24, 120, 128, 1000, 1024, 4096, 4104, 5000, 8192, 16384, 16400]))
+        adt, wdt = (f16, f16) if case % 3 == 0 else (f16, f32) if case % 3 == 1 else (f32, f32)
+        pad = int(rng.choice([0, 8, 3]))
+        x, y = Guarded(gpu, rng, (n, d), adt, pad), Guarded(gpu, rng, (n, d), adt, int(rng.choice([0, 8])))
+        w, b = Guarded(gpu, rng, (d,), wdt, 0), Guarded(gpu, rng, (d,), wdt, 0)
+        say("random rms_norm/layer_norm %d: n=%d d=%d pad=%d %s/%s" % (case, n, d, pad, adt.__name__, wdt.__name__))
+        rms.launch(ophip.RmsNormArgs(y.layout, y.ptr, x.layout, x.ptr, w.layout, w.ptr, 1e-5), None, stream)
+        got = y.fetch(stream)
+        ref = oracle.rms_norm(np.empty((n, d), adt), x.view(), w.view(), 1e-5)
+        if adt is f16: assert_close_f16(got, ref, "rms_norm")
+        else: np.testing.assert_allclose(got, ref, rtol=3e-5, atol=3e-6)
+        ln.launch(ophip.LayerNormArgs(y.layout, y.ptr, x.layout, x.ptr, w.layout, w.ptr, b.layout, b.ptr, 1e-5), None, stream)
+        got = y.fetch(stream)
+        ref = oracle.layer_norm(np.empty((n, d), adt), x.view(), w.view(), b.view(), 1e-5)
+        if adt is f16: assert_close_f16(got, ref, "layer_norm", abs_tol=4e-3)
+        else: np.testing.assert_allclose(got, ref, rtol=1e-4, atol=1e-4)
+
+
+def test_random_softmax_swiglu_gelu(gpu, stream):
+    rng = np.random.default_rng(101)
+    sm, sw, ge = ophip.FusedSoftmax(gpu), ophip.Swiglu(gpu), ophip.Gelu(gpu)
+    for case in range(30):
+        nh, seq = int(rng.integers(1, 5)), int(rng.integers(1, 20))
+        att = seq + int(rng.choice([0, 1, 7, 100, 500, 2040, 2049, 5000]))
+        pad = int(rng.choice([0, 8, 5]))
+        a = Guarded(gpu, rng, (nh, seq, att), f16, pad, scale=2.0)
+        mask = ophip.AttnMask.CAUSAL if case % 4 else ophip.AttnMask.NONE
+        say("random softmax %d: nh=%d seq=%d att=%d pad=%d mask=%d" % (case, nh, seq, att, pad, mask))
+        sm.launch(ophip.FusedSoftmaxArgs(mask, a.layout, a.ptr), None, stream)
+        got = a.fetch(stream)
+        ref = oracle.fused_softmax(a.view().copy(), causal=bool(mask))
+        assert_close_f16(got, ref, "softmax")
+        assert np.array_equal(got == 0, ref == 0)
+        n, d = int(rng.integers(1, 40)), int(rng.choice([8, 40, 1001, 2048, 11008]))
+        g, u = Guarded(gpu, rng, (n, d), f16, pad, scale=2.0), Guarded(gpu, rng, (n, d), f16, int(rng.choice([0, 8])))
+        say("random swiglu/gelu %d: n=%d d=%d" % (case, n, d))
+        sw.launch(ophip.SwigluArgs(g.layout, g.ptr, u.layout, u.ptr), None, stream)
+        assert_close_f16(g.fetch(stream), oracle.swiglu(g.view().copy(), u.view()), "swiglu")
+        ge.launch(ophip.GeluArgs(u.layout, u.ptr), None, stream)
+        assert_close_f16(u.fetch(stream), oracle.gelu(u.view().copy()), "gelu")
+
+
+def test_random_rope(gpu, stream):
+    rng = np.random.default_rng(102)
+    rope = ophip.Rope(gpu)
+    for case in range(20):
+        nt, nh = int(rng.integers(1, 40)), int(rng.integers(1, 9))
+        dh = int(rng.choice([2, 8, 20, 64, 128, 256]))
+        pad = int(rng.choice([0, 8, 2]))
+        t = Guarded(gpu, rng, (nt, nh, dh), f16, pad)
+        pdt = np.uint32 if case % 2 else np.uint64
+        pos = rng.integers(0, 5000, nt).astype(pdt)
+        pd = gpu.from_host(pos)
+        empty = TensorLayout(dt.F16, [0, dh], [2 * dh, 2])
+        say("random rope %d: nt=%d nh=%d dh=%d pad=%d %s" % (case, nt, nh, dh, pad, pdt.__name__))
+        rope.launch(ophip.RopeArgs(t.layout, t.ptr, TensorLayout.of(pos), pd, empty, None, empty, None, 1e4), None, stream)
+        assert_close_f16(t.fetch(stream), oracle.rope(t.view().copy(), pos, 1e4), "rope")
+
+
+def test_random_rearrange_and_add(gpu, stream):
+    rng = np.random.default_rng(103)
+    re, ad = ophip.Rearrange(gpu), ophip.Add(gpu)
+    for case in range(30):
+        nd = int(rng.integers(1, 5))
+        shape = [int(rng.integers(1, 9)) for _ in range(nd - 1)] + [int(rng.choice([1, 3, 8, 16, 40]))]
+        perm = list(rng.permutation(nd))
+        src = Guarded(gpu, rng, shape, f16, int(rng.choice([0, 8, 1])))
+        dst_store = Guarded(gpu, rng, [shape[p] for p in perm], f16, int(rng.choice([0, 8])), fill=0)
+        inv = list(np.argsort(perm))
+        dst_layout = TensorLayout(dt.F16, shape, [dst_store.strides[inv[i]] for i in range(nd)])
+        say("random rearrange %d: shape=%s perm=%s" % (case, shape, perm))
+        re.launch(ophip.RearrangeArgs(dst_layout, dst_store.ptr, src.layout, src.ptr), None, stream)
+        got = dst_store.fetch(stream)
+        assert np.array_equal(got.view(np.uint16), src.view().transpose(perm).view(np.uint16))
+        b = Guarded(gpu, rng, shape, f16, int(rng.choice([0, 8])))
+        c = Guarded(gpu, rng, shape, f16, int(rng.choice([0, 8])), fill=0)
+        bl = b.layout
+        if nd > 1 and case % 3 == 0:  # broadcast b over the first dimension
+            bl = TensorLayout(dt.F16, shape, [0] + list(b.strides[1:]))
+        say("random add %d" % case)
+        ad.launch(ophip.AddArgs(c.layout, c.ptr, src.layout, src.ptr, bl, b.ptr), None, stream)
+        bv = b.view() if bl is b.layout else np.broadcast_to(b.view()[:1], shape)
+        assert np.array_equal(c.fetch(stream), (src.view().astype(f32) + bv.astype(f32)).astype(f16))
+
+
+def test_random_mat_mul(gpu, stream):
+    """Shapes straddle the kernel boundaries: 64 / 65 rows, widths that are not multiples of 8 or 128, K that is
+    not a multiple of 32, tile-sized multiples of 128 / 256, batches with broadcast b."""
+    rng = np.random.default_rng(104)
+    mm = ophip.MatMul(gpu)
+    oracle.set_threads(8)
+    try:
+        for case in range(40):
+            m = int(rng.choice([1, 5, 16, 17, 33, 64, 65, 100, 128, 256, 384]))
+            n = int(rng.choice([8, 24, 100, 128, 136, 256, 512, 1000]))
+            k = int(rng.choice([1, 7, 32, 64, 96, 100, 128, 512, 1000]))
+            bt = int(rng.choice([1, 1, 2, 3]))
+            ta, tb, tc = (bool(rng.integers(0, 2)) for _ in range(3))
+            pa, pb, pc = (int(rng.choice([0, 8])) for _ in range(3))
+            A = Guarded(gpu, rng, (bt, k, m) if ta else (bt, m, k), f16, pa)
+            B = Guarded(gpu, rng, (bt, n, k) if tb else (bt, k, n), f16, pb, scale=0.1)
+            C = Guarded(gpu, rng, (bt, n, m) if tc else (bt, m, n), f16, pc)
+            tr = lambda g, t: (TensorLayout(dt.F16, [g.shape[0], g.shape[2], g.shape[1]], [g.strides[0], g.strides[2], g.strides[1]]),
+                               g.view().transpose(0, 2, 1)) if t else (g.layout, g.view())
+            (al, av), (bl, bv), (cl, cv) = tr(A, ta), tr(B, tb), tr(C, tc)
+            if bt > 1 and case % 4 == 0:  # one b for every batch
+                bl = TensorLayout(dt.F16, bl.shape, [0] + list(bl.strides[1:]))
+                bv = np.broadcast_to(bv[:1], bv.shape)
+            alpha, beta = float(rng.choice([1.0, 0.5, -1.25])), float(rng.choice([0.0, 1.0, 0.5]))
+            args = ophip.MatMulArgs(cl, C.ptr, beta, al, A.ptr, bl, B.ptr, alpha)
+            say("random mat_mul %d: bt=%d m=%d n=%d k=%d t=%d%d%d pads=%d%d%d a=%g b=%g [%s]" % (
+                case, bt, m, n, k, ta, tb, tc, pa, pb, pc, alpha, beta, mm.describe(args)))
+            ref = cv.copy()
+            oracle.mat_mul(ref, beta, av, np.ascontiguousarray(bv) if bv.strides[0] == 0 and bt > 1 else bv, alpha)
+            mm.launch(args, None, stream)
+            got = C.fetch(stream)
+            got = got.transpose(0, 2, 1) if tc else got
+            scale = float(np.abs(ref.astype(np.float64)).max()) + 1e-3
+            err = np.abs(got.astype(np.float64) - ref.astype(np.float64)).max()
+            assert err <= 2e-3 + 4e-3 * scale, (err, scale)
+    finally:
+        oracle.set_threads(1)
