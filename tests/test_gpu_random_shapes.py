@@ -2,6 +2,8 @@
 Each device tensor sits inside a buffer with 4 KiB of guard bytes on both sides and random
 padding between rows; after the launch everything outside the tensor's elements must be
 unchanged, so a stray store is caught as a failed assertion."""
+import os
+
 import numpy as np
 import pytest
 
@@ -14,6 +16,8 @@ pytestmark = pytest.mark.gpu
 
 f16, f32 = np.float16, np.float32
 GUARD = 4096
+# OPHIP_TEST_SWEEPS=<n> repeats every sweep with n different seeds (default 1)
+SWEEPS = pytest.mark.parametrize("sweep", range(int(os.environ.get("OPHIP_TEST_SWEEPS", "1"))))
 
 
 def say(msg):
@@ -58,8 +62,9 @@ class Guarded:
         return self.view(got)
 
 
-def test_random_rms_norm_and_layer_norm(gpu, stream):
-    rng = np.random.default_rng(100)
+@SWEEPS
+def test_random_rms_norm_and_layer_norm(gpu, stream, sweep):
+    rng = np.random.default_rng(100 + 1000 * sweep)
     rms, ln = ophip.RmsNorm(gpu), ophip.LayerNorm(gpu)
     for case in range(30):
         n = int(rng.integers(1, 70))
@@ -81,8 +86,9 @@ def test_random_rms_norm_and_layer_norm(gpu, stream):
         else: np.testing.assert_allclose(got, ref, rtol=1e-4, atol=1e-4)
 
 
-def test_random_softmax_swiglu_gelu(gpu, stream):
-    rng = np.random.default_rng(101)
+@SWEEPS
+def test_random_softmax_swiglu_gelu(gpu, stream, sweep):
+    rng = np.random.default_rng(101 + 1000 * sweep)
     sm, sw, ge = ophip.FusedSoftmax(gpu), ophip.Swiglu(gpu), ophip.Gelu(gpu)
     for case in range(30):
         nh, seq = int(rng.integers(1, 5)), int(rng.integers(1, 20))
@@ -105,8 +111,9 @@ def test_random_softmax_swiglu_gelu(gpu, stream):
         assert_close_f16(u.fetch(stream), oracle.gelu(u.view().copy()), "gelu")
 
 
-def test_random_rope(gpu, stream):
-    rng = np.random.default_rng(102)
+@SWEEPS
+def test_random_rope(gpu, stream, sweep):
+    rng = np.random.default_rng(102 + 1000 * sweep)
     rope = ophip.Rope(gpu)
     for case in range(20):
         nt, nh = int(rng.integers(1, 40)), int(rng.integers(1, 9))
@@ -122,8 +129,9 @@ def test_random_rope(gpu, stream):
         assert_close_f16(t.fetch(stream), oracle.rope(t.view().copy(), pos, 1e4), "rope")
 
 
-def test_random_rearrange_and_add(gpu, stream):
-    rng = np.random.default_rng(103)
+@SWEEPS
+def test_random_rearrange_and_add(gpu, stream, sweep):
+    rng = np.random.default_rng(103 + 1000 * sweep)
     re, ad = ophip.Rearrange(gpu), ophip.Add(gpu)
     for case in range(30):
         nd = int(rng.integers(1, 5))
@@ -148,10 +156,11 @@ def test_random_rearrange_and_add(gpu, stream):
         assert np.array_equal(c.fetch(stream), (src.view().astype(f32) + bv.astype(f32)).astype(f16))
 
 
-def test_random_mat_mul(gpu, stream):
+@SWEEPS
+def test_random_mat_mul(gpu, stream, sweep):
     """Shapes straddle the kernel boundaries: 64 / 65 rows, widths that are not multiples of 8 or 128, K that is
     not a multiple of 32, tile-sized multiples of 128 / 256, batches with broadcast b."""
-    rng = np.random.default_rng(104)
+    rng = np.random.default_rng(104 + 1000 * sweep)
     mm = ophip.MatMul(gpu)
     oracle.set_threads(8)
     try:
