@@ -40,18 +40,24 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 // simply take 32 consecutive slots and the epilogue maps slots back to rows with
 // row(s) = (s % (R / 8)) * 8 + s / (R / 8).
 //
-// Within an LDS row.  TK = 32: rows are padded to 40 halves (80 bytes), so that 16-byte
-// reads of consecutive rows spread over the banks.  TK = 64: rows are exactly 128 bytes and
-// the eight 16-byte groups of row s are stored at position (group ^ (s & 7)): measured, a
-// wave's ds_read_b128 of 32 rows x 2 groups runs 1.6x faster on this layout than on padded
-// rows, the transposing stores stay conflict-free, and the tile needs 128 KiB instead of 144.
+// Within an LDS row.  Measured with SQ_LDS_BANK_CONFLICT / SQ_LDS_IDX_ACTIVE: a ds_read_b128
+// is served 16 lanes per cycle over 64 banks of 4 bytes (4 cycles when conflict-free), a
+// ds_write_b128 8 lanes per cycle over 128 bytes (8 cycles).  So 16 consecutive rows read at
+// the same k must land on 16 different 16-byte groups modulo 256 bytes, and the 8 consecutive
+// rows a transposing store touches on 8 different groups modulo 128 bytes.
+// TK = 32: rows are padded to 40 halves (80 bytes).  TK = 64: rows are exactly 128 bytes and
+// the eight 16-byte groups of row s are stored at position group ^ key(s),
+// key(s) = (s & 7) ^ ((s >> 3) & 1): distinct over any 8 consecutive rows, and rows s, s + 8
+// (same parity, hence the same 128-byte half of the 256-byte bank line) differ in the low
+// bit.  The fragment reads, the 16-byte stores of K-contiguous operands (8 lanes per row) and
+// the transposing stores are all conflict-free, and the tile needs 128 KiB instead of 144.
 template <int TK>
 struct TileRow {
     static constexpr bool SWIZZLE = TK == 64;
     static constexpr int LDK = SWIZZLE ? TK : TK + 8;  // row pitch in halves
     // offset in halves of 16-byte group `g` of LDS row `s`
     __device__ static __forceinline__ uint32_t at(uint32_t s, uint32_t g) {
-        return s * LDK + (SWIZZLE ? (g ^ (s & 7)) : g) * 8;
+        return s * LDK + (SWIZZLE ? (g ^ (s & 7) ^ ((s >> 3) & 1)) : g) * 8;
     }
 };
 
@@ -206,11 +212,11 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
     __syncthreads();
 
     Pack8 a[2][TM], b[2][TN];
-    // Fragment addresses.  Every slot a lane reads has the same low three bits (l32 & 7), so
+    // Fragment addresses.  Every slot a lane reads has the same low four bits (l32 & 15), so
     // the position of k-step kk's group inside the row is one value per kk for all fragments.
     uint32_t koff[KK];
 #pragma unroll
-    for (int kk = 0; kk < KK; ++kk) koff[kk] = TileRow<TK>::at(l32 & 7, 2 * kk + lk) - (l32 & 7) * LDK;
+    for (int kk = 0; kk < KK; ++kk) koff[kk] = TileRow<TK>::at(l32 & 15, 2 * kk + lk) - (l32 & 15) * LDK;
     const uint32_t a_row = LP::reader_slot(wm, 0, l32) * LDK;
     const uint32_t b_row = BM * LDK + LQ::reader_slot(wn, 0, l32) * LDK;
     // fragment r of k-step kk of the tile at `tile`: r < TM is a P fragment, the rest are Q's
