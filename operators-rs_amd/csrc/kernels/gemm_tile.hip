@@ -99,7 +99,10 @@ struct TileLoader {
 
     // `tile` (wave-uniform) points at element (row0, k0) of the operand.  The copy is cut
     // into NV pieces so that the main loop can place them one by one between MFMAs.
+    // The empty asm keeps the compiler from widening the offset to 64 bits outside the loop: as
+    // "uniform base + 32-bit lane offset" the load needs no address arithmetic.
     __device__ __forceinline__ void fetch_piece(const f16 *tile, int v) {
+        asm volatile("" : "+v"(voff[v]));
         reg[v] = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(tile) + voff[v]);
     }
     __device__ __forceinline__ void fetch(const f16 *tile) {
@@ -144,7 +147,13 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
     constexpr int LDK = TileRow<TK>::LDK;
     constexpr int WM = BM / 2, WN = BN / 2;  // wave tile
     constexpr int TM = WM / 32, TN = WN / 32;
-    __shared__ f16 lds[2][(BM + BN) * LDK];
+    // LDS: P buffer 0, P buffer 1, Q buffer 0, Q buffer 1.  Both buffers of an operand are within
+    // 64 KiB of each other, so one address register per lane serves both through the
+    // instruction's immediate offset.
+    __shared__ f16 lds[2 * (BM + BN) * LDK];
+    constexpr uint32_t Q_REGION = 2 * BM * LDK;
+    auto p_buf = [&](int b) { return lds + b * (BM * LDK); };
+    auto q_buf = [&](int b) { return lds + Q_REGION + b * (BN * LDK); };
 
     // XCD-aware tile order: ids are dealt round-robin over 8 XCDs; give each XCD a
     // contiguous run of tiles, walked in groups of 8 tile-rows so panels are reused.
@@ -201,13 +210,24 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
     // The code below is written in exactly that order, one memory operation of each kind
     // after each MFMA, and sched_barrier(0) after every such group keeps the compiler from
     // regrouping them.
-    lp.fetch(ptile);
-    lq.fetch(qtile);
-    lp.commit(lds[0]);
-    lq.commit(lds[0] + BM * LDK);
-    if (ksteps > 1) {
-        lp.fetch(ptile + pstep);
-        lq.fetch(qtile + qstep);
+    // Copy piece i in the order the main loop uses (the waits the compiler derives for the loop
+    // merge the prologue's order with the loop's: they must agree or the loop waits too long).
+    constexpr bool Q_FIRST = PK && !QK, ALTERNATE = PK && QK && LP::NV == LQ::NV;
+    auto piece_is_q = [&](int i) { return ALTERNATE ? bool(i & 1) : ((i >= LP::NV) != Q_FIRST) ; };
+    auto piece_v = [&](int i) { return ALTERNATE ? i / 2 : (Q_FIRST ? (i < LQ::NV ? i : i - LQ::NV) : (i < LP::NV ? i : i - LP::NV)); };
+    auto fetch_all = [&](const f16 *pt, const f16 *qt) {
+#pragma unroll
+        for (int i = 0; i < LP::NV + LQ::NV; ++i) {
+            if (piece_is_q(i)) lq.fetch_piece(qt, piece_v(i));
+            else lp.fetch_piece(pt, piece_v(i));
+        }
+    };
+    fetch_all(ptile, qtile);
+    lp.commit(p_buf(0));
+    lq.commit(q_buf(0));
+    {
+        const uint32_t k1 = min(1u, ksteps - 1);
+        fetch_all(ptile + k1 * pstep, qtile + k1 * qstep);
     }
     __syncthreads();
 
@@ -218,13 +238,14 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) koff[kk] = TileRow<TK>::at(l32 & 15, 2 * kk + lk) - (l32 & 15) * LDK;
     const uint32_t a_row = LP::reader_slot(wm, 0, l32) * LDK;
-    const uint32_t b_row = BM * LDK + LQ::reader_slot(wn, 0, l32) * LDK;
+    const uint32_t b_row = Q_REGION + LQ::reader_slot(wn, 0, l32) * LDK;
     // fragment r of k-step kk of the tile at `tile`: r < TM is a P fragment, the rest are Q's
-    auto read_one = [&](int buf, const f16 *tile, int kk, int r) {
+    // `from`: LDS buffer 0 or 1
+    auto read_one = [&](int buf, int from, int kk, int r) {
         if (r < TM)
-            a[buf][r].u = ld128(tile + a_row + koff[kk] + (LP::reader_slot(wm, r, l32) - LP::reader_slot(wm, 0, l32)) * LDK);
+            a[buf][r].u = ld128(lds + (a_row + koff[kk]) + from * (BM * LDK) + (LP::reader_slot(wm, r, l32) - LP::reader_slot(wm, 0, l32)) * LDK);
         else
-            b[buf][r - TM].u = ld128(tile + b_row + koff[kk] + (LQ::reader_slot(wn, r - TM, l32) - LQ::reader_slot(wn, 0, l32)) * LDK);
+            b[buf][r - TM].u = ld128(lds + (b_row + koff[kk]) + from * (BN * LDK) + (LQ::reader_slot(wn, r - TM, l32) - LQ::reader_slot(wn, 0, l32)) * LDK);
     };
     auto mfma_one = [&](int buf, int m) {
         const int tm = m / TN, tn = m % TN;
@@ -233,58 +254,100 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
     constexpr int NMFMA = TM * TN, NREAD = TM + TN, NLOAD = LP::NV + LQ::NV;
     static_assert(NREAD <= NMFMA && NLOAD <= NMFMA, "one memory operation of a kind per MFMA at most");
     static_assert(KK >= 2 && KK % 2 == 0, "fragment buffers alternate per k-step");
-    // STORE: tile ks+1 exists (it is in `reg`); LOAD: tile ks+2 exists.
-    auto step = [&](uint32_t ks, auto store, auto load) {
-        constexpr bool STORE = decltype(store)::value, LOAD = decltype(load)::value;
-        f16 *cur = lds[ks & 1], *nxt = lds[(ks + 1) & 1];
-        const f16 *pnext = ptile + (ks + 2) * pstep, *qnext = qtile + (ks + 2) * qstep;
+    // Issue budget.  The wave issues in order and an MFMA occupies its pipe for 32 cycles, so
+    // whatever stands between two MFMAs must issue in less than that or the pipe runs dry:
+    // a ds_write_b128 alone takes about 20 cycles, a global load with its address arithmetic
+    // about 16, a ds_read_b128 4.  Hence at most one memory operation per MFMA: fragment reads
+    // after the even-numbered MFMAs of a tile, stores and loads after the odd-numbered ones.
+    //   256 x 256 x 64 (4 k-steps of 16 MFMAs, 16 copy pieces): odd position o = 0..31 of a tile's
+    //   loop holds the store of piece ST[i] = o or the load of piece LD[i] = o, pieces numbered
+    //   in store order.  Stores end before the barrier (o < 24).  Both operands K-contiguous:
+    //   two stores, then the load that refills the first of them, and so on, which leaves a
+    //   load 19 to 30 positions (of 64 cycles) to arrive.  Otherwise: all stores, then all
+    //   loads, the row-contiguous operand first, because each of its stores reads all of its
+    //   registers.
+    struct Sched { int st[16], ld[16]; };
+    constexpr Sched SCH = (PK && QK) ? Sched{{0, 1, 3, 4, 6, 7, 9, 10, 12, 13, 15, 16, 18, 19, 21, 22},
+                                             {2, 5, 8, 11, 14, 17, 20, 23, 24, 25, 26, 27, 28, 29, 30, 31}}
+                                     : Sched{{0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15},
+                                             {16, 17, 18, 19, 20, 21, 22, 23, 24, 25, 26, 27, 28, 29, 30, 31}};
+    static_assert(KK == 2 || (LP::NV == 8 && LQ::NV == 8 && NMFMA == 16 && KK == 4), "tables are for the 256 x 256 x 64 tile");
+    // fragments in the order the next k-step's MFMAs want them: a0 b0 b1 b2 b3 a1 a2 a3
+    constexpr int RORDER[8] = {0, TM, TM + 1, TM + 2, TM + 3, 1, 2, 3};
+    // Every tile runs the same code: past the end of K the loads fetch the last tile again, the
+    // stores put it into the buffer nobody reads any more and the fragment reads of a tile that
+    // does not exist are not used.  (Separate code for the last two tiles costs more in
+    // registers, through the extra control flow, than the few redundant copies.)
+    auto step = [&](uint32_t ks, auto parity) {
+        constexpr bool STORE = true, LOAD = true;
+        constexpr int cur = decltype(parity)::value, nxt = 1 - cur;  // = ks % 2
+        const uint32_t knext = min(ks + 2, ksteps - 1);
+        const f16 *pnext = ptile + knext * pstep, *qnext = qtile + knext * qstep;
+        auto piece_op = [&](int i, bool is_store) {
+            const bool is_q = piece_is_q(i);
+            const int v = piece_v(i);
+            if (is_store) {
+                if (is_q) lq.commit_piece(q_buf(nxt), v);
+                else lp.commit_piece(p_buf(nxt), v);
+            } else {
+                if (is_q) lq.fetch_piece(qnext, v);
+                else lp.fetch_piece(pnext, v);
+            }
+        };
+        // what follows MFMA number `slot` of the tile (KK == 4)
+        auto after_mfma = [&](int slot, bool reads, int next_buf, int from, int next_kk) {
+            if (slot % 2 == 0) {
+                if (reads) read_one(next_buf, from, next_kk, RORDER[(slot % NMFMA) / 2]);
+            } else {
+                const int o = slot / 2;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    if (STORE && SCH.st[i] == o) piece_op(i, true);
+                    if (LOAD && SCH.ld[i] == o) piece_op(i, false);
+                }
+            }
+        };
 #pragma unroll
         for (int kk = 0; kk < KK - 1; ++kk) {
 #pragma unroll
             for (int m = 0; m < NMFMA; ++m) {
                 mfma_one(kk & 1, m);
-                if (m < NREAD) read_one((kk + 1) & 1, cur, kk + 1, m);
-                if (STORE && kk == 0 && m < NLOAD) {
-                    if (m < LP::NV) lp.commit_piece(nxt, m);
-                    else lq.commit_piece(nxt + BM * LDK, m - LP::NV);
-                }
-                if constexpr (LOAD && KK > 2) {
-                    // The global loads are spread over k-steps 1 .. KK-2, one every SPREAD MFMAs: a
-                    // 1 KiB load occupies the CU's address path for 16 cycles, and a burst of them
-                    // blocks the issuing wave (and with it the MFMA pipe).  They stay a k-step behind
-                    // the LDS stores of the registers they refill: a load issued right after the
-                    // store of its register has to wait for that store to drain.
-                    constexpr int SLOTS = (KK - 2) * NMFMA, SPREAD = SLOTS / NLOAD;
-                    const int slot = (kk - 1) * NMFMA + m;
-                    if (kk >= 1 && slot % SPREAD == 0 && slot / SPREAD < NLOAD) {
-                        const int piece = slot / SPREAD;
-                        if (piece < LP::NV) lp.fetch_piece(pnext, piece);
-                        else lq.fetch_piece(qnext, piece - LP::NV);
-                    }
+                if constexpr (KK > 2) {
+                    after_mfma(kk * NMFMA + m, true, (kk + 1) & 1, cur, kk + 1);
+                } else {
+                    // two k-steps of 4 MFMAs per tile: reads and stores under the first, then all loads
+                    if (m < NREAD) read_one((kk + 1) & 1, cur, kk + 1, m);
+                    if (STORE && m < NLOAD) piece_op(m, true);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (LOAD && KK == 2 && kk == 0) {
-                lp.fetch(pnext);
-                lq.fetch(qnext);
+                fetch_all(pnext, qnext);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
+        // every store of this tile's loop is above this line
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int m = 0; m < NMFMA; ++m) {
             mfma_one((KK - 1) & 1, m);
-            if (STORE && m < NREAD) read_one(0, nxt, 0, m);
+            if constexpr (KK > 2) after_mfma((KK - 1) * NMFMA + m, STORE, 0, nxt, 0);
+            else if (STORE && m < NREAD) read_one(0, nxt, 0, m);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
 #pragma unroll
-    for (int r = 0; r < NREAD; ++r) read_one(0, lds[0], 0, r);
+    for (int r = 0; r < NREAD; ++r) read_one(0, 0, 0, KK > 2 ? RORDER[r % 8] : r);
+    // Two tiles per trip so that the LDS buffer of every access is a compile-time constant.
+    constexpr std::integral_constant<int, 0> EVEN{};
+    constexpr std::integral_constant<int, 1> ODD{};
     uint32_t ks = 0;
-    for (; ks + 2 < ksteps; ++ks) step(ks, std::true_type{}, std::true_type{});
-    if (ks + 1 < ksteps) step(ks++, std::true_type{}, std::false_type{});
-    step(ks, std::false_type{}, std::false_type{});
+    for (; ks + 2 <= ksteps; ks += 2) {
+        step(ks, EVEN);
+        step(ks + 1, ODD);
+    }
+    if (ks < ksteps) step(ks, EVEN);
 
     // 32x32 accumulator tile: lane holds slot-column l32 and slot-rows 8*(e/4) + 4*lk + e%4.
     f16 *db = reinterpret_cast<f16 *>(p.d) + (int64_t)bat * p.d_sb;
