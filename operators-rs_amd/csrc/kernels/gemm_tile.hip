@@ -10,8 +10,8 @@
 // K-contiguous in memory is copied 16 bytes at a time; one that is contiguous
 // along i / j (e.g. a weight stored [K, N]) is loaded as 16-byte rows of 8
 // columns and transposed inside the lane's registers before the LDS store.
-// Global loads for step s+1 are issued before the MFMAs of step s and written to
-// the other LDS buffer afterwards: one barrier per step.
+// Tile s+1 waits in registers while tile s is multiplied and goes to the other LDS
+// buffer under its MFMAs, the loads of tile s+2 refill the registers: one barrier per tile.
 // Workgroup ids are remapped so that the 8 XCDs (ids are dealt round-robin to
 // them) each work on a compact block of tiles and share operand panels in
 // their own L2.
@@ -25,10 +25,7 @@
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-// TK = K per step (32 or 64); LDS row pitch = TK + 8 halves (80 or 144 bytes: an odd
-// multiple of 16, so 16-byte reads of consecutive rows spread over all banks).
-
-// Copies one R x 32 operand tile from global memory to registers (`fetch`) and
+// Copies one R x TK operand tile from global memory to registers (`fetch`) and
 // from registers to LDS (`commit`).  KCONTIG: rows are K-contiguous in memory.
 //
 // LDS row order.  A K-contiguous operand keeps its rows in order.  A row-contiguous
@@ -203,13 +200,12 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
     // One wave per SIMD: nothing hides a stall, so the loop is software-pipelined by hand.
     //   registers  : tile s+1 waits in `reg` while tile s is multiplied; MFMA fragments are
     //                double-buffered, the LDS reads of k-step kk+1 run under the MFMAs of kk
-    //   k-step 0   : tile s+1 goes from registers to the other LDS buffer
-    //   k-steps 1..: the global loads of tile s+2 refill the registers, spread out evenly
+    //   stores     : tile s+1 goes from registers to the other LDS buffer, piece by piece
+    //   loads      : the global loads of tile s+2 refill the registers behind the stores
     //   barrier    : before the last k-step (whose fragments are already in registers), so
     //                that step's MFMAs cover the first fragment reads of tile s+1
-    // The code below is written in exactly that order, one memory operation of each kind
-    // after each MFMA, and sched_barrier(0) after every such group keeps the compiler from
-    // regrouping them.
+    // The code below is written in exactly that order, one memory operation after each MFMA,
+    // and sched_barrier(0) after every such pair keeps the compiler from regrouping them.
     // Copy piece i in the order the main loop uses (the waits the compiler derives for the loop
     // merge the prologue's order with the loop's: they must agree or the loop waits too long).
     constexpr bool Q_FIRST = PK && !QK, ALTERNATE = PK && QK && LP::NV == LQ::NV;
