@@ -123,15 +123,30 @@ struct TileLoader {
                 f16 *dst = lds + TileRow<TK>::at(c * (R / 8) + cb, kb * NV / 8) + kb * NV % 8;
                 uint32_t w[NV / 2];
 #pragma unroll
-                for (int d = 0; d < NV / 2; ++d) {
-                    const uint32_t a0 = reg[2 * d][c / 2], a1 = reg[2 * d + 1][c / 2];
-                    w[d] = (c & 1) ? ((a0 >> 16) | (a1 & 0xffff0000u)) : ((a0 & 0xffffu) | (a1 << 16));
-                }
+                for (int d = 0; d < NV / 2; ++d) w[d] = pair(reg[2 * d][c / 2], reg[2 * d + 1][c / 2], c & 1);
                 if constexpr (NV == 8) *reinterpret_cast<u32x4 *>(dst) = u32x4{w[0], w[1], w[2], w[3]};
                 else if constexpr (NV == 4) *reinterpret_cast<u32x2 *>(dst) = u32x2{w[0], w[1]};
                 else *reinterpret_cast<uint32_t *>(dst) = w[0];
             }
         }
+    }
+    // halves `hi` of a0 and a1 in one register: a single byte permute
+    __device__ static __forceinline__ uint32_t pair(uint32_t a0, uint32_t a1, bool hi) {
+        return __builtin_amdgcn_perm(a1, a0, hi ? 0x07060302u : 0x05040100u);
+    }
+    // A row-contiguous piece in two halves, so that the main loop can put the permutes and
+    // the store behind different MFMAs (NV == 8: piece v is column v, one 16-byte store).
+    __device__ __forceinline__ u32x4 pack_piece(int v) const {
+        static_assert(KCONTIG || NV == 8 || NV <= 4, "pack_piece is for the 8-register case");
+        u32x4 w;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) w[d] = pair(reg[(2 * d) % NV][v / 2], reg[(2 * d + 1) % NV][v / 2], v & 1);
+        return w;
+    }
+    __device__ __forceinline__ void store_packed(f16 *lds, int v, u32x4 w) const {
+        const uint32_t t = threadIdx.x;
+        const uint32_t cb = t % (R / 8), kb = t / (R / 8);
+        st128(lds + TileRow<TK>::at(v * (R / 8) + cb, kb * NV / 8) + kb * NV % 8, w);
     }
     __device__ __forceinline__ void commit(f16 *lds) const {
 #pragma unroll
@@ -279,12 +294,25 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
         constexpr int cur = decltype(parity)::value, nxt = 1 - cur;  // = ks % 2
         const uint32_t knext = min(ks + 2, ksteps - 1);
         const f16 *pnext = ptile + knext * pstep, *qnext = qtile + knext * qstep;
+        u32x4 packed;
+        // the permutes of a row-contiguous piece, one slot ahead of its store
+        auto piece_pack = [&](int i) {
+            const bool is_q = piece_is_q(i);
+            const int v = piece_v(i);
+            if (is_q) { if constexpr (!QK && LQ::NV == 8) packed = lq.pack_piece(v); }
+            else { if constexpr (!PK && LP::NV == 8) packed = lp.pack_piece(v); }
+        };
         auto piece_op = [&](int i, bool is_store) {
             const bool is_q = piece_is_q(i);
             const int v = piece_v(i);
             if (is_store) {
-                if (is_q) lq.commit_piece(q_buf(nxt), v);
-                else lp.commit_piece(p_buf(nxt), v);
+                if (is_q) {
+                    if constexpr (!QK && LQ::NV == 8) lq.store_packed(q_buf(nxt), v, packed);
+                    else lq.commit_piece(q_buf(nxt), v);
+                } else {
+                    if constexpr (!PK && LP::NV == 8) lp.store_packed(p_buf(nxt), v, packed);
+                    else lp.commit_piece(p_buf(nxt), v);
+                }
             } else {
                 if (is_q) lq.fetch_piece(qnext, v);
                 else lp.fetch_piece(pnext, v);
@@ -294,6 +322,9 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
         auto after_mfma = [&](int slot, bool reads, int next_buf, int from, int next_kk) {
             if (slot % 2 == 0) {
                 if (reads) read_one(next_buf, from, next_kk, RORDER[(slot % NMFMA) / 2]);
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+                    if (STORE && SCH.st[i] == slot / 2) piece_pack(i);
             } else {
                 const int o = slot / 2;
 #pragma unroll
