@@ -208,6 +208,18 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
     };
     for (uint32_t b : {256u, 128u}) {
         int best = -1;
+        // Tiles for less than half the CUs (a CU holds one 256 tile or two 128 tiles): split K,
+        // keeping at least 8 K-steps per workgroup; the f32 partials are summed by
+        // gemm_splitk_reduce, which wants the orientation whose D is j-contiguous.
+        size_t split = 1;
+        {
+            const size_t wgs = (size_t)(L.m / b) * (L.n / b) * L.batch, target = b == 256 ? cus : 2 * (size_t)cus;
+            const size_t ksteps = L.k / (b == 256 ? 64 : 32);
+            if (wgs > 0 && wgs * 2 <= cus)
+                split = std::min<size_t>({target / wgs, (size_t)8, std::max<size_t>(1, ksteps / 8)});
+            if (const char *e = std::getenv("OPHIP_GEMM_TILE_SPLITK")) split = std::max(1, std::atoi(e));
+            split = std::max<size_t>(1, std::min(split, ksteps));
+        }
         for (int attempt = 0; attempt < 2; ++attempt) {
             orient(attempt == 1);
             if (!tile_ok(b)) continue;
@@ -217,7 +229,7 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
             if (b == 256 && !(force && std::atoi(force) == 256) &&
                 (size_t)(p.M / b) * (p.N / b) * p.batch < cus / 2 && p.M % 128 == 0 && p.N % 128 == 0)
                 continue;
-            const bool wide = (p.q_sl != 1 && p.d_sj == 1) || (p.p_sl == 1 && p.d_si == 1);
+            const bool wide = split > 1 ? p.d_sj == 1 : (p.q_sl != 1 && p.d_sj == 1) || (p.p_sl == 1 && p.d_si == 1);
             if (best < 0 || wide) best = attempt;
             if (wide) break;
         }
@@ -227,6 +239,14 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
             g.tile = (int)b;
             g.pk = p.p_sl == 1;
             g.qk = p.q_sl == 1;
+            const size_t tk = b == 256 ? 64 : 32, ksteps = p.K / tk;
+            if (split > 1) {
+                const size_t sps = (ksteps + split - 1) / split;
+                split = (ksteps + sps - 1) / sps;
+                p.k_per_split = (uint32_t)(sps * tk);
+                p.split_k = (uint32_t)split;
+                g.workspace = split > 1 ? split * p.batch * (size_t)p.M * p.N * sizeof(float) : 0;
+            }
             return g;
         }
     }
@@ -327,7 +347,7 @@ int ophip_mat_mul_describe(const ophip_mat_mul *op, const ophip_mat_mul_args *ar
         if (g.kind == GemmPlan::Skinny)
             std::snprintf(out, len, "skinny rows<=%d q%s split_k=%u", 16 * g.mt, g.qmode ? "K" : "N", g.p.split_k);
         else if (g.kind == GemmPlan::Tile)
-            std::snprintf(out, len, "tile%d p%s q%s", g.tile, g.pk ? "K" : "M", g.qk ? "K" : "N");
+            std::snprintf(out, len, "tile%d p%s q%s split_k=%u", g.tile, g.pk ? "K" : "M", g.qk ? "K" : "N", g.p.split_k);
         else
             std::snprintf(out, len, "generic");
     });
@@ -360,8 +380,14 @@ int ophip_mat_mul_launch(const ophip_mat_mul *op, const ophip_mat_mul_args *args
             return;
         }
         if (g.kind == GemmPlan::Tile) {
+            Workspace ws(qa, workspace, workspace_len, g.workspace);
+            g.p.partial = ws.ptr();
             const unsigned tiles = (p.M / g.tile) * (p.N / g.tile);
-            launch(op->tile[g.tile == 256 ? 0 : 1][g.pk][g.qk], Dim3{tiles, 1, p.batch}, Dim3{256}, 0, stream, g.p);
+            launch(op->tile[g.tile == 256 ? 0 : 1][g.pk][g.qk], Dim3{tiles, p.split_k, p.batch}, Dim3{256}, 0, stream, g.p);
+            if (p.split_k > 1) {
+                const size_t total = (size_t)p.batch * p.M * (p.N / 8);
+                launch(op->reduce, Dim3{(unsigned)((total + 255) / 256)}, Dim3{256}, 0, stream, g.p);
+            }
             return;
         }
         const unsigned gx = (p.N + 63) / 64, gy = (p.M + 63) / 64;

@@ -206,11 +206,15 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
     typedef TileLoader<BN, QK, TK> LQ;
     LP lp;
     LQ lq;
-    const uint32_t ksteps = p.K / TK;
+    // split K: workgroup blockIdx.y multiplies K-range [kbeg, kbeg + klen) and leaves f32 partials
+    const uint32_t split = blockIdx.y;
+    const uint32_t kbeg = split * p.k_per_split, klen = min(p.K - kbeg, p.k_per_split);
+    const uint32_t ksteps = klen / TK;
     constexpr int KK = TK / 16;  // MFMA k-steps per LDS tile
     lp.init(p.p_si, p.p_sl);
     lq.init(p.q_sj, p.q_sl);
-    const f16 *ptile = pb + (int64_t)i0 * p.p_si, *qtile = qb + (int64_t)j0 * p.q_sj;
+    const f16 *ptile = pb + (int64_t)i0 * p.p_si + (int64_t)kbeg * p.p_sl;
+    const f16 *qtile = qb + (int64_t)j0 * p.q_sj + (int64_t)kbeg * p.q_sl;
     const int64_t pstep = (int64_t)TK * p.p_sl, qstep = (int64_t)TK * p.q_sl;
     // One wave per SIMD: nothing hides a stall, so the loop is software-pipelined by hand.
     //   registers  : tile s+1 waits in `reg` while tile s is multiplied; MFMA fragments are
@@ -377,6 +381,30 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
     if (ks < ksteps) step(ks, EVEN);
 
     // 32x32 accumulator tile: lane holds slot-column l32 and slot-rows 8*(e/4) + 4*lk + e%4.
+    if (p.split_k > 1) {
+        // f32 partials [split][batch][M][N]; gemm_splitk_reduce sums them and applies alpha, beta
+        float *part = reinterpret_cast<float *>(p.partial) + ((size_t)split * p.batch + bat) * p.M * (size_t)p.N;
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const uint32_t i = i0 + LP::row_of_slot(LP::reader_slot(wm, tm, 8 * (e / 4) + 4 * lk + (e % 4)));
+                float *row = part + (size_t)i * p.N + j0;
+                if constexpr (LQ::PERMUTED) {
+                    // the lane's TN tiles are TN adjacent columns
+                    float *dst = row + LQ::row_of_slot(LQ::reader_slot(wn, 0, l32));
+                    if constexpr (TN == 4) *reinterpret_cast<f32x4 *>(dst) = f32x4{acc[tm][0][e], acc[tm][1][e], acc[tm][2][e], acc[tm][3][e]};
+                    else {
+#pragma unroll
+                        for (int tn = 0; tn < TN; ++tn) dst[tn] = acc[tm][tn][e];
+                    }
+                } else {
+#pragma unroll
+                    for (int tn = 0; tn < TN; ++tn) row[LQ::row_of_slot(LQ::reader_slot(wn, tn, l32))] = acc[tm][tn][e];
+                }
+            }
+        return;
+    }
     f16 *db = reinterpret_cast<f16 *>(p.d) + (int64_t)bat * p.d_sb;
     if (LQ::PERMUTED && p.d_sj == 1) {
         // the lane's TN tiles are TN adjacent columns of D: one 4*TN/2-byte store per row

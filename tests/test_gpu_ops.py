@@ -872,6 +872,32 @@ def test_mat_mul_mfma_256_tile_kernel_layouts(gpu, stream, monkeypatch, ta, tb, 
     check_mat_mul(out, cv, av, bv, 0.75, 0.5, "mat_mul 256-tile layouts")
 
 
+@pytest.mark.parametrize("ta", [False, True])
+@pytest.mark.parametrize("tb", [False, True])
+@pytest.mark.parametrize("tc", [False, True])
+@pytest.mark.parametrize("m,n,k,bt,force256", [(256, 384, 2048, 1, False), (128, 256, 1056, 2, False), (256, 512, 1088, 1, True)])
+def test_mat_mul_tile_kernel_split_k(gpu, stream, monkeypatch, ta, tb, tc, m, n, k, bt, force256):
+    """Few tiles and a long K: the tile kernels split K (evenly or not), write f32 partials to the
+    workspace and the reduce kernel applies alpha and beta, in every operand layout."""
+    if force256:
+        monkeypatch.setenv("OPHIP_GEMM_TILE", "256")
+    rng = np.random.default_rng(m + n + k + 4 * ta + 2 * tb + tc)
+    a = (rng.standard_normal((bt, k, m) if ta else (bt, m, k)) * 0.25).astype(f32).astype(f16)
+    b = (rng.standard_normal((bt, n, k) if tb else (bt, k, n)) * 0.25).astype(f32).astype(f16)
+    c = rng.standard_normal((bt, n, m) if tc else (bt, m, n)).astype(f32).astype(f16)
+    av = a.transpose(0, 2, 1) if ta else a
+    bv = b.transpose(0, 2, 1) if tb else b
+    cv = c.transpose(0, 2, 1) if tc else c
+    args = ophip.MatMulArgs(TensorLayout.of(cv), None, 0.5, TensorLayout.of(av), None, TensorLayout.of(bv), None, 0.75)
+    op = ophip.MatMul(gpu)
+    what = op.describe(args)
+    say("mat_mul tile split-k ta=%s tb=%s tc=%s %dx%dx%d: %s" % (ta, tb, tc, m, n, k, what))
+    assert what.startswith("tile256" if force256 else "tile128") and int(what.split("split_k=")[1]) > 1, what
+    assert op.scheme(args, 2 ** 40) == int(what.split("split_k=")[1]) * bt * m * n * 4
+    out = run_mat_mul(gpu, stream, cv, av, bv, 0.75, 0.5)
+    check_mat_mul(out, cv, av, bv, 0.75, 0.5, "mat_mul tile split-k")
+
+
 def test_mat_mul_compute_bound_shape(gpu, stream):
     rng = np.random.default_rng(12)
     n = 2048
