@@ -187,12 +187,8 @@ def copy_ceiling(ophip, gpu, stream):
             "hbm_frac": round((2 << 30) / (us * 1e-6) / HBM_PEAK, 4)}
 
 
-def standalone_ops(ophip, gpu, stream, rng, reps):
-    """Every operator at its benchmark shape plus a scaled shape that does not fit the Infinity Cache."""
-    o, L, F16 = ophip, ophip.TensorLayout, ophip.dt.F16
-    c = lambda *s: L.new_contiguous(F16, list(s))
-    out = []
-
+def adder(out):
+    """Returns add(name, shape, bytes, us, flops, note): appends one per-operator record to `out` and logs it."""
     def add(name, shape, nbytes, us, flops=0, note=None):
         rec = {"op": name, "shape": shape, "us": round(us, 3), "bytes": nbytes,
                "GBps": round(nbytes / us / 1e3, 1), "hbm_frac": round(nbytes / (us * 1e-6) / HBM_PEAK, 4)}
@@ -207,6 +203,45 @@ def standalone_ops(ophip, gpu, stream, rng, reps):
         log("  %-28s %-22s %10.2f us %9.1f GB/s  %5.1f%% HBM%s" % (
             name, shape, us, rec["GBps"], 100 * rec["hbm_frac"],
             ("  %.1f TFLOP/s %.1f%% MFMA" % (rec["TFLOPs"], 100 * rec["mfma_frac"])) if flops else ""))
+
+    return add
+
+
+def mat_mul_lines(o, gpu, stream, rng, add, launches=0):
+    """Compute-bound mat_mul: square shapes in both layouts of B and the prefill GEMMs of a Llama-7B layer
+    at 512 tokens.  `launches` > 0: that many plain launches per shape and nothing else (counter runs)."""
+    from ophip import TensorLayout as L, dt
+    c = lambda *s: L.new_contiguous(dt.F16, list(s))
+    mm = o.MatMul(gpu)
+    shapes = [(4096, 4096, 4096, False), (4096, 4096, 4096, True), (8192, 8192, 8192, False), (8192, 8192, 8192, True),
+              (512, 12288, 4096, False), (512, 22016, 4096, False), (512, 4096, 11008, False)]
+    for m, n, k, b_nk in shapes:
+        A_, B_, C_ = gpu.from_host(normal_f16(rng, (m, k), 1.0)), gpu.from_host(normal_f16(rng, (k, n), 0.02)), \
+            gpu.malloc(m * n * 2)
+        bl = L(dt.F16, [k, n], [2, k * 2]) if b_nk else c(k, n)  # the same bytes read as B[N, K] transposed
+        a = o.MatMulArgs(c(m, n), C_, 0.0, c(m, k), A_, bl, B_, 1.0)
+        ws = gpu.malloc(max(mm.scheme(a, 1 << 32), 1))
+        shape = "%dx%dx%d%s" % (m, n, k, ", B stored [N,K]" if b_nk else "")
+        nbytes, flops = 2 * (m * k + k * n + m * n), 2 * m * n * k
+        if launches:
+            us = time_launches(gpu, stream, lambda: mm.launch(a, ws, stream), launches, warm=1)
+            add("mat_mul", shape, nbytes, us, flops=flops, note="%d launches, %s" % (launches, mm.describe(a)))
+        else:
+            if m == n == k:
+                us = time_launches(gpu, stream, lambda: mm.launch(a, ws, stream), 10, warm=2)
+                add("mat_mul", shape, nbytes, us, flops=flops, note="10 launches from idle clocks")
+            us = time_sustained(gpu, stream, lambda: mm.launch(a, ws, stream))
+            add("mat_mul", shape, nbytes, us, flops=flops, note="steady state (0.3 s warm-up), " + mm.describe(a))
+        A_.free(); B_.free(); C_.free(); ws.free()
+
+
+def standalone_ops(ophip, gpu, stream, rng, reps):
+    """Every operator at its benchmark shape plus a scaled shape that does not fit the Infinity Cache."""
+    o, L, F16 = ophip, ophip.TensorLayout, ophip.dt.F16
+    c = lambda *s: L.new_contiguous(F16, list(s))
+    out = []
+
+    add = adder(out)
 
     # rms_norm: [64, 4096] and [65536, 4096]
     rms = o.RmsNorm(gpu)
@@ -331,18 +366,7 @@ def standalone_ops(ophip, gpu, stream, rng, reps):
     us = time_launches(gpu, stream, lambda: akv.launch(a, ws, stream), reps)
     add("attention_kv_cached", "nh32 seq16 pos2032 dh128", 2 * NH * KV * DH * 2 + 8 * nt * D * 2, us,
         note="composite of 7 launches; bytes = both caches read once + q, k, v, o and the appended rows")
-    # compute-bound mat_mul: 4096^3 and 8192^3
-    mm = o.MatMul(gpu)
-    for n in (4096, 8192):
-        A_, B_, C_ = gpu.from_host(normal_f16(rng, (n, n), 1.0)), gpu.from_host(normal_f16(rng, (n, n), 0.02)), \
-            gpu.malloc(n * n * 2)
-        a = o.MatMulArgs(c(n, n), C_, 0.0, c(n, n), A_, c(n, n), B_, 1.0)
-        mm.scheme(a, 0)
-        us = time_launches(gpu, stream, lambda: mm.launch(a, None, stream), 10, warm=2)
-        add("mat_mul", "%d^3" % n, 3 * n * n * 2, us, flops=2 * n ** 3, note="10 launches from idle clocks")
-        us = time_sustained(gpu, stream, lambda: mm.launch(a, None, stream))
-        add("mat_mul", "%d^3" % n, 3 * n * n * 2, us, flops=2 * n ** 3, note="steady state (0.3 s warm-up)")
-        A_.free(); B_.free(); C_.free()
+    mat_mul_lines(o, gpu, stream, rng, add)
     return out
 
 
@@ -379,6 +403,9 @@ def main():
     ap.add_argument("--reps", type=int, default=100, help="launches per standalone-operator timing")
     ap.add_argument("--no-per-op", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--mat-mul-only", type=int, nargs="?", const=0, default=None, metavar="LAUNCHES",
+                    help="only the compute-bound mat_mul shapes (not the benchmark line); with a number, that many "
+                         "plain launches per shape, for hardware-counter runs")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -392,6 +419,11 @@ def main():
     log("device: %s (%s), %d CUs" % (info.name.decode(), info.arch.decode(), info.compute_units))
     stream = gpu.stream()
     rng = np.random.default_rng(0)
+    if args.mat_mul_only is not None:
+        lines = []
+        mat_mul_lines(ophip, gpu, stream, rng, adder(lines), launches=args.mat_mul_only)
+        print(json.dumps({"mat_mul": lines}))
+        return
 
     # two layers' worth of distinct weights (2 x 404 MB), alternated per step, so no
     # step finds its weights in the 256 MiB Infinity Cache

@@ -96,7 +96,7 @@ struct GemmPlan {
     GemmParams p{};
     enum Kind { Generic, Skinny, Tile } kind = Generic;
     int mt = 1, qmode = 0;
-    int tile = 256, pk = 1, qk = 1;  // Tile: block size and whether P / Q are K-contiguous
+    int tile = 256, tk = 64, pk = 1, qk = 1;  // Tile: block size, K-step, and whether P / Q are K-contiguous
     size_t workspace = 0;
 };
 
@@ -214,7 +214,7 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
         size_t split = 1;
         {
             const size_t wgs = (size_t)(L.m / b) * (L.n / b) * L.batch, target = b == 256 ? cus : 2 * (size_t)cus;
-            const size_t ksteps = L.k / (b == 256 ? 64 : 32);
+            const size_t ksteps = L.k / (L.k % 64 == 0 ? 64 : 32);
             if (wgs > 0 && wgs * 2 <= cus)
                 split = std::min<size_t>({target / wgs, (size_t)8, std::max<size_t>(1, ksteps / 8)});
             if (const char *e = std::getenv("OPHIP_GEMM_TILE_SPLITK")) split = std::max(1, std::atoi(e));
@@ -239,7 +239,8 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
             g.tile = (int)b;
             g.pk = p.p_sl == 1;
             g.qk = p.q_sl == 1;
-            const size_t tk = b == 256 ? 64 : 32, ksteps = p.K / tk;
+            const size_t tk = p.K % 64 == 0 ? 64 : 32, ksteps = p.K / tk;
+            g.tk = (int)tk;
             if (split > 1) {
                 const size_t sps = (ksteps + split - 1) / split;
                 split = (ksteps + sps - 1) / sps;
@@ -264,7 +265,7 @@ struct ophip_mat_mul {
     ophip_device *dev;
     hipFunction_t skinny[3][2];  // [mt index 1,2,4][qmode]
     hipFunction_t reduce, generic_f16, generic_f32;
-    hipFunction_t tile[2][2][2];  // [256 / 128][P K-contiguous][Q K-contiguous]
+    hipFunction_t tile[3][2][2];  // [256 x 64 / 128 x 64 / 128 x 32 (K-step)][P K-contiguous][Q K-contiguous]
     // Arrival counters live in a buffer owned by the operator, one per stream:
     // launches on one stream run in order and every kernel leaves its counters at
     // zero, so the buffer is zeroed once, when a stream is first seen.
@@ -288,10 +289,10 @@ struct ophip_mat_mul {
             for (int q = 0; q < 2; ++q)
                 skinny[i][q] =
                     d->kernel("gemm", ("gemm_skinny_m" + std::to_string(mts[i]) + "_q" + std::to_string(q)).c_str());
-        for (int b = 0; b < 2; ++b)
+        for (int b = 0; b < 3; ++b)
             for (int pk = 0; pk < 2; ++pk)
                 for (int qk = 0; qk < 2; ++qk) {
-                    const std::string sz = b == 0 ? "256x256" : "128x128";
+                    const std::string sz = b == 0 ? "256x256" : b == 1 ? "128x128" : "128x128k32";
                     tile[b][pk][qk] = d->kernel(
                         "gemm_tile", ("gemm_tile_" + sz + "_p" + std::to_string(pk) + "_q" + std::to_string(qk)).c_str());
                 }
@@ -347,7 +348,7 @@ int ophip_mat_mul_describe(const ophip_mat_mul *op, const ophip_mat_mul_args *ar
         if (g.kind == GemmPlan::Skinny)
             std::snprintf(out, len, "skinny rows<=%d q%s split_k=%u", 16 * g.mt, g.qmode ? "K" : "N", g.p.split_k);
         else if (g.kind == GemmPlan::Tile)
-            std::snprintf(out, len, "tile%d p%s q%s split_k=%u", g.tile, g.pk ? "K" : "M", g.qk ? "K" : "N", g.p.split_k);
+            std::snprintf(out, len, "tile%dx%d p%s q%s split_k=%u", g.tile, g.tk, g.pk ? "K" : "M", g.qk ? "K" : "N", g.p.split_k);
         else
             std::snprintf(out, len, "generic");
     });
@@ -383,7 +384,7 @@ int ophip_mat_mul_launch(const ophip_mat_mul *op, const ophip_mat_mul_args *args
             Workspace ws(qa, workspace, workspace_len, g.workspace);
             g.p.partial = ws.ptr();
             const unsigned tiles = (p.M / g.tile) * (p.N / g.tile);
-            launch(op->tile[g.tile == 256 ? 0 : 1][g.pk][g.qk], Dim3{tiles, p.split_k, p.batch}, Dim3{256}, 0, stream, g.p);
+            launch(op->tile[g.tile == 256 ? 0 : g.tk == 64 ? 1 : 2][g.pk][g.qk], Dim3{tiles, p.split_k, p.batch}, Dim3{256}, 0, stream, g.p);
             if (p.split_k > 1) {
                 const size_t total = (size_t)p.batch * p.M * (p.N / 8);
                 launch(op->reduce, Dim3{(unsigned)((total + 255) / 256)}, Dim3{256}, 0, stream, g.p);

@@ -154,7 +154,8 @@ struct TileLoader {
     }
 };
 
-template <int BM, int BN, bool PK, bool QK, int TK>
+// DEPTH: operand tiles kept in flight in registers (1: the next one; 2: the next two, in two register sets).
+template <int BM, int BN, bool PK, bool QK, int TK, int DEPTH>
 __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
     constexpr int LDK = TileRow<TK>::LDK;
     constexpr int WM = BM / 2, WN = BN / 2;  // wave tile
@@ -204,15 +205,18 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
 
     typedef TileLoader<BM, PK, TK> LP;
     typedef TileLoader<BN, QK, TK> LQ;
-    LP lp;
-    LQ lq;
+    LP lp[DEPTH];
+    LQ lq[DEPTH];
     // split K: workgroup blockIdx.y multiplies K-range [kbeg, kbeg + klen) and leaves f32 partials
     const uint32_t split = blockIdx.y;
     const uint32_t kbeg = split * p.k_per_split, klen = min(p.K - kbeg, p.k_per_split);
     const uint32_t ksteps = klen / TK;
     constexpr int KK = TK / 16;  // MFMA k-steps per LDS tile
-    lp.init(p.p_si, p.p_sl);
-    lq.init(p.q_sj, p.q_sl);
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+        lp[d].init(p.p_si, p.p_sl);
+        lq[d].init(p.q_sj, p.q_sl);
+    }
     const f16 *ptile = pb + (int64_t)i0 * p.p_si + (int64_t)kbeg * p.p_sl;
     const f16 *qtile = qb + (int64_t)j0 * p.q_sj + (int64_t)kbeg * p.q_sl;
     const int64_t pstep = (int64_t)TK * p.p_sl, qstep = (int64_t)TK * p.q_sl;
@@ -230,19 +234,21 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
     constexpr bool Q_FIRST = PK && !QK, ALTERNATE = PK && QK && LP::NV == LQ::NV;
     auto piece_is_q = [&](int i) { return ALTERNATE ? bool(i & 1) : ((i >= LP::NV) != Q_FIRST) ; };
     auto piece_v = [&](int i) { return ALTERNATE ? i / 2 : (Q_FIRST ? (i < LQ::NV ? i : i - LQ::NV) : (i < LP::NV ? i : i - LP::NV)); };
-    auto fetch_all = [&](const f16 *pt, const f16 *qt) {
+    auto fetch_all = [&](int set, const f16 *pt, const f16 *qt) {
 #pragma unroll
         for (int i = 0; i < LP::NV + LQ::NV; ++i) {
-            if (piece_is_q(i)) lq.fetch_piece(qt, piece_v(i));
-            else lp.fetch_piece(pt, piece_v(i));
+            if (piece_is_q(i)) lq[set].fetch_piece(qt, piece_v(i));
+            else lp[set].fetch_piece(pt, piece_v(i));
         }
     };
-    fetch_all(ptile, qtile);
-    lp.commit(p_buf(0));
-    lq.commit(q_buf(0));
-    {
-        const uint32_t k1 = min(1u, ksteps - 1);
-        fetch_all(ptile + k1 * pstep, qtile + k1 * qstep);
+    // operand tile t travels through register set t % DEPTH
+    fetch_all(0, ptile, qtile);
+    lp[0].commit(p_buf(0));
+    lq[0].commit(q_buf(0));
+#pragma unroll
+    for (int d = 1; d <= DEPTH; ++d) {
+        const uint32_t kd = min((uint32_t)d, ksteps - 1);
+        fetch_all(d % DEPTH, ptile + kd * pstep, qtile + kd * qstep);
     }
     __syncthreads();
 
@@ -267,7 +273,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
         acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[buf][tm].h, b[buf][tn].h, acc[tm][tn], 0, 0, 0);
     };
     constexpr int NMFMA = TM * TN, NREAD = TM + TN, NLOAD = LP::NV + LQ::NV;
-    static_assert(NREAD <= NMFMA && NLOAD <= NMFMA, "one memory operation of a kind per MFMA at most");
+    static_assert(NREAD <= NMFMA && NLOAD <= NMFMA * (KK / 2), "the copy pieces must fit the slots of half a tile");
     static_assert(KK >= 2 && KK % 2 == 0, "fragment buffers alternate per k-step");
     // Issue budget.  The wave issues in order and an MFMA occupies its pipe for 32 cycles, so
     // whatever stands between two MFMAs must issue in less than that or the pipe runs dry:
@@ -286,9 +292,15 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
                                              {2, 5, 8, 11, 14, 17, 20, 23, 24, 25, 26, 27, 28, 29, 30, 31}}
                                      : Sched{{0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15},
                                              {16, 17, 18, 19, 20, 21, 22, 23, 24, 25, 26, 27, 28, 29, 30, 31}};
-    static_assert(KK == 2 || (LP::NV == 8 && LQ::NV == 8 && NMFMA == 16 && KK == 4), "tables are for the 256 x 256 x 64 tile");
-    // fragments in the order the next k-step's MFMAs want them: a0 b0 b1 b2 b3 a1 a2 a3
-    constexpr int RORDER[8] = {0, TM, TM + 1, TM + 2, TM + 3, 1, 2, 3};
+    //   128 x 128 x 64 (4 k-steps of 4 MFMAs, 8 copy pieces, two such workgroups per CU so the other
+    //   wave of the SIMD fills what one wave's issue leaves open): a fragment read after every
+    //   MFMA, the stores after MFMAs 0..7, the loads after 8..15; with DEPTH = 2 a load has a
+    //   tile and a half to arrive.
+    //   128 x 128 x 32 (K not a multiple of 64): two k-steps, stores under the first, then the loads.
+    constexpr bool BIG = NMFMA == 16 && KK == 4, MID = NMFMA == 4 && KK == 4;
+    static_assert(KK == 2 || (BIG && LP::NV == 8 && LQ::NV == 8) || (MID && LP::NV == 4 && LQ::NV == 4), "no slot table for this tile");
+    // fragments in the order the next k-step's MFMAs want them: a0 b0 b1 b2 b3 a1 a2 a3 (a0 b0 b1 a1)
+    constexpr int RORDER[8] = {0, TM, TM + 1, BIG ? TM + 2 : 1, TM + 3, 1, 2, 3};
     // Every tile runs the same code: past the end of K the loads fetch the last tile again, the
     // stores put it into the buffer nobody reads any more and the fragment reads of a tile that
     // does not exist are not used.  (Separate code for the last two tiles costs more in
@@ -296,35 +308,40 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
     auto step = [&](uint32_t ks, auto parity) {
         constexpr bool STORE = true, LOAD = true;
         constexpr int cur = decltype(parity)::value, nxt = 1 - cur;  // = ks % 2
-        const uint32_t knext = min(ks + 2, ksteps - 1);
+        constexpr int SET = DEPTH == 2 ? nxt : 0;  // register set of tile ks + 1, refilled with tile ks + 1 + DEPTH
+        const uint32_t knext = min(ks + 1 + DEPTH, ksteps - 1);
         const f16 *pnext = ptile + knext * pstep, *qnext = qtile + knext * qstep;
         u32x4 packed;
         // the permutes of a row-contiguous piece, one slot ahead of its store
         auto piece_pack = [&](int i) {
             const bool is_q = piece_is_q(i);
             const int v = piece_v(i);
-            if (is_q) { if constexpr (!QK && LQ::NV == 8) packed = lq.pack_piece(v); }
-            else { if constexpr (!PK && LP::NV == 8) packed = lp.pack_piece(v); }
+            if (is_q) { if constexpr (!QK && LQ::NV == 8) packed = lq[SET].pack_piece(v); }
+            else { if constexpr (!PK && LP::NV == 8) packed = lp[SET].pack_piece(v); }
         };
         auto piece_op = [&](int i, bool is_store) {
             const bool is_q = piece_is_q(i);
             const int v = piece_v(i);
             if (is_store) {
                 if (is_q) {
-                    if constexpr (!QK && LQ::NV == 8) lq.store_packed(q_buf(nxt), v, packed);
-                    else lq.commit_piece(q_buf(nxt), v);
+                    if constexpr (!QK && LQ::NV == 8) lq[SET].store_packed(q_buf(nxt), v, packed);
+                    else lq[SET].commit_piece(q_buf(nxt), v);
                 } else {
-                    if constexpr (!PK && LP::NV == 8) lp.store_packed(p_buf(nxt), v, packed);
-                    else lp.commit_piece(p_buf(nxt), v);
+                    if constexpr (!PK && LP::NV == 8) lp[SET].store_packed(p_buf(nxt), v, packed);
+                    else lp[SET].commit_piece(p_buf(nxt), v);
                 }
             } else {
-                if (is_q) lq.fetch_piece(qnext, v);
-                else lp.fetch_piece(pnext, v);
+                if (is_q) lq[SET].fetch_piece(qnext, v);
+                else lp[SET].fetch_piece(pnext, v);
             }
         };
         // what follows MFMA number `slot` of the tile (KK == 4)
         auto after_mfma = [&](int slot, bool reads, int next_buf, int from, int next_kk) {
-            if (slot % 2 == 0) {
+            if constexpr (MID) {
+                if (reads) read_one(next_buf, from, next_kk, RORDER[slot % NMFMA]);
+                if (slot < NLOAD) piece_op(slot, true);
+                else piece_op(slot - NLOAD, false);
+            } else if (slot % 2 == 0) {
                 if (reads) read_one(next_buf, from, next_kk, RORDER[(slot % NMFMA) / 2]);
 #pragma unroll
                 for (int i = 0; i < 16; ++i)
@@ -353,7 +370,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (LOAD && KK == 2 && kk == 0) {
-                fetch_all(pnext, qnext);
+                fetch_all(SET, pnext, qnext);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -370,6 +387,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
     };
 #pragma unroll
     for (int r = 0; r < NREAD; ++r) read_one(0, 0, 0, KK > 2 ? RORDER[r % 8] : r);
+    static_assert(!MID || NLOAD == 8, "MID: 8 stores, then 8 loads, in the 16 slots of a tile");
     // Two tiles per trip so that the LDS buffer of every access is a compile-time constant.
     constexpr std::integral_constant<int, 0> EVEN{};
     constexpr std::integral_constant<int, 1> ODD{};
@@ -469,16 +487,20 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
     }
 }
 
-#define GEMM_TILE(BM, BN, PK, QK, TK)                                                                    \
-    extern "C" __global__ void __launch_bounds__(256) gemm_tile_##BM##x##BN##_p##PK##_q##QK(GemmParams p) { \
-        gemm_tile<BM, BN, PK, QK, TK>(p);                                                                \
+#define GEMM_TILE(NAME, BM, BN, PK, QK, TK, DEPTH)                                                 \
+    extern "C" __global__ void __launch_bounds__(256) gemm_tile_##NAME##_p##PK##_q##QK(GemmParams p) { \
+        gemm_tile<BM, BN, PK, QK, TK, DEPTH>(p);                                                   \
     }
 
-GEMM_TILE(256, 256, 1, 1, 64)
-GEMM_TILE(256, 256, 1, 0, 64)
-GEMM_TILE(256, 256, 0, 1, 64)
-GEMM_TILE(256, 256, 0, 0, 64)
-GEMM_TILE(128, 128, 1, 1, 32)
-GEMM_TILE(128, 128, 1, 0, 32)
-GEMM_TILE(128, 128, 0, 1, 32)
-GEMM_TILE(128, 128, 0, 0, 32)
+GEMM_TILE(256x256, 256, 256, 1, 1, 64, 1)
+GEMM_TILE(256x256, 256, 256, 1, 0, 64, 1)
+GEMM_TILE(256x256, 256, 256, 0, 1, 64, 1)
+GEMM_TILE(256x256, 256, 256, 0, 0, 64, 1)
+GEMM_TILE(128x128, 128, 128, 1, 1, 64, 2)
+GEMM_TILE(128x128, 128, 128, 1, 0, 64, 2)
+GEMM_TILE(128x128, 128, 128, 0, 1, 64, 2)
+GEMM_TILE(128x128, 128, 128, 0, 0, 64, 2)
+GEMM_TILE(128x128k32, 128, 128, 1, 1, 32, 1)
+GEMM_TILE(128x128k32, 128, 128, 1, 0, 32, 1)
+GEMM_TILE(128x128k32, 128, 128, 0, 1, 32, 1)
+GEMM_TILE(128x128k32, 128, 128, 0, 0, 32, 1)

@@ -192,3 +192,21 @@ def test_offset_calculator_best_fit_and_coalescing():
     assert c.take(4096) == (0x10000, 0x10000 + 4096)
     c.put(*a)
     assert c.take(1024) == (0x40000, 0x40000 + 1024)
+
+
+def test_tile_gemm_code_objects_keep_accumulators_in_registers():
+    """A tile-GEMM loop that fails to unroll puts its 256 accumulators into scratch memory and the kernel
+    runs an order of magnitude slower without any error: check the private segment size in the built code
+    object's metadata.  Skipped where the build directory or the ROCm binutils are absent."""
+    import shutil
+    import subprocess
+    hsaco = os.path.join(os.path.dirname(ophip.__file__), "..", "csrc", "build", "gemm_tile.hsaco")
+    readelf = shutil.which("llvm-readelf") or "/opt/rocm/llvm/bin/llvm-readelf"
+    if not os.path.exists(hsaco) or not os.path.exists(readelf):
+        pytest.skip("no built code object or no llvm-readelf here")
+    notes = subprocess.run([readelf, "--notes", hsaco], capture_output=True, text=True, check=True).stdout
+    names = re.findall(r"\.name:\s+(\S+)", notes)
+    scratch = [int(v) for v in re.findall(r"\.private_segment_fixed_size:\s+(\d+)", notes)]
+    assert len(names) == len(scratch) == 12, (names, scratch)
+    for name, size in zip(names, scratch):
+        assert size <= 512, "%s uses %d bytes of scratch per lane" % (name, size)
