@@ -1,0 +1,1 @@
+impl_op!(hip, Hip);
