@@ -223,11 +223,13 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
         for (int attempt = 0; attempt < 2; ++attempt) {
             orient(attempt == 1);
             if (!tile_ok(b)) continue;
-            // too few 256-tiles to fill the machine: let the 128 pass take it
-            // (OPHIP_GEMM_TILE=256 keeps the large tile, for tests of that kernel on small shapes)
+            // 256-tiles for less than 60 % of the CUs: the 128 pass is faster (measured on 512 .. 2048 row
+            // shapes: at half the CUs the large tile loses by 10 - 50 %, at two thirds it wins by 10 %)
+            // (OPHIP_GEMM_TILE=256 / 128 keeps one tile size, for tests and sweeps)
             const char *force = std::getenv("OPHIP_GEMM_TILE");
-            if (b == 256 && !(force && std::atoi(force) == 256) &&
-                (size_t)(p.M / b) * (p.N / b) * p.batch < cus / 2 && p.M % 128 == 0 && p.N % 128 == 0)
+            if (force && (uint32_t)std::atoi(force) != b) continue;
+            if (b == 256 && !force && (size_t)(p.M / b) * (p.N / b) * p.batch * 5 < (size_t)cus * 3 && p.M % 128 == 0 &&
+                p.N % 128 == 0)
                 continue;
             const bool wide = split > 1 ? p.d_sj == 1 : (p.q_sl != 1 && p.d_sj == 1) || (p.p_sl == 1 && p.d_si == 1);
             if (best < 0 || wide) best = attempt;
