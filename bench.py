@@ -3,9 +3,9 @@
 
 One "step" is one pass of the Llama-7B-shape decode layer (16 tokens, d = 4096,
 32 heads x 128, KV length 2048, FFN 11008) through the operator API: rms_norm,
-QKV mat_mul, rope(q), rope(k), QK^T mat_mul, causal softmax, PV mat_mul, O-proj
-mat_mul, rms_norm, gate/up mat_mul, swiglu, down mat_mul - twelve launches on one
-stream, inputs resident in HBM, synthetic data.  `value` is the layer's
+QKV mat_mul, rope (q and k in one launch: they are adjacent heads of the qkv rows),
+QK^T mat_mul, causal softmax, PV mat_mul, O-proj mat_mul, rms_norm, gate/up mat_mul,
+swiglu, down mat_mul - eleven launches on one stream, inputs resident in HBM, synthetic data.  `value` is the layer's
 algorithmic bytes divided by the measured time per step.
 
 Beside it the script reports, in the same JSON line:
@@ -71,7 +71,6 @@ class Layer:
             self.h = {k: v for k, v in h.items() if k in ("x",)}  # drop host weights
 
         c = lambda *s: L.new_contiguous(F16, list(s))
-        q_lay = L(F16, [NT, NH, DH], [3 * D * 2, DH * 2, 2])          # q / k views inside qkv
         qb_lay = L(F16, [NH, NT, DH], [DH * 2, 3 * D * 2, 2])         # q as [head, token, dh]
         kt_lay = L(F16, [NH, DH, KV], [KV * DH * 2, 2, DH * 2])       # K-cache as K^T
         ob_lay = L(F16, [NH, NT, DH], [DH * 2, D * 2, 2])             # attention output as [token, head*dh]
@@ -83,9 +82,10 @@ class Layer:
         A = self.args = {}
         A["rms_norm_1"] = ("rms", o.RmsNormArgs(c(NT, D), d["xn"], c(NT, D), d["x"], c(D), d["w_norm1"], 1e-5))
         A["qkv"] = ("mm", o.MatMulArgs(c(NT, 3 * D), d["qkv"], 0.0, c(NT, D), d["xn"], c(D, 3 * D), d["w_qkv"], 1.0))
-        A["rope_q"] = ("rope", o.RopeArgs(q_lay, d["qkv"].ptr, c(NT), d["pos"], empty, None, empty, None, 1e4))
-        A["rope_k"] = ("rope", o.RopeArgs(q_lay, d["qkv"].ptr + D * 2, c(NT), d["pos"], empty, None, empty, None, 1e4))
-        A["rope_q"][1].p_layout = A["rope_k"][1].p_layout = L(o.dt.U32, [NT], [4])
+        # q and k sit side by side in every token's qkv row: one rope launch over both, as 2 * NH heads
+        qk_lay = L(F16, [NT, 2 * NH, DH], [3 * D * 2, DH * 2, 2])
+        A["rope"] = ("rope", o.RopeArgs(qk_lay, d["qkv"].ptr, c(NT), d["pos"], empty, None, empty, None, 1e4))
+        A["rope"][1].p_layout = L(o.dt.U32, [NT], [4])
         A["qk_t"] = ("mm", o.MatMulArgs(c(NH, NT, KV), d["att"], 0.0, qb_lay, d["qkv"].ptr, kt_lay, d["k_cache"],
                                         float(1.0 / np.sqrt(DH))))
         A["softmax"] = ("sm", o.FusedSoftmaxArgs(o.AttnMask.CAUSAL, c(NH, NT, KV), d["att"]))
@@ -95,7 +95,7 @@ class Layer:
         A["gate_up"] = ("mm", o.MatMulArgs(c(NT, 2 * DI), d["gu"], 0.0, c(NT, D), d["yn"], c(D, 2 * DI), d["w_gu"], 1.0))
         A["swiglu"] = ("sw", o.SwigluArgs(half, d["gu"].ptr, half, d["gu"].ptr + DI * 2))
         A["down"] = ("mm", o.MatMulArgs(c(NT, D), d["out"], 0.0, half, d["gu"].ptr, c(DI, D), d["w_d"], 1.0))
-        self.order = ["rms_norm_1", "qkv", "rope_q", "rope_k", "qk_t", "softmax", "pv", "o_proj", "rms_norm_2",
+        self.order = ["rms_norm_1", "qkv", "rope", "qk_t", "softmax", "pv", "o_proj", "rms_norm_2",
                       "gate_up", "swiglu", "down"]
         for name in self.order:
             kind, a = A[name]
@@ -121,8 +121,7 @@ def layer_work():
     w = {
         "rms_norm_1": (2 * NT * D * 2 + D * 2, 0),
         "qkv": gemm(NT, 3 * D, D),
-        "rope_q": (2 * NT * NH * DH * 2 + NT * 4, 0),
-        "rope_k": (2 * NT * NH * DH * 2 + NT * 4, 0),
+        "rope": (2 * (2 * NT * NH * DH * 2 + NT * 4), 0),  # q and k, the position vector counted for each
         "qk_t": gemm(NT, KV, DH, NH),
         "softmax": (2 * NH * NT * KV * 2, 0),
         "pv": gemm(NT, DH, KV, NH),
@@ -371,7 +370,7 @@ def standalone_ops(ophip, gpu, stream, rng, reps):
 
 
 def cpu_layer_step(oracle, h, threads):
-    """The same twelve operations through the CPU oracle (threads on the axes the reference hands to rayon)."""
+    """The same operations through the CPU oracle (threads on the axes the reference hands to rayon)."""
     oracle.set_threads(threads)
     xn = oracle.rms_norm(np.empty_like(h["x"]), h["x"], h["w_norm1"], 1e-5)
     qkv = oracle.mat_mul(np.zeros((NT, 3 * D), f16), 0.0, xn, h["w_qkv"], 1.0)
