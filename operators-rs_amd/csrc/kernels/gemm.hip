@@ -277,17 +277,18 @@ __device__ __forceinline__ void gemm_skinny(const GemmParams &p) {
                     float sum[8] = {0, 0, 0, 0, 0, 0, 0, 0};
                     const size_t sstride = (size_t)p.batch * p.M * p.N;  // floats between splits
                     const float *src0 = reinterpret_cast<const float *>(p.partial) + ((size_t)bat * p.M + i) * p.N + col0;
-                    for (uint32_t s0 = 0; s0 < p.split_k; s0 += 4) {  // four splits' loads in flight, summed in order
-                        float v[4][8];
+                    constexpr int FLY = MT == 1 ? 8 : 4;  // splits whose loads are in flight together, summed in order
+                    for (uint32_t s0 = 0; s0 < p.split_k; s0 += FLY) {
+                        float v[FLY][8];
 #pragma unroll
-                        for (int u = 0; u < 4; ++u)
+                        for (int u = 0; u < FLY; ++u)
 #pragma unroll
                             for (int t = 0; t < 8; t += 2) {
                                 v[u][t] = v[u][t + 1] = 0.f;
                                 if (s0 + u < p.split_k) partial_load(src0 + (s0 + u) * sstride + t, v[u][t], v[u][t + 1]);
                             }
 #pragma unroll
-                        for (int u = 0; u < 4; ++u)
+                        for (int u = 0; u < FLY; ++u)
                             if (s0 + u < p.split_k) {
 #pragma unroll
                                 for (int t = 0; t < 8; ++t) sum[t] += v[u][t];
