@@ -11,7 +11,8 @@ algorithmic bytes divided by the measured time per step.
 Beside it the script reports, in the same JSON line:
   per_op       every operator at its benchmark shape (and a scaled shape large
                enough to leave the 256 MiB Infinity Cache): us/op, GB/s or
-               TFLOP/s, fraction of the roofline;
+               TFLOP/s, fraction of the roofline; at the benchmark shapes of the single
+               operators also `cpu_us`, the CPU oracle's time on the same shape;
   roofline     the dominant kernel of the step (the gate/up weight-streaming
                mat_mul), timed with HIP events inside the timed region;
   cpu_baseline the CPU oracle (a port of the crate's CPU backend) timed on the
@@ -369,6 +370,44 @@ def standalone_ops(ophip, gpu, stream, rng, reps):
     return out
 
 
+def cpu_per_op(oracle, threads):
+    """The CPU oracle on the benchmark configurations of the single operators (BASELINE.json configs 1 - 4),
+    best of three runs each; keys are (operator, shape) as in `per_op`."""
+    rng = np.random.default_rng(0)
+    oracle.set_threads(threads)
+    out = {}
+
+    def best(fn):
+        ts = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        return min(ts) * 1e6
+
+    try:
+        x, w = normal_f16(rng, (64, D), 1.0), (rng.random(D, dtype=np.float32) + 0.5).astype(f16)
+        y = np.zeros_like(x)
+        out[("rms_norm", "[64,%d]" % D)] = best(lambda: oracle.rms_norm(y, x, w, 1e-5))
+        t, pos = normal_f16(rng, (512, NH, DH), 1.0), np.arange(512, dtype=np.uint32)
+        out[("rope", "[512,%d,%d]" % (NH, DH))] = best(lambda: oracle.rope(t, pos, 1e4))
+        src = normal_f16(rng, (32, 512, DH), 1.0)
+        dst = np.zeros((512, 32, DH), f16)
+        out[("rearrange", "[32,512,%d]->T" % DH)] = best(lambda: oracle.rearrange(dst.transpose(1, 0, 2), src))
+        for seq, al in ((512, 512), (1, 2048)):
+            att = normal_f16(rng, (32, seq, al), 2.0)
+            out[("fused_softmax", "[32,%d,%d]" % (seq, al))] = best(lambda: oracle.fused_softmax(att, True))
+        gu = normal_f16(rng, (16, 2 * DI), 1.0)
+        out[("swiglu", "[16,%d]" % DI)] = best(lambda: oracle.swiglu(gu[:, :DI], gu[:, DI:]))
+        logits = normal_f16(rng, (16, 32000), np.sqrt(3.0))
+        out[("random_sample argmax", "16 x [32000]")] = best(lambda: [oracle.argmax(r) for r in logits])
+        out[("random_sample top-k 50 / top-p 0.9", "16 x [32000]")] = best(
+            lambda: [oracle.random_sample(r, 0.8, 0.9, 50, 0.37) for r in logits])
+    finally:
+        oracle.set_threads(1)
+    return out
+
+
 def cpu_layer_step(oracle, h, threads):
     """The same operations through the CPU oracle (threads on the axes the reference hands to rayon)."""
     oracle.set_threads(threads)
@@ -480,6 +519,11 @@ def main():
             cpu_layer_step(oracle, h, threads)
             t_cpu += time.perf_counter() - c0
             n_cpu += 1
+        # the same oracle on the single-operator configurations, beside their GPU lines
+        for (op_name, shape), us in cpu_per_op(oracle, threads).items():
+            for rec in per_op:
+                if rec["op"] == op_name and rec["shape"] == shape:
+                    rec["cpu_us"], rec["cpu_threads"] = round(us, 1), threads
         cpu = {"value": round(layer_bytes / (t_cpu / n_cpu) / 1e9, 3), "unit": "GB/s", "cores": threads,
                "kind": "port", "ms_per_step": round(t_cpu / n_cpu * 1e3, 2),
                "sample": "%d full decode-layer steps of the same workload through the CPU oracle" % n_cpu}
