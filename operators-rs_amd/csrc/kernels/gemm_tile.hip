@@ -306,7 +306,6 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
     // does not exist are not used.  (Separate code for the last two tiles costs more in
     // registers, through the extra control flow, than the few redundant copies.)
     auto step = [&](uint32_t ks, auto parity) {
-        constexpr bool STORE = true, LOAD = true;
         constexpr int cur = decltype(parity)::value, nxt = 1 - cur;  // = ks % 2
         constexpr int SET = DEPTH == 2 ? nxt : 0;  // register set of tile ks + 1, refilled with tile ks + 1 + DEPTH
         const uint32_t knext = min(ks + 1 + DEPTH, ksteps - 1);
@@ -336,22 +335,22 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
             }
         };
         // what follows MFMA number `slot` of the tile (KK == 4)
-        auto after_mfma = [&](int slot, bool reads, int next_buf, int from, int next_kk) {
+        auto after_mfma = [&](int slot, int next_buf, int from, int next_kk) {
             if constexpr (MID) {
-                if (reads) read_one(next_buf, from, next_kk, RORDER[slot % NMFMA]);
+                read_one(next_buf, from, next_kk, RORDER[slot % NMFMA]);
                 if (slot < NLOAD) piece_op(slot, true);
                 else piece_op(slot - NLOAD, false);
             } else if (slot % 2 == 0) {
-                if (reads) read_one(next_buf, from, next_kk, RORDER[(slot % NMFMA) / 2]);
+                read_one(next_buf, from, next_kk, RORDER[(slot % NMFMA) / 2]);
 #pragma unroll
                 for (int i = 0; i < 16; ++i)
-                    if (STORE && SCH.st[i] == slot / 2) piece_pack(i);
+                    if (SCH.st[i] == slot / 2) piece_pack(i);
             } else {
                 const int o = slot / 2;
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
-                    if (STORE && SCH.st[i] == o) piece_op(i, true);
-                    if (LOAD && SCH.ld[i] == o) piece_op(i, false);
+                    if (SCH.st[i] == o) piece_op(i, true);
+                    if (SCH.ld[i] == o) piece_op(i, false);
                 }
             }
         };
@@ -361,15 +360,15 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
             for (int m = 0; m < NMFMA; ++m) {
                 mfma_one(kk & 1, m);
                 if constexpr (KK > 2) {
-                    after_mfma(kk * NMFMA + m, true, (kk + 1) & 1, cur, kk + 1);
+                    after_mfma(kk * NMFMA + m, (kk + 1) & 1, cur, kk + 1);
                 } else {
                     // two k-steps of 4 MFMAs per tile: reads and stores under the first, then all loads
                     if (m < NREAD) read_one((kk + 1) & 1, cur, kk + 1, m);
-                    if (STORE && m < NLOAD) piece_op(m, true);
+                    if (m < NLOAD) piece_op(m, true);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (LOAD && KK == 2 && kk == 0) {
+            if (KK == 2 && kk == 0) {
                 fetch_all(SET, pnext, qnext);
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -380,8 +379,8 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
 #pragma unroll
         for (int m = 0; m < NMFMA; ++m) {
             mfma_one((KK - 1) & 1, m);
-            if constexpr (KK > 2) after_mfma((KK - 1) * NMFMA + m, STORE, 0, nxt, 0);
-            else if (STORE && m < NREAD) read_one(0, nxt, 0, m);
+            if constexpr (KK > 2) after_mfma((KK - 1) * NMFMA + m, 0, nxt, 0);
+            else if (m < NREAD) read_one(0, nxt, 0, m);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
