@@ -187,6 +187,20 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
             split = (slabs + sps - 1) / sps;
             p.k_per_split = (uint32_t)(sps * 32);
             p.split_k = (uint32_t)split;
+            // A long l-contiguous Q (a weight stored [N, K]): the mode that reads 256 contiguous bytes per
+            // column, in K-chunks of 128 dealt to the four waves; needs whole chunks and at least one per wave.
+            if (g.qmode == 1 && p.N % 128 == 0 && p.K % 128 == 0) {
+                // (cold-weight sweeps: at least 8 chunks per split, i.e. two per wave, or the split costs more than it hides)
+                const size_t chunks = p.K / 128;
+                if (!std::getenv("OPHIP_GEMM_SPLITK")) split = std::min(split, std::max<size_t>(1, chunks / 8));
+                const size_t cps = (chunks + split - 1) / split;  // chunks per split
+                if (cps >= 4) {
+                    g.qmode = 2;
+                    split = (chunks + cps - 1) / cps;
+                    p.k_per_split = (uint32_t)(cps * 128);
+                    p.split_k = (uint32_t)split;
+                }
+            }
             g.workspace = split > 1 ? split * p.batch * (size_t)p.M * p.N * sizeof(float) : 0;
             return g;
         }
@@ -265,7 +279,7 @@ constexpr size_t SPLITK_COUNTERS = 1 << 16;
 
 struct ophip_mat_mul {
     ophip_device *dev;
-    hipFunction_t skinny[3][2];  // [mt index 1,2,4][qmode]
+    hipFunction_t skinny[3][3];  // [mt index 1,2,4][qmode]
     hipFunction_t reduce, generic_f16, generic_f32;
     hipFunction_t tile[3][2][2];  // [256 x 64 / 128 x 64 / 128 x 32 (K-step)][P K-contiguous][Q K-contiguous]
     // Arrival counters live in a buffer owned by the operator, one per stream:
@@ -288,7 +302,7 @@ struct ophip_mat_mul {
         ophip_device_retain(d);
         static const int mts[3] = {1, 2, 4};
         for (int i = 0; i < 3; ++i)
-            for (int q = 0; q < 2; ++q)
+            for (int q = 0; q < 3; ++q)
                 skinny[i][q] =
                     d->kernel("gemm", ("gemm_skinny_m" + std::to_string(mts[i]) + "_q" + std::to_string(q)).c_str());
         for (int b = 0; b < 3; ++b)
@@ -348,7 +362,8 @@ int ophip_mat_mul_describe(const ophip_mat_mul *op, const ophip_mat_mul_args *ar
         if (L.dt != OPHIP_DT_F16 && L.dt != OPHIP_DT_F32) throw type_not_support("mat_mul supports f16 and f32");
         const GemmPlan g = make_plan(*args, L, (unsigned)op->dev->props.multiProcessorCount);
         if (g.kind == GemmPlan::Skinny)
-            std::snprintf(out, len, "skinny rows<=%d q%s split_k=%u", 16 * g.mt, g.qmode ? "K" : "N", g.p.split_k);
+            std::snprintf(out, len, "skinny rows<=%d q%s split_k=%u", 16 * g.mt, g.qmode == 0 ? "N" : g.qmode == 1 ? "K" : "K256",
+                          g.p.split_k);
         else if (g.kind == GemmPlan::Tile)
             std::snprintf(out, len, "tile%dx%d p%s q%s split_k=%u", g.tile, g.tk, g.pk ? "K" : "M", g.qk ? "K" : "N", g.p.split_k);
         else

@@ -25,6 +25,13 @@
 //     per column offset t.
 //   QMODE 1 (Q is l-contiguous, e.g. K-cache used as K^T): one 16-byte load per
 //     column offset t already is the B operand.
+//   QMODE 2 (Q is l-contiguous and long in l, e.g. a weight stored [N, K]): QMODE 1 reads 64
+//     bytes per column and instruction.  Here a wave step is 128 of K x 32 columns: the 16 lanes
+//     l % 16 read 256 contiguous bytes of one column, an instruction covers 4 columns, and the
+//     tile goes through a wave-private LDS buffer to reach the MFMA operand layout (8 writes and
+//     8 reads of 16 bytes per lane and step; LDS operations of one wave stay in order, so the
+//     buffer needs no barrier).  Step cg of a K-chunk holds the columns 8n + 2cg + {0, 1},
+//     n = 0..15, so the accumulators end up exactly as in the other modes.
 // MFMA number t multiplies the 16 rows of P with the 16 columns {n0 + 8j + t};
 // after the eight of them a lane holds, for 4 rows, 8 consecutive columns: one
 // 16-byte store per row.
@@ -121,9 +128,12 @@ __device__ __forceinline__ void skinny_store(const GemmParams &p, uint32_t bat, 
     }
 }
 
+constexpr int SK_TR_PITCH = 272;  // bytes per LDS row of the QMODE 2 transposition buffer: 256 + 16 (an odd number of 16-byte units)
+
 template <int MT, int QMODE>
 __device__ __forceinline__ void gemm_skinny(const GemmParams &p) {
     __shared__ float red[SK_WAVES][32][WAVE];
+    __shared__ __attribute__((aligned(16))) char tr_all[QMODE == 2 ? SK_WAVES * 32 * SK_TR_PITCH : 16];
 
     const uint32_t wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
     const uint32_t j16 = lane % 16, g = lane / 16;
@@ -148,78 +158,158 @@ __device__ __forceinline__ void gemm_skinny(const GemmParams &p) {
     for (int mt = 0; mt < MT; ++mt) prow[mt] = pb + (int64_t)min(mt * 16 + j16, p.M - 1) * p.p_si + 8 * g;
     const uint32_t colc = min(col0, p.N - 8);
 
-    auto step = [&](const u32x4(&w)[8], const u32x4(&a)[MT]) {
-        u32x4 b[8];
-        if constexpr (QMODE == 0) {
-            transpose8x8(w, b);
-        } else {
-#pragma unroll
-            for (int t = 0; t < 8; ++t) b[t] = w[t];
-        }
+    if constexpr (QMODE == 2) {
+        // The host guarantees: Q l-contiguous, N a multiple of 128, this split's K range a multiple of 128.
+        char *tr = tr_all + wave * (32 * SK_TR_PITCH);
+        const uint32_t chunks = (kend - kbeg) / 128;
+        const uint32_t cnt = chunks > wave ? (chunks - wave + SK_WAVES - 1) / SK_WAVES : 0;  // K-chunks of this wave
+        // load t of a step: local column lc = 4t + g = (n, cb) = (lc / 2, lc % 2) -> column n0 + 8n + cb (+ 2cg),
+        // 8 of K at 8 * j16; LDS row cb * 16 + n
+        const f16 *qrow[8];
+        uint32_t wr_off[8];
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
-            Pack8 bt;
-            bt.u = b[t];
+            const uint32_t lc = 4 * t + g, n = lc / 2, cb = lc % 2;
+            qrow[t] = qb + (int64_t)(n0 + 8 * n + cb) * p.q_sj + 8 * j16;
+            wr_off[t] = (cb * 16 + n) * SK_TR_PITCH + j16 * 16;
+        }
+        const uint32_t rd_off = j16 * SK_TR_PITCH + g * 16;  // + cb * 16 rows + kb4 * 64 bytes
+        const int64_t cg_stride = 2 * p.q_sj;
+        u32x4 wbuf[4][8], a_cur[MT][4], a_nxt[MT][4];
+        auto kc_of = [&](uint32_t i) { return kbeg + 128 * (wave + SK_WAVES * min(i, cnt - 1)); };
+        auto issue_w = [&](auto U, uint32_t i, int cg) {
+            constexpr int u = decltype(U)::value;
+            const uint32_t kc = kc_of(i);
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                Pack8 at;
-                at.u = a[mt];
-                acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(at.h, bt.h, acc[mt][t], 0, 0, 0);
+            for (int t = 0; t < 8; ++t) wbuf[u][t] = ld128_nt(qrow[t] + cg * cg_stride + kc);
+        };
+        auto issue_a = [&](u32x4(&a)[MT][4], uint32_t i) {
+            const uint32_t kc = kc_of(i);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int kb4 = 0; kb4 < 4; ++kb4) a[mt][kb4] = ld128(prow[mt] + kc + 32 * kb4);
+        };
+        auto compute = [&](auto U, int cg) {
+            constexpr int u = decltype(U)::value;
+#pragma unroll
+            for (int t = 0; t < 8; ++t) st128(tr + wr_off[t], wbuf[u][t]);
+#pragma unroll
+            for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+                for (int kb4 = 0; kb4 < 4; ++kb4) {
+                    Pack8 bt;
+                    bt.u = ld128(tr + rd_off + cb * (16 * SK_TR_PITCH) + kb4 * 64);
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt) {
+                        Pack8 at;
+                        at.u = a_cur[mt][kb4];
+                        acc[mt][2 * cg + cb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(at.h, bt.h, acc[mt][2 * cg + cb], 0, 0, 0);
+                    }
+                }
+        };
+        using I0 = std::integral_constant<int, 0>;
+        using I1 = std::integral_constant<int, 1>;
+        using I2 = std::integral_constant<int, 2>;
+        using I3 = std::integral_constant<int, 3>;
+        if (cnt > 0) {
+            issue_a(a_cur, 0);
+            issue_w(I0{}, 0, 0);
+            issue_w(I1{}, 0, 1);
+            issue_w(I2{}, 0, 2);
+            // Four steps (one K-chunk) per trip; the loads of the next three steps are in flight.  Past the
+            // last chunk the loads fetch it again and nobody uses them.
+            for (uint32_t i = 0; i < cnt; ++i) {
+                issue_w(I3{}, i, 3);
+                issue_a(a_nxt, i + 1);
+                compute(I0{}, 0);
+                issue_w(I0{}, i + 1, 0);
+                compute(I1{}, 1);
+                issue_w(I1{}, i + 1, 1);
+                compute(I2{}, 2);
+                issue_w(I2{}, i + 1, 2);
+                compute(I3{}, 3);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                    for (int kb4 = 0; kb4 < 4; ++kb4) a_cur[mt][kb4] = a_nxt[mt][kb4];
             }
         }
-    };
-
-    // Full K-steps run through a ring of three register buffers: while one step is
-    // being multiplied, the loads of the next two are in flight (16 KB per wave).
-    const uint32_t kfull = kbeg + (kend - kbeg) / 32 * 32;  // end of the full steps
-    constexpr uint32_t STRIDE = 32 * SK_WAVES;
-    const uint32_t kb0 = kbeg + 32 * wave;
-    const uint32_t cnt = kfull > kb0 ? (kfull - kb0 + STRIDE - 1) / STRIDE : 0;  // full steps of this wave
-    u32x4 wbuf[3][8], abuf[3][MT];
-    auto issue = [&](auto U, uint32_t idx) {
-        constexpr int u = decltype(U)::value;
-        const uint32_t kb = kb0 + idx * STRIDE;
+    } else {
+    auto step = [&](const u32x4(&w)[8], const u32x4(&a)[MT]) {
+            u32x4 b[8];
+            if constexpr (QMODE == 0) {
+                transpose8x8(w, b);
+            } else {
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) abuf[u][mt] = ld128(prow[mt] + kb);
-        skinny_load_q<QMODE>(p, qb, kb, colc, g, wbuf[u]);
-    };
-    using I0 = std::integral_constant<int, 0>;
-    using I1 = std::integral_constant<int, 1>;
-    using I2 = std::integral_constant<int, 2>;
-    uint32_t issued = 0, done = 0;
-    if (cnt > 0) { issue(I0{}, 0); issued = 1; }
-    if (cnt > 1) { issue(I1{}, 1); issued = 2; }
-    while (issued + 3 <= cnt) {
-        issue(I2{}, issued);
-        step(wbuf[0], abuf[0]);
-        issue(I0{}, issued + 1);
-        step(wbuf[1], abuf[1]);
-        issue(I1{}, issued + 2);
-        step(wbuf[2], abuf[2]);
-        issued += 3;
-        done += 3;
-    }
-    const uint32_t rem = cnt - issued;  // 0, 1 or 2 steps still to load
-    if (done < cnt) {
-        if (rem >= 1) issue(I2{}, issued);
-        step(wbuf[0], abuf[0]);
-    }
-    if (done + 1 < cnt) {
-        if (rem >= 2) issue(I0{}, issued + 1);
-        step(wbuf[1], abuf[1]);
-    }
-    if (rem >= 1) step(wbuf[2], abuf[2]);
-    if (rem >= 2) step(wbuf[0], abuf[0]);
-
-    if (kfull < kend && kb0 + cnt * STRIDE == kfull) {  // the ragged last step belongs to exactly one wave
-        const uint32_t kb = kfull;
+                for (int t = 0; t < 8; ++t) b[t] = w[t];
+            }
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            abuf[0][mt] = u32x4{0, 0, 0, 0};
-            if (kb + 8 * g < kend) abuf[0][mt] = ld128(prow[mt] + kb);
+            for (int t = 0; t < 8; ++t) {
+                Pack8 bt;
+                bt.u = b[t];
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    Pack8 at;
+                    at.u = a[mt];
+                    acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(at.h, bt.h, acc[mt][t], 0, 0, 0);
+                }
+            }
+        };
+
+        // Full K-steps run through a ring of three register buffers: while one step is
+        // being multiplied, the loads of the next two are in flight (16 KB per wave).
+        const uint32_t kfull = kbeg + (kend - kbeg) / 32 * 32;  // end of the full steps
+        constexpr uint32_t STRIDE = 32 * SK_WAVES;
+        const uint32_t kb0 = kbeg + 32 * wave;
+        const uint32_t cnt = kfull > kb0 ? (kfull - kb0 + STRIDE - 1) / STRIDE : 0;  // full steps of this wave
+        u32x4 wbuf[3][8], abuf[3][MT];
+        auto issue = [&](auto U, uint32_t idx) {
+            constexpr int u = decltype(U)::value;
+            const uint32_t kb = kb0 + idx * STRIDE;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) abuf[u][mt] = ld128(prow[mt] + kb);
+            skinny_load_q<QMODE>(p, qb, kb, colc, g, wbuf[u]);
+        };
+        using I0 = std::integral_constant<int, 0>;
+        using I1 = std::integral_constant<int, 1>;
+        using I2 = std::integral_constant<int, 2>;
+        uint32_t issued = 0, done = 0;
+        if (cnt > 0) { issue(I0{}, 0); issued = 1; }
+        if (cnt > 1) { issue(I1{}, 1); issued = 2; }
+        while (issued + 3 <= cnt) {
+            issue(I2{}, issued);
+            step(wbuf[0], abuf[0]);
+            issue(I0{}, issued + 1);
+            step(wbuf[1], abuf[1]);
+            issue(I1{}, issued + 2);
+            step(wbuf[2], abuf[2]);
+            issued += 3;
+            done += 3;
         }
-        skinny_load_q_tail<QMODE>(p, qb, kb, kend, colc, g, wbuf[0]);
-        step(wbuf[0], abuf[0]);
+        const uint32_t rem = cnt - issued;  // 0, 1 or 2 steps still to load
+        if (done < cnt) {
+            if (rem >= 1) issue(I2{}, issued);
+            step(wbuf[0], abuf[0]);
+        }
+        if (done + 1 < cnt) {
+            if (rem >= 2) issue(I0{}, issued + 1);
+            step(wbuf[1], abuf[1]);
+        }
+        if (rem >= 1) step(wbuf[2], abuf[2]);
+        if (rem >= 2) step(wbuf[0], abuf[0]);
+
+        if (kfull < kend && kb0 + cnt * STRIDE == kfull) {  // the ragged last step belongs to exactly one wave
+            const uint32_t kb = kfull;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                abuf[0][mt] = u32x4{0, 0, 0, 0};
+                if (kb + 8 * g < kend) abuf[0][mt] = ld128(prow[mt] + kb);
+            }
+            skinny_load_q_tail<QMODE>(p, qb, kb, kend, colc, g, wbuf[0]);
+            step(wbuf[0], abuf[0]);
+        }
+
     }
 
     // combine the 4 waves, then row = mt*16 + 4g + wave, columns col0 .. col0+7
@@ -312,6 +402,9 @@ GEMM_SKINNY(4, 0)
 GEMM_SKINNY(1, 1)
 GEMM_SKINNY(2, 1)
 GEMM_SKINNY(4, 1)
+GEMM_SKINNY(1, 2)
+GEMM_SKINNY(2, 2)
+GEMM_SKINNY(4, 2)
 
 // One thread per (batch, row, 8 columns): partial sums in ascending split order.
 extern "C" __global__ void __launch_bounds__(256) gemm_splitk_reduce(GemmParams p) {

@@ -810,6 +810,30 @@ def test_mat_mul_decode_layer_shapes(gpu, stream, name, bt, m, n, k, b_transpose
         oracle.set_threads(1)
 
 
+@pytest.mark.parametrize("m,n,k,bt,beta", [(16, 12288, 4096, 1, 0.0), (16, 4096, 11008, 1, 0.5), (16, 4096, 4096, 1, 0.0),
+                                           (24, 1024, 2048, 2, 1.0), (40, 512, 1024, 1, 0.0), (64, 384, 512, 3, 0.5)])
+def test_mat_mul_weights_stored_n_by_k(gpu, stream, m, n, k, bt, beta):
+    """Weights kept as [N, K] (K-contiguous, the layout of a PyTorch Linear): the weight-streaming kernel's
+    mode that reads 256 contiguous bytes per column and transposes through LDS, for 16, 32 and 64-row blocks,
+    with and without split K, batched, with beta."""
+    rng = np.random.default_rng(m + n + k)
+    shape = lambda *s: (bt,) + s if bt > 1 else s
+    a = normal_f16(rng, shape(m, k), std=1.0)
+    w = normal_f16(rng, shape(n, k), std=0.02)
+    b = w.swapaxes(-1, -2)
+    c = normal_f16(rng, shape(m, n), std=1.0)
+    args = ophip.MatMulArgs(TensorLayout.of(c), None, beta, TensorLayout.of(a), None, TensorLayout.of(b), None, 1.0)
+    what = ophip.MatMul(gpu).describe(args)
+    say("mat_mul [N,K] weights %dx%dx%d bt=%d: %s" % (m, n, k, bt, what))
+    assert "qK256" in what, what
+    oracle.set_threads(8)
+    try:
+        out = run_mat_mul(gpu, stream, c, a, b, 1.0, beta)
+        check_mat_mul(out, c, a, b, 1.0, beta, "mat_mul [N,K] weights")
+    finally:
+        oracle.set_threads(1)
+
+
 @pytest.mark.parametrize("ta", [False, True])
 @pytest.mark.parametrize("tb", [False, True])
 @pytest.mark.parametrize("tc", [False, True])
