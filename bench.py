@@ -366,6 +366,27 @@ def standalone_ops(ophip, gpu, stream, rng, reps):
     us = time_launches(gpu, stream, lambda: akv.launch(a, ws, stream), reps)
     add("attention_kv_cached", "nh32 seq16 pos2032 dh128", 2 * NH * KV * DH * 2 + 8 * nt * D * 2, us,
         note="composite of 7 launches; bytes = both caches read once + q, k, v, o and the appended rows")
+    # the dominant decode GEMM (gate/up) on its own, weights stored [K, N] and [N, K]: two copies of the
+    # weights alternate so that no launch finds them in the Infinity Cache
+    mm = o.MatMul(gpu)
+    xa = gpu.from_host(normal_f16(rng, (nt, D), 1.0))
+    ya = gpu.malloc(nt * 2 * DI * 2)
+    w2 = [gpu.from_host(normal_f16(rng, (D, 2 * DI), 0.02)) for _ in range(2)]
+    wsb = gpu.malloc(64 << 20)
+    for b_nk in (False, True):
+        bl = L(F16, [D, 2 * DI], [2, D * 2]) if b_nk else c(D, 2 * DI)
+        pair = [o.MatMulArgs(c(nt, 2 * DI), ya, 0.0, c(nt, D), xa, bl, w, 1.0) for w in w2]
+        flip = [0]
+
+        def run():
+            flip[0] ^= 1
+            mm.launch(pair[flip[0]], wsb, stream)
+        us = time_launches(gpu, stream, run, reps)
+        add("mat_mul", "%dx%dx%d%s" % (nt, 2 * DI, D, ", B stored [N,K]" if b_nk else ""),
+            2 * (nt * D + D * 2 * DI + nt * 2 * DI), us, flops=2 * nt * D * 2 * DI, note="cold weights, " + mm.describe(pair[0]))
+    for w in w2:
+        w.free()
+    wsb.free(); xa.free(); ya.free()
     mat_mul_lines(o, gpu, stream, rng, add)
     return out
 
