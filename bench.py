@@ -392,8 +392,8 @@ def standalone_ops(ophip, gpu, stream, rng, reps):
 
 
 def cpu_per_op(oracle, threads):
-    """The CPU oracle on the benchmark configurations of the single operators (BASELINE.json configs 1 - 4),
-    best of three runs each; keys are (operator, shape) as in `per_op`."""
+    """The CPU oracle on the benchmark configurations of the single operators (rms_norm, rope and rearrange,
+    causal softmax, random_sample), best of three runs each; keys are (operator, shape) as in `per_op`."""
     rng = np.random.default_rng(0)
     oracle.set_threads(threads)
     out = {}

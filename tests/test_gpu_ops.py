@@ -783,12 +783,13 @@ DECODE_GEMMS = [
     ("down", 1, 16, 4096, 11008, False),
     ("qk_t", 32, 16, 2048, 128, True),
     ("pv", 32, 16, 128, 2048, False),
+    ("wide_288_strips", 1, 16, 36864, 1024, False),  # a few more column strips than CUs: K is halved
 ]
 
 
 @pytest.mark.parametrize("name,bt,m,n,k,b_transposed", DECODE_GEMMS)
 def test_mat_mul_decode_layer_shapes(gpu, stream, name, bt, m, n, k, b_transposed):
-    """The six GEMMs of a Llama-7B decode layer, 16 tokens, weights ~ N(0, 0.02) (std 0.02)."""
+    """The six GEMMs of a Llama-7B decode layer, 16 tokens, weights ~ N(0, 0.02) (std 0.02), and one wider weight."""
     rng = np.random.default_rng(len(name) + n)
     shape = lambda *s: (bt,) + s if bt > 1 else s
     if name in ("qk_t", "pv"):
