@@ -208,13 +208,15 @@ def adder(out):
 
 
 def mat_mul_lines(o, gpu, stream, rng, add, launches=0):
-    """Compute-bound mat_mul: square shapes in both layouts of B and the prefill GEMMs of a Llama-7B layer
-    at 512 tokens.  `launches` > 0: that many plain launches per shape and nothing else (counter runs)."""
+    """Compute-bound mat_mul: square shapes in both layouts of B, the prefill GEMMs of a Llama-7B layer
+    at 512 tokens, and two shapes that are no multiples of the tile (509 tokens; 4000 x 4000).
+    `launches` > 0: that many plain launches per shape and nothing else (counter runs)."""
     from ophip import TensorLayout as L, dt
     c = lambda *s: L.new_contiguous(dt.F16, list(s))
     mm = o.MatMul(gpu)
     shapes = [(4096, 4096, 4096, False), (4096, 4096, 4096, True), (8192, 8192, 8192, False), (8192, 8192, 8192, True),
-              (512, 12288, 4096, False), (512, 22016, 4096, False), (512, 4096, 11008, False)]
+              (512, 12288, 4096, False), (512, 22016, 4096, False), (512, 4096, 11008, False),
+              (509, 12288, 4096, False), (4000, 4000, 4096, False)]
     for m, n, k, b_nk in shapes:
         A_, B_, C_ = gpu.from_host(normal_f16(rng, (m, k), 1.0)), gpu.from_host(normal_f16(rng, (k, n), 0.02)), \
             gpu.malloc(m * n * 2)

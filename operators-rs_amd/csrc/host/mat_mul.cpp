@@ -211,8 +211,11 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
     }
     // Compute-bound shapes: the LDS-tiled MFMA kernel.  Of the two orientations take
     // the one whose epilogue can store several adjacent outputs per lane.
+    // M and N need not be whole tiles: the last tiles load clamped rows and store what exists; 16-byte
+    // loads along a contiguous i or j need that dimension in whole groups of 8.
     auto tile_ok = [&](uint32_t b) {
-        if (!f16 || p.K == 0 || p.K % (b == 256 ? 64 : 32) != 0 || p.M % b != 0 || p.N % b != 0) return false;
+        if (!f16 || p.K == 0 || p.K % (b == 256 ? 64 : 32) != 0) return false;
+        if ((p.p_sl != 1 && p.M % 8 != 0) || (p.q_sl != 1 && p.N % 8 != 0)) return false;
         if (!aligned16(p.p) || !aligned16(p.q) || !aligned16(p.d)) return false;
         if (!mult8(p.p_sb) || !mult8(p.q_sb) || !mult8(p.d_sb)) return false;
         if (!(p.p_sl == 1 ? mult8(p.p_si) : mult8(p.p_sl))) return false;
@@ -231,12 +234,13 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
         // gemm_splitk_reduce, which wants the orientation whose D is j-contiguous.
         size_t split = 1;
         {
-            const size_t wgs = (size_t)(L.m / b) * (L.n / b) * L.batch, target = b == 256 ? cus : 2 * (size_t)cus;
+            const size_t wgs = ((L.m + b - 1) / b) * ((L.n + b - 1) / b) * L.batch, target = b == 256 ? cus : 2 * (size_t)cus;
             const size_t ksteps = L.k / (L.k % 64 == 0 ? 64 : 32);
             if (wgs > 0 && wgs * 2 <= cus)
                 split = std::min<size_t>({target / wgs, (size_t)8, std::max<size_t>(1, ksteps / 8)});
             if (const char *e = std::getenv("OPHIP_GEMM_TILE_SPLITK")) split = std::max(1, std::atoi(e));
             split = std::max<size_t>(1, std::min(split, ksteps));
+            if (L.m % 8 != 0 || L.n % 8 != 0) split = 1;  // gemm_splitk_reduce works on groups of 8 columns
         }
         for (int attempt = 0; attempt < 2; ++attempt) {
             orient(attempt == 1);
@@ -246,9 +250,12 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
             // (OPHIP_GEMM_TILE=256 / 128 keeps one tile size, for tests and sweeps)
             const char *force = std::getenv("OPHIP_GEMM_TILE");
             if (force && (uint32_t)std::atoi(force) != b) continue;
-            if (b == 256 && !force && (size_t)(p.M / b) * (p.N / b) * p.batch * 5 < (size_t)cus * 3 && p.M % 128 == 0 &&
-                p.N % 128 == 0)
-                continue;
+            // and when the part of the last tiles that lies outside the matrix costs more than the large tile's
+            // advantage (about 1.4 x per multiply at these sizes)
+            if (b == 256 && !force) {
+                const size_t t256 = (size_t)((p.M + 255) / 256) * ((p.N + 255) / 256), t128 = (size_t)((p.M + 127) / 128) * ((p.N + 127) / 128);
+                if (t256 * p.batch * 5 < (size_t)cus * 3 || t256 * 4 * 5 > t128 * 7) continue;
+            }
             const bool wide = split > 1 ? p.d_sj == 1 : (p.q_sl != 1 && p.d_sj == 1) || (p.p_sl == 1 && p.d_si == 1);
             if (best < 0 || wide) best = attempt;
             if (wide) break;
@@ -285,7 +292,8 @@ struct ophip_mat_mul {
     ophip_device *dev;
     hipFunction_t skinny[3][3];  // [mt index 1,2,4][qmode]
     hipFunction_t reduce, generic_f16, generic_f32;
-    hipFunction_t tile[3][2][2];  // [256 x 64 / 128 x 64 / 128 x 32 (K-step)][P K-contiguous][Q K-contiguous]
+    // [256 x 64 / 128 x 64 / 128 x 32 (K-step)][M or N not in whole tiles][P K-contiguous][Q K-contiguous]
+    hipFunction_t tile[3][2][2][2];
     // Arrival counters live in a buffer owned by the operator, one per stream:
     // launches on one stream run in order and every kernel leaves its counters at
     // zero, so the buffer is zeroed once, when a stream is first seen.
@@ -310,12 +318,13 @@ struct ophip_mat_mul {
                 skinny[i][q] =
                     d->kernel("gemm", ("gemm_skinny_m" + std::to_string(mts[i]) + "_q" + std::to_string(q)).c_str());
         for (int b = 0; b < 3; ++b)
-            for (int pk = 0; pk < 2; ++pk)
-                for (int qk = 0; qk < 2; ++qk) {
-                    const std::string sz = b == 0 ? "256x256" : b == 1 ? "128x128" : "128x128k32";
-                    tile[b][pk][qk] = d->kernel(
-                        "gemm_tile", ("gemm_tile_" + sz + "_p" + std::to_string(pk) + "_q" + std::to_string(qk)).c_str());
-                }
+            for (int r = 0; r < 2; ++r)
+                for (int pk = 0; pk < 2; ++pk)
+                    for (int qk = 0; qk < 2; ++qk) {
+                        const std::string sz = b == 0 ? "256x256" : b == 1 ? "128x128" : "128x128k32";
+                        tile[b][r][pk][qk] = d->kernel("gemm_tile", ("gemm_tile_" + sz + (r ? "r" : "") + "_p" + std::to_string(pk) +
+                                                                    "_q" + std::to_string(qk)).c_str());
+                    }
         reduce = d->kernel("gemm", "gemm_splitk_reduce");
         generic_f16 = d->kernel("gemm", "gemm_generic_f16");
         generic_f32 = d->kernel("gemm", "gemm_generic_f32");
@@ -369,7 +378,8 @@ int ophip_mat_mul_describe(const ophip_mat_mul *op, const ophip_mat_mul_args *ar
             std::snprintf(out, len, "skinny rows<=%d q%s split_k=%u", 16 * g.mt, g.qmode == 0 ? "N" : g.qmode == 1 ? "K" : "K256",
                           g.p.split_k);
         else if (g.kind == GemmPlan::Tile)
-            std::snprintf(out, len, "tile%dx%d p%s q%s split_k=%u", g.tile, g.tk, g.pk ? "K" : "M", g.qk ? "K" : "N", g.p.split_k);
+            std::snprintf(out, len, "tile%dx%d%s p%s q%s split_k=%u", g.tile, g.tk,
+                          g.p.M % g.tile != 0 || g.p.N % g.tile != 0 ? " ragged" : "", g.pk ? "K" : "M", g.qk ? "K" : "N", g.p.split_k);
         else
             std::snprintf(out, len, "generic");
     });
@@ -404,8 +414,10 @@ int ophip_mat_mul_launch(const ophip_mat_mul *op, const ophip_mat_mul_args *args
         if (g.kind == GemmPlan::Tile) {
             Workspace ws(qa, workspace, workspace_len, g.workspace);
             g.p.partial = ws.ptr();
-            const unsigned tiles = (p.M / g.tile) * (p.N / g.tile);
-            launch(op->tile[g.tile == 256 ? 0 : g.tk == 64 ? 1 : 2][g.pk][g.qk], Dim3{tiles, p.split_k, p.batch}, Dim3{256}, 0, stream, g.p);
+            const unsigned tiles = ((p.M + g.tile - 1) / g.tile) * ((p.N + g.tile - 1) / g.tile);
+            const int ragged = p.M % g.tile != 0 || p.N % g.tile != 0;
+            launch(op->tile[g.tile == 256 ? 0 : g.tk == 64 ? 1 : 2][ragged][g.pk][g.qk], Dim3{tiles, p.split_k, p.batch}, Dim3{256}, 0,
+                   stream, g.p);
             if (p.split_k > 1) {
                 const size_t total = (size_t)p.batch * p.M * (p.N / 8);
                 launch(op->reduce, Dim3{(unsigned)((total + 255) / 256)}, Dim3{256}, 0, stream, g.p);

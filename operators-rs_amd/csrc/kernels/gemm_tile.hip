@@ -16,9 +16,10 @@
 // them) each work on a compact block of tiles and share operand panels in
 // their own L2.
 //
-// Requirements checked by the host: M % BM == 0, N % BN == 0, K % TK == 0 (TK = 64 for the
-// 256 tiles, 32 for the 128 tiles),
-// 16-byte aligned bases and strides.  Everything else runs on the generic kernel.
+// Requirements checked by the host: K % TK == 0 (TK = 64 for the 256 tiles, 64 or 32 for the
+// 128 tiles), 16-byte aligned bases and strides; M and N in whole tiles for the plain kernels, any
+// M and N for the `r` kernels (a dimension along which an operand is contiguous must be a multiple
+// of 8).  Everything else runs on the generic kernel.
 #include <type_traits>
 
 #include "device_util.h"
@@ -80,15 +81,22 @@ struct TileLoader {
 
     // s_row: stride between rows (i or j), s_k: stride along K, in elements; one of them is 1.
     // The host guarantees that offsets inside a tile fit 32 bits.
-    __device__ __forceinline__ void init(int64_t s_row, int64_t s_k) {
+    // CLAMP: only `rows` of the tile's R rows exist (the last tile of a dimension that is not a
+    // multiple of R).  The threads of the missing rows load an existing row instead (the last one,
+    // or for a row-contiguous operand the last group of 8: there the host guarantees rows % 8 == 0);
+    // what they store to LDS only reaches accumulators that the epilogue drops.
+    template <bool CLAMP>
+    __device__ __forceinline__ void init(int64_t s_row, int64_t s_k, uint32_t rows) {
         const uint32_t t = threadIdx.x;
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
             if constexpr (KCONTIG) {
-                const uint32_t idx = t + v * 256, row = idx / KV, kv = idx % KV;
+                const uint32_t idx = t + v * 256, kv = idx % KV;
+                const uint32_t row = CLAMP ? min(idx / KV, rows - 1) : idx / KV;
                 voff[v] = (row * (uint32_t)s_row + kv * 8) * 2;
             } else {
-                const uint32_t cb = t % (R / 8), kb = t / (R / 8);
+                const uint32_t kb = t / (R / 8);
+                const uint32_t cb = CLAMP ? min(t % (R / 8), rows / 8 - 1) : t % (R / 8);
                 voff[v] = ((kb * NV + v) * (uint32_t)s_k + cb * 8) * 2;
             }
         }
@@ -155,7 +163,9 @@ struct TileLoader {
 };
 
 // DEPTH: operand tiles kept in flight in registers (1: the next one; 2: the next two, in two register sets).
-template <int BM, int BN, bool PK, bool QK, int TK, int DEPTH>
+// RAGGED: M and N need not be multiples of the tile; the last tiles load clamped rows and the
+// epilogue stores only what exists.
+template <int BM, int BN, bool PK, bool QK, int TK, int DEPTH, bool RAGGED>
 __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
     constexpr int LDK = TileRow<TK>::LDK;
     constexpr int WM = BM / 2, WN = BN / 2;  // wave tile
@@ -170,7 +180,8 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
 
     // XCD-aware tile order: ids are dealt round-robin over 8 XCDs; give each XCD a
     // contiguous run of tiles, walked in groups of 8 tile-rows so panels are reused.
-    const uint32_t tiles_m = p.M / BM, tiles_n = p.N / BN, tiles = tiles_m * tiles_n;
+    const uint32_t tiles_m = RAGGED ? (p.M + BM - 1) / BM : p.M / BM, tiles_n = RAGGED ? (p.N + BN - 1) / BN : p.N / BN;
+    const uint32_t tiles = tiles_m * tiles_n;
     uint32_t id = blockIdx.x;
     {
         const uint32_t per_xcd = (tiles + 7) / 8;
@@ -214,8 +225,8 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
     constexpr int KK = TK / 16;  // MFMA k-steps per LDS tile
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
-        lp[d].init(p.p_si, p.p_sl);
-        lq[d].init(p.q_sj, p.q_sl);
+        lp[d].template init<RAGGED>(p.p_si, p.p_sl, min((uint32_t)BM, p.M - i0));
+        lq[d].template init<RAGGED>(p.q_sj, p.q_sl, min((uint32_t)BN, p.N - j0));
     }
     const f16 *ptile = pb + (int64_t)i0 * p.p_si + (int64_t)kbeg * p.p_sl;
     const f16 *qtile = qb + (int64_t)j0 * p.q_sj + (int64_t)kbeg * p.q_sl;
@@ -406,10 +417,13 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 const uint32_t i = i0 + LP::row_of_slot(LP::reader_slot(wm, tm, 8 * (e / 4) + 4 * lk + (e % 4)));
+                if (RAGGED && i >= p.M) continue;
                 float *row = part + (size_t)i * p.N + j0;
                 if constexpr (LQ::PERMUTED) {
-                    // the lane's TN tiles are TN adjacent columns
-                    float *dst = row + LQ::row_of_slot(LQ::reader_slot(wn, 0, l32));
+                    // the lane's TN tiles are TN adjacent columns (all inside N or all outside: N % 8 == 0)
+                    const uint32_t jl = LQ::row_of_slot(LQ::reader_slot(wn, 0, l32));
+                    if (RAGGED && j0 + jl >= p.N) continue;
+                    float *dst = row + jl;
                     if constexpr (TN == 4) *reinterpret_cast<f32x4 *>(dst) = f32x4{acc[tm][0][e], acc[tm][1][e], acc[tm][2][e], acc[tm][3][e]};
                     else {
 #pragma unroll
@@ -417,7 +431,10 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
                     }
                 } else {
 #pragma unroll
-                    for (int tn = 0; tn < TN; ++tn) row[LQ::row_of_slot(LQ::reader_slot(wn, tn, l32))] = acc[tm][tn][e];
+                    for (int tn = 0; tn < TN; ++tn) {
+                        const uint32_t jl = LQ::row_of_slot(LQ::reader_slot(wn, tn, l32));
+                        if (!RAGGED || j0 + jl < p.N) row[jl] = acc[tm][tn][e];
+                    }
                 }
             }
         return;
@@ -431,6 +448,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 const uint32_t i = i0 + LP::row_of_slot(LP::reader_slot(wm, tm, 8 * (e / 4) + 4 * lk + (e % 4)));
+                if (RAGGED && (i >= p.M || j >= p.N)) continue;  // j .. j + TN - 1 are inside N together: N % 8 == 0
                 f16 *dst = db + (int64_t)i * p.d_si + j;
                 union { f16 h[TN]; uint32_t u[TN / 2]; } o, c;
                 if (p.read_dst) {
@@ -446,7 +464,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
 #pragma unroll
                 for (int w = 0; w < TN / 2; ++w) reinterpret_cast<uint32_t *>(dst)[w] = o.u[w];
             }
-    } else if (!LP::PERMUTED && p.d_si == 1) {
+    } else if (!LP::PERMUTED && p.d_si == 1 && (!RAGGED || p.M % 4 == 0)) {
         // four consecutive accumulator rows are four adjacent rows of D: 8-byte stores
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm)
@@ -456,6 +474,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
                     const uint32_t i = i0 + wm * WM + tm * 32 + 8 * q + 4 * lk;
+                    if (RAGGED && (i >= p.M || j >= p.N)) continue;
                     f16 *dst = db + i + (int64_t)j * p.d_sj;
                     union { f16 h[4]; u32x2 u; } o, c;
                     if (p.read_dst) c.u = *reinterpret_cast<const u32x2 *>(dst);
@@ -477,6 +496,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     const uint32_t i = i0 + LP::row_of_slot(LP::reader_slot(wm, tm, 8 * (e / 4) + 4 * lk + (e % 4)));
+                    if (RAGGED && (i >= p.M || j >= p.N)) continue;
                     f16 *dst = db + (int64_t)i * p.d_si + (int64_t)j * p.d_sj;
                     float v = p.alpha * acc[tm][tn][e];
                     if (p.read_dst) v = p.beta * h2f(*dst) + v;
@@ -486,9 +506,15 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
     }
 }
 
-#define GEMM_TILE(NAME, BM, BN, PK, QK, TK, DEPTH)                                                 \
-    extern "C" __global__ void __launch_bounds__(256) gemm_tile_##NAME##_p##PK##_q##QK(GemmParams p) { \
-        gemm_tile<BM, BN, PK, QK, TK, DEPTH>(p);                                                   \
+// Every tile in two builds: for M and N in whole tiles (no clamps, no store guards), and `r` for the rest.
+// (One build with the guards switched by a kernel argument runs the whole-tile shapes 3 - 4 % slower:
+// the guards change the register allocation of the main loop.)
+#define GEMM_TILE(NAME, BM, BN, PK, QK, TK, DEPTH)                                                    \
+    extern "C" __global__ void __launch_bounds__(256) gemm_tile_##NAME##_p##PK##_q##QK(GemmParams p) {    \
+        gemm_tile<BM, BN, PK, QK, TK, DEPTH, false>(p);                                               \
+    }                                                                                                 \
+    extern "C" __global__ void __launch_bounds__(256) gemm_tile_##NAME##r_p##PK##_q##QK(GemmParams p) {   \
+        gemm_tile<BM, BN, PK, QK, TK, DEPTH, true>(p);                                                \
     }
 
 GEMM_TILE(256x256, 256, 256, 1, 1, 64, 1)

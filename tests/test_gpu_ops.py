@@ -942,6 +942,28 @@ def test_mat_mul_compute_bound_shape(gpu, stream):
     assert_close_f16(out[:64], sub, "2048^3 rows 0..63", abs_tol=2e-3 + 4e-3 * float(np.abs(sub).max()))
 
 
+@pytest.mark.parametrize("tokens,n,k,b_transposed,beta", [(509, 1536, 1024, False, 0.0), (509, 1536, 1024, True, 0.5),
+                                                          (100, 12288, 4096, False, 0.0), (300, 1000, 2048, True, 1.0),
+                                                          (65, 136, 64, False, 0.0)])
+def test_mat_mul_prefill_with_any_token_count(gpu, stream, tokens, n, k, b_transposed, beta):
+    """A prefill GEMM whose token count is no multiple of the tile (and a weight whose width is not either):
+    still the MFMA tile kernel, with its last tiles cut."""
+    rng = np.random.default_rng(tokens + n)
+    a = normal_f16(rng, (tokens, k), std=1.0)
+    b = normal_f16(rng, (n, k), std=0.02).T if b_transposed else normal_f16(rng, (k, n), std=0.02)
+    c = normal_f16(rng, (tokens, n), std=1.0)
+    args = ophip.MatMulArgs(TensorLayout.of(c), None, beta, TensorLayout.of(a), None, TensorLayout.of(b), None, 1.0)
+    what = ophip.MatMul(gpu).describe(args)
+    say("mat_mul prefill %d x %d x %d [%s]" % (tokens, n, k, what))
+    assert what.startswith("tile") and "ragged" in what, what
+    oracle.set_threads(8)
+    try:
+        out = run_mat_mul(gpu, stream, c, a, b, 1.0, beta)
+        check_mat_mul(out, c, a, b, 1.0, beta, "prefill %d tokens" % tokens)
+    finally:
+        oracle.set_threads(1)
+
+
 def test_mat_mul_beta_zero_never_reads_c_and_scalars_round_to_f16(gpu, stream):
     a = np.ones((16, 2048), f16)
     a[:, 2047] = 0  # 2047 ones per row

@@ -244,3 +244,53 @@ def test_random_mat_mul_tile_shapes(gpu, stream, monkeypatch, sweep):
     finally:
         oracle.set_threads(1)
     say("tile kernels exercised: %s" % sorted(seen))
+
+
+@SWEEPS
+def test_random_mat_mul_ragged_tile_shapes(gpu, stream, monkeypatch, sweep):
+    """More than 64 rows and columns that are no multiples of the 128 tile: the last tiles of the MFMA kernel load
+    clamped rows and store only what exists (guard zones around C catch a store past M or N).  Two thirds of the
+    cases have M and N in multiples of 8 with every operand layout; the others an odd M with A and C row-major
+    (nothing is contiguous along M then).  Some have few tiles and a long K (split K over ragged tiles).  Every
+    fourth case keeps the 256 x 256 tile, which the library would only choose for much larger outputs."""
+    rng = np.random.default_rng(731 + 1000 * sweep)
+    mm = ophip.MatMul(gpu)
+    oracle.set_threads(8)
+    try:
+        for case in range(24):
+            odd_m = case % 3 == 2
+            big = case % 4 == 1
+            if big:
+                monkeypatch.setenv("OPHIP_GEMM_TILE", "256")
+            else:
+                monkeypatch.delenv("OPHIP_GEMM_TILE", raising=False)
+            n = 8 * int(rng.integers(9, 90))
+            m = 2 * int(rng.integers(33, 350)) + 1 if odd_m else 8 * int(rng.integers(9, 90))
+            k = int(rng.choice([64, 192, 1088, 2048]) if big else rng.choice([32, 64, 96, 192, 1056, 2048, 4096]))
+            bt = int(rng.choice([1, 1, 2]))
+            ta, tb, tc = (bool(rng.integers(0, 2)) for _ in range(3))
+            if odd_m:
+                ta = tc = False
+            pa, pb, pc = (int(rng.choice([0, 8])) for _ in range(3))
+            A = Guarded(gpu, rng, (bt, k, m) if ta else (bt, m, k), f16, pa, scale=0.25)
+            B = Guarded(gpu, rng, (bt, n, k) if tb else (bt, k, n), f16, pb, scale=0.25)
+            C = Guarded(gpu, rng, (bt, n, m) if tc else (bt, m, n), f16, pc)
+            tr = lambda g, t: (TensorLayout(dt.F16, [g.shape[0], g.shape[2], g.shape[1]], [g.strides[0], g.strides[2], g.strides[1]]),
+                               g.view().transpose(0, 2, 1)) if t else (g.layout, g.view())
+            (al, av), (bl, bv), (cl, cv) = tr(A, ta), tr(B, tb), tr(C, tc)
+            alpha, beta = float(rng.choice([1.0, 0.5])), float(rng.choice([0.0, 1.0, 0.5]))
+            args = ophip.MatMulArgs(cl, C.ptr, beta, al, A.ptr, bl, B.ptr, alpha)
+            what = mm.describe(args)
+            say("random ragged mat_mul %d: bt=%d m=%d n=%d k=%d t=%d%d%d pads=%d%d%d a=%g b=%g [%s]" % (
+                case, bt, m, n, k, ta, tb, tc, pa, pb, pc, alpha, beta, what))
+            assert what.startswith("tile256" if big else "tile128") and "ragged" in what, what
+            ref = cv.copy()
+            oracle.mat_mul(ref, beta, av, bv, alpha)
+            mm.launch(args, None, stream)
+            got = C.fetch(stream)
+            got = got.transpose(0, 2, 1) if tc else got
+            scale = float(np.abs(ref.astype(np.float64)).max()) + 1e-3
+            err = np.abs(got.astype(np.float64) - ref.astype(np.float64)).max()
+            assert err <= 2e-3 + 4e-3 * scale, (err, scale)
+    finally:
+        oracle.set_threads(1)
