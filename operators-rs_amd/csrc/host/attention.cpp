@@ -25,6 +25,17 @@ struct Lay3 {
         const ptrdiff_t e = (ptrdiff_t)ophip_dtype_nbytes(dt);
         return Lay3{{a, b, c}, {(ptrdiff_t)(b * c) * e, (ptrdiff_t)c * e, e}};
     }
+    // rows of c elements, each starting on a 16-byte boundary: what the MFMA mat_mul kernels need of a
+    // K-contiguous operand.  The score matrix lives in the operator's own workspace, so its row pitch is
+    // the operator's choice (the reference keeps it dense).
+    static size_t padded_row(uint64_t dt, size_t c) {
+        const size_t e = ophip_dtype_nbytes(dt), per16 = e && 16 % e == 0 ? 16 / e : 1;
+        return (c + per16 - 1) / per16 * per16;
+    }
+    static Lay3 padded_rows(uint64_t dt, size_t a, size_t b, size_t c) {
+        const ptrdiff_t e = (ptrdiff_t)ophip_dtype_nbytes(dt), ld = (ptrdiff_t)padded_row(dt, c);
+        return Lay3{{a, b, c}, {(ptrdiff_t)b * ld * e, ld * e, e}};
+    }
     static Lay3 dyn(size_t a, size_t b, size_t c) {  // TensorLayout::new_dyn with dynamic strides
         return Lay3{{a, b, c}, {OPHIP_DYN_ISIZE, OPHIP_DYN_ISIZE, OPHIP_DYN_ISIZE}};
     }
@@ -124,8 +135,8 @@ size_t attention_scheme(ophip_attention *op, const ophip_attention_args &args, s
         return wc.calculate(max_ws);
     }
     const size_t ele = ophip_dtype_nbytes(m.dt);
-    const Lay3 att = Lay3::contiguous(m.dt, m.nh, m.seq, m.att);
-    const size_t q_size = m.nh * m.seq * m.dh * ele, att_size = m.nh * m.seq * m.att * ele;
+    const Lay3 att = Lay3::padded_rows(m.dt, m.nh, m.seq, m.att);
+    const size_t q_size = m.nh * m.seq * m.dh * ele, att_size = m.nh * m.seq * Lay3::padded_row(m.dt, m.att) * ele;
     const size_t rest = max_ws > q_size + att_size ? max_ws - (q_size + att_size) : 0;  // saturating_sub
     wc.push_base(q_size);
     wc.push_base(att_size);
@@ -171,7 +182,7 @@ void attention_launch(const ophip_attention *op, const ophip_attention_args &arg
     const Lay3 kt{{nkvh, dh, att}, {nkvh_sk, dh_sk, att_sk}};
 
     const size_t q_size = merged ? 0 : nh * seq * dh * ele;
-    const size_t att_size = nh * seq * att * ele;
+    const size_t att_size = nh * seq * Lay3::padded_row(dt, att) * ele;
     Workspace ws(qa, workspace, workspace_len, q_size + att_size);
     char *q_buf = static_cast<char *>(ws.ptr());
     char *att_buf = q_buf + q_size;
@@ -195,8 +206,8 @@ void attention_launch(const ophip_attention *op, const ophip_attention_args &arg
         qx_lay = Lay3{{nkvh, head_group * seq, dh}, {(ptrdiff_t)(head_group * seq) * row_sq, row_sq, dh_sq}};
         q_base = args.q_base;
     }
-    const Lay3 att_mm = Lay3::contiguous(dt, nkvh, head_group * seq, att);
-    const Lay3 att_sm = Lay3::contiguous(dt, nh, seq, att);
+    const Lay3 att_mm = Lay3::padded_rows(dt, nkvh, head_group * seq, att);
+    const Lay3 att_sm = Lay3::padded_rows(dt, nh, seq, att);
 
     // att = q . k^T
     const ophip_mat_mul_args qk{att_mm.tl(dt), att_buf, 0.f, qx_lay.tl(dt), q_base, kt.tl(dt), args.k_base,

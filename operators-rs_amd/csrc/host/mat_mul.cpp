@@ -97,6 +97,7 @@ struct GemmPlan {
     enum Kind { Generic, Skinny, Tile } kind = Generic;
     int mt = 1, qmode = 0;
     int tile = 256, tk = 64, pk = 1, qk = 1;  // Tile: block size, K-step, and whether P / Q are K-contiguous
+    bool ragged = false;                      // Tile: M or N not in whole tiles, or K not in whole K-steps
     size_t workspace = 0;
 };
 
@@ -211,10 +212,13 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
     }
     // Compute-bound shapes: the LDS-tiled MFMA kernel.  Of the two orientations take
     // the one whose epilogue can store several adjacent outputs per lane.
+    // K-step of the tile kernels: 64, or 32 for a K in whole steps of 32 only; any other K from 64 on runs
+    // the 64 step with a partial last one; 0: K too short.
+    const size_t tile_tk = L.k % 64 == 0 ? 64 : L.k % 32 == 0 ? 32 : L.k >= 64 ? 64 : 0;
     // M and N need not be whole tiles: the last tiles load clamped rows and store what exists; 16-byte
     // loads along a contiguous i or j need that dimension in whole groups of 8.
     auto tile_ok = [&](uint32_t b) {
-        if (!f16 || p.K == 0 || p.K % (b == 256 ? 64 : 32) != 0) return false;
+        if (!f16 || p.K == 0 || tile_tk == 0 || (b == 256 && tile_tk != 64)) return false;
         if ((p.p_sl != 1 && p.M % 8 != 0) || (p.q_sl != 1 && p.N % 8 != 0)) return false;
         if (!aligned16(p.p) || !aligned16(p.q) || !aligned16(p.d)) return false;
         if (!mult8(p.p_sb) || !mult8(p.q_sb) || !mult8(p.d_sb)) return false;
@@ -235,7 +239,7 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
         size_t split = 1;
         {
             const size_t wgs = ((L.m + b - 1) / b) * ((L.n + b - 1) / b) * L.batch, target = b == 256 ? cus : 2 * (size_t)cus;
-            const size_t ksteps = L.k / (L.k % 64 == 0 ? 64 : 32);
+            const size_t ksteps = tile_tk ? L.k / tile_tk : 1;
             if (wgs > 0 && wgs * 2 <= cus)
                 split = std::min<size_t>({target / wgs, (size_t)8, std::max<size_t>(1, ksteps / 8)});
             if (const char *e = std::getenv("OPHIP_GEMM_TILE_SPLITK")) split = std::max(1, std::atoi(e));
@@ -266,8 +270,9 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
             g.tile = (int)b;
             g.pk = p.p_sl == 1;
             g.qk = p.q_sl == 1;
-            const size_t tk = p.K % 64 == 0 ? 64 : 32, ksteps = p.K / tk;
+            const size_t tk = tile_tk, ksteps = p.K / tk;
             g.tk = (int)tk;
+            g.ragged = p.M % b != 0 || p.N % b != 0 || p.K % tk != 0;
             if (split > 1) {
                 const size_t sps = (ksteps + split - 1) / split;
                 split = (ksteps + sps - 1) / sps;
@@ -379,7 +384,7 @@ int ophip_mat_mul_describe(const ophip_mat_mul *op, const ophip_mat_mul_args *ar
                           g.p.split_k);
         else if (g.kind == GemmPlan::Tile)
             std::snprintf(out, len, "tile%dx%d%s p%s q%s split_k=%u", g.tile, g.tk,
-                          g.p.M % g.tile != 0 || g.p.N % g.tile != 0 ? " ragged" : "", g.pk ? "K" : "M", g.qk ? "K" : "N", g.p.split_k);
+                          g.ragged ? " ragged" : "", g.pk ? "K" : "M", g.qk ? "K" : "N", g.p.split_k);
         else
             std::snprintf(out, len, "generic");
     });
@@ -415,8 +420,7 @@ int ophip_mat_mul_launch(const ophip_mat_mul *op, const ophip_mat_mul_args *args
             Workspace ws(qa, workspace, workspace_len, g.workspace);
             g.p.partial = ws.ptr();
             const unsigned tiles = ((p.M + g.tile - 1) / g.tile) * ((p.N + g.tile - 1) / g.tile);
-            const int ragged = p.M % g.tile != 0 || p.N % g.tile != 0;
-            launch(op->tile[g.tile == 256 ? 0 : g.tk == 64 ? 1 : 2][ragged][g.pk][g.qk], Dim3{tiles, p.split_k, p.batch}, Dim3{256}, 0,
+            launch(op->tile[g.tile == 256 ? 0 : g.tk == 64 ? 1 : 2][g.ragged][g.pk][g.qk], Dim3{tiles, p.split_k, p.batch}, Dim3{256}, 0,
                    stream, g.p);
             if (p.split_k > 1) {
                 const size_t total = (size_t)p.batch * p.M * (p.N / 8);

@@ -346,7 +346,7 @@ extern "C" int ophip_fused_softmax_launch(const ophip_fused_softmax *op, const o
         p.att_len = (uint32_t)att;
         p.causal = causal;
 
-        const bool vec = att % 8 == 0 && aligned16(p.att) && mult16(sh) && mult16(ss);
+        const bool vec = aligned16(p.att) && mult16(sh) && mult16(ss);
         const int want_vec = vec ? 8 : 1;
         // narrowest group that holds the row in registers; with few rows prefer a
         // whole workgroup per row so more lanes pull on memory

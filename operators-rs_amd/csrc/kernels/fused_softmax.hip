@@ -16,7 +16,8 @@ __device__ __forceinline__ uint32_t kept_columns(const SoftmaxParams &p, uint32_
     return p.causal ? p.att_len - p.seq + r + 1 : p.att_len;
 }
 
-// VEC = 8: 16-byte accesses (att_len % 8 == 0, 16-byte aligned rows); VEC = 1: element-wise.
+// VEC = 8: 16-byte accesses (16-byte aligned rows; the last, partial group of an att_len that is no
+// multiple of 8 goes element by element, so nothing past att_len is read or written); VEC = 1: element-wise.
 // PT = register slots per thread (vectors or elements).
 template <int VEC, int PT, int G>
 __device__ __forceinline__ void softmax_reg(const SoftmaxParams &p) {
@@ -41,7 +42,13 @@ __device__ __forceinline__ void softmax_reg(const SoftmaxParams &p) {
         if constexpr (VEC == 8) {
             Pack8 v;
             v.u = u32x4{0, 0, 0, 0};
-            if (col0 < kept) v.u = ld128(row + col0);
+            if (col0 + 8 <= p.att_len) {
+                if (col0 < kept) v.u = ld128(row + col0);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 7; ++e)
+                    if (col0 + e < kept) v.e[e] = row[col0 + e];
+            }
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 x[i][e] = col0 + e < kept ? h2f(v.e[e]) : -INFINITY;
@@ -79,7 +86,13 @@ __device__ __forceinline__ void softmax_reg(const SoftmaxParams &p) {
                 Pack8 o;
 #pragma unroll
                 for (int e = 0; e < 8; ++e) o.e[e] = col0 + e < kept ? f2h(x[i][e] * inv) : (f16)0.f;
-                st128(row + col0, o.u);
+                if (col0 + 8 <= p.att_len) {
+                    st128(row + col0, o.u);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 7; ++e)
+                        if (col0 + e < p.att_len) row[col0 + e] = o.e[e];
+                }
             } else {
                 row[col0] = col0 < kept ? f2h(x[i][0] * inv) : (f16)0.f;
             }

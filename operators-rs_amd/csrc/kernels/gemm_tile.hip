@@ -16,9 +16,9 @@
 // them) each work on a compact block of tiles and share operand panels in
 // their own L2.
 //
-// Requirements checked by the host: K % TK == 0 (TK = 64 for the 256 tiles, 64 or 32 for the
-// 128 tiles), 16-byte aligned bases and strides; M and N in whole tiles for the plain kernels, any
-// M and N for the `r` kernels (a dimension along which an operand is contiguous must be a multiple
+// Requirements checked by the host: 16-byte aligned bases and strides; for the plain kernels M and N
+// in whole tiles and K % TK == 0 (TK = 64 for the 256 tiles, 64 or 32 for the 128 tiles); the `r`
+// kernels take any M, N and K >= TK (M or N along which an operand is contiguous must be a multiple
 // of 8).  Everything else runs on the generic kernel.
 #include <type_traits>
 
@@ -114,6 +114,30 @@ struct TileLoader {
 #pragma unroll
         for (int v = 0; v < NV; ++v) fetch_piece(tile, v);
     }
+    // The last, partial K-step of a K that is no multiple of TK: only `kvalid` (< TK) of the tile's k exist,
+    // the rest is filled with zeros.  Runs once per workgroup, outside the pipelined loop.
+    __device__ __forceinline__ void fetch_tail(const f16 *tile, uint32_t kvalid) {
+        const uint32_t t = threadIdx.x;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const char *src = reinterpret_cast<const char *>(tile) + voff[v];
+            reg[v] = u32x4{0, 0, 0, 0};
+            if constexpr (KCONTIG) {
+                const uint32_t k0 = ((t + v * 256) % KV) * 8;  // first k of this vector
+                if (k0 + 8 <= kvalid) {
+                    reg[v] = *reinterpret_cast<const u32x4 *>(src);
+                } else if (k0 < kvalid) {
+                    const uint16_t *h = reinterpret_cast<const uint16_t *>(src);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if (k0 + e < kvalid) reg[v][e / 2] |= (uint32_t)h[e] << (16 * (e & 1));
+                }
+            } else {
+                const uint32_t k = (t / (R / 8)) * NV + v;  // this register's k-row
+                if (k < kvalid) reg[v] = *reinterpret_cast<const u32x4 *>(src);
+            }
+        }
+    }
 
     // Piece v of the register -> LDS copy.  K-contiguous: vector v.  Row-contiguous: reg[v]
     // holds k-row (kb*NV + v), columns cb*8 .. +8, and piece v writes columns
@@ -163,8 +187,9 @@ struct TileLoader {
 };
 
 // DEPTH: operand tiles kept in flight in registers (1: the next one; 2: the next two, in two register sets).
-// RAGGED: M and N need not be multiples of the tile; the last tiles load clamped rows and the
-// epilogue stores only what exists.
+// RAGGED: M and N need not be multiples of the tile (the last tiles load clamped rows and the
+// epilogue stores only what exists) nor K of TK (a last, partial K-step is loaded with zeros for
+// the missing k and multiplied after the pipelined loop); K >= TK.
 template <int BM, int BN, bool PK, bool QK, int TK, int DEPTH, bool RAGGED>
 __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
     constexpr int LDK = TileRow<TK>::LDK;
@@ -220,7 +245,8 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
     LQ lq[DEPTH];
     // split K: workgroup blockIdx.y multiplies K-range [kbeg, kbeg + klen) and leaves f32 partials
     const uint32_t split = blockIdx.y;
-    const uint32_t kbeg = split * p.k_per_split, klen = min(p.K - kbeg, p.k_per_split);
+    // (the last split also takes what is left of a K that is no multiple of TK; only the ragged builds see one)
+    const uint32_t kbeg = split * p.k_per_split, klen = split + 1 == p.split_k ? p.K - kbeg : p.k_per_split;
     const uint32_t ksteps = klen / TK;
     constexpr int KK = TK / 16;  // MFMA k-steps per LDS tile
 #pragma unroll
@@ -407,6 +433,24 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
         step(ks + 1, ODD);
     }
     if (ks < ksteps) step(ks, EVEN);
+    if constexpr (RAGGED) {
+        const uint32_t ktail = klen % TK;
+        if (ktail != 0) {  // workgroup-uniform
+            __syncthreads();  // every wave is done with the LDS buffers
+            lp[0].fetch_tail(ptile + ksteps * pstep, ktail);
+            lq[0].fetch_tail(qtile + ksteps * qstep, ktail);
+            lp[0].commit(p_buf(0));
+            lq[0].commit(q_buf(0));
+            __syncthreads();
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk) {
+#pragma unroll
+                for (int r = 0; r < NREAD; ++r) read_one(0, 0, kk, r);
+#pragma unroll
+                for (int m = 0; m < NMFMA; ++m) mfma_one(0, m);
+            }
+        }
+    }
 
     // 32x32 accumulator tile: lane holds slot-column l32 and slot-rows 8*(e/4) + 4*lk + e%4.
     if (p.split_k > 1) {
@@ -464,8 +508,9 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
 #pragma unroll
                 for (int w = 0; w < TN / 2; ++w) reinterpret_cast<uint32_t *>(dst)[w] = o.u[w];
             }
-    } else if (!LP::PERMUTED && p.d_si == 1 && (!RAGGED || p.M % 4 == 0)) {
-        // four consecutive accumulator rows are four adjacent rows of D: 8-byte stores
+    } else if (!LP::PERMUTED && p.d_si == 1) {
+        // four consecutive accumulator rows are four adjacent rows of D: 8-byte stores (the group that
+        // straddles a ragged M goes element by element)
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm)
 #pragma unroll
@@ -476,6 +521,16 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
                     const uint32_t i = i0 + wm * WM + tm * 32 + 8 * q + 4 * lk;
                     if (RAGGED && (i >= p.M || j >= p.N)) continue;
                     f16 *dst = db + i + (int64_t)j * p.d_sj;
+                    if (RAGGED && i + 4 > p.M) {
+#pragma unroll
+                        for (int r = 0; r < 3; ++r) {
+                            if (i + r >= p.M) break;
+                            float v = p.alpha * acc[tm][tn][4 * q + r];
+                            if (p.read_dst) v = p.beta * h2f(dst[r]) + v;
+                            dst[r] = f2h(v);
+                        }
+                        continue;
+                    }
                     union { f16 h[4]; u32x2 u; } o, c;
                     if (p.read_dst) c.u = *reinterpret_cast<const u32x2 *>(dst);
 #pragma unroll

@@ -43,7 +43,11 @@ def download(gpu, stream, mem, like):
 
 
 @pytest.mark.parametrize("nh,nkvh,seq,att,dh,mask", [(32, 4, 7, 127, 64, CAUSAL), (8, 8, 33, 33, 128, CAUSAL),
-                                                     (6, 2, 3, 40, 16, NONE), (4, 1, 1, 300, 64, CAUSAL)])
+                                                     (6, 2, 3, 40, 16, NONE), (4, 1, 1, 300, 64, CAUSAL),
+                                                     # prefill: more than 64 rows per kv head, odd att (the MFMA tile
+                                                     # kernels with cut last tiles and a partial last K-step)
+                                                     (8, 2, 200, 333, 64, CAUSAL), (4, 4, 509, 509, 128, CAUSAL),
+                                                     (4, 2, 100, 1001, 128, NONE)])
 def test_attention_contiguous(gpu, stream, nh, nkvh, seq, att, dh, mask):
     rng = np.random.default_rng(nh * 1000 + att)
     q, k, v = (rng.random(s).astype(f16) for s in ((nh, seq, dh), (nkvh, att, dh), (nkvh, att, dh)))
@@ -101,7 +105,8 @@ def test_attention_scheme_workspace_rules(gpu):
     c = lambda *s: TensorLayout.new_contiguous(dt.F16, list(s))
     args = ophip.AttentionArgs(c(nh, seq, dh), None, c(nkvh, att, dh), None, c(nkvh, att, dh), None, c(nh, seq, dh),
                                None, CAUSAL)
-    q_size, att_size = nh * seq * dh * 2, nh * seq * att * 2
+    # score rows are padded to 16 bytes (127 -> 128 columns): the operator's own buffer, MFMA-friendly
+    q_size, att_size = nh * seq * dh * 2, nh * seq * ((att + 7) // 8 * 8) * 2
     assert op.scheme(args, 2 ** 40) >= q_size + att_size
     assert op.scheme(args, q_size + att_size) == q_size + att_size
     assert op.scheme(args, q_size + att_size - 1) == q_size

@@ -252,7 +252,9 @@ def test_random_mat_mul_ragged_tile_shapes(gpu, stream, monkeypatch, sweep):
     clamped rows and store only what exists (guard zones around C catch a store past M or N).  Two thirds of the
     cases have M and N in multiples of 8 with every operand layout; the others an odd M with A and C row-major
     (nothing is contiguous along M then).  Some have few tiles and a long K (split K over ragged tiles).  Every
-    fourth case keeps the 256 x 256 tile, which the library would only choose for much larger outputs."""
+    fourth case keeps the 256 x 256 tile, which the library would only choose for much larger outputs.  Half of
+    the cases have a K that is no multiple of the kernel's K-step, some of them odd (rows along K are then
+    padded to whole groups of 8, which is what the kernel's 16-byte loads need)."""
     rng = np.random.default_rng(731 + 1000 * sweep)
     mm = ophip.MatMul(gpu)
     oracle.set_threads(8)
@@ -266,15 +268,19 @@ def test_random_mat_mul_ragged_tile_shapes(gpu, stream, monkeypatch, sweep):
                 monkeypatch.delenv("OPHIP_GEMM_TILE", raising=False)
             n = 8 * int(rng.integers(9, 90))
             m = 2 * int(rng.integers(33, 350)) + 1 if odd_m else 8 * int(rng.integers(9, 90))
-            k = int(rng.choice([64, 192, 1088, 2048]) if big else rng.choice([32, 64, 96, 192, 1056, 2048, 4096]))
+            if case % 2 == 0:
+                k = int(rng.choice([64, 192, 1088, 2048]) if big else rng.choice([32, 64, 96, 192, 1056, 2048, 4096]))
+            else:
+                k = int(rng.choice([72, 100, 136, 509, 1000, 2056, 4095]))
             bt = int(rng.choice([1, 1, 2]))
             ta, tb, tc = (bool(rng.integers(0, 2)) for _ in range(3))
             if odd_m:
                 ta = tc = False
-            pa, pb, pc = (int(rng.choice([0, 8])) for _ in range(3))
-            A = Guarded(gpu, rng, (bt, k, m) if ta else (bt, m, k), f16, pa, scale=0.25)
-            B = Guarded(gpu, rng, (bt, n, k) if tb else (bt, k, n), f16, pb, scale=0.25)
-            C = Guarded(gpu, rng, (bt, n, m) if tc else (bt, m, n), f16, pc)
+            sa, sb, sc = ((bt, k, m) if ta else (bt, m, k)), ((bt, n, k) if tb else (bt, k, n)), ((bt, n, m) if tc else (bt, m, n))
+            pa, pb, pc = ((-sh[-1]) % 8 + int(rng.choice([0, 8])) for sh in (sa, sb, sc))
+            A = Guarded(gpu, rng, sa, f16, pa, scale=0.25)
+            B = Guarded(gpu, rng, sb, f16, pb, scale=0.25)
+            C = Guarded(gpu, rng, sc, f16, pc)
             tr = lambda g, t: (TensorLayout(dt.F16, [g.shape[0], g.shape[2], g.shape[1]], [g.strides[0], g.strides[2], g.strides[1]]),
                                g.view().transpose(0, 2, 1)) if t else (g.layout, g.view())
             (al, av), (bl, bv), (cl, cv) = tr(A, ta), tr(B, tb), tr(C, tc)
