@@ -154,12 +154,12 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
     auto skinny_ok = [&]() {
         if (!f16 || p.M == 0 || p.M > 64 || p.K == 0) return false;
         if (p.p_sl != 1 || !mult8(p.p_si) || !mult8(p.p_sb) || !aligned16(p.p)) return false;
-        if (p.K % 8 != 0 || p.N % 8 != 0) return false;
+        if (p.N % 8 != 0) return false;
         if (!aligned16(p.q) || !mult8(p.q_sb)) return false;
-        if (p.q_sj == 1) {
+        if (p.q_sj == 1) {  // any K: the last K-step masks P element by element and Q by rows
             if (!mult8(p.q_sl)) return false;
         } else if (p.q_sl == 1) {
-            if (!mult8(p.q_sj)) return false;
+            if (p.K % 8 != 0 || !mult8(p.q_sj)) return false;
         } else {
             return false;
         }

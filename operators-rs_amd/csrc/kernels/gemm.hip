@@ -304,7 +304,14 @@ __device__ __forceinline__ void gemm_skinny(const GemmParams &p) {
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
                 abuf[0][mt] = u32x4{0, 0, 0, 0};
-                if (kb + 8 * g < kend) abuf[0][mt] = ld128(prow[mt] + kb);
+                if (kb + 8 * g + 8 <= kend) {
+                    abuf[0][mt] = ld128(prow[mt] + kb);
+                } else if (kb + 8 * g < kend) {  // K cuts this group of 8 (K % 8 != 0): element by element
+                    const uint16_t *h = reinterpret_cast<const uint16_t *>(prow[mt] + kb);
+#pragma unroll
+                    for (int e = 0; e < 7; ++e)
+                        if (kb + 8 * g + e < kend) abuf[0][mt][e / 2] |= (uint32_t)h[e] << (16 * (e & 1));
+                }
             }
             skinny_load_q_tail<QMODE>(p, qb, kb, kend, colc, g, wbuf[0]);
             step(wbuf[0], abuf[0]);

@@ -964,6 +964,24 @@ def test_mat_mul_prefill_with_any_token_count(gpu, stream, tokens, n, k, b_trans
         oracle.set_threads(1)
 
 
+@pytest.mark.parametrize("bt,m,n,k", [(32, 16, 128, 2047), (4, 16, 128, 301), (2, 40, 256, 1001), (1, 7, 64, 33)])
+def test_mat_mul_few_rows_with_any_k(gpu, stream, bt, m, n, k):
+    """The PV product of a decode step: a handful of score rows (padded to 16 bytes, as the attention operator
+    keeps them) times V[att, dh] for an att that is no multiple of 8.  Still the weight-streaming kernel: its
+    last K-step masks the scores element by element and V by rows."""
+    rng = np.random.default_rng(k)
+    ld = (k + 7) // 8 * 8
+    a = normal_f16(rng, (bt, m, ld), std=0.05)[:, :, :k]
+    b = normal_f16(rng, (bt, k, n), std=1.0)
+    c = np.zeros((bt, m, n), f16)
+    args = ophip.MatMulArgs(TensorLayout.of(c), None, 0.0, TensorLayout.of(a), None, TensorLayout.of(b), None, 1.0)
+    what = ophip.MatMul(gpu).describe(args)
+    say("mat_mul %d x [%d x %d x %d] [%s]" % (bt, m, n, k, what))
+    assert what.startswith("skinny"), what
+    out = run_mat_mul(gpu, stream, c, a, b, 1.0, 0.0)
+    check_mat_mul(out, c, a, b, 1.0, 0.0, "few rows, k = %d" % k)
+
+
 def test_mat_mul_beta_zero_never_reads_c_and_scalars_round_to_f16(gpu, stream):
     a = np.ones((16, 2048), f16)
     a[:, 2047] = 0  # 2047 ones per row
