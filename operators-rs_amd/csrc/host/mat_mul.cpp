@@ -169,6 +169,7 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
 
     // prefer the orientation whose row count is the small dimension
     const bool first_transposed = L.n <= L.m;
+    auto plan_skinny = [&]() {
     for (int attempt = 0; attempt < 2; ++attempt) {
         orient(attempt == 0 ? first_transposed : !first_transposed);
         if (skinny_ok()) {
@@ -207,9 +208,11 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
                 }
             }
             g.workspace = split > 1 ? split * p.batch * (size_t)p.M * p.N * sizeof(float) : 0;
-            return g;
+            return true;
         }
     }
+    return false;
+    };
     // Compute-bound shapes: the LDS-tiled MFMA kernel.  Of the two orientations take
     // the one whose epilogue can store several adjacent outputs per lane.
     // K-step of the tile kernels: 64, or 32 for a K in whole steps of 32 only; any other K from 64 on runs
@@ -231,8 +234,10 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
             if (st <= 0 || st >= lim) return false;
         return true;
     };
+    auto plan_tile = [&]() {
     for (uint32_t b : {256u, 128u}) {
         int best = -1;
+        bool best_splits = false;
         // Tiles for less than half the CUs (a CU holds one 256 tile or two 128 tiles): split K,
         // keeping at least 8 K-steps per workgroup; the f32 partials are summed by
         // gemm_splitk_reduce, which wants the orientation whose D is j-contiguous.
@@ -244,7 +249,6 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
                 split = std::min<size_t>({target / wgs, (size_t)8, std::max<size_t>(1, ksteps / 8)});
             if (const char *e = std::getenv("OPHIP_GEMM_TILE_SPLITK")) split = std::max(1, std::atoi(e));
             split = std::max<size_t>(1, std::min(split, ksteps));
-            if (L.m % 8 != 0 || L.n % 8 != 0) split = 1;  // gemm_splitk_reduce works on groups of 8 columns
         }
         for (int attempt = 0; attempt < 2; ++attempt) {
             orient(attempt == 1);
@@ -260,12 +264,18 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
                 const size_t t256 = (size_t)((p.M + 255) / 256) * ((p.N + 255) / 256), t128 = (size_t)((p.M + 127) / 128) * ((p.N + 127) / 128);
                 if (t256 * p.batch * 5 < (size_t)cus * 3 || t256 * 4 * 5 > t128 * 7) continue;
             }
-            const bool wide = split > 1 ? p.d_sj == 1 : (p.q_sl != 1 && p.d_sj == 1) || (p.p_sl == 1 && p.d_si == 1);
-            if (best < 0 || wide) best = attempt;
+            // (gemm_splitk_reduce works on groups of 8 columns: an orientation whose N is no multiple of 8 cannot split)
+            const bool can_split = split > 1 && p.N % 8 == 0;
+            const bool wide = split > 1 ? can_split && p.d_sj == 1 : (p.q_sl != 1 && p.d_sj == 1) || (p.p_sl == 1 && p.d_si == 1);
+            if (best < 0 || wide || (can_split && !best_splits)) {
+                best = attempt;
+                best_splits = can_split;
+            }
             if (wide) break;
         }
         if (best >= 0) {
             orient(best == 1);
+            if (!best_splits) split = 1;
             g.kind = GemmPlan::Tile;
             g.tile = (int)b;
             g.pk = p.p_sl == 1;
@@ -280,10 +290,19 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
                 p.split_k = (uint32_t)split;
                 g.workspace = split > 1 ? split * p.batch * (size_t)p.M * p.N * sizeof(float) : 0;
             }
-            return g;
+            return true;
         }
     }
-    orient(false);
+    return false;
+    };
+    // The streaming kernel slows down with its row count (every wave re-reads the rows of P for its K-steps
+    // and multiplies 16 of them at a time); cold-weight sweeps over the decode GEMMs of a 7B layer put the
+    // crossover to the 128 tile at 48 rows, at 32 for a weight of less than 64 MB (16 .. 64 rows against the
+    // tile kernel at 65: 4096 x 22016 37 / 43 / 46 / 49 against 45 us; 4096 x 4096 13 / 18 / 22 / 26 against 18 us).
+    const size_t rows = std::min(L.m, L.n), weight_bytes = (size_t)L.k * std::max(L.m, L.n) * 2;
+    const bool tile_first = L.batch == 1 && rows > (weight_bytes < ((size_t)64 << 20) ? 32u : 48u);
+    if (tile_first ? plan_tile() || plan_skinny() : plan_skinny() || plan_tile()) return g;
+    orient(false);  // neither planner touches the split fields unless it succeeds
     g.kind = GemmPlan::Generic;
     return g;
 }

@@ -812,7 +812,7 @@ def test_mat_mul_decode_layer_shapes(gpu, stream, name, bt, m, n, k, b_transpose
 
 
 @pytest.mark.parametrize("m,n,k,bt,beta", [(16, 12288, 4096, 1, 0.0), (16, 4096, 11008, 1, 0.5), (16, 4096, 4096, 1, 0.0),
-                                           (24, 1024, 2048, 2, 1.0), (40, 512, 1024, 1, 0.0), (64, 384, 512, 3, 0.5)])
+                                           (24, 1024, 2048, 2, 1.0), (40, 512, 1024, 2, 0.0), (64, 384, 512, 3, 0.5)])
 def test_mat_mul_weights_stored_n_by_k(gpu, stream, m, n, k, bt, beta):
     """Weights kept as [N, K] (K-contiguous, the layout of a PyTorch Linear): the weight-streaming kernel's
     mode that reads 256 contiguous bytes per column and transposes through LDS, for 16, 32 and 64-row blocks,
