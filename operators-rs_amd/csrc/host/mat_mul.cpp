@@ -170,53 +170,53 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
     // prefer the orientation whose row count is the small dimension
     const bool first_transposed = L.n <= L.m;
     auto plan_skinny = [&]() {
-    for (int attempt = 0; attempt < 2; ++attempt) {
-        orient(attempt == 0 ? first_transposed : !first_transposed);
-        if (skinny_ok()) {
-            g.kind = GemmPlan::Skinny;
-            g.mt = p.M <= 16 ? 1 : p.M <= 32 ? 2 : 4;
-            g.qmode = p.q_sj == 1 ? 0 : 1;
-            // The kernel is latency-bound per CU, so a CU that holds two workgroups takes
-            // twice as long as one that holds one: split K only as far as one workgroup
-            // per CU (rounding down), keeping at least 16 K-steps per workgroup (the in-kernel
-            // reduction of a split costs a few microseconds of tail).
-            const size_t ntiles = (p.N + 127) / 128, slabs = (p.K + 31) / 32;
-            const size_t base = ntiles * p.batch;
-            size_t split = std::max<size_t>(1, (size_t)cus / base);
-            split = std::min(split, std::max<size_t>(1, slabs / 16));
-            // Slightly more workgroups than CUs is the worst case (the CUs that hold two finish last, at twice
-            // the time): halving the workgroups evens the load out a little (measured on 16 x 4096 x 36864 and
-            // 40960: 71 -> 65 and 72 -> 68 us; from 1.5 workgroups per CU on, a split only costs).
-            if (base > (size_t)cus && base * 4 <= (size_t)cus * 5 && slabs >= 32) split = 2;
-            if (const char *e = std::getenv("OPHIP_GEMM_SPLITK")) split = std::max(1, std::atoi(e));
-            size_t sps = (slabs + split - 1) / split;  // K-steps per split
-            split = (slabs + sps - 1) / sps;
-            p.k_per_split = (uint32_t)(sps * 32);
-            p.split_k = (uint32_t)split;
-            // A long l-contiguous Q (a weight stored [N, K]): the mode that reads 256 contiguous bytes per
-            // column, in K-chunks of 128 dealt to the four waves; needs whole chunks and at least one per wave.
-            if (g.qmode == 1 && p.N % 128 == 0 && p.K % 128 == 0) {
-                // (cold-weight sweeps: at least 8 chunks per split, i.e. two per wave, or the split costs more than it hides)
-                const size_t chunks = p.K / 128;
-                if (!std::getenv("OPHIP_GEMM_SPLITK")) split = std::min(split, std::max<size_t>(1, chunks / 8));
-                const size_t cps = (chunks + split - 1) / split;  // chunks per split
-                if (cps >= 4) {
-                    g.qmode = 2;
-                    split = (chunks + cps - 1) / cps;
-                    p.k_per_split = (uint32_t)(cps * 128);
-                    p.split_k = (uint32_t)split;
+        for (int attempt = 0; attempt < 2; ++attempt) {
+            orient(attempt == 0 ? first_transposed : !first_transposed);
+            if (skinny_ok()) {
+                g.kind = GemmPlan::Skinny;
+                g.mt = p.M <= 16 ? 1 : p.M <= 32 ? 2 : 4;
+                g.qmode = p.q_sj == 1 ? 0 : 1;
+                // The kernel is latency-bound per CU, so a CU that holds two workgroups takes
+                // twice as long as one that holds one: split K only as far as one workgroup
+                // per CU (rounding down), keeping at least 16 K-steps per workgroup (the in-kernel
+                // reduction of a split costs a few microseconds of tail).
+                const size_t ntiles = (p.N + 127) / 128, slabs = (p.K + 31) / 32;
+                const size_t base = ntiles * p.batch;
+                size_t split = std::max<size_t>(1, (size_t)cus / base);
+                split = std::min(split, std::max<size_t>(1, slabs / 16));
+                // Slightly more workgroups than CUs is the worst case (the CUs that hold two finish last, at twice
+                // the time): halving the workgroups evens the load out a little (measured on 16 x 4096 x 36864 and
+                // 40960: 71 -> 65 and 72 -> 68 us; from 1.5 workgroups per CU on, a split only costs).
+                if (base > (size_t)cus && base * 4 <= (size_t)cus * 5 && slabs >= 32) split = 2;
+                if (const char *e = std::getenv("OPHIP_GEMM_SPLITK")) split = std::max(1, std::atoi(e));
+                size_t sps = (slabs + split - 1) / split;  // K-steps per split
+                split = (slabs + sps - 1) / sps;
+                p.k_per_split = (uint32_t)(sps * 32);
+                p.split_k = (uint32_t)split;
+                // A long l-contiguous Q (a weight stored [N, K]): the mode that reads 256 contiguous bytes per
+                // column, in K-chunks of 128 dealt to the four waves; needs whole chunks and at least one per wave.
+                if (g.qmode == 1 && p.N % 128 == 0 && p.K % 128 == 0) {
+                    // (cold-weight sweeps: at least 8 chunks per split, i.e. two per wave, or the split costs more than it hides)
+                    const size_t chunks = p.K / 128;
+                    if (!std::getenv("OPHIP_GEMM_SPLITK")) split = std::min(split, std::max<size_t>(1, chunks / 8));
+                    const size_t cps = (chunks + split - 1) / split;  // chunks per split
+                    if (cps >= 4) {
+                        g.qmode = 2;
+                        split = (chunks + cps - 1) / cps;
+                        p.k_per_split = (uint32_t)(cps * 128);
+                        p.split_k = (uint32_t)split;
+                    }
                 }
+                // N-contiguous weight, long K range in whole groups of 8 steps: the build that deals the steps to the
+                // waves in pairs and requests both halves of P's cache lines together (same box, cold weights,
+                // 16 / 32 rows: 4096 x 22016 37.0 -> 35.9 / 42.2 -> 39.1 us, 4096 x 12288 split 2 23.4 -> 22.6 / 27.5 -> 26.3;
+                // K = 4096 split 8 and 11008 split 8 lose 2 - 4 %, so they keep the plain dealing)
+                if (g.qmode == 0 && p.k_per_split % 256 == 0 && p.k_per_split >= 1024 && p.K % p.k_per_split == 0) g.qmode = 3;
+                g.workspace = split > 1 ? split * p.batch * (size_t)p.M * p.N * sizeof(float) : 0;
+                return true;
             }
-            // N-contiguous weight, long K range in whole groups of 8 steps: the build that deals the steps to the
-            // waves in pairs and requests both halves of P's cache lines together (same box, cold weights,
-            // 16 / 32 rows: 4096 x 22016 37.0 -> 35.9 / 42.2 -> 39.1 us, 4096 x 12288 split 2 23.4 -> 22.6 / 27.5 -> 26.3;
-            // K = 4096 split 8 and 11008 split 8 lose 2 - 4 %, so they keep the plain dealing)
-            if (g.qmode == 0 && p.k_per_split % 256 == 0 && p.k_per_split >= 1024 && p.K % p.k_per_split == 0) g.qmode = 3;
-            g.workspace = split > 1 ? split * p.batch * (size_t)p.M * p.N * sizeof(float) : 0;
-            return true;
         }
-    }
-    return false;
+        return false;
     };
     // Compute-bound shapes: the LDS-tiled MFMA kernel.  Of the two orientations take
     // the one whose epilogue can store several adjacent outputs per lane.
@@ -240,65 +240,67 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
         return true;
     };
     auto plan_tile = [&]() {
-    for (uint32_t b : {256u, 128u}) {
-        int best = -1;
-        bool best_splits = false;
-        // Tiles for less than half the CUs (a CU holds one 256 tile or two 128 tiles): split K,
-        // keeping at least 8 K-steps per workgroup; the f32 partials are summed by
-        // gemm_splitk_reduce, which wants the orientation whose D is j-contiguous.
-        size_t split = 1;
-        {
-            const size_t wgs = ((L.m + b - 1) / b) * ((L.n + b - 1) / b) * L.batch, target = b == 256 ? cus : 2 * (size_t)cus;
-            const size_t ksteps = tile_tk ? L.k / tile_tk : 1;
-            if (wgs > 0 && wgs * 2 <= cus)
-                split = std::min<size_t>({target / wgs, (size_t)8, std::max<size_t>(1, ksteps / 8)});
-            if (const char *e = std::getenv("OPHIP_GEMM_TILE_SPLITK")) split = std::max(1, std::atoi(e));
-            split = std::max<size_t>(1, std::min(split, ksteps));
-        }
-        for (int attempt = 0; attempt < 2; ++attempt) {
-            orient(attempt == 1);
-            if (!tile_ok(b)) continue;
-            // 256-tiles for less than 60 % of the CUs: the 128 pass is faster (measured on 512 .. 2048 row
-            // shapes: at half the CUs the large tile loses by 10 - 50 %, at two thirds it wins by 10 %)
-            // (OPHIP_GEMM_TILE=256 / 128 keeps one tile size, for tests and sweeps)
-            const char *force = std::getenv("OPHIP_GEMM_TILE");
-            if (force && (uint32_t)std::atoi(force) != b) continue;
-            // and when the part of the last tiles that lies outside the matrix costs more than the large tile's
-            // advantage (about 1.4 x per multiply at these sizes)
-            if (b == 256 && !force) {
-                const size_t t256 = (size_t)((p.M + 255) / 256) * ((p.N + 255) / 256), t128 = (size_t)((p.M + 127) / 128) * ((p.N + 127) / 128);
-                if (t256 * p.batch * 5 < (size_t)cus * 3 || t256 * 4 * 5 > t128 * 7) continue;
+        for (uint32_t b : {256u, 128u}) {
+            int best = -1;
+            bool best_splits = false;
+            // Tiles for less than half the CUs (a CU holds one 256 tile or two 128 tiles): split K,
+            // keeping at least 8 K-steps per workgroup; the f32 partials are summed by
+            // gemm_splitk_reduce, which wants the orientation whose D is j-contiguous.
+            size_t split = 1;
+            {
+                const size_t wgs = ((L.m + b - 1) / b) * ((L.n + b - 1) / b) * L.batch, target = b == 256 ? cus : 2 * (size_t)cus;
+                const size_t ksteps = tile_tk ? L.k / tile_tk : 1;
+                if (wgs > 0 && wgs * 2 <= cus)
+                    split = std::min<size_t>({target / wgs, (size_t)8, std::max<size_t>(1, ksteps / 8)});
+                if (const char *e = std::getenv("OPHIP_GEMM_TILE_SPLITK")) split = std::max(1, std::atoi(e));
+                split = std::max<size_t>(1, std::min(split, ksteps));
             }
-            // (gemm_splitk_reduce works on groups of 8 columns: an orientation whose N is no multiple of 8 cannot split)
-            const bool can_split = split > 1 && p.N % 8 == 0;
-            const bool wide = split > 1 ? can_split && p.d_sj == 1 : (p.q_sl != 1 && p.d_sj == 1) || (p.p_sl == 1 && p.d_si == 1);
-            if (best < 0 || wide || (can_split && !best_splits)) {
-                best = attempt;
-                best_splits = can_split;
+            for (int attempt = 0; attempt < 2; ++attempt) {
+                orient(attempt == 1);
+                if (!tile_ok(b)) continue;
+                // 256-tiles for less than 60 % of the CUs: the 128 pass is faster (measured on 512 .. 2048 row
+                // shapes: at half the CUs the large tile loses by 10 - 50 %, at two thirds it wins by 10 %)
+                // (OPHIP_GEMM_TILE=256 / 128 keeps one tile size, for tests and sweeps)
+                const char *force = std::getenv("OPHIP_GEMM_TILE");
+                if (force && (uint32_t)std::atoi(force) != b) continue;
+                // and when the part of the last tiles that lies outside the matrix costs more than the large tile's
+                // advantage (about 1.4 x per multiply at these sizes)
+                if (b == 256 && !force) {
+                    const size_t t256 = (size_t)((p.M + 255) / 256) * ((p.N + 255) / 256);
+                    const size_t t128 = (size_t)((p.M + 127) / 128) * ((p.N + 127) / 128);
+                    if (t256 * p.batch * 5 < (size_t)cus * 3 || t256 * 4 * 5 > t128 * 7) continue;
+                }
+                // (gemm_splitk_reduce works on groups of 8 columns: an orientation whose N is no multiple of 8 cannot split)
+                const bool can_split = split > 1 && p.N % 8 == 0;
+                const bool wide = split > 1 ? can_split && p.d_sj == 1
+                                            : (p.q_sl != 1 && p.d_sj == 1) || (p.p_sl == 1 && p.d_si == 1);
+                if (best < 0 || wide || (can_split && !best_splits)) {
+                    best = attempt;
+                    best_splits = can_split;
+                }
+                if (wide) break;
             }
-            if (wide) break;
-        }
-        if (best >= 0) {
-            orient(best == 1);
-            if (!best_splits) split = 1;
-            g.kind = GemmPlan::Tile;
-            g.tile = (int)b;
-            g.pk = p.p_sl == 1;
-            g.qk = p.q_sl == 1;
-            const size_t tk = tile_tk, ksteps = p.K / tk;
-            g.tk = (int)tk;
-            g.ragged = p.M % b != 0 || p.N % b != 0 || p.K % tk != 0;
-            if (split > 1) {
-                const size_t sps = (ksteps + split - 1) / split;
-                split = (ksteps + sps - 1) / sps;
-                p.k_per_split = (uint32_t)(sps * tk);
-                p.split_k = (uint32_t)split;
-                g.workspace = split > 1 ? split * p.batch * (size_t)p.M * p.N * sizeof(float) : 0;
+            if (best >= 0) {
+                orient(best == 1);
+                if (!best_splits) split = 1;
+                g.kind = GemmPlan::Tile;
+                g.tile = (int)b;
+                g.pk = p.p_sl == 1;
+                g.qk = p.q_sl == 1;
+                const size_t tk = tile_tk, ksteps = p.K / tk;
+                g.tk = (int)tk;
+                g.ragged = p.M % b != 0 || p.N % b != 0 || p.K % tk != 0;
+                if (split > 1) {
+                    const size_t sps = (ksteps + split - 1) / split;
+                    split = (ksteps + sps - 1) / sps;
+                    p.k_per_split = (uint32_t)(sps * tk);
+                    p.split_k = (uint32_t)split;
+                    g.workspace = split > 1 ? split * p.batch * (size_t)p.M * p.N * sizeof(float) : 0;
+                }
+                return true;
             }
-            return true;
         }
-    }
-    return false;
+        return false;
     };
     // The streaming kernel slows down with its row count (every wave re-reads the rows of P for its K-steps
     // and multiplies 16 of them at a time); cold-weight sweeps over the decode GEMMs of a 7B layer put the
@@ -344,7 +346,8 @@ struct ophip_mat_mul {
         static const int mts[3] = {1, 2, 4};
         for (int i = 0; i < 3; ++i)
             for (int q = 0; q < 4; ++q)
-                skinny[i][q] = d->kernel("gemm", ("gemm_skinny_m" + std::to_string(mts[i]) + "_q" + (q == 3 ? "0p" : std::to_string(q))).c_str());
+                skinny[i][q] = d->kernel(
+                    "gemm", ("gemm_skinny_m" + std::to_string(mts[i]) + "_q" + (q == 3 ? "0p" : std::to_string(q))).c_str());
         for (int b = 0; b < 3; ++b)
             for (int r = 0; r < 2; ++r)
                 for (int pk = 0; pk < 2; ++pk)
@@ -403,7 +406,8 @@ int ophip_mat_mul_describe(const ophip_mat_mul *op, const ophip_mat_mul_args *ar
         if (L.dt != OPHIP_DT_F16 && L.dt != OPHIP_DT_F32) throw type_not_support("mat_mul supports f16 and f32");
         const GemmPlan g = make_plan(*args, L, (unsigned)op->dev->props.multiProcessorCount);
         if (g.kind == GemmPlan::Skinny)
-            std::snprintf(out, len, "skinny rows<=%d q%s split_k=%u", 16 * g.mt, g.qmode == 0 ? "N" : g.qmode == 1 ? "K" : g.qmode == 2 ? "K256" : "N paired",
+            std::snprintf(out, len, "skinny rows<=%d q%s split_k=%u", 16 * g.mt,
+                          g.qmode == 0 ? "N" : g.qmode == 1 ? "K" : g.qmode == 2 ? "K256" : "N paired",
                           g.p.split_k);
         else if (g.kind == GemmPlan::Tile)
             std::snprintf(out, len, "tile%dx%d%s p%s q%s split_k=%u", g.tile, g.tk,
