@@ -391,7 +391,8 @@ OPHIP_API int ophip_mat_mul_launch(const ophip_mat_mul *op, const ophip_mat_mul_
                                    const ophip_queue_alloc *queue_alloc);
 OPHIP_API void ophip_mat_mul_destroy(ophip_mat_mul *op);
 /* Diagnostics, no counterpart in the reference: writes the name of the kernel family launch()
- * would pick for these arguments on this device ("skinny rows<=16 qN split_k=2", "tile256x64 pK qN split_k=1",
+ * would pick for these arguments on this device ("skinny rows<=16 qN split_k=8", "skinny rows<=16 qN paired split_k=1",
+ * "skinny rows<=32 qK256 split_k=2", "tile256x64 pK qN split_k=1",
  * "tile128x64 ragged pK qK split_k=1" when M or N is not in whole tiles, "tile128x32 ...", "generic") into out[0..len). */
 OPHIP_API int ophip_mat_mul_describe(const ophip_mat_mul *op, const ophip_mat_mul_args *args, char *out, size_t len);
 
