@@ -298,25 +298,29 @@ def standalone_ops(ophip, gpu, stream, rng, reps):
         us = time_launches(gpu, stream, lambda: sw.launch(a, None, stream), reps)
         add("swiglu", "[%d,%d]" % (n, DI), 3 * n * DI * 2, us)
         gu.free()
-    # random_sample: 16 rows x [32000], one launch per row as the API prescribes
+    # random_sample: 16 rows x [32000], one launch per row as the API prescribes; then a vocabulary of today's
+    # models, which a workgroup cannot keep in its registers
     rs = o.RandomSample(gpu)
-    logits = gpu.from_host(normal_f16(rng, (16, 32000), np.sqrt(3.0)))
-    kv = gpu.malloc(16 * 8)
-    for mode, cfg, seed in (("argmax", o.SampleArgs.argmax(), 0.0), ("top-k 50 / top-p 0.9", o.SampleArgs(0.8, 0.9, 50), 0.37)):
-        arg_rows = []
-        for r in range(16):
-            a = o.RandomSampleArgs.layout(F16, 32000)
-            a.kv_pair_base, a.logits_base, a.config, a.seed = kv.ptr + 8 * r, logits.ptr + r * 64000, cfg, seed
-            arg_rows.append(a)
+    for vocab in (32000, 128256):
+        logits = gpu.from_host(normal_f16(rng, (16, vocab), np.sqrt(3.0)))
+        kv = gpu.malloc(16 * 8)
+        shape = "16 x [%d]" % vocab
+        for mode, cfg, seed in (("argmax", o.SampleArgs.argmax(), 0.0), ("top-k 50 / top-p 0.9", o.SampleArgs(0.8, 0.9, 50), 0.37)):
+            arg_rows = []
+            for r in range(16):
+                a = o.RandomSampleArgs.layout(F16, vocab)
+                a.kv_pair_base, a.logits_base, a.config, a.seed = kv.ptr + 8 * r, logits.ptr + r * vocab * 2, cfg, seed
+                arg_rows.append(a)
 
-        def run16():
-            for a in arg_rows:
-                rs.launch(a, None, stream)
-        us = time_launches(gpu, stream, run16, max(reps // 4, 5))
-        add("random_sample " + mode, "16 x [32000]", 16 * (32000 * 2 + 8), us, note="16 launches")
-        b = arg_rows[0]
-        us = time_launches(gpu, stream, lambda: rs.launch_batch(b, 16, 64000, None, None, stream), reps)
-        add("random_sample " + mode, "16 x [32000]", 16 * (32000 * 2 + 8), us, note="1 batched launch (extension)")
+            def run16():
+                for a in arg_rows:
+                    rs.launch(a, None, stream)
+            us = time_launches(gpu, stream, run16, max(reps // 4, 5))
+            add("random_sample " + mode, shape, 16 * (vocab * 2 + 8), us, note="16 launches")
+            b = arg_rows[0]
+            us = time_launches(gpu, stream, lambda: rs.launch_batch(b, 16, vocab * 2, None, None, stream), reps)
+            add("random_sample " + mode, shape, 16 * (vocab * 2 + 8), us, note="1 batched launch (extension)")
+        logits.free(); kv.free()
     # the remaining single-device operators, small and out-of-cache
     ln = o.LayerNorm(gpu)
     for n in (64, 65536):

@@ -20,6 +20,9 @@
 //      order, each term being exp() evaluated in f64 and rounded once to f32, so
 //      cum[0..k) follows the sequential definition; the sum over all n entries
 //      (needed for top_p) is a parallel f32 reduction in a fixed order.
+// sampling, top_k <= 1024, rows that do not fit the registers (`sample_topk_list`): after the first digit the
+// elements that can still matter (the chosen bucket and everything above it) are copied to a short list in
+// LDS, in the same sweep that sums the exponentials of the whole row; the rest runs on the list.
 // sampling, any top_k (`sample_full`): full bitonic sort in a global workspace,
 // then the same sequential scan over all n entries.
 #include "device_util.h"
@@ -476,6 +479,225 @@ __device__ __forceinline__ void sample_topk_impl(const SampleParams &p) {
 
 extern "C" __global__ void __launch_bounds__(SB) sample_topk_f16(SampleParams p) { sample_topk_impl<f16>(p); }
 extern "C" __global__ void __launch_bounds__(SB) sample_topk_f32(SampleParams p) { sample_topk_impl<float>(p); }
+
+constexpr uint32_t LIST_CAP = 2048;  // entries of the short list a row is cut down to after the first digit
+
+// sample_topk for a row that does not fit the registers (more than 32768 logits, or not 16-byte aligned): every
+// sweep reads it from memory at one CU's pace, so the row is cut down to a short list in LDS as early as possible.
+// (For a row held in registers building the list costs more than the sweeps it saves: that case keeps
+// sample_topk_impl above.)
+template <typename T>
+__device__ __forceinline__ void sample_topk_list_impl(const SampleParams &p) {
+    typedef Logit<T> L;
+    const char *row = reinterpret_cast<const char *>(p.logits) + (int64_t)blockIdx.x * p.row_stride;
+    const uint32_t n = p.n;
+    auto sweep_row = [&](auto &&f) { for_each_logit<T>(row, n, f); };  // f(index, raw bits) for every element
+    __shared__ uint32_t hist[256];
+    __shared__ uint32_t hist_w[SB / WAVE][256];  // one histogram per wave: 16x less contention on hot bins
+    __shared__ uint32_t s_wtot[4];
+    __shared__ uint32_t s_sel[2];
+    __shared__ uint32_t s_cnt;
+    __shared__ uint64_t cand[SB];
+    __shared__ uint64_t list[LIST_CAP];
+    __shared__ float s_cum[SB];
+    __shared__ float s_red[SB / WAVE];
+    __shared__ uint32_t s_kmax[SB / WAVE];
+    const uint32_t k = p.k_eff;
+    const float t = p.temperature, inv_t = 1.0f / t;
+
+    // 1a. k-th largest key, one 8-bit digit per sweep.  The first sweep also finds the largest key (the
+    // maximum every exponent is taken against).  If few enough elements share the first digit of the
+    // k-th key or lie above it, a second sweep copies them to a short list in LDS, summing the
+    // exponentials of the whole row on the way, and every later sweep runs over that list: two passes
+    // over the row instead of five or more, which is what a row too long for registers pays for.
+    uint32_t prefix = 0, krem = k, eq_count = 0, nlist = 0;
+    bool use_list = false;  // workgroup-uniform
+    float total = 0.f, mx = 0.f;
+    // f(index, key) for every element still in play
+    auto each = [&](auto &&f) {
+        if (use_list) {
+            for (uint32_t e = threadIdx.x; e < nlist; e += SB) {
+                const uint64_t c = list[e];
+                f(comp_idx(c), comp_key(c));
+            }
+        } else {
+            sweep_row([&](uint32_t i, uint32_t bits) { f(i, L::key(bits)); });
+        }
+    };
+    for (int shift = L::KEY_BITS - 8; shift >= 0; shift -= 8) {
+        for (uint32_t i = threadIdx.x; i < (SB / WAVE) * 256; i += SB) (&hist_w[0][0])[i] = 0;
+        __syncthreads();
+        const bool first = shift == L::KEY_BITS - 8;
+        const uint32_t hi_mask = first ? 0u : (0xffffffffu << (shift + 8));
+        uint32_t *my_hist = hist_w[threadIdx.x / WAVE];
+        uint32_t kmax = 0;
+        each([&](uint32_t, uint32_t key) {
+            if (first) kmax = max(kmax, key);
+            if (((key ^ prefix) & hi_mask) == 0) atomicAdd(&my_hist[(key >> shift) & 255u], 1u);
+        });
+        if (first) {
+#pragma unroll
+            for (int o = WAVE / 2; o > 0; o >>= 1) kmax = max(kmax, (uint32_t)__shfl_xor((int)kmax, o, WAVE));
+            if (threadIdx.x % WAVE == 0) s_kmax[threadIdx.x / WAVE] = kmax;
+        }
+        __syncthreads();
+        if (threadIdx.x < 256) {
+            uint32_t c = 0;
+#pragma unroll
+            for (int w = 0; w < SB / WAVE; ++w) c += hist_w[w][threadIdx.x];
+            hist[threadIdx.x] = c;
+        }
+        __syncthreads();
+        pick_bucket(hist, krem, true, s_wtot, s_sel);
+        const uint32_t above = krem - s_sel[1];  // elements in the buckets above the chosen one
+        prefix |= s_sel[0] << shift;
+        krem = s_sel[1];
+        eq_count = hist[s_sel[0]];
+        if (first) {
+            uint32_t km = 0;
+#pragma unroll
+            for (int w = 0; w < SB / WAVE; ++w) km = max(km, s_kmax[w]);
+            mx = L::value(L::unkey(km));
+            // the chosen bucket and everything above it: `above + eq_count` elements
+            if (above + eq_count <= LIST_CAP) {
+                if (threadIdx.x == 0) s_cnt = 0;
+                __syncthreads();
+                const uint32_t floor_digit = s_sel[0];
+                float part = 0.f;
+                // (the total only feeds the top_p bound: hardware exp2 and a reciprocal keep this sweep cheap)
+                sweep_row([&](uint32_t i, uint32_t bits) {
+                    part += fast_exp((L::value(bits) - mx) * inv_t);
+                    const uint32_t key = L::key(bits);
+                    if ((key >> shift) >= floor_digit) list[atomicAdd(&s_cnt, 1u)] = composite(key, i);
+                });
+                total = block_sum_f32(part, s_red);
+                __syncthreads();
+                nlist = s_cnt;
+                use_list = true;  // (the elements above the chosen bucket are in the list for the gather step)
+            }
+        }
+        __syncthreads();
+    }
+    const uint32_t kstar = prefix;  // k-th largest key; `krem` of the `eq_count` ties are wanted
+
+    // 1b. among the ties, the krem-th smallest index
+    uint32_t istar = 0xffffffffu;
+    if (eq_count > krem) {  // uniform branch
+        uint32_t ipre = 0, irem = krem;
+        for (int shift = 24; shift >= 0; shift -= 8) {
+            if (threadIdx.x < 256) hist[threadIdx.x] = 0;
+            __syncthreads();
+            const uint32_t hi_mask = shift == 24 ? 0u : (0xffffffffu << (shift + 8));
+            each([&](uint32_t i, uint32_t key) {
+                if (key == kstar && ((i ^ ipre) & hi_mask) == 0) atomicAdd(&hist[(i >> shift) & 255u], 1u);
+            });
+            __syncthreads();
+            pick_bucket(hist, irem, false, s_wtot, s_sel);
+            ipre |= s_sel[0] << shift;
+            irem = s_sel[1];
+            __syncthreads();
+        }
+        istar = ipre;
+    }
+
+    // 2. gather exactly k candidates, pad to a power of two
+    uint32_t P = 64;
+    while (P < k) P <<= 1;
+    if (threadIdx.x == 0) s_cnt = 0;
+    for (uint32_t i = threadIdx.x; i < P; i += SB) cand[i] = 0;
+    __syncthreads();
+    each([&](uint32_t i, uint32_t key) {
+        if (key > kstar || (key == kstar && i <= istar)) {
+            const uint32_t slot = atomicAdd(&s_cnt, 1u);
+            if (slot < SB) cand[slot] = composite(key, i);
+        }
+    });
+    __syncthreads();
+    if (!use_list) {  // the sweep the short-list path has already made
+        float part = 0.f;
+        sweep_row([&](uint32_t, uint32_t bits) { part += fast_exp((L::value(bits) - mx) * inv_t); });
+        total = block_sum_f32(part, s_red);
+    }
+
+    if (P == 64) {
+        // k <= 64: sort, prefix and search live in the registers of wave 0
+        const uint32_t lane = threadIdx.x % WAVE;
+        uint64_t x = 0;
+        if (threadIdx.x < WAVE) {
+            x = cand[lane];
+#pragma unroll
+            for (int k2 = 2; k2 <= WAVE; k2 <<= 1)
+#pragma unroll
+                for (int j = k2 >> 1; j > 0; j >>= 1) {
+                    const uint64_t y = shfl_xor_u64(x, j);
+                    const bool desc = (lane & k2) == 0, lower = (lane & j) == 0;
+                    x = (lower == desc) ? (x > y ? x : y) : (x < y ? x : y);
+                }
+        }
+        if (threadIdx.x < WAVE) {
+            float e = 0.f;
+            if (lane > 0 && lane < k) e = exp_cr((L::value(L::unkey(comp_key(x))) - mx) / t);
+            // cum[i] = cum[i-1] + e[i], strictly in order, every lane replaying the same chain
+            float c = 1.0f, mine = 1.0f;
+#pragma unroll
+            for (int i = 1; i < WAVE; ++i) {
+                c = c + __shfl(e, i, WAVE);
+                if (lane == (uint32_t)i) mine = c;
+            }
+            const float pk = c;  // terms past k are zero, so the chain ends at cum[k-1]
+            const float plimit = row_seed(p) * fminf(pk, total * p.top_p);
+            const uint64_t hit = __ballot(lane < k && mine >= plimit);
+            const uint32_t ans = hit ? (uint32_t)__ffsll((long long)hit) - 1 : k - 1;
+            if (lane == ans) {
+                KvPair *out = reinterpret_cast<KvPair *>(p.kv) + blockIdx.x;
+                out->idx = comp_idx(x);
+                out->val = L::from_f32(mine);
+            }
+        }
+        return;
+    }
+
+    bitonic_lds(cand, P, 2, P, P, 0);
+    // 3. running sums
+    if (threadIdx.x < P)
+        s_cum[threadIdx.x] = threadIdx.x == 0   ? 1.0f
+                             : threadIdx.x < k ? exp_cr((L::value(L::unkey(comp_key(cand[threadIdx.x]))) - mx) / t)
+                                               : 0.f;
+    __syncthreads();
+    if (threadIdx.x < WAVE) {
+        // wave 0 replays the sequential sum 64 entries at a time, carrying the running value
+        const uint32_t lane = threadIdx.x;
+        float c = 0.f;
+        for (uint32_t base = 0; base < P; base += WAVE) {
+            const float e = s_cum[base + lane];
+            float mine = 0.f;
+#pragma unroll
+            for (int i = 0; i < WAVE; ++i) {
+                c = c + __shfl(e, i, WAVE);
+                if (lane == (uint32_t)i) mine = c;
+            }
+            s_cum[base + lane] = mine;
+        }
+        const float pk = c;  // entries past k add zero
+        const float plimit = row_seed(p) * fminf(pk, total * p.top_p);
+        uint32_t ans = k - 1;
+        for (uint32_t base = 0; base < P; base += WAVE) {
+            const uint64_t hit = __ballot(base + lane < k && s_cum[base + lane] >= plimit);
+            if (hit) {
+                ans = base + (uint32_t)__ffsll((long long)hit) - 1;
+                break;
+            }
+        }
+        if (lane == 0) {
+            KvPair *out = reinterpret_cast<KvPair *>(p.kv) + blockIdx.x;
+            out->idx = comp_idx(cand[ans]);
+            out->val = L::from_f32(s_cum[ans]);
+        }
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(SB) sample_topk_list_f16(SampleParams p) { sample_topk_list_impl<f16>(p); }
+extern "C" __global__ void __launch_bounds__(SB) sample_topk_list_f32(SampleParams p) { sample_topk_list_impl<float>(p); }
 
 // Full sort.  Workspace per row: npow2 u64 sort keys, then n f32 running sums.
 constexpr uint32_t TILE = 2048;  // u64 entries sorted per LDS tile (16 KB)

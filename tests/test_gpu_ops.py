@@ -658,6 +658,44 @@ def test_random_sample_randomised_against_oracle(gpu, stream, dtype):
     assert agree >= 58
 
 
+@pytest.mark.parametrize("dtype", [f16, f32])
+def test_random_sample_long_and_misaligned_rows(gpu, stream, dtype):
+    """Rows that do not fit the workgroup's registers (more than 32768 logits, or not on a 16-byte boundary) go
+    through the short-list kernel: vocabularies of today's models, with smooth logits (few candidates after the
+    first radix digit), with logits rounded to a few levels (ties at the k-th value; the candidates overflow the
+    list and the kernel falls back to sweeping the row), and a short row that starts 2 or 4 bytes off."""
+    rng = np.random.default_rng(11)
+    op = ophip.RandomSample(gpu)
+    agree = trials = 0
+    for n, off in [(40000, 0), (50257, 0), (128256, 0), (151936, 0), (32000, 1), (5000, 1), (70001, 1)]:
+        for rounded in (False, True):
+            x = (rng.standard_normal(n + off) * rng.choice([1.7, 4.0])).astype(f32).astype(dtype)
+            if rounded:
+                x = np.round(x).astype(dtype)
+            for top_k in (50, 200, 1024):
+                t, top_p, seed = float(rng.uniform(0.3, 2.0)), float(rng.uniform(0.05, 1.0)), float(rng.uniform(0, 1))
+                say("long row n=%d off=%d rounded=%d k=%d t=%.3f p=%.3f seed=%.4f" % (n, off, rounded, top_k, t, top_p, seed))
+                ld = gpu.from_host(x)
+                kvd = gpu.from_host(np.array([0xFFFFFFFF, 0xFFFFFFFF], np.uint32))
+                args = ophip.RandomSampleArgs.layout(ophip.NP_DT[np.dtype(dtype)], n)
+                args.kv_pair_base, args.logits_base = kvd, ld.ptr + off * x.itemsize
+                args.config, args.seed = ophip.SampleArgs(t, top_p, top_k), seed
+                op.launch(args, None, stream)
+                kv = gpu.to_host(kvd, np.uint32, 2, stream=stream)
+                idx, val = int(kv[0]), int(kv[1])
+                row = x[off:]
+                ridx, rval = oracle.random_sample(row, t, top_p, top_k, seed)
+                lo = oracle.random_sample(row, t, top_p, top_k, seed * (1 - 1e-5))[0]
+                hi = oracle.random_sample(row, t, top_p, top_k, min(seed * (1 + 1e-5), 1.0))[0]
+                assert idx in (ridx, lo, hi), (idx, ridx, lo, hi)
+                trials += 1
+                if idx == ridx:
+                    agree += 1
+                    rv = val_of(rval, dtype)
+                    assert abs(val_of(val, dtype) - rv) <= 2e-3 + 1e-2 * abs(rv)
+    assert agree >= trials - 2
+
+
 def test_random_sample_all_equal_and_edge_draws(gpu, stream):
     op = ophip.RandomSample(gpu)
     x = np.full(5000, 1.25, f16)  # the k-th value is tied 5000 ways: indices 0..k-1 are the candidates
