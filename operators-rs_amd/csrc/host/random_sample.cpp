@@ -41,13 +41,15 @@ size_t full_sort_workspace(size_t n) { return next_pow2(n) * 8 + ((n * 4 + 15) &
 
 struct ophip_random_sample {
     ophip_device *dev;
-    hipFunction_t argmax[2], topk[2], topk_list[2], full[2];  // [0] f16, [1] f32
+    hipFunction_t argmax[2], topk_k64[2], topk[2], topk_list[2], full[2];  // [0] f16, [1] f32
     explicit ophip_random_sample(ophip_device *d) : dev(d) {
         ophip_device_retain(d);
         argmax[0] = d->kernel("random_sample", "argmax_f16");
         argmax[1] = d->kernel("random_sample", "argmax_f32");
         topk[0] = d->kernel("random_sample", "sample_topk_f16");
         topk[1] = d->kernel("random_sample", "sample_topk_f32");
+        topk_k64[0] = d->kernel("random_sample", "sample_topk_k64_f16");
+        topk_k64[1] = d->kernel("random_sample", "sample_topk_k64_f32");
         topk_list[0] = d->kernel("random_sample", "sample_topk_list_f16");
         topk_list[1] = d->kernel("random_sample", "sample_topk_list_f32");
         full[0] = d->kernel("random_sample", "sample_full_f16");
@@ -134,7 +136,8 @@ static void sample_launch(const ophip_random_sample *op, const ophip_random_samp
         // rows of up to 32768 logits on 16-byte boundaries stay in the workgroup's registers; longer ones are
         // cut down to a short list in LDS after the first radix digit
         const bool in_registers = n <= 32768 && aligned16(p.logits) && (rows == 1 || row_stride % 16 == 0);
-        launch(in_registers ? op->topk[ti] : op->topk_list[ti], grid, Dim3{1024}, 0, stream_of(qa), p);
+        // (top_k <= 64, the common case, has a kernel of its own among the register-row ones)
+        launch(!in_registers ? op->topk_list[ti] : k_eff <= 64 ? op->topk_k64[ti] : op->topk[ti], grid, Dim3{1024}, 0, stream_of(qa), p);
         return;
     }
     p.npow2 = (uint32_t)next_pow2(n);

@@ -305,7 +305,74 @@ __device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t v, int m) {
     return ((uint64_t)hi << 32) | lo;
 }
 
-template <typename T>
+// Among the elements whose key is `kstar` (there are eq_count of them), the index of the krem-th smallest
+// (krem >= 1), written to *out.  each(f) calls f(index, key) for every element in play.  The tied indices
+// are collected in `scratch` (LDS, room for SB of them) in one sweep and ranked by counting: ties at the k-th
+// value are common with f16 logits and larger k, and are nearly always a handful.  Returns false, with nothing
+// done, when there are more than SB of them: the caller then selects digit by digit.
+template <typename Each>
+__device__ __forceinline__ bool kth_tied_index(Each &&each, uint32_t kstar, uint32_t krem, uint32_t eq_count,
+                                               uint32_t *scratch, uint32_t *counter, uint32_t *out) {
+    if (eq_count > SB) return false;  // workgroup-uniform
+    if (threadIdx.x == 0) *counter = 0;
+    __syncthreads();
+    each([&](uint32_t i, uint32_t key) {
+        if (key == kstar) scratch[atomicAdd(counter, 1u)] = i;
+    });
+    __syncthreads();
+    if (threadIdx.x < eq_count) {
+        const uint32_t mine = scratch[threadIdx.x];
+        uint32_t smaller = 0;
+        for (uint32_t u = 0; u < eq_count; ++u) smaller += scratch[u] < mine ? 1u : 0u;
+        if (smaller == krem - 1) *out = mine;
+    }
+    __syncthreads();
+    return true;
+}
+
+// Descending sort of `cnt` <= 256 (a power of two, >= 64) u64 values in LDS by wave 0 alone: four values per
+// lane in registers, exchanges inside a lane or by shuffle, no barrier per stage (the LDS network above
+// spends most of its time in its 36 barriers at this size).  All threads call; the result is in `a` after return.
+__device__ __forceinline__ void sort_desc_256(uint64_t *a, uint32_t cnt) {
+    if (threadIdx.x < WAVE) {
+        const uint32_t lane = threadIdx.x;
+        uint64_t x[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) x[r] = lane * 4 + r < cnt ? a[lane * 4 + r] : 0;  // zeros sort to the end
+#pragma unroll
+        for (int k2 = 2; k2 <= 256; k2 <<= 1)
+#pragma unroll
+            for (int j = k2 >> 1; j > 0; j >>= 1) {
+                if (j >= 4) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const uint32_t i = lane * 4 + r;
+                        const uint64_t y = shfl_xor_u64(x[r], j / 4);
+                        const bool desc = (i & k2) == 0, lower = (i & j) == 0;
+                        x[r] = (lower == desc) ? (x[r] > y ? x[r] : y) : (x[r] < y ? x[r] : y);
+                    }
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        if ((r & j) != 0) continue;  // r is the lower of the pair (r, r + j)
+                        const uint32_t i = lane * 4 + r;
+                        const bool desc = (i & k2) == 0;
+                        const uint64_t lo = x[r] < x[r + j] ? x[r] : x[r + j], hi = x[r] < x[r + j] ? x[r + j] : x[r];
+                        x[r] = desc ? hi : lo;
+                        x[r + j] = desc ? lo : hi;
+                    }
+                }
+            }
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            if (lane * 4 + r < cnt) a[lane * 4 + r] = x[r];
+    }
+    __syncthreads();
+}
+
+// SMALLK: top_k <= 64, the common case (sort, prefix and search in the registers of wave 0) as a kernel of its own:
+// it is short, and the code of the general case beside it cost it 3 % even unexecuted.
+template <typename T, bool SMALLK>
 __device__ __forceinline__ void sample_topk_impl(const SampleParams &p) {
     typedef Logit<T> L;
     __shared__ uint32_t hist[256];
@@ -353,7 +420,16 @@ __device__ __forceinline__ void sample_topk_impl(const SampleParams &p) {
 
     // 1b. among the ties, the krem-th smallest index
     uint32_t istar = 0xffffffffu;
-    if (eq_count > krem) {  // uniform branch
+    bool ranked = false;
+    if constexpr (!SMALLK) {
+        if (eq_count > krem) {
+            ranked = kth_tied_index([&](auto &&f) { rc.for_each(row, n, [&](uint32_t i, uint32_t bits) { f(i, L::key(bits)); }); },
+                                    kstar, krem, eq_count, reinterpret_cast<uint32_t *>(cand), &s_cnt, &s_sel[0]);
+            if (ranked) istar = s_sel[0];
+            __syncthreads();
+        }
+    }
+    if (eq_count > krem && !ranked) {  // uniform branch
         uint32_t ipre = 0, irem = krem;
         for (int shift = 24; shift >= 0; shift -= 8) {
             if (threadIdx.x < 256) hist[threadIdx.x] = 0;
@@ -373,7 +449,8 @@ __device__ __forceinline__ void sample_topk_impl(const SampleParams &p) {
 
     // 2. gather exactly k candidates, pad to a power of two
     uint32_t P = 64;
-    while (P < k) P <<= 1;
+    if constexpr (!SMALLK)
+        while (P < k) P <<= 1;
     if (threadIdx.x == 0) s_cnt = 0;
     for (uint32_t i = threadIdx.x; i < P; i += SB) cand[i] = 0;
     __syncthreads();
@@ -387,7 +464,7 @@ __device__ __forceinline__ void sample_topk_impl(const SampleParams &p) {
     __syncthreads();
 
     const float t = p.temperature;
-    if (P == 64) {
+    if (SMALLK || P == 64) {
         // k <= 64: sort, prefix and search live in the registers of wave 0
         const uint32_t lane = threadIdx.x % WAVE;
         uint64_t x = 0;
@@ -433,52 +510,57 @@ __device__ __forceinline__ void sample_topk_impl(const SampleParams &p) {
         return;
     }
 
-    bitonic_lds(cand, P, 2, P, P, 0);
-    // 3. running sums
-    const float mx = L::value(L::unkey(comp_key(cand[0])));
-    float part = 0.f;
-    const float inv_t = 1.0f / t;
-    rc.for_each(row, n, [&](uint32_t, uint32_t bits) { part += fast_exp((L::value(bits) - mx) * inv_t); });
-    const float total = block_sum_f32(part, s_red);
-    if (threadIdx.x < P)
-        s_cum[threadIdx.x] = threadIdx.x == 0   ? 1.0f
-                             : threadIdx.x < k ? exp_cr((L::value(L::unkey(comp_key(cand[threadIdx.x]))) - mx) / t)
-                                               : 0.f;
-    __syncthreads();
-    if (threadIdx.x < WAVE) {
-        // wave 0 replays the sequential sum 64 entries at a time, carrying the running value
-        const uint32_t lane = threadIdx.x;
-        float c = 0.f;
-        for (uint32_t base = 0; base < P; base += WAVE) {
-            const float e = s_cum[base + lane];
-            float mine = 0.f;
-#pragma unroll
-            for (int i = 0; i < WAVE; ++i) {
-                c = c + __shfl(e, i, WAVE);
-                if (lane == (uint32_t)i) mine = c;
+    if constexpr (!SMALLK) {
+        if (P <= 256) sort_desc_256(cand, P);
+        else bitonic_lds(cand, P, 2, P, P, 0);
+        // 3. running sums
+        const float mx = L::value(L::unkey(comp_key(cand[0])));
+        float part = 0.f;
+        const float inv_t = 1.0f / t;
+        rc.for_each(row, n, [&](uint32_t, uint32_t bits) { part += fast_exp((L::value(bits) - mx) * inv_t); });
+        const float total = block_sum_f32(part, s_red);
+        if (threadIdx.x < P)
+            s_cum[threadIdx.x] = threadIdx.x == 0   ? 1.0f
+                                 : threadIdx.x < k ? exp_cr((L::value(L::unkey(comp_key(cand[threadIdx.x]))) - mx) / t)
+                                                   : 0.f;
+        __syncthreads();
+        if (threadIdx.x < WAVE) {
+            // wave 0 replays the sequential sum 64 entries at a time, carrying the running value
+            const uint32_t lane = threadIdx.x;
+            float c = 0.f;
+            for (uint32_t base = 0; base < P; base += WAVE) {
+                const float e = s_cum[base + lane];
+                float mine = 0.f;
+    #pragma unroll
+                for (int i = 0; i < WAVE; ++i) {
+                    c = c + __shfl(e, i, WAVE);
+                    if (lane == (uint32_t)i) mine = c;
+                }
+                s_cum[base + lane] = mine;
             }
-            s_cum[base + lane] = mine;
-        }
-        const float pk = c;  // entries past k add zero
-        const float plimit = row_seed(p) * fminf(pk, total * p.top_p);
-        uint32_t ans = k - 1;
-        for (uint32_t base = 0; base < P; base += WAVE) {
-            const uint64_t hit = __ballot(base + lane < k && s_cum[base + lane] >= plimit);
-            if (hit) {
-                ans = base + (uint32_t)__ffsll((long long)hit) - 1;
-                break;
+            const float pk = c;  // entries past k add zero
+            const float plimit = row_seed(p) * fminf(pk, total * p.top_p);
+            uint32_t ans = k - 1;
+            for (uint32_t base = 0; base < P; base += WAVE) {
+                const uint64_t hit = __ballot(base + lane < k && s_cum[base + lane] >= plimit);
+                if (hit) {
+                    ans = base + (uint32_t)__ffsll((long long)hit) - 1;
+                    break;
+                }
             }
-        }
-        if (lane == 0) {
-            KvPair *out = reinterpret_cast<KvPair *>(p.kv) + blockIdx.x;
-            out->idx = comp_idx(cand[ans]);
-            out->val = L::from_f32(s_cum[ans]);
+            if (lane == 0) {
+                KvPair *out = reinterpret_cast<KvPair *>(p.kv) + blockIdx.x;
+                out->idx = comp_idx(cand[ans]);
+                out->val = L::from_f32(s_cum[ans]);
+            }
         }
     }
 }
 
-extern "C" __global__ void __launch_bounds__(SB) sample_topk_f16(SampleParams p) { sample_topk_impl<f16>(p); }
-extern "C" __global__ void __launch_bounds__(SB) sample_topk_f32(SampleParams p) { sample_topk_impl<float>(p); }
+extern "C" __global__ void __launch_bounds__(SB) sample_topk_k64_f16(SampleParams p) { sample_topk_impl<f16, true>(p); }
+extern "C" __global__ void __launch_bounds__(SB) sample_topk_k64_f32(SampleParams p) { sample_topk_impl<float, true>(p); }
+extern "C" __global__ void __launch_bounds__(SB) sample_topk_f16(SampleParams p) { sample_topk_impl<f16, false>(p); }
+extern "C" __global__ void __launch_bounds__(SB) sample_topk_f32(SampleParams p) { sample_topk_impl<float, false>(p); }
 
 constexpr uint32_t LIST_CAP = 2048;  // entries of the short list a row is cut down to after the first digit
 
@@ -582,7 +664,13 @@ __device__ __forceinline__ void sample_topk_list_impl(const SampleParams &p) {
 
     // 1b. among the ties, the krem-th smallest index
     uint32_t istar = 0xffffffffu;
-    if (eq_count > krem) {  // uniform branch
+    bool ranked = false;
+    if (eq_count > krem) {
+        ranked = kth_tied_index(each, kstar, krem, eq_count, reinterpret_cast<uint32_t *>(cand), &s_cnt, &s_sel[0]);
+        if (ranked) istar = s_sel[0];
+        __syncthreads();
+    }
+    if (eq_count > krem && !ranked) {  // uniform branch
         uint32_t ipre = 0, irem = krem;
         for (int shift = 24; shift >= 0; shift -= 8) {
             if (threadIdx.x < 256) hist[threadIdx.x] = 0;
@@ -657,7 +745,8 @@ __device__ __forceinline__ void sample_topk_list_impl(const SampleParams &p) {
         return;
     }
 
-    bitonic_lds(cand, P, 2, P, P, 0);
+    if (P <= 256) sort_desc_256(cand, P);
+    else bitonic_lds(cand, P, 2, P, P, 0);
     // 3. running sums
     if (threadIdx.x < P)
         s_cum[threadIdx.x] = threadIdx.x == 0   ? 1.0f
