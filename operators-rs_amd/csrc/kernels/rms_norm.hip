@@ -31,6 +31,34 @@ __device__ __forceinline__ float load_w(const void *w, uint32_t j) {
     return (float)reinterpret_cast<const TW *>(w)[j];
 }
 
+// The same in two steps, so that the load can be issued before the row's reduction and the conversion done
+// after it: N consecutive weights are N * sizeof(TW) / 16 vectors of 16 bytes.
+template <typename TW, int N>
+struct RawW {
+    static constexpr int NV = N * sizeof(TW) / 16;
+    u32x4 v[NV];
+    __device__ __forceinline__ void load(const void *w, uint32_t j) {
+#pragma unroll
+        for (int c = 0; c < NV; ++c) v[c] = ld128(reinterpret_cast<const TW *>(w) + j + c * (16 / sizeof(TW)));
+    }
+    __device__ __forceinline__ void get(float (&out)[N]) const {
+        if constexpr (sizeof(TW) == 2) {
+            Pack8 p;
+            p.u = v[0];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) out[i] = h2f(p.e[i]);
+        } else {
+#pragma unroll
+            for (int c = 0; c < NV; ++c) {
+                Pack4f p;
+                p.u = v[c];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) out[4 * c + i] = p.e[i];
+            }
+        }
+    }
+};
+
 // N consecutive weights starting at element j (j multiple of N, base 16-byte aligned)
 template <typename TW, int N>
 __device__ __forceinline__ void load_w_vec(const void *w, uint32_t j, float (&out)[N]) {
@@ -69,12 +97,17 @@ __device__ __forceinline__ void rms_norm_vec(const RmsNormParams &p) {
     const uint32_t nvec = p.d / N;
 
     Vec<TA> cache[CACHE];
+    // w for the cached vectors is requested together with x: asked for after the reduction (a barrier the
+    // compiler will not move a load across) it would put a second memory latency into a kernel that, on a
+    // few rows, is nothing but latency
+    RawW<TW, N> wraw[CACHE];
     float ss = 0.f;
 #pragma unroll
     for (int c = 0; c < CACHE; ++c) {
         const uint32_t v = lane + c * G;
         if (v < nvec) {
             cache[c].v.u = ld128(xr + (size_t)v * 16);
+            wraw[c].load(p.w, v * N);
 #pragma unroll
             for (int i = 0; i < N; ++i) {
                 const float f = cache[c].get(i);
@@ -99,7 +132,7 @@ __device__ __forceinline__ void rms_norm_vec(const RmsNormParams &p) {
         const uint32_t v = lane + c * G;
         if (v < nvec) {
             float w[N];
-            load_w_vec<TW, N>(p.w, v * N, w);
+            wraw[c].get(w);
             Vec<TA> o;
 #pragma unroll
             for (int i = 0; i < N; ++i) o.set(i, (k * w[i]) * cache[c].get(i));

@@ -30,17 +30,24 @@ __device__ __forceinline__ void rope_fill_table(const RopeParams &p, uint32_t to
 
 extern "C" __global__ void __launch_bounds__(256) rope_f16_vec(RopeParams p) {
     const uint32_t token = blockIdx.x;
-    rope_fill_table(p, token);
     const uint32_t cpv = p.dh / 8;  // 16-byte chunks per head
     const uint32_t h0 = blockIdx.y * p.heads_per_block;
     const uint32_t h1 = min(h0 + p.heads_per_block, p.nh);
     const uint32_t total = (h1 - h0) * cpv;
     char *base = reinterpret_cast<char *>(p.t) + (int64_t)token * p.st;
+    auto chunk = [&](uint32_t v) { return base + (int64_t)(h0 + v / cpv) * p.sh + (size_t)(v % cpv) * 16; };
+    // The thread's first chunk is requested before the table is filled (a load of pos, the transcendentals, a
+    // barrier): on a few tokens the kernel is nothing but latency, and this takes one memory latency out of it.
+    Pack8 first;
+    first.u = u32x4{0, 0, 0, 0};
+    if (threadIdx.x < total) first.u = ld128(chunk(threadIdx.x));
+    rope_fill_table(p, token);
     for (uint32_t v = threadIdx.x; v < total; v += blockDim.x) {
-        const uint32_t h = h0 + v / cpv, c = v % cpv;
-        char *ptr = base + (int64_t)h * p.sh + (size_t)c * 16;
+        const uint32_t c = v % cpv;
+        char *ptr = chunk(v);
         Pack8 x, o;
-        x.u = ld128(ptr);
+        if (v == threadIdx.x) x.u = first.u;
+        else x.u = ld128(ptr);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const float2 sc = rope_sc[4 * c + i];
