@@ -822,6 +822,8 @@ DECODE_GEMMS = [
     ("qk_t", 32, 16, 2048, 128, True),
     ("pv", 32, 16, 128, 2048, False),
     ("wide_288_strips", 1, 16, 36864, 1024, False),  # a few more column strips than CUs: K is halved
+    ("qkv_32_rows", 1, 32, 12288, 4096, False),  # the 32- and 64-row builds of the paired-step streaming kernel
+    ("gate_up_48_rows", 1, 48, 22016, 4096, False),
 ]
 
 
@@ -841,6 +843,10 @@ def test_mat_mul_decode_layer_shapes(gpu, stream, name, bt, m, n, k, b_transpose
     b = bfull.swapaxes(-1, -2) if b_transposed else bfull
     c = np.zeros(shape(m, n), f16)
     say("mat_mul decode %s" % name)
+    if name in ("qkv", "gate_up", "qkv_32_rows", "gate_up_48_rows"):
+        args = ophip.MatMulArgs(TensorLayout.of(c), None, 0.0, TensorLayout.of(a), None, TensorLayout.of(b), None, alpha)
+        what = ophip.MatMul(gpu).describe(args)
+        assert what.startswith("skinny") and "paired" in what, what
     oracle.set_threads(8)
     try:
         out = run_mat_mul(gpu, stream, c, a, b, alpha, 0.0)
