@@ -10,7 +10,7 @@ using namespace ophip;
 
 namespace {
 
-constexpr size_t TOPK_FAST_MAX = 1024;  // candidates the single-workgroup top-k kernel sorts in LDS
+constexpr size_t TOPK_FAST_MAX = 8192;  // candidates the single-workgroup top-k kernels sort in LDS (KCAP in random_sample.hip)
 
 struct SampleMeta {
     uint64_t dt;
@@ -140,9 +140,25 @@ static void sample_launch(const ophip_random_sample *op, const ophip_random_samp
         launch(!in_registers ? op->topk_list[ti] : k_eff <= 64 ? op->topk_k64[ti] : op->topk[ti], grid, Dim3{1024}, 0, stream_of(qa), p);
         return;
     }
+    // top_k beyond the LDS kernels (or none): they try first, with 64, 1024 and then 8192 candidates, and leave a
+    // word per row saying whether those candidates already hold top_p of the probability; each kernel in line
+    // only does the rows still open, the full sort last (on the peaked distributions of a language model the
+    // first try settles every row)
     p.npow2 = (uint32_t)next_pow2(n);
     Workspace ws(qa, workspace, workspace_len, rows * full_sort_workspace(n));
     p.workspace = ws.ptr();
+    const bool in_registers = n <= 32768 && aligned16(p.logits) && (rows == 1 || row_stride % 16 == 0);
+    const hipFunction_t attempt = in_registers ? op->topk[ti] : op->topk_list[ti];
+    SampleParams first = p;
+    first.k_eff = 64;
+    first.verify_cover = 1;
+    launch(attempt, grid, Dim3{1024}, 0, stream_of(qa), first);
+    first.verify_cover = 3;
+    for (size_t k : {(size_t)1024, TOPK_FAST_MAX}) {
+        first.k_eff = (uint32_t)k;
+        launch(attempt, grid, Dim3{1024}, 0, stream_of(qa), first);
+    }
+    p.verify_cover = 2;
     launch(op->full[ti], grid, Dim3{1024}, 0, stream_of(qa), p);
 }
 

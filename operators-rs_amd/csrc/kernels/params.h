@@ -69,6 +69,11 @@ struct SampleParams {
     uint32_t k_eff;      // min(top_k, n)
     float temperature, top_p, seed;
     uint32_t npow2;      // general path: n rounded up to a power of two
+    // top_k beyond what the single-workgroup kernels sort (or no top_k at all): they try first, with 64, 1024 and then
+    // 8192 candidates, and report in the first word of the row's workspace whether those candidates already
+    // hold top_p of the probability (0: the result is written; 1: the next kernel in line has to do the row).
+    // Bit 0: write that word; bit 1: read it first and leave the row alone if it is 0.
+    uint32_t verify_cover;
 };
 
 // Canonical GEMM seen by the kernels:

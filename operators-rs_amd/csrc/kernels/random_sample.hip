@@ -10,7 +10,7 @@
 // together with the index of the last NaN; only if a NaN exists does a second
 // sweep redo the search on the suffix after it.
 //
-// sampling, top_k <= 1024 (`sample_topk`): the reference's answer always lies
+// sampling, top_k <= 8192 (`sample_topk`, `sample_topk_k64` for top_k <= 64): the reference's answer always lies
 // in the first min(top_k, n) entries of the order (value descending, index
 // ascending), so no full sort is needed:
 //   1. radix-select the k-th largest key (8-bit digits through an LDS histogram),
@@ -20,11 +20,15 @@
 //      order, each term being exp() evaluated in f64 and rounded once to f32, so
 //      cum[0..k) follows the sequential definition; the sum over all n entries
 //      (needed for top_p) is a parallel f32 reduction in a fixed order.
-// sampling, top_k <= 1024, rows that do not fit the registers (`sample_topk_list`): after the first digit the
+// the same for rows that do not fit the registers (`sample_topk_list`): after the first digit the
 // elements that can still matter (the chosen bucket and everything above it) are copied to a short list in
 // LDS, in the same sweep that sums the exponentials of the whole row; the rest runs on the list.
-// sampling, any top_k (`sample_full`): full bitonic sort in a global workspace,
-// then the same sequential scan over all n entries.
+// sampling, any top_k (`sample_full`): full bitonic sort in a global workspace, then the same sequential scan
+// over all n entries (by wave 0, 64 terms at a time).  The host puts the top-k kernels in front of it with 64,
+// 1024 and 8192 candidates standing in for the larger top_k: a try whose candidates already hold top_p of
+// the probability gives the same answer and settles the row (a word per row in the workspace says so), and
+// the kernels behind it leave that row alone.  On the peaked distributions of a language model the first
+// try does; the full sort is for flat ones.
 #include "device_util.h"
 
 struct KvPair {
@@ -76,6 +80,21 @@ struct Logit<float> {
 };
 
 constexpr int SB = 1024;  // workgroup size of every kernel in this file
+// the full-sort workspace of the row this workgroup serves (npow2 u64 sort keys, then n f32 running sums)
+__device__ __forceinline__ char *sample_row_workspace(const SampleParams &p) {
+    const size_t ws_row = (size_t)p.npow2 * 8 + (((size_t)p.n * 4 + 15) & ~(size_t)15);
+    return reinterpret_cast<char *>(p.workspace) + blockIdx.x * ws_row;
+}
+
+// An earlier kernel in line has finished this row (all threads call; workgroup-uniform).
+__device__ __forceinline__ bool sample_row_done(const SampleParams &p) {
+    if (!(p.verify_cover & 2)) return false;
+    const uint32_t todo = *reinterpret_cast<const uint32_t *>(sample_row_workspace(p));
+    __syncthreads();  // everybody has read the word before anybody writes it again
+    return todo == 0;
+}
+
+constexpr uint32_t KCAP = 8192;  // largest top_k the single-workgroup kernels sort in LDS (the host's TOPK_FAST_MAX)
 
 // Calls f(index, raw bits) for every element of the row, 16 bytes per load when the
 // row is 16-byte aligned (8 f16 or 4 f32 per thread and step), else element-wise.
@@ -380,11 +399,14 @@ __device__ __forceinline__ void sample_topk_impl(const SampleParams &p) {
     __shared__ uint32_t s_wtot[4];
     __shared__ uint32_t s_sel[2];
     __shared__ uint32_t s_cnt;
-    __shared__ uint64_t cand[SB];
-    __shared__ float s_cum[SB];
+    constexpr uint32_t KC = SMALLK ? SB : KCAP;  // candidates the kernel has room for
+    __shared__ uint64_t cand[KC];
+    __shared__ float s_cum[KC];
     __shared__ float s_red[SB / WAVE];
     __shared__ float s_mx;
 
+    if constexpr (!SMALLK)
+        if (sample_row_done(p)) return;
     const char *row = reinterpret_cast<const char *>(p.logits) + (int64_t)blockIdx.x * p.row_stride;
     const uint32_t n = p.n, k = p.k_eff;
     RowCache<T> rc;
@@ -458,7 +480,7 @@ __device__ __forceinline__ void sample_topk_impl(const SampleParams &p) {
         const uint32_t key = L::key(bits);
         if (key > kstar || (key == kstar && i <= istar)) {
             const uint32_t slot = atomicAdd(&s_cnt, 1u);
-            if (slot < SB) cand[slot] = composite(key, i);
+            if (slot < KC) cand[slot] = composite(key, i);
         }
     });
     __syncthreads();
@@ -498,6 +520,13 @@ __device__ __forceinline__ void sample_topk_impl(const SampleParams &p) {
                 if (lane == (uint32_t)i) mine = c;
             }
             const float pk = c;  // terms past k are zero, so the chain ends at cum[k-1]
+            if constexpr (!SMALLK) {
+                if (p.verify_cover & 1) {  // k stands in for a larger top_k: do these candidates hold top_p of the mass?
+                    const bool uncovered = pk < total * p.top_p;
+                    if (lane == 0) *reinterpret_cast<uint32_t *>(sample_row_workspace(p)) = uncovered ? 1u : 0u;
+                    if (uncovered) return;  // the next kernel in line does this row
+                }
+            }
             const float plimit = row_seed(p) * fminf(pk, total * p.top_p);
             const uint64_t hit = __ballot(lane < k && mine >= plimit);
             const uint32_t ans = hit ? (uint32_t)__ffsll((long long)hit) - 1 : k - 1;
@@ -519,10 +548,8 @@ __device__ __forceinline__ void sample_topk_impl(const SampleParams &p) {
         const float inv_t = 1.0f / t;
         rc.for_each(row, n, [&](uint32_t, uint32_t bits) { part += fast_exp((L::value(bits) - mx) * inv_t); });
         const float total = block_sum_f32(part, s_red);
-        if (threadIdx.x < P)
-            s_cum[threadIdx.x] = threadIdx.x == 0   ? 1.0f
-                                 : threadIdx.x < k ? exp_cr((L::value(L::unkey(comp_key(cand[threadIdx.x]))) - mx) / t)
-                                                   : 0.f;
+        for (uint32_t i = threadIdx.x; i < P; i += SB)
+            s_cum[i] = i == 0 ? 1.0f : i < k ? exp_cr((L::value(L::unkey(comp_key(cand[i]))) - mx) / t) : 0.f;
         __syncthreads();
         if (threadIdx.x < WAVE) {
             // wave 0 replays the sequential sum 64 entries at a time, carrying the running value
@@ -539,6 +566,11 @@ __device__ __forceinline__ void sample_topk_impl(const SampleParams &p) {
                 s_cum[base + lane] = mine;
             }
             const float pk = c;  // entries past k add zero
+            if (p.verify_cover & 1) {  // k stands in for a larger top_k: do these candidates hold top_p of the mass?
+                const bool uncovered = pk < total * p.top_p;
+                if (lane == 0) *reinterpret_cast<uint32_t *>(sample_row_workspace(p)) = uncovered ? 1u : 0u;
+                if (uncovered) return;  // the full-sort kernel does this row
+            }
             const float plimit = row_seed(p) * fminf(pk, total * p.top_p);
             uint32_t ans = k - 1;
             for (uint32_t base = 0; base < P; base += WAVE) {
@@ -571,6 +603,7 @@ constexpr uint32_t LIST_CAP = 2048;  // entries of the short list a row is cut d
 template <typename T>
 __device__ __forceinline__ void sample_topk_list_impl(const SampleParams &p) {
     typedef Logit<T> L;
+    if (sample_row_done(p)) return;
     const char *row = reinterpret_cast<const char *>(p.logits) + (int64_t)blockIdx.x * p.row_stride;
     const uint32_t n = p.n;
     auto sweep_row = [&](auto &&f) { for_each_logit<T>(row, n, f); };  // f(index, raw bits) for every element
@@ -579,9 +612,10 @@ __device__ __forceinline__ void sample_topk_list_impl(const SampleParams &p) {
     __shared__ uint32_t s_wtot[4];
     __shared__ uint32_t s_sel[2];
     __shared__ uint32_t s_cnt;
-    __shared__ uint64_t cand[SB];
+    constexpr uint32_t KC = KCAP;
+    __shared__ uint64_t cand[KC];
     __shared__ uint64_t list[LIST_CAP];
-    __shared__ float s_cum[SB];
+    __shared__ float s_cum[KC];
     __shared__ float s_red[SB / WAVE];
     __shared__ uint32_t s_kmax[SB / WAVE];
     const uint32_t k = p.k_eff;
@@ -697,7 +731,7 @@ __device__ __forceinline__ void sample_topk_list_impl(const SampleParams &p) {
     each([&](uint32_t i, uint32_t key) {
         if (key > kstar || (key == kstar && i <= istar)) {
             const uint32_t slot = atomicAdd(&s_cnt, 1u);
-            if (slot < SB) cand[slot] = composite(key, i);
+            if (slot < KC) cand[slot] = composite(key, i);
         }
     });
     __syncthreads();
@@ -733,6 +767,11 @@ __device__ __forceinline__ void sample_topk_list_impl(const SampleParams &p) {
                 if (lane == (uint32_t)i) mine = c;
             }
             const float pk = c;  // terms past k are zero, so the chain ends at cum[k-1]
+            if (p.verify_cover & 1) {  // k stands in for a larger top_k: do these candidates hold top_p of the mass?
+                const bool uncovered = pk < total * p.top_p;
+                if (lane == 0) *reinterpret_cast<uint32_t *>(sample_row_workspace(p)) = uncovered ? 1u : 0u;
+                if (uncovered) return;  // the next kernel in line does this row
+            }
             const float plimit = row_seed(p) * fminf(pk, total * p.top_p);
             const uint64_t hit = __ballot(lane < k && mine >= plimit);
             const uint32_t ans = hit ? (uint32_t)__ffsll((long long)hit) - 1 : k - 1;
@@ -748,10 +787,8 @@ __device__ __forceinline__ void sample_topk_list_impl(const SampleParams &p) {
     if (P <= 256) sort_desc_256(cand, P);
     else bitonic_lds(cand, P, 2, P, P, 0);
     // 3. running sums
-    if (threadIdx.x < P)
-        s_cum[threadIdx.x] = threadIdx.x == 0   ? 1.0f
-                             : threadIdx.x < k ? exp_cr((L::value(L::unkey(comp_key(cand[threadIdx.x]))) - mx) / t)
-                                               : 0.f;
+    for (uint32_t i = threadIdx.x; i < P; i += SB)
+        s_cum[i] = i == 0 ? 1.0f : i < k ? exp_cr((L::value(L::unkey(comp_key(cand[i]))) - mx) / t) : 0.f;
     __syncthreads();
     if (threadIdx.x < WAVE) {
         // wave 0 replays the sequential sum 64 entries at a time, carrying the running value
@@ -768,6 +805,11 @@ __device__ __forceinline__ void sample_topk_list_impl(const SampleParams &p) {
             s_cum[base + lane] = mine;
         }
         const float pk = c;  // entries past k add zero
+        if (p.verify_cover & 1) {  // k stands in for a larger top_k: do these candidates hold top_p of the mass?
+            const bool uncovered = pk < total * p.top_p;
+            if (lane == 0) *reinterpret_cast<uint32_t *>(sample_row_workspace(p)) = uncovered ? 1u : 0u;
+            if (uncovered) return;  // the full-sort kernel does this row
+        }
         const float plimit = row_seed(p) * fminf(pk, total * p.top_p);
         uint32_t ans = k - 1;
         for (uint32_t base = 0; base < P; base += WAVE) {
@@ -800,9 +842,9 @@ __device__ __forceinline__ void sample_full_impl(const SampleParams &p) {
 
     const uint32_t n = p.n, np2 = p.npow2;
     const char *row = reinterpret_cast<const char *>(p.logits) + (int64_t)blockIdx.x * p.row_stride;
-    const size_t ws_row = (size_t)np2 * 8 + (((size_t)n * 4 + 15) & ~(size_t)15);
-    uint64_t *keys = reinterpret_cast<uint64_t *>(reinterpret_cast<char *>(p.workspace) + blockIdx.x * ws_row);
+    uint64_t *keys = reinterpret_cast<uint64_t *>(sample_row_workspace(p));
     float *cum = reinterpret_cast<float *>(keys + np2);
+    if (sample_row_done(p)) return;  // a top-k kernel ran first and finished the row
 
     for (uint32_t i = threadIdx.x; i < np2; i += SB)
         keys[i] = i < n ? composite(L::key(L::bits(row, i)), i) : 0;
@@ -845,13 +887,26 @@ __device__ __forceinline__ void sample_full_impl(const SampleParams &p) {
     for (uint32_t i = threadIdx.x; i < n; i += SB)
         cum[i] = i == 0 ? 1.0f : exp_cr((L::value(L::unkey(comp_key(keys[i]))) - mx) / t);
     __syncthreads();
-    if (threadIdx.x == 0) {
-        float c = 1.0f;
-        for (uint32_t i = 1; i < n; ++i) {
-            c = c + cum[i];
-            cum[i] = c;
+    if (threadIdx.x < WAVE) {
+        // the sequential f32 running sum, by wave 0: 64 terms at a time are loaded together (the next 64 already
+        // on their way), then every lane replays the same chain of 64 additions and keeps its own prefix
+        // (0 + cum[0] is exactly the 1.0 the sum starts from; lanes past n add zeros)
+        const uint32_t lane = threadIdx.x;
+        float c = 0.f;
+        float e = lane < n ? cum[lane] : 0.f;
+        for (uint32_t base = 0; base < n; base += WAVE) {
+            const uint32_t nxt = base + WAVE + lane;
+            const float e_next = nxt < n ? cum[nxt] : 0.f;
+            float mine = 0.f;
+#pragma unroll
+            for (int i = 0; i < WAVE; ++i) {
+                c = c + __shfl(e, i, WAVE);
+                if (lane == (uint32_t)i) mine = c;
+            }
+            if (base + lane < n) cum[base + lane] = mine;
+            e = e_next;
         }
-        s_ans = n - 1;
+        if (lane == 0) s_ans = n - 1;
     }
     __syncthreads();
     const float pk = cum[p.k_eff - 1];

@@ -708,12 +708,17 @@ def test_random_sample_all_equal_and_edge_draws(gpu, stream):
     assert run_sample(gpu, stream, y, ophip.SampleArgs(0.8, 0.9, 50), 0.0, op=op)[0] == int(np.argmax(y))
 
 
-@pytest.mark.parametrize("top_k", [1025, 5000, ophip.DYN_USIZE])
+@pytest.mark.parametrize("top_k", [1025, 5000, 8192, 8193, ophip.DYN_USIZE])
 def test_random_sample_large_top_k_full_sort(gpu, stream, top_k):
+    """top_k up to 8192 is sorted in LDS; beyond that (or with no top_k) the row is tried with 1024 and 8192
+    candidates first and only goes through the full sort when those do not hold top_p of the probability:
+    peaked logits (std 6) settle in the first try, std 1.7 in the second on 32000 logits, flat ones
+    (std 0.3) need the full sort."""
     rng = np.random.default_rng(8)
     op = ophip.RandomSample(gpu)
-    for n, dtype in [(32000, f16), (3000, f32), (50257, f16)]:
-        x = (rng.standard_normal(n) * 1.7).astype(f32).astype(dtype)
+    for n, dtype, std in [(32000, f16, 1.7), (3000, f32, 1.7), (50257, f16, 1.7), (32000, f16, 6.0), (128256, f16, 6.0),
+                          (20000, f32, 0.3), (40000, f16, 0.3)]:
+        x = (rng.standard_normal(n) * std).astype(f32).astype(dtype)
         args = ophip.RandomSampleArgs.layout(ophip.NP_DT[np.dtype(dtype)], n)
         need = op.scheme(args, 2 ** 40)
         assert need > 0
