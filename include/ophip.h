@@ -145,6 +145,11 @@ OPHIP_API int ophip_event_record(ophip_device *dev, ophip_event ev, ophip_stream
 OPHIP_API int ophip_event_synchronize(ophip_device *dev, ophip_event ev);
 OPHIP_API int ophip_event_elapsed_ms(ophip_device *dev, ophip_event start, ophip_event stop,
                                      float *ms);
+/* Measurement aid, no counterpart in the reference: the next kernel this thread launches on `stream` (through any
+ * operator of this library) records its own begin into `start` and its own end into `stop`, so that
+ * ophip_event_elapsed_ms(start, stop) is the kernel's duration on the device, without the cost of two separate event
+ * records around it.  An operator that launches several kernels times its first. */
+OPHIP_API int ophip_time_next_launch(ophip_device *dev, ophip_stream stream, ophip_event start, ophip_event stop);
 
 /* Launch graphs (no counterpart in the reference's driver crate): a fixed sequence of launch()
  * calls on `stream` between begin and end is recorded instead of run, and replayed by

@@ -1145,6 +1145,29 @@ def test_recorded_launch_sequence_replays_like_eager_launches(gpu, stream):
     graph.destroy()
 
 
+def test_time_next_launch_gives_the_kernels_own_duration(gpu, stream):
+    """ophip_time_next_launch: the next kernel on the stream records its own begin and end; the one after is an
+    ordinary launch again, and results are unaffected."""
+    rng = np.random.default_rng(3)
+    x = normal_f16(rng, (64, 4096))
+    w = rng.uniform(0.5, 1.5, 4096).astype(f32).astype(f16)
+    xd, wd, yd = gpu.from_host(x), gpu.from_host(w), gpu.malloc(x.nbytes)
+    c = lambda *s: TensorLayout.new_contiguous(dt.F16, list(s))
+    op = ophip.RmsNorm(gpu)
+    a = ophip.RmsNormArgs(c(64, 4096), yd, c(64, 4096), xd, c(4096), wd, 1e-5)
+    op.launch(a, None, stream)
+    e0, e1 = gpu.event(), gpu.event()
+    gpu.time_next_launch(stream, e0, e1)
+    op.launch(a, None, stream)
+    op.launch(a, None, stream)
+    stream.synchronize()
+    us = e0.elapsed_ms(e1) * 1e3
+    say("rms_norm [64, 4096] by its own events: %.2f us" % us)
+    assert 0.5 < us < 200.0
+    got = gpu.to_host(yd, f16, x.size, stream=stream).reshape(x.shape)
+    assert_close_f16(got, oracle.rms_norm(np.empty_like(x), x, w, 1e-5), "rms_norm after a timed launch")
+
+
 # ------------------------------------------------------------- threading ----
 
 def test_one_operator_instance_launched_from_several_threads(gpu):
