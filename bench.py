@@ -507,25 +507,24 @@ def main():
     stream.synchronize()
 
     # The dominant kernel is timed on every EVERY-th step only (an odd stride, so both weight sets are sampled):
-    # on steps 0, 7, .. its launch carries two events that the kernel itself records at its begin and its end
-    # (the figure the rocprofv3 trace must agree with); on steps 3, 10, .. two separate event records bracket the
-    # launch, which reads longer by most of what an empty pair of records reads.
+    # its launch carries two events that the kernel itself records at its begin and its end (the figure the
+    # rocprofv3 trace must agree with).
     DOM, EVERY = "gate_up", 7
     own = [(gpu.event(), gpu.event()) for _ in range(0, args.steps, EVERY)]
-    pairs = [(gpu.event(), gpu.event()) for _ in range(3, args.steps, EVERY)]
     t0 = time.perf_counter()
     for i in range(args.steps):
-        if i % EVERY == 0:
-            layers[i % 2].step(stream, own={DOM: own[i // EVERY]})
-        elif i % EVERY == 3:
-            layers[i % 2].step(stream, around={DOM: pairs[i // EVERY]})
-        else:
-            layers[i % 2].step(stream)
+        layers[i % 2].step(stream, own={DOM: own[i // EVERY]} if i % EVERY == 0 else None)
     stream.synchronize()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / args.steps
     dom_us = float(np.mean([a.elapsed_ms(b) for a, b in own])) * 1e3
-    bracketed_us = float(np.mean([a.elapsed_ms(b) for a, b in pairs])) * 1e3 if pairs else None
+    # For comparison, outside the timed region: two separate event records around the same launch, which read
+    # longer by most of what an empty pair of records reads.
+    pairs = [(gpu.event(), gpu.event()) for _ in range(20)]
+    for i, pr in enumerate(pairs):
+        layers[i % 2].step(stream, around={DOM: pr})
+    stream.synchronize()
+    bracketed_us = float(np.mean([a.elapsed_ms(b) for a, b in pairs])) * 1e3
     # What a pair of event records reads with nothing between them, in the same position of the layer
     # (after rms_norm_2): the part of the bracketed time that is not the kernel.
     empties = [(gpu.event(), gpu.event()) for _ in range(40)]
@@ -602,8 +601,9 @@ def main():
                      "bracketed_us": round(bracketed_us, 3) if bracketed_us is not None else None,
                      "event_pair_us": round(event_pair_us, 3),
                      "note": "us is between two events the kernel's own launch records at its begin and end, inside the "
-                             "timed steps; bracketed_us is between two separate event records around the launch, "
-                             "event_pair_us what such a pair reads with no kernel between them"},
+                             "timed steps; bracketed_us is between two separate event records around the launch (20 "
+                             "more steps after the timed ones), event_pair_us what such a pair reads with no kernel "
+                             "between them"},
         "cpu_baseline": cpu,
         "copy_ceiling": ceiling,
         "per_op_layer": per_layer,
