@@ -509,7 +509,7 @@ def main():
     # The dominant kernel is timed on every EVERY-th step only (an odd stride, so both weight sets are sampled):
     # its launch carries two events that the kernel itself records at its begin and its end (the figure the
     # rocprofv3 trace must agree with).
-    DOM, EVERY = "gate_up", 7
+    DOM, EVERY = "gate_up", 25  # (a launch that carries events costs the step about 4 us)
     own = [(gpu.event(), gpu.event()) for _ in range(0, args.steps, EVERY)]
     t0 = time.perf_counter()
     for i in range(args.steps):
