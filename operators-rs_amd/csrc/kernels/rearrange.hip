@@ -44,12 +44,7 @@ __device__ __forceinline__ void rearrange32(const RearrangeParams &p) {
             const uint32_t c = g - u * p.chunks_per_unit;
             uint32_t rem = u;
             int64_t d = (int64_t)c * B, s = (int64_t)c * B;
-            // (unrolled over the most dimensions there can be, so that every kernel argument sits at a fixed
-            // offset and all of them are fetched up front: indexed by a loop counter each would be a scalar load
-            // in the middle of the chain that leads to the thread's first load)
-#pragma unroll
-            for (uint32_t q = 0; q < OPHIP_REARRANGE_MAXD; ++q) {
-                if (q >= p.ndim) break;
+            for (uint32_t q = 0; q < p.ndim; ++q) {
                 const uint32_t k = fastdiv(rem, p.idx_div[q]);
                 rem -= k * p.idx_div[q].d;
                 d += (int64_t)k * p.dst_s[q];
