@@ -446,7 +446,12 @@ __device__ __forceinline__ void gemm_skinny(const GemmParams &p) {
         // arrival order) and resets the counter for the next launch.
         // The partials were written with device-scope (write-through) stores; once
         // every thread has seen its stores acknowledged the count may be published.
+        // A workgroup-scope fence does not wait for them (within one CU memory operations stay in
+        // order without that), and the count travels to another L2 channel than the partials: without
+        // the explicit wait it can overtake them, and a workgroup that arrives last right then sums
+        // whatever the buffer held before.
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         uint32_t *counter = reinterpret_cast<uint32_t *>(p.counters) + (size_t)bat * gridDim.x + blockIdx.x;
         if (threadIdx.x == 0) s_last = atomicAdd(counter, 1u) == p.split_k - 1 ? 1u : 0u;

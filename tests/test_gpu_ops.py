@@ -1063,6 +1063,38 @@ def test_mat_mul_split_k_workspace_paths(gpu, stream):
         assert_close_f16(out, ref, "split-k", abs_tol=4e-3)
 
 
+@pytest.mark.parametrize("m,n,k", [(16, 12288, 4096), (16, 1024, 4096), (48, 4096, 11008), (16, 1160, 2048)])
+def test_mat_mul_split_k_ignores_what_the_workspace_held(gpu, stream, m, n, k):
+    """The workgroup of a column strip that arrives last sums the partial sums of all K ranges: it must
+    see the other workgroups' partial sums, not what the workspace held before (NaNs here), however close
+    together they finish.  Many launches, each bit-identical to the first, which is checked against the oracle."""
+    rng = np.random.default_rng(m + n + k)
+    a = normal_f16(rng, (m, k))
+    b = normal_f16(rng, (k, n), std=0.02)
+    c = np.zeros((m, n), f16)
+    op = ophip.MatMul(gpu)
+    cd, ad, bd = gpu.from_host(c), gpu.from_host(a), gpu.from_host(b)
+    args = ophip.MatMulArgs(TensorLayout.of(c), cd, 0.0, TensorLayout.of(a), ad, TensorLayout.of(b), bd, 1.0)
+    what = op.describe(args)
+    assert what.startswith("skinny") and "split_k=1" not in what, what
+    need = op.scheme(args, 2 ** 40)
+    assert need > 0
+    ws = gpu.malloc(need)
+    say("mat_mul split-k over a dirty workspace %dx%dx%d: %s" % (m, n, k, what))
+    ref = c.copy()
+    oracle.mat_mul(ref, 0.0, a, b, 1.0)
+    first = None
+    for it in range(40):
+        gpu.memset(ws, 0xFF, stream=stream)
+        op.launch(args, ws, stream)
+        out = gpu.to_host(cd, f16, c.size, stream=stream).reshape(c.shape)
+        if first is None:
+            first = out
+            assert_close_f16(out, ref, "split-k over a dirty workspace", abs_tol=4e-3)
+        else:
+            assert np.array_equal(out.view(np.uint16), first.view(np.uint16)), "launch %d differs from the first" % it
+
+
 def run_mat_mul_with(gpu, stream, c, a, b, op, ws, qa):
     cd, ad, bd = gpu.from_host(c), gpu.from_host(a), gpu.from_host(b)
     args = ophip.MatMulArgs(TensorLayout.of(c), cd, 1.0, TensorLayout.of(a), ad, TensorLayout.of(b), bd, 1.0)
