@@ -322,22 +322,33 @@ constexpr size_t SPLITK_COUNTERS = 1 << 16;
 struct ophip_mat_mul {
     ophip_device *dev;
     hipFunction_t skinny[3][4];  // [mt index 1,2,4][qmode; 3 = mode 0 with paired K-steps]
-    hipFunction_t reduce, generic_f16, generic_f32;
+    hipFunction_t reduce, fill, generic_f16, generic_f32;
     // [256 x 64 / 128 x 64 / 128 x 32 (K-step)][M or N not in whole tiles][P K-contiguous][Q K-contiguous]
     hipFunction_t tile[3][2][2][2];
     // Arrival counters live in a buffer owned by the operator, one per stream:
     // launches on one stream run in order and every kernel leaves its counters at
-    // zero, so the buffer is zeroed once, when a stream is first seen.
+    // zero, so a buffer is zeroed once.  The first stream gets the buffer made (and cleared) with the operator,
+    // which costs no device work at launch time: that launch may be recorded into a graph.  A further stream
+    // gets a new buffer, cleared by a kernel on that stream; allocating is not possible while a stream records,
+    // so an operator's first split-K product on a second stream has to be an ordinary launch.
     mutable std::mutex mu;
     mutable std::unordered_map<hipStream_t, void *> counters;
+    mutable void *spare = nullptr;
 
     void *counters_for(hipStream_t stream) const {
         std::lock_guard<std::mutex> lock(mu);
         auto it = counters.find(stream);
         if (it != counters.end()) return it->second;
+        if (spare) {
+            void *buf = spare;
+            spare = nullptr;
+            counters[stream] = buf;
+            return buf;
+        }
         void *buf = nullptr;
         check_hip(hipMalloc(&buf, SPLITK_COUNTERS * sizeof(uint32_t)), "hipMalloc");
-        check_hip(hipMemsetAsync(buf, 0, SPLITK_COUNTERS * sizeof(uint32_t), stream), "hipMemsetAsync");
+        FillU32Params f{buf, (uint32_t)SPLITK_COUNTERS, 0u};
+        launch(fill, Dim3{(unsigned)(SPLITK_COUNTERS / 256)}, Dim3{256}, 0, stream, f);
         counters[stream] = buf;
         return buf;
     }
@@ -357,11 +368,22 @@ struct ophip_mat_mul {
                                                                     "_q" + std::to_string(qk)).c_str());
                     }
         reduce = d->kernel("gemm", "gemm_splitk_reduce");
+        fill = d->kernel("gemm", "gemm_fill_u32");
+        d->make_current();
+        check_hip(hipMalloc(&spare, SPLITK_COUNTERS * sizeof(uint32_t)), "hipMalloc");
+        const hipError_t e = hipMemset(spare, 0, SPLITK_COUNTERS * sizeof(uint32_t));
+        const hipError_t e2 = e == hipSuccess ? hipStreamSynchronize(nullptr) : e;
+        if (e2 != hipSuccess) {
+            (void)hipFree(spare);
+            ophip_device_release(d);
+            check_hip(e2, "hipMemset");
+        }
         generic_f16 = d->kernel("gemm", "gemm_generic_f16");
         generic_f32 = d->kernel("gemm", "gemm_generic_f32");
     }
     ~ophip_mat_mul() {
         for (auto &c : counters) (void)hipFree(c.second);
+        if (spare) (void)hipFree(spare);
         ophip_device_release(dev);
     }
 };

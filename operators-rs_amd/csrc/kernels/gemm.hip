@@ -596,5 +596,12 @@ __device__ __forceinline__ void gemm_generic(const GemmParams &p) {
         }
 }
 
+// Clears a fresh buffer of arrival counters.  A kernel rather than a memset: it can be recorded into a launch graph
+// like any other launch when an operator's first split-K product on a stream happens during recording.
+extern "C" __global__ void __launch_bounds__(256) gemm_fill_u32(FillU32Params p) {
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (i < p.count) reinterpret_cast<uint32_t *>(p.dst)[i] = p.value;
+}
+
 extern "C" __global__ void __launch_bounds__(256) gemm_generic_f16(GemmParams p) { gemm_generic<f16>(p); }
 extern "C" __global__ void __launch_bounds__(256) gemm_generic_f32(GemmParams p) { gemm_generic<float>(p); }

@@ -95,6 +95,13 @@ struct GemmParams {
     uint32_t k_per_split;  // multiple of 32
 };
 
+// dst[0 .. count) = value, 32-bit words (the split-K arrival counters start at zero)
+struct FillU32Params {
+    void *dst;
+    uint32_t count;
+    uint32_t value;
+};
+
 struct LayerNormParams {
     void *y;
     const void *x;

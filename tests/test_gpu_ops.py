@@ -1161,7 +1161,7 @@ def test_recorded_launch_sequence_replays_like_eager_launches(gpu, stream):
         sw.launch(a_sw, None, stream)
 
     say("launch graph: eager reference")
-    sequence()  # also lets mat_mul set up its per-stream counters before recording
+    sequence()
     want = gpu.to_host(gu, f16, 16 * 2048, stream=stream).copy()
     stream.begin_capture()
     sequence()
@@ -1174,6 +1174,36 @@ def test_recorded_launch_sequence_replays_like_eager_launches(gpu, stream):
         assert np.array_equal(got, want), "replay %d differs from the eager result" % rep
         rms.launch(a_rms, None, stream)  # eager work between replays
         stream.synchronize()
+    graph.destroy()
+
+
+def test_first_split_k_product_of_an_operator_may_be_recorded(gpu, stream):
+    """An operator that has never launched on the stream sets up its arrival counters with its first split-K
+    product; when that launch is being recorded, the set-up is part of the recording and every replay is right."""
+    rng = np.random.default_rng(22)
+    a, b = normal_f16(rng, (16, 4096)), normal_f16(rng, (4096, 1024), std=0.02)
+    ad, bd = gpu.from_host(a), gpu.from_host(b)
+    cd = gpu.malloc(16 * 1024 * 2)
+    c = lambda *s: TensorLayout.new_contiguous(dt.F16, list(s))
+    args = ophip.MatMulArgs(c(16, 1024), cd, 0.0, c(16, 4096), ad, c(4096, 1024), bd, 1.0)
+    eager = ophip.MatMul(gpu)
+    assert "split_k=1" not in eager.describe(args)
+    ws = gpu.malloc(eager.scheme(args, 1 << 30))
+    eager.launch(args, ws, stream)
+    want = gpu.to_host(cd, f16, 16 * 1024, stream=stream).copy()
+    fresh = ophip.MatMul(gpu)
+    say("launch graph: an operator's first split-K product, recorded")
+    stream.begin_capture()
+    fresh.launch(args, ws, stream)
+    graph = stream.end_capture()
+    for rep in range(4):
+        gpu.memset(cd, 0xFF, stream=stream)
+        gpu.memset(ws, 0xFF, stream=stream)
+        graph.launch(stream)
+        got = gpu.to_host(cd, f16, 16 * 1024, stream=stream)
+        assert np.array_equal(got, want), "replay %d differs from the eager result" % rep
+        fresh.launch(args, ws, stream)  # the same operator, eagerly, between replays
+        assert np.array_equal(gpu.to_host(cd, f16, 16 * 1024, stream=stream), want)
     graph.destroy()
 
 
