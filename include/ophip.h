@@ -129,7 +129,8 @@ typedef void *ophip_event;  /* hipEvent_t  */
 OPHIP_API int ophip_malloc(ophip_device *dev, size_t size, void **out);
 OPHIP_API int ophip_free(ophip_device *dev, void *ptr);
 /* Copies and fills: queued on `stream` when one is given; with a null stream the call returns
- * when the data is in place, so work queued afterwards on any stream sees it. */
+ * when the data is in place, so work queued afterwards on any stream sees it.  A fill on a stream
+ * is a kernel launch (any address and size), so it can be recorded into a graph like the operators. */
 OPHIP_API int ophip_memcpy_h2d(ophip_device *dev, void *dst, const void *src, size_t size,
                                ophip_stream stream);
 OPHIP_API int ophip_memcpy_d2h(ophip_device *dev, void *dst, const void *src, size_t size,

@@ -95,6 +95,16 @@ struct GemmParams {
     uint32_t k_per_split;  // multiple of 32
 };
 
+// dst[0 .. size) = value, bytes: the first `head` bytes (up to 16-byte alignment) and the last `tail` bytes one at a
+// time, `body` 16-byte units between them
+struct FillBytesParams {
+    void *dst;
+    uint64_t body;
+    uint32_t head, tail;
+    uint32_t value;  // the byte, repeated four times
+    uint32_t _pad;
+};
+
 // dst[0 .. count) = value, 32-bit words (the split-K arrival counters start at zero)
 struct FillU32Params {
     void *dst;

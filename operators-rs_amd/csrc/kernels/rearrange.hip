@@ -93,3 +93,14 @@ REARRANGE(8)
 REARRANGE(4)
 REARRANGE(2)
 REARRANGE(1)
+
+// memset on a stream, as a kernel: it is recorded into a launch graph like any other launch.
+extern "C" __global__ void __launch_bounds__(256) fill_bytes(FillBytesParams p) {
+    const uint64_t gid = (uint64_t)blockIdx.x * 256 + threadIdx.x, stride = (uint64_t)gridDim.x * 256;
+    char *dst = reinterpret_cast<char *>(p.dst);
+    if (gid < p.head) dst[gid] = (char)p.value;
+    char *body = dst + p.head;
+    const u32x4 v = u32x4{p.value, p.value, p.value, p.value};
+    for (uint64_t i = gid; i < p.body; i += stride) st128(body + 16 * i, v);
+    if (gid < p.tail) body[16 * p.body + gid] = (char)p.value;
+}

@@ -472,9 +472,9 @@ class Gpu:
                 stream.synchronize()
         return out
 
-    def memset(self, mem, value, size=None, stream=None):
-        _check(lib().ophip_memset(self.handle, ctypes.c_void_p(mem.ptr), int(value),
-                                  ctypes.c_size_t(mem.size if size is None else size),
+    def memset(self, mem, value, size=None, stream=None, offset=0):
+        _check(lib().ophip_memset(self.handle, ctypes.c_void_p(mem.ptr + offset), int(value),
+                                  ctypes.c_size_t(mem.size - offset if size is None else size),
                                   stream.handle if stream else None))
 
     def release(self):

@@ -1207,6 +1207,32 @@ def test_first_split_k_product_of_an_operator_may_be_recorded(gpu, stream):
     graph.destroy()
 
 
+def test_memset_on_a_stream_any_alignment_and_recorded(gpu, stream):
+    """ophip_memset with a stream is a kernel launch: any offset and length, bytes around the range untouched,
+    and a recorded fill replays (over changed contents) like the eager one."""
+    size = 1 << 16
+    buf = gpu.malloc(size)
+    for off, n, val in [(0, size, 0xAB), (1, 1, 0x01), (3, 29, 0x7F), (16, 4096, 0x00), (17, 4097, 0xFF), (5, 7, 0x3C),
+                        (15, 1, 0x11), (15, 17, 0x22), (32, 15, 0x33), (1, size - 2, 0x5A)]:
+        gpu.memset(buf, 0xEE)
+        gpu.memset(buf, val, n, stream=stream, offset=off)
+        got = gpu.to_host(buf, np.uint8, size, stream=stream)
+        want = np.full(size, 0xEE, np.uint8)
+        want[off:off + n] = val
+        assert np.array_equal(got, want), (off, n, val)
+    stream.begin_capture()
+    gpu.memset(buf, 0x42, 1000, stream=stream, offset=7)
+    graph = stream.end_capture()
+    for rep in range(3):
+        gpu.memset(buf, rep, stream=stream)
+        graph.launch(stream)
+        got = gpu.to_host(buf, np.uint8, size, stream=stream)
+        want = np.full(size, rep, np.uint8)
+        want[7:1007] = 0x42
+        assert np.array_equal(got, want), "replay %d" % rep
+    graph.destroy()
+
+
 def test_time_next_launch_gives_the_kernels_own_duration(gpu, stream):
     """ophip_time_next_launch: the next kernel on the stream records its own begin and end; the one after is an
     ordinary launch again, and results are unaffected."""
