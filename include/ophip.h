@@ -157,8 +157,9 @@ OPHIP_API int ophip_time_next_launch(ophip_device *dev, ophip_stream stream, oph
 /* Launch graphs (no counterpart in the reference's driver crate): a fixed sequence of launch()
  * calls on `stream` between begin and end is recorded instead of run, and replayed by
  * ophip_graph_launch without per-launch host cost.  Give every recorded launch a workspace of
- * its own (scheme() reports the size) and launch mat_mul once on the stream before recording:
- * its first launch on a stream allocates. */
+ * its own (scheme() reports the size).  A mat_mul operator used on more than one stream has to be
+ * launched once on each further stream before that stream records: its first split-K launch on a
+ * stream other than the first allocates, which HIP refuses while a stream records. */
 typedef void *ophip_graph; /* hipGraphExec_t */
 OPHIP_API int ophip_stream_begin_capture(ophip_device *dev, ophip_stream stream);
 OPHIP_API int ophip_stream_end_capture(ophip_device *dev, ophip_stream stream, ophip_graph *out);
