@@ -19,6 +19,9 @@
  *     them, launch() answers OPHIP_DYNAMIC_NOT_SUPPORT.
  *   - launch() only enqueues work on the queue's stream and returns; nothing
  *     synchronises.  A caller-provided workspace must outlive the enqueued work.
+ *     The kernels address a workspace 16 bytes at a time: a workspace that does
+ *     not start on a 16-byte boundary is used from the next boundary on, and
+ *     counts as too small when what is left there is less than scheme() asked for.
  *   - Return value: OPHIP_OK, one of the nine scheme error kinds (1..9, the
  *     declaration order of SchemeErrorKind), or OPHIP_EXECUTION_FAILED.  The
  *     text of the last error raised on the calling thread is available from

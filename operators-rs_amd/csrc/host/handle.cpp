@@ -102,9 +102,18 @@ void launch_raw(hipFunction_t fn, Dim3 grid, Dim3 block, size_t smem, hipStream_
 }
 
 Workspace::Workspace(const ophip_queue_alloc *qa, void *ext, size_t ext_len, size_t need) {
-    if (need == 0 || (ext && ext_len >= need)) {
+    if (need == 0) {
         ptr_ = ext;
         return;
+    }
+    // The kernels move 16 bytes at a time and use 64-bit atomics inside a workspace: a caller's slice that does not
+    // start on a 16-byte boundary is used from the next boundary on, if enough of it is left.
+    if (ext) {
+        const uintptr_t a = reinterpret_cast<uintptr_t>(ext), up = (a + 15) & ~(uintptr_t)15;
+        if (ext_len >= (up - a) && ext_len - (up - a) >= need) {
+            ptr_ = reinterpret_cast<void *>(up);
+            return;
+        }
     }
     if (!qa || !qa->alloc) throw execution_failed("workspace too small and no queue allocator given");
     ptr_ = qa->alloc(qa->ctx, need);

@@ -103,7 +103,25 @@ struct GemmPlan {
 
 bool mult8(int64_t v) { return (v & 7) == 0; }
 
-GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L, unsigned cus) {
+// Test and sweep knobs, read from the environment once, when an operator is created
+// (OPHIP_GEMM_SPLITK, OPHIP_GEMM_TILE_SPLITK, OPHIP_GEMM_TILE); 0 = not set.
+struct GemmKnobs {
+    int skinny_split = 0, tile_split = 0, tile = 0;
+    static GemmKnobs from_env() {
+        GemmKnobs k;
+        auto num = [](const char *name) {
+            const char *e = std::getenv(name);
+            const int v = e ? std::atoi(e) : 0;
+            return v > 0 ? v : 0;
+        };
+        k.skinny_split = num("OPHIP_GEMM_SPLITK");
+        k.tile_split = num("OPHIP_GEMM_TILE_SPLITK");
+        k.tile = num("OPHIP_GEMM_TILE");
+        return k;
+    }
+};
+
+GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L, unsigned cus, const GemmKnobs &knobs) {
     const void *a = L.ab_swap ? args.b_base : args.a_base;
     const void *b = L.ab_swap ? args.a_base : args.b_base;
     const int64_t a_si = L.a_trans ? L.a_ld : 1, a_sl = L.a_trans ? 1 : L.a_ld;
@@ -188,7 +206,7 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
                 // the time): halving the workgroups evens the load out a little (measured on 16 x 4096 x 36864 and
                 // 40960: 71 -> 65 and 72 -> 68 us; from 1.5 workgroups per CU on, a split only costs).
                 if (base > (size_t)cus && base * 4 <= (size_t)cus * 5 && slabs >= 32) split = 2;
-                if (const char *e = std::getenv("OPHIP_GEMM_SPLITK")) split = std::max(1, std::atoi(e));
+                if (knobs.skinny_split) split = (size_t)knobs.skinny_split;
                 size_t sps = (slabs + split - 1) / split;  // K-steps per split
                 split = (slabs + sps - 1) / sps;
                 p.k_per_split = (uint32_t)(sps * 32);
@@ -198,7 +216,7 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
                 if (g.qmode == 1 && p.N % 128 == 0 && p.K % 128 == 0) {
                     // (cold-weight sweeps: at least 8 chunks per split, i.e. two per wave, or the split costs more than it hides)
                     const size_t chunks = p.K / 128;
-                    if (!std::getenv("OPHIP_GEMM_SPLITK")) split = std::min(split, std::max<size_t>(1, chunks / 8));
+                    if (!knobs.skinny_split) split = std::min(split, std::max<size_t>(1, chunks / 8));
                     const size_t cps = (chunks + split - 1) / split;  // chunks per split
                     if (cps >= 4) {
                         g.qmode = 2;
@@ -252,7 +270,7 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
                 const size_t ksteps = tile_tk ? L.k / tile_tk : 1;
                 if (wgs > 0 && wgs * 2 <= cus)
                     split = std::min<size_t>({target / wgs, (size_t)8, std::max<size_t>(1, ksteps / 8)});
-                if (const char *e = std::getenv("OPHIP_GEMM_TILE_SPLITK")) split = std::max(1, std::atoi(e));
+                if (knobs.tile_split) split = (size_t)knobs.tile_split;
                 split = std::max<size_t>(1, std::min(split, ksteps));
             }
             for (int attempt = 0; attempt < 2; ++attempt) {
@@ -261,8 +279,8 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
                 // 256-tiles for less than 60 % of the CUs: the 128 pass is faster (measured on 512 .. 2048 row
                 // shapes: at half the CUs the large tile loses by 10 - 50 %, at two thirds it wins by 10 %)
                 // (OPHIP_GEMM_TILE=256 / 128 keeps one tile size, for tests and sweeps)
-                const char *force = std::getenv("OPHIP_GEMM_TILE");
-                if (force && (uint32_t)std::atoi(force) != b) continue;
+                const bool force = knobs.tile != 0;
+                if (force && (uint32_t)knobs.tile != b) continue;
                 // and when the part of the last tiles that lies outside the matrix costs more than the large tile's
                 // advantage (about 1.4 x per multiply at these sizes)
                 if (b == 256 && !force) {
@@ -321,6 +339,7 @@ constexpr size_t SPLITK_COUNTERS = 1 << 16;
 
 struct ophip_mat_mul {
     ophip_device *dev;
+    GemmKnobs knobs = GemmKnobs::from_env();
     hipFunction_t skinny[3][4];  // [mt index 1,2,4][qmode; 3 = mode 0 with paired K-steps]
     hipFunction_t reduce, fill, generic_f16, generic_f32;
     // [256 x 64 / 128 x 64 / 128 x 32 (K-step)][M or N not in whole tiles][P K-contiguous][Q K-contiguous]
@@ -414,7 +433,7 @@ int ophip_mat_mul_scheme(ophip_mat_mul *op, const ophip_mat_mul_args *args, size
         try {
             const ophip_mat_mul_layout L = mat_mul_layout(*args);
             if (L.dt != OPHIP_DT_F16 && L.dt != OPHIP_DT_F32) return;
-            const GemmPlan g = make_plan(*args, L, (unsigned)op->dev->props.multiProcessorCount);
+            const GemmPlan g = make_plan(*args, L, (unsigned)op->dev->props.multiProcessorCount, op->knobs);
             if (ws && g.workspace <= max_ws) *ws = g.workspace;
         } catch (const Error &) {
         }
@@ -426,7 +445,7 @@ int ophip_mat_mul_describe(const ophip_mat_mul *op, const ophip_mat_mul_args *ar
         if (!op || !args || !out || len == 0) throw args_not_support("null argument");
         const ophip_mat_mul_layout L = mat_mul_layout(*args);
         if (L.dt != OPHIP_DT_F16 && L.dt != OPHIP_DT_F32) throw type_not_support("mat_mul supports f16 and f32");
-        const GemmPlan g = make_plan(*args, L, (unsigned)op->dev->props.multiProcessorCount);
+        const GemmPlan g = make_plan(*args, L, (unsigned)op->dev->props.multiProcessorCount, op->knobs);
         if (g.kind == GemmPlan::Skinny)
             std::snprintf(out, len, "skinny rows<=%d q%s split_k=%u", 16 * g.mt,
                           g.qmode == 0 ? "N" : g.qmode == 1 ? "K" : g.qmode == 2 ? "K256" : "N paired",
@@ -448,7 +467,7 @@ int ophip_mat_mul_launch(const ophip_mat_mul *op, const ophip_mat_mul_args *args
         if (L.m == 0 || L.n == 0 || L.batch == 0) return;
         if (L.m > 0x7fffffffu || L.n > 0x7fffffffu || L.k > 0x7fffffffu || L.batch > 65535)
             throw shape_not_support("mat_mul dimension too large");
-        GemmPlan g = make_plan(*args, L, (unsigned)op->dev->props.multiProcessorCount);
+        GemmPlan g = make_plan(*args, L, (unsigned)op->dev->props.multiProcessorCount, op->knobs);
         const GemmParams &p = g.p;
         hipStream_t stream = stream_of(qa);
         op->dev->make_current();

@@ -1061,6 +1061,12 @@ def test_mat_mul_split_k_workspace_paths(gpu, stream):
     for ws, qa in [(None, stream), (gpu.malloc(need), stream), (None, pool)]:
         out = run_mat_mul_with(gpu, stream, c, a, b, op, ws, qa)
         assert_close_f16(out, ref, "split-k", abs_tol=4e-3)
+    # a caller's slice that starts off a 16-byte boundary: used from the next boundary on when enough of it is
+    # left, otherwise it counts as too small and the queue allocator serves the launch
+    slab = gpu.malloc(need + 64)
+    for off, length in [(2, need + 14), (6, need + 32), (2, need), (12, need + 3)]:
+        out = run_mat_mul_with(gpu, stream, c, a, b, op, (slab.ptr + off, length), stream)
+        assert_close_f16(out, ref, "split-k, workspace at +%d" % off, abs_tol=4e-3)
 
 
 @pytest.mark.parametrize("m,n,k", [(16, 12288, 4096), (16, 1024, 4096), (48, 4096, 11008), (16, 1160, 2048)])

@@ -210,10 +210,12 @@ def test_random_mat_mul_tile_shapes(gpu, stream, monkeypatch, sweep):
             big = case % 3 == 0
             if big:
                 monkeypatch.setenv("OPHIP_GEMM_TILE", "256")
+                mm = ophip.MatMul(gpu)  # the knob is read when an operator is created
                 m, n = int(rng.choice([256, 512, 768])), int(rng.choice([256, 512, 1024]))
                 k = int(rng.choice([64, 128, 192, 1088, 2048]))
             else:
                 monkeypatch.delenv("OPHIP_GEMM_TILE", raising=False)
+                mm = ophip.MatMul(gpu)
                 m = int(rng.choice([128, 256, 384, 512, 1024]))
                 n = int(rng.choice([128, 256, 384, 768, 1024]))
                 k = int(rng.choice([32, 64, 96, 192, 1056, 2048]))
@@ -266,6 +268,7 @@ def test_random_mat_mul_ragged_tile_shapes(gpu, stream, monkeypatch, sweep):
                 monkeypatch.setenv("OPHIP_GEMM_TILE", "256")
             else:
                 monkeypatch.delenv("OPHIP_GEMM_TILE", raising=False)
+            mm = ophip.MatMul(gpu)  # the knob is read when an operator is created
             n = 8 * int(rng.integers(9, 90))
             m = 2 * int(rng.integers(33, 350)) + 1 if odd_m else 8 * int(rng.integers(9, 90))
             if case % 2 == 0:
