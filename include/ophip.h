@@ -402,6 +402,16 @@ OPHIP_API int ophip_mat_mul_launch(const ophip_mat_mul *op, const ophip_mat_mul_
                                    void *workspace, size_t workspace_len,
                                    const ophip_queue_alloc *queue_alloc);
 OPHIP_API void ophip_mat_mul_destroy(ophip_mat_mul *op);
+/* No counterpart in the reference.  For callers that cannot allocate device memory (a stream that is
+ * being recorded into a graph, a tight serving loop, a harness that forbids hipMalloc): the same product as
+ * ophip_mat_mul_launch, queued on `stream`, with no workspace argument and no queue allocator.  The split-K
+ * scratch (f32 partials and arrival counters) is a device array inside this library, 32 MiB + 256 KiB, held by
+ * every GPU the library runs on until the process ends; nothing is allocated or freed by the call.  A product
+ * whose partials need more than 32 MiB (ophip_mat_mul_scheme reports the need) is refused with
+ * OPHIP_ARGS_NOT_SUPPORT.  All calls on one GPU share the array: two of them that overlap in time (on
+ * different streams, or from two threads) race; calls on one stream are ordered and safe. */
+OPHIP_API int ophip_mat_mul_launch_static(const ophip_mat_mul *op, const ophip_mat_mul_args *args,
+                                          ophip_stream stream);
 /* Diagnostics, no counterpart in the reference: writes the name of the kernel family launch()
  * would pick for these arguments on this device ("skinny rows<=16 qN split_k=8", "skinny rows<=16 qN paired split_k=1",
  * "skinny rows<=32 qK256 split_k=2", "tile256x64 pK qN split_k=1",

@@ -1,4 +1,5 @@
 #include "handle.hpp"
+#include "static_scratch.hpp"
 #include "../kernels/params.h"
 
 #include <algorithm>
@@ -225,6 +226,7 @@ int ophip_device_create(int ordinal, const ophip_config *cfg, ophip_device **out
             if (std::strncmp(d->props.gcnArchName, "gfx950", 6) != 0)
                 throw execution_failed(std::string("this library carries gfx950 code only, device is ") +
                                        d->props.gcnArchName);
+            static_scratch_resolve(ordinal);  // the device is current: its copy of the library's scratch array
         } catch (...) {
             delete d;
             throw;

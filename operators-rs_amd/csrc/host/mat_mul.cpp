@@ -10,6 +10,7 @@
 
 #include "../kernels/params.h"
 #include "handle.hpp"
+#include "static_scratch.hpp"
 
 using namespace ophip;
 
@@ -407,6 +408,75 @@ struct ophip_mat_mul {
     }
 };
 
+// One launch.  `fixed_counters` null: the ordinary entry point (workspace from the caller or the queue allocator,
+// arrival counters owned by the operator).  Otherwise the caller of this function brings every byte of scratch:
+// `workspace` holds the f32 partials, `fixed_counters` the arrival counters (cleared here, by a kernel, as far as
+// this launch uses them), and nothing is allocated.
+static void mat_mul_launch_impl(const ophip_mat_mul *op, const ophip_mat_mul_args *args, void *workspace,
+                                size_t workspace_len, const ophip_queue_alloc *qa, void *fixed_counters,
+                                size_t fixed_counter_count, hipStream_t stream) {
+    if (!op || !args) throw args_not_support("null argument");
+    const ophip_mat_mul_layout L = mat_mul_layout(*args);
+    if (L.dt != OPHIP_DT_F16 && L.dt != OPHIP_DT_F32) throw type_not_support("mat_mul supports f16 and f32");
+    if (is_dyn(args->alpha) || is_dyn(args->beta)) throw dyn_not_support("");
+    if (L.m == 0 || L.n == 0 || L.batch == 0) return;
+    if (L.m > 0x7fffffffu || L.n > 0x7fffffffu || L.k > 0x7fffffffu || L.batch > 65535)
+        throw shape_not_support("mat_mul dimension too large");
+    GemmPlan g = make_plan(*args, L, (unsigned)op->dev->props.multiProcessorCount, op->knobs);
+    const GemmParams &p = g.p;
+    const bool fixed = fixed_counters != nullptr;
+    if (fixed && g.workspace > workspace_len)
+        throw args_not_support("this product needs " + std::to_string(g.workspace) +
+                               " bytes of split-K scratch, the library's static buffer holds " +
+                               std::to_string(workspace_len));
+    op->dev->make_current();
+    if (g.kind == GemmPlan::Skinny) {
+        Workspace ws(fixed ? nullptr : qa, workspace, workspace_len, g.workspace);
+        g.p.partial = ws.ptr();
+        const size_t tiles = (size_t)((p.N + 127) / 128) * p.batch;
+        if (fixed) {
+            g.p.counters = (p.split_k > 1 && tiles <= fixed_counter_count) ? fixed_counters : nullptr;
+            if (g.p.counters) {  // the static buffer keeps what the last call left: start this launch's counters at zero
+                FillU32Params f{fixed_counters, (uint32_t)tiles, 0u};
+                launch(op->fill, Dim3{(unsigned)((tiles + 255) / 256)}, Dim3{256}, 0, stream, f);
+            }
+        } else {
+            g.p.counters = (p.split_k > 1 && tiles <= SPLITK_COUNTERS) ? op->counters_for(stream) : nullptr;
+        }
+        const int mi = g.mt == 1 ? 0 : g.mt == 2 ? 1 : 2;
+        launch(op->skinny[mi][g.qmode], Dim3{(p.N + 127) / 128, p.split_k, p.batch}, Dim3{256}, 0, stream, g.p);
+        if (p.split_k > 1 && !g.p.counters) {
+            const size_t total = (size_t)p.batch * p.M * (p.N / 8);
+            launch(op->reduce, Dim3{(unsigned)((total + 255) / 256)}, Dim3{256}, 0, stream, g.p);
+        }
+        return;
+    }
+    if (g.kind == GemmPlan::Tile) {
+        Workspace ws(fixed ? nullptr : qa, workspace, workspace_len, g.workspace);
+        g.p.partial = ws.ptr();
+        const unsigned tiles = ((p.M + g.tile - 1) / g.tile) * ((p.N + g.tile - 1) / g.tile);
+        launch(op->tile[g.tile == 256 ? 0 : g.tk == 64 ? 1 : 2][g.ragged][g.pk][g.qk], Dim3{tiles, p.split_k, p.batch}, Dim3{256}, 0,
+               stream, g.p);
+        if (p.split_k > 1) {
+            const size_t total = (size_t)p.batch * p.M * (p.N / 8);
+            launch(op->reduce, Dim3{(unsigned)((total + 255) / 256)}, Dim3{256}, 0, stream, g.p);
+        }
+        return;
+    }
+    const unsigned gx = (p.N + 63) / 64, gy = (p.M + 63) / 64;
+    if (gy > 65535) throw shape_not_support("mat_mul dimension too large for the generic kernel");
+    launch(L.dt == OPHIP_DT_F16 ? op->generic_f16 : op->generic_f32, Dim3{gx, gy, p.batch}, Dim3{256}, 0, stream,
+           g.p);
+}
+
+namespace ophip {
+void mat_mul_launch_fixed_scratch(const ophip_mat_mul *op, const ophip_mat_mul_args *args, void *partials,
+                                  size_t partial_bytes, void *counters, size_t counter_count, hipStream_t stream) {
+    mat_mul_launch_impl(op, args, partials, partial_bytes, nullptr, counters, counter_count, stream);
+}
+const ophip_device *mat_mul_device(const ophip_mat_mul *op) { return op->dev; }
+}  // namespace ophip
+
 extern "C" {
 
 int ophip_mat_mul_plan(const ophip_mat_mul_args *args, ophip_mat_mul_layout *out) {
@@ -460,47 +530,7 @@ int ophip_mat_mul_describe(const ophip_mat_mul *op, const ophip_mat_mul_args *ar
 
 int ophip_mat_mul_launch(const ophip_mat_mul *op, const ophip_mat_mul_args *args, void *workspace,
                          size_t workspace_len, const ophip_queue_alloc *qa) {
-    return guard([&] {
-        const ophip_mat_mul_layout L = mat_mul_layout(*args);
-        if (L.dt != OPHIP_DT_F16 && L.dt != OPHIP_DT_F32) throw type_not_support("mat_mul supports f16 and f32");
-        if (is_dyn(args->alpha) || is_dyn(args->beta)) throw dyn_not_support("");
-        if (L.m == 0 || L.n == 0 || L.batch == 0) return;
-        if (L.m > 0x7fffffffu || L.n > 0x7fffffffu || L.k > 0x7fffffffu || L.batch > 65535)
-            throw shape_not_support("mat_mul dimension too large");
-        GemmPlan g = make_plan(*args, L, (unsigned)op->dev->props.multiProcessorCount, op->knobs);
-        const GemmParams &p = g.p;
-        hipStream_t stream = stream_of(qa);
-        op->dev->make_current();
-        if (g.kind == GemmPlan::Skinny) {
-            Workspace ws(qa, workspace, workspace_len, g.workspace);
-            g.p.partial = ws.ptr();
-            const size_t tiles = (size_t)((p.N + 127) / 128) * p.batch;
-            g.p.counters = (p.split_k > 1 && tiles <= SPLITK_COUNTERS) ? op->counters_for(stream) : nullptr;
-            const int mi = g.mt == 1 ? 0 : g.mt == 2 ? 1 : 2;
-            launch(op->skinny[mi][g.qmode], Dim3{(p.N + 127) / 128, p.split_k, p.batch}, Dim3{256}, 0, stream, g.p);
-            if (p.split_k > 1 && !g.p.counters) {
-                const size_t total = (size_t)p.batch * p.M * (p.N / 8);
-                launch(op->reduce, Dim3{(unsigned)((total + 255) / 256)}, Dim3{256}, 0, stream, g.p);
-            }
-            return;
-        }
-        if (g.kind == GemmPlan::Tile) {
-            Workspace ws(qa, workspace, workspace_len, g.workspace);
-            g.p.partial = ws.ptr();
-            const unsigned tiles = ((p.M + g.tile - 1) / g.tile) * ((p.N + g.tile - 1) / g.tile);
-            launch(op->tile[g.tile == 256 ? 0 : g.tk == 64 ? 1 : 2][g.ragged][g.pk][g.qk], Dim3{tiles, p.split_k, p.batch}, Dim3{256}, 0,
-                   stream, g.p);
-            if (p.split_k > 1) {
-                const size_t total = (size_t)p.batch * p.M * (p.N / 8);
-                launch(op->reduce, Dim3{(unsigned)((total + 255) / 256)}, Dim3{256}, 0, stream, g.p);
-            }
-            return;
-        }
-        const unsigned gx = (p.N + 63) / 64, gy = (p.M + 63) / 64;
-        if (gy > 65535) throw shape_not_support("mat_mul dimension too large for the generic kernel");
-        launch(L.dt == OPHIP_DT_F16 ? op->generic_f16 : op->generic_f32, Dim3{gx, gy, p.batch}, Dim3{256}, 0, stream,
-               g.p);
-    });
+    return guard([&] { mat_mul_launch_impl(op, args, workspace, workspace_len, qa, nullptr, 0, stream_of(qa)); });
 }
 
 }  // extern "C"

@@ -222,7 +222,7 @@ EXPORTS = [
     "ophip_random_sample_create", "ophip_random_sample_scheme", "ophip_random_sample_launch",
     "ophip_random_sample_destroy", "ophip_random_sample_build_indices", "ophip_random_sample_launch_batch",
     "ophip_mat_mul_plan", "ophip_mat_mul_create", "ophip_mat_mul_scheme", "ophip_mat_mul_launch",
-    "ophip_mat_mul_destroy", "ophip_mat_mul_describe",
+    "ophip_mat_mul_destroy", "ophip_mat_mul_describe", "ophip_mat_mul_launch_static",
     "ophip_attention_create", "ophip_attention_scheme", "ophip_attention_launch", "ophip_attention_destroy",
     "ophip_attention_kv_cached_create", "ophip_attention_kv_cached_scheme", "ophip_attention_kv_cached_launch",
     "ophip_attention_kv_cached_destroy",
@@ -859,3 +859,7 @@ class MatMul(_Operator):
         buf = ctypes.create_string_buffer(96)
         _check(lib().ophip_mat_mul_describe(self.handle, ctypes.byref(args.c()), buf, ctypes.c_size_t(96)))
         return buf.value.decode()
+
+    def launch_static(self, args, stream):
+        """The same product with the library's own scratch array: no workspace, no allocator, nothing allocated."""
+        _check(lib().ophip_mat_mul_launch_static(self.handle, ctypes.byref(args.c()), stream.handle), launch=True)
