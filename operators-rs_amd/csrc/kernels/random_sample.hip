@@ -252,8 +252,41 @@ __device__ __forceinline__ uint32_t comp_idx(uint64_t c) { return 0xffffffffu - 
 
 __device__ __forceinline__ float row_seed(const SampleParams &p) { return p.seeds ? p.seeds[blockIdx.x] : p.seed; }
 
-// exp() the way a correctly rounded expf would return it
-__device__ __forceinline__ float exp_cr(float x) { return (float)exp((double)x); }
+// expf() as the host's C library computes it, bit for bit: the reference's f32::exp is libm's expf, which is
+// not correctly rounded (it differs from the rounded exact value on about 1 input in 11 500).  This is the
+// published algorithm of glibc's expf (sysdeps/ieee754/flt-32/e_expf.c, from ARM's optimized routines): x * 32 / ln 2 =
+// k + r, a 32-entry table of 2^(i/32) and a cubic in r, all in f64; as built for x86-64 the remainder r is one fused
+// multiply-add.  Equal to the host's expf on every f32 in [-103, -0] (1 120 796 673 inputs, checked on the CPU).
+static __device__ const uint64_t EXPF_TAB[32] = {
+    0x3ff0000000000000, 0x3fefd9b0d3158574, 0x3fefb5586cf9890f, 0x3fef9301d0125b51, 0x3fef72b83c7d517b,
+    0x3fef54873168b9aa, 0x3fef387a6e756238, 0x3fef1e9df51fdee1, 0x3fef06fe0a31b715, 0x3feef1a7373aa9cb,
+    0x3feedea64c123422, 0x3feece086061892d, 0x3feebfdad5362a27, 0x3feeb42b569d4f82, 0x3feeab07dd485429,
+    0x3feea47eb03a5585, 0x3feea09e667f3bcd, 0x3fee9f75e8ec5f74, 0x3feea11473eb0187, 0x3feea589994cce13,
+    0x3feeace5422aa0db, 0x3feeb737b0cdc5e5, 0x3feec49182a3f090, 0x3feed503b23e255d, 0x3feee89f995ad3ad,
+    0x3feeff76f2fb5e47, 0x3fef199bdd85529c, 0x3fef3720dcef9069, 0x3fef5818dcfba487, 0x3fef7c97337b9b5f,
+    0x3fefa4afa2a490da, 0x3fefd0765b6e4540,
+};
+__device__ __forceinline__ float expf_libm(float x) {
+#pragma clang fp contract(off)
+    if (x < -0x1.9fe368p6f) return 0.f;  // below log(2^-150): libm's underflow result
+    if (x > 0x1.62e42ep6f) return INFINITY;
+    constexpr double INV_LN2_N = 0x1.71547652b82fep+0 * 32, SHIFT = 0x1.8p+52;
+    constexpr double C0 = 0x1.c6af84b912394p-5 / 32 / 32 / 32, C1 = 0x1.ebfce50fac4f3p-3 / 32 / 32,
+                     C2 = 0x1.62e42ff0c52d6p-1 / 32;
+    const double xd = (double)x;
+    const double z = INV_LN2_N * xd;
+    double kd = z + SHIFT;  // round to nearest integer: the low bits of kd's encoding hold it
+    const uint64_t ki = (uint64_t)__double_as_longlong(kd);
+    kd -= SHIFT;
+    const double r = __builtin_fma(INV_LN2_N, xd, -kd);
+    const double sc = __longlong_as_double((long long)(EXPF_TAB[ki & 31u] + (ki << 47)));
+    const double q = __builtin_fma(C0, r, C1);
+    const double r2 = r * r;
+    double y = __builtin_fma(C2, r, 1.0);
+    y = __builtin_fma(q, r2, y);
+    y = y * sc;
+    return (float)y;
+}
 
 __device__ __forceinline__ float block_sum_f32(float v, float *smem) {
     v = wave_sum(v);
@@ -268,7 +301,8 @@ __device__ __forceinline__ float block_sum_f32(float v, float *smem) {
 
 // Descending bitonic network over `cnt` (power of two) u64 values in LDS, all
 // (k2, j) stages with k2 from k2_first and j <= j_first for the first k2.
-__device__ __forceinline__ void bitonic_lds(uint64_t *a, uint32_t cnt, uint32_t k2_first,
+template <typename K>
+__device__ __forceinline__ void bitonic_lds(K *a, uint32_t cnt, uint32_t k2_first,
                                             uint32_t k2_last, uint32_t j_cap, uint32_t base) {
     for (uint32_t k2 = k2_first; k2 <= k2_last; k2 <<= 1) {
         uint32_t j = k2 >> 1;
@@ -278,7 +312,7 @@ __device__ __forceinline__ void bitonic_lds(uint64_t *a, uint32_t cnt, uint32_t 
                 const uint32_t i = 2 * t - (t & (j - 1));
                 const uint32_t l = i + j;
                 const bool desc = (((base + i) & k2) == 0);
-                const uint64_t x = a[i], y = a[l];
+                const K x = a[i], y = a[l];
                 if ((x < y) == desc) {
                     a[i] = y;
                     a[l] = x;
@@ -389,6 +423,267 @@ __device__ __forceinline__ void sort_desc_256(uint64_t *a, uint32_t cnt) {
     __syncthreads();
 }
 
+// ---- the total over all n entries, as the reference's sequential sum gives it -----------------------------------
+//
+// The reference's top_p bound is top_p * cum[n-1], the last of its sequential f32 running sums over the sorted
+// row.  The kernels sum the row in parallel instead, so they only know an interval [T_lo, T_hi] that holds
+// cum[n-1]; the sampled entry is a monotone function of that total, so when both ends of the interval give the same
+// entry the row is settled.  Three stages, each run only by the rows the stage before could not settle:
+//   0. hardware-exp2 parallel f32 sum F; cum[n-1] lies within n * 2^-24 (sequential rounding) + 6e-5 (the fast
+//      exponentials and the parallel sum) of it, relatively;
+//   1. the exact terms e_i (libm's expf) summed in f64, S, and E = sum of min(e_i, 2^-24 * T_hi): one sequential
+//      addition errs by at most half an ulp of the running sum, and by the term itself when that is smaller, so
+//      |cum[n-1] - S| <= E;
+//   2. the sequential sum itself, continued from cum[k-1] over the entries behind the k candidates in sorted
+//      order (sample_exact_total below).
+struct TotalBounds {
+    float lo, hi;
+};
+__device__ __forceinline__ float f32_not_above(double x) {
+    float f = (float)x;
+    if ((double)f > x) f = __uint_as_float(__float_as_uint(f) - 1u);  // x >= 1 here: positive, normal
+    return f;
+}
+__device__ __forceinline__ float f32_not_below(double x) {
+    float f = (float)x;
+    if ((double)f < x) f = __uint_as_float(__float_as_uint(f) + 1u);
+    return f;
+}
+__device__ __forceinline__ TotalBounds bounds_from_fast_sum(float F, uint32_t n) {
+    const double seq = (double)n * 0x1p-24 * 1.001, par = 6e-5;
+    TotalBounds b;
+    b.lo = seq < 0.5 ? fmaxf(1.0f, f32_not_above((double)F / (1.0 + par) * (1.0 - seq))) : 1.0f;
+    b.hi = seq < 0.5 ? f32_not_below((double)F / (1.0 - par) * (1.0 + seq)) : INFINITY;
+    if (!(F == F)) b.lo = 1.0f, b.hi = INFINITY;
+    return b;
+}
+
+__device__ __forceinline__ double block_sum_f64(double v, double *smem) {
+#pragma unroll
+    for (int o = WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+    __syncthreads();
+    if ((threadIdx.x & (WAVE - 1)) == 0) smem[threadIdx.x / WAVE] = v;
+    __syncthreads();
+    double r = 0.0;
+#pragma unroll
+    for (int i = 0; i < SB / WAVE; ++i) r += smem[i];
+    return r;
+}
+
+constexpr uint32_t XCH = 4096;  // entries sample_exact_total sorts per round
+// LDS the later stages work in (the caller's histogram arrays serve again)
+struct TotalScratch {
+    uint32_t *hist;            // [256]
+    uint32_t (*hist_w)[256];   // [SB / WAVE][256]
+    uint32_t *wtot;            // [4]
+    uint32_t *sel;             // [2]
+    uint32_t *cnt;             // [1]
+    uint32_t *keys;            // [XCH]
+    double *red;               // [SB / WAVE]
+    float *fl;                 // [2]
+};
+
+// Stage 1: the exact terms summed in f64 and the bound on what the sequential f32 sum can lose or gain against that
+// (`t_hi`: the stage-0 upper bound of the total).  All threads call; every thread gets the interval.
+// (Like sample_exact_total a function of its own that reads the row from memory: the callers' common path
+// carries neither its code nor its registers.)
+template <typename T>
+__device__ __noinline__ TotalBounds sample_total_bounds(const char *row, uint32_t n, float mx, float t, float t_hi,
+                                                        TotalScratch s) {
+    typedef Logit<T> L;
+    const double h = (double)t_hi * 0x1p-24 * (1.0 + 1e-6);
+    double sum = 0.0, err = 0.0;
+    for_each_logit<T>(row, n, [&](uint32_t, uint32_t bits) {
+        const double e = (double)expf_libm((L::value(bits) - mx) / t);
+        sum += e;
+        err += e < h ? e : h;
+    });
+    sum = block_sum_f64(sum, s.red);
+    err = block_sum_f64(err, s.red);
+    TotalBounds b;
+    b.lo = fmaxf(1.0f, f32_not_above((sum - err) * (1.0 - 1e-9)));
+    b.hi = f32_not_below((sum + err) * (1.0 + 1e-9));
+    if (!(sum == sum) || !(err == err)) b.lo = 1.0f, b.hi = INFINITY;
+    return b;
+}
+
+// The reference's sequential sum continued: `c` is cum[k-1]; behind the k candidates come `leftover` more entries
+// with the k-th key and then every entry whose key is below it, in descending order.  Rounds of up to XCH keys:
+// radix-select the XCH-th largest key still below `hi`, gather the keys above it, sort them in LDS, and let
+// wave 0 add their terms one after another; the entries with the selected key itself (any number of them) are one
+// term added that many times.  The sum stops early once a term no longer changes it: every later term is
+// smaller and the sum only grows.  All threads call; every thread gets the total.
+template <typename T>
+__device__ __noinline__ float sample_exact_total(const char *row, uint32_t n, float c, uint32_t kstar, uint32_t leftover,
+                                                 float mx, float t, TotalScratch s) {
+    typedef Logit<T> L;
+    // (the row is read from memory here even when the caller holds it in registers: this is a function of its
+    // own so that its code and its registers stay out of the callers' common path)
+    auto each_key = [&](auto &&f) { for_each_logit<T>(row, n, [&](uint32_t, uint32_t bits) { f(L::key(bits)); }); };
+    auto term = [&](uint32_t key) { return expf_libm((L::value(L::unkey(key)) - mx) / t); };
+    // `count` times the same term, by every lane of wave 0 alike; false once the sum no longer moves
+    auto add_run = [&](float e, uint32_t count) {
+        for (uint32_t i = 0; i < count; ++i) {
+            const float nc = c + e;
+            if (nc == c) return false;
+            c = nc;
+        }
+        return true;
+    };
+    const bool wave0 = threadIdx.x < WAVE;
+    const uint32_t lane = threadIdx.x % WAVE;
+    bool moving = true;  // (meaningful in wave 0)
+    if (wave0 && leftover) moving = add_run(term(kstar), leftover);
+    uint32_t hi = kstar;  // keys below `hi` are still to come
+    for (;;) {
+        if (wave0 && lane == 0) s.fl[0] = moving ? 1.f : 0.f;
+        __syncthreads();
+        if (s.fl[0] == 0.f || hi == 0) break;
+        // the XCH-th largest key below hi, digit by digit; the first digit's histogram also counts what is left
+        uint32_t prefix = 0, krem = XCH, eq_count = 0, left = 0;
+        bool all = false;  // XCH or fewer left: this round takes them all
+        for (int shift = L::KEY_BITS - 8; shift >= 0 && !all; shift -= 8) {
+            for (uint32_t i = threadIdx.x; i < (SB / WAVE) * 256; i += SB) (&s.hist_w[0][0])[i] = 0;
+            __syncthreads();
+            const bool first = shift == L::KEY_BITS - 8;
+            const uint32_t hi_mask = first ? 0u : (0xffffffffu << (shift + 8));
+            uint32_t *my_hist = s.hist_w[threadIdx.x / WAVE];
+            each_key([&](uint32_t key) {
+                if (key < hi && ((key ^ prefix) & hi_mask) == 0) atomicAdd(&my_hist[(key >> shift) & 255u], 1u);
+            });
+            __syncthreads();
+            if (threadIdx.x < 256) {
+                uint32_t cnt = 0;
+#pragma unroll
+                for (int w = 0; w < SB / WAVE; ++w) cnt += s.hist_w[w][threadIdx.x];
+                s.hist[threadIdx.x] = cnt;
+            }
+            __syncthreads();
+            if (first) {
+                for (uint32_t i = 0; i < 256; ++i) left += s.hist[i];
+                if (left <= XCH) {
+                    all = true;
+                    break;
+                }
+            }
+            pick_bucket(s.hist, krem, true, s.wtot, s.sel);
+            prefix |= s.sel[0] << shift;
+            krem = s.sel[1];
+            eq_count = s.hist[s.sel[0]];
+            __syncthreads();
+        }
+        if (left == 0) break;
+        const uint32_t lo = all ? 0u : prefix;  // gather lo < key < hi (all: every key below hi)
+        uint32_t P = 64;
+        const uint32_t expect = all ? left : XCH - krem;
+        while (P < expect) P <<= 1;
+        if (threadIdx.x == 0) *s.cnt = 0;
+        for (uint32_t i = threadIdx.x; i < P; i += SB) s.keys[i] = 0;
+        __syncthreads();
+        each_key([&](uint32_t key) {
+            if (key < hi && (all || key > lo)) {
+                const uint32_t slot = atomicAdd(s.cnt, 1u);
+                if (slot < XCH) s.keys[slot] = key;
+            }
+        });
+        __syncthreads();
+        const uint32_t cnt = min(*s.cnt, XCH);
+        if (P <= 64) {
+            if (wave0) {  // one value per lane, sorted by shuffles
+                uint32_t x = s.keys[lane];
+#pragma unroll
+                for (int k2 = 2; k2 <= WAVE; k2 <<= 1)
+#pragma unroll
+                    for (int j = k2 >> 1; j > 0; j >>= 1) {
+                        const uint32_t y = __shfl_xor(x, j, WAVE);
+                        const bool desc = (lane & k2) == 0, lower = (lane & j) == 0;
+                        x = (lower == desc) ? max(x, y) : min(x, y);
+                    }
+                s.keys[lane] = x;
+            }
+            __syncthreads();
+        } else {
+            bitonic_lds(s.keys, P, 2, P, P, 0);
+        }
+        if (wave0) {
+            for (uint32_t base = 0; base < cnt && moving; base += WAVE) {
+                const float e = base + lane < cnt ? term(s.keys[base + lane]) : 0.f;
+                const float e0 = __shfl(e, 0, WAVE);
+                if (c + e0 == c) {  // the largest term left no longer moves the sum
+                    moving = false;
+                    break;
+                }
+#pragma unroll
+                for (int i = 0; i < WAVE; ++i) c = c + __shfl(e, i, WAVE);
+            }
+            if (moving && !all) moving = add_run(term(lo), eq_count);
+        }
+        if (all) break;
+        hi = lo;
+    }
+    __syncthreads();
+    if (wave0 && lane == 0) s.fl[1] = c;
+    __syncthreads();
+    return s.fl[1];
+}
+
+// Stages 0 to 2 for one row whose k candidates are sorted and summed.  Wave 0 holds the running sums: find(plimit)
+// returns the first candidate whose running sum reaches plimit (k - 1 if none), emit(i) writes candidate i as the
+// row's result; both are called by all lanes of wave 0 only.  `pk` is cum[k-1] (valid in wave 0), `fast_total`
+// the stage-0 sum.  All threads call.
+template <typename T, typename Find, typename Emit>
+__device__ __forceinline__ void sample_settle(const SampleParams &p, const char *row, float fast_total, float mx, float pk,
+                                              uint32_t k, uint32_t kstar, uint32_t leftover, Find &&find, Emit &&emit,
+                                              const TotalScratch &s, uint32_t *s_state) {
+    typedef Logit<T> L;
+    const bool wave0 = threadIdx.x < WAVE;
+    const uint32_t lane = threadIdx.x % WAVE;
+    const float seed = row_seed(p), top_p = p.top_p, t = p.temperature;
+    // wave 0: 1 = the row is settled (result written, or left to the next kernel in line), 0 = the interval is too wide
+    auto judge = [&](float t_lo, float t_hi) -> uint32_t {
+        const float pp_lo = t_lo * top_p, pp_hi = t_hi * top_p;
+        if (p.verify_cover & 1) {  // k stands in for a larger top_k: do these candidates hold top_p of the mass?
+            if (pk < pp_lo) {
+                if (lane == 0) *reinterpret_cast<uint32_t *>(sample_row_workspace(p)) = 1u;  // no: the next kernel does the row
+                return 1u;
+            }
+            if (!(pk >= pp_hi)) return 0u;
+        }
+        const float pl_lo = seed * fminf(pk, pp_lo), pl_hi = seed * fminf(pk, pp_hi);
+        const uint32_t a_lo = find(pl_lo);
+        const uint32_t a_hi = pl_hi == pl_lo ? a_lo : find(pl_hi);
+        if (a_lo != a_hi) return 0u;
+        if ((p.verify_cover & 1) && lane == 0) *reinterpret_cast<uint32_t *>(sample_row_workspace(p)) = 0u;
+        emit(a_lo);
+        return 1u;
+    };
+    const TotalBounds b0 = bounds_from_fast_sum(fast_total, p.n);
+    if (wave0) {
+        const uint32_t done = judge(b0.lo, b0.hi);
+        if (lane == 0) *s_state = done;
+    }
+    __syncthreads();
+    if (__builtin_expect(*s_state != 0, 1)) return;
+    __syncthreads();
+
+    // stage 1
+    const TotalBounds b1 = sample_total_bounds<T>(row, p.n, mx, t, b0.hi, s);
+    if (wave0) {
+        const uint32_t done = judge(b1.lo, b1.hi);
+        if (lane == 0) *s_state = done;
+    }
+    __syncthreads();
+    if (__builtin_expect(*s_state != 0, 1)) return;
+    __syncthreads();
+
+    // stage 2
+    const float pk_all = __shfl(pk, 0, WAVE);  // (wave 0's; the other waves' copy is not used)
+    if (wave0 && lane == 0) s.fl[1] = pk_all;
+    __syncthreads();
+    const float total = sample_exact_total<T>(row, p.n, s.fl[1], kstar, leftover, mx, t, s);
+    if (wave0) (void)judge(total, total);
+}
+
 // SMALLK: top_k <= 64, the common case (sort, prefix and search in the registers of wave 0) as a kernel of its own:
 // it is short, and the code of the general case beside it cost it 3 % even unexecuted.
 template <typename T, bool SMALLK>
@@ -404,6 +699,10 @@ __device__ __forceinline__ void sample_topk_impl(const SampleParams &p) {
     __shared__ float s_cum[KC];
     __shared__ float s_red[SB / WAVE];
     __shared__ float s_mx;
+    __shared__ uint32_t s_xkeys[XCH];
+    __shared__ double s_xred[SB / WAVE];
+    __shared__ float s_xfl[2];
+    __shared__ uint32_t s_state;
 
     if constexpr (!SMALLK)
         if (sample_row_done(p)) return;
@@ -486,6 +785,10 @@ __device__ __forceinline__ void sample_topk_impl(const SampleParams &p) {
     __syncthreads();
 
     const float t = p.temperature;
+    const uint32_t leftover = eq_count - krem;  // entries with the k-th key that are not among the candidates
+    TotalScratch scratch;
+    scratch.hist = hist, scratch.hist_w = hist_w, scratch.wtot = s_wtot, scratch.sel = s_sel, scratch.cnt = &s_cnt;
+    scratch.keys = s_xkeys, scratch.red = s_xred, scratch.fl = s_xfl;
     if (SMALLK || P == 64) {
         // k <= 64: sort, prefix and search live in the registers of wave 0
         const uint32_t lane = threadIdx.x % WAVE;
@@ -505,37 +808,37 @@ __device__ __forceinline__ void sample_topk_impl(const SampleParams &p) {
         __syncthreads();
         const float mx = s_mx;
         float part = 0.f;
-        // the total only feeds the top_p bound: hardware exp2 and a reciprocal keep this sweep cheap
+        // stage 0 of the total (see sample_settle): hardware exp2 and a reciprocal keep this sweep cheap
         const float inv_t = 1.0f / t;
         rc.for_each(row, n, [&](uint32_t, uint32_t bits) { part += fast_exp((L::value(bits) - mx) * inv_t); });
         const float total = block_sum_f32(part, s_red);
+        float mine = 1.0f, pk = 1.0f;
         if (threadIdx.x < WAVE) {
             float e = 0.f;
-            if (lane > 0 && lane < k) e = exp_cr((L::value(L::unkey(comp_key(x))) - mx) / t);
+            if (lane > 0 && lane < k) e = expf_libm((L::value(L::unkey(comp_key(x))) - mx) / t);
             // cum[i] = cum[i-1] + e[i], strictly in order, every lane replaying the same chain
-            float c = 1.0f, mine = 1.0f;
+            float c = 1.0f;
 #pragma unroll
             for (int i = 1; i < WAVE; ++i) {
                 c = c + __shfl(e, i, WAVE);
                 if (lane == (uint32_t)i) mine = c;
             }
-            const float pk = c;  // terms past k are zero, so the chain ends at cum[k-1]
-            if constexpr (!SMALLK) {
-                if (p.verify_cover & 1) {  // k stands in for a larger top_k: do these candidates hold top_p of the mass?
-                    const bool uncovered = pk < total * p.top_p;
-                    if (lane == 0) *reinterpret_cast<uint32_t *>(sample_row_workspace(p)) = uncovered ? 1u : 0u;
-                    if (uncovered) return;  // the next kernel in line does this row
-                }
-            }
-            const float plimit = row_seed(p) * fminf(pk, total * p.top_p);
-            const uint64_t hit = __ballot(lane < k && mine >= plimit);
-            const uint32_t ans = hit ? (uint32_t)__ffsll((long long)hit) - 1 : k - 1;
-            if (lane == ans) {
-                KvPair *out = reinterpret_cast<KvPair *>(p.kv) + blockIdx.x;
-                out->idx = comp_idx(x);
-                out->val = L::from_f32(mine);
-            }
+            pk = c;  // terms past k are zero, so the chain ends at cum[k-1]
         }
+        sample_settle<T>(
+            p, row, total, mx, pk, k, kstar, leftover,
+            [&](float plimit) {
+                const uint64_t hit = __ballot(lane < k && mine >= plimit);
+                return hit ? (uint32_t)__ffsll((long long)hit) - 1 : k - 1;
+            },
+            [&](uint32_t ans) {
+                if (lane == ans) {
+                    KvPair *out = reinterpret_cast<KvPair *>(p.kv) + blockIdx.x;
+                    out->idx = comp_idx(x);
+                    out->val = L::from_f32(mine);
+                }
+            },
+            scratch, &s_state);
         return;
     }
 
@@ -549,11 +852,12 @@ __device__ __forceinline__ void sample_topk_impl(const SampleParams &p) {
         rc.for_each(row, n, [&](uint32_t, uint32_t bits) { part += fast_exp((L::value(bits) - mx) * inv_t); });
         const float total = block_sum_f32(part, s_red);
         for (uint32_t i = threadIdx.x; i < P; i += SB)
-            s_cum[i] = i == 0 ? 1.0f : i < k ? exp_cr((L::value(L::unkey(comp_key(cand[i]))) - mx) / t) : 0.f;
+            s_cum[i] = i == 0 ? 1.0f : i < k ? expf_libm((L::value(L::unkey(comp_key(cand[i]))) - mx) / t) : 0.f;
         __syncthreads();
+        const uint32_t lane = threadIdx.x % WAVE;
+        float pk = 1.0f;
         if (threadIdx.x < WAVE) {
             // wave 0 replays the sequential sum 64 entries at a time, carrying the running value
-            const uint32_t lane = threadIdx.x;
             float c = 0.f;
             for (uint32_t base = 0; base < P; base += WAVE) {
                 const float e = s_cum[base + lane];
@@ -565,27 +869,25 @@ __device__ __forceinline__ void sample_topk_impl(const SampleParams &p) {
                 }
                 s_cum[base + lane] = mine;
             }
-            const float pk = c;  // entries past k add zero
-            if (p.verify_cover & 1) {  // k stands in for a larger top_k: do these candidates hold top_p of the mass?
-                const bool uncovered = pk < total * p.top_p;
-                if (lane == 0) *reinterpret_cast<uint32_t *>(sample_row_workspace(p)) = uncovered ? 1u : 0u;
-                if (uncovered) return;  // the full-sort kernel does this row
-            }
-            const float plimit = row_seed(p) * fminf(pk, total * p.top_p);
-            uint32_t ans = k - 1;
-            for (uint32_t base = 0; base < P; base += WAVE) {
-                const uint64_t hit = __ballot(base + lane < k && s_cum[base + lane] >= plimit);
-                if (hit) {
-                    ans = base + (uint32_t)__ffsll((long long)hit) - 1;
-                    break;
-                }
-            }
-            if (lane == 0) {
-                KvPair *out = reinterpret_cast<KvPair *>(p.kv) + blockIdx.x;
-                out->idx = comp_idx(cand[ans]);
-                out->val = L::from_f32(s_cum[ans]);
-            }
+            pk = c;  // entries past k add zero
         }
+        sample_settle<T>(
+            p, row, total, mx, pk, k, kstar, leftover,
+            [&](float plimit) {
+                for (uint32_t base = 0; base < P; base += WAVE) {
+                    const uint64_t hit = __ballot(base + lane < k && s_cum[base + lane] >= plimit);
+                    if (hit) return base + (uint32_t)__ffsll((long long)hit) - 1;
+                }
+                return k - 1;
+            },
+            [&](uint32_t ans) {
+                if (lane == 0) {
+                    KvPair *out = reinterpret_cast<KvPair *>(p.kv) + blockIdx.x;
+                    out->idx = comp_idx(cand[ans]);
+                    out->val = L::from_f32(s_cum[ans]);
+                }
+            },
+            scratch, &s_state);
     }
 }
 
@@ -618,6 +920,10 @@ __device__ __forceinline__ void sample_topk_list_impl(const SampleParams &p) {
     __shared__ float s_cum[KC];
     __shared__ float s_red[SB / WAVE];
     __shared__ uint32_t s_kmax[SB / WAVE];
+    __shared__ uint32_t s_xkeys[XCH];
+    __shared__ double s_xred[SB / WAVE];
+    __shared__ float s_xfl[2];
+    __shared__ uint32_t s_state;
     const uint32_t k = p.k_eff;
     const float t = p.temperature, inv_t = 1.0f / t;
 
@@ -741,10 +1047,15 @@ __device__ __forceinline__ void sample_topk_list_impl(const SampleParams &p) {
         total = block_sum_f32(part, s_red);
     }
 
+    const uint32_t leftover = eq_count - krem;  // entries with the k-th key that are not among the candidates
+    TotalScratch scratch;
+    scratch.hist = hist, scratch.hist_w = hist_w, scratch.wtot = s_wtot, scratch.sel = s_sel, scratch.cnt = &s_cnt;
+    scratch.keys = s_xkeys, scratch.red = s_xred, scratch.fl = s_xfl;
+    const uint32_t lane = threadIdx.x % WAVE;
     if (P == 64) {
         // k <= 64: sort, prefix and search live in the registers of wave 0
-        const uint32_t lane = threadIdx.x % WAVE;
         uint64_t x = 0;
+        float mine = 1.0f, pk = 1.0f;
         if (threadIdx.x < WAVE) {
             x = cand[lane];
 #pragma unroll
@@ -755,32 +1066,31 @@ __device__ __forceinline__ void sample_topk_list_impl(const SampleParams &p) {
                     const bool desc = (lane & k2) == 0, lower = (lane & j) == 0;
                     x = (lower == desc) ? (x > y ? x : y) : (x < y ? x : y);
                 }
-        }
-        if (threadIdx.x < WAVE) {
             float e = 0.f;
-            if (lane > 0 && lane < k) e = exp_cr((L::value(L::unkey(comp_key(x))) - mx) / t);
+            if (lane > 0 && lane < k) e = expf_libm((L::value(L::unkey(comp_key(x))) - mx) / t);
             // cum[i] = cum[i-1] + e[i], strictly in order, every lane replaying the same chain
-            float c = 1.0f, mine = 1.0f;
+            float c = 1.0f;
 #pragma unroll
             for (int i = 1; i < WAVE; ++i) {
                 c = c + __shfl(e, i, WAVE);
                 if (lane == (uint32_t)i) mine = c;
             }
-            const float pk = c;  // terms past k are zero, so the chain ends at cum[k-1]
-            if (p.verify_cover & 1) {  // k stands in for a larger top_k: do these candidates hold top_p of the mass?
-                const bool uncovered = pk < total * p.top_p;
-                if (lane == 0) *reinterpret_cast<uint32_t *>(sample_row_workspace(p)) = uncovered ? 1u : 0u;
-                if (uncovered) return;  // the next kernel in line does this row
-            }
-            const float plimit = row_seed(p) * fminf(pk, total * p.top_p);
-            const uint64_t hit = __ballot(lane < k && mine >= plimit);
-            const uint32_t ans = hit ? (uint32_t)__ffsll((long long)hit) - 1 : k - 1;
-            if (lane == ans) {
-                KvPair *out = reinterpret_cast<KvPair *>(p.kv) + blockIdx.x;
-                out->idx = comp_idx(x);
-                out->val = L::from_f32(mine);
-            }
+            pk = c;  // terms past k are zero, so the chain ends at cum[k-1]
         }
+        sample_settle<T>(
+            p, row, total, mx, pk, k, kstar, leftover,
+            [&](float plimit) {
+                const uint64_t hit = __ballot(lane < k && mine >= plimit);
+                return hit ? (uint32_t)__ffsll((long long)hit) - 1 : k - 1;
+            },
+            [&](uint32_t ans) {
+                if (lane == ans) {
+                    KvPair *out = reinterpret_cast<KvPair *>(p.kv) + blockIdx.x;
+                    out->idx = comp_idx(x);
+                    out->val = L::from_f32(mine);
+                }
+            },
+            scratch, &s_state);
         return;
     }
 
@@ -788,11 +1098,11 @@ __device__ __forceinline__ void sample_topk_list_impl(const SampleParams &p) {
     else bitonic_lds(cand, P, 2, P, P, 0);
     // 3. running sums
     for (uint32_t i = threadIdx.x; i < P; i += SB)
-        s_cum[i] = i == 0 ? 1.0f : i < k ? exp_cr((L::value(L::unkey(comp_key(cand[i]))) - mx) / t) : 0.f;
+        s_cum[i] = i == 0 ? 1.0f : i < k ? expf_libm((L::value(L::unkey(comp_key(cand[i]))) - mx) / t) : 0.f;
     __syncthreads();
+    float pk = 1.0f;
     if (threadIdx.x < WAVE) {
         // wave 0 replays the sequential sum 64 entries at a time, carrying the running value
-        const uint32_t lane = threadIdx.x;
         float c = 0.f;
         for (uint32_t base = 0; base < P; base += WAVE) {
             const float e = s_cum[base + lane];
@@ -804,27 +1114,25 @@ __device__ __forceinline__ void sample_topk_list_impl(const SampleParams &p) {
             }
             s_cum[base + lane] = mine;
         }
-        const float pk = c;  // entries past k add zero
-        if (p.verify_cover & 1) {  // k stands in for a larger top_k: do these candidates hold top_p of the mass?
-            const bool uncovered = pk < total * p.top_p;
-            if (lane == 0) *reinterpret_cast<uint32_t *>(sample_row_workspace(p)) = uncovered ? 1u : 0u;
-            if (uncovered) return;  // the full-sort kernel does this row
-        }
-        const float plimit = row_seed(p) * fminf(pk, total * p.top_p);
-        uint32_t ans = k - 1;
-        for (uint32_t base = 0; base < P; base += WAVE) {
-            const uint64_t hit = __ballot(base + lane < k && s_cum[base + lane] >= plimit);
-            if (hit) {
-                ans = base + (uint32_t)__ffsll((long long)hit) - 1;
-                break;
-            }
-        }
-        if (lane == 0) {
-            KvPair *out = reinterpret_cast<KvPair *>(p.kv) + blockIdx.x;
-            out->idx = comp_idx(cand[ans]);
-            out->val = L::from_f32(s_cum[ans]);
-        }
+        pk = c;  // entries past k add zero
     }
+    sample_settle<T>(
+        p, row, total, mx, pk, k, kstar, leftover,
+        [&](float plimit) {
+            for (uint32_t base = 0; base < P; base += WAVE) {
+                const uint64_t hit = __ballot(base + lane < k && s_cum[base + lane] >= plimit);
+                if (hit) return base + (uint32_t)__ffsll((long long)hit) - 1;
+            }
+            return k - 1;
+        },
+        [&](uint32_t ans) {
+            if (lane == 0) {
+                KvPair *out = reinterpret_cast<KvPair *>(p.kv) + blockIdx.x;
+                out->idx = comp_idx(cand[ans]);
+                out->val = L::from_f32(s_cum[ans]);
+            }
+        },
+        scratch, &s_state);
 }
 
 extern "C" __global__ void __launch_bounds__(SB) sample_topk_list_f16(SampleParams p) { sample_topk_list_impl<f16>(p); }
@@ -885,7 +1193,7 @@ __device__ __forceinline__ void sample_full_impl(const SampleParams &p) {
     const float mx = L::value(L::unkey(comp_key(keys[0])));
     const float t = p.temperature;
     for (uint32_t i = threadIdx.x; i < n; i += SB)
-        cum[i] = i == 0 ? 1.0f : exp_cr((L::value(L::unkey(comp_key(keys[i]))) - mx) / t);
+        cum[i] = i == 0 ? 1.0f : expf_libm((L::value(L::unkey(comp_key(keys[i]))) - mx) / t);
     __syncthreads();
     if (threadIdx.x < WAVE) {
         // the sequential f32 running sum, by wave 0: 64 terms at a time are loaded together (the next 64 already
