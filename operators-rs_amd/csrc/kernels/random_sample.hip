@@ -17,9 +17,10 @@
 //      and, if the k-th value is tied, radix-select on the index among the ties;
 //   2. gather exactly k candidates, bitonic-sort them in LDS by (value desc, idx asc);
 //   3. the f32 running sum over those k entries is done by ONE lane in sorted
-//      order, each term being exp() evaluated in f64 and rounded once to f32, so
-//      cum[0..k) follows the sequential definition; the sum over all n entries
-//      (needed for top_p) is a parallel f32 reduction in a fixed order.
+//      order, each term being libm's expf restated bit for bit, so cum[0..k) is the
+//      reference's; the sum over all n entries (needed for top_p) is known as an
+//      interval around a parallel sum, and only a row whose draw falls between two
+//      entries inside that interval pays for the sequential total (sample_settle).
 // the same for rows that do not fit the registers (`sample_topk_list`): after the first digit the
 // elements that can still matter (the chosen bucket and everything above it) are copied to a short list in
 // LDS, in the same sweep that sums the exponentials of the whole row; the rest runs on the list.
@@ -423,6 +424,63 @@ __device__ __forceinline__ void sort_desc_256(uint64_t *a, uint32_t cnt) {
     __syncthreads();
 }
 
+__device__ __forceinline__ uint32_t shfl_xor_key(uint32_t v, int m) { return __shfl_xor(v, m, WAVE); }
+__device__ __forceinline__ uint64_t shfl_xor_key(uint64_t v, int m) { return shfl_xor_u64(v, m); }
+
+// Descending sort of P (a power of two, 64 <= P <= SB * PER) keys in LDS by the whole workgroup: PER consecutive
+// keys per thread in registers; exchanges at a distance below PER stay inside the thread, below 64 * PER they are
+// shuffles inside the wave, and only the few stages with longer distances go through LDS with barriers (for
+// 4096 keys: 10 of 78 stages; the all-LDS network above takes 36 us for them, this one 4).
+// All threads call; `a` holds the result after return.
+template <typename K, int PER>
+__device__ __forceinline__ void block_sort_desc(K *a, uint32_t P) {
+    const uint32_t first = threadIdx.x * PER;
+    K x[PER];
+#pragma unroll
+    for (int r = 0; r < PER; ++r) x[r] = first + r < P ? a[first + r] : (K)0;
+    auto settle = [&](K &mine, K other, uint32_t i, uint32_t k2, uint32_t j) {
+        const bool desc = (i & k2) == 0, lower = (i & j) == 0;
+        mine = (lower == desc) ? (mine > other ? mine : other) : (mine < other ? mine : other);
+    };
+    for (uint32_t k2 = 2; k2 <= P; k2 <<= 1)
+        for (uint32_t j = k2 >> 1; j > 0; j >>= 1) {
+            if (j >= (uint32_t)PER * WAVE) {
+                __syncthreads();
+#pragma unroll
+                for (int r = 0; r < PER; ++r)
+                    if (first + r < P) a[first + r] = x[r];
+                __syncthreads();
+#pragma unroll
+                for (int r = 0; r < PER; ++r)
+                    if (first + r < P) settle(x[r], a[(first + r) ^ j], first + r, k2, j);
+            } else if (j >= (uint32_t)PER) {
+                K y[PER];  // all the exchanges are requested before the first is used
+#pragma unroll
+                for (int r = 0; r < PER; ++r) y[r] = shfl_xor_key(x[r], (int)(j / PER));
+#pragma unroll
+                for (int r = 0; r < PER; ++r) settle(x[r], y[r], first + r, k2, j);
+            } else {
+#pragma unroll
+                for (int jj = PER / 2; jj >= 1; jj >>= 1)
+                    if (j == (uint32_t)jj) {
+#pragma unroll
+                        for (int r = 0; r < PER; ++r)
+                            if ((r & jj) == 0) {
+                                const bool desc = ((first + r) & k2) == 0;
+                                const K lo = x[r] < x[r + jj] ? x[r] : x[r + jj], hi = x[r] < x[r + jj] ? x[r + jj] : x[r];
+                                x[r] = desc ? hi : lo;
+                                x[r + jj] = desc ? lo : hi;
+                            }
+                    }
+            }
+        }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < PER; ++r)
+        if (first + r < P) a[first + r] = x[r];
+    __syncthreads();
+}
+
 // ---- the total over all n entries, as the reference's sequential sum gives it -----------------------------------
 //
 // The reference's top_p bound is top_p * cum[n-1], the last of its sequential f32 running sums over the sorted
@@ -471,16 +529,30 @@ __device__ __forceinline__ double block_sum_f64(double v, double *smem) {
 }
 
 constexpr uint32_t XCH = 4096;  // entries sample_exact_total sorts per round
-// LDS the later stages work in (the caller's histogram arrays serve again)
+// LDS the later stages work in (the caller's histogram arrays serve again).  The members are LDS pointers by type:
+// handed to a function that is not inlined as plain pointers they would make every access a flat one.
+#define LDS_PTR(T) __attribute__((address_space(3))) T *
+struct TotalScratchLds {
+    LDS_PTR(uint32_t) hist;    // [256]
+    LDS_PTR(uint32_t) hist_w;  // [SB / WAVE][256]
+    LDS_PTR(uint32_t) wtot;    // [4]
+    LDS_PTR(uint32_t) sel;     // [2]
+    LDS_PTR(uint32_t) cnt;     // [1]
+    LDS_PTR(uint32_t) keys;    // [XCH]
+    LDS_PTR(double) red;       // [SB / WAVE]
+    LDS_PTR(float) fl;         // [2]
+};
+// the same as plain pointers, made from the above inside a function (the compiler keeps track of where they point)
 struct TotalScratch {
-    uint32_t *hist;            // [256]
-    uint32_t (*hist_w)[256];   // [SB / WAVE][256]
-    uint32_t *wtot;            // [4]
-    uint32_t *sel;             // [2]
-    uint32_t *cnt;             // [1]
-    uint32_t *keys;            // [XCH]
-    double *red;               // [SB / WAVE]
-    float *fl;                 // [2]
+    uint32_t *hist;
+    uint32_t (*hist_w)[256];
+    uint32_t *wtot, *sel, *cnt, *keys;
+    double *red;
+    float *fl;
+    __device__ __forceinline__ explicit TotalScratch(const TotalScratchLds &l)
+        : hist((uint32_t *)l.hist), hist_w((uint32_t(*)[256])l.hist_w), wtot((uint32_t *)l.wtot), sel((uint32_t *)l.sel),
+          cnt((uint32_t *)l.cnt), keys((uint32_t *)l.keys), red((double *)l.red), fl((float *)l.fl) {
+    }
 };
 
 // Stage 1: the exact terms summed in f64 and the bound on what the sequential f32 sum can lose or gain against that
@@ -489,8 +561,9 @@ struct TotalScratch {
 // carries neither its code nor its registers.)
 template <typename T>
 __device__ __noinline__ TotalBounds sample_total_bounds(const char *row, uint32_t n, float mx, float t, float t_hi,
-                                                        TotalScratch s) {
+                                                        TotalScratchLds lds) {
     typedef Logit<T> L;
+    const TotalScratch s(lds);
     const double h = (double)t_hi * 0x1p-24 * (1.0 + 1e-6);
     double sum = 0.0, err = 0.0;
     for_each_logit<T>(row, n, [&](uint32_t, uint32_t bits) {
@@ -508,15 +581,18 @@ __device__ __noinline__ TotalBounds sample_total_bounds(const char *row, uint32_
 }
 
 // The reference's sequential sum continued: `c` is cum[k-1]; behind the k candidates come `leftover` more entries
-// with the k-th key and then every entry whose key is below it, in descending order.  Rounds of up to XCH keys:
-// radix-select the XCH-th largest key still below `hi`, gather the keys above it, sort them in LDS, and let
-// wave 0 add their terms one after another; the entries with the selected key itself (any number of them) are one
-// term added that many times.  The sum stops early once a term no longer changes it: every later term is
-// smaller and the sum only grows.  All threads call; every thread gets the total.
+// with the k-th key and then every entry whose key is below it, in descending order.  They are taken in rounds of up
+// to XCH keys: gathered into LDS, sorted, and added in order (add_sorted below).  The rounds' key ranges come from one
+// histogram of the keys' top 12 bits (a range of whole bins that holds at most XCH keys); a row with more than XCH keys
+// in one bin (heavy ties) is cut by radix-selecting the XCH-th largest key still to come instead, the entries
+// with that key itself (any number of them) being one term added that many times.  The sum stops early once a term
+// no longer changes it: every later term is smaller and the sum only grows.  All threads call; every thread gets
+// the total.
 template <typename T>
 __device__ __noinline__ float sample_exact_total(const char *row, uint32_t n, float c, uint32_t kstar, uint32_t leftover,
-                                                 float mx, float t, TotalScratch s) {
+                                                 float mx, float t, TotalScratchLds lds) {
     typedef Logit<T> L;
+    const TotalScratch s(lds);
     // (the row is read from memory here even when the caller holds it in registers: this is a function of its
     // own so that its code and its registers stay out of the callers' common path)
     auto each_key = [&](auto &&f) { for_each_logit<T>(row, n, [&](uint32_t, uint32_t bits) { f(L::key(bits)); }); };
@@ -531,95 +607,247 @@ __device__ __noinline__ float sample_exact_total(const char *row, uint32_t n, fl
         return true;
     };
     const bool wave0 = threadIdx.x < WAVE;
-    const uint32_t lane = threadIdx.x % WAVE;
-    bool moving = true;  // (meaningful in wave 0)
-    if (wave0 && leftover) moving = add_run(term(kstar), leftover);
-    uint32_t hi = kstar;  // keys below `hi` are still to come
-    for (;;) {
+    const uint32_t lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+    bool moving = true;  // between rounds wave 0 holds the sum and this flag; keep_going() tells everybody
+    auto keep_going = [&]() {
         if (wave0 && lane == 0) s.fl[0] = moving ? 1.f : 0.f;
         __syncthreads();
-        if (s.fl[0] == 0.f || hi == 0) break;
-        // the XCH-th largest key below hi, digit by digit; the first digit's histogram also counts what is left
-        uint32_t prefix = 0, krem = XCH, eq_count = 0, left = 0;
-        bool all = false;  // XCH or fewer left: this round takes them all
-        for (int shift = L::KEY_BITS - 8; shift >= 0 && !all; shift -= 8) {
-            for (uint32_t i = threadIdx.x; i < (SB / WAVE) * 256; i += SB) (&s.hist_w[0][0])[i] = 0;
-            __syncthreads();
-            const bool first = shift == L::KEY_BITS - 8;
-            const uint32_t hi_mask = first ? 0u : (0xffffffffu << (shift + 8));
-            uint32_t *my_hist = s.hist_w[threadIdx.x / WAVE];
-            each_key([&](uint32_t key) {
-                if (key < hi && ((key ^ prefix) & hi_mask) == 0) atomicAdd(&my_hist[(key >> shift) & 255u], 1u);
-            });
-            __syncthreads();
-            if (threadIdx.x < 256) {
-                uint32_t cnt = 0;
-#pragma unroll
-                for (int w = 0; w < SB / WAVE; ++w) cnt += s.hist_w[w][threadIdx.x];
-                s.hist[threadIdx.x] = cnt;
+        const bool go = s.fl[0] != 0.f;
+        __syncthreads();
+        return go;
+    };
+
+    // The `cnt` keys in s.keys, sorted descending, are added in parallel, yet with the sequential sum's roundings.
+    // While the sum stays in one binade [2^b, 2^(b+1)), it is an integer M of 24 bits times u = 2^(b-23), and adding a
+    // term e adds an integer number of u: d = e / u rounded to nearest, a fixed number except on an exact tie
+    // (e / u = q + 1/2), where round-to-even makes it depend on M's parity: q + (q & 1) for even M, q + ((q + 1) & 1)
+    // for odd M.  So every term is a pair (d for even M, d for odd M); pairs compose, in order, to pairs, and an
+    // ordered scan gives M in front of every term.  The first term that carries M to 2^24 leaves the binade: it is
+    // added in floating point, and the scan starts again behind it with the next binade's u.
+    auto add_sorted = [&](uint32_t cnt) {
+        for (uint32_t pos = 0; pos < cnt;) {  // (workgroup-uniform)
+            if (wave0 && lane == 0) {
+                const float e0 = term(s.keys[pos]);
+                s.fl[0] = (c + e0 == c) ? 0.f : 1.f;  // the largest term left no longer moves the sum
+                s.fl[1] = c;
+                s.sel[0] = cnt;  // index of the first term that leaves the binade
             }
             __syncthreads();
-            if (first) {
-                for (uint32_t i = 0; i < 256; ++i) left += s.hist[i];
-                if (left <= XCH) {
-                    all = true;
-                    break;
+            if (s.fl[0] == 0.f) {
+                moving = false;
+                break;
+            }
+            const float c_now = s.fl[1];
+            const uint32_t cbits = __float_as_uint(c_now);
+            const uint32_t bexp = cbits >> 23;  // biased exponent of the sum (it is >= 1.0)
+            const uint32_t M = (cbits & 0x7fffffu) | 0x800000u;
+            const double scale = __longlong_as_double((long long)(1023 + 23 + 127 - (int)bexp) << 52);  // 1 / u
+            constexpr uint32_t PER = XCH / SB;
+            uint32_t f0[PER], f1[PER];
+            uint32_t t0 = 0, t1 = 0;  // this thread's terms composed
+#pragma unroll
+            for (uint32_t j = 0; j < PER; ++j) {
+                const uint32_t i = pos + threadIdx.x * PER + j;
+                f0[j] = f1[j] = 0;
+                if (i < cnt) {
+                    const double es = (double)term(s.keys[i]) * scale;
+                    const double fl = floor(es);
+                    const uint32_t q = (uint32_t)fl;
+                    const double frac = es - fl;
+                    if (frac == 0.5) f0[j] = q + (q & 1u), f1[j] = q + ((q + 1u) & 1u);
+                    else f0[j] = f1[j] = q + (frac > 0.5 ? 1u : 0u);
+                }
+                const uint32_t n0 = t0 + ((t0 & 1u) ? f1[j] : f0[j]);
+                const uint32_t n1 = t1 + (((t1 + 1u) & 1u) ? f1[j] : f0[j]);
+                t0 = n0, t1 = n1;
+            }
+            // ordered inclusive scan over the threads: (l0, l1) from the left is applied first
+            uint32_t i0 = t0, i1 = t1;
+#pragma unroll
+            for (int o = 1; o < WAVE; o <<= 1) {
+                const uint32_t l0 = __shfl_up(i0, o, WAVE), l1 = __shfl_up(i1, o, WAVE);
+                if (lane >= (uint32_t)o) {
+                    const uint32_t n0 = l0 + ((l0 & 1u) ? i1 : i0);
+                    const uint32_t n1 = l1 + (((l1 + 1u) & 1u) ? i1 : i0);
+                    i0 = n0, i1 = n1;
                 }
             }
-            pick_bucket(s.hist, krem, true, s.wtot, s.sel);
-            prefix |= s.sel[0] << shift;
-            krem = s.sel[1];
-            eq_count = s.hist[s.sel[0]];
+            if (lane == WAVE - 1) s.hist[2 * wave] = i0, s.hist[2 * wave + 1] = i1;
+            __syncthreads();
+            uint32_t w0 = 0, w1 = 0;  // the waves to the left composed
+            for (uint32_t w = 0; w < wave; ++w) {
+                const uint32_t g0 = s.hist[2 * w], g1 = s.hist[2 * w + 1];
+                const uint32_t n0 = w0 + ((w0 & 1u) ? g1 : g0);
+                const uint32_t n1 = w1 + (((w1 + 1u) & 1u) ? g1 : g0);
+                w0 = n0, w1 = n1;
+            }
+            // exclusive prefix of this thread: waves to the left, then lanes to the left
+            uint32_t x0 = __shfl_up(i0, 1, WAVE), x1 = __shfl_up(i1, 1, WAVE);
+            if (lane == 0) x0 = x1 = 0;
+            const uint32_t Mw = M + ((M & 1u) ? w1 : w0);
+            const uint32_t Mt = Mw + ((Mw & 1u) ? x1 : x0);  // M in front of this thread's first term
+            uint32_t Mi = Mt;
+#pragma unroll
+            for (uint32_t j = 0; j < PER; ++j) {
+                const uint32_t i = pos + threadIdx.x * PER + j;
+                if (i < cnt) {
+                    const uint32_t d = (Mi & 1u) ? f1[j] : f0[j];
+                    if (Mi + d >= 0x1000000u || Mi >= 0x1000000u) {
+                        atomicMin(&s.sel[0], i);
+                        break;
+                    }
+                    Mi += d;
+                }
+            }
+            __syncthreads();
+            const uint32_t cross = s.sel[0];
+            __syncthreads();
+            if (cross >= cnt) {  // the whole piece stays in the binade: the last thread's M is the sum
+                if (threadIdx.x == SB - 1) s.fl[1] = __uint_as_float((bexp << 23) | (Mi & 0x7fffffu));
+                __syncthreads();
+                c = s.fl[1];
+                __syncthreads();
+                break;
+            }
+            // the thread that owns term `cross` has M in front of it: that one term is added in floating point
+            if (threadIdx.x == (cross - pos) / PER) {
+                uint32_t Mc = Mt;
+#pragma unroll
+                for (uint32_t j = 0; j < PER; ++j)
+                    if (j < (cross - pos) % PER) Mc += (Mc & 1u) ? f1[j] : f0[j];
+                s.fl[1] = __uint_as_float((bexp << 23) | (Mc & 0x7fffffu)) + term(s.keys[cross]);
+            }
+            __syncthreads();
+            c = s.fl[1];
+            pos = cross + 1;
             __syncthreads();
         }
-        if (left == 0) break;
-        const uint32_t lo = all ? 0u : prefix;  // gather lo < key < hi (all: every key below hi)
+    };
+    // keys picked by `take` into s.keys (up to XCH of them), sorted descending; returns how many
+    auto gather_sorted = [&](uint32_t expect, auto &&take) {
         uint32_t P = 64;
-        const uint32_t expect = all ? left : XCH - krem;
         while (P < expect) P <<= 1;
         if (threadIdx.x == 0) *s.cnt = 0;
         for (uint32_t i = threadIdx.x; i < P; i += SB) s.keys[i] = 0;
         __syncthreads();
         each_key([&](uint32_t key) {
-            if (key < hi && (all || key > lo)) {
+            if (take(key)) {
                 const uint32_t slot = atomicAdd(s.cnt, 1u);
                 if (slot < XCH) s.keys[slot] = key;
             }
         });
         __syncthreads();
         const uint32_t cnt = min(*s.cnt, XCH);
-        if (P <= 64) {
-            if (wave0) {  // one value per lane, sorted by shuffles
-                uint32_t x = s.keys[lane];
+        block_sort_desc<uint32_t, XCH / SB>(s.keys, P);
+        return cnt;
+    };
+
+    if (wave0 && leftover) moving = add_run(term(kstar), leftover);
+
+    // histogram of the keys below kstar by their top 12 bits, then in place: tail[b] = keys in bins >= b
+    constexpr int BSH = L::KEY_BITS - 12;
+    constexpr uint32_t NBIN = 4096, BPT = NBIN / SB;
+    uint32_t *tail = &s.hist_w[0][0];
+    for (uint32_t i = threadIdx.x; i < NBIN; i += SB) tail[i] = 0;
+    if (threadIdx.x == 0) s.sel[1] = 0;
+    __syncthreads();
+    each_key([&](uint32_t key) {
+        if (key < kstar) atomicAdd(&tail[key >> BSH], 1u);
+    });
+    __syncthreads();
+    {
+        uint32_t mine[BPT], sum = 0, big = 0;
 #pragma unroll
-                for (int k2 = 2; k2 <= WAVE; k2 <<= 1)
+        for (uint32_t j = 0; j < BPT; ++j) {  // this thread's bins, highest first
+            mine[j] = tail[NBIN - 1 - (threadIdx.x * BPT + j)];
+            big = max(big, mine[j]);
+            sum += mine[j];
+            mine[j] = sum;
+        }
+        uint32_t incl = sum;
 #pragma unroll
-                    for (int j = k2 >> 1; j > 0; j >>= 1) {
-                        const uint32_t y = __shfl_xor(x, j, WAVE);
-                        const bool desc = (lane & k2) == 0, lower = (lane & j) == 0;
-                        x = (lower == desc) ? max(x, y) : min(x, y);
-                    }
-                s.keys[lane] = x;
+        for (int o = 1; o < WAVE; o <<= 1) {
+            const uint32_t l = __shfl_up(incl, o, WAVE);
+            if (lane >= (uint32_t)o) incl += l;
+        }
+        if (lane == WAVE - 1) s.hist[wave] = incl;
+        atomicMax(&s.sel[1], big);
+        __syncthreads();
+        uint32_t base = incl - sum;
+        for (uint32_t w = 0; w < wave; ++w) base += s.hist[w];
+#pragma unroll
+        for (uint32_t j = 0; j < BPT; ++j) tail[NBIN - 1 - (threadIdx.x * BPT + j)] = base + mine[j];
+        __syncthreads();
+    }
+    const bool heavy = s.sel[1] > XCH;  // a bin alone overflows a round
+    __syncthreads();
+
+    if (!heavy) {
+        uint32_t done = 0, bin_hi = NBIN;  // keys taken so far; bins below bin_hi are still to come
+        while (keep_going() && bin_hi > 0 && tail[0] > done) {
+            // the lowest bin down to which everything still to come fits one round
+            uint32_t lo_b = 0, hi_b = bin_hi - 1;
+            while (lo_b < hi_b) {
+                const uint32_t mid = (lo_b + hi_b) / 2;
+                if (tail[mid] - done <= XCH) hi_b = mid;
+                else lo_b = mid + 1;
             }
+            const uint32_t bin_lo = lo_b, expect = tail[bin_lo] - done;
             __syncthreads();
-        } else {
-            bitonic_lds(s.keys, P, 2, P, P, 0);
-        }
-        if (wave0) {
-            for (uint32_t base = 0; base < cnt && moving; base += WAVE) {
-                const float e = base + lane < cnt ? term(s.keys[base + lane]) : 0.f;
-                const float e0 = __shfl(e, 0, WAVE);
-                if (c + e0 == c) {  // the largest term left no longer moves the sum
-                    moving = false;
-                    break;
-                }
-#pragma unroll
-                for (int i = 0; i < WAVE; ++i) c = c + __shfl(e, i, WAVE);
+            if (expect) {
+                const uint32_t cnt = gather_sorted(expect, [&](uint32_t key) {
+                    const uint32_t bin = key >> BSH;
+                    return key < kstar && bin >= bin_lo && bin < bin_hi;
+                });
+                add_sorted(cnt);
             }
-            if (moving && !all) moving = add_run(term(lo), eq_count);
+            done += expect;
+            bin_hi = bin_lo;
         }
-        if (all) break;
-        hi = lo;
+    } else {
+        uint32_t hi = kstar;  // keys below `hi` are still to come
+        while (keep_going() && hi > 0) {
+            // the XCH-th largest key below hi, digit by digit; the first digit's histogram also counts what is left
+            uint32_t prefix = 0, krem = XCH, eq_count = 0, left = 0;
+            bool all = false;  // XCH or fewer left: this round takes them all
+            for (int shift = L::KEY_BITS - 8; shift >= 0 && !all; shift -= 8) {
+                for (uint32_t i = threadIdx.x; i < (SB / WAVE) * 256; i += SB) (&s.hist_w[0][0])[i] = 0;
+                __syncthreads();
+                const bool first = shift == L::KEY_BITS - 8;
+                const uint32_t hi_mask = first ? 0u : (0xffffffffu << (shift + 8));
+                uint32_t *my_hist = s.hist_w[wave];
+                each_key([&](uint32_t key) {
+                    if (key < hi && ((key ^ prefix) & hi_mask) == 0) atomicAdd(&my_hist[(key >> shift) & 255u], 1u);
+                });
+                __syncthreads();
+                if (threadIdx.x < 256) {
+                    uint32_t cnt = 0;
+#pragma unroll
+                    for (int w = 0; w < SB / WAVE; ++w) cnt += s.hist_w[w][threadIdx.x];
+                    s.hist[threadIdx.x] = cnt;
+                }
+                __syncthreads();
+                if (first) {
+                    for (uint32_t i = 0; i < 256; ++i) left += s.hist[i];
+                    if (left <= XCH) {
+                        all = true;
+                        break;
+                    }
+                }
+                pick_bucket(s.hist, krem, true, s.wtot, s.sel);
+                prefix |= s.sel[0] << shift;
+                krem = s.sel[1];
+                eq_count = s.hist[s.sel[0]];
+                __syncthreads();
+            }
+            if (left == 0) break;
+            const uint32_t lo = all ? 0u : prefix;  // gather lo < key < hi (all: every key below hi)
+            const uint32_t cnt = gather_sorted(all ? left : XCH - krem, [&](uint32_t key) { return key < hi && (all || key > lo); });
+            add_sorted(cnt);
+            if (all) break;
+            if (wave0 && moving) moving = add_run(term(lo), eq_count);  // the entries with the selected key itself
+            hi = lo;
+        }
     }
     __syncthreads();
     if (wave0 && lane == 0) s.fl[1] = c;
@@ -634,7 +862,7 @@ __device__ __noinline__ float sample_exact_total(const char *row, uint32_t n, fl
 template <typename T, typename Find, typename Emit>
 __device__ __forceinline__ void sample_settle(const SampleParams &p, const char *row, float fast_total, float mx, float pk,
                                               uint32_t k, uint32_t kstar, uint32_t leftover, Find &&find, Emit &&emit,
-                                              const TotalScratch &s, uint32_t *s_state) {
+                                              const TotalScratchLds &s, uint32_t *s_state) {
     typedef Logit<T> L;
     const bool wave0 = threadIdx.x < WAVE;
     const uint32_t lane = threadIdx.x % WAVE;
@@ -786,9 +1014,10 @@ __device__ __forceinline__ void sample_topk_impl(const SampleParams &p) {
 
     const float t = p.temperature;
     const uint32_t leftover = eq_count - krem;  // entries with the k-th key that are not among the candidates
-    TotalScratch scratch;
-    scratch.hist = hist, scratch.hist_w = hist_w, scratch.wtot = s_wtot, scratch.sel = s_sel, scratch.cnt = &s_cnt;
-    scratch.keys = s_xkeys, scratch.red = s_xred, scratch.fl = s_xfl;
+    TotalScratchLds scratch;
+    scratch.hist = (LDS_PTR(uint32_t))hist, scratch.hist_w = (LDS_PTR(uint32_t)) & hist_w[0][0];
+    scratch.wtot = (LDS_PTR(uint32_t))s_wtot, scratch.sel = (LDS_PTR(uint32_t))s_sel, scratch.cnt = (LDS_PTR(uint32_t)) & s_cnt;
+    scratch.keys = (LDS_PTR(uint32_t))s_xkeys, scratch.red = (LDS_PTR(double))s_xred, scratch.fl = (LDS_PTR(float))s_xfl;
     if (SMALLK || P == 64) {
         // k <= 64: sort, prefix and search live in the registers of wave 0
         const uint32_t lane = threadIdx.x % WAVE;
@@ -1048,9 +1277,10 @@ __device__ __forceinline__ void sample_topk_list_impl(const SampleParams &p) {
     }
 
     const uint32_t leftover = eq_count - krem;  // entries with the k-th key that are not among the candidates
-    TotalScratch scratch;
-    scratch.hist = hist, scratch.hist_w = hist_w, scratch.wtot = s_wtot, scratch.sel = s_sel, scratch.cnt = &s_cnt;
-    scratch.keys = s_xkeys, scratch.red = s_xred, scratch.fl = s_xfl;
+    TotalScratchLds scratch;
+    scratch.hist = (LDS_PTR(uint32_t))hist, scratch.hist_w = (LDS_PTR(uint32_t)) & hist_w[0][0];
+    scratch.wtot = (LDS_PTR(uint32_t))s_wtot, scratch.sel = (LDS_PTR(uint32_t))s_sel, scratch.cnt = (LDS_PTR(uint32_t)) & s_cnt;
+    scratch.keys = (LDS_PTR(uint32_t))s_xkeys, scratch.red = (LDS_PTR(double))s_xred, scratch.fl = (LDS_PTR(float))s_xfl;
     const uint32_t lane = threadIdx.x % WAVE;
     if (P == 64) {
         // k <= 64: sort, prefix and search live in the registers of wave 0
