@@ -220,3 +220,164 @@ extern "C" {
     pub fn ophip_stream_synchronize(dev: *mut ophip_device, stream: ophip_stream) -> c_int;
     pub fn ophip_queue_alloc_from_stream(dev: *mut ophip_device, stream: ophip_stream, out: *mut ophip_queue_alloc) -> c_int;
 }
+
+// ---- the rest of include/ophip.h: everything the header declares is declared here too -------------
+#[repr(C)]
+pub struct ophip_mem_pool {
+    _opaque: [u8; 0],
+}
+#[repr(C)]
+pub struct ophip_offset_calculator {
+    _opaque: [u8; 0],
+}
+#[repr(C)]
+pub struct ophip_attention {
+    _opaque: [u8; 0],
+}
+#[repr(C)]
+pub struct ophip_attention_kv_cached {
+    _opaque: [u8; 0],
+}
+#[repr(C)]
+pub struct ophip_conv {
+    _opaque: [u8; 0],
+}
+#[repr(C)]
+#[derive(Clone, Copy)]
+pub struct ophip_rope_seq {
+    pub pos: usize,
+    pub len: usize,
+}
+#[repr(C)]
+#[derive(Clone, Copy)]
+pub struct ophip_kv_pair {
+    pub idx: u32,
+    pub val: u32,
+}
+#[repr(C)]
+#[derive(Clone, Copy)]
+pub struct ophip_mat_mul_layout {
+    pub dt: u64,
+    pub ab_swap: i32,
+    pub a_trans: i32,
+    pub b_trans: i32,
+    pub _pad: i32,
+    pub batch: usize,
+    pub m: usize,
+    pub n: usize,
+    pub k: usize,
+    pub c_stride: isize,
+    pub c_ld: isize,
+    pub a_stride: isize,
+    pub a_ld: isize,
+    pub b_stride: isize,
+    pub b_ld: isize,
+}
+#[repr(C)]
+#[derive(Clone, Copy)]
+pub struct ophip_attention_args {
+    pub q_layout: ophip_tensor_layout,
+    pub q_base: *mut c_void,
+    pub k_layout: ophip_tensor_layout,
+    pub k_base: *const c_void,
+    pub v_layout: ophip_tensor_layout,
+    pub v_base: *const c_void,
+    pub o_layout: ophip_tensor_layout,
+    pub o_base: *mut c_void,
+    pub mask: u8,
+}
+#[repr(C)]
+#[derive(Clone, Copy)]
+pub struct ophip_attention_kv_cached_args {
+    pub q_layout: ophip_tensor_layout,
+    pub q_base: *mut c_void,
+    pub k_layout: ophip_tensor_layout,
+    pub k_base: *const c_void,
+    pub v_layout: ophip_tensor_layout,
+    pub v_base: *const c_void,
+    pub o_layout: ophip_tensor_layout,
+    pub o_base: *mut c_void,
+    pub k_cache_layout: ophip_tensor_layout,
+    pub k_cache_base: *mut c_void,
+    pub v_cache_layout: ophip_tensor_layout,
+    pub v_cache_base: *mut c_void,
+    pub mask: u8,
+    pub pos: usize,
+}
+#[repr(C)]
+#[derive(Clone, Copy)]
+pub struct ophip_conv_args {
+    pub y_layout: ophip_tensor_layout,
+    pub y_base: *mut c_void,
+    pub x_layout: ophip_tensor_layout,
+    pub x_base: *const c_void,
+    pub w_layout: ophip_tensor_layout,
+    pub w_base: *const c_void,
+    pub b_layout: ophip_tensor_layout,
+    pub b_base: *const c_void,
+    pub strides: [usize; 2],
+    pub dilations: [usize; 2],
+    pub pads: [usize; 4],
+}
+#[link(name = "ophip")]
+extern "C" {
+    pub fn ophip_status_name(status: c_int) -> *const c_char;
+    pub fn ophip_dtype_nbytes(dt: u64) -> usize;
+    pub fn ophip_device_retain(dev: *mut ophip_device);
+    pub fn ophip_memset(dev: *mut ophip_device, dst: *mut c_void, value: c_int, size: usize, stream: *mut c_void) -> c_int;
+    pub fn ophip_event_create(dev: *mut ophip_device, out: *mut *mut c_void) -> c_int;
+    pub fn ophip_event_destroy(dev: *mut ophip_device, ev: *mut c_void) -> c_int;
+    pub fn ophip_event_record(dev: *mut ophip_device, ev: *mut c_void, stream: *mut c_void) -> c_int;
+    pub fn ophip_event_synchronize(dev: *mut ophip_device, ev: *mut c_void) -> c_int;
+    pub fn ophip_event_elapsed_ms(dev: *mut ophip_device, start: *mut c_void, stop: *mut c_void, ms: *mut f32) -> c_int;
+    pub fn ophip_time_next_launch(dev: *mut ophip_device, stream: *mut c_void, start: *mut c_void, stop: *mut c_void) -> c_int;
+    pub fn ophip_stream_begin_capture(dev: *mut ophip_device, stream: *mut c_void) -> c_int;
+    pub fn ophip_stream_end_capture(dev: *mut ophip_device, stream: *mut c_void, out: *mut *mut c_void) -> c_int;
+    pub fn ophip_graph_launch(dev: *mut ophip_device, graph: *mut c_void, stream: *mut c_void) -> c_int;
+    pub fn ophip_graph_destroy(dev: *mut ophip_device, graph: *mut c_void) -> c_int;
+    pub fn ophip_mem_pool_create(dev: *mut ophip_device, stream: *mut c_void, out: *mut *mut ophip_mem_pool) -> c_int;
+    pub fn ophip_mem_pool_put(pool: *mut ophip_mem_pool, size: usize) -> c_int;
+    pub fn ophip_mem_pool_queue_alloc(pool: *mut ophip_mem_pool, out: *mut ophip_queue_alloc) -> c_int;
+    pub fn ophip_mem_pool_destroy(pool: *mut ophip_mem_pool);
+    pub fn ophip_offset_calculator_create(alignment: usize) -> *mut ophip_offset_calculator;
+    pub fn ophip_offset_calculator_destroy(c: *mut ophip_offset_calculator);
+    pub fn ophip_offset_calculator_put(c: *mut ophip_offset_calculator, start: usize, end: usize);
+    pub fn ophip_offset_calculator_take(c: *mut ophip_offset_calculator, size: usize, start: *mut usize,
+        end: *mut usize) -> c_int;
+    pub fn ophip_rope_build_pos(dt: u64, nt: usize, seqs: *const ophip_rope_seq, nseq: usize,
+        queue_alloc: *const ophip_queue_alloc, out: *mut *mut c_void) -> c_int;
+    pub fn ophip_rope_build_sincos(dt: u64, nctx: usize, dh: usize, queue_alloc: *const ophip_queue_alloc,
+        nctx_out: *mut usize, out: *mut *mut c_void) -> c_int;
+    pub fn ophip_rearrange_plan(args: *const ophip_rearrange_args, out: *mut isize, ndim_out: *mut usize) -> c_int;
+    pub fn ophip_sample_args_new(temperature: f32, top_p: f32, top_k: usize, out: *mut ophip_sample_args) -> c_int;
+    pub fn ophip_sample_args_argmax() -> ophip_sample_args;
+    pub fn ophip_random_sample_launch_batch(op: *const ophip_random_sample, args: *const ophip_random_sample_args,
+        rows: usize, row_stride: isize, seeds: *const f32, workspace: *mut c_void, workspace_len: usize,
+        queue_alloc: *const ophip_queue_alloc) -> c_int;
+    pub fn ophip_random_sample_build_indices(n: usize, queue_alloc: *const ophip_queue_alloc, out: *mut *mut c_void) -> c_int;
+    pub fn ophip_mat_mul_plan(args: *const ophip_mat_mul_args, out: *mut ophip_mat_mul_layout) -> c_int;
+    pub fn ophip_mat_mul_launch_static(op: *const ophip_mat_mul, args: *const ophip_mat_mul_args,
+        stream: *mut c_void) -> c_int;
+    pub fn ophip_mat_mul_describe(op: *const ophip_mat_mul, args: *const ophip_mat_mul_args, out: *mut c_char,
+        len: usize) -> c_int;
+    pub fn ophip_attention_create(dev: *mut ophip_device, out: *mut *mut ophip_attention) -> c_int;
+    pub fn ophip_attention_scheme(op: *mut ophip_attention, args: *const ophip_attention_args,
+        max_workspace_size: usize, workspace_size: *mut usize) -> c_int;
+    pub fn ophip_attention_launch(op: *const ophip_attention, args: *const ophip_attention_args,
+        workspace: *mut c_void, workspace_len: usize, queue_alloc: *const ophip_queue_alloc) -> c_int;
+    pub fn ophip_attention_destroy(op: *mut ophip_attention);
+    pub fn ophip_attention_kv_cached_create(dev: *mut ophip_device, out: *mut *mut ophip_attention_kv_cached) -> c_int;
+    pub fn ophip_attention_kv_cached_scheme(op: *mut ophip_attention_kv_cached,
+        args: *const ophip_attention_kv_cached_args, max_workspace_size: usize, workspace_size: *mut usize) -> c_int;
+    pub fn ophip_attention_kv_cached_launch(op: *const ophip_attention_kv_cached,
+        args: *const ophip_attention_kv_cached_args, workspace: *mut c_void, workspace_len: usize,
+        queue_alloc: *const ophip_queue_alloc) -> c_int;
+    pub fn ophip_attention_kv_cached_destroy(op: *mut ophip_attention_kv_cached);
+    pub fn ophip_add_plan(args: *const ophip_add_args, out: *mut isize, ndim_out: *mut usize) -> c_int;
+    pub fn ophip_conv_create(dev: *mut ophip_device, out: *mut *mut ophip_conv) -> c_int;
+    pub fn ophip_conv_scheme(op: *mut ophip_conv, args: *const ophip_conv_args, max_workspace_size: usize,
+        workspace_size: *mut usize) -> c_int;
+    pub fn ophip_conv_launch(op: *const ophip_conv, args: *const ophip_conv_args, workspace: *mut c_void,
+        workspace_len: usize, queue_alloc: *const ophip_queue_alloc) -> c_int;
+    pub fn ophip_conv_destroy(op: *mut ophip_conv);
+}

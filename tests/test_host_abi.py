@@ -210,3 +210,95 @@ def test_tile_gemm_code_objects_keep_accumulators_in_registers():
     assert len(names) == len(scratch) == 24, (names, scratch)  # 3 tiles x 4 operand layouts, whole-tile and ragged builds
     for name, size in zip(names, scratch):
         assert size <= 512, "%s uses %d bytes of scratch per lane" % (name, size)
+
+
+# ---- the Rust side's declarations against the header, as text (no rustc, no C compiler needed) ----------------
+
+SHIM = os.path.join(ROOT, "operators-rs_amd", "rust_shim", "operators", "src")
+
+
+def _both_sides():
+    import abi_text
+
+    hs, hf, he, ho = abi_text.parse_header(open(os.path.join(ROOT, "include", "ophip.h")).read())
+    rs, rf, ro = abi_text.parse_rust_ffi(open(os.path.join(SHIM, "handle", "hip", "ffi.rs")).read())
+    return hs, hf, he, ho, rs, rf, ro
+
+
+def test_rust_ffi_structs_mirror_the_header():
+    """Every struct of include/ophip.h exists in ffi.rs with the same fields, in the same order, of the same types
+    (C spelling mapped to Rust: size_t = usize, ptrdiff_t = isize, const T * = *const T ...), and ffi.rs has none
+    the header lacks."""
+    hs, _, _, ho, rs, _, ro = _both_sides()
+    assert len(hs) >= 20 and set(hs) == set(rs), (sorted(set(hs) - set(rs)), sorted(set(rs) - set(hs)))
+    for name, fields in hs.items():
+        assert rs[name] == fields, "%s:\n  header %s\n  ffi.rs %s" % (name, fields, rs[name])
+    assert set(ho) == set(ro) - {"ophip_device"} | ({"ophip_device"} & set(ho)), (sorted(set(ho) ^ set(ro)))
+
+
+def test_rust_ffi_functions_mirror_the_header():
+    """Every OPHIP_API function is declared in ffi.rs (the four verbs of an operator through the `verbs!` macro, which
+    the reader expands) with the same argument count, order and types and the same return type."""
+    _, hf, _, _, _, rf, _ = _both_sides()
+    assert len(hf) >= 100 and set(hf) == set(rf), (sorted(set(hf) - set(rf)), sorted(set(rf) - set(hf)))
+    for name, sig in hf.items():
+        assert rf[name] == sig, "%s:\n  header %s\n  ffi.rs %s" % (name, sig, rf[name])
+    assert set(hf) == set(ophip.EXPORTS)
+
+
+def test_rust_side_uses_the_headers_codes():
+    """The status codes the Rust side turns into SchemeErrorKind and the dtype codes it sends are the header's."""
+    _, _, he, _, _, _, _ = _both_sides()
+    mod = open(os.path.join(SHIM, "handle", "hip", "mod.rs")).read()
+    # fn scheme_kind: `1 => TypeNotSupport,` ...
+    body = mod[mod.index("fn scheme_kind"):]
+    body = body[:body.index("\n}\n")]
+    rust_status = {name: int(code) for code, name in re.findall(r"(\d+)\s*=>\s*(\w+)\s*,", body)}
+    camel = lambda c: "".join(w.capitalize() for w in c[len("OPHIP_"):].lower().split("_"))
+    header_status = {camel(k): v for k, v in he["ophip_status"].items() if 1 <= v <= 9}
+    assert rust_status == header_status and len(rust_status) == 9
+    L = ophip.lib()
+    for name, code in rust_status.items():
+        assert L.ophip_status_name(code).decode() == name  # and the library names them the same way
+    # fn dt_code: `(ty::F16, 1),` ... and the KVPair code
+    body = mod[mod.index("fn dt_code"):]
+    body = body[:body.index("\n}\n")]
+    rust_dt = {name.upper(): int(code) for name, code in re.findall(r"\(ty::(\w+),\s*(\d+)\)", body)}
+    rust_dt["KVPAIR"] = int(re.search(r"KVPair[^\n]*\{\s*return\s+(\d+);", body, flags=re.S).group(1))
+    header_dt = {k[len("OPHIP_DT_"):]: v for k, v in he["ophip_dtype"].items()}
+    assert rust_dt == header_dt, (rust_dt, header_dt)
+    assert he["ophip_attn_mask"] == {"OPHIP_MASK_NONE": 0, "OPHIP_MASK_CAUSAL": 1}
+
+
+def test_every_operator_of_the_rust_side_names_what_the_header_has():
+    """The per-operator modules hand `ophip_*` names to the `hip_operator!` macro and build the argument structs
+    field by field: every name is a function, struct or opaque type of the header, and every struct literal sets
+    exactly the header's fields."""
+    hs, hf, _, ho, _, _, _ = _both_sides()
+    known = set(hf) | set(hs) | set(ho) | {"ophip_stream", "ophip_event", "ophip_graph"}  # (the three pointer typedefs)
+    used, literals = set(), 0
+    for d, _, files in os.walk(SHIM):
+        for f in files:
+            if not f.endswith(".rs") or f == "ffi.rs":
+                continue
+            text = re.sub(r"//[^\n]*", " ", open(os.path.join(d, f)).read())
+            used |= set(re.findall(r"\b(ophip_[a-z0-9_]+)\b", text))
+            for m in re.finditer(r"ffi::(ophip_\w+)\s*\{", text):
+                name, depth, top, i = m.group(1), 1, "", m.end()
+                if name not in hs:  # `-> *mut ffi::ophip_device {`: a function body, not a literal
+                    continue
+                while depth:  # the literal's own level, nested literals left out
+                    ch = text[i]
+                    depth += (ch == "{") - (ch == "}")
+                    if depth == 1 and ch not in "{}":
+                        top += ch
+                    i += 1
+                if ".." in top:  # `{ .. }` in a doc example
+                    continue
+                fields = re.findall(r"(?:^|,)\s*(\w+)\s*:(?!:)", top)
+                if not fields:  # `-> ffi::ophip_device_info {`: a function body again
+                    continue
+                assert fields == [n for n, _ in hs[name]], (f, name, fields)
+                literals += 1
+    assert len(used) >= 60 and literals >= 11
+    assert used <= known, sorted(used - known)
