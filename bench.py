@@ -192,11 +192,79 @@ def copy_ceiling(ophip, gpu, stream):
             "hbm_frac": round((2 << 30) / (us * 1e-6) / HBM_PEAK, 4)}
 
 
-def adder(out):
-    """Returns add(name, shape, bytes, us, flops, note): appends one per-operator record to `out` and logs it."""
+def read_power():
+    """Board power in watts from the amdgpu hwmon files, or None when they cannot be read."""
+    import glob
+    for pat in ("/sys/class/drm/card*/device/hwmon/hwmon*/power1_average", "/sys/class/drm/card*/device/hwmon/hwmon*/power1_input"):
+        for f in sorted(glob.glob(pat)):
+            try:
+                return int(open(f).read().strip()) / 1e6
+            except (OSError, ValueError):
+                pass
+    return None
+
+
+def ceilings(ophip, gpu, stream):
+    """What this machine gives a plain stream of 1 GiB (hipMemcpyAsync, and the library's probe kernels: read,
+    read with non-temporal loads, write, copy; best grid of a few) and a bare MFMA loop (random-looking and all-zero
+    operands, from idle clocks and in steady state, with the board power where the driver shows it)."""
+    out = {"copy_hipMemcpyAsync": copy_ceiling(ophip, gpu, stream)}
+    nbytes = 1 << 30
+    a_, b_ = gpu.malloc(nbytes), gpu.malloc(nbytes)
+    gpu.memset(a_, 0x3C)
+    gpu.memset(b_, 0)
+    probe = lambda kind, blocks, iters=0, seed=1, dst=None: ophip._check(ophip.lib().ophip_probe(
+        gpu.handle, kind.encode(), ctypes.c_void_p((dst or b_).ptr), ctypes.c_void_p(a_.ptr), ctypes.c_size_t(nbytes),
+        ctypes.c_uint(iters), ctypes.c_uint(seed), ctypes.c_uint(blocks), stream.handle))
+    for kind, moved in (("read", nbytes), ("read_nt", nbytes), ("write", nbytes), ("copy", 2 * nbytes)):
+        best = None
+        for blocks in (1024, 2048, 4096, 8192, 16384, 65536):
+            us = time_launches(gpu, stream, lambda: probe(kind, blocks), 10, warm=2)
+            if best is None or us < best[0]:
+                best = (us, blocks)
+        us, blocks = best
+        out[kind] = {"bytes": moved, "us": round(us, 2), "GBps": round(moved / us / 1e3, 1), "blocks": blocks,
+                     "hbm_frac": round(moved / (us * 1e-6) / HBM_PEAK, 4)}
+        log("  probe %-8s 1 GiB: %8.1f us, %7.1f GB/s (%.1f%% of 8 TB/s), %d workgroups" % (
+            kind, us, moved / us / 1e3, 100 * moved / (us * 1e-6) / HBM_PEAK, blocks))
+    # bare MFMA loop: 2048 workgroups of 4 waves, 512 trips of 128 MFMA 32x32x16 each
+    blocks, iters = 2048, 512
+    flop = blocks * 4 * iters * 128 * 32768
+    scratch = gpu.malloc(blocks * 1024)
+    for name, seed in (("mfma_random", 12345), ("mfma_zero", 0)):
+        run = lambda: probe("mfma", blocks, iters, seed, dst=scratch)
+        time.sleep(0.5)
+        idle_us = time_launches(gpu, stream, run, 5, warm=0)
+        n, t0, watts = 0, time.perf_counter(), []
+        while time.perf_counter() - t0 < 2.0:   # two seconds of load: clocks and power settle
+            for _ in range(4):
+                run()
+            stream.synchronize()
+            n += 4
+            w = read_power()
+            if w:
+                watts.append(w)
+        us = time_launches(gpu, stream, run, 20, warm=0)
+        out[name] = {"flop": flop, "us_from_idle": round(idle_us, 1), "TFLOPs_from_idle": round(flop / idle_us / 1e6, 1),
+                     "us_steady": round(us, 1), "TFLOPs_steady": round(flop / us / 1e6, 1),
+                     "mfma_frac_steady": round(flop / (us * 1e-6) / MFMA_F16_PEAK, 4),
+                     "watts": round(sum(watts[len(watts) // 2:]) / max(1, len(watts[len(watts) // 2:])), 0) if watts else None}
+        log("  probe %-12s %7.1f TFLOP/s from idle clocks, %7.1f TFLOP/s steady (%.1f%% of 2.5 PFLOP/s)%s" % (
+            name, flop / idle_us / 1e6, flop / us / 1e6, 100 * flop / (us * 1e-6) / MFMA_F16_PEAK,
+            ", %.0f W" % out[name]["watts"] if out[name]["watts"] else ""))
+    a_.free(); b_.free(); scratch.free()
+    return out
+
+
+def adder(out, ceiling=None):
+    """Returns add(name, shape, bytes, us, flops, note): appends one per-operator record to `out` and logs it.
+    `ceiling`: the copy_ceiling record; with it every record carries `ceiling_frac`, its rate against what a plain
+    copy reaches on this machine (the practical ceiling of a stream), beside `hbm_frac` (against the 8 TB/s nameplate)."""
     def add(name, shape, nbytes, us, flops=0, note=None):
         rec = {"op": name, "shape": shape, "us": round(us, 3), "bytes": nbytes,
                "GBps": round(nbytes / us / 1e3, 1), "hbm_frac": round(nbytes / (us * 1e-6) / HBM_PEAK, 4)}
+        if ceiling:
+            rec["ceiling_frac"] = round(nbytes / us / 1e3 / ceiling["GBps"], 4)
         if flops:
             rec["TFLOPs"] = round(flops / us / 1e6, 2)
             rec["mfma_frac"] = round(flops / (us * 1e-6) / MFMA_F16_PEAK, 4)
@@ -242,13 +310,13 @@ def mat_mul_lines(o, gpu, stream, rng, add, launches=0):
         A_.free(); B_.free(); C_.free(); ws.free()
 
 
-def standalone_ops(ophip, gpu, stream, rng, reps):
+def standalone_ops(ophip, gpu, stream, rng, reps, ceiling=None):
     """Every operator at its benchmark shape plus a scaled shape that does not fit the Infinity Cache."""
     o, L, F16 = ophip, ophip.TensorLayout, ophip.dt.F16
     c = lambda *s: L.new_contiguous(F16, list(s))
     out = []
 
-    add = adder(out)
+    add = adder(out, ceiling)
 
     # rms_norm: [64, 4096] and [65536, 4096]
     rms = o.RmsNorm(gpu)
@@ -476,6 +544,8 @@ def main():
     ap.add_argument("--mat-mul-only", type=int, nargs="?", const=0, default=None, metavar="LAUNCHES",
                     help="only the compute-bound mat_mul shapes (not the benchmark line); with a number, that many "
                          "plain launches per shape, for hardware-counter runs")
+    ap.add_argument("--ceilings", action="store_true",
+                    help="only the machine's ceilings: stream probes (read, write, copy) and the bare MFMA loop")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -489,6 +559,9 @@ def main():
     log("device: %s (%s), %d CUs" % (info.name.decode(), info.arch.decode(), info.compute_units))
     stream = gpu.stream()
     rng = np.random.default_rng(0)
+    if args.ceilings:
+        print(json.dumps({"ceilings": ceilings(ophip, gpu, stream)}))
+        return
     if args.mat_mul_only is not None:
         lines = []
         mat_mul_lines(ophip, gpu, stream, rng, adder(lines), launches=args.mat_mul_only)
@@ -506,10 +579,12 @@ def main():
         layers[i % 2].step(stream)
     stream.synchronize()
 
-    # The dominant kernel is timed on every EVERY-th step only (an odd stride, so both weight sets are sampled):
+    # The dominant kernel is timed on every EVERY-th step only (an odd stride, so both weight sets are sampled;
+    # `roofline.samples` says how many launches that was):
     # its launch carries two events that the kernel itself records at its begin and its end (the figure the
     # rocprofv3 trace must agree with).
-    DOM, EVERY = "gate_up", 25  # (a launch that carries events costs the step about 4 us)
+    DOM = "gate_up"  # (a launch that carries events costs the step about 4 us: at most a quarter of the steps carry them)
+    EVERY = max(1, min(25, args.steps // 4)) | 1
     own = [(gpu.event(), gpu.event()) for _ in range(0, args.steps, EVERY)]
     t0 = time.perf_counter()
     for i in range(args.steps):
@@ -537,6 +612,7 @@ def main():
     event_pair_us = float(np.mean([a.elapsed_ms(b) for a, b in empties])) * 1e3
     dom_bytes = work[DOM][0]
 
+    ceiling = copy_ceiling(ophip, gpu, stream)
     # per-op times inside the layer (back-to-back launches of one op; small ops are cache-resident)
     per_layer = []
     log("decode layer, per op:")
@@ -544,7 +620,8 @@ def main():
         us = time_launches(gpu, stream, lambda: layers[0].launch(name, stream), args.reps)
         b, f = work[name]
         rec = {"op": name, "us": round(us, 3), "bytes": b, "GBps": round(b / us / 1e3, 1),
-               "hbm_frac": round(b / (us * 1e-6) / HBM_PEAK, 4)}
+               "hbm_frac": round(b / (us * 1e-6) / HBM_PEAK, 4),
+               "ceiling_frac": round(b / us / 1e3 / ceiling["GBps"], 4)}
         if f:
             rec["TFLOPs"] = round(f / us / 1e6, 2)
         if b < (256 << 20):
@@ -552,11 +629,10 @@ def main():
         per_layer.append(rec)
         log("  %-12s %9.2f us %9.1f GB/s %5.1f%% HBM" % (name, us, rec["GBps"], 100 * rec["hbm_frac"]))
 
-    ceiling = copy_ceiling(ophip, gpu, stream)
     per_op = []
     if not args.no_per_op:
         log("standalone operators:")
-        per_op = standalone_ops(ophip, gpu, stream, rng, args.reps)
+        per_op = standalone_ops(ophip, gpu, stream, rng, args.reps, ceiling)
 
     cpu = None
     if not args.no_cpu:
@@ -597,7 +673,7 @@ def main():
         "roofline": {"bound": "hbm", "kernel": "gemm_skinny (gate/up mat_mul 16x4096 . 4096x22016)",
                      "achieved": round(dom_bytes / (dom_us * 1e-6) / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(dom_bytes / (dom_us * 1e-6) / HBM_PEAK, 4), "traffic": profiled_traffic(),
-                     "us": round(dom_us, 3), "algorithmic_bytes": dom_bytes,
+                     "us": round(dom_us, 3), "samples": len(own), "algorithmic_bytes": dom_bytes,
                      "bracketed_us": round(bracketed_us, 3) if bracketed_us is not None else None,
                      "event_pair_us": round(event_pair_us, 3),
                      "note": "us is between two events the kernel's own launch records at its begin and end, inside the "

@@ -157,6 +157,14 @@ OPHIP_API int ophip_event_elapsed_ms(ophip_device *dev, ophip_event start, ophip
  * records around it.  An operator that launches several kernels times its first. */
 OPHIP_API int ophip_time_next_launch(ophip_device *dev, ophip_stream stream, ophip_event start, ophip_event stop);
 
+/* Measurement aid, no counterpart in the reference: one launch of a probe kernel, for ceilings measured on the machine
+ * at hand.  kind = "read", "read_nt" (non-temporal loads), "write", "copy": `blocks` workgroups of 256 threads stream
+ * `bytes` (a multiple of 16) from `src` and / or into `dst` (16-byte aligned; a read-only probe writes at most 16 bytes
+ * to dst).  kind = "mfma": `blocks` workgroups run `iters` trips of 128 v_mfma_f32_32x32x16_f16 per wave on operands made
+ * in registers from `seed` (0: all-zero operands) = blocks * 4 * iters * 128 * 32768 flop; dst needs blocks * 1024 bytes. */
+OPHIP_API int ophip_probe(ophip_device *dev, const char *kind, void *dst, const void *src, size_t bytes,
+                          unsigned iters, unsigned seed, unsigned blocks, ophip_stream stream);
+
 /* Launch graphs (no counterpart in the reference's driver crate): a fixed sequence of launch()
  * calls on `stream` between begin and end is recorded instead of run, and replayed by
  * ophip_graph_launch without per-launch host cost.  Give every recorded launch a workspace of

@@ -4,7 +4,9 @@
 // kernels: they plan workspace, build views and launch the three operators in the
 // reference's order, so the work lands on the queue exactly as the crate would put it.
 #include <cmath>
+#include <cstdlib>
 
+#include "../kernels/params.h"
 #include "handle.hpp"
 
 using namespace ophip;
@@ -232,11 +234,25 @@ struct ophip_attention_kv_cached {
     ophip_device *dev;
     ophip_rearrange *rearrange = nullptr;
     ophip_attention *attention = nullptr;
+    // the one-pass kernels for decode shapes: [16 * {1, 2, 4} query rows per kv head][dh 64 / 128]
+    hipFunction_t decode[3][2][2], combine[3][2];  // decode: [..][..][256 / 128 keys per workgroup]
+    bool one_pass = true;  // OPHIP_ATTN_ONE_PASS=0 keeps the composite (tests, comparisons); read once, here
+    int force_chunk = 0;   // OPHIP_ATTN_CHUNK=256|128 keeps one chunk size (sweeps)
     explicit ophip_attention_kv_cached(ophip_device *d) : dev(d) {
         ophip_device_retain(d);
         try {
             sub(ophip_rearrange_create(d, &rearrange));
             sub(ophip_attention_create(d, &attention));
+            static const char *mt_tag[3] = {"m1", "m2", "m4"}, *dh_tag[2] = {"d64", "d128"};
+            for (int i = 0; i < 3; ++i)
+                for (int j = 0; j < 2; ++j) {
+                    const std::string tail = std::string(mt_tag[i]) + "_" + dh_tag[j];
+                    decode[i][j][0] = d->kernel("attention_decode", ("attn_decode_" + tail + "_k64").c_str());
+                    decode[i][j][1] = d->kernel("attention_decode", ("attn_decode_" + tail + "_k32").c_str());
+                    combine[i][j] = d->kernel("attention_decode", ("attn_decode_combine_" + tail).c_str());
+                }
+            if (const char *e = std::getenv("OPHIP_ATTN_ONE_PASS")) one_pass = std::atoi(e) != 0;
+            if (const char *e = std::getenv("OPHIP_ATTN_CHUNK")) force_chunk = std::atoi(e);
         } catch (...) {
             release();
             throw;
@@ -279,6 +295,23 @@ KvCachedMeta kv_cached_meta(const ophip_attention_kv_cached_args &a) {
     return m;
 }
 
+// Keys per workgroup of the one-pass kernel: 256, or 128 when that leaves CUs without a workgroup (measured: the
+// decode layer, 32 kv heads x 2048 keys, 15.5 us with 256 keys against 17.0; 8 kv heads x 4096 keys 12.3 against 10.7).
+size_t decode_chunk(size_t nkvh, size_t att, unsigned cus, int force) {
+    if (force == 256 || force == 128) return (size_t)force;
+    return (att + 255) / 256 * nkvh < (size_t)cus ? 128 : 256;
+}
+
+// Workspace of the one-pass kernel for these sizes, or SIZE_MAX when it does not serve them (the shapes alone
+// decide here; launch also looks at strides and alignment).
+size_t one_pass_workspace(uint64_t dt, size_t nh, size_t nkvh, size_t seq, size_t att, size_t dh, size_t chunk) {
+    if (dt != OPHIP_DT_F16 || (dh != 64 && dh != 128) || nkvh == 0 || nh % nkvh != 0 || seq == 0 || att == 0) return SIZE_MAX;
+    const size_t rows = nh / nkvh * seq;
+    if (rows > 64 || att > 0x7fffffffu) return SIZE_MAX;
+    const size_t nchunk = (att + chunk - 1) / chunk, rp = rows <= 16 ? 16 : rows <= 32 ? 32 : 64;
+    return nchunk == 1 ? 0 : nkvh * nchunk * rp * (dh + 2) * sizeof(float);
+}
+
 // Operator::scheme (attention_kv_cached/operator.rs:42-77)
 size_t kv_cached_scheme(ophip_attention_kv_cached *op, const ophip_attention_kv_cached_args &args, size_t max_ws) {
     const KvCachedMeta m = kv_cached_meta(args);
@@ -297,7 +330,62 @@ size_t kv_cached_scheme(ophip_attention_kv_cached *op, const ophip_attention_kv_
     at.mask = args.mask;
     need = attention_scheme(op->attention, at, max_ws);
     wc.push_sub(need);
-    return wc.calculate(max_ws);
+    size_t ans = wc.calculate(max_ws);
+    // a launch of these sizes may run on the one-pass kernel instead: a workspace that serves either
+    if (op->one_pass && !is_dyn(m.nh) && !is_dyn(m.nkvh) && !is_dyn(m.dh) && !is_dyn(att)) {
+        const size_t fused = one_pass_workspace(m.dt, m.nh, m.nkvh, m.seq, att, m.dh,
+                                                decode_chunk(m.nkvh, att, (unsigned)op->dev->props.multiProcessorCount, op->force_chunk));
+        if (fused != SIZE_MAX && fused <= max_ws) ans = std::max(ans, fused);
+    }
+    return ans;
+}
+
+// The one-pass kernel (attention_decode.hip) when it serves this call; false, with nothing done, otherwise.
+bool kv_cached_one_pass(const ophip_attention_kv_cached *op, const ophip_attention_kv_cached_args &args, const KvCachedMeta &m,
+                        size_t pos, size_t att, void *workspace, size_t workspace_len, const ophip_queue_alloc *qa) {
+    if (!op->one_pass) return false;
+    const size_t nh = static_of(m.nh), nkvh = static_of(m.nkvh), seq = static_of(m.seq), dh = static_of(m.dh);
+    const size_t chunk = decode_chunk(nkvh, att, (unsigned)op->dev->props.multiProcessorCount, op->force_chunk);
+    const size_t need = one_pass_workspace(m.dt, nh, nkvh, seq, att, dh, chunk);
+    if (need == SIZE_MAX || (args.mask != OPHIP_MASK_NONE && args.mask != OPHIP_MASK_CAUSAL)) return false;
+    // every tensor: dh contiguous, rows and heads on 16-byte boundaries
+    auto fits = [](const ophip_tensor_layout &l, const void *base) {
+        for (int i = 0; i < 3; ++i)
+            if (is_dyn(l.strides[i])) return false;
+        return l.strides[2] == 2 && mult16(l.strides[0]) && mult16(l.strides[1]) && aligned16(base);
+    };
+    if (!fits(args.q_layout, args.q_base) || !fits(args.o_layout, args.o_base) || !fits(args.k_layout, args.k_base) ||
+        !fits(args.v_layout, args.v_base) || !fits(args.k_cache_layout, args.k_cache_base) || !aligned16(args.v_cache_base))
+        return false;
+    const size_t group = nh / nkvh, rows = group * seq;
+    AttnDecodeParams p{};
+    p.q = args.q_base;
+    p.o = args.o_base;
+    // the reference overwrites q with the result when q's heads and tokens merge (attention/operator.rs:186-239)
+    const ptrdiff_t nh_sq = args.q_layout.strides[0], seq_sq = args.q_layout.strides[1];
+    const bool merged = nh == 1 || seq == 1 || nh_sq == (ptrdiff_t)seq * seq_sq;
+    p.q_out = merged && args.q_base != args.o_base ? args.q_base : nullptr;
+    p.k_new = args.k_base;
+    p.v_new = args.v_base;
+    p.k_cache = args.k_cache_base;
+    p.v_cache = args.v_cache_base;
+    p.q_sh = nh_sq / 2, p.q_ss = seq_sq / 2;
+    p.o_sh = args.o_layout.strides[0] / 2, p.o_ss = args.o_layout.strides[1] / 2;
+    p.kn_sh = args.k_layout.strides[0] / 2, p.kn_ss = args.k_layout.strides[1] / 2;
+    p.vn_sh = args.v_layout.strides[0] / 2, p.vn_ss = args.v_layout.strides[1] / 2;
+    p.kc_sh = args.k_cache_layout.strides[0] / 2, p.kc_ss = args.k_cache_layout.strides[1] / 2;
+    p.nkvh = (uint32_t)nkvh, p.group = (uint32_t)group, p.seq = (uint32_t)seq, p.att = (uint32_t)att, p.pos = (uint32_t)pos;
+    p.nchunk = (uint32_t)((att + chunk - 1) / chunk);
+    p.causal = args.mask == OPHIP_MASK_CAUSAL;
+    p.scale = round_to_f16(1.0f / std::sqrt((float)dh));  // the reference's mat_mul rounds alpha to the data type
+    if (p.nchunk > 65535 || nkvh > 65535) return false;
+    Workspace ws(qa, workspace, workspace_len, need);
+    p.partial = static_cast<float *>(ws.ptr());
+    const int mi = rows <= 16 ? 0 : rows <= 32 ? 1 : 2, di = dh == 64 ? 0 : 1;
+    op->dev->make_current();
+    launch(op->decode[mi][di][chunk == 256 ? 0 : 1], Dim3{p.nchunk, (unsigned)nkvh}, Dim3{256}, 0, stream_of(qa), p);
+    if (p.nchunk > 1) launch(op->combine[mi][di], Dim3{(unsigned)(nkvh * rows)}, Dim3{256}, 0, stream_of(qa), p);
+    return true;
 }
 
 // Operator::launch (attention_kv_cached/operator.rs:79-183).  As in the reference, the
@@ -318,6 +406,7 @@ void kv_cached_launch(const ophip_attention_kv_cached *op, const ophip_attention
     // cache capacity
     const size_t att = pos + seq;
     if (buf_k < att || buf_v < att) throw shape_mismatch("Out of cache buffer");
+    if (kv_cached_one_pass(op, args, m, pos, att, workspace, workspace_len, qa)) return;
     // concatenate the new rows onto the caches: slice(1, pos, 1, seq)
     const Lay3 k_cat{{nkvh, seq, dh}, {nkvh_skc, buf_skc, dh_skc}};
     const Lay3 v_cat{{nkvh, seq, dh}, {nkvh_svc, buf_svc, dh_svc}};

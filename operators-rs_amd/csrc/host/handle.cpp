@@ -380,6 +380,24 @@ int ophip_time_next_launch(ophip_device *dev, ophip_stream stream, ophip_event s
     });
 }
 
+// Measurement probes (probe.hip): one launch of the named probe over `bytes` of memory (streams) or with `iters`
+// trips (mfma), `blocks` workgroups of 256 threads.
+int ophip_probe(ophip_device *dev, const char *kind, void *dst, const void *src, size_t bytes, unsigned iters,
+                unsigned seed, unsigned blocks, ophip_stream stream) {
+    return guard([&] {
+        if (!dev || !kind) throw args_not_support("null argument");
+        const std::string k = kind;
+        const bool reads = k == "read" || k == "read_nt" || k == "copy", writes = k == "write" || k == "copy";
+        if (!reads && !writes && k != "mfma") throw args_not_support("unknown probe: " + k);
+        if ((reads && !src) || !dst || blocks == 0) throw args_not_support("probe: null buffer or empty grid");
+        if ((reads || writes) && (bytes % 16 != 0 || !aligned16(dst) || (reads && !aligned16(src))))
+            throw args_not_support("probe: buffers in whole 16-byte vectors");
+        ProbeParams p{dst, src, (uint64_t)bytes, iters, seed};
+        dev->make_current();
+        launch(dev->kernel("probe", ("probe_" + k).c_str()), Dim3{blocks}, Dim3{256}, 0, (hipStream_t)stream, p);
+    });
+}
+
 // ---- launch graphs ------------------------------------------------------------
 // Every launch() of this library only enqueues kernels (and stream-ordered allocations) on
 // the caller's stream, so a fixed sequence of them can be recorded once and replayed.

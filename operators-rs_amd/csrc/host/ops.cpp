@@ -2,7 +2,9 @@
 // argument validation as in the reference's Args::meta / Scheme::new, kernel
 // selection, and asynchronous launch on the caller's queue.
 #include <algorithm>
+#include <cmath>
 #include <cstring>
+#include <mutex>
 
 #include "../kernels/params.h"
 #include "handle.hpp"
@@ -11,7 +13,7 @@ using namespace ophip;
 
 namespace {
 
-const char *dt_tag(uint64_t dt) { return dt == OPHIP_DT_F16 ? "f16" : dt == OPHIP_DT_F32 ? "f32" : "?"; }
+const char *dt_tag(uint64_t dt) { return dt == OPHIP_DT_F16 ? "f16" : dt == OPHIP_DT_F32 ? "f32" : dt == OPHIP_DT_F64 ? "f64" : "?"; }
 
 }  // namespace
 
@@ -37,9 +39,10 @@ static RmsNormMeta rms_norm_meta(const ophip_rms_norm_args &a) {
 }
 
 static void rms_norm_check_types(uint64_t dt_a, uint64_t dt_w) {
+    // the pairs of the CPU backend (rms_norm/common_cpu/mod.rs:84-90); anything else is `todo!()` there
     const bool ok = (dt_a == OPHIP_DT_F16 && (dt_w == OPHIP_DT_F16 || dt_w == OPHIP_DT_F32)) ||
-                    (dt_a == OPHIP_DT_F32 && dt_w == OPHIP_DT_F32);
-    if (!ok) throw type_not_support("rms_norm supports (a, w) in {(f16, f16), (f16, f32), (f32, f32)}");
+                    (dt_a == OPHIP_DT_F32 && dt_w == OPHIP_DT_F32) || (dt_a == OPHIP_DT_F64 && dt_w == OPHIP_DT_F64);
+    if (!ok) throw type_not_support("rms_norm supports (a, w) in {(f16, f16), (f16, f32), (f32, f32), (f64, f64)}");
 }
 
 struct RmsKey {
@@ -62,7 +65,11 @@ struct ophip_rms_norm : OpBase {
     RmsScheme scheme_for(const RmsKey &key) const {
         return schemes.get_or_insert(key, [&] {
             const std::string base = std::string("rms_norm_") + dt_tag(key.dt_a) + "_" + dt_tag(key.dt_w);
-            RmsScheme s;
+            RmsScheme s{};
+            if (key.dt_a == OPHIP_DT_F64) {  // one kernel only
+                s.scalar = dev->kernel("rms_norm", (base + "_scalar").c_str());
+                return s;
+            }
             s.g64 = dev->kernel("rms_norm", (base + "_g64").c_str());
             s.g256 = dev->kernel("rms_norm", (base + "_g256").c_str());
             s.g1024 = dev->kernel("rms_norm", (base + "_g1024").c_str());
@@ -105,6 +112,7 @@ extern "C" int ophip_rms_norm_launch(const ophip_rms_norm *op, const ophip_rms_n
             throw strides_not_support("rms_norm needs contiguous inner dimensions");
         if (n == 0 || d == 0) return;
         if (n > 0x7fffffffu || d > 0x7fffffffu) throw shape_not_support("rms_norm dimension too large");
+        if (!args->y_base || !args->x_base || !args->w_base) throw args_not_support("rms_norm: null base pointer");
 
         const RmsScheme s = op->scheme_for(RmsKey{m.dt_a, m.dt_w, d});
         RmsNormParams p{};
@@ -118,7 +126,7 @@ extern "C" int ophip_rms_norm_launch(const ophip_rms_norm *op, const ophip_rms_n
         p.epsilon = args->epsilon;
 
         const size_t vec_elems = 16 / (size_t)unit;
-        const bool vec = d % vec_elems == 0 && aligned16(p.y) && aligned16(p.x) && aligned16(p.w) && mult16(nsy) &&
+        const bool vec = m.dt_a != OPHIP_DT_F64 && d % vec_elems == 0 && aligned16(p.y) && aligned16(p.x) && aligned16(p.w) && mult16(nsy) &&
                          mult16(nsx);
         op->dev->make_current();
         if (!vec) {
@@ -170,6 +178,20 @@ static RopeMeta rope_meta(const ophip_rope_args &a) {
 
 struct ophip_rope : OpBase {
     hipFunction_t f16_vec, f16_pairs, f32_pairs;
+    // theta^(k / (dh/2)) of the last (theta, dh) launched: a model has one such pair
+    mutable std::mutex den_mu;
+    mutable float den_theta = 0.f;
+    mutable size_t den_half = 0;
+    mutable float den[128];
+    void denominators(float theta, size_t half, float *out) const {
+        std::lock_guard<std::mutex> lock(den_mu);
+        if (den_half != half || den_theta != theta) {
+            for (size_t k = 0; k < half; ++k) den[k] = std::pow(theta, (float)k / (float)half);  // powf, as the reference's
+            den_theta = theta;
+            den_half = half;
+        }
+        std::memcpy(out, den, half * sizeof(float));
+    }
     explicit ophip_rope(ophip_device *d) : OpBase(d) {
         f16_vec = d->kernel("rope", "rope_f16_vec");
         f16_pairs = d->kernel("rope", "rope_f16_pairs");
@@ -220,6 +242,8 @@ extern "C" int ophip_rope_launch(const ophip_rope *op, const ophip_rope_args *ar
         p.dh = (uint32_t)dh;
         p.theta = args->theta;
         p.pos_is_u64 = m.dt_p == OPHIP_DT_U64;
+        p.has_den = dh / 2 <= 128;
+        if (p.has_den) op->denominators(args->theta, dh / 2, p.den);
 
         const bool vec = m.dt_t == OPHIP_DT_F16 && dh % 8 == 0 && aligned16(p.t) && mult16(st) && mult16(sh);
         // split a token's heads over blockIdx.y when there are few tokens, keeping >= 256 items per block
@@ -287,7 +311,7 @@ struct SoftmaxVariant {
 
 struct ophip_fused_softmax : OpBase {
     std::vector<SoftmaxVariant> variants;
-    hipFunction_t stream_fn;
+    hipFunction_t stream_fn, rows4[2];  // rows4: four rows per wave, 1 or 2 vectors per lane and row
     explicit ophip_fused_softmax(ophip_device *d) : OpBase(d) {
         static const int table[][3] = {{8, 1, 64},  {8, 2, 64},   {8, 4, 64},   {8, 1, 256},  {8, 2, 256},
                                        {8, 4, 256}, {8, 8, 256},  {8, 4, 1024}, {8, 8, 1024}, {1, 8, 64},
@@ -298,6 +322,8 @@ struct ophip_fused_softmax : OpBase {
             variants.push_back({t[0], t[1], t[2], d->kernel("fused_softmax", name.c_str())});
         }
         stream_fn = d->kernel("fused_softmax", "softmax_f16_stream");
+        rows4[0] = d->kernel("fused_softmax", "softmax_f16_rows4_p1");
+        rows4[1] = d->kernel("fused_softmax", "softmax_f16_rows4_p2");
     }
 };
 
@@ -358,6 +384,13 @@ extern "C" int ophip_fused_softmax_launch(const ophip_fused_softmax *op, const o
             if (!pick || v.g < pick->g || (v.g == pick->g && v.pt < pick->pt)) pick = &v;
         }
         op->dev->make_current();
+        if (vec && att <= 1024 && rows >= 8192) {
+            // many short rows: four per wave, their loads in flight together (16384 waves of one 512-column row
+            // each cost more in start-up than in traffic: [32, 512, 512] causal 9.6 -> see the kernel's note)
+            const size_t waves = nh * ((seq + 3) / 4);
+            launch(op->rows4[att <= 512 ? 0 : 1], Dim3{ceil_div(waves, 4)}, Dim3{256}, 0, stream_of(qa), p);
+            return;
+        }
         if (!pick) {
             launch(op->stream_fn, Dim3{(unsigned)rows}, Dim3{1024}, 0, stream_of(qa), p);
             return;
@@ -459,11 +492,12 @@ extern "C" int ophip_rearrange_plan(const ophip_rearrange_args *args, ptrdiff_t 
 }
 
 struct ophip_rearrange : OpBase {
-    hipFunction_t k32[5], k64[5];  // chunk sizes 16, 8, 4, 2, 1
+    hipFunction_t k32[5], k32_one[5], k64[5];  // chunk sizes 16, 8, 4, 2, 1; k32_one: one chunk per thread
     explicit ophip_rearrange(ophip_device *d) : OpBase(d) {
         static const int sizes[5] = {16, 8, 4, 2, 1};
         for (int i = 0; i < 5; ++i) {
             k32[i] = d->kernel("rearrange", ("rearrange_b" + std::to_string(sizes[i])).c_str());
+            k32_one[i] = d->kernel("rearrange", ("rearrange1_b" + std::to_string(sizes[i])).c_str());
             k64[i] = d->kernel("rearrange", ("rearrange64_b" + std::to_string(sizes[i])).c_str());
         }
     }
@@ -575,8 +609,11 @@ extern "C" int ophip_rearrange_launch(const ophip_rearrange *op, const ophip_rea
         if (small) {
             p.cpu_div = make_fastdiv((uint32_t)cpu);
             for (size_t i = 0; i < nd; ++i) p.idx_div[i] = make_fastdiv((uint32_t)o_idx[i + 1]);
-            const unsigned per_block = 256 * 4;  // RE_ITEMS chunks per thread
-            launch(op->k32[ci], Dim3{ceil_div(p.total, per_block)}, Dim3{256}, 0, stream_of(qa), p);
+            // four chunks per thread, unless that leaves fewer than eight workgroups per CU: then one
+            const unsigned cus = (unsigned)op->dev->props.multiProcessorCount;
+            const bool one = p.total < (uint64_t)cus * 8 * 256 * 4;
+            launch(one ? op->k32_one[ci] : op->k32[ci], Dim3{ceil_div(p.total, one ? 256 : 256 * 4)}, Dim3{256}, 0,
+                   stream_of(qa), p);
         } else {
             if (cpu > 0xffffffffu) throw shape_not_support("rearrange unit too large");
             const uint64_t blocks = std::min<uint64_t>((p.total + 255) / 256, 1u << 20);

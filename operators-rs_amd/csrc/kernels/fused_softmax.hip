@@ -100,6 +100,111 @@ __device__ __forceinline__ void softmax_reg(const SoftmaxParams &p) {
     }
 }
 
+// Many short rows (a prefill's [nh, seq, att <= 1024] scores): a wave that serves one row of 512 columns lives for
+// one load, two reductions and one store, and 16384 such waves cost more in start-up than in traffic.  Here a wave
+// takes four rows at once, all their loads in flight together; under a causal mask the four are two pairs
+// (r, seq - 1 - r), so every wave moves the same number of bytes whatever its place in the triangle.
+// 16-byte aligned rows only; PT 16-byte vectors per lane and row (att_len <= 512 * PT).
+template <int PT>
+__device__ __forceinline__ void softmax_rows4(const SoftmaxParams &p) {
+    constexpr int ROWS = 4;
+    const uint32_t lane = threadIdx.x % WAVE;
+    const uint32_t per_head = (p.seq + ROWS - 1) / ROWS;  // waves per head
+    const uint32_t w = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+    if (w >= p.nh * per_head) return;  // (no barrier in this kernel)
+    const uint32_t h = w / per_head, j = w - h * per_head;
+    const bool paired = p.seq % ROWS == 0;
+
+    f16 *row[ROWS];
+    uint32_t kept[ROWS];
+    bool live[ROWS];
+    float x[ROWS][PT][8];
+    float mx[ROWS];
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i) {
+        uint32_t r = paired ? (i % 2 == 0 ? 2 * j + i / 2 : p.seq - 1 - (2 * j + i / 2)) : ROWS * j + i;
+        live[i] = r < p.seq;
+        if (!live[i]) r = p.seq - 1;
+        kept[i] = kept_columns(p, r);
+        row[i] = reinterpret_cast<f16 *>(reinterpret_cast<char *>(p.att) + (int64_t)h * p.sh + (int64_t)r * p.ss);
+    }
+    Pack8 v[ROWS][PT];
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i)
+#pragma unroll
+        for (int q = 0; q < PT; ++q) {
+            const uint32_t col0 = (lane + q * WAVE) * 8;
+            v[i][q].u = u32x4{0, 0, 0, 0};
+            if (col0 + 8 <= p.att_len) {
+                if (col0 < kept[i]) v[i][q].u = ld128(row[i] + col0);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 7; ++e)
+                    if (col0 + e < kept[i]) v[i][q].e[e] = row[i][col0 + e];
+            }
+        }
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i) {
+        mx[i] = -INFINITY;
+#pragma unroll
+        for (int q = 0; q < PT; ++q)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const uint32_t col = (lane + q * WAVE) * 8 + e;
+                x[i][q][e] = col < kept[i] ? h2f(v[i][q].e[e]) : -INFINITY;
+                mx[i] = fmaxf(mx[i], x[i][q][e]);
+            }
+    }
+#pragma unroll
+    for (int o = WAVE / 2; o > 0; o >>= 1)
+#pragma unroll
+        for (int i = 0; i < ROWS; ++i) mx[i] = fmaxf(mx[i], __shfl_xor(mx[i], o, WAVE));
+    float sum[ROWS];
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i) {
+        sum[i] = 0.f;
+#pragma unroll
+        for (int q = 0; q < PT; ++q)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const uint32_t col = (lane + q * WAVE) * 8 + e;
+                if (col < kept[i]) {
+                    const float ex = fast_exp(x[i][q][e] - mx[i]);
+                    sum[i] += ex;
+                    x[i][q][e] = h2f(f2h(ex));  // the reference stores f16(e) and re-reads it
+                } else {
+                    x[i][q][e] = 0.f;
+                }
+            }
+    }
+#pragma unroll
+    for (int o = WAVE / 2; o > 0; o >>= 1)
+#pragma unroll
+        for (int i = 0; i < ROWS; ++i) sum[i] += __shfl_xor(sum[i], o, WAVE);
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i) {
+        const float inv = 1.0f / sum[i];
+#pragma unroll
+        for (int q = 0; q < PT; ++q) {
+            const uint32_t col0 = (lane + q * WAVE) * 8;
+            if (col0 < p.att_len && live[i]) {
+                Pack8 o;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o.e[e] = col0 + e < kept[i] ? f2h(x[i][q][e] * inv) : (f16)0.f;
+                if (col0 + 8 <= p.att_len) {
+                    st128(row[i] + col0, o.u);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 7; ++e)
+                        if (col0 + e < p.att_len) row[i][col0 + e] = o.e[e];
+                }
+            }
+        }
+    }
+}
+extern "C" __global__ void __launch_bounds__(256) softmax_f16_rows4_p1(SoftmaxParams p) { softmax_rows4<1>(p); }
+extern "C" __global__ void __launch_bounds__(256) softmax_f16_rows4_p2(SoftmaxParams p) { softmax_rows4<2>(p); }
+
 // Any att_len: one 1024-thread workgroup per row, three sweeps (max; exp + sum,
 // storing f16(e); scale), O(1) LDS.
 extern "C" __global__ void __launch_bounds__(1024) softmax_f16_stream(SoftmaxParams p) {

@@ -36,6 +36,10 @@ struct RopeParams {
     float theta;
     uint32_t pos_is_u64;
     uint32_t heads_per_block;
+    // theta^(k / (dh/2)) for k < dh/2, evaluated by the host's powf (what the reference's CPU backend divides by) when
+    // dh <= 256; has_den = 0: the kernel evaluates powf itself
+    uint32_t has_den;
+    float den[128];
 };
 
 struct SoftmaxParams {
@@ -74,6 +78,27 @@ struct SampleParams {
     // hold top_p of the probability (0: the result is written; 1: the next kernel in line has to do the row).
     // Bit 0: write that word; bit 1: read it first and leave the row alone if it is 0.
     uint32_t verify_cover;
+};
+
+// attention_kv_cached in one pass (attention_decode.hip).  Strides in elements; the v-cache is addressed with the
+// k-cache's strides, as in the reference.
+struct AttnDecodeParams {
+    const void *q;
+    void *q_out;  // q again when the reference would overwrite it with the result (its heads and tokens merge), else null
+    void *o;
+    const void *k_new, *v_new;  // the rows being appended: [nkvh, seq, dh]
+    void *k_cache, *v_cache;
+    float *partial;  // several chunks: [nkvh][nchunk] blocks of 16 * MT rows x (dh + 2) floats
+    int64_t q_sh, q_ss, o_sh, o_ss, kn_sh, kn_ss, vn_sh, vn_ss, kc_sh, kc_ss;
+    uint32_t nkvh, group, seq, att, pos, nchunk, causal;
+    float scale;
+};
+
+struct ProbeParams {  // probe.hip
+    void *dst;
+    const void *src;
+    uint64_t bytes;
+    uint32_t iters, seed;
 };
 
 // Canonical GEMM seen by the kernels:

@@ -25,9 +25,9 @@ struct Chunk<2> { typedef uint16_t T; };
 template <>
 struct Chunk<1> { typedef uint8_t T; };
 
-constexpr int RE_ITEMS = 4;  // chunks per thread, loads issued before stores
-
-template <int B>
+// RE_ITEMS chunks per thread, loads issued before stores: 4 for large copies; 1 for mid-size ones, which would
+// otherwise leave the machine with one workgroup per CU or less (8 MB: 256 workgroups at 4 chunks per thread).
+template <int B, int RE_ITEMS>
 __device__ __forceinline__ void rearrange32(const RearrangeParams &p) {
     typedef typename Chunk<B>::T T;
     const uint32_t total = (uint32_t)p.total;
@@ -82,7 +82,10 @@ __device__ __forceinline__ void rearrange64(const RearrangeParams &p) {
 
 #define REARRANGE(B)                                                                             \
     extern "C" __global__ void __launch_bounds__(256) rearrange_b##B(RearrangeParams p) {       \
-        rearrange32<B>(p);                                                                       \
+        rearrange32<B, 4>(p);                                                                    \
+    }                                                                                            \
+    extern "C" __global__ void __launch_bounds__(256) rearrange1_b##B(RearrangeParams p) {      \
+        rearrange32<B, 1>(p);                                                                    \
     }                                                                                            \
     extern "C" __global__ void __launch_bounds__(256) rearrange64_b##B(RearrangeParams p) {     \
         rearrange64<B>(p);                                                                       \

@@ -276,3 +276,23 @@ RMS_VEC(rms_norm_f32_f32_g1024, float, float, 1024)
 RMS_SCALAR(rms_norm_f16_f16_scalar, f16, f16)
 RMS_SCALAR(rms_norm_f16_f32_scalar, f16, float)
 RMS_SCALAR(rms_norm_f32_f32_scalar, float, float)
+
+// f64 rows with f64 weights (rms_norm/common_cpu/mod.rs:84-90 lists the pair): all arithmetic in f64, as the
+// reference's, one workgroup per row.  No vector variant: the hot path is f16.
+extern "C" __global__ void __launch_bounds__(256) rms_norm_f64_f64_scalar(RmsNormParams p) {
+    constexpr int G = 256;
+    __shared__ double smem[G / WAVE];
+    const uint32_t row = blockIdx.x;
+    const double *xr = reinterpret_cast<const double *>(reinterpret_cast<const char *>(p.x) + (int64_t)row * p.nsx);
+    double *yr = reinterpret_cast<double *>(reinterpret_cast<char *>(p.y) + (int64_t)row * p.nsy);
+    const double *w = reinterpret_cast<const double *>(p.w);
+    double ss = 0.0;
+    for (uint32_t j = threadIdx.x; j < p.d; j += G) ss += xr[j] * xr[j];
+#pragma unroll
+    for (int o = WAVE / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, WAVE);
+    if ((threadIdx.x & (WAVE - 1)) == 0) smem[threadIdx.x / WAVE] = ss;
+    __syncthreads();
+    ss = (smem[0] + smem[1]) + (smem[2] + smem[3]);
+    const double k = 1.0 / sqrt(ss / (double)p.d + (double)p.epsilon);
+    for (uint32_t j = threadIdx.x; j < p.d; j += G) yr[j] = (k * w[j]) * xr[j];
+}

@@ -21,9 +21,13 @@ __device__ __forceinline__ float rope_pos(const RopeParams &p, uint32_t token) {
 __device__ __forceinline__ void rope_fill_table(const RopeParams &p, uint32_t token) {
     const uint32_t H = p.dh / 2;
     const float pos = rope_pos(p, token);
-    for (uint32_t k = threadIdx.x; k < H; k += blockDim.x) {
-        const float ang = pos / powf(p.theta, (float)k / (float)H);
-        rope_sc[k] = make_float2(sinf(ang), cosf(ang));
+    // one entry of the table per thread, the sines by the first H threads and the cosines by the next H: the
+    // table is the kernel's critical path (everything else waits for it at the barrier)
+    float *flat = reinterpret_cast<float *>(rope_sc);
+    for (uint32_t e = threadIdx.x; e < 2 * H; e += blockDim.x) {
+        const uint32_t k = e < H ? e : e - H;
+        const float ang = pos / (p.has_den ? p.den[k] : powf(p.theta, (float)k / (float)H));
+        flat[2 * k + (e < H ? 0 : 1)] = e < H ? sinf(ang) : cosf(ang);
     }
     __syncthreads();
 }

@@ -204,7 +204,7 @@ EXPORTS = [
     "ophip_malloc", "ophip_free", "ophip_memcpy_h2d", "ophip_memcpy_d2h", "ophip_memcpy_d2d", "ophip_memset",
     "ophip_stream_create", "ophip_stream_destroy", "ophip_stream_synchronize",
     "ophip_event_create", "ophip_event_destroy", "ophip_event_record", "ophip_event_synchronize",
-    "ophip_event_elapsed_ms", "ophip_time_next_launch",
+    "ophip_event_elapsed_ms", "ophip_time_next_launch", "ophip_probe",
     "ophip_stream_begin_capture", "ophip_stream_end_capture", "ophip_graph_launch", "ophip_graph_destroy",
     "ophip_queue_alloc_from_stream", "ophip_mem_pool_create", "ophip_mem_pool_put",
     "ophip_mem_pool_queue_alloc", "ophip_mem_pool_destroy",

@@ -4,7 +4,7 @@ types), so that a test can compare them declaration by declaration without a C o
 import re
 
 _SCALARS = {
-    "void": "c_void", "int": "c_int", "char": "c_char", "float": "f32", "double": "f64", "size_t": "usize",
+    "void": "c_void", "int": "c_int", "unsigned": "c_uint", "char": "c_char", "float": "f32", "double": "f64", "size_t": "usize",
     "ptrdiff_t": "isize", "uint8_t": "u8", "uint16_t": "u16", "uint32_t": "u32", "uint64_t": "u64", "int32_t": "i32",
     "int64_t": "i64",
 }

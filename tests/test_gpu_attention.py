@@ -159,6 +159,81 @@ def test_attention_kv_cached(gpu, stream, nh, nkvh, seq, dh, buf, pos):
     assert_close_f16(out, attention_f64(q, kc_ref[:, :pos + seq], vc_ref[:, :pos + seq], True), "kv cached vs f64")
 
 
+def kv_cached_case(gpu, stream, op, nh, nkvh, seq, dh, buf, pos, mask, rng, strided=False):
+    """One launch on fresh buffers; returns (o, q afterwards, k cache, v cache) and the host inputs."""
+    q, k, v = normal_f16(rng, (nh, seq, dh)), normal_f16(rng, (nkvh, seq, dh)), normal_f16(rng, (nkvh, seq, dh))
+    kc, vc = normal_f16(rng, (nkvh, buf, dh)), normal_f16(rng, (nkvh, buf, dh))
+    lay = TensorLayout.of
+    if strided:
+        # q, k, v as the head-major views of one token-major [seq, (nh + 2 nkvh) * dh] buffer (a fused QKV
+        # product), o as the same view of a [seq, nh * dh] buffer: heads and tokens do not merge
+        row = (nh + 2 * nkvh) * dh
+        qkv = np.zeros((seq, row), f16)
+        qkv[:, :nh * dh] = q.transpose(1, 0, 2).reshape(seq, nh * dh)
+        qkv[:, nh * dh:(nh + nkvh) * dh] = k.transpose(1, 0, 2).reshape(seq, nkvh * dh)
+        qkv[:, (nh + nkvh) * dh:] = v.transpose(1, 0, 2).reshape(seq, nkvh * dh)
+        qkv_d = upload(gpu, qkv)
+        q_lay = TensorLayout(dt.F16, [nh, seq, dh], [dh * 2, row * 2, 2])
+        kv_lay = TensorLayout(dt.F16, [nkvh, seq, dh], [dh * 2, row * 2, 2])
+        o_lay = TensorLayout(dt.F16, [nh, seq, dh], [dh * 2, nh * dh * 2, 2])
+        qd, kd, vd = qkv_d.ptr, qkv_d.ptr + nh * dh * 2, qkv_d.ptr + (nh + nkvh) * dh * 2
+        k_lay = v_lay = kv_lay
+    else:
+        qd, kd, vd = (upload(gpu, a) for a in (q, k, v))
+        q_lay, k_lay, v_lay, o_lay = lay(q), lay(k), lay(v), lay(q)
+    kcd, vcd = upload(gpu, kc), upload(gpu, vc)
+    od = gpu.malloc(q.nbytes)
+    gpu.memset(od, 0)
+    args = ophip.AttnKVCachedArgs(q_lay, qd, k_lay, kd, v_lay, vd, o_lay, od, lay(kc), kcd, lay(vc), vcd, mask, pos)
+    op.scheme(args, 2 ** 40)
+    op.launch(args, None, stream)
+    if strided:
+        out = download(gpu, stream, od, np.zeros((seq, nh, dh), f16)).transpose(1, 0, 2)
+        q_after = download(gpu, stream, qkv_d, qkv)[:, :nh * dh].reshape(seq, nh, dh).transpose(1, 0, 2)
+    else:
+        out, q_after = download(gpu, stream, od, q), download(gpu, stream, qd, q)
+    return out, q_after, download(gpu, stream, kcd, kc), download(gpu, stream, vcd, vc), (q, k, v, kc, vc)
+
+
+@pytest.mark.parametrize("nh,nkvh,seq,dh,buf,pos,mask,strided", [
+    (32, 32, 16, 128, 2048, 2032, CAUSAL, True),    # the decode layer, q / k / v inside a fused QKV buffer
+    (32, 8, 1, 128, 4096, 4095, CAUSAL, False),     # one token, grouped heads: 4 rows per kv head, 16 chunks
+    (32, 4, 7, 64, 160, 120, CAUSAL, False),        # attention_kv_cached/cuda.rs: 56 rows per kv head, one chunk
+    (32, 4, 7, 64, 1500, 1017, CAUSAL, True),       # the same over 4 chunks, the last one ragged (att 1024)
+    (8, 8, 16, 64, 700, 0, CAUSAL, False),          # empty cache: everything comes from k and v
+    (12, 4, 5, 128, 300, 251, NONE, False),         # no mask: 15 rows, att 256 = exactly one chunk
+    (12, 4, 5, 128, 300, 252, NONE, False),         # att 257: a second chunk with one key
+    (16, 2, 8, 128, 520, 500, CAUSAL, False),       # 64 rows per kv head, the append straddles chunks 1 and 2
+    (3, 3, 33, 64, 100, 10, CAUSAL, False),         # 33 rows per kv head
+])
+def test_attention_kv_cached_one_pass(gpu, stream, monkeypatch, nh, nkvh, seq, dh, buf, pos, mask, strided):
+    """Decode shapes run on the one-pass kernel: against the oracle's composite (which rounds the scores and the
+    probabilities to f16 between the steps), against f64, and against the composite of launches
+    (OPHIP_ATTN_ONE_PASS=0) for everything the reference makes observable: o, the appended cache rows bit for bit
+    and the rest of the caches untouched, q overwritten with the result when its heads and tokens merge and left
+    alone when they do not."""
+    say("kv cached one pass nh=%d nkvh=%d seq=%d dh=%d buf=%d pos=%d strided=%s" % (nh, nkvh, seq, dh, buf, pos, strided))
+    fused = ophip.AttnKVCached(gpu)
+    monkeypatch.setenv("OPHIP_ATTN_ONE_PASS", "0")
+    composite = ophip.AttnKVCached(gpu)  # the switch is read when an operator is created
+    monkeypatch.delenv("OPHIP_ATTN_ONE_PASS")
+    seed = nh * 7919 + buf * 31 + pos
+    out, q_after, kc_out, vc_out, (q, k, v, kc, vc) = kv_cached_case(gpu, stream, fused, nh, nkvh, seq, dh, buf, pos, mask,
+                                                                     np.random.default_rng(seed), strided)
+    out_c, q_after_c, kc_c, vc_c, _ = kv_cached_case(gpu, stream, composite, nh, nkvh, seq, dh, buf, pos, mask,
+                                                     np.random.default_rng(seed), strided)
+    kc_ref, vc_ref = kc.copy(), vc.copy()
+    ref = oracle.attention_kv_cached(q.copy(), k, v, np.zeros_like(q), kc_ref, vc_ref, pos, causal=(mask == CAUSAL))
+    assert np.array_equal(kc_out, kc_ref) and np.array_equal(vc_out, vc_ref)
+    assert np.array_equal(kc_c, kc_ref) and np.array_equal(vc_c, vc_ref)
+    assert_close_f16(out, ref, "one pass vs oracle")
+    assert_close_f16(out, attention_f64(q, kc_ref[:, :pos + seq], vc_ref[:, :pos + seq], mask == CAUSAL), "one pass vs f64")
+    assert_close_f16(out, out_c, "one pass vs composite")
+    merged = not strided or nh == 1 or seq == 1
+    assert np.array_equal(q_after, out if merged else q)
+    assert np.array_equal(q_after_c, out_c if merged else q)
+
+
 def test_attention_kv_cached_errors_and_scheme(gpu, stream):
     op = ophip.AttnKVCached(gpu)
     c = lambda *s: TensorLayout.new_contiguous(dt.F16, list(s))

@@ -78,6 +78,35 @@ def test_attention_repeats_bit_for_bit(gpu, stream, nh, nkvh, seq, att, dh):
     assert not np.isnan(out.view(f16)).any(), what
 
 
+@pytest.mark.parametrize("nh,nkvh,seq,dh,buf,pos", [(32, 32, 16, 128, 2048, 2032), (32, 4, 7, 64, 1500, 1017),
+                                                    (64, 8, 1, 128, 8192, 8000)])
+def test_attention_kv_cached_one_pass_repeats_bit_for_bit(gpu, stream, nh, nkvh, seq, dh, buf, pos):
+    """The one-pass kernel hands every chunk's maximum, sum and partial output to a second launch through the
+    workspace (8, 4 and 63 chunks here; the last case takes 128 keys per workgroup): the same bits every time, o and
+    both caches, over a workspace of NaNs."""
+    rng = np.random.default_rng(nh + buf + pos)
+    q, k, v = normal_f16(rng, (nh, seq, dh)), normal_f16(rng, (nkvh, seq, dh)), normal_f16(rng, (nkvh, seq, dh))
+    kc, vc = normal_f16(rng, (nkvh, buf, dh)), normal_f16(rng, (nkvh, buf, dh))
+    o = np.zeros((nh, seq, dh), f16)
+    qd, kd, vd, od, kcd, vcd = (gpu.from_host(x) for x in (q, k, v, o, kc, vc))
+    lay = TensorLayout.of
+    op = ophip.AttnKVCached(gpu)
+    args = ophip.AttnKVCachedArgs(lay(q), qd, lay(k), kd, lay(v), vd, lay(o), od, lay(kc), kcd, lay(vc), vcd, 1, pos)
+    ws = gpu.malloc(max(op.scheme(args, 2 ** 40), 16))
+    what = "attention_kv_cached one pass %s" % ((nh, nkvh, seq, dh, buf, pos),)
+    print(what, flush=True)
+
+    def launch():
+        gpu.upload(qd, q, stream=stream)  # the operator leaves its result in q as well
+        stream.synchronize()
+        op.launch(args, ws, stream)
+
+    out = repeat(gpu, stream, launch, od, o.nbytes, ws, what)
+    assert not np.isnan(out.view(f16)).any(), what
+    k_after = gpu.to_host(kcd, f16, kc.size, stream=stream).reshape(kc.shape)
+    assert np.array_equal(k_after[:, pos:pos + seq], k) and np.array_equal(k_after[:, :pos], kc[:, :pos])
+
+
 @pytest.mark.parametrize("rows,n,top_k,top_p", [(16, 32000, 50, 0.9), (4, 128256, 50, 0.9), (4, 32000, 2000, 0.95),
                                                 (2, 50000, 2 ** 62, 0.9)])
 def test_random_sample_repeats_bit_for_bit(gpu, stream, rows, n, top_k, top_p):
