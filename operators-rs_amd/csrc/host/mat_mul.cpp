@@ -435,13 +435,14 @@ static void mat_mul_launch_impl(const ophip_mat_mul *op, const ophip_mat_mul_arg
         g.p.partial = ws.ptr();
         const size_t tiles = (size_t)((p.N + 127) / 128) * p.batch;
         if (fixed) {
-            g.p.counters = (p.split_k > 1 && tiles <= fixed_counter_count) ? fixed_counters : nullptr;
+            g.p.counters = (p.split_k > 1 && tiles <= fixed_counter_count && g.workspace < ((size_t)1 << 32)) ? fixed_counters : nullptr;
             if (g.p.counters) {  // the static buffer keeps what the last call left: start this launch's counters at zero
                 FillU32Params f{fixed_counters, (uint32_t)tiles, 0u};
                 launch(op->fill, Dim3{(unsigned)((tiles + 255) / 256)}, Dim3{256}, 0, stream, f);
             }
         } else {
-            g.p.counters = (p.split_k > 1 && tiles <= SPLITK_COUNTERS) ? op->counters_for(stream) : nullptr;
+            // (the in-kernel reduction addresses the partials with 32-bit offsets)
+            g.p.counters = (p.split_k > 1 && tiles <= SPLITK_COUNTERS && g.workspace < ((size_t)1 << 32)) ? op->counters_for(stream) : nullptr;
         }
         const int mi = g.mt == 1 ? 0 : g.mt == 2 ? 1 : 2;
         launch(op->skinny[mi][g.qmode], Dim3{(p.N + 127) / 128, p.split_k, p.batch}, Dim3{256}, 0, stream, g.p);

@@ -86,19 +86,26 @@ __device__ __forceinline__ void transpose8x8(const u32x4 (&w)[8], u32x4 (&b)[8])
 }
 
 // Split-K partials cross workgroups that may sit on different XCDs (each with its
-// own L2), inside one kernel.  They are moved with device-scope relaxed atomics
-// (64-bit, write-through / L2-bypassing accesses) instead of plain accesses plus
-// device-scope fences: a device-scope fence writes back and invalidates the whole
+// own L2), inside one kernel.  They are moved with write-through / L2-bypassing accesses
+// (the sc1 cache policy the compiler gives device-scope relaxed atomics) instead of plain
+// accesses plus device-scope fences: a device-scope fence writes back and invalidates the whole
 // L2, which is ruinous while the same L2 is streaming weights.
-__device__ __forceinline__ void partial_store(float *dst, float a, float b) {
-    const unsigned long long v = (unsigned long long)__float_as_uint(a) | ((unsigned long long)__float_as_uint(b) << 32);
-    __hip_atomic_store(reinterpret_cast<unsigned long long *>(dst), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+// They go 16 bytes at a time through buffer instructions, which take the cache policy as an operand: a lane's 8
+// partial sums are two stores, and 16 lanes write 512 contiguous bytes (as four 64-bit atomic stores per lane the
+// hardware counted four times the bytes written).  Offsets are 32-bit: the host keeps this path for workspaces
+// below 4 GiB.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t partial_rsrc(void *base) {
+    return __builtin_amdgcn_make_buffer_rsrc(base, 0, 0xffffffff, 0x00020000);
 }
-__device__ __forceinline__ void partial_load(const float *src, float &a, float &b) {
-    const unsigned long long v = __hip_atomic_load(reinterpret_cast<const unsigned long long *>(src), __ATOMIC_RELAXED,
-                                                   __HIP_MEMORY_SCOPE_AGENT);
-    a = __uint_as_float((uint32_t)v);
-    b = __uint_as_float((uint32_t)(v >> 32));
+constexpr int PARTIAL_SC1 = 16;  // the cache-policy operand of the buffer builtins: bit 4 = sc1
+__device__ __forceinline__ void partial_store4(__amdgpu_buffer_rsrc_t r, uint32_t byte_off, float a, float b, float c, float d) {
+    const u32x4 v = {__float_as_uint(a), __float_as_uint(b), __float_as_uint(c), __float_as_uint(d)};
+    __builtin_amdgcn_raw_buffer_store_b128(v, r, byte_off, 0, PARTIAL_SC1);
+}
+__device__ __forceinline__ void partial_load4(__amdgpu_buffer_rsrc_t r, uint32_t byte_off, float (&out)[4]) {
+    const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, PARTIAL_SC1);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) out[t] = __uint_as_float(v[t]);
 }
 
 // D[i, col0 .. col0+7] = alpha * sum + beta * D, rounded once to f16
@@ -425,11 +432,12 @@ __device__ __forceinline__ void gemm_skinny(const GemmParams &p) {
         const uint32_t i = mt * 16 + 4 * g + wave;
         if (i < p.M && col0 < p.N) {
             if (p.split_k > 1) {
-                float *dst = reinterpret_cast<float *>(p.partial) +
-                             (((size_t)split * p.batch + bat) * p.M + i) * p.N + col0;
+                const size_t elem = (((size_t)split * p.batch + bat) * p.M + i) * p.N + col0;
+                float *dst = reinterpret_cast<float *>(p.partial) + elem;
                 if (p.counters) {
-#pragma unroll
-                    for (int t = 0; t < 8; t += 2) partial_store(dst + t, sum[t], sum[t + 1]);
+                    const __amdgpu_buffer_rsrc_t r = partial_rsrc(p.partial);
+                    partial_store4(r, (uint32_t)(elem * 4), sum[0], sum[1], sum[2], sum[3]);
+                    partial_store4(r, (uint32_t)(elem * 4 + 16), sum[4], sum[5], sum[6], sum[7]);
                 } else {
                     *reinterpret_cast<f32x4 *>(dst) = f32x4{sum[0], sum[1], sum[2], sum[3]};
                     *reinterpret_cast<f32x4 *>(dst + 4) = f32x4{sum[4], sum[5], sum[6], sum[7]};
@@ -463,17 +471,22 @@ __device__ __forceinline__ void gemm_skinny(const GemmParams &p) {
                 if (i < p.M && col0 < p.N) {
                     float sum[8] = {0, 0, 0, 0, 0, 0, 0, 0};
                     const size_t sstride = (size_t)p.batch * p.M * p.N;  // floats between splits
-                    const float *src0 = reinterpret_cast<const float *>(p.partial) + ((size_t)bat * p.M + i) * p.N + col0;
+                    const size_t elem0 = ((size_t)bat * p.M + i) * p.N + col0;
+                    const __amdgpu_buffer_rsrc_t r = partial_rsrc(p.partial);
                     constexpr int FLY = MT == 1 ? 8 : 4;  // splits whose loads are in flight together, summed in order
                     for (uint32_t s0 = 0; s0 < p.split_k; s0 += FLY) {
                         float v[FLY][8];
 #pragma unroll
-                        for (int u = 0; u < FLY; ++u)
-#pragma unroll
-                            for (int t = 0; t < 8; t += 2) {
-                                v[u][t] = v[u][t + 1] = 0.f;
-                                if (s0 + u < p.split_k) partial_load(src0 + (s0 + u) * sstride + t, v[u][t], v[u][t + 1]);
+                        for (int u = 0; u < FLY; ++u) {
+                            float lo[4] = {0.f, 0.f, 0.f, 0.f}, hi[4] = {0.f, 0.f, 0.f, 0.f};
+                            if (s0 + u < p.split_k) {
+                                const uint32_t off = (uint32_t)((elem0 + (s0 + u) * sstride) * 4);
+                                partial_load4(r, off, lo);
+                                partial_load4(r, off + 16, hi);
                             }
+#pragma unroll
+                            for (int t = 0; t < 4; ++t) v[u][t] = lo[t], v[u][4 + t] = hi[t];
+                        }
 #pragma unroll
                         for (int u = 0; u < FLY; ++u)
                             if (s0 + u < p.split_k) {
