@@ -170,7 +170,13 @@ OPHIP_API int ophip_probe(ophip_device *dev, const char *kind, void *dst, const 
  * ophip_graph_launch without per-launch host cost.  Give every recorded launch a workspace of
  * its own (scheme() reports the size).  A mat_mul operator used on more than one stream has to be
  * launched once on each further stream before that stream records: its first split-K launch on a
- * stream other than the first allocates, which HIP refuses while a stream records. */
+ * stream other than the first allocates, which HIP refuses while a stream records.
+ * A recorded split-K mat_mul carries the address of the arrival counters the operator keeps for the
+ * stream it was recorded on.  Hence: replay a graph on the stream it was recorded on (on another stream,
+ * while that one also runs split-K products of the same operator, two kernels would share one set of
+ * counters and sum wrongly), and destroy a graph before the operators recorded into it (the operator
+ * frees its counters).  An operator keeps one 256 KiB counter buffer per stream it has ever been
+ * launched on, until it is destroyed. */
 typedef void *ophip_graph; /* hipGraphExec_t */
 OPHIP_API int ophip_stream_begin_capture(ophip_device *dev, ophip_stream stream);
 OPHIP_API int ophip_stream_end_capture(ophip_device *dev, ophip_stream stream, ophip_graph *out);
