@@ -256,6 +256,110 @@ def ceilings(ophip, gpu, stream):
     return out
 
 
+def gemm_floors(ophip, gpu, stream, rng, reps):
+    """The six GEMMs of the decode layer on cold operands (copies of the weight or cache operand rotate through more than
+    600 MB), each beside what a bare read of the same bytes takes: the library's read probe (non-temporal loads) over
+    the same cold copies, with as many workgroups as the GEMM launches and with the best of a few grids, and beside an
+    empty launch.  What separates a GEMM from its bare read is MFMA work, the activation loads and, with split K, the
+    exchange of partial sums."""
+    import copy
+    layer = Layer(ophip, gpu, rng)
+    mm = layer.ops["mm"]
+    out = []
+    one = gpu.malloc(4096)
+    probe = lambda kind, dst, src, nbytes, blocks: ophip._check(ophip.lib().ophip_probe(
+        gpu.handle, kind.encode(), ctypes.c_void_p(dst.ptr), ctypes.c_void_p(src.ptr if src else dst.ptr),
+        ctypes.c_size_t(nbytes), ctypes.c_uint(0), ctypes.c_uint(1), ctypes.c_uint(blocks), stream.handle))
+    empty_us = time_launches(gpu, stream, lambda: probe("write", one, None, 16, 1), 200, warm=10)
+    log("  empty launch (16 bytes written by one workgroup), back to back: %.2f us" % empty_us)
+    work = layer_work()
+    operand = {"qkv": ("w_qkv", D * 3 * D * 2), "qk_t": ("k_cache", NH * KV * DH * 2), "pv": ("v_cache", NH * KV * DH * 2),
+               "o_proj": ("w_o", D * D * 2), "gate_up": ("w_gu", D * 2 * DI * 2), "down": ("w_d", DI * D * 2)}
+    for name in ("qkv", "qk_t", "pv", "o_proj", "gate_up", "down"):
+        buf_name, nbytes = operand[name]
+        ncopy = max(2, (600 << 20) // nbytes + 1)
+        copies = [gpu.malloc(nbytes) for _ in range(ncopy)]
+        for cbuf in copies:
+            ophip._check(ophip.lib().ophip_memcpy_d2d(gpu.handle, ctypes.c_void_p(cbuf.ptr), ctypes.c_void_p(layer.d[buf_name].ptr),
+                                                      ctypes.c_size_t(nbytes), stream.handle))
+        stream.synchronize()
+        kind, base = layer.args[name]
+        variants = []
+        for cbuf in copies:
+            a = copy.copy(base)
+            a.b_base = cbuf
+            variants.append(a)
+        what = mm.describe(base)
+        split = int(what.split("split_k=")[1]) if "split_k=" in what else 1
+        m, n = (NT, {"qkv": 3 * D, "o_proj": D, "gate_up": 2 * DI, "down": D}.get(name, KV if name == "qk_t" else DH))
+        batch = NH if name in ("qk_t", "pv") else 1
+        wgs = (n + 127) // 128 * split * batch
+        it = [0]
+
+        def run_gemm():
+            mm.launch(variants[it[0] % ncopy], layer.d["ws"], stream)
+            it[0] += 1
+
+        def run_probe(blocks):
+            def f():
+                probe("read_nt", one, copies[it[0] % ncopy], nbytes, blocks)
+                it[0] += 1
+            return f
+        gemm_us = time_launches(gpu, stream, run_gemm, reps, warm=ncopy)
+        same_us = time_launches(gpu, stream, run_probe(wgs), reps, warm=ncopy)
+        best = min((time_launches(gpu, stream, run_probe(b), reps, warm=4), b) for b in (256, 512, 1024, 2048))
+        rec = {"op": name, "kernel": what, "workgroups": wgs, "operand_bytes": nbytes, "algorithmic_bytes": work[name][0],
+               "gemm_us": round(gemm_us, 2), "bare_read_same_grid_us": round(same_us, 2),
+               "bare_read_best_us": round(best[0], 2), "bare_read_best_workgroups": best[1], "copies": ncopy}
+        out.append(rec)
+        log("  %-8s %-34s %4d workgroups: %6.2f us | bare read of the operand (%5.1f MB), same grid %6.2f us, best %6.2f us (%d workgroups)" % (
+            name, what, wgs, gemm_us, nbytes / 1e6, same_us, best[0], best[1]))
+        for cbuf in copies:
+            cbuf.free()
+    # The weight-streaming kernel without a K split, one workgroup per 128-column strip, on 64 .. 288 strips (cold
+    # weights): what one CU pulls, and how the launch's rate follows the number of CUs that hold a workgroup.
+    L, F16 = ophip.TensorLayout, ophip.dt.F16
+    prev = os.environ.get("OPHIP_GEMM_SPLITK")
+    os.environ["OPHIP_GEMM_SPLITK"] = "1"
+    unsplit = ophip.MatMul(gpu)
+    if prev is None:
+        del os.environ["OPHIP_GEMM_SPLITK"]
+    else:
+        os.environ["OPHIP_GEMM_SPLITK"] = prev
+    strips_out = []
+    x = layer.d["xn"]
+    for strips in (64, 128, 172, 192, 224, 250, 256, 288):
+        n = 128 * strips
+        nbytes = D * n * 2
+        ncopy = max(2, (600 << 20) // nbytes + 1)
+        copies = [gpu.malloc(nbytes) for _ in range(ncopy)]
+        src_bytes = D * 2 * DI * 2
+        for cbuf in copies:  # any finite f16 will do: the layer's gate/up weight, again and again
+            for off in range(0, nbytes, src_bytes):
+                ophip._check(ophip.lib().ophip_memcpy_d2d(gpu.handle, ctypes.c_void_p(cbuf.ptr + off), ctypes.c_void_p(layer.d["w_gu"].ptr),
+                                                          ctypes.c_size_t(min(nbytes - off, src_bytes)), stream.handle))
+        dst = gpu.malloc(NT * n * 2)
+        variants = [ophip.MatMulArgs(L.new_contiguous(F16, [NT, n]), dst, 0.0, L.new_contiguous(F16, [NT, D]), x,
+                                     L.new_contiguous(F16, [D, n]), cbuf, 1.0) for cbuf in copies]
+        what = unsplit.describe(variants[0])
+        it = [0]
+
+        def run_strips():
+            unsplit.launch(variants[it[0] % ncopy], layer.d["ws"], stream)
+            it[0] += 1
+        us = time_launches(gpu, stream, run_strips, reps, warm=ncopy)
+        busy = min(strips, 256)
+        rec = {"strips": strips, "kernel": what, "weight_bytes": nbytes, "us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
+               "GBps_per_busy_cu": round(nbytes / us / 1e3 / busy, 2)}
+        strips_out.append(rec)
+        log("  %3d strips (%s): %6.2f us, %6.1f GB/s, %5.2f GB/s per CU that holds a workgroup" % (
+            strips, what, us, rec["GBps"], rec["GBps_per_busy_cu"]))
+        for cbuf in copies:
+            cbuf.free()
+        dst.free()
+    return {"empty_launch_us": round(empty_us, 2), "gemms": out, "unsplit_strips": strips_out}
+
+
 def adder(out, ceiling=None):
     """Returns add(name, shape, bytes, us, flops, note): appends one per-operator record to `out` and logs it.
     `ceiling`: the copy_ceiling record; with it every record carries `ceiling_frac`, its rate against what a plain
@@ -544,6 +648,8 @@ def main():
     ap.add_argument("--mat-mul-only", type=int, nargs="?", const=0, default=None, metavar="LAUNCHES",
                     help="only the compute-bound mat_mul shapes (not the benchmark line); with a number, that many "
                          "plain launches per shape, for hardware-counter runs")
+    ap.add_argument("--floors", action="store_true",
+                    help="only the decode layer's GEMMs on cold operands, each beside a bare read of the same bytes")
     ap.add_argument("--ceilings", action="store_true",
                     help="only the machine's ceilings: stream probes (read, write, copy) and the bare MFMA loop")
     args = ap.parse_args()
@@ -559,6 +665,9 @@ def main():
     log("device: %s (%s), %d CUs" % (info.name.decode(), info.arch.decode(), info.compute_units))
     stream = gpu.stream()
     rng = np.random.default_rng(0)
+    if args.floors:
+        print(json.dumps({"floors": gemm_floors(ophip, gpu, stream, rng, args.reps)}))
+        return
     if args.ceilings:
         print(json.dumps({"ceilings": ceilings(ophip, gpu, stream)}))
         return
@@ -593,6 +702,21 @@ def main():
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / args.steps
     dom_us = float(np.mean([a.elapsed_ms(b) for a, b in own])) * 1e3
+    # The same steps replayed from a recorded launch graph (two steps, one per weight set, per replay): what the
+    # host's launch calls cost the step, if anything.  Reported beside `ms_per_step`, which stays the eager figure.
+    stream.begin_capture()
+    for lay in layers:
+        lay.step(stream)
+    graph = stream.end_capture()
+    for _ in range(max(1, args.warmup // 2)):
+        graph.launch(stream)
+    stream.synchronize()
+    t0g = time.perf_counter()
+    for _ in range(args.steps // 2):
+        graph.launch(stream)
+    stream.synchronize()
+    graph_ms_per_step = (time.perf_counter() - t0g) * 1e3 / (2 * (args.steps // 2)) if args.steps >= 2 else None
+    graph.destroy()
     # For comparison, outside the timed region: two separate event records around the same launch, which read
     # longer by most of what an empty pair of records reads.
     pairs = [(gpu.event(), gpu.event()) for _ in range(20)]
@@ -662,6 +786,7 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 5),
+        "graph_replay_ms_per_step": round(graph_ms_per_step, 5) if graph_ms_per_step else None,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
