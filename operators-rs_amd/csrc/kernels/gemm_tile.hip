@@ -76,6 +76,19 @@ struct TileLoader {
     // Row-contiguous: thread (cb, kb) takes NV k-rows x 8 columns.
     static constexpr int KV = TK / 8;
     static constexpr int NV = R * KV / 256;
+    // Row-contiguous operand: which 8 columns (cb) and which NV k-rows (kb) thread t holds.  With NV = 4 a thread's
+    // transposing stores are 8 bytes wide and the hardware takes 16 lanes of such a store per cycle over 128 bytes: 16
+    // lanes on 16 consecutive LDS rows would meet only 8 different swizzle keys (rows s and s + 8 collide; measured as
+    // 1.3 conflict cycles per LDS instruction of the 128 tile).  So a group of 16 lanes takes 8 column groups of two
+    // neighbouring kb instead: 8 rows x the two 8-byte halves of one 16-byte group.
+    __device__ static __forceinline__ uint32_t cb_of(uint32_t t) {
+        if constexpr (NV == 4 && R == 128 && TK == 64) return (t & 7) | ((t >> 1) & 8);
+        return t % (R / 8);
+    }
+    __device__ static __forceinline__ uint32_t kb_of(uint32_t t) {
+        if constexpr (NV == 4 && R == 128 && TK == 64) return ((t >> 3) & 1) | ((t >> 5) << 1);
+        return t / (R / 8);
+    }
     u32x4 reg[NV];
     uint32_t voff[NV];  // byte offset of each of the thread's vectors from the tile's first element
 
@@ -95,8 +108,8 @@ struct TileLoader {
                 const uint32_t row = CLAMP ? min(idx / KV, rows - 1) : idx / KV;
                 voff[v] = (row * (uint32_t)s_row + kv * 8) * 2;
             } else {
-                const uint32_t kb = t / (R / 8);
-                const uint32_t cb = CLAMP ? min(t % (R / 8), rows / 8 - 1) : t % (R / 8);
+                const uint32_t kb = kb_of(t);
+                const uint32_t cb = CLAMP ? min(cb_of(t), rows / 8 - 1) : cb_of(t);
                 voff[v] = ((kb * NV + v) * (uint32_t)s_k + cb * 8) * 2;
             }
         }
@@ -133,7 +146,7 @@ struct TileLoader {
                         if (k0 + e < kvalid) reg[v][e / 2] |= (uint32_t)h[e] << (16 * (e & 1));
                 }
             } else {
-                const uint32_t k = (t / (R / 8)) * NV + v;  // this register's k-row
+                const uint32_t k = kb_of(t) * NV + v;  // this register's k-row
                 if (k < kvalid) reg[v] = *reinterpret_cast<const u32x4 *>(src);
             }
         }
@@ -149,7 +162,7 @@ struct TileLoader {
             const uint32_t idx = t + v * 256, row = idx / KV, kv = idx % KV;
             st128(lds + TileRow<TK>::at(row, kv), reg[v]);
         } else {
-            const uint32_t cb = t % (R / 8), kb = t / (R / 8);
+            const uint32_t cb = cb_of(t), kb = kb_of(t);
 #pragma unroll
             for (int c = v * 8 / NV; c < (v + 1) * 8 / NV; ++c) {
                 f16 *dst = lds + TileRow<TK>::at(c * (R / 8) + cb, kb * NV / 8) + kb * NV % 8;
@@ -177,7 +190,7 @@ struct TileLoader {
     }
     __device__ __forceinline__ void store_packed(f16 *lds, int v, u32x4 w) const {
         const uint32_t t = threadIdx.x;
-        const uint32_t cb = t % (R / 8), kb = t / (R / 8);
+        const uint32_t cb = cb_of(t), kb = kb_of(t);
         st128(lds + TileRow<TK>::at(v * (R / 8) + cb, kb * NV / 8) + kb * NV % 8, w);
     }
     __device__ __forceinline__ void commit(f16 *lds) const {
@@ -269,7 +282,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
     // Copy piece i in the order the main loop uses (the waits the compiler derives for the loop
     // merge the prologue's order with the loop's: they must agree or the loop waits too long).
     constexpr bool Q_FIRST = PK && !QK, ALTERNATE = PK && QK && LP::NV == LQ::NV;
-    auto piece_is_q = [&](int i) { return ALTERNATE ? bool(i & 1) : ((i >= LP::NV) != Q_FIRST) ; };
+    auto piece_is_q = [&](int i) { return ALTERNATE ? bool(i & 1) : (Q_FIRST ? i < LQ::NV : i >= LP::NV); };
     auto piece_v = [&](int i) { return ALTERNATE ? i / 2 : (Q_FIRST ? (i < LQ::NV ? i : i - LQ::NV) : (i < LP::NV ? i : i - LP::NV)); };
     auto fetch_all = [&](int set, const f16 *pt, const f16 *qt) {
 #pragma unroll
