@@ -357,7 +357,55 @@ def gemm_floors(ophip, gpu, stream, rng, reps):
         for cbuf in copies:
             cbuf.free()
         dst.free()
-    return {"empty_launch_us": round(empty_us, 2), "gemms": out, "unsplit_strips": strips_out}
+    # The streaming kernel's access pattern and nothing else (probe "strips": 128-column strips x equal K ranges, four waves
+    # per workgroup on every fourth group of 32 rows, three groups in flight per wave; no MFMA, no activations, no
+    # epilogue, no exchange of partial sums) on the four weight shapes, at 1 .. 16 K ranges.
+    pattern = []
+    for name, n, k in (("qkv", 3 * D, D), ("o_proj", D, D), ("gate_up", 2 * DI, D), ("down", D, DI)):
+        nbytes = n * k * 2
+        ncopy = max(2, (700 << 20) // nbytes + 1)
+        copies = [gpu.malloc(nbytes) for _ in range(ncopy)]
+        for cbuf in copies:
+            gpu.memset(cbuf, 0x3C)
+        row = {"op": name, "bytes": nbytes, "us_by_k_ranges": {}}
+        for ranges in (1, 2, 4, 8, 16):
+            if k % (32 * ranges):
+                continue
+            it = [0]
+
+            def run_pattern():
+                ophip._check(ophip.lib().ophip_probe(gpu.handle, b"strips", ctypes.c_void_p(one.ptr), ctypes.c_void_p(copies[it[0] % ncopy].ptr),
+                                                     ctypes.c_size_t(nbytes), ctypes.c_uint(n), ctypes.c_uint(k), ctypes.c_uint(ranges), stream.handle))
+                it[0] += 1
+            row["us_by_k_ranges"][ranges] = round(time_launches(gpu, stream, run_pattern, reps, warm=ncopy), 2)
+        pattern.append(row)
+        log("  pattern %-8s %6.1f MB: %s" % (name, nbytes / 1e6, "  ".join("%d ranges (%d workgroups) %6.2f us" % (
+            r, (n + 127) // 128 * r, us) for r, us in row["us_by_k_ranges"].items())))
+        for cbuf in copies:
+            cbuf.free()
+    # What one CU pulls with nothing but loads: the read probes on 1 MB per workgroup (as a strip above), 64 / 128 / 256
+    # workgroups, 4 or 16 vectors in flight per thread, plain or non-temporal loads.
+    per_cu = []
+    for blocks in (64, 128, 256):
+        nbytes = blocks << 20
+        npool = (768 << 20) // nbytes + 1  # more than three times the 256 MiB cache in rotation
+        pool = [gpu.malloc(nbytes) for _ in range(npool)]
+        for pbuf in pool:
+            gpu.memset(pbuf, 0x3C)
+        for kind in ("read", "read_nt", "read16", "read_nt16"):
+            it = [0]
+
+            def run_probe_kind():
+                probe(kind, one, pool[it[0] % npool], nbytes, blocks)
+                it[0] += 1
+            us = time_launches(gpu, stream, run_probe_kind, reps, warm=npool)
+            per_cu.append({"kind": kind, "workgroups": blocks, "bytes": nbytes, "us": round(us, 2),
+                           "GBps_per_workgroup": round(nbytes / us / 1e3 / blocks, 2)})
+            log("  probe %-9s %3d workgroups x 1 MB: %6.2f us, %5.2f GB/s per workgroup" % (kind, blocks, us, nbytes / us / 1e3 / blocks))
+        for pbuf in pool:
+            pbuf.free()
+    return {"empty_launch_us": round(empty_us, 2), "gemms": out, "unsplit_strips": strips_out, "access_pattern": pattern,
+            "probe_per_workgroup": per_cu}
 
 
 def adder(out, ceiling=None):

@@ -387,13 +387,19 @@ int ophip_probe(ophip_device *dev, const char *kind, void *dst, const void *src,
     return guard([&] {
         if (!dev || !kind) throw args_not_support("null argument");
         const std::string k = kind;
-        const bool reads = k == "read" || k == "read_nt" || k == "copy", writes = k == "write" || k == "copy";
-        if (!reads && !writes && k != "mfma") throw args_not_support("unknown probe: " + k);
+        const bool reads = k == "read" || k == "read_nt" || k == "read16" || k == "read_nt16" || k == "copy", writes = k == "write" || k == "copy";
+        if (!reads && !writes && k != "mfma" && k != "strips") throw args_not_support("unknown probe: " + k);
         if ((reads && !src) || !dst || blocks == 0) throw args_not_support("probe: null buffer or empty grid");
         if ((reads || writes) && (bytes % 16 != 0 || !aligned16(dst) || (reads && !aligned16(src))))
             throw args_not_support("probe: buffers in whole 16-byte vectors");
         ProbeParams p{dst, src, (uint64_t)bytes, iters, seed};
         dev->make_current();
+        if (k == "strips") {  // `src`: [seed rows][iters columns] f16, `blocks` row ranges; one workgroup per 128-column strip and range
+            if (!src || !dst || iters < 8 || iters % 8 != 0 || blocks == 0 || seed % (32 * blocks) != 0 || (size_t)iters * seed * 2 > bytes || !aligned16(src))
+                throw args_not_support("probe strips: [seed][iters] f16 inside `bytes`, rows in whole groups of 32 per range");
+            launch(dev->kernel("probe", "probe_strips"), Dim3{(iters + 127) / 128, blocks}, Dim3{256}, 0, (hipStream_t)stream, p);
+            return;
+        }
         launch(dev->kernel("probe", ("probe_" + k).c_str()), Dim3{blocks}, Dim3{256}, 0, (hipStream_t)stream, p);
     });
 }

@@ -384,7 +384,7 @@ extern "C" int ophip_fused_softmax_launch(const ophip_fused_softmax *op, const o
             if (!pick || v.g < pick->g || (v.g == pick->g && v.pt < pick->pt)) pick = &v;
         }
         op->dev->make_current();
-        if (vec && att <= 1024 && rows >= 8192) {
+        if (vec && att % 8 == 0 && att <= 1024 && rows >= 8192) {
             // many short rows: four per wave, their loads in flight together (16384 waves of one 512-column row
             // each cost more in start-up than in traffic: [32, 512, 512] causal 9.6 -> see the kernel's note)
             const size_t waves = nh * ((seq + 3) / 4);

@@ -51,6 +51,33 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
+// The same reductions with the first four steps as DPP operand modifiers (lane ^ 1, lane ^ 2, mirror inside 8, mirror
+// inside 16: no LDS crossbar, no extra instruction) and only the last two as cross-lane reads: a third of the
+// instructions, for kernels whose reductions are a visible share of their work.  Every lane ends with the result.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+constexpr int DPP_XOR1 = 0xB1, DPP_XOR2 = 0x4E, DPP_HALF_MIRROR = 0x141, DPP_MIRROR = 0x140;
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+    v += dpp_move<DPP_XOR1>(v);
+    v += dpp_move<DPP_XOR2>(v);
+    v += dpp_move<DPP_HALF_MIRROR>(v);
+    v += dpp_move<DPP_MIRROR>(v);
+    v += __shfl_xor(v, 16, WAVE);
+    v += __shfl_xor(v, 32, WAVE);
+    return v;
+}
+__device__ __forceinline__ float wave_max_dpp(float v) {
+    v = fmaxf(v, dpp_move<DPP_XOR1>(v));
+    v = fmaxf(v, dpp_move<DPP_XOR2>(v));
+    v = fmaxf(v, dpp_move<DPP_HALF_MIRROR>(v));
+    v = fmaxf(v, dpp_move<DPP_MIRROR>(v));
+    v = fmaxf(v, __shfl_xor(v, 16, WAVE));
+    v = fmaxf(v, __shfl_xor(v, 32, WAVE));
+    return v;
+}
+
 // Sum over a group of G consecutive threads (G = 64 * 2^k, G <= blockDim).
 // Groups wider than a wave combine their per-wave partials through `smem`
 // (one float per wave of the block) in a fixed order; all threads must call.

@@ -104,7 +104,7 @@ __device__ __forceinline__ void softmax_reg(const SoftmaxParams &p) {
 // one load, two reductions and one store, and 16384 such waves cost more in start-up than in traffic.  Here a wave
 // takes four rows at once, all their loads in flight together; under a causal mask the four are two pairs
 // (r, seq - 1 - r), so every wave moves the same number of bytes whatever its place in the triangle.
-// 16-byte aligned rows only; PT 16-byte vectors per lane and row (att_len <= 512 * PT).
+// 16-byte aligned rows of a multiple of 8 columns only; PT 16-byte vectors per lane and row (att_len <= 512 * PT).
 template <int PT>
 __device__ __forceinline__ void softmax_rows4(const SoftmaxParams &p) {
     constexpr int ROWS = 4;
@@ -116,71 +116,63 @@ __device__ __forceinline__ void softmax_rows4(const SoftmaxParams &p) {
     const bool paired = p.seq % ROWS == 0;
 
     f16 *row[ROWS];
-    uint32_t kept[ROWS];
+    int kept[ROWS];
     bool live[ROWS];
-    float x[ROWS][PT][8];
-    float mx[ROWS];
 #pragma unroll
     for (int i = 0; i < ROWS; ++i) {
         uint32_t r = paired ? (i % 2 == 0 ? 2 * j + i / 2 : p.seq - 1 - (2 * j + i / 2)) : ROWS * j + i;
         live[i] = r < p.seq;
         if (!live[i]) r = p.seq - 1;
-        kept[i] = kept_columns(p, r);
+        kept[i] = (int)kept_columns(p, r);
         row[i] = reinterpret_cast<f16 *>(reinterpret_cast<char *>(p.att) + (int64_t)h * p.sh + (int64_t)r * p.ss);
     }
+    // att_len is a multiple of 8 (the host sends other lengths to the general kernel): a lane's vector is inside the
+    // row or outside it, and what a row keeps of it is the first `n` of its 8 columns, n = kept - col0.
     Pack8 v[ROWS][PT];
 #pragma unroll
     for (int i = 0; i < ROWS; ++i)
 #pragma unroll
         for (int q = 0; q < PT; ++q) {
-            const uint32_t col0 = (lane + q * WAVE) * 8;
+            const int col0 = (int)(lane + q * WAVE) * 8;
             v[i][q].u = u32x4{0, 0, 0, 0};
-            if (col0 + 8 <= p.att_len) {
-                if (col0 < kept[i]) v[i][q].u = ld128(row[i] + col0);
-            } else {
-#pragma unroll
-                for (int e = 0; e < 7; ++e)
-                    if (col0 + e < kept[i]) v[i][q].e[e] = row[i][col0 + e];
-            }
+            if (col0 < kept[i]) v[i][q].u = ld128(row[i] + col0);
         }
+    // Masked columns become -inf once, here; from then on they take care of themselves: they never win the maximum,
+    // their exponential is 0, they add nothing to the sum and 0 / sum is the 0 the mask asks for.
+    float x[ROWS][PT][8];
+    float mx[ROWS];
 #pragma unroll
     for (int i = 0; i < ROWS; ++i) {
         mx[i] = -INFINITY;
 #pragma unroll
-        for (int q = 0; q < PT; ++q)
+        for (int q = 0; q < PT; ++q) {
+            const int n = kept[i] - (int)(lane + q * WAVE) * 8;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const uint32_t col = (lane + q * WAVE) * 8 + e;
-                x[i][q][e] = col < kept[i] ? h2f(v[i][q].e[e]) : -INFINITY;
+                x[i][q][e] = e < n ? h2f(v[i][q].e[e]) : -INFINITY;
                 mx[i] = fmaxf(mx[i], x[i][q][e]);
             }
+        }
     }
 #pragma unroll
-    for (int o = WAVE / 2; o > 0; o >>= 1)
-#pragma unroll
-        for (int i = 0; i < ROWS; ++i) mx[i] = fmaxf(mx[i], __shfl_xor(mx[i], o, WAVE));
+    for (int i = 0; i < ROWS; ++i) mx[i] = wave_max_dpp(mx[i]);
     float sum[ROWS];
 #pragma unroll
     for (int i = 0; i < ROWS; ++i) {
         sum[i] = 0.f;
+        constexpr float LOG2E = 1.44269504088896340736f;
+        const float shift = -mx[i] * LOG2E;  // exp(x - mx) = 2^(x * log2(e) - mx * log2(e)): one fused multiply-add per element
 #pragma unroll
         for (int q = 0; q < PT; ++q)
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const uint32_t col = (lane + q * WAVE) * 8 + e;
-                if (col < kept[i]) {
-                    const float ex = fast_exp(x[i][q][e] - mx[i]);
-                    sum[i] += ex;
-                    x[i][q][e] = h2f(f2h(ex));  // the reference stores f16(e) and re-reads it
-                } else {
-                    x[i][q][e] = 0.f;
-                }
+                const float ex = __builtin_amdgcn_exp2f(__builtin_fmaf(x[i][q][e], LOG2E, shift));
+                sum[i] += ex;
+                x[i][q][e] = h2f(f2h(ex));  // the reference stores f16(e) and re-reads it
             }
     }
 #pragma unroll
-    for (int o = WAVE / 2; o > 0; o >>= 1)
-#pragma unroll
-        for (int i = 0; i < ROWS; ++i) sum[i] += __shfl_xor(sum[i], o, WAVE);
+    for (int i = 0; i < ROWS; ++i) sum[i] = wave_sum_dpp(sum[i]);
 #pragma unroll
     for (int i = 0; i < ROWS; ++i) {
         const float inv = 1.0f / sum[i];
@@ -190,14 +182,8 @@ __device__ __forceinline__ void softmax_rows4(const SoftmaxParams &p) {
             if (col0 < p.att_len && live[i]) {
                 Pack8 o;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) o.e[e] = col0 + e < kept[i] ? f2h(x[i][q][e] * inv) : (f16)0.f;
-                if (col0 + 8 <= p.att_len) {
-                    st128(row[i] + col0, o.u);
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 7; ++e)
-                        if (col0 + e < p.att_len) row[i][col0 + e] = o.e[e];
-                }
+                for (int e = 0; e < 8; ++e) o.e[e] = f2h(x[i][q][e] * inv);
+                st128(row[i] + col0, o.u);
             }
         }
     }

@@ -3,6 +3,7 @@
 // against nameplate figures.  Launched by ophip_probe; bench.py --ceilings runs them.
 //   probe_read / probe_read_nt : every thread pulls 16-byte vectors, four loads in flight, grid-stride
 //                                (`_nt`: with the non-temporal hint the GEMM weight loads carry)
+//   probe_read16 / probe_read_nt16 : the same with sixteen loads in flight
 //   probe_write                : 16-byte stores, grid-stride
 //   probe_copy                 : loads four vectors, then stores them (the element-wise kernels' pattern)
 //   probe_mfma                 : v_mfma_f32_32x32x16_f16 back to back on 16 independent accumulators per wave, the
@@ -33,6 +34,55 @@ extern "C" __global__ void __launch_bounds__(256) probe_read_nt(ProbeParams p) {
         acc ^= a ^ b ^ c ^ d;
     }
     for (; i < nvec; i += st) acc ^= ld128_nt(w + i);
+    if (acc[0] == 0x12345678u && acc[1] == 0x9abcdef0u) *reinterpret_cast<u32x4 *>(p.dst) = acc;
+}
+
+// The same read with 16 vectors in flight per thread (64 KB per workgroup, the depth of the weight-streaming GEMM's
+// register ring): what one CU can pull when the depth of its queue is not the limit.
+template <bool NT>
+__device__ __forceinline__ void probe_read_deep(const ProbeParams &p) {
+    const u32x4 *w = reinterpret_cast<const u32x4 *>(p.src);
+    const size_t nvec = p.bytes / 16, st = (size_t)gridDim.x * blockDim.x;
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    u32x4 acc = {0, 0, 0, 0};
+    for (; i + 15 * st < nvec; i += 16 * st) {
+        u32x4 v[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) v[u] = NT ? ld128_nt(w + i + u * st) : w[i + u * st];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) acc ^= v[u];
+    }
+    for (; i < nvec; i += st) acc ^= NT ? ld128_nt(w + i) : w[i];
+    if (acc[0] == 0x12345678u && acc[1] == 0x9abcdef0u) *reinterpret_cast<u32x4 *>(p.dst) = acc;
+}
+extern "C" __global__ void __launch_bounds__(256) probe_read16(ProbeParams p) { probe_read_deep<false>(p); }
+extern "C" __global__ void __launch_bounds__(256) probe_read_nt16(ProbeParams p) { probe_read_deep<true>(p); }
+
+// The weight-streaming GEMM's access pattern and nothing else: `src` is a row-major [seed rows][iters columns] f16
+// matrix; workgroup (x, y) reads the 128-column strip x over the y-th of gridDim.y equal row ranges, its four waves
+// taking every fourth group of 32 rows, a lane 8 rows x 16 bytes per group, three groups in flight per wave.
+extern "C" __global__ void __launch_bounds__(256) probe_strips(ProbeParams p) {
+    const uint32_t wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, j = lane % 16, g = lane / 16;
+    const uint32_t n = p.iters, rows = p.seed;
+    const uint32_t per = rows / gridDim.y, kbeg = blockIdx.y * per, kend = kbeg + per;
+    const uint32_t col = min(blockIdx.x * 128 + 8 * j, n - 8);
+    const f16 *w = reinterpret_cast<const f16 *>(p.src) + col;
+    u32x4 acc = {0, 0, 0, 0};
+    uint32_t kb = kbeg + 32 * wave;
+    for (; kb + 2 * 128 + 32 <= kend; kb += 3 * 128) {
+        u32x4 v[3][8];
+#pragma unroll
+        for (int u = 0; u < 3; ++u)
+#pragma unroll
+            for (int r = 0; r < 8; ++r) v[u][r] = ld128_nt(w + (size_t)(kb + 128 * u + 8 * g + r) * n);
+#pragma unroll
+        for (int u = 0; u < 3; ++u)
+#pragma unroll
+            for (int r = 0; r < 8; ++r) acc ^= v[u][r];
+    }
+    for (; kb + 32 <= kend; kb += 128)
+#pragma unroll
+        for (int r = 0; r < 8; ++r) acc ^= ld128_nt(w + (size_t)(kb + 8 * g + r) * n);
     if (acc[0] == 0x12345678u && acc[1] == 0x9abcdef0u) *reinterpret_cast<u32x4 *>(p.dst) = acc;
 }
 
