@@ -175,8 +175,9 @@ OPHIP_API int ophip_probe(ophip_device *dev, const char *kind, void *dst, const 
  * stream it was recorded on.  Hence: replay a graph on the stream it was recorded on (on another stream,
  * while that one also runs split-K products of the same operator, two kernels would share one set of
  * counters and sum wrongly), and destroy a graph before the operators recorded into it (the operator
- * frees its counters).  An operator keeps one 256 KiB counter buffer per stream it has ever been
- * launched on, until it is destroyed. */
+ * frees its counters).  An operator keeps one 256 KiB counter buffer per stream it is launched on; a
+ * stream ended with ophip_stream_destroy (which then waits for the stream's work first) hands its
+ * buffer to the next new stream, the rest is freed with the operator. */
 typedef void *ophip_graph; /* hipGraphExec_t */
 OPHIP_API int ophip_stream_begin_capture(ophip_device *dev, ophip_stream stream);
 OPHIP_API int ophip_stream_end_capture(ophip_device *dev, ophip_stream stream, ophip_graph *out);

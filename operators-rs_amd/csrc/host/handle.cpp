@@ -328,6 +328,14 @@ int ophip_stream_create(ophip_device *dev, ophip_stream *out) {
 int ophip_stream_destroy(ophip_device *dev, ophip_stream stream) {
     return guard([&] {
         dev->make_current();
+        {
+            std::lock_guard<std::mutex> lock(dev->hooks_mu);
+            if (!dev->stream_gone.empty()) {
+                // what the hooks hand on to other streams must be at rest first
+                check_hip(hipStreamSynchronize((hipStream_t)stream), "hipStreamSynchronize");
+                for (auto &h : dev->stream_gone) h.second((hipStream_t)stream);
+            }
+        }
         check_hip(hipStreamDestroy((hipStream_t)stream), "hipStreamDestroy");
     });
 }

@@ -9,6 +9,7 @@
 #include <hip/hip_runtime_api.h>
 
 #include <atomic>
+#include <functional>
 #include <map>
 #include <shared_mutex>
 #include <string>
@@ -25,6 +26,10 @@ struct ophip_device {
     std::shared_mutex mu;
     std::map<std::string, hipModule_t> modules;
     std::map<std::string, hipFunction_t> functions;
+
+    // Operators that keep per-stream state (mat_mul's arrival counters) ask to be told when a stream goes away.
+    std::mutex hooks_mu;
+    std::map<const void *, std::function<void(hipStream_t)>> stream_gone;
 
     // Function `kernel` of the embedded code object `module`; throws ExecutionFailed.
     hipFunction_t kernel(const char *module, const char *kernel);

@@ -7,6 +7,7 @@
 #include <cstdlib>
 #include <mutex>
 #include <unordered_map>
+#include <vector>
 
 #include "../kernels/params.h"
 #include "handle.hpp"
@@ -351,17 +352,25 @@ struct ophip_mat_mul {
     // which costs no device work at launch time: that launch may be recorded into a graph.  A further stream
     // gets a new buffer, cleared by a kernel on that stream; allocating is not possible while a stream records,
     // so an operator's first split-K product on a second stream has to be an ordinary launch.
+    // A stream that is destroyed (ophip_stream_destroy synchronises it first) gives its buffer back: all zero, ready
+    // for the next stream.
     mutable std::mutex mu;
     mutable std::unordered_map<hipStream_t, void *> counters;
+    mutable std::vector<void *> idle;
     mutable void *spare = nullptr;
 
     void *counters_for(hipStream_t stream) const {
         std::lock_guard<std::mutex> lock(mu);
         auto it = counters.find(stream);
         if (it != counters.end()) return it->second;
-        if (spare) {
+        if (spare || !idle.empty()) {
             void *buf = spare;
-            spare = nullptr;
+            if (spare) {
+                spare = nullptr;
+            } else {
+                buf = idle.back();
+                idle.pop_back();
+            }
             counters[stream] = buf;
             return buf;
         }
@@ -400,8 +409,21 @@ struct ophip_mat_mul {
         }
         generic_f16 = d->kernel("gemm", "gemm_generic_f16");
         generic_f32 = d->kernel("gemm", "gemm_generic_f32");
+        std::lock_guard<std::mutex> lock(d->hooks_mu);
+        d->stream_gone[this] = [this](hipStream_t s) {
+            std::lock_guard<std::mutex> l(mu);
+            auto it = counters.find(s);
+            if (it == counters.end()) return;
+            idle.push_back(it->second);
+            counters.erase(it);
+        };
     }
     ~ophip_mat_mul() {
+        {
+            std::lock_guard<std::mutex> lock(dev->hooks_mu);
+            dev->stream_gone.erase(this);
+        }
+        for (void *b : idle) (void)hipFree(b);
         for (auto &c : counters) (void)hipFree(c.second);
         if (spare) (void)hipFree(spare);
         ophip_device_release(dev);

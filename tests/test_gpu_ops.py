@@ -1167,6 +1167,38 @@ def test_mat_mul_split_k_ignores_what_the_workspace_held(gpu, stream, m, n, k):
             assert np.array_equal(out.view(np.uint16), first.view(np.uint16)), "launch %d differs from the first" % it
 
 
+def test_mat_mul_split_k_on_streams_that_come_and_go(gpu, stream):
+    """The arrival counters of a split-K product belong to the operator, one buffer per stream.  A stream that is
+    destroyed hands its buffer on: products on a row of short-lived streams, interleaved with the long-lived one, all
+    match the first."""
+    rng = np.random.default_rng(5)
+    a = normal_f16(rng, (16, 4096))
+    b = normal_f16(rng, (4096, 4096), std=0.02)
+    c = np.zeros((16, 4096), f16)
+    op = ophip.MatMul(gpu)
+    cd, ad, bd = gpu.from_host(c), gpu.from_host(a), gpu.from_host(b)
+    args = ophip.MatMulArgs(TensorLayout.of(c), cd, 0.0, TensorLayout.of(a), ad, TensorLayout.of(b), bd, 1.0)
+    assert "split_k=1" not in op.describe(args)
+    ws = gpu.malloc(op.scheme(args, 2 ** 40))
+    ref = c.copy()
+    oracle.mat_mul(ref, 0.0, a, b, 1.0)
+    say("mat_mul split-k on streams that come and go")
+    op.launch(args, ws, stream)
+    first = gpu.to_host(cd, f16, c.size, stream=stream).reshape(c.shape)
+    assert_close_f16(first, ref, "split-k, first stream", abs_tol=4e-3)
+    for it in range(6):
+        other = gpu.stream()
+        gpu.memset(cd, 0xFF, stream=other)
+        op.launch(args, ws, other)
+        out = gpu.to_host(cd, f16, c.size, stream=other).reshape(c.shape)
+        other.destroy()
+        assert np.array_equal(out.view(np.uint16), first.view(np.uint16)), "stream %d differs" % it
+        gpu.memset(cd, 0xFF, stream=stream)
+        op.launch(args, ws, stream)
+        out = gpu.to_host(cd, f16, c.size, stream=stream).reshape(c.shape)
+        assert np.array_equal(out.view(np.uint16), first.view(np.uint16)), "back on the first stream, round %d" % it
+
+
 def run_mat_mul_with(gpu, stream, c, a, b, op, ws, qa):
     cd, ad, bd = gpu.from_host(c), gpu.from_host(a), gpu.from_host(b)
     args = ophip.MatMulArgs(TensorLayout.of(c), cd, 1.0, TensorLayout.of(a), ad, TensorLayout.of(b), bd, 1.0)
