@@ -317,7 +317,11 @@ def test_softmax_reference_shapes(gpu, stream, seq, al):
 @pytest.mark.parametrize("shape,causal", [((2, 3, 8), True), ((1, 1, 1), True), ((3, 5, 5), True),
                                           ((2, 4, 1000), False), ((2, 4, 4096), True), ((1, 3, 9000), True),
                                           ((1, 2, 16384), True), ((1, 2, 40000), True), ((1, 2, 70001), True),
-                                          ((4, 300, 300), True), ((2, 2, 1023), False), ((1, 2, 5000), True)])
+                                          ((4, 300, 300), True), ((2, 2, 1023), False), ((1, 2, 5000), True),
+                                          # many short rows, four to a wave: a row count that is no multiple of four, two
+                                          # vectors per lane, more columns than rows, no mask, a single vector per row
+                                          ((32, 257, 264), True), ((16, 514, 1024), True), ((16, 512, 1000), True),
+                                          ((32, 256, 512), False), ((64, 130, 136), True), ((1100, 8, 8), True), ((33, 250, 256), True)])
 def test_softmax_shapes(gpu, stream, shape, causal):
     rng = np.random.default_rng(sum(shape))
     att = normal_f16(rng, shape, std=2.0)
