@@ -343,7 +343,7 @@ struct ophip_mat_mul {
     ophip_device *dev;
     GemmKnobs knobs = GemmKnobs::from_env();
     hipFunction_t skinny[3][4];  // [mt index 1,2,4][qmode; 3 = mode 0 with paired K-steps]
-    hipFunction_t reduce, fill, generic_f16, generic_f32;
+    hipFunction_t reduce, fill, generic_f16, generic_f32, generic_f64;
     // [256 x 64 / 128 x 64 / 128 x 32 (K-step)][M or N not in whole tiles][P K-contiguous][Q K-contiguous]
     hipFunction_t tile[3][2][2][2];
     // Arrival counters live in a buffer owned by the operator, one per stream:
@@ -409,6 +409,7 @@ struct ophip_mat_mul {
         }
         generic_f16 = d->kernel("gemm", "gemm_generic_f16");
         generic_f32 = d->kernel("gemm", "gemm_generic_f32");
+        generic_f64 = d->kernel("gemm", "gemm_generic_f64");
         std::lock_guard<std::mutex> lock(d->hooks_mu);
         d->stream_gone[this] = [this](hipStream_t s) {
             std::lock_guard<std::mutex> l(mu);
@@ -439,7 +440,7 @@ static void mat_mul_launch_impl(const ophip_mat_mul *op, const ophip_mat_mul_arg
                                 size_t fixed_counter_count, hipStream_t stream) {
     if (!op || !args) throw args_not_support("null argument");
     const ophip_mat_mul_layout L = mat_mul_layout(*args);
-    if (L.dt != OPHIP_DT_F16 && L.dt != OPHIP_DT_F32) throw type_not_support("mat_mul supports f16 and f32");
+    if (L.dt != OPHIP_DT_F16 && L.dt != OPHIP_DT_F32 && L.dt != OPHIP_DT_F64) throw type_not_support("mat_mul supports f16, f32 and f64");
     if (is_dyn(args->alpha) || is_dyn(args->beta)) throw dyn_not_support("");
     if (L.m == 0 || L.n == 0 || L.batch == 0) return;
     if (L.m > 0x7fffffffu || L.n > 0x7fffffffu || L.k > 0x7fffffffu || L.batch > 65535)
@@ -451,6 +452,7 @@ static void mat_mul_launch_impl(const ophip_mat_mul *op, const ophip_mat_mul_arg
         throw args_not_support("this product needs " + std::to_string(g.workspace) +
                                " bytes of split-K scratch, the library's static buffer holds " +
                                std::to_string(workspace_len));
+    if (!args->c_base || !args->a_base || !args->b_base) throw args_not_support("null base address");
     op->dev->make_current();
     if (g.kind == GemmPlan::Skinny) {
         Workspace ws(fixed ? nullptr : qa, workspace, workspace_len, g.workspace);
@@ -488,7 +490,7 @@ static void mat_mul_launch_impl(const ophip_mat_mul *op, const ophip_mat_mul_arg
     }
     const unsigned gx = (p.N + 63) / 64, gy = (p.M + 63) / 64;
     if (gy > 65535) throw shape_not_support("mat_mul dimension too large for the generic kernel");
-    launch(L.dt == OPHIP_DT_F16 ? op->generic_f16 : op->generic_f32, Dim3{gx, gy, p.batch}, Dim3{256}, 0, stream,
+    launch(L.dt == OPHIP_DT_F16 ? op->generic_f16 : L.dt == OPHIP_DT_F32 ? op->generic_f32 : op->generic_f64, Dim3{gx, gy, p.batch}, Dim3{256}, 0, stream,
            g.p);
 }
 
@@ -525,7 +527,7 @@ int ophip_mat_mul_scheme(ophip_mat_mul *op, const ophip_mat_mul_args *args, size
         if (!op || !args) return;
         try {
             const ophip_mat_mul_layout L = mat_mul_layout(*args);
-            if (L.dt != OPHIP_DT_F16 && L.dt != OPHIP_DT_F32) return;
+            if (L.dt != OPHIP_DT_F16 && L.dt != OPHIP_DT_F32 && L.dt != OPHIP_DT_F64) return;
             const GemmPlan g = make_plan(*args, L, (unsigned)op->dev->props.multiProcessorCount, op->knobs);
             if (ws && g.workspace <= max_ws) *ws = g.workspace;
         } catch (const Error &) {
@@ -537,7 +539,7 @@ int ophip_mat_mul_describe(const ophip_mat_mul *op, const ophip_mat_mul_args *ar
     return guard([&] {
         if (!op || !args || !out || len == 0) throw args_not_support("null argument");
         const ophip_mat_mul_layout L = mat_mul_layout(*args);
-        if (L.dt != OPHIP_DT_F16 && L.dt != OPHIP_DT_F32) throw type_not_support("mat_mul supports f16 and f32");
+        if (L.dt != OPHIP_DT_F16 && L.dt != OPHIP_DT_F32 && L.dt != OPHIP_DT_F64) throw type_not_support("mat_mul supports f16, f32 and f64");
         const GemmPlan g = make_plan(*args, L, (unsigned)op->dev->props.multiProcessorCount, op->knobs);
         if (g.kind == GemmPlan::Skinny)
             std::snprintf(out, len, "skinny rows<=%d q%s split_k=%u", 16 * g.mt,

@@ -177,7 +177,7 @@ static RopeMeta rope_meta(const ophip_rope_args &a) {
 }
 
 struct ophip_rope : OpBase {
-    hipFunction_t f16_vec, f16_pairs, f32_pairs;
+    hipFunction_t f16_vec, f16_pairs, f32_pairs, f64_pairs;
     // theta^(k / (dh/2)) of the last (theta, dh) launched: a model has one such pair
     mutable std::mutex den_mu;
     mutable float den_theta = 0.f;
@@ -196,6 +196,7 @@ struct ophip_rope : OpBase {
         f16_vec = d->kernel("rope", "rope_f16_vec");
         f16_pairs = d->kernel("rope", "rope_f16_pairs");
         f32_pairs = d->kernel("rope", "rope_f32_pairs");
+        f64_pairs = d->kernel("rope", "rope_f64_pairs");
     }
 };
 
@@ -218,7 +219,8 @@ extern "C" int ophip_rope_launch(const ophip_rope *op, const ophip_rope_args *ar
                                  const ophip_queue_alloc *qa) {
     return guard([&] {
         const RopeMeta m = rope_meta(*args);
-        if (m.dt_t != OPHIP_DT_F16 && m.dt_t != OPHIP_DT_F32) throw type_not_support("rope supports f16 and f32 tokens");
+        if (m.dt_t != OPHIP_DT_F16 && m.dt_t != OPHIP_DT_F32 && m.dt_t != OPHIP_DT_F64)
+            throw type_not_support("rope supports f16, f32 and f64 tokens");
         if (m.dt_p != OPHIP_DT_U32 && m.dt_p != OPHIP_DT_U64) throw type_not_support("rope supports u32 and u64 positions");
         const size_t nt = static_of(m.nt), nh = static_of(args->t_layout.shape[1]), dh = static_of(m.dh);
         const ptrdiff_t st = static_of(args->t_layout.strides[0]), sh = static_of(args->t_layout.strides[1]),
@@ -228,8 +230,9 @@ extern "C" int ophip_rope_launch(const ophip_rope *op, const ophip_rope_args *ar
         if (sp % punit != 0 || st % unit != 0 || sh % unit != 0) throw strides_not_support("misaligned strides");
         if (nt == 0 || nh == 0 || dh < 2) return;
         if (nt > 0x7fffffffu || nh > 0xffffffu || dh > 0xffffffu) throw shape_not_support("rope dimension too large");
-        const size_t smem = (dh / 2) * 8;
+        const size_t smem = (dh / 2) * (m.dt_t == OPHIP_DT_F64 ? 16 : 8);
         if (smem > 64 * 1024) throw shape_not_support("rope head dimension too large");
+        if (!args->t_base || !args->p_base) throw args_not_support("null base address");
 
         RopeParams p{};
         p.t = args->t_base;
@@ -255,7 +258,7 @@ extern "C" int ophip_rope_launch(const ophip_rope *op, const ophip_rope_args *ar
         by = (nh + hpb - 1) / hpb;
         if (by > 65535) throw shape_not_support("too many heads");
         p.heads_per_block = (uint32_t)hpb;
-        hipFunction_t fn = vec ? op->f16_vec : (m.dt_t == OPHIP_DT_F16 ? op->f16_pairs : op->f32_pairs);
+        hipFunction_t fn = vec ? op->f16_vec : m.dt_t == OPHIP_DT_F16 ? op->f16_pairs : m.dt_t == OPHIP_DT_F32 ? op->f32_pairs : op->f64_pairs;
         op->dev->make_current();
         launch(fn, Dim3{(unsigned)nt, (unsigned)by}, Dim3{256}, smem, stream_of(qa), p);
     });
@@ -311,7 +314,7 @@ struct SoftmaxVariant {
 
 struct ophip_fused_softmax : OpBase {
     std::vector<SoftmaxVariant> variants;
-    hipFunction_t stream_fn, rows4[2];  // rows4: four rows per wave, 1 or 2 vectors per lane and row
+    hipFunction_t stream_fn, stream_f32, stream_f64, rows4[2];  // rows4: four rows per wave, 1 or 2 vectors per lane and row
     explicit ophip_fused_softmax(ophip_device *d) : OpBase(d) {
         static const int table[][3] = {{8, 1, 64},  {8, 2, 64},   {8, 4, 64},   {8, 1, 256},  {8, 2, 256},
                                        {8, 4, 256}, {8, 8, 256},  {8, 4, 1024}, {8, 8, 1024}, {1, 8, 64},
@@ -322,6 +325,8 @@ struct ophip_fused_softmax : OpBase {
             variants.push_back({t[0], t[1], t[2], d->kernel("fused_softmax", name.c_str())});
         }
         stream_fn = d->kernel("fused_softmax", "softmax_f16_stream");
+        stream_f32 = d->kernel("fused_softmax", "softmax_f32_stream");
+        stream_f64 = d->kernel("fused_softmax", "softmax_f64_stream");
         rows4[0] = d->kernel("fused_softmax", "softmax_f16_rows4_p1");
         rows4[1] = d->kernel("fused_softmax", "softmax_f16_rows4_p2");
     }
@@ -340,7 +345,8 @@ extern "C" int ophip_fused_softmax_scheme(ophip_fused_softmax *, const ophip_fus
     return guard([&] {
         if (ws) *ws = 0;
         if (args->att_layout.ndim != 3) throw rank_not_support("");
-        if (args->att_layout.dt != OPHIP_DT_F16) throw type_not_support("fused softmax supports f16");
+        const uint64_t dt = args->att_layout.dt;
+        if (dt != OPHIP_DT_F16 && dt != OPHIP_DT_F32 && dt != OPHIP_DT_F64) throw type_not_support("fused softmax supports f16, f32 and f64");
     });
 }
 
@@ -349,13 +355,14 @@ extern "C" int ophip_fused_softmax_launch(const ophip_fused_softmax *op, const o
     return guard([&] {
         const ophip_tensor_layout &l = args->att_layout;
         if (l.ndim != 3) throw rank_not_support("");
-        if (l.dt != OPHIP_DT_F16) throw type_not_support("fused softmax supports f16");
+        if (l.dt != OPHIP_DT_F16 && l.dt != OPHIP_DT_F32 && l.dt != OPHIP_DT_F64) throw type_not_support("fused softmax supports f16, f32 and f64");
+        const ptrdiff_t unit = (ptrdiff_t)ophip_dtype_nbytes(l.dt);
         if (args->att_mask != OPHIP_MASK_NONE && args->att_mask != OPHIP_MASK_CAUSAL)
             throw args_not_support("unknown attention mask");
         const size_t nh = static_of(l.shape[0]), seq = static_of(l.shape[1]), att = static_of(l.shape[2]);
         const ptrdiff_t sh = static_of(l.strides[0]), ss = static_of(l.strides[1]), sa = static_of(l.strides[2]);
-        if (sa != 2) throw strides_not_support("fused softmax needs a contiguous last dimension");
-        if (sh % 2 != 0 || ss % 2 != 0) throw strides_not_support("misaligned strides");
+        if (sa != unit) throw strides_not_support("fused softmax needs a contiguous last dimension");
+        if (sh % unit != 0 || ss % unit != 0) throw strides_not_support("misaligned strides");
         const size_t rows = nh * seq;
         if (rows == 0) return;
         const bool causal = args->att_mask == OPHIP_MASK_CAUSAL;
@@ -372,6 +379,12 @@ extern "C" int ophip_fused_softmax_launch(const ophip_fused_softmax *op, const o
         p.att_len = (uint32_t)att;
         p.causal = causal;
 
+        if (!p.att) throw args_not_support("null base address");
+        if (l.dt != OPHIP_DT_F16) {
+            op->dev->make_current();
+            launch(l.dt == OPHIP_DT_F32 ? op->stream_f32 : op->stream_f64, Dim3{(unsigned)rows}, Dim3{1024}, 0, stream_of(qa), p);
+            return;
+        }
         const bool vec = aligned16(p.att) && mult16(sh) && mult16(ss);
         const int want_vec = vec ? 8 : 1;
         // narrowest group that holds the row in registers; with few rows prefer a
@@ -626,11 +639,12 @@ extern "C" int ophip_rearrange_launch(const ophip_rearrange *op, const ophip_rea
 // Args::meta: swiglu/args.rs:31-50; launch checks: swiglu/cuda/mod.rs:53-98.
 
 struct ophip_swiglu : OpBase {
-    hipFunction_t f16_vec, f16_scalar, f32_scalar;
+    hipFunction_t f16_vec, f16_scalar, f32_scalar, f64_scalar;
     explicit ophip_swiglu(ophip_device *d) : OpBase(d) {
         f16_vec = d->kernel("swiglu", "swiglu_f16_vec");
         f16_scalar = d->kernel("swiglu", "swiglu_f16_scalar");
         f32_scalar = d->kernel("swiglu", "swiglu_f32_scalar");
+        f64_scalar = d->kernel("swiglu", "swiglu_f64_scalar");
     }
 };
 
@@ -667,7 +681,7 @@ extern "C" int ophip_swiglu_launch(const ophip_swiglu *op, const ophip_swiglu_ar
                                    const ophip_queue_alloc *qa) {
     return guard([&] {
         const SwigluMeta m = swiglu_meta(*args);
-        if (m.dt != OPHIP_DT_F16 && m.dt != OPHIP_DT_F32) throw type_not_support("swiglu supports f16 and f32");
+        if (m.dt != OPHIP_DT_F16 && m.dt != OPHIP_DT_F32 && m.dt != OPHIP_DT_F64) throw type_not_support("swiglu supports f16, f32 and f64");
         const size_t n = static_of(m.n), d = static_of(m.d);
         const ptrdiff_t sgn = static_of(args->gate_layout.strides[0]), sgd = static_of(args->gate_layout.strides[1]);
         const ptrdiff_t sun = static_of(args->up_layout.strides[0]), sud = static_of(args->up_layout.strides[1]);
@@ -688,7 +702,8 @@ extern "C" int ophip_swiglu_launch(const ophip_swiglu *op, const ophip_swiglu_ar
         const size_t items = vec ? d / 8 : d;
         const unsigned gx = std::min<unsigned>(ceil_div(items, 256), 65535u);
         const unsigned gy = (unsigned)std::min<size_t>(n, 65535);
-        hipFunction_t fn = vec ? op->f16_vec : (m.dt == OPHIP_DT_F16 ? op->f16_scalar : op->f32_scalar);
+        hipFunction_t fn = vec ? op->f16_vec : m.dt == OPHIP_DT_F16 ? op->f16_scalar : m.dt == OPHIP_DT_F32 ? op->f32_scalar : op->f64_scalar;
+        if (!p.gate || !p.up) throw args_not_support("null base address");
         op->dev->make_current();
         launch(fn, Dim3{gx, gy}, Dim3{256}, 0, stream_of(qa), p);
     });

@@ -11,7 +11,7 @@ using namespace ophip;
 
 namespace {
 
-const char *dt_tag(uint64_t dt) { return dt == OPHIP_DT_F16 ? "f16" : dt == OPHIP_DT_F32 ? "f32" : "?"; }
+const char *dt_tag(uint64_t dt) { return dt == OPHIP_DT_F16 ? "f16" : dt == OPHIP_DT_F32 ? "f32" : dt == OPHIP_DT_F64 ? "f64" : "?"; }
 
 }  // namespace
 
@@ -68,9 +68,10 @@ extern "C" int ophip_layer_norm_launch(const ophip_layer_norm *op, const ophip_l
         const ptrdiff_t nsy = static_of(args->y_layout.strides[0]), dsy = static_of(args->y_layout.strides[1]);
         const ptrdiff_t nsx = static_of(args->x_layout.strides[0]), dsx = static_of(args->x_layout.strides[1]);
         const ptrdiff_t dss = static_of(args->scale_layout.strides[0]), dsb = static_of(args->bias_layout.strides[0]);
+        const bool f64 = m.dt_a == OPHIP_DT_F64 && m.dt_w == OPHIP_DT_F64;
         const bool ok = (m.dt_a == OPHIP_DT_F16 && (m.dt_w == OPHIP_DT_F16 || m.dt_w == OPHIP_DT_F32)) ||
-                        (m.dt_a == OPHIP_DT_F32 && m.dt_w == OPHIP_DT_F32);
-        if (!ok) throw type_not_support("layer_norm supports (scale, x) in (f16,f16), (f32,f16), (f32,f32)");
+                        (m.dt_a == OPHIP_DT_F32 && m.dt_w == OPHIP_DT_F32) || f64;
+        if (!ok) throw type_not_support("layer_norm supports (scale, x) in (f16,f16), (f32,f16), (f32,f32), (f64,f64)");
         const ptrdiff_t unit = (ptrdiff_t)ophip_dtype_nbytes(m.dt_a), wunit = (ptrdiff_t)ophip_dtype_nbytes(m.dt_w);
         if (dsy != unit || dsx != unit || dss != wunit || dsb != wunit)
             throw strides_not_support("layer_norm needs contiguous inner dimensions");
@@ -90,8 +91,9 @@ extern "C" int ophip_layer_norm_launch(const ophip_layer_norm *op, const ophip_l
         p.epsilon = args->epsilon;
         const std::string base = std::string("layer_norm_") + dt_tag(m.dt_a) + "_" + dt_tag(m.dt_w);
         const size_t vec_elems = 16 / (size_t)unit;
-        const bool vec = d % vec_elems == 0 && aligned16(p.y) && aligned16(p.x) && aligned16(p.scale) &&
+        const bool vec = !f64 && d % vec_elems == 0 && aligned16(p.y) && aligned16(p.x) && aligned16(p.scale) &&
                          aligned16(p.bias) && mult16(nsy) && mult16(nsx);
+        if (!p.y || !p.x || !p.scale || !p.bias) throw args_not_support("null base address");
         op->dev->make_current();
         if (!vec) {
             launch(op->dev->kernel("layer_norm", (base + "_scalar").c_str()), Dim3{(unsigned)n}, Dim3{256}, 0,
@@ -146,7 +148,7 @@ extern "C" int ophip_gelu_launch(const ophip_gelu *op, const ophip_gelu_args *ar
         const uint64_t dt = args->layout.dt;
         const size_t n = static_of(args->layout.shape[0]), d = static_of(args->layout.shape[1]);
         const ptrdiff_t sn = static_of(args->layout.strides[0]), sd = static_of(args->layout.strides[1]);
-        if (dt != OPHIP_DT_F16 && dt != OPHIP_DT_F32) throw type_not_support("gelu supports f16 and f32");
+        if (dt != OPHIP_DT_F16 && dt != OPHIP_DT_F32 && dt != OPHIP_DT_F64) throw type_not_support("gelu supports f16, f32 and f64");
         const ptrdiff_t unit = (ptrdiff_t)ophip_dtype_nbytes(dt);
         if (sd != unit) throw strides_not_support("gelu needs a contiguous inner dimension");
         if (sn % unit != 0) throw strides_not_support("misaligned strides");
@@ -161,7 +163,8 @@ extern "C" int ophip_gelu_launch(const ophip_gelu *op, const ophip_gelu_args *ar
         const size_t items = vec ? d / 8 : d;
         const unsigned gx = std::min<unsigned>(ceil_div(items, 256), 65535u);
         const unsigned gy = (unsigned)std::min<size_t>(n, 65535);
-        const char *name = vec ? "gelu_f16_vec" : dt == OPHIP_DT_F16 ? "gelu_f16_scalar" : "gelu_f32_scalar";
+        const char *name = vec ? "gelu_f16_vec" : dt == OPHIP_DT_F16 ? "gelu_f16_scalar" : dt == OPHIP_DT_F32 ? "gelu_f32_scalar" : "gelu_f64_scalar";
+        if (!p.base) throw args_not_support("null base address");
         op->dev->make_current();
         launch(op->dev->kernel("gelu", name), Dim3{gx, gy}, Dim3{256}, 0, stream_of(qa), p);
     });
@@ -266,7 +269,7 @@ extern "C" int ophip_add_launch(const ophip_add *op, const ophip_add_args *args,
                                 const ophip_queue_alloc *qa) {
     return guard([&] {
         AddScheme s = add_scheme(*args);
-        if (s.dt != OPHIP_DT_F16 && s.dt != OPHIP_DT_F32) throw type_not_support("add supports f16 and f32");
+        if (s.dt != OPHIP_DT_F16 && s.dt != OPHIP_DT_F32 && s.dt != OPHIP_DT_F64) throw type_not_support("add supports f16, f32 and f64");
         if (s.dims.size() > OPHIP_REARRANGE_MAXD)
             throw rank_not_support("add supports at most " + std::to_string(OPHIP_REARRANGE_MAXD) +
                                    " non-mergeable dimensions");
@@ -284,7 +287,7 @@ extern "C" int ophip_add_launch(const ophip_add *op, const ophip_add_args *args,
         const size_t per = 16 / unit;
         if (!s.dims.empty()) {
             AddDim &in = s.dims.back();
-            vec = in.c == (ptrdiff_t)unit && in.a == (ptrdiff_t)unit && in.b == (ptrdiff_t)unit && in.d % per == 0 &&
+            vec = s.dt != OPHIP_DT_F64 && in.c == (ptrdiff_t)unit && in.a == (ptrdiff_t)unit && in.b == (ptrdiff_t)unit && in.d % per == 0 &&
                   aligned16(p.c) && aligned16(p.a) && aligned16(p.b);
             for (size_t i = 0; vec && i + 1 < s.dims.size(); ++i)
                 vec = mult16(s.dims[i].c) && mult16(s.dims[i].a) && mult16(s.dims[i].b);
@@ -304,6 +307,7 @@ extern "C" int ophip_add_launch(const ophip_add *op, const ophip_add_args *args,
         }
         const std::string name = std::string("add_") + dt_tag(s.dt) + (vec ? "_vec" : "_scalar");
         const unsigned blocks = (unsigned)std::min<size_t>(ceil_div(total, 256), 1u << 20);
+        if (!p.c || !p.a || !p.b) throw args_not_support("null base address");
         op->dev->make_current();
         launch(op->dev->kernel("add", name.c_str()), Dim3{blocks}, Dim3{256}, 0, stream_of(qa), p);
     });
@@ -369,7 +373,7 @@ extern "C" int ophip_add_rows_launch(const ophip_add_rows *op, const ophip_add_r
                         nsd = static_of(args->dst_layout.strides[2]);
         const ptrdiff_t bsi = static_of(args->idx_layout.strides[0]), msi = static_of(args->idx_layout.strides[1]);
         const ptrdiff_t kss = static_of(args->src_layout.strides[0]), nss = static_of(args->src_layout.strides[1]);
-        if (r.dt != OPHIP_DT_F16 && r.dt != OPHIP_DT_F32) throw type_not_support("add_rows supports f16 and f32");
+        if (r.dt != OPHIP_DT_F16 && r.dt != OPHIP_DT_F32 && r.dt != OPHIP_DT_F64) throw type_not_support("add_rows supports f16, f32 and f64");
         if (r.dt_idx != OPHIP_DT_U32 && r.dt_idx != OPHIP_DT_U64) throw type_not_support("idx must be u32 or u64");
         const ptrdiff_t unit = (ptrdiff_t)ophip_dtype_nbytes(r.dt), iunit = (ptrdiff_t)ophip_dtype_nbytes(r.dt_idx);
         for (ptrdiff_t st : {bsd, msd, nsd, kss, nss})
@@ -400,11 +404,12 @@ extern "C" int ophip_add_rows_launch(const ophip_add_rows *op, const ophip_add_r
         const size_t items = vec ? n / 8 : n;
         const unsigned gx = std::min<unsigned>(ceil_div(items, 256), 65535u);
         const unsigned gy = (unsigned)std::min<size_t>(batch * m, 65535);
+        if (!p.dst || !p.src || !p.idx) throw args_not_support("null base address");
         op->dev->make_current();
         if (vec) {
             launch(op->dev->kernel("add_rows", "add_rows_f16_vec"), Dim3{gx, gy}, Dim3{256}, 0, stream_of(qa), p);
         } else {
-            const char *name = r.dt == OPHIP_DT_F16 ? "add_rows_f16_scalar" : "add_rows_f32_scalar";
+            const char *name = r.dt == OPHIP_DT_F16 ? "add_rows_f16_scalar" : r.dt == OPHIP_DT_F32 ? "add_rows_f32_scalar" : "add_rows_f64_scalar";
             launch(op->dev->kernel("add_rows", name), Dim3{gx, gy}, Dim3{256}, 0, stream_of(qa), q);
         }
     });

@@ -6,6 +6,8 @@
 // multiply-high divisions; dimensions are ordered by descending c stride, so consecutive
 // threads write ascending addresses.  f16 sums are formed in f32 and rounded once, as
 // half's `f16 + f16` does.
+#include <type_traits>
+
 #include "device_util.h"
 
 struct AddOffsets {
@@ -52,11 +54,13 @@ template <typename T>
 __device__ __forceinline__ void add_scalar(const AddParams &p) {
     for (uint32_t g = blockIdx.x * blockDim.x + threadIdx.x; g < p.total; g += gridDim.x * blockDim.x) {
         const AddOffsets o = add_decode(p, g);
-        const float a = (float)*reinterpret_cast<const T *>(reinterpret_cast<const char *>(p.a) + o.a);
-        const float b = (float)*reinterpret_cast<const T *>(reinterpret_cast<const char *>(p.b) + o.b);
+        using Calc = std::conditional_t<sizeof(T) == 8, double, float>;  // f64 data adds in f64
+        const Calc a = (Calc)*reinterpret_cast<const T *>(reinterpret_cast<const char *>(p.a) + o.a);
+        const Calc b = (Calc)*reinterpret_cast<const T *>(reinterpret_cast<const char *>(p.b) + o.b);
         *reinterpret_cast<T *>(reinterpret_cast<char *>(p.c) + o.c) = (T)(a + b);
     }
 }
 
 extern "C" __global__ void __launch_bounds__(256) add_f16_scalar(AddParams p) { add_scalar<f16>(p); }
 extern "C" __global__ void __launch_bounds__(256) add_f32_scalar(AddParams p) { add_scalar<float>(p); }
+extern "C" __global__ void __launch_bounds__(256) add_f64_scalar(AddParams p) { add_scalar<double>(p); }

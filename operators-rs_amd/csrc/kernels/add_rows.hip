@@ -3,6 +3,8 @@
 // blockIdx.y walks the b * m destination rows, blockIdx.x the row in 16-byte vectors (or single
 // elements when the row is not 16-byte friendly).  The row index is read once per workgroup.
 // An index >= k (the reference asserts) leaves the destination row unchanged.
+#include <type_traits>
+
 #include "device_util.h"
 
 __device__ __forceinline__ bool add_rows_locate(const AddRowsParams &p, uint32_t bm, char *&dst, const char *&src) {
@@ -42,7 +44,8 @@ __device__ __forceinline__ void add_rows_scalar(const AddRowsParams &p, int64_t 
         for (uint32_t j = blockIdx.x * blockDim.x + threadIdx.x; j < p.n; j += gridDim.x * blockDim.x) {
             T *d = reinterpret_cast<T *>(dst + (int64_t)j * nsd);
             const T *s = reinterpret_cast<const T *>(src + (int64_t)j * nss);
-            *d = (T)((float)*d + (float)*s);
+            using Calc = std::conditional_t<sizeof(T) == 8, double, float>;  // f64 data adds in f64
+            *d = (T)((Calc)*d + (Calc)*s);
         }
     }
 }
@@ -56,4 +59,7 @@ extern "C" __global__ void __launch_bounds__(256) add_rows_f16_scalar(AddRowsSca
 }
 extern "C" __global__ void __launch_bounds__(256) add_rows_f32_scalar(AddRowsScalarParams q) {
     add_rows_scalar<float>(q.p, q.nsd, q.nss);
+}
+extern "C" __global__ void __launch_bounds__(256) add_rows_f64_scalar(AddRowsScalarParams q) {
+    add_rows_scalar<double>(q.p, q.nsd, q.nss);
 }

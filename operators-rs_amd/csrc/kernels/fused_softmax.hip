@@ -215,6 +215,47 @@ extern "C" __global__ void __launch_bounds__(1024) softmax_f16_stream(SoftmaxPar
     for (uint32_t c = kept + threadIdx.x; c < p.att_len; c += G) row[c] = (f16)0.f;
 }
 
+// f32 and f64 rows (fuesd_softmax/common_cpu/mod.rs:147-193): the same three sweeps in the element's own arithmetic, the
+// library's exp; one 1024-thread workgroup per row.  No register-resident variants: the hot path is f16.
+template <typename T>
+__device__ __forceinline__ void softmax_stream_wide(const SoftmaxParams &p) {
+    constexpr int G = 1024;
+    __shared__ T smem[G / WAVE];
+    const uint32_t flat = blockIdx.x;
+    const uint32_t h = flat / p.seq, r = flat % p.seq;
+    const uint32_t kept = kept_columns(p, r);
+    T *row = reinterpret_cast<T *>(reinterpret_cast<char *>(p.att) + (int64_t)h * p.sh + (int64_t)r * p.ss);
+    const uint32_t wave = threadIdx.x / WAVE;
+    auto across = [&](T v, auto op) {  // every thread ends with op over the whole workgroup, combined in a fixed order
+#pragma unroll
+        for (int o = WAVE / 2; o > 0; o >>= 1) v = op(v, __shfl_xor(v, o, WAVE));
+        __syncthreads();
+        if ((threadIdx.x & (WAVE - 1)) == 0) smem[wave] = v;
+        __syncthreads();
+        T s = smem[0];
+#pragma unroll
+        for (int i = 1; i < G / WAVE; ++i) s = op(s, smem[i]);
+        return s;
+    };
+    T mx = -INFINITY;
+    for (uint32_t c = threadIdx.x; c < kept; c += G) mx = row[c] > mx ? row[c] : mx;
+    mx = across(mx, [](T a, T b) { return a > b ? a : b; });
+    T sum = 0;
+    for (uint32_t c = threadIdx.x; c < kept; c += G) {
+        T ex;
+        if constexpr (sizeof(T) == 8) ex = exp(row[c] - mx);
+        else ex = expf(row[c] - mx);
+        sum += ex;
+        row[c] = ex;
+    }
+    sum = across(sum, [](T a, T b) { return a + b; });
+    const T inv = (T)1 / sum;
+    for (uint32_t c = threadIdx.x; c < kept; c += G) row[c] = row[c] * inv;
+    for (uint32_t c = kept + threadIdx.x; c < p.att_len; c += G) row[c] = (T)0;
+}
+extern "C" __global__ void __launch_bounds__(1024) softmax_f32_stream(SoftmaxParams p) { softmax_stream_wide<float>(p); }
+extern "C" __global__ void __launch_bounds__(1024) softmax_f64_stream(SoftmaxParams p) { softmax_stream_wide<double>(p); }
+
 #define SOFTMAX_REG(VEC, PT, G)                                                                  \
     extern "C" __global__ void __launch_bounds__((G) < 256 ? 256 : (G))                          \
         softmax_f16_v##VEC##_p##PT##_g##G(SoftmaxParams p) {                                     \

@@ -25,14 +25,23 @@ extern "C" __global__ void __launch_bounds__(256) gelu_f16_vec(GeluParams p) {
     }
 }
 
+// f64 data in f64 (gelu/common_cpu/mod.rs:62-64), sqrt(2 / pi) from the f64 constant
+__device__ __forceinline__ double gelu_f64(double x) {
+    const double c = 0.79788456080286535588;
+    return 0.5 * x * (1.0 + tanh(c * (x + 0.044715 * (x * x * x))));
+}
+
 template <typename T>
 __device__ __forceinline__ void gelu_scalar(const GeluParams &p) {
     for (uint32_t row = blockIdx.y; row < p.n; row += gridDim.y) {
         T *r = reinterpret_cast<T *>(reinterpret_cast<char *>(p.base) + (int64_t)row * p.sn);
-        for (uint32_t j = blockIdx.x * blockDim.x + threadIdx.x; j < p.d; j += gridDim.x * blockDim.x)
-            r[j] = (T)gelu_f32((float)r[j]);
+        for (uint32_t j = blockIdx.x * blockDim.x + threadIdx.x; j < p.d; j += gridDim.x * blockDim.x) {
+            if constexpr (sizeof(T) == 8) r[j] = gelu_f64(r[j]);
+            else r[j] = (T)gelu_f32((float)r[j]);
+        }
     }
 }
 
 extern "C" __global__ void __launch_bounds__(256) gelu_f16_scalar(GeluParams p) { gelu_scalar<f16>(p); }
 extern "C" __global__ void __launch_bounds__(256) gelu_f32_scalar(GeluParams p) { gelu_scalar<float>(p); }
+extern "C" __global__ void __launch_bounds__(256) gelu_f64_scalar(GeluParams p) { gelu_scalar<double>(p); }

@@ -558,32 +558,33 @@ extern "C" __global__ void __launch_bounds__(256) gemm_splitk_reduce(GemmParams 
 template <typename T>
 __device__ __forceinline__ void gemm_generic(const GemmParams &p) {
     constexpr int BM = 64, BN = 64, BK = 16;
-    __shared__ float Ps[BK][BM + 4];
-    __shared__ float Qs[BK][BN + 4];
+    using Acc = std::conditional_t<sizeof(T) == 8, double, float>;  // f64 data multiplies and adds in f64
+    __shared__ Acc Ps[BK][BM + 4];
+    __shared__ Acc Qs[BK][BN + 4];
     const uint32_t bat = blockIdx.z;
     const uint32_t i0 = blockIdx.y * BM, j0 = blockIdx.x * BN;
     const T *pb = reinterpret_cast<const T *>(p.p) + (int64_t)bat * p.p_sb;
     const T *qb = reinterpret_cast<const T *>(p.q) + (int64_t)bat * p.q_sb;
     T *db = reinterpret_cast<T *>(p.d) + (int64_t)bat * p.d_sb;
     const uint32_t tx = threadIdx.x % 16, ty = threadIdx.x / 16;
-    float acc[4][4] = {};
+    Acc acc[4][4] = {};
     for (uint32_t k0 = 0; k0 < p.K; k0 += BK) {
         for (uint32_t e = threadIdx.x; e < BM * BK; e += 256) {
             uint32_t li, ll;
             if (p.p_sl == 1) { ll = e % BK; li = e / BK; } else { li = e % BM; ll = e / BM; }
             const uint32_t i = i0 + li, l = k0 + ll;
-            Ps[ll][li] = (i < p.M && l < p.K) ? (float)pb[(int64_t)i * p.p_si + (int64_t)l * p.p_sl] : 0.f;
+            Ps[ll][li] = (i < p.M && l < p.K) ? (Acc)pb[(int64_t)i * p.p_si + (int64_t)l * p.p_sl] : (Acc)0;
         }
         for (uint32_t e = threadIdx.x; e < BN * BK; e += 256) {
             uint32_t lj, ll;
             if (p.q_sl == 1) { ll = e % BK; lj = e / BK; } else { lj = e % BN; ll = e / BN; }
             const uint32_t j = j0 + lj, l = k0 + ll;
-            Qs[ll][lj] = (j < p.N && l < p.K) ? (float)qb[(int64_t)l * p.q_sl + (int64_t)j * p.q_sj] : 0.f;
+            Qs[ll][lj] = (j < p.N && l < p.K) ? (Acc)qb[(int64_t)l * p.q_sl + (int64_t)j * p.q_sj] : (Acc)0;
         }
         __syncthreads();
 #pragma unroll
         for (int l = 0; l < BK; ++l) {
-            float a[4], b[4];
+            Acc a[4], b[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) a[r] = Ps[l][ty * 4 + r];
 #pragma unroll
@@ -602,8 +603,8 @@ __device__ __forceinline__ void gemm_generic(const GemmParams &p) {
             const uint32_t i = i0 + ty * 4 + r, j = j0 + tx * 4 + c;
             if (i < p.M && j < p.N) {
                 T *e = db + (int64_t)i * p.d_si + (int64_t)j * p.d_sj;
-                float v = p.alpha * acc[r][c];
-                if (p.read_dst) v = p.beta * (float)*e + v;
+                Acc v = (Acc)p.alpha * acc[r][c];
+                if (p.read_dst) v = (Acc)p.beta * (Acc)*e + v;
                 *e = (T)v;
             }
         }
@@ -616,5 +617,6 @@ extern "C" __global__ void __launch_bounds__(256) gemm_fill_u32(FillU32Params p)
     if (i < p.count) reinterpret_cast<uint32_t *>(p.dst)[i] = p.value;
 }
 
+extern "C" __global__ void __launch_bounds__(256) gemm_generic_f64(GemmParams p) { gemm_generic<double>(p); }
 extern "C" __global__ void __launch_bounds__(256) gemm_generic_f16(GemmParams p) { gemm_generic<f16>(p); }
 extern "C" __global__ void __launch_bounds__(256) gemm_generic_f32(GemmParams p) { gemm_generic<float>(p); }

@@ -235,3 +235,35 @@ extern "C" __global__ void __launch_bounds__(256) layer_norm_f16_f32_rows(LayerN
 LAYER_NORM(f16_f16, f16, f16)
 LAYER_NORM(f16_f32, f16, float)
 LAYER_NORM(f32_f32, float, float)
+
+// f64 rows with f64 scale and bias (layer_norm/common_cpu/mod.rs:97 lists the pair): all arithmetic in f64, as the
+// reference's, one workgroup per row.  No vector variant: the hot path is f16.
+extern "C" __global__ void __launch_bounds__(256) layer_norm_f64_f64_scalar(LayerNormParams p) {
+    constexpr int G = 256;
+    __shared__ double smem[2][G / WAVE];
+    const uint32_t row = blockIdx.x;
+    const double *xr = reinterpret_cast<const double *>(reinterpret_cast<const char *>(p.x) + (int64_t)row * p.nsx);
+    double *yr = reinterpret_cast<double *>(reinterpret_cast<char *>(p.y) + (int64_t)row * p.nsy);
+    double s1 = 0.0, s2 = 0.0;
+    for (uint32_t j = threadIdx.x; j < p.d; j += G) {
+        const double f = xr[j];
+        s1 += f;
+        s2 += f * f;
+    }
+#pragma unroll
+    for (int o = WAVE / 2; o > 0; o >>= 1) {
+        s1 += __shfl_xor(s1, o, WAVE);
+        s2 += __shfl_xor(s2, o, WAVE);
+    }
+    if ((threadIdx.x & (WAVE - 1)) == 0) {
+        smem[0][threadIdx.x / WAVE] = s1;
+        smem[1][threadIdx.x / WAVE] = s2;
+    }
+    __syncthreads();
+    s1 = (smem[0][0] + smem[0][1]) + (smem[0][2] + smem[0][3]);
+    s2 = (smem[1][0] + smem[1][1]) + (smem[1][2] + smem[1][3]);
+    const double n = (double)p.d, e = s1 / n, e2 = s2 / n;
+    const double k = 1.0 / (sqrt(e2 - e * e) + (double)p.epsilon);
+    const double *sc = reinterpret_cast<const double *>(p.scale), *bi = reinterpret_cast<const double *>(p.bias);
+    for (uint32_t j = threadIdx.x; j < p.d; j += G) yr[j] = fma(xr[j] - e, sc[j] * k, bi[j]);
+}

@@ -84,3 +84,30 @@ __device__ __forceinline__ void rope_pairs(const RopeParams &p) {
 
 extern "C" __global__ void __launch_bounds__(256) rope_f16_pairs(RopeParams p) { rope_pairs<f16>(p); }
 extern "C" __global__ void __launch_bounds__(256) rope_f32_pairs(RopeParams p) { rope_pairs<float>(p); }
+
+// f64 tokens (rope/common_cpu/mod.rs:125-126): position, angle, sine and cosine in f64, as the reference computes them;
+// the table holds dh/2 (sin, cos) pairs of 16 bytes.
+extern "C" __global__ void __launch_bounds__(256) rope_f64_pairs(RopeParams p) {
+    double2 *table = reinterpret_cast<double2 *>(rope_sc);
+    const uint32_t token = blockIdx.x;
+    const uint32_t H = p.dh / 2;
+    const char *pp = reinterpret_cast<const char *>(p.pos) + (int64_t)token * p.sp;
+    const double pos = p.pos_is_u64 ? (double)*reinterpret_cast<const uint64_t *>(pp) : (double)*reinterpret_cast<const uint32_t *>(pp);
+    for (uint32_t k = threadIdx.x; k < H; k += blockDim.x) {
+        const double ang = pos / pow((double)p.theta, (double)k / (double)H);
+        table[k] = double2{sin(ang), cos(ang)};
+    }
+    __syncthreads();
+    const uint32_t h0 = blockIdx.y * p.heads_per_block;
+    const uint32_t h1 = min(h0 + p.heads_per_block, p.nh);
+    const uint32_t total = (h1 - h0) * H;
+    char *base = reinterpret_cast<char *>(p.t) + (int64_t)token * p.st;
+    for (uint32_t v = threadIdx.x; v < total; v += blockDim.x) {
+        const uint32_t h = h0 + v / H, k = v % H;
+        double *ptr = reinterpret_cast<double *>(base + (int64_t)h * p.sh) + 2 * k;
+        const double2 sc = table[k];
+        const double a = ptr[0], b = ptr[1];
+        ptr[0] = a * sc.y - b * sc.x;
+        ptr[1] = a * sc.x + b * sc.y;
+    }
+}

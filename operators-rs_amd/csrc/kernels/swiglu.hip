@@ -28,15 +28,21 @@ extern "C" __global__ void __launch_bounds__(256) swiglu_f16_vec(SwigluParams p)
     }
 }
 
+// f64 data is computed in f64, as the reference does (swiglu/common_cpu/mod.rs:74-76): the library's exp, an IEEE division
+__device__ __forceinline__ double swiglu_f64(double a, double b) { return (a * (1.0 / (1.0 + exp(-a)))) * b; }
+
 template <typename T>
 __device__ __forceinline__ void swiglu_scalar(const SwigluParams &p) {
     for (uint32_t row = blockIdx.y; row < p.n; row += gridDim.y) {
         T *g = reinterpret_cast<T *>(reinterpret_cast<char *>(p.gate) + (int64_t)row * p.sgn);
         const T *u = reinterpret_cast<const T *>(reinterpret_cast<const char *>(p.up) + (int64_t)row * p.sun);
-        for (uint32_t j = blockIdx.x * blockDim.x + threadIdx.x; j < p.d; j += gridDim.x * blockDim.x)
-            g[j] = (T)swiglu_f32((float)g[j], (float)u[j]);
+        for (uint32_t j = blockIdx.x * blockDim.x + threadIdx.x; j < p.d; j += gridDim.x * blockDim.x) {
+            if constexpr (sizeof(T) == 8) g[j] = swiglu_f64(g[j], u[j]);
+            else g[j] = (T)swiglu_f32((float)g[j], (float)u[j]);
+        }
     }
 }
 
 extern "C" __global__ void __launch_bounds__(256) swiglu_f16_scalar(SwigluParams p) { swiglu_scalar<f16>(p); }
 extern "C" __global__ void __launch_bounds__(256) swiglu_f32_scalar(SwigluParams p) { swiglu_scalar<float>(p); }
+extern "C" __global__ void __launch_bounds__(256) swiglu_f64_scalar(SwigluParams p) { swiglu_scalar<double>(p); }

@@ -281,10 +281,16 @@ static inline int32_t f32_total_key(float f) {
     v ^= (int32_t)(((uint32_t)(v >> 31)) >> 1);
     return v;
 }
+static inline int64_t f64_total_key(double f) {
+    int64_t v;
+    memcpy(&v, &f, 8);
+    v ^= (int64_t)(((uint64_t)(v >> 63)) >> 1);
+    return v;
+}
 
 /*
  * operators/src/fuesd_softmax/common_cpu/mod.rs:99-114 (row loop, rayon over
- * nh*seq rows) and :117-145 (f16), :147-169 (f32).
+ * nh*seq rows) and :117-145 (f16), :147-169 (f32), :171-193 (f64: the f32 code in f64).
  * Row (h, r) keeps `causal = att_len - seq_len + r + 1` columns (mask 1) or all
  * (mask 0).  f16: max by total order; e = exp(f32(x) - max) is stored as f16
  * while the un-rounded e is summed sequentially; the stored f16 is re-read and
@@ -296,7 +302,7 @@ static inline int32_t f32_total_key(float f) {
  */
 ORACLE_API int oracle_fused_softmax(void *att, ptrdiff_t sh, ptrdiff_t ss, ptrdiff_t sa, size_t nh,
                                     size_t seq_len, size_t att_len, int mask, int dt) {
-    if (dt != ORACLE_F16 && dt != ORACLE_F32) return ORACLE_TYPE_NOT_SUPPORT;
+    if (dt != ORACLE_F16 && dt != ORACLE_F32 && dt != ORACLE_F64) return ORACLE_TYPE_NOT_SUPPORT;
     if (mask == 1 && att_len < seq_len) return ORACLE_SHAPE_NOT_SUPPORT;
     if (att_len == 0 && nh * seq_len != 0) return ORACLE_SHAPE_NOT_SUPPORT;
     char *base = (char *)att;
@@ -330,6 +336,22 @@ ORACLE_API int oracle_fused_softmax(void *att, ptrdiff_t sh, ptrdiff_t ss, ptrdi
                 uint16_t z = 0;
                 memcpy(row + c * sa, &z, 2);
             }
+        } else if (dt == ORACLE_F64) {
+            double best = ld_f64(row);
+            for (ptrdiff_t c = 1; c < causal; c++) {
+                double v = ld_f64(row + c * sa);
+                if (!(f64_total_key(best) > f64_total_key(v))) best = v;
+            }
+            double sum = 0.0;
+            for (ptrdiff_t c = 0; c < causal; c++) {
+                double e = exp(ld_f64(row + c * sa) - best);
+                st_f64(row + c * sa, e);
+                sum = sum + e;
+            }
+            double div = 1.0 / sum;
+            for (ptrdiff_t c = 0; c < causal; c++)
+                st_f64(row + c * sa, ld_f64(row + c * sa) * div);
+            for (ptrdiff_t c = causal; c < (ptrdiff_t)att_len; c++) st_f64(row + c * sa, 0.0);
         } else {
             float best = ld_f32(row);
             for (ptrdiff_t c = 1; c < causal; c++) {

@@ -350,7 +350,7 @@ def test_softmax_errors(gpu, stream):
         op.scheme(ophip.FusedSoftmaxArgs(1, L(dt.F16, [4, 4], [8, 2]), None), 0)
     assert e.value.kind == "RankNotSupport"
     with pytest.raises(ophip.SchemeError) as e:
-        op.scheme(ophip.FusedSoftmaxArgs(1, L(dt.F32, [1, 4, 4], [64, 16, 4]), None), 0)
+        op.scheme(ophip.FusedSoftmaxArgs(1, L(dt.BF16, [1, 4, 4], [32, 8, 2]), None), 0)
     assert e.value.kind == "TypeNotSupport"
     with pytest.raises(ophip.LaunchError) as e:
         op.launch(ophip.FusedSoftmaxArgs(1, L(dt.F16, [1, 4, 4], [64, 16, 4]), None), None, stream)
@@ -1218,8 +1218,8 @@ def test_mat_mul_errors(gpu, stream):
                                    L(dt.F16, [3, 7], [14, 2]), None, 1.0), None, stream)
     assert e.value.kind == "ShapeMismatch"
     with pytest.raises(ophip.LaunchError) as e:
-        op.launch(ophip.MatMulArgs(L(dt.F64, [5, 7], [56, 8]), None, 0.0, L(dt.F64, [5, 3], [24, 8]), None,
-                                   L(dt.F64, [3, 7], [56, 8]), None, 1.0), None, stream)
+        op.launch(ophip.MatMulArgs(L(dt.BF16, [5, 7], [14, 2]), None, 0.0, L(dt.BF16, [5, 3], [6, 2]), None,
+                                   L(dt.BF16, [3, 7], [14, 2]), None, 1.0), None, stream)
     assert e.value.kind == "TypeNotSupport"
     with pytest.raises(ophip.LaunchError) as e:
         op.launch(ophip.MatMulArgs(L(dt.F16, [5, None], [14, 2]), None, 0.0, L(dt.F16, [5, 3], [6, 2]), None,

@@ -243,6 +243,33 @@ def test_softmax_shift_invariance_and_double_rounding():
     assert np.abs(out.astype(f64) - want.astype(f64)).max() <= float(ulp16(want).max())  # libm expf vs numpy exp
 
 
+@pytest.mark.parametrize("dtype", [f32, f64])
+def test_softmax_f32_and_f64_closed_form(dtype):
+    """fuesd_softmax/common_cpu/mod.rs:147-193: the same algorithm in the element's own arithmetic."""
+    rng = np.random.default_rng(4)
+    eps = float(np.finfo(dtype).eps)
+    for seq, al in [(1, 37), (6, 6), (5, 64)]:
+        att = (rng.standard_normal((2, seq, al)) * 2).astype(dtype)
+        out = oracle.fused_softmax(att.copy(), causal=True)
+        ref = softmax_ref64(att, True)
+        for r in range(seq):
+            m = al - seq + r + 1
+            assert (out[:, r, m:] == 0).all() and not np.signbit(out[:, r, m:]).any()  # exactly +0
+        # exp of a difference of magnitude <= ~16: a few ulp from the argument, then sum and product
+        assert (np.abs(out.astype(f64) - ref) <= 24 * eps * ref + 1e-300).all()
+        np.testing.assert_allclose(out.astype(f64).sum(axis=2), 1.0, atol=al * eps)
+    sq = oracle.fused_softmax(np.array([[[-7.0, 1.0], [2.0, 2.0]]], dtype), causal=True)
+    assert sq[0, 0].tolist() == [1.0, 0.0] and sq[0, 1].tolist() == [0.5, 0.5]
+    nomask = oracle.fused_softmax(np.array([[[1.0, 1.0, 1.0, 1.0]]], dtype), causal=False)
+    assert nomask[0, 0].tolist() == [0.25] * 4
+    # the scale is the rounded reciprocal of the sum, not a division: 1 / 3 rounds down in f32 and in f64, and
+    # 3 equal logits give exactly that rounded reciprocal
+    three = oracle.fused_softmax(np.array([[[0.5, 0.5, 0.5]]], dtype), causal=False)
+    assert three[0, 0, 0] == dtype(1) / dtype(3)
+    x = (rng.integers(-32, 32, (2, 4, 24)) / 8.0).astype(dtype)  # multiples of 1/8: + 2 is exact
+    assert np.array_equal(oracle.fused_softmax(x.copy(), causal=True), oracle.fused_softmax(x + dtype(2), causal=True))
+
+
 def test_softmax_strided_rows():
     rng = np.random.default_rng(3)
     big = (rng.standard_normal((2, 6, 48)) * 2).astype(f16)
