@@ -505,12 +505,13 @@ extern "C" int ophip_rearrange_plan(const ophip_rearrange_args *args, ptrdiff_t 
 }
 
 struct ophip_rearrange : OpBase {
-    hipFunction_t k32[5], k32_one[5], k64[5];  // chunk sizes 16, 8, 4, 2, 1; k32_one: one chunk per thread
+    hipFunction_t k32[5], k32_nt[5], k32_one[5], k64[5];  // chunk sizes 16, 8, 4, 2, 1; k32_one: one chunk per thread; k32_nt: non-temporal stores
     explicit ophip_rearrange(ophip_device *d) : OpBase(d) {
         static const int sizes[5] = {16, 8, 4, 2, 1};
         for (int i = 0; i < 5; ++i) {
             k32[i] = d->kernel("rearrange", ("rearrange_b" + std::to_string(sizes[i])).c_str());
             k32_one[i] = d->kernel("rearrange", ("rearrange1_b" + std::to_string(sizes[i])).c_str());
+            k32_nt[i] = d->kernel("rearrange", ("rearrange_nt_b" + std::to_string(sizes[i])).c_str());
             k64[i] = d->kernel("rearrange", ("rearrange64_b" + std::to_string(sizes[i])).c_str());
         }
     }
@@ -625,7 +626,8 @@ extern "C" int ophip_rearrange_launch(const ophip_rearrange *op, const ophip_rea
             // four chunks per thread, unless that leaves fewer than eight workgroups per CU: then one
             const unsigned cus = (unsigned)op->dev->props.multiProcessorCount;
             const bool one = p.total < (uint64_t)cus * 8 * 256 * 4;
-            launch(one ? op->k32_one[ci] : op->k32[ci], Dim3{ceil_div(p.total, one ? 256 : 256 * 4)}, Dim3{256}, 0,
+            const bool nt = p.total * B >= ((uint64_t)64 << 20);  // more than the caches hold
+            launch(one ? op->k32_one[ci] : nt ? op->k32_nt[ci] : op->k32[ci], Dim3{ceil_div(p.total, one ? 256 : 256 * 4)}, Dim3{256}, 0,
                    stream_of(qa), p);
         } else {
             if (cpu > 0xffffffffu) throw shape_not_support("rearrange unit too large");
@@ -639,12 +641,13 @@ extern "C" int ophip_rearrange_launch(const ophip_rearrange *op, const ophip_rea
 // Args::meta: swiglu/args.rs:31-50; launch checks: swiglu/cuda/mod.rs:53-98.
 
 struct ophip_swiglu : OpBase {
-    hipFunction_t f16_vec, f16_scalar, f32_scalar, f64_scalar;
+    hipFunction_t f16_vec, f16_vec_nt, f16_scalar, f32_scalar, f64_scalar;
     explicit ophip_swiglu(ophip_device *d) : OpBase(d) {
         f16_vec = d->kernel("swiglu", "swiglu_f16_vec");
         f16_scalar = d->kernel("swiglu", "swiglu_f16_scalar");
         f32_scalar = d->kernel("swiglu", "swiglu_f32_scalar");
         f64_scalar = d->kernel("swiglu", "swiglu_f64_scalar");
+        f16_vec_nt = d->kernel("swiglu", "swiglu_f16_vec_nt");
     }
 };
 
@@ -702,7 +705,8 @@ extern "C" int ophip_swiglu_launch(const ophip_swiglu *op, const ophip_swiglu_ar
         const size_t items = vec ? d / 8 : d;
         const unsigned gx = std::min<unsigned>(ceil_div(items, 256), 65535u);
         const unsigned gy = (unsigned)std::min<size_t>(n, 65535);
-        hipFunction_t fn = vec ? op->f16_vec : m.dt == OPHIP_DT_F16 ? op->f16_scalar : m.dt == OPHIP_DT_F32 ? op->f32_scalar : op->f64_scalar;
+        const bool big = n * d * (size_t)unit >= ((size_t)64 << 20);  // more than the caches hold
+        hipFunction_t fn = vec ? (big ? op->f16_vec_nt : op->f16_vec) : m.dt == OPHIP_DT_F16 ? op->f16_scalar : m.dt == OPHIP_DT_F32 ? op->f32_scalar : op->f64_scalar;
         if (!p.gate || !p.up) throw args_not_support("null base address");
         op->dev->make_current();
         launch(fn, Dim3{gx, gy}, Dim3{256}, 0, stream_of(qa), p);

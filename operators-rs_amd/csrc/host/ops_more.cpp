@@ -297,6 +297,7 @@ extern "C" int ophip_add_launch(const ophip_add *op, const ophip_add_args *args,
         if (total > 0x7fffffffu) throw shape_not_support("add: too many elements");
         p.total = (uint32_t)total;
         p.ndim = (uint32_t)s.dims.size();
+
         size_t items = 1;  // items per step of dimension i = product of the dimensions after it
         for (size_t i = s.dims.size(); i-- > 0;) {
             p.idx_div[i] = make_fastdiv((uint32_t)items);
@@ -305,7 +306,9 @@ extern "C" int ophip_add_launch(const ophip_add *op, const ophip_add_args *args,
             p.b_s[i] = s.dims[i].b;
             items *= s.dims[i].d;
         }
-        const std::string name = std::string("add_") + dt_tag(s.dt) + (vec ? "_vec" : "_scalar");
+        // (more output than the caches hold: the build that stores with the non-temporal hint)
+        const bool nt = vec && total * 16 >= ((size_t)64 << 20);
+        const std::string name = std::string("add_") + dt_tag(s.dt) + (vec ? (nt ? "_vec_nt" : "_vec") : "_scalar");
         const unsigned blocks = (unsigned)std::min<size_t>(ceil_div(total, 256), 1u << 20);
         if (!p.c || !p.a || !p.b) throw args_not_support("null base address");
         op->dev->make_current();

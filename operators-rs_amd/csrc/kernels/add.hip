@@ -27,28 +27,38 @@ __device__ __forceinline__ AddOffsets add_decode(const AddParams &p, uint32_t g)
     return o;
 }
 
-extern "C" __global__ void __launch_bounds__(256) add_f16_vec(AddParams p) {
+// NT: a sum larger than the caches (the host decides): stores with the non-temporal hint.  (Separate builds: a flag
+// in the parameters would make the compiler merge the two stores of an if / else and drop the hint.)
+template <bool NT>
+__device__ __forceinline__ void add_f16_vec_impl(const AddParams &p) {
     for (uint32_t g = blockIdx.x * blockDim.x + threadIdx.x; g < p.total; g += gridDim.x * blockDim.x) {
         const AddOffsets o = add_decode(p, g);
         Pack8 a, b, c;
-        a.u = ld128(reinterpret_cast<const char *>(p.a) + o.a);
-        b.u = ld128(reinterpret_cast<const char *>(p.b) + o.b);
+        a.u = ld128_nt(reinterpret_cast<const char *>(p.a) + o.a);
+        b.u = ld128_nt(reinterpret_cast<const char *>(p.b) + o.b);
 #pragma unroll
         for (int i = 0; i < 8; ++i) c.e[i] = f2h(h2f(a.e[i]) + h2f(b.e[i]));
-        st128(reinterpret_cast<char *>(p.c) + o.c, c.u);
+        if constexpr (NT) st128_nt(reinterpret_cast<char *>(p.c) + o.c, c.u);
+        else st128(reinterpret_cast<char *>(p.c) + o.c, c.u);
     }
 }
+extern "C" __global__ void __launch_bounds__(256) add_f16_vec(AddParams p) { add_f16_vec_impl<false>(p); }
+extern "C" __global__ void __launch_bounds__(256) add_f16_vec_nt(AddParams p) { add_f16_vec_impl<true>(p); }
 
-extern "C" __global__ void __launch_bounds__(256) add_f32_vec(AddParams p) {
+template <bool NT>
+__device__ __forceinline__ void add_f32_vec_impl(const AddParams &p) {
     for (uint32_t g = blockIdx.x * blockDim.x + threadIdx.x; g < p.total; g += gridDim.x * blockDim.x) {
         const AddOffsets o = add_decode(p, g);
         Pack4f a, b, c;
-        a.u = ld128(reinterpret_cast<const char *>(p.a) + o.a);
-        b.u = ld128(reinterpret_cast<const char *>(p.b) + o.b);
+        a.u = ld128_nt(reinterpret_cast<const char *>(p.a) + o.a);
+        b.u = ld128_nt(reinterpret_cast<const char *>(p.b) + o.b);
         c.f = a.f + b.f;
-        st128(reinterpret_cast<char *>(p.c) + o.c, c.u);
+        if constexpr (NT) st128_nt(reinterpret_cast<char *>(p.c) + o.c, c.u);
+        else st128(reinterpret_cast<char *>(p.c) + o.c, c.u);
     }
 }
+extern "C" __global__ void __launch_bounds__(256) add_f32_vec(AddParams p) { add_f32_vec_impl<false>(p); }
+extern "C" __global__ void __launch_bounds__(256) add_f32_vec_nt(AddParams p) { add_f32_vec_impl<true>(p); }
 
 template <typename T>
 __device__ __forceinline__ void add_scalar(const AddParams &p) {

@@ -25,7 +25,7 @@ extern "C" __global__ void __launch_bounds__(256) add_rows_f16_vec(AddRowsParams
         if (!add_rows_locate(p, bm, dst, src)) continue;
         for (uint32_t v = blockIdx.x * blockDim.x + threadIdx.x; v < nvec; v += gridDim.x * blockDim.x) {
             Pack8 d, s;
-            d.u = ld128(dst + (size_t)v * 16);
+            d.u = ld128_nt(dst + (size_t)v * 16);
             s.u = ld128(src + (size_t)v * 16);
 #pragma unroll
             for (int i = 0; i < 8; ++i) d.e[i] = f2h(h2f(d.e[i]) + h2f(s.e[i]));

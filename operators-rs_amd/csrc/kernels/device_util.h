@@ -19,6 +19,9 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ u32x4 ld128(const void *p) { return *reinterpret_cast<const u32x4 *>(p); }
 __device__ __forceinline__ void st128(void *p, u32x4 v) { *reinterpret_cast<u32x4 *>(p) = v; }
+// the same with the non-temporal hint: for output that the kernel writes once and that is too large to be found in a
+// cache by whoever reads it next
+__device__ __forceinline__ void st128_nt(void *p, u32x4 v) { __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(p)); }
 // Streaming load for data touched once per launch (GEMM weights): the non-temporal hint keeps
 // such lines from displacing reusable ones in L2 and the Infinity Cache, and raises read-only
 // streaming bandwidth (5.8 -> 6.6 TB/s measured on 1 GiB).

@@ -43,7 +43,7 @@ __device__ __forceinline__ void softmax_reg(const SoftmaxParams &p) {
             Pack8 v;
             v.u = u32x4{0, 0, 0, 0};
             if (col0 + 8 <= p.att_len) {
-                if (col0 < kept) v.u = ld128(row + col0);
+                if (col0 < kept) v.u = ld128_nt(row + col0);
             } else {
 #pragma unroll
                 for (int e = 0; e < 7; ++e)
@@ -135,7 +135,7 @@ __device__ __forceinline__ void softmax_rows4(const SoftmaxParams &p) {
         for (int q = 0; q < PT; ++q) {
             const int col0 = (int)(lane + q * WAVE) * 8;
             v[i][q].u = u32x4{0, 0, 0, 0};
-            if (col0 < kept[i]) v[i][q].u = ld128(row[i] + col0);
+            if (col0 < kept[i]) v[i][q].u = ld128_nt(row[i] + col0);
         }
     // Masked columns become -inf once, here; from then on they take care of themselves: they never win the maximum,
     // their exponential is 0, they add nothing to the sum and 0 / sum is the 0 the mask asks for.

@@ -75,7 +75,7 @@ __device__ __forceinline__ void layer_norm_vec(const LayerNormParams &p) {
     for (int c = 0; c < CACHE; ++c) {
         const uint32_t v = lane + c * G;
         if (v < nvec) {
-            cache[c].v.u = ld128(xr + (size_t)v * 16);
+            cache[c].v.u = ld128_nt(xr + (size_t)v * 16);
 #pragma unroll
             for (int i = 0; i < N; ++i) {
                 const float f = cache[c].get(i);
@@ -86,7 +86,7 @@ __device__ __forceinline__ void layer_norm_vec(const LayerNormParams &p) {
     }
     for (uint32_t v = lane + CACHE * G; v < nvec; v += G) {
         Vec<TA> t;
-        t.v.u = ld128(xr + (size_t)v * 16);
+        t.v.u = ld128_nt(xr + (size_t)v * 16);
 #pragma unroll
         for (int i = 0; i < N; ++i) {
             const float f = t.get(i);
@@ -115,7 +115,7 @@ __device__ __forceinline__ void layer_norm_vec(const LayerNormParams &p) {
     }
     for (uint32_t v = lane + CACHE * G; v < nvec; v += G) {
         Vec<TA> t;
-        t.v.u = ld128(xr + (size_t)v * 16);
+        t.v.u = ld128_nt(xr + (size_t)v * 16);
         emit(t, v);
     }
 }
@@ -169,7 +169,7 @@ __device__ __forceinline__ void layer_norm_rows(const LayerNormParams &p) {
 #pragma unroll
         for (int c = 0; c < CACHE; ++c) {
             const uint32_t v = lane + c * WAVE;
-            if (v < nvec) cur[c].u = ld128(xr + (size_t)v * 16);
+            if (v < nvec) cur[c].u = ld128_nt(xr + (size_t)v * 16);
         }
     }
     for (; row < p.n; row += waves) {
@@ -179,7 +179,7 @@ __device__ __forceinline__ void layer_norm_rows(const LayerNormParams &p) {
 #pragma unroll
             for (int c = 0; c < CACHE; ++c) {
                 const uint32_t v = lane + c * WAVE;
-                if (v < nvec) nxt[c].u = ld128(xn + (size_t)v * 16);
+                if (v < nvec) nxt[c].u = ld128_nt(xn + (size_t)v * 16);
             }
         }
         float s1 = 0.f, s2 = 0.f;
@@ -208,7 +208,7 @@ __device__ __forceinline__ void layer_norm_rows(const LayerNormParams &p) {
 #pragma unroll
                 for (int i = 0; i < 8; ++i)
                     o.e[i] = f2h(__builtin_fmaf(h2f(cur[c].e[i]) - e, s_scale[v * 8 + i] * k, s_bias[v * 8 + i]));
-                st128(yr + (size_t)v * 16, o.u);
+                st128_nt(yr + (size_t)v * 16, o.u);
             }
         }
 #pragma unroll

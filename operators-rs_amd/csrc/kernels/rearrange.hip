@@ -27,7 +27,10 @@ struct Chunk<1> { typedef uint8_t T; };
 
 // RE_ITEMS chunks per thread, loads issued before stores: 4 for large copies; 1 for mid-size ones, which would
 // otherwise leave the machine with one workgroup per CU or less (8 MB: 256 workgroups at 4 chunks per thread).
-template <int B, int RE_ITEMS>
+// NT: a copy larger than the caches (the host decides): what it writes is not found in them by the next reader
+// anyway, and the non-temporal hint on the stores is worth 3 % on such a copy.  (A flag in the parameters does
+// not do: the compiler merges the two stores of an if / else and drops the hint.)
+template <int B, int RE_ITEMS, bool NT = false>
 __device__ __forceinline__ void rearrange32(const RearrangeParams &p) {
     typedef typename Chunk<B>::T T;
     const uint32_t total = (uint32_t)p.total;
@@ -51,12 +54,15 @@ __device__ __forceinline__ void rearrange32(const RearrangeParams &p) {
                 s += (int64_t)k * p.src_s[q];
             }
             doff[it] = d;
-            val[it] = *reinterpret_cast<const T *>(reinterpret_cast<const char *>(p.src) + s);
+            val[it] = __builtin_nontemporal_load(reinterpret_cast<const T *>(reinterpret_cast<const char *>(p.src) + s));
         }
     }
 #pragma unroll
     for (int it = 0; it < RE_ITEMS; ++it)
-        if (ok[it]) *reinterpret_cast<T *>(reinterpret_cast<char *>(p.dst) + doff[it]) = val[it];
+        if (ok[it]) {
+            if constexpr (NT) __builtin_nontemporal_store(val[it], reinterpret_cast<T *>(reinterpret_cast<char *>(p.dst) + doff[it]));
+            else *reinterpret_cast<T *>(reinterpret_cast<char *>(p.dst) + doff[it]) = val[it];
+        }
 }
 
 // 64-bit indices: more than 2^32 chunks or an index stride beyond 32 bits.
@@ -83,6 +89,9 @@ __device__ __forceinline__ void rearrange64(const RearrangeParams &p) {
 #define REARRANGE(B)                                                                             \
     extern "C" __global__ void __launch_bounds__(256) rearrange_b##B(RearrangeParams p) {       \
         rearrange32<B, 4>(p);                                                                    \
+    }                                                                                            \
+    extern "C" __global__ void __launch_bounds__(256) rearrange_nt_b##B(RearrangeParams p) {    \
+        rearrange32<B, 4, true>(p);                                                              \
     }                                                                                            \
     extern "C" __global__ void __launch_bounds__(256) rearrange1_b##B(RearrangeParams p) {      \
         rearrange32<B, 1>(p);                                                                    \

@@ -211,7 +211,7 @@ __device__ __forceinline__ void rms_norm_rows(const RmsNormParams &p) {
 #pragma unroll
         for (int c = 0; c < CACHE; ++c) {
             const uint32_t v = lane + c * WAVE;
-            if (v < nvec) cur[c].u = ld128(xr + (size_t)v * 16);
+            if (v < nvec) cur[c].u = ld128_nt(xr + (size_t)v * 16);
         }
     }
     for (; row < p.n; row += waves) {
@@ -221,7 +221,7 @@ __device__ __forceinline__ void rms_norm_rows(const RmsNormParams &p) {
 #pragma unroll
             for (int c = 0; c < CACHE; ++c) {
                 const uint32_t v = lane + c * WAVE;
-                if (v < nvec) nxt[c].u = ld128(xn + (size_t)v * 16);
+                if (v < nvec) nxt[c].u = ld128_nt(xn + (size_t)v * 16);
             }
         }
         float ss = 0.f;
@@ -246,7 +246,7 @@ __device__ __forceinline__ void rms_norm_rows(const RmsNormParams &p) {
                 Pack8 o;
 #pragma unroll
                 for (int i = 0; i < 8; ++i) o.e[i] = f2h((k * w[c].get(i)) * h2f(cur[c].e[i]));
-                st128(yr + (size_t)v * 16, o.u);
+                st128_nt(yr + (size_t)v * 16, o.u);
             }
         }
 #pragma unroll
