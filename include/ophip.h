@@ -158,9 +158,12 @@ OPHIP_API int ophip_event_elapsed_ms(ophip_device *dev, ophip_event start, ophip
 OPHIP_API int ophip_time_next_launch(ophip_device *dev, ophip_stream stream, ophip_event start, ophip_event stop);
 
 /* Measurement aid, no counterpart in the reference: one launch of a probe kernel, for ceilings measured on the machine
- * at hand.  kind = "read", "read_nt" (non-temporal loads), "write", "copy": `blocks` workgroups of 256 threads stream
+ * at hand.  kind = "read", "read_nt" (non-temporal loads), "read16", "read_nt16" (sixteen instead of four 16-byte loads
+ * in flight per thread), "write", "copy": `blocks` workgroups of 256 threads stream
  * `bytes` (a multiple of 16) from `src` and / or into `dst` (16-byte aligned; a read-only probe writes at most 16 bytes
- * to dst).  kind = "mfma": `blocks` workgroups run `iters` trips of 128 v_mfma_f32_32x32x16_f16 per wave on operands made
+ * to dst).  kind = "strips": the weight-streaming mat_mul's access pattern alone; `src` is a row-major f16 matrix of `seed`
+ * rows and `iters` columns (a multiple of 8) inside `bytes`, read in 128-column strips by one workgroup per strip and
+ * per each of `blocks` equal row ranges (`seed` a multiple of 32 * blocks).  kind = "mfma": `blocks` workgroups run `iters` trips of 128 v_mfma_f32_32x32x16_f16 per wave on operands made
  * in registers from `seed` (0: all-zero operands) = blocks * 4 * iters * 128 * 32768 flop; dst needs blocks * 1024 bytes. */
 OPHIP_API int ophip_probe(ophip_device *dev, const char *kind, void *dst, const void *src, size_t bytes,
                           unsigned iters, unsigned seed, unsigned blocks, ophip_stream stream);
