@@ -596,7 +596,28 @@ def standalone_ops(ophip, gpu, stream, rng, reps, ceiling=None):
     ws = gpu.malloc(max(akv.scheme(a, 1 << 30), 1))
     us = time_launches(gpu, stream, lambda: akv.launch(a, ws, stream), reps)
     add("attention_kv_cached", "nh32 seq16 pos2032 dh128", 2 * NH * KV * DH * 2 + 8 * nt * D * 2, us,
-        note="composite of 7 launches; bytes = both caches read once + q, k, v, o and the appended rows")
+        note="one pass over the caches + the merge of its chunks (the crate's composite: 7 launches); bytes = both caches "
+             "read once + q, k, v, o and the appended rows; the same two caches every launch (34.6 MB: they stay in the 256 MiB cache)")
+    # the same with ten sets of caches in rotation (346 MB), as the layers of a model present them: every launch reads HBM
+    sets = [(kc, vc)] + [(gpu.malloc(NH * KV * DH * 2), gpu.malloc(NH * KV * DH * 2)) for _ in range(9)]
+    for kb_, vb_ in sets[1:]:
+        for dst_, src_ in ((kb_, kc), (vb_, vc)):
+            ophip._check(ophip.lib().ophip_memcpy_d2d(gpu.handle, ctypes.c_void_p(dst_.ptr), ctypes.c_void_p(src_.ptr),
+                                                      ctypes.c_size_t(NH * KV * DH * 2), stream.handle))
+    stream.synchronize()
+    rot = [o.AttnKVCachedArgs(head_major(3 * D * 2), qkv.ptr, head_major(3 * D * 2), qkv.ptr + D * 2,
+                              head_major(3 * D * 2), qkv.ptr + 2 * D * 2, head_major(D * 2), obuf,
+                              c(NH, KV, DH), kb_, c(NH, KV, DH), vb_, o.AttnMask.CAUSAL, pos) for kb_, vb_ in sets]
+    turn = [0]
+
+    def launch_rotating():
+        akv.launch(rot[turn[0] % len(rot)], ws, stream)
+        turn[0] += 1
+    us = time_launches(gpu, stream, launch_rotating, max(reps, 2 * len(rot)), warm=len(rot))
+    add("attention_kv_cached", "nh32 seq16 pos2032 dh128, ten cache sets in rotation", 2 * NH * KV * DH * 2 + 8 * nt * D * 2, us,
+        note="as above on caches that come from HBM")
+    for kb_, vb_ in sets[1:]:
+        kb_.free(); vb_.free()
     # the dominant decode GEMM (gate/up) on its own, weights stored [K, N] and [N, K]: two copies of the
     # weights alternate so that no launch finds them in the Infinity Cache
     mm = o.MatMul(gpu)
