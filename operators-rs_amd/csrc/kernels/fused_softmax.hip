@@ -108,10 +108,23 @@ __device__ __forceinline__ void softmax_reg(const SoftmaxParams &p) {
 template <int PT>
 __device__ __forceinline__ void softmax_rows4(const SoftmaxParams &p) {
     constexpr int ROWS = 4;
+    // keep[n]: the 16 bytes that keep the first n of a vector's 8 columns.  What a row masks becomes -inf with one
+    // bit-field insert per register, before anything is converted; from then on masked columns take care of
+    // themselves: they never win the maximum, their exponential is 0, they add nothing to the sum, and 0 / sum is
+    // the +0 the mask asks for.
+    __shared__ u32x4 keep[9];
+    if (threadIdx.x < 9) {
+        const uint32_t n = threadIdx.x;
+        u32x4 m;
+#pragma unroll
+        for (uint32_t w = 0; w < 4; ++w) m[w] = n >= 2 * w + 2 ? 0xffffffffu : n == 2 * w + 1 ? 0x0000ffffu : 0u;
+        keep[n] = m;
+    }
+    __syncthreads();
     const uint32_t lane = threadIdx.x % WAVE;
     const uint32_t per_head = (p.seq + ROWS - 1) / ROWS;  // waves per head
     const uint32_t w = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
-    if (w >= p.nh * per_head) return;  // (no barrier in this kernel)
+    if (w >= p.nh * per_head) return;  // (no barrier below this line)
     const uint32_t h = w / per_head, j = w - h * per_head;
     const bool paired = p.seq % ROWS == 0;
 
@@ -127,7 +140,7 @@ __device__ __forceinline__ void softmax_rows4(const SoftmaxParams &p) {
         row[i] = reinterpret_cast<f16 *>(reinterpret_cast<char *>(p.att) + (int64_t)h * p.sh + (int64_t)r * p.ss);
     }
     // att_len is a multiple of 8 (the host sends other lengths to the general kernel): a lane's vector is inside the
-    // row or outside it, and what a row keeps of it is the first `n` of its 8 columns, n = kept - col0.
+    // row or outside it, and what a row keeps of it is the first n of its 8 columns, n = kept - col0.
     Pack8 v[ROWS][PT];
 #pragma unroll
     for (int i = 0; i < ROWS; ++i)
@@ -137,25 +150,26 @@ __device__ __forceinline__ void softmax_rows4(const SoftmaxParams &p) {
             v[i][q].u = u32x4{0, 0, 0, 0};
             if (col0 < kept[i]) v[i][q].u = ld128_nt(row[i] + col0);
         }
-    // Masked columns become -inf once, here; from then on they take care of themselves: they never win the maximum,
-    // their exponential is 0, they add nothing to the sum and 0 / sum is the 0 the mask asks for.
-    float x[ROWS][PT][8];
+    constexpr uint32_t NEG_INF2 = 0xfc00fc00u;  // two f16 -inf
     float mx[ROWS];
 #pragma unroll
     for (int i = 0; i < ROWS; ++i) {
-        mx[i] = -INFINITY;
+        f16x2 m2 = __builtin_bit_cast(f16x2, NEG_INF2);
 #pragma unroll
         for (int q = 0; q < PT; ++q) {
-            const int n = kept[i] - (int)(lane + q * WAVE) * 8;
+            const int n = min(max(kept[i] - (int)(lane + q * WAVE) * 8, 0), 8);
+            const u32x4 m = keep[n];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                x[i][q][e] = e < n ? h2f(v[i][q].e[e]) : -INFINITY;
-                mx[i] = fmaxf(mx[i], x[i][q][e]);
+            for (int c = 0; c < 4; ++c) {
+                v[i][q].u[c] = (v[i][q].u[c] & m[c]) | (NEG_INF2 & ~m[c]);
+                m2 = __builtin_elementwise_max(m2, __builtin_bit_cast(f16x2, v[i][q].u[c]));  // exact: the maximum is one of them
             }
         }
+        mx[i] = fmaxf(h2f(m2[0]), h2f(m2[1]));
     }
 #pragma unroll
     for (int i = 0; i < ROWS; ++i) mx[i] = wave_max_dpp(mx[i]);
+    float x[ROWS][PT][8];
     float sum[ROWS];
 #pragma unroll
     for (int i = 0; i < ROWS; ++i) {
@@ -166,7 +180,7 @@ __device__ __forceinline__ void softmax_rows4(const SoftmaxParams &p) {
         for (int q = 0; q < PT; ++q)
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const float ex = __builtin_amdgcn_exp2f(__builtin_fmaf(x[i][q][e], LOG2E, shift));
+                const float ex = __builtin_amdgcn_exp2f(__builtin_fmaf(h2f(v[i][q].e[e]), LOG2E, shift));
                 sum[i] += ex;
                 x[i][q][e] = h2f(f2h(ex));  // the reference stores f16(e) and re-reads it
             }
