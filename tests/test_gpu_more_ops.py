@@ -163,7 +163,7 @@ def run_add(gpu, stream, c_view, c_buf, a_view, a_buf, b_view, b_buf):
 
 
 @pytest.mark.parametrize("dtype", [f16, f32])
-@pytest.mark.parametrize("shape", [(1, 768), (16, 4096), (3, 5, 7), (1000, 33)])
+@pytest.mark.parametrize("shape", [(1, 768), (16, 4096), (3, 5, 7), (1000, 33), (8200, 4096)])  # the last: a sum of more than 64 MiB
 def test_add_contiguous(gpu, stream, dtype, shape):
     rng = np.random.default_rng(sum(shape))
     a, b = (rng.standard_normal(shape).astype(f32).astype(dtype) for _ in range(2))
