@@ -13,7 +13,9 @@ using namespace ophip;
 
 namespace {
 
-const char *dt_tag(uint64_t dt) { return dt == OPHIP_DT_F16 ? "f16" : dt == OPHIP_DT_F32 ? "f32" : dt == OPHIP_DT_F64 ? "f64" : "?"; }
+const char *dt_tag(uint64_t dt) {
+    return dt == OPHIP_DT_F16 ? "f16" : dt == OPHIP_DT_BF16 ? "bf16" : dt == OPHIP_DT_F32 ? "f32" : dt == OPHIP_DT_F64 ? "f64" : "?";
+}
 
 }  // namespace
 
@@ -39,10 +41,14 @@ static RmsNormMeta rms_norm_meta(const ophip_rms_norm_args &a) {
 }
 
 static void rms_norm_check_types(uint64_t dt_a, uint64_t dt_w) {
-    // the pairs of the CPU backend (rms_norm/common_cpu/mod.rs:84-90); anything else is `todo!()` there
+    // the pairs of the CPU backend (rms_norm/common_cpu/mod.rs:84-90; anything else is `todo!()` there), and bf16
+    // activations with bf16 or f32 weights, which the CUDA backend compiles a kernel for like for any other pair of
+    // named types (rms_norm/cuda/mod.rs:146-147)
     const bool ok = (dt_a == OPHIP_DT_F16 && (dt_w == OPHIP_DT_F16 || dt_w == OPHIP_DT_F32)) ||
+                    (dt_a == OPHIP_DT_BF16 && (dt_w == OPHIP_DT_BF16 || dt_w == OPHIP_DT_F32)) ||
                     (dt_a == OPHIP_DT_F32 && dt_w == OPHIP_DT_F32) || (dt_a == OPHIP_DT_F64 && dt_w == OPHIP_DT_F64);
-    if (!ok) throw type_not_support("rms_norm supports (a, w) in {(f16, f16), (f16, f32), (f32, f32), (f64, f64)}");
+    if (!ok)
+        throw type_not_support("rms_norm supports (a, w) in {(f16, f16), (f16, f32), (bf16, bf16), (bf16, f32), (f32, f32), (f64, f64)}");
 }
 
 struct RmsKey {
@@ -55,7 +61,7 @@ struct RmsKeyHash {
 };
 struct RmsScheme {  // kernels for one (dt_a, dt_w, d): a vector variant per group width plus the scalar one
     hipFunction_t g64, g256, g1024, scalar;
-    hipFunction_t rows;  // f16 activations only: one wave per row over many rows
+    hipFunction_t rows;  // f16 and bf16 activations only: one wave per row over many rows
 };
 
 struct ophip_rms_norm : OpBase {
@@ -74,7 +80,7 @@ struct ophip_rms_norm : OpBase {
             s.g256 = dev->kernel("rms_norm", (base + "_g256").c_str());
             s.g1024 = dev->kernel("rms_norm", (base + "_g1024").c_str());
             s.scalar = dev->kernel("rms_norm", (base + "_scalar").c_str());
-            s.rows = key.dt_a == OPHIP_DT_F16 ? dev->kernel("rms_norm", (base + "_rows").c_str()) : nullptr;
+            s.rows = key.dt_a == OPHIP_DT_F16 || key.dt_a == OPHIP_DT_BF16 ? dev->kernel("rms_norm", (base + "_rows").c_str()) : nullptr;
             return s;
         });
     }
@@ -141,8 +147,8 @@ extern "C" int ophip_rms_norm_launch(const ophip_rms_norm *op, const ophip_rms_n
         const unsigned cus = (unsigned)op->dev->props.multiProcessorCount;
         if (G == 64 && s.rows && n >= (size_t)cus * 64) {
             // enough rows for several per wave: as many waves as stay resident (registers allow
-            // 16 per CU with f16 weights, 12 with f32), each streaming rows with w held in registers
-            const unsigned per_cu = m.dt_w == OPHIP_DT_F16 ? 4 : 3;
+            // 16 per CU with two-byte weights, 12 with f32), each streaming rows with w held in registers
+            const unsigned per_cu = m.dt_w == OPHIP_DT_F32 ? 3 : 4;
             launch(s.rows, Dim3{cus * per_cu}, Dim3{256}, 0, stream_of(qa), p);
             return;
         }

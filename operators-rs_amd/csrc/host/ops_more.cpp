@@ -11,7 +11,9 @@ using namespace ophip;
 
 namespace {
 
-const char *dt_tag(uint64_t dt) { return dt == OPHIP_DT_F16 ? "f16" : dt == OPHIP_DT_F32 ? "f32" : dt == OPHIP_DT_F64 ? "f64" : "?"; }
+const char *dt_tag(uint64_t dt) {
+    return dt == OPHIP_DT_F16 ? "f16" : dt == OPHIP_DT_BF16 ? "bf16" : dt == OPHIP_DT_F32 ? "f32" : dt == OPHIP_DT_F64 ? "f64" : "?";
+}
 
 }  // namespace
 
@@ -69,9 +71,13 @@ extern "C" int ophip_layer_norm_launch(const ophip_layer_norm *op, const ophip_l
         const ptrdiff_t nsx = static_of(args->x_layout.strides[0]), dsx = static_of(args->x_layout.strides[1]);
         const ptrdiff_t dss = static_of(args->scale_layout.strides[0]), dsb = static_of(args->bias_layout.strides[0]);
         const bool f64 = m.dt_a == OPHIP_DT_F64 && m.dt_w == OPHIP_DT_F64;
+        // the CPU backend's pairs (layer_norm/common_cpu/mod.rs:94-97), and bf16 rows with bf16 or f32 parameters, which
+        // the CUDA backend compiles a kernel for like for any other named types (layer_norm/cuda/mod.rs:158-159)
         const bool ok = (m.dt_a == OPHIP_DT_F16 && (m.dt_w == OPHIP_DT_F16 || m.dt_w == OPHIP_DT_F32)) ||
+                        (m.dt_a == OPHIP_DT_BF16 && (m.dt_w == OPHIP_DT_BF16 || m.dt_w == OPHIP_DT_F32)) ||
                         (m.dt_a == OPHIP_DT_F32 && m.dt_w == OPHIP_DT_F32) || f64;
-        if (!ok) throw type_not_support("layer_norm supports (scale, x) in (f16,f16), (f32,f16), (f32,f32), (f64,f64)");
+        if (!ok)
+            throw type_not_support("layer_norm supports (scale, x) in (f16,f16), (f32,f16), (bf16,bf16), (f32,bf16), (f32,f32), (f64,f64)");
         const ptrdiff_t unit = (ptrdiff_t)ophip_dtype_nbytes(m.dt_a), wunit = (ptrdiff_t)ophip_dtype_nbytes(m.dt_w);
         if (dsy != unit || dsx != unit || dss != wunit || dsb != wunit)
             throw strides_not_support("layer_norm needs contiguous inner dimensions");
@@ -106,7 +112,7 @@ extern "C" int ophip_layer_norm_launch(const ophip_layer_norm *op, const ophip_l
         unsigned G = nvec <= 64 * 8 ? 64 : nvec <= 256 * 8 ? 256 : 1024;
         while (G < 1024 && n * (G / 64) < 2048 && nvec >= 4 * (size_t)G) G *= 4;
         const unsigned cus = (unsigned)op->dev->props.multiProcessorCount;
-        if (G == 64 && m.dt_a == OPHIP_DT_F16 && d <= 4096 && n >= (size_t)cus * 64 &&
+        if (G == 64 && unit == 2 && d <= 4096 && n >= (size_t)cus * 64 &&
             n * d * (size_t)unit >= ((size_t)32 << 20)) {
             // many rows and more bytes than the L2s hold: persistent workgroups (four per CU: 32 KiB
             // of LDS each for scale and bias) whose waves stream rows
@@ -269,7 +275,9 @@ extern "C" int ophip_add_launch(const ophip_add *op, const ophip_add_args *args,
                                 const ophip_queue_alloc *qa) {
     return guard([&] {
         AddScheme s = add_scheme(*args);
-        if (s.dt != OPHIP_DT_F16 && s.dt != OPHIP_DT_F32 && s.dt != OPHIP_DT_F64) throw type_not_support("add supports f16, f32 and f64");
+        // (bf16: no CPU kernel in the reference, but its CUDA backend adds any named type, add/cuda/mod.rs:105-123)
+        if (s.dt != OPHIP_DT_F16 && s.dt != OPHIP_DT_BF16 && s.dt != OPHIP_DT_F32 && s.dt != OPHIP_DT_F64)
+            throw type_not_support("add supports f16, bf16, f32 and f64");
         if (s.dims.size() > OPHIP_REARRANGE_MAXD)
             throw rank_not_support("add supports at most " + std::to_string(OPHIP_REARRANGE_MAXD) +
                                    " non-mergeable dimensions");
@@ -376,7 +384,9 @@ extern "C" int ophip_add_rows_launch(const ophip_add_rows *op, const ophip_add_r
                         nsd = static_of(args->dst_layout.strides[2]);
         const ptrdiff_t bsi = static_of(args->idx_layout.strides[0]), msi = static_of(args->idx_layout.strides[1]);
         const ptrdiff_t kss = static_of(args->src_layout.strides[0]), nss = static_of(args->src_layout.strides[1]);
-        if (r.dt != OPHIP_DT_F16 && r.dt != OPHIP_DT_F32 && r.dt != OPHIP_DT_F64) throw type_not_support("add_rows supports f16, f32 and f64");
+        // (bf16: no CPU kernel in the reference, but its CUDA backend compiles one for any named type, add_rows/cuda/mod.rs:135-163)
+        if (r.dt != OPHIP_DT_F16 && r.dt != OPHIP_DT_BF16 && r.dt != OPHIP_DT_F32 && r.dt != OPHIP_DT_F64)
+            throw type_not_support("add_rows supports f16, bf16, f32 and f64");
         if (r.dt_idx != OPHIP_DT_U32 && r.dt_idx != OPHIP_DT_U64) throw type_not_support("idx must be u32 or u64");
         const ptrdiff_t unit = (ptrdiff_t)ophip_dtype_nbytes(r.dt), iunit = (ptrdiff_t)ophip_dtype_nbytes(r.dt_idx);
         for (ptrdiff_t st : {bsd, msd, nsd, kss, nss})
@@ -402,7 +412,7 @@ extern "C" int ophip_add_rows_launch(const ophip_add_rows *op, const ophip_add_r
         p.idx_is_u64 = r.dt_idx == OPHIP_DT_U64;
         q.nsd = nsd;
         q.nss = nss;
-        const bool vec = r.dt == OPHIP_DT_F16 && nsd == unit && nss == unit && n % 8 == 0 && aligned16(p.dst) &&
+        const bool vec = unit == 2 && nsd == unit && nss == unit && n % 8 == 0 && aligned16(p.dst) &&
                          aligned16(p.src) && mult16(bsd) && mult16(msd) && mult16(kss);
         const size_t items = vec ? n / 8 : n;
         const unsigned gx = std::min<unsigned>(ceil_div(items, 256), 65535u);
@@ -410,10 +420,11 @@ extern "C" int ophip_add_rows_launch(const ophip_add_rows *op, const ophip_add_r
         if (!p.dst || !p.src || !p.idx) throw args_not_support("null base address");
         op->dev->make_current();
         if (vec) {
-            launch(op->dev->kernel("add_rows", "add_rows_f16_vec"), Dim3{gx, gy}, Dim3{256}, 0, stream_of(qa), p);
+            launch(op->dev->kernel("add_rows", r.dt == OPHIP_DT_F16 ? "add_rows_f16_vec" : "add_rows_bf16_vec"), Dim3{gx, gy}, Dim3{256}, 0,
+               stream_of(qa), p);
         } else {
-            const char *name = r.dt == OPHIP_DT_F16 ? "add_rows_f16_scalar" : r.dt == OPHIP_DT_F32 ? "add_rows_f32_scalar" : "add_rows_f64_scalar";
-            launch(op->dev->kernel("add_rows", name), Dim3{gx, gy}, Dim3{256}, 0, stream_of(qa), q);
+            const std::string name = std::string("add_rows_") + dt_tag(r.dt) + "_scalar";
+            launch(op->dev->kernel("add_rows", name.c_str()), Dim3{gx, gy}, Dim3{256}, 0, stream_of(qa), q);
         }
     });
 }

@@ -4,7 +4,7 @@
 // items in the innermost one: single elements, or 16-byte vectors when that dimension is
 // contiguous in all three tensors.  Item g is decoded into per-dimension indices with
 // multiply-high divisions; dimensions are ordered by descending c stride, so consecutive
-// threads write ascending addresses.  f16 sums are formed in f32 and rounded once, as
+// threads write ascending addresses.  f16 (and bf16) sums are formed in f32 and rounded once, as
 // half's `f16 + f16` does.
 #include <type_traits>
 
@@ -29,21 +29,24 @@ __device__ __forceinline__ AddOffsets add_decode(const AddParams &p, uint32_t g)
 
 // NT: a sum larger than the caches (the host decides): stores with the non-temporal hint.  (Separate builds: a flag
 // in the parameters would make the compiler merge the two stores of an if / else and drop the hint.)
-template <bool NT>
-__device__ __forceinline__ void add_f16_vec_impl(const AddParams &p) {
+template <typename T, bool NT>
+__device__ __forceinline__ void add_h_vec_impl(const AddParams &p) {  // T: f16 or bf16
     for (uint32_t g = blockIdx.x * blockDim.x + threadIdx.x; g < p.total; g += gridDim.x * blockDim.x) {
         const AddOffsets o = add_decode(p, g);
-        Pack8 a, b, c;
+        PackOf<T> a, b, c;
         a.u = ld128_nt(reinterpret_cast<const char *>(p.a) + o.a);
         b.u = ld128_nt(reinterpret_cast<const char *>(p.b) + o.b);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) c.e[i] = f2h(h2f(a.e[i]) + h2f(b.e[i]));
+        for (int i = 0; i < 8; ++i) c.e[i] = (T)((float)a.e[i] + (float)b.e[i]);
         if constexpr (NT) st128_nt(reinterpret_cast<char *>(p.c) + o.c, c.u);
         else st128(reinterpret_cast<char *>(p.c) + o.c, c.u);
     }
 }
-extern "C" __global__ void __launch_bounds__(256) add_f16_vec(AddParams p) { add_f16_vec_impl<false>(p); }
-extern "C" __global__ void __launch_bounds__(256) add_f16_vec_nt(AddParams p) { add_f16_vec_impl<true>(p); }
+extern "C" __global__ void __launch_bounds__(256) add_f16_vec(AddParams p) { add_h_vec_impl<f16, false>(p); }
+extern "C" __global__ void __launch_bounds__(256) add_f16_vec_nt(AddParams p) { add_h_vec_impl<f16, true>(p); }
+// bf16: the reference's CUDA backend adds any named type (add/cuda/mod.rs:105-123); its CPU backend has no bf16
+extern "C" __global__ void __launch_bounds__(256) add_bf16_vec(AddParams p) { add_h_vec_impl<bf16, false>(p); }
+extern "C" __global__ void __launch_bounds__(256) add_bf16_vec_nt(AddParams p) { add_h_vec_impl<bf16, true>(p); }
 
 template <bool NT>
 __device__ __forceinline__ void add_f32_vec_impl(const AddParams &p) {
@@ -72,5 +75,6 @@ __device__ __forceinline__ void add_scalar(const AddParams &p) {
 }
 
 extern "C" __global__ void __launch_bounds__(256) add_f16_scalar(AddParams p) { add_scalar<f16>(p); }
+extern "C" __global__ void __launch_bounds__(256) add_bf16_scalar(AddParams p) { add_scalar<bf16>(p); }
 extern "C" __global__ void __launch_bounds__(256) add_f32_scalar(AddParams p) { add_scalar<float>(p); }
 extern "C" __global__ void __launch_bounds__(256) add_f64_scalar(AddParams p) { add_scalar<double>(p); }

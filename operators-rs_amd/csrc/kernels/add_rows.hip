@@ -17,22 +17,27 @@ __device__ __forceinline__ bool add_rows_locate(const AddRowsParams &p, uint32_t
     return true;
 }
 
-extern "C" __global__ void __launch_bounds__(256) add_rows_f16_vec(AddRowsParams p) {
+template <typename T>
+__device__ __forceinline__ void add_rows_h_vec(const AddRowsParams &p) {  // T: f16 or bf16
     const uint32_t nvec = p.n / 8;
     for (uint32_t bm = blockIdx.y; bm < p.batch * p.m; bm += gridDim.y) {
         char *dst;
         const char *src;
         if (!add_rows_locate(p, bm, dst, src)) continue;
         for (uint32_t v = blockIdx.x * blockDim.x + threadIdx.x; v < nvec; v += gridDim.x * blockDim.x) {
-            Pack8 d, s;
+            PackOf<T> d, s;
             d.u = ld128_nt(dst + (size_t)v * 16);
             s.u = ld128(src + (size_t)v * 16);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) d.e[i] = f2h(h2f(d.e[i]) + h2f(s.e[i]));
+            for (int i = 0; i < 8; ++i) d.e[i] = (T)((float)d.e[i] + (float)s.e[i]);
             st128(dst + (size_t)v * 16, d.u);
         }
     }
 }
+extern "C" __global__ void __launch_bounds__(256) add_rows_f16_vec(AddRowsParams p) { add_rows_h_vec<f16>(p); }
+// bf16: the reference's CUDA backend compiles add_rows for any named type (add_rows/cuda/mod.rs:135-163); its CPU
+// backend has no bf16
+extern "C" __global__ void __launch_bounds__(256) add_rows_bf16_vec(AddRowsParams p) { add_rows_h_vec<bf16>(p); }
 
 // element-wise; nsd / nss are the element strides of dst and src rows in bytes
 template <typename T>
@@ -56,6 +61,9 @@ struct AddRowsScalarParams {
 };
 extern "C" __global__ void __launch_bounds__(256) add_rows_f16_scalar(AddRowsScalarParams q) {
     add_rows_scalar<f16>(q.p, q.nsd, q.nss);
+}
+extern "C" __global__ void __launch_bounds__(256) add_rows_bf16_scalar(AddRowsScalarParams q) {
+    add_rows_scalar<bf16>(q.p, q.nsd, q.nss);
 }
 extern "C" __global__ void __launch_bounds__(256) add_rows_f32_scalar(AddRowsScalarParams q) {
     add_rows_scalar<float>(q.p, q.nsd, q.nss);

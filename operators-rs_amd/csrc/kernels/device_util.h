@@ -7,6 +7,7 @@
 #include "params.h"
 
 typedef _Float16 f16;
+typedef __bf16 bf16;  // conversions from and to float are the hardware's (to bf16: nearest even)
 typedef f16 f16x2 __attribute__((ext_vector_type(2)));
 typedef f16 f16x4 __attribute__((ext_vector_type(4)));
 typedef f16 f16x8 __attribute__((ext_vector_type(8)));
@@ -40,6 +41,12 @@ union Pack4f {
     u32x4 u;
     f32x4 f;
     float e[4];
+};
+// 16 bytes of T (f16, bf16: 8 elements; f32: 4)
+template <typename T>
+union PackOf {
+    u32x4 u;
+    T e[16 / sizeof(T)];
 };
 
 template <typename T>

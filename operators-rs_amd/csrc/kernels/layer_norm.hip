@@ -9,39 +9,23 @@
 #include "device_util.h"
 
 template <typename TA>
-struct Vec;  // 16 bytes of TA
-template <>
-struct Vec<f16> {
-    static constexpr int N = 8;
-    Pack8 v;
-    __device__ __forceinline__ float get(int i) const { return h2f(v.e[i]); }
-    __device__ __forceinline__ void set(int i, float f) { v.e[i] = f2h(f); }
-};
-template <>
-struct Vec<float> {
-    static constexpr int N = 4;
-    Pack4f v;
-    __device__ __forceinline__ float get(int i) const { return v.e[i]; }
-    __device__ __forceinline__ void set(int i, float f) { v.e[i] = f; }
+struct Vec {  // 16 bytes of TA
+    static constexpr int N = 16 / sizeof(TA);
+    PackOf<TA> v;
+    __device__ __forceinline__ float get(int i) const { return (float)v.e[i]; }
+    __device__ __forceinline__ void set(int i, float f) { v.e[i] = (TA)f; }
 };
 
 // N consecutive parameters starting at element j (j multiple of N, base 16-byte aligned)
 template <typename TW, int N>
 __device__ __forceinline__ void load_param_vec(const void *w, uint32_t j, float (&out)[N]) {
-    if constexpr (sizeof(TW) == 2) {
-        static_assert(N == 8, "");
-        Pack8 p;
-        p.u = ld128(reinterpret_cast<const f16 *>(w) + j);
+    constexpr int PER = 16 / sizeof(TW);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) out[i] = h2f(p.e[i]);
-    } else {
+    for (int c = 0; c < N / PER; ++c) {
+        PackOf<TW> p;
+        p.u = ld128(reinterpret_cast<const TW *>(w) + j + PER * c);
 #pragma unroll
-        for (int c = 0; c < N / 4; ++c) {
-            Pack4f p;
-            p.u = ld128(reinterpret_cast<const float *>(w) + j + 4 * c);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) out[4 * c + i] = p.e[i];
-        }
+        for (int i = 0; i < PER; ++i) out[PER * c + i] = (float)p.e[i];
     }
 }
 
@@ -143,11 +127,11 @@ __device__ __forceinline__ void layer_norm_scalar(const LayerNormParams &p) {
         yr[j] = (TA)__builtin_fmaf((float)xr[j] - e, (float)sc[j] * k, (float)bi[j]);
 }
 
-// Many short rows of f16 (d <= 4096): a persistent workgroup converts scale and bias to f32
+// Many short rows of f16 or bf16 (d <= 4096): a persistent workgroup converts scale and bias to f32
 // once into LDS, then each of its waves streams rows (dealt round-robin over all waves of the
 // grid) with the next row's loads in flight while the current one is reduced and written.
 // Per row the only global traffic left is x in and y out.
-template <typename TW>
+template <typename TA, typename TW>
 __device__ __forceinline__ void layer_norm_rows(const LayerNormParams &p) {
     constexpr int CACHE = 8, MAXD = 4096;
     __shared__ float s_scale[MAXD], s_bias[MAXD];
@@ -163,7 +147,7 @@ __device__ __forceinline__ void layer_norm_rows(const LayerNormParams &p) {
     const uint32_t nvec = p.d / 8;
     if (row >= p.n) return;
 
-    Pack8 cur[CACHE], nxt[CACHE];
+    PackOf<TA> cur[CACHE], nxt[CACHE];
     {
         const char *xr = reinterpret_cast<const char *>(p.x) + (int64_t)row * p.nsx;
 #pragma unroll
@@ -189,7 +173,7 @@ __device__ __forceinline__ void layer_norm_rows(const LayerNormParams &p) {
             if (v < nvec) {
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
-                    const float f = h2f(cur[c].e[i]);
+                    const float f = (float)cur[c].e[i];
                     s1 += f;
                     s2 += f * f;
                 }
@@ -204,10 +188,10 @@ __device__ __forceinline__ void layer_norm_rows(const LayerNormParams &p) {
         for (int c = 0; c < CACHE; ++c) {
             const uint32_t v = lane + c * WAVE;
             if (v < nvec) {
-                Pack8 o;
+                PackOf<TA> o;
 #pragma unroll
                 for (int i = 0; i < 8; ++i)
-                    o.e[i] = f2h(__builtin_fmaf(h2f(cur[c].e[i]) - e, s_scale[v * 8 + i] * k, s_bias[v * 8 + i]));
+                    o.e[i] = (TA)__builtin_fmaf((float)cur[c].e[i] - e, s_scale[v * 8 + i] * k, s_bias[v * 8 + i]);
                 st128_nt(yr + (size_t)v * 16, o.u);
             }
         }
@@ -216,8 +200,10 @@ __device__ __forceinline__ void layer_norm_rows(const LayerNormParams &p) {
     }
 }
 
-extern "C" __global__ void __launch_bounds__(256) layer_norm_f16_f16_rows(LayerNormParams p) { layer_norm_rows<f16>(p); }
-extern "C" __global__ void __launch_bounds__(256) layer_norm_f16_f32_rows(LayerNormParams p) { layer_norm_rows<float>(p); }
+extern "C" __global__ void __launch_bounds__(256) layer_norm_f16_f16_rows(LayerNormParams p) { layer_norm_rows<f16, f16>(p); }
+extern "C" __global__ void __launch_bounds__(256) layer_norm_f16_f32_rows(LayerNormParams p) { layer_norm_rows<f16, float>(p); }
+extern "C" __global__ void __launch_bounds__(256) layer_norm_bf16_bf16_rows(LayerNormParams p) { layer_norm_rows<bf16, bf16>(p); }
+extern "C" __global__ void __launch_bounds__(256) layer_norm_bf16_f32_rows(LayerNormParams p) { layer_norm_rows<bf16, float>(p); }
 
 #define LAYER_NORM(NAME, TA, TW)                                                                                  \
     extern "C" __global__ void __launch_bounds__(256) layer_norm_##NAME##_g64(LayerNormParams p) {                \
@@ -235,6 +221,10 @@ extern "C" __global__ void __launch_bounds__(256) layer_norm_f16_f32_rows(LayerN
 LAYER_NORM(f16_f16, f16, f16)
 LAYER_NORM(f16_f32, f16, float)
 LAYER_NORM(f32_f32, float, float)
+// bf16 rows with bf16 or f32 scale and bias: pairs the reference's CUDA backend compiles a kernel for like for any
+// other named types (layer_norm/cuda/mod.rs:158-159); its CPU backend has none.  f32 arithmetic, result rounded to bf16.
+LAYER_NORM(bf16_bf16, bf16, bf16)
+LAYER_NORM(bf16_f32, bf16, float)
 
 // f64 rows with f64 scale and bias (layer_norm/common_cpu/mod.rs:97 lists the pair): all arithmetic in f64, as the
 // reference's, one workgroup per row.  No vector variant: the hot path is f16.

@@ -10,20 +10,11 @@
 #include "device_util.h"
 
 template <typename TA>
-struct Vec;  // 16 bytes of TA
-template <>
-struct Vec<f16> {
-    static constexpr int N = 8;
-    Pack8 v;
-    __device__ __forceinline__ float get(int i) const { return h2f(v.e[i]); }
-    __device__ __forceinline__ void set(int i, float f) { v.e[i] = f2h(f); }
-};
-template <>
-struct Vec<float> {
-    static constexpr int N = 4;
-    Pack4f v;
-    __device__ __forceinline__ float get(int i) const { return v.e[i]; }
-    __device__ __forceinline__ void set(int i, float f) { v.e[i] = f; }
+struct Vec {
+    static constexpr int N = 16 / sizeof(TA);
+    PackOf<TA> v;
+    __device__ __forceinline__ float get(int i) const { return (float)v.e[i]; }
+    __device__ __forceinline__ void set(int i, float f) { v.e[i] = (TA)f; }
 };
 
 template <typename TW>
@@ -42,19 +33,13 @@ struct RawW {
         for (int c = 0; c < NV; ++c) v[c] = ld128(reinterpret_cast<const TW *>(w) + j + c * (16 / sizeof(TW)));
     }
     __device__ __forceinline__ void get(float (&out)[N]) const {
-        if constexpr (sizeof(TW) == 2) {
-            Pack8 p;
-            p.u = v[0];
+        constexpr int PER = 16 / sizeof(TW);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) out[i] = h2f(p.e[i]);
-        } else {
+        for (int c = 0; c < NV; ++c) {
+            PackOf<TW> p;
+            p.u = v[c];
 #pragma unroll
-            for (int c = 0; c < NV; ++c) {
-                Pack4f p;
-                p.u = v[c];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) out[4 * c + i] = p.e[i];
-            }
+            for (int i = 0; i < PER; ++i) out[PER * c + i] = (float)p.e[i];
         }
     }
 };
@@ -62,21 +47,9 @@ struct RawW {
 // N consecutive weights starting at element j (j multiple of N, base 16-byte aligned)
 template <typename TW, int N>
 __device__ __forceinline__ void load_w_vec(const void *w, uint32_t j, float (&out)[N]) {
-    if constexpr (sizeof(TW) == 2) {
-        static_assert(N == 8, "");
-        Pack8 p;
-        p.u = ld128(reinterpret_cast<const f16 *>(w) + j);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) out[i] = h2f(p.e[i]);
-    } else {
-#pragma unroll
-        for (int c = 0; c < N / 4; ++c) {
-            Pack4f p;
-            p.u = ld128(reinterpret_cast<const float *>(w) + j + 4 * c);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) out[4 * c + i] = p.e[i];
-        }
-    }
+    RawW<TW, N> raw;
+    raw.load(w, j);
+    raw.get(out);
 }
 
 template <typename TA, typename TW, int G>
@@ -170,11 +143,11 @@ __device__ __forceinline__ void rms_norm_scalar(const RmsNormParams &p) {
 }
 
 
-// Many short rows (d <= 4096 halves): one wave per row, rows dealt round-robin to a
+// Many short rows (d <= 4096 elements of two bytes): one wave per row, rows dealt round-robin to a
 // fixed number of waves.  w is converted once and stays in registers for all rows
 // of the wave; the next row's x is already in flight while the current one is reduced
 // and written, so each wave keeps reads and writes streaming.
-template <typename TW>
+template <typename TA, typename TW>
 __device__ __forceinline__ void rms_norm_rows(const RmsNormParams &p) {
     constexpr int CACHE = 8;
     const uint32_t lane = threadIdx.x % WAVE;
@@ -183,14 +156,14 @@ __device__ __forceinline__ void rms_norm_rows(const RmsNormParams &p) {
     const uint32_t nvec = p.d / 8;
     if (row >= p.n) return;
 
-    // w stays in its storage type (f16 weights: 4 registers per vector) and is widened on use
+    // w stays in its storage type (two-byte weights: 4 registers per vector) and is widened on use
     struct WVec {
         u32x4 raw[sizeof(TW) / 2];
         __device__ __forceinline__ float get(int i) const {
             if constexpr (sizeof(TW) == 2) {
-                Pack8 t;
+                PackOf<TW> t;
                 t.u = raw[0];
-                return h2f(t.e[i]);
+                return (float)t.e[i];
             } else {
                 return __uint_as_float(raw[i / 4][i % 4]);
             }
@@ -205,7 +178,7 @@ __device__ __forceinline__ void rms_norm_rows(const RmsNormParams &p) {
                 w[c].raw[q] = ld128(reinterpret_cast<const char *>(p.w) + ((size_t)v * 8 * sizeof(TW)) + 16 * q);
         }
     }
-    Pack8 cur[CACHE], nxt[CACHE];
+    PackOf<TA> cur[CACHE], nxt[CACHE];
     {
         const char *xr = reinterpret_cast<const char *>(p.x) + (int64_t)row * p.nsx;
 #pragma unroll
@@ -231,7 +204,7 @@ __device__ __forceinline__ void rms_norm_rows(const RmsNormParams &p) {
             if (v < nvec) {
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
-                    const float f = h2f(cur[c].e[i]);
+                    const float f = (float)cur[c].e[i];
                     ss += f * f;
                 }
             }
@@ -243,9 +216,9 @@ __device__ __forceinline__ void rms_norm_rows(const RmsNormParams &p) {
         for (int c = 0; c < CACHE; ++c) {
             const uint32_t v = lane + c * WAVE;
             if (v < nvec) {
-                Pack8 o;
+                PackOf<TA> o;
 #pragma unroll
-                for (int i = 0; i < 8; ++i) o.e[i] = f2h((k * w[c].get(i)) * h2f(cur[c].e[i]));
+                for (int i = 0; i < 8; ++i) o.e[i] = (TA)((k * w[c].get(i)) * (float)cur[c].e[i]);
                 st128_nt(yr + (size_t)v * 16, o.u);
             }
         }
@@ -254,8 +227,10 @@ __device__ __forceinline__ void rms_norm_rows(const RmsNormParams &p) {
     }
 }
 
-extern "C" __global__ void __launch_bounds__(256) rms_norm_f16_f16_rows(RmsNormParams p) { rms_norm_rows<f16>(p); }
-extern "C" __global__ void __launch_bounds__(256) rms_norm_f16_f32_rows(RmsNormParams p) { rms_norm_rows<float>(p); }
+extern "C" __global__ void __launch_bounds__(256) rms_norm_f16_f16_rows(RmsNormParams p) { rms_norm_rows<f16, f16>(p); }
+extern "C" __global__ void __launch_bounds__(256) rms_norm_f16_f32_rows(RmsNormParams p) { rms_norm_rows<f16, float>(p); }
+extern "C" __global__ void __launch_bounds__(256) rms_norm_bf16_bf16_rows(RmsNormParams p) { rms_norm_rows<bf16, bf16>(p); }
+extern "C" __global__ void __launch_bounds__(256) rms_norm_bf16_f32_rows(RmsNormParams p) { rms_norm_rows<bf16, float>(p); }
 
 #define RMS_VEC(NAME, TA, TW, G)                                                        \
     extern "C" __global__ void __launch_bounds__((G) < 256 ? 256 : (G)) NAME(RmsNormParams p) { \
@@ -273,6 +248,17 @@ RMS_VEC(rms_norm_f16_f32_g1024, f16, float, 1024)
 RMS_VEC(rms_norm_f32_f32_g64, float, float, 64)
 RMS_VEC(rms_norm_f32_f32_g256, float, float, 256)
 RMS_VEC(rms_norm_f32_f32_g1024, float, float, 1024)
+// bf16 activations with bf16 or f32 weights: what the reference's CUDA backend also compiles a kernel for
+// (rms_norm/cuda/mod.rs:146-147 through handle/cuda/mod.rs:204); its CPU backend has no such pair.  Same arithmetic:
+// f32 throughout, the result rounded to bf16 (nearest even).
+RMS_VEC(rms_norm_bf16_bf16_g64, bf16, bf16, 64)
+RMS_VEC(rms_norm_bf16_bf16_g256, bf16, bf16, 256)
+RMS_VEC(rms_norm_bf16_bf16_g1024, bf16, bf16, 1024)
+RMS_VEC(rms_norm_bf16_f32_g64, bf16, float, 64)
+RMS_VEC(rms_norm_bf16_f32_g256, bf16, float, 256)
+RMS_VEC(rms_norm_bf16_f32_g1024, bf16, float, 1024)
+RMS_SCALAR(rms_norm_bf16_bf16_scalar, bf16, bf16)
+RMS_SCALAR(rms_norm_bf16_f32_scalar, bf16, float)
 RMS_SCALAR(rms_norm_f16_f16_scalar, f16, f16)
 RMS_SCALAR(rms_norm_f16_f32_scalar, f16, float)
 RMS_SCALAR(rms_norm_f32_f32_scalar, float, float)

@@ -137,8 +137,8 @@ def test_rms_norm_errors(gpu, stream):
         op.scheme(mk(good, L(dt.F32, [4, 256], [1024, 4]), L(dt.F16, [256], [2])), 0)
     assert e.value.kind == "TypeMismatch"
     # pairs of (activation, weight) types outside the CPU backend's list (rms_norm/common_cpu/mod.rs:84-90, where
-    # they are `todo!()`): refused by scheme and launch alike
-    for dta, dtw in [(dt.BF16, dt.BF16), (dt.F16, dt.F64), (dt.F32, dt.F16), (dt.F64, dt.F32), (dt.U32, dt.U32)]:
+    # they are `todo!()`) and the two bf16 pairs (tests/test_gpu_bf16.py): refused by scheme and launch alike
+    for dta, dtw in [(dt.BF16, dt.F16), (dt.F16, dt.BF16), (dt.F16, dt.F64), (dt.F32, dt.F16), (dt.F64, dt.F32), (dt.U32, dt.U32)]:
         na, nw = ophip.dtype_nbytes(dta), ophip.dtype_nbytes(dtw)
         a = mk(L(dta, [4, 256], [256 * na, na]), L(dta, [4, 256], [256 * na, na]), L(dtw, [256], [nw]))
         with pytest.raises(ophip.SchemeError) as e:
