@@ -441,14 +441,21 @@ def mat_mul_lines(o, gpu, stream, rng, add, launches=0):
     mm = o.MatMul(gpu)
     shapes = [(4096, 4096, 4096, False), (4096, 4096, 4096, True), (8192, 8192, 8192, False), (8192, 8192, 8192, True),
               (512, 12288, 4096, False), (512, 22016, 4096, False), (512, 4096, 11008, False),
-              (509, 12288, 4096, False), (4000, 4000, 4096, False)]
-    for m, n, k, b_nk in shapes:
-        A_, B_, C_ = gpu.from_host(normal_f16(rng, (m, k), 1.0)), gpu.from_host(normal_f16(rng, (k, n), 0.02)), \
+              (509, 12288, 4096, False), (4000, 4000, 4096, False), (8192, 8192, 8192, True, dt.BF16)]
+    for m, n, k, b_nk, *et in shapes:
+        et = et[0] if et else dt.F16
+        if launches and et != dt.F16:
+            continue  # (the bf16 build's kernels carry the f16 build's names: a counter run would mix the two)
+        # (bf16: the top halves of f32 normals, which are bf16 normals of the same spread)
+        mk = normal_f16 if et == dt.F16 else lambda r, sh, std: np.ascontiguousarray(
+            (r.standard_normal(sh, dtype=np.float32) * np.float32(std)).view(np.uint32) >> 16).astype(np.uint16)
+        c = lambda *s, et=et: L.new_contiguous(et, list(s))
+        A_, B_, C_ = gpu.from_host(mk(rng, (m, k), 1.0)), gpu.from_host(mk(rng, (k, n), 0.02)), \
             gpu.malloc(m * n * 2)
-        bl = L(dt.F16, [k, n], [2, k * 2]) if b_nk else c(k, n)  # the same bytes read as B[N, K] transposed
+        bl = L(et, [k, n], [2, k * 2]) if b_nk else c(k, n)  # the same bytes read as B[N, K] transposed
         a = o.MatMulArgs(c(m, n), C_, 0.0, c(m, k), A_, bl, B_, 1.0)
         ws = gpu.malloc(max(mm.scheme(a, 1 << 32), 1))
-        shape = "%dx%dx%d%s" % (m, n, k, ", B stored [N,K]" if b_nk else "")
+        shape = "%dx%dx%d%s%s" % (m, n, k, ", B stored [N,K]" if b_nk else "", ", bf16" if et != dt.F16 else "")
         nbytes, flops = 2 * (m * k + k * n + m * n), 2 * m * n * k
         if launches:
             us = time_launches(gpu, stream, lambda: mm.launch(a, ws, stream), launches, warm=1)
@@ -625,16 +632,19 @@ def standalone_ops(ophip, gpu, stream, rng, reps, ceiling=None):
     ya = gpu.malloc(nt * 2 * DI * 2)
     w2 = [gpu.from_host(normal_f16(rng, (D, 2 * DI), 0.02)) for _ in range(2)]
     wsb = gpu.malloc(64 << 20)
-    for b_nk in (False, True):
-        bl = L(F16, [D, 2 * DI], [2, D * 2]) if b_nk else c(D, 2 * DI)
-        pair = [o.MatMulArgs(c(nt, 2 * DI), ya, 0.0, c(nt, D), xa, bl, w, 1.0) for w in w2]
+    # (the third line: the same buffers read as bf16 numbers -- every f16 pattern here is a finite bf16 -- by the bf16
+    # build of the same kernel)
+    for b_nk, et in ((False, F16), (True, F16), (False, o.dt.BF16)):
+        ce = lambda *s_: L.new_contiguous(et, list(s_))
+        bl = L(et, [D, 2 * DI], [2, D * 2]) if b_nk else ce(D, 2 * DI)
+        pair = [o.MatMulArgs(ce(nt, 2 * DI), ya, 0.0, ce(nt, D), xa, bl, w, 1.0) for w in w2]
         flip = [0]
 
         def run():
             flip[0] ^= 1
             mm.launch(pair[flip[0]], wsb, stream)
         us = time_launches(gpu, stream, run, reps)
-        add("mat_mul", "%dx%dx%d%s" % (nt, 2 * DI, D, ", B stored [N,K]" if b_nk else ""),
+        add("mat_mul", "%dx%dx%d%s%s" % (nt, 2 * DI, D, ", B stored [N,K]" if b_nk else "", ", bf16" if et != F16 else ""),
             2 * (nt * D + D * 2 * DI + nt * 2 * DI), us, flops=2 * nt * D * 2 * DI, note="cold weights, " + mm.describe(pair[0]))
     for w in w2:
         w.free()

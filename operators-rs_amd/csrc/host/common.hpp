@@ -124,6 +124,7 @@ inline bool mult16(ptrdiff_t v) { return (v & 15) == 0; }
 
 // f32 -> f16 -> f32 (round to nearest even), for the scalars the reference rounds to f16
 float round_to_f16(float f);
+float round_to_bf16(float f);  // nearest even; NaN and infinity unchanged
 
 // Least-recently-used map guarded by a mutex: the shape of the reference's
 // Mutex<LruCache<SchemeKey, Scheme>> (e.g. rms_norm/cuda/mod.rs:14-17).

@@ -19,6 +19,16 @@ void check_hip(hipError_t e, const char *what) {
                                ") " + hipGetErrorString(e));
 }
 
+float round_to_bf16(float f) {
+    uint32_t x;
+    std::memcpy(&x, &f, 4);
+    if (((x >> 23) & 0xffu) == 0xffu) return f;
+    x = (x + 0x7fffu + ((x >> 16) & 1u)) & 0xffff0000u;
+    float r;
+    std::memcpy(&r, &x, 4);
+    return r;
+}
+
 float round_to_f16(float f) {
     // software round-to-nearest-even f32 -> f16 -> f32
     uint32_t x;

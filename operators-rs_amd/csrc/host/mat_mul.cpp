@@ -123,6 +123,10 @@ struct GemmKnobs {
     }
 };
 
+// f16, f32, f64: the CPU backend's types (mat_mul/common_cpu/mod.rs:99-103).  bf16: neither backend of the reference
+// multiplies it (its CUDA backend checks for F16, mat_mul/cuda/mod.rs:73); taken here because the matrix cores do.
+bool mat_mul_takes(uint64_t dt) { return dt == OPHIP_DT_F16 || dt == OPHIP_DT_BF16 || dt == OPHIP_DT_F32 || dt == OPHIP_DT_F64; }
+
 GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L, unsigned cus, const GemmKnobs &knobs) {
     const void *a = L.ab_swap ? args.b_base : args.a_base;
     const void *b = L.ab_swap ? args.a_base : args.b_base;
@@ -135,9 +139,12 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
     p.K = (uint32_t)L.k;
     p.d = args.c_base;
     p.d_sb = L.c_stride;
-    const bool f16 = L.dt == OPHIP_DT_F16;
-    p.alpha = f16 ? round_to_f16(args.alpha) : args.alpha;
-    p.beta = f16 ? round_to_f16(args.beta) : args.beta;
+    // f16 and bf16 take the same MFMA kernels (two builds of one source); alpha and beta are rounded to the data's type
+    // first, as the reference does for f16 (mat_mul/common_cpu/mod.rs:60-105)
+    const bool f16 = L.dt == OPHIP_DT_F16 || L.dt == OPHIP_DT_BF16;
+    auto rounded = [&](float v) { return L.dt == OPHIP_DT_F16 ? round_to_f16(v) : L.dt == OPHIP_DT_BF16 ? round_to_bf16(v) : v; };
+    p.alpha = rounded(args.alpha);
+    p.beta = rounded(args.beta);
     p.read_dst = args.beta != 0.f;
     p.split_k = 1;
     p.k_per_split = (uint32_t)((L.k + 31) / 32 * 32);
@@ -342,10 +349,11 @@ constexpr size_t SPLITK_COUNTERS = 1 << 16;
 struct ophip_mat_mul {
     ophip_device *dev;
     GemmKnobs knobs = GemmKnobs::from_env();
-    hipFunction_t skinny[3][4];  // [mt index 1,2,4][qmode; 3 = mode 0 with paired K-steps]
-    hipFunction_t reduce, fill, generic_f16, generic_f32, generic_f64;
+    // the MFMA kernels exist twice, [0] on f16 and [1] on bf16 elements
+    hipFunction_t skinny[2][3][4];  // [mt index 1,2,4][qmode; 3 = mode 0 with paired K-steps]
+    hipFunction_t reduce[2], fill, generic_f16, generic_bf16, generic_f32, generic_f64;
     // [256 x 64 / 128 x 64 / 128 x 32 (K-step)][M or N not in whole tiles][P K-contiguous][Q K-contiguous]
-    hipFunction_t tile[3][2][2][2];
+    hipFunction_t tile[2][3][2][2][2];
     // Arrival counters live in a buffer owned by the operator, one per stream:
     // launches on one stream run in order and every kernel leaves its counters at
     // zero, so a buffer is zeroed once.  The first stream gets the buffer made (and cleared) with the operator,
@@ -384,19 +392,22 @@ struct ophip_mat_mul {
     explicit ophip_mat_mul(ophip_device *d) : dev(d) {
         ophip_device_retain(d);
         static const int mts[3] = {1, 2, 4};
-        for (int i = 0; i < 3; ++i)
-            for (int q = 0; q < 4; ++q)
-                skinny[i][q] = d->kernel(
-                    "gemm", ("gemm_skinny_m" + std::to_string(mts[i]) + "_q" + (q == 3 ? "0p" : std::to_string(q))).c_str());
-        for (int b = 0; b < 3; ++b)
-            for (int r = 0; r < 2; ++r)
-                for (int pk = 0; pk < 2; ++pk)
-                    for (int qk = 0; qk < 2; ++qk) {
-                        const std::string sz = b == 0 ? "256x256" : b == 1 ? "128x128" : "128x128k32";
-                        tile[b][r][pk][qk] = d->kernel("gemm_tile", ("gemm_tile_" + sz + (r ? "r" : "") + "_p" + std::to_string(pk) +
-                                                                    "_q" + std::to_string(qk)).c_str());
-                    }
-        reduce = d->kernel("gemm", "gemm_splitk_reduce");
+        for (int e = 0; e < 2; ++e) {
+            const char *gemm = e ? "gemm_bf16" : "gemm", *gemm_tile = e ? "gemm_tile_bf16" : "gemm_tile";
+            for (int i = 0; i < 3; ++i)
+                for (int q = 0; q < 4; ++q)
+                    skinny[e][i][q] = d->kernel(
+                        gemm, ("gemm_skinny_m" + std::to_string(mts[i]) + "_q" + (q == 3 ? "0p" : std::to_string(q))).c_str());
+            for (int b = 0; b < 3; ++b)
+                for (int r = 0; r < 2; ++r)
+                    for (int pk = 0; pk < 2; ++pk)
+                        for (int qk = 0; qk < 2; ++qk) {
+                            const std::string sz = b == 0 ? "256x256" : b == 1 ? "128x128" : "128x128k32";
+                            tile[e][b][r][pk][qk] = d->kernel(gemm_tile, ("gemm_tile_" + sz + (r ? "r" : "") + "_p" + std::to_string(pk) +
+                                                                          "_q" + std::to_string(qk)).c_str());
+                        }
+            reduce[e] = d->kernel(gemm, "gemm_splitk_reduce");
+        }
         fill = d->kernel("gemm", "gemm_fill_u32");
         d->make_current();
         check_hip(hipMalloc(&spare, SPLITK_COUNTERS * sizeof(uint32_t)), "hipMalloc");
@@ -408,6 +419,7 @@ struct ophip_mat_mul {
             check_hip(e2, "hipMemset");
         }
         generic_f16 = d->kernel("gemm", "gemm_generic_f16");
+        generic_bf16 = d->kernel("gemm_bf16", "gemm_generic_bf16");
         generic_f32 = d->kernel("gemm", "gemm_generic_f32");
         generic_f64 = d->kernel("gemm", "gemm_generic_f64");
         std::lock_guard<std::mutex> lock(d->hooks_mu);
@@ -440,7 +452,7 @@ static void mat_mul_launch_impl(const ophip_mat_mul *op, const ophip_mat_mul_arg
                                 size_t fixed_counter_count, hipStream_t stream) {
     if (!op || !args) throw args_not_support("null argument");
     const ophip_mat_mul_layout L = mat_mul_layout(*args);
-    if (L.dt != OPHIP_DT_F16 && L.dt != OPHIP_DT_F32 && L.dt != OPHIP_DT_F64) throw type_not_support("mat_mul supports f16, f32 and f64");
+    if (!mat_mul_takes(L.dt)) throw type_not_support("mat_mul supports f16, bf16, f32 and f64");
     if (is_dyn(args->alpha) || is_dyn(args->beta)) throw dyn_not_support("");
     if (L.m == 0 || L.n == 0 || L.batch == 0) return;
     if (L.m > 0x7fffffffu || L.n > 0x7fffffffu || L.k > 0x7fffffffu || L.batch > 65535)
@@ -448,6 +460,7 @@ static void mat_mul_launch_impl(const ophip_mat_mul *op, const ophip_mat_mul_arg
     GemmPlan g = make_plan(*args, L, (unsigned)op->dev->props.multiProcessorCount, op->knobs);
     const GemmParams &p = g.p;
     const bool fixed = fixed_counters != nullptr;
+    const int e = L.dt == OPHIP_DT_BF16 ? 1 : 0;
     if (fixed && g.workspace > workspace_len)
         throw args_not_support("this product needs " + std::to_string(g.workspace) +
                                " bytes of split-K scratch, the library's static buffer holds " +
@@ -469,10 +482,10 @@ static void mat_mul_launch_impl(const ophip_mat_mul *op, const ophip_mat_mul_arg
             g.p.counters = (p.split_k > 1 && tiles <= SPLITK_COUNTERS && g.workspace < ((size_t)1 << 32)) ? op->counters_for(stream) : nullptr;
         }
         const int mi = g.mt == 1 ? 0 : g.mt == 2 ? 1 : 2;
-        launch(op->skinny[mi][g.qmode], Dim3{(p.N + 127) / 128, p.split_k, p.batch}, Dim3{256}, 0, stream, g.p);
+        launch(op->skinny[e][mi][g.qmode], Dim3{(p.N + 127) / 128, p.split_k, p.batch}, Dim3{256}, 0, stream, g.p);
         if (p.split_k > 1 && !g.p.counters) {
             const size_t total = (size_t)p.batch * p.M * (p.N / 8);
-            launch(op->reduce, Dim3{(unsigned)((total + 255) / 256)}, Dim3{256}, 0, stream, g.p);
+            launch(op->reduce[e], Dim3{(unsigned)((total + 255) / 256)}, Dim3{256}, 0, stream, g.p);
         }
         return;
     }
@@ -480,18 +493,18 @@ static void mat_mul_launch_impl(const ophip_mat_mul *op, const ophip_mat_mul_arg
         Workspace ws(fixed ? nullptr : qa, workspace, workspace_len, g.workspace);
         g.p.partial = ws.ptr();
         const unsigned tiles = ((p.M + g.tile - 1) / g.tile) * ((p.N + g.tile - 1) / g.tile);
-        launch(op->tile[g.tile == 256 ? 0 : g.tk == 64 ? 1 : 2][g.ragged][g.pk][g.qk], Dim3{tiles, p.split_k, p.batch}, Dim3{256}, 0,
+        launch(op->tile[e][g.tile == 256 ? 0 : g.tk == 64 ? 1 : 2][g.ragged][g.pk][g.qk], Dim3{tiles, p.split_k, p.batch}, Dim3{256}, 0,
                stream, g.p);
         if (p.split_k > 1) {
             const size_t total = (size_t)p.batch * p.M * (p.N / 8);
-            launch(op->reduce, Dim3{(unsigned)((total + 255) / 256)}, Dim3{256}, 0, stream, g.p);
+            launch(op->reduce[e], Dim3{(unsigned)((total + 255) / 256)}, Dim3{256}, 0, stream, g.p);
         }
         return;
     }
     const unsigned gx = (p.N + 63) / 64, gy = (p.M + 63) / 64;
     if (gy > 65535) throw shape_not_support("mat_mul dimension too large for the generic kernel");
-    launch(L.dt == OPHIP_DT_F16 ? op->generic_f16 : L.dt == OPHIP_DT_F32 ? op->generic_f32 : op->generic_f64, Dim3{gx, gy, p.batch}, Dim3{256}, 0, stream,
-           g.p);
+    launch(L.dt == OPHIP_DT_F16 ? op->generic_f16 : L.dt == OPHIP_DT_BF16 ? op->generic_bf16 : L.dt == OPHIP_DT_F32 ? op->generic_f32 : op->generic_f64,
+           Dim3{gx, gy, p.batch}, Dim3{256}, 0, stream, g.p);
 }
 
 namespace ophip {
@@ -527,7 +540,7 @@ int ophip_mat_mul_scheme(ophip_mat_mul *op, const ophip_mat_mul_args *args, size
         if (!op || !args) return;
         try {
             const ophip_mat_mul_layout L = mat_mul_layout(*args);
-            if (L.dt != OPHIP_DT_F16 && L.dt != OPHIP_DT_F32 && L.dt != OPHIP_DT_F64) return;
+            if (!mat_mul_takes(L.dt)) return;
             const GemmPlan g = make_plan(*args, L, (unsigned)op->dev->props.multiProcessorCount, op->knobs);
             if (ws && g.workspace <= max_ws) *ws = g.workspace;
         } catch (const Error &) {
@@ -539,7 +552,7 @@ int ophip_mat_mul_describe(const ophip_mat_mul *op, const ophip_mat_mul_args *ar
     return guard([&] {
         if (!op || !args || !out || len == 0) throw args_not_support("null argument");
         const ophip_mat_mul_layout L = mat_mul_layout(*args);
-        if (L.dt != OPHIP_DT_F16 && L.dt != OPHIP_DT_F32 && L.dt != OPHIP_DT_F64) throw type_not_support("mat_mul supports f16, f32 and f64");
+        if (!mat_mul_takes(L.dt)) throw type_not_support("mat_mul supports f16, bf16, f32 and f64");
         const GemmPlan g = make_plan(*args, L, (unsigned)op->dev->props.multiProcessorCount, op->knobs);
         if (g.kind == GemmPlan::Skinny)
             std::snprintf(out, len, "skinny rows<=%d q%s split_k=%u", 16 * g.mt,

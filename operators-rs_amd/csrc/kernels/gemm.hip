@@ -1,4 +1,5 @@
-// mat_mul kernels for gfx950 (f16 storage, f32 accumulation).
+// mat_mul kernels for gfx950 (f16 storage, f32 accumulation; compiled a second time on bf16 elements, see
+// gemm_elem.h: `elem` below is the element type of the build).
 //
 // Canonical problem (the host maps the reference's column-major descriptor onto it):
 //     D[i, j] = alpha * sum_l P[i, l] * Q[l, j] + (read_dst ? beta * D[i, j] : 0)
@@ -6,13 +7,13 @@
 //  gemm_skinny_*  : M <= 64 rows (decode: a handful of tokens against a weight
 //                   matrix).  HBM-bound: Q is streamed exactly once with 16-byte
 //                   loads straight into MFMA operand registers, P (tiny) comes
-//                   from L2, the product runs on v_mfma_f32_16x16x32_f16.
+//                   from L2, the product runs on v_mfma_f32_16x16x32_f16 (_bf16).
 //  gemm_generic_* : any strides / alignment, LDS-tiled FMA; the safety net.
 //  gemm_splitk_reduce : sums the f32 partials of a split-K skinny launch in a
 //                   fixed order and applies alpha / beta.
 #include <type_traits>
 
-#include "device_util.h"
+#include "gemm_elem.h"
 
 // ----------------------------------------------------------- skinny (MFMA) --
 //
@@ -44,7 +45,7 @@ constexpr int SK_WAVES = 4;
 // clamped into the matrix (lanes past N load valid memory and their results are
 // dropped at the store), so the steady-state loop carries no branches.
 template <int QMODE>
-__device__ __forceinline__ void skinny_load_q(const GemmParams &p, const f16 *qb, uint32_t kb, uint32_t colc,
+__device__ __forceinline__ void skinny_load_q(const GemmParams &p, const elem *qb, uint32_t kb, uint32_t colc,
                                               uint32_t g, u32x4 (&w)[8]) {
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
@@ -58,7 +59,7 @@ __device__ __forceinline__ void skinny_load_q(const GemmParams &p, const f16 *qb
 }
 // Same, for a final K-step that reaches past kend: rows beyond it read as zero.
 template <int QMODE>
-__device__ __forceinline__ void skinny_load_q_tail(const GemmParams &p, const f16 *qb, uint32_t kb, uint32_t kend,
+__device__ __forceinline__ void skinny_load_q_tail(const GemmParams &p, const elem *qb, uint32_t kb, uint32_t kend,
                                                    uint32_t colc, uint32_t g, u32x4 (&w)[8]) {
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
@@ -111,26 +112,26 @@ __device__ __forceinline__ void partial_load4(__amdgpu_buffer_rsrc_t r, uint32_t
 // D[i, col0 .. col0+7] = alpha * sum + beta * D, rounded once to f16
 __device__ __forceinline__ void skinny_store(const GemmParams &p, uint32_t bat, uint32_t i, uint32_t col0,
                                              const float (&sum)[8]) {
-    f16 *dst = reinterpret_cast<f16 *>(p.d) + (int64_t)bat * p.d_sb + (int64_t)i * p.d_si;
+    elem *dst = reinterpret_cast<elem *>(p.d) + (int64_t)bat * p.d_sb + (int64_t)i * p.d_si;
     if (p.d_sj == 1) {
-        Pack8 o;
+        PackE o;
         if (p.read_dst) {
-            Pack8 c;
+            PackE c;
             c.u = ld128(dst + col0);
 #pragma unroll
-            for (int t = 0; t < 8; ++t) o.e[t] = f2h(p.beta * h2f(c.e[t]) + p.alpha * sum[t]);
+            for (int t = 0; t < 8; ++t) o.e[t] = f2e(p.beta * e2f(c.e[t]) + p.alpha * sum[t]);
         } else {
 #pragma unroll
-            for (int t = 0; t < 8; ++t) o.e[t] = f2h(p.alpha * sum[t]);
+            for (int t = 0; t < 8; ++t) o.e[t] = f2e(p.alpha * sum[t]);
         }
         st128(dst + col0, o.u);
     } else {
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
-            f16 *e = dst + (int64_t)(col0 + t) * p.d_sj;
+            elem *e = dst + (int64_t)(col0 + t) * p.d_sj;
             float r = p.alpha * sum[t];
-            if (p.read_dst) r = p.beta * h2f(*e) + r;
-            *e = f2h(r);
+            if (p.read_dst) r = p.beta * e2f(*e) + r;
+            *e = f2e(r);
         }
     }
 }
@@ -150,8 +151,8 @@ __device__ __forceinline__ void gemm_skinny(const GemmParams &p) {
     const uint32_t kend = min(p.K, kbeg + p.k_per_split);
     const uint32_t col0 = n0 + 8 * j16;
 
-    const f16 *qb = reinterpret_cast<const f16 *>(p.q) + (int64_t)bat * p.q_sb;
-    const f16 *pb = reinterpret_cast<const f16 *>(p.p) + (int64_t)bat * p.p_sb;
+    const elem *qb = reinterpret_cast<const elem *>(p.q) + (int64_t)bat * p.q_sb;
+    const elem *pb = reinterpret_cast<const elem *>(p.p) + (int64_t)bat * p.p_sb;
 
     f32x4 acc[MT][8];
 #pragma unroll
@@ -160,7 +161,7 @@ __device__ __forceinline__ void gemm_skinny(const GemmParams &p) {
         for (int t = 0; t < 8; ++t) acc[mt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     // rows of P this lane feeds (clamped: rows past M only produce output rows that are never stored)
-    const f16 *prow[MT];
+    const elem *prow[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) prow[mt] = pb + (int64_t)min(mt * 16 + j16, p.M - 1) * p.p_si + 8 * g;
     const uint32_t colc = min(col0, p.N - 8);
@@ -172,7 +173,7 @@ __device__ __forceinline__ void gemm_skinny(const GemmParams &p) {
         const uint32_t cnt = chunks > wave ? (chunks - wave + SK_WAVES - 1) / SK_WAVES : 0;  // K-chunks of this wave
         // load t of a step: local column lc = 4t + g = (n, cb) = (lc / 2, lc % 2) -> column n0 + 8n + cb (+ 2cg),
         // 8 of K at 8 * j16; LDS row cb * 16 + n
-        const f16 *qrow[8];
+        const elem *qrow[8];
         uint32_t wr_off[8];
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
@@ -205,13 +206,13 @@ __device__ __forceinline__ void gemm_skinny(const GemmParams &p) {
             for (int cb = 0; cb < 2; ++cb)
 #pragma unroll
                 for (int kb4 = 0; kb4 < 4; ++kb4) {
-                    Pack8 bt;
+                    PackE bt;
                     bt.u = ld128(tr + rd_off + cb * (16 * SK_TR_PITCH) + kb4 * 64);
 #pragma unroll
                     for (int mt = 0; mt < MT; ++mt) {
-                        Pack8 at;
+                        PackE at;
                         at.u = a_cur[mt][kb4];
-                        acc[mt][2 * cg + cb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(at.h, bt.h, acc[mt][2 * cg + cb], 0, 0, 0);
+                        acc[mt][2 * cg + cb] = mfma_16x16x32(at.h, bt.h, acc[mt][2 * cg + cb]);
                     }
                 }
         };
@@ -253,13 +254,13 @@ __device__ __forceinline__ void gemm_skinny(const GemmParams &p) {
             }
 #pragma unroll
             for (int t = 0; t < 8; ++t) {
-                Pack8 bt;
+                PackE bt;
                 bt.u = b[t];
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) {
-                    Pack8 at;
+                    PackE at;
                     at.u = a[mt];
-                    acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(at.h, bt.h, acc[mt][t], 0, 0, 0);
+                    acc[mt][t] = mfma_16x16x32(at.h, bt.h, acc[mt][t]);
                 }
             }
         };
@@ -432,12 +433,12 @@ __device__ __forceinline__ void gemm_skinny(const GemmParams &p) {
         const uint32_t i = mt * 16 + 4 * g + wave;
         if (i < p.M && col0 < p.N) {
             if (p.split_k > 1) {
-                const size_t elem = (((size_t)split * p.batch + bat) * p.M + i) * p.N + col0;
-                float *dst = reinterpret_cast<float *>(p.partial) + elem;
+                const size_t first = (((size_t)split * p.batch + bat) * p.M + i) * p.N + col0;
+                float *dst = reinterpret_cast<float *>(p.partial) + first;
                 if (p.counters) {
                     const __amdgpu_buffer_rsrc_t r = partial_rsrc(p.partial);
-                    partial_store4(r, (uint32_t)(elem * 4), sum[0], sum[1], sum[2], sum[3]);
-                    partial_store4(r, (uint32_t)(elem * 4 + 16), sum[4], sum[5], sum[6], sum[7]);
+                    partial_store4(r, (uint32_t)(first * 4), sum[0], sum[1], sum[2], sum[3]);
+                    partial_store4(r, (uint32_t)(first * 4 + 16), sum[4], sum[5], sum[6], sum[7]);
                 } else {
                     *reinterpret_cast<f32x4 *>(dst) = f32x4{sum[0], sum[1], sum[2], sum[3]};
                     *reinterpret_cast<f32x4 *>(dst + 4) = f32x4{sum[4], sum[5], sum[6], sum[7]};
@@ -610,6 +611,10 @@ __device__ __forceinline__ void gemm_generic(const GemmParams &p) {
         }
 }
 
+#ifdef GEMM_ELEM_BF16
+extern "C" __global__ void __launch_bounds__(256) gemm_generic_bf16(GemmParams p) { gemm_generic<bf16>(p); }
+#else
+// (the kernels that do not depend on the build's element type are part of the f16 build only)
 // Clears a fresh buffer of arrival counters.  A kernel rather than a memset: it can be recorded into a launch graph
 // like any other launch when an operator's first split-K product on a stream happens during recording.
 extern "C" __global__ void __launch_bounds__(256) gemm_fill_u32(FillU32Params p) {
@@ -620,3 +625,4 @@ extern "C" __global__ void __launch_bounds__(256) gemm_fill_u32(FillU32Params p)
 extern "C" __global__ void __launch_bounds__(256) gemm_generic_f64(GemmParams p) { gemm_generic<double>(p); }
 extern "C" __global__ void __launch_bounds__(256) gemm_generic_f16(GemmParams p) { gemm_generic<f16>(p); }
 extern "C" __global__ void __launch_bounds__(256) gemm_generic_f32(GemmParams p) { gemm_generic<float>(p); }
+#endif

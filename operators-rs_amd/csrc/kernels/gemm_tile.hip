@@ -1,4 +1,5 @@
-// Compute-bound mat_mul for gfx950: LDS-tiled MFMA kernel (f16 in, f32 accumulate).
+// Compute-bound mat_mul for gfx950: LDS-tiled MFMA kernel (f16 in, f32 accumulate; compiled a second time on bf16
+// elements, see gemm_elem.h: `elem` below is the element type of the build).
 //
 //     D[i, j] = alpha * sum_l P[i, l] * Q[l, j] + (read_dst ? beta * D[i, j] : 0)
 //
@@ -22,9 +23,8 @@
 // of 8).  Everything else runs on the generic kernel.
 #include <type_traits>
 
-#include "device_util.h"
+#include "gemm_elem.h"
 
-typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 // Copies one R x TK operand tile from global memory to registers (`fetch`) and
 // from registers to LDS (`commit`).  KCONTIG: rows are K-contiguous in memory.
@@ -119,17 +119,17 @@ struct TileLoader {
     // into NV pieces so that the main loop can place them one by one between MFMAs.
     // The empty asm keeps the compiler from widening the offset to 64 bits outside the loop: as
     // "uniform base + 32-bit lane offset" the load needs no address arithmetic.
-    __device__ __forceinline__ void fetch_piece(const f16 *tile, int v) {
+    __device__ __forceinline__ void fetch_piece(const elem *tile, int v) {
         asm volatile("" : "+v"(voff[v]));
         reg[v] = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(tile) + voff[v]);
     }
-    __device__ __forceinline__ void fetch(const f16 *tile) {
+    __device__ __forceinline__ void fetch(const elem *tile) {
 #pragma unroll
         for (int v = 0; v < NV; ++v) fetch_piece(tile, v);
     }
     // The last, partial K-step of a K that is no multiple of TK: only `kvalid` (< TK) of the tile's k exist,
     // the rest is filled with zeros.  Runs once per workgroup, outside the pipelined loop.
-    __device__ __forceinline__ void fetch_tail(const f16 *tile, uint32_t kvalid) {
+    __device__ __forceinline__ void fetch_tail(const elem *tile, uint32_t kvalid) {
         const uint32_t t = threadIdx.x;
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
@@ -156,7 +156,7 @@ struct TileLoader {
     // holds k-row (kb*NV + v), columns cb*8 .. +8, and piece v writes columns
     // v*8/NV .. (v+1)*8/NV, each as the NV halves the thread holds of it (so every piece
     // reads all NV registers: refill them only after the last piece).
-    __device__ __forceinline__ void commit_piece(f16 *lds, int v) const {
+    __device__ __forceinline__ void commit_piece(elem *lds, int v) const {
         const uint32_t t = threadIdx.x;
         if constexpr (KCONTIG) {
             const uint32_t idx = t + v * 256, row = idx / KV, kv = idx % KV;
@@ -165,7 +165,7 @@ struct TileLoader {
             const uint32_t cb = cb_of(t), kb = kb_of(t);
 #pragma unroll
             for (int c = v * 8 / NV; c < (v + 1) * 8 / NV; ++c) {
-                f16 *dst = lds + TileRow<TK>::at(c * (R / 8) + cb, kb * NV / 8) + kb * NV % 8;
+                elem *dst = lds + TileRow<TK>::at(c * (R / 8) + cb, kb * NV / 8) + kb * NV % 8;
                 uint32_t w[NV / 2];
 #pragma unroll
                 for (int d = 0; d < NV / 2; ++d) w[d] = pair(reg[2 * d][c / 2], reg[2 * d + 1][c / 2], c & 1);
@@ -188,12 +188,12 @@ struct TileLoader {
         for (int d = 0; d < 4; ++d) w[d] = pair(reg[(2 * d) % NV][v / 2], reg[(2 * d + 1) % NV][v / 2], v & 1);
         return w;
     }
-    __device__ __forceinline__ void store_packed(f16 *lds, int v, u32x4 w) const {
+    __device__ __forceinline__ void store_packed(elem *lds, int v, u32x4 w) const {
         const uint32_t t = threadIdx.x;
         const uint32_t cb = cb_of(t), kb = kb_of(t);
         st128(lds + TileRow<TK>::at(v * (R / 8) + cb, kb * NV / 8) + kb * NV % 8, w);
     }
-    __device__ __forceinline__ void commit(f16 *lds) const {
+    __device__ __forceinline__ void commit(elem *lds) const {
 #pragma unroll
         for (int v = 0; v < NV; ++v) commit_piece(lds, v);
     }
@@ -211,7 +211,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
     // LDS: P buffer 0, P buffer 1, Q buffer 0, Q buffer 1.  Both buffers of an operand are within
     // 64 KiB of each other, so one address register per lane serves both through the
     // instruction's immediate offset.
-    __shared__ f16 lds[2 * (BM + BN) * LDK];
+    __shared__ elem lds[2 * (BM + BN) * LDK];
     constexpr uint32_t Q_REGION = 2 * BM * LDK;
     auto p_buf = [&](int b) { return lds + b * (BM * LDK); };
     auto q_buf = [&](int b) { return lds + Q_REGION + b * (BN * LDK); };
@@ -236,8 +236,8 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
     const uint32_t tile_n = (id % group_size) / rows_in_group;
     const uint32_t bat = blockIdx.z;
 
-    const f16 *pb = reinterpret_cast<const f16 *>(p.p) + (int64_t)bat * p.p_sb;
-    const f16 *qb = reinterpret_cast<const f16 *>(p.q) + (int64_t)bat * p.q_sb;
+    const elem *pb = reinterpret_cast<const elem *>(p.p) + (int64_t)bat * p.p_sb;
+    const elem *qb = reinterpret_cast<const elem *>(p.q) + (int64_t)bat * p.q_sb;
     const uint32_t i0 = tile_m * BM, j0 = tile_n * BN;
 
     const uint32_t wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
@@ -267,8 +267,8 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
         lp[d].template init<RAGGED>(p.p_si, p.p_sl, min((uint32_t)BM, p.M - i0));
         lq[d].template init<RAGGED>(p.q_sj, p.q_sl, min((uint32_t)BN, p.N - j0));
     }
-    const f16 *ptile = pb + (int64_t)i0 * p.p_si + (int64_t)kbeg * p.p_sl;
-    const f16 *qtile = qb + (int64_t)j0 * p.q_sj + (int64_t)kbeg * p.q_sl;
+    const elem *ptile = pb + (int64_t)i0 * p.p_si + (int64_t)kbeg * p.p_sl;
+    const elem *qtile = qb + (int64_t)j0 * p.q_sj + (int64_t)kbeg * p.q_sl;
     const int64_t pstep = (int64_t)TK * p.p_sl, qstep = (int64_t)TK * p.q_sl;
     // One wave per SIMD: nothing hides a stall, so the loop is software-pipelined by hand.
     //   registers  : tile s+1 waits in `reg` while tile s is multiplied; MFMA fragments are
@@ -284,7 +284,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
     constexpr bool Q_FIRST = PK && !QK, ALTERNATE = PK && QK && LP::NV == LQ::NV;
     auto piece_is_q = [&](int i) { return ALTERNATE ? bool(i & 1) : (Q_FIRST ? i < LQ::NV : i >= LP::NV); };
     auto piece_v = [&](int i) { return ALTERNATE ? i / 2 : (Q_FIRST ? (i < LQ::NV ? i : i - LQ::NV) : (i < LP::NV ? i : i - LP::NV)); };
-    auto fetch_all = [&](int set, const f16 *pt, const f16 *qt) {
+    auto fetch_all = [&](int set, const elem *pt, const elem *qt) {
 #pragma unroll
         for (int i = 0; i < LP::NV + LQ::NV; ++i) {
             if (piece_is_q(i)) lq[set].fetch_piece(qt, piece_v(i));
@@ -302,7 +302,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
     }
     __syncthreads();
 
-    Pack8 a[2][TM], b[2][TN];
+    PackE a[2][TM], b[2][TN];
     // Fragment addresses.  Every slot a lane reads has the same low four bits (l32 & 15), so
     // the position of k-step kk's group inside the row is one value per kk for all fragments.
     uint32_t koff[KK];
@@ -320,7 +320,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
     };
     auto mfma_one = [&](int buf, int m) {
         const int tm = m / TN, tn = m % TN;
-        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[buf][tm].h, b[buf][tn].h, acc[tm][tn], 0, 0, 0);
+        acc[tm][tn] = mfma_32x32x16(a[buf][tm].h, b[buf][tn].h, acc[tm][tn]);
     };
     constexpr int NMFMA = TM * TN, NREAD = TM + TN, NLOAD = LP::NV + LQ::NV;
     static_assert(NREAD <= NMFMA && NLOAD <= NMFMA * (KK / 2), "the copy pieces must fit the slots of half a tile");
@@ -359,7 +359,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
         constexpr int cur = decltype(parity)::value, nxt = 1 - cur;  // = ks % 2
         constexpr int SET = DEPTH == 2 ? nxt : 0;  // register set of tile ks + 1, refilled with tile ks + 1 + DEPTH
         const uint32_t knext = min(ks + 1 + DEPTH, ksteps - 1);
-        const f16 *pnext = ptile + knext * pstep, *qnext = qtile + knext * qstep;
+        const elem *pnext = ptile + knext * pstep, *qnext = qtile + knext * qstep;
         u32x4 packed;
         // the permutes of a row-contiguous piece, one slot ahead of its store
         auto piece_pack = [&](int i) {
@@ -496,7 +496,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
             }
         return;
     }
-    f16 *db = reinterpret_cast<f16 *>(p.d) + (int64_t)bat * p.d_sb;
+    elem *db = reinterpret_cast<elem *>(p.d) + (int64_t)bat * p.d_sb;
     if (LQ::PERMUTED && p.d_sj == 1) {
         // the lane's TN tiles are TN adjacent columns of D: one 4*TN/2-byte store per row
         const uint32_t j = j0 + LQ::row_of_slot(LQ::reader_slot(wn, 0, l32));
@@ -506,8 +506,8 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
             for (int e = 0; e < 16; ++e) {
                 const uint32_t i = i0 + LP::row_of_slot(LP::reader_slot(wm, tm, 8 * (e / 4) + 4 * lk + (e % 4)));
                 if (RAGGED && (i >= p.M || j >= p.N)) continue;  // j .. j + TN - 1 are inside N together: N % 8 == 0
-                f16 *dst = db + (int64_t)i * p.d_si + j;
-                union { f16 h[TN]; uint32_t u[TN / 2]; } o, c;
+                elem *dst = db + (int64_t)i * p.d_si + j;
+                union { elem h[TN]; uint32_t u[TN / 2]; } o, c;
                 if (p.read_dst) {
 #pragma unroll
                     for (int w = 0; w < TN / 2; ++w) c.u[w] = reinterpret_cast<const uint32_t *>(dst)[w];
@@ -515,8 +515,8 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
 #pragma unroll
                 for (int tn = 0; tn < TN; ++tn) {
                     float v = p.alpha * acc[tm][tn][e];
-                    if (p.read_dst) v = p.beta * h2f(c.h[tn]) + v;
-                    o.h[tn] = f2h(v);
+                    if (p.read_dst) v = p.beta * e2f(c.h[tn]) + v;
+                    o.h[tn] = f2e(v);
                 }
 #pragma unroll
                 for (int w = 0; w < TN / 2; ++w) reinterpret_cast<uint32_t *>(dst)[w] = o.u[w];
@@ -533,24 +533,24 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
                 for (int q = 0; q < 4; ++q) {
                     const uint32_t i = i0 + wm * WM + tm * 32 + 8 * q + 4 * lk;
                     if (RAGGED && (i >= p.M || j >= p.N)) continue;
-                    f16 *dst = db + i + (int64_t)j * p.d_sj;
+                    elem *dst = db + i + (int64_t)j * p.d_sj;
                     if (RAGGED && i + 4 > p.M) {
 #pragma unroll
                         for (int r = 0; r < 3; ++r) {
                             if (i + r >= p.M) break;
                             float v = p.alpha * acc[tm][tn][4 * q + r];
-                            if (p.read_dst) v = p.beta * h2f(dst[r]) + v;
-                            dst[r] = f2h(v);
+                            if (p.read_dst) v = p.beta * e2f(dst[r]) + v;
+                            dst[r] = f2e(v);
                         }
                         continue;
                     }
-                    union { f16 h[4]; u32x2 u; } o, c;
+                    union { elem h[4]; u32x2 u; } o, c;
                     if (p.read_dst) c.u = *reinterpret_cast<const u32x2 *>(dst);
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
                         float v = p.alpha * acc[tm][tn][4 * q + r];
-                        if (p.read_dst) v = p.beta * h2f(c.h[r]) + v;
-                        o.h[r] = f2h(v);
+                        if (p.read_dst) v = p.beta * e2f(c.h[r]) + v;
+                        o.h[r] = f2e(v);
                     }
                     *reinterpret_cast<u32x2 *>(dst) = o.u;
                 }
@@ -565,10 +565,10 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
                 for (int e = 0; e < 16; ++e) {
                     const uint32_t i = i0 + LP::row_of_slot(LP::reader_slot(wm, tm, 8 * (e / 4) + 4 * lk + (e % 4)));
                     if (RAGGED && (i >= p.M || j >= p.N)) continue;
-                    f16 *dst = db + (int64_t)i * p.d_si + (int64_t)j * p.d_sj;
+                    elem *dst = db + (int64_t)i * p.d_si + (int64_t)j * p.d_sj;
                     float v = p.alpha * acc[tm][tn][e];
-                    if (p.read_dst) v = p.beta * h2f(*dst) + v;
-                    *dst = f2h(v);
+                    if (p.read_dst) v = p.beta * e2f(*dst) + v;
+                    *dst = f2e(v);
                 }
             }
     }

@@ -1,4 +1,4 @@
-"""bf16 data on rms_norm, layer_norm, add and add_rows, through the C ABI.
+"""bf16 data on rms_norm, layer_norm, add, add_rows and (further down) mat_mul, through the C ABI.
 
 The reference's CUDA backend compiles these four for any pair of named types, bf16 included (handle/cuda/mod.rs:188-210
 with rms_norm/cuda/mod.rs:146-147, layer_norm/cuda/mod.rs:158-159, add/cuda/mod.rs:105-123, add_rows/cuda/mod.rs:135-163);
@@ -177,3 +177,110 @@ def test_bf16_still_refused_where_no_backend_of_the_reference_takes_it(gpu, stre
     with pytest.raises(ophip.SchemeError) as e:
         ophip.FusedSoftmax(gpu).scheme(ophip.FusedSoftmaxArgs(ophip.AttnMask.CAUSAL, c(1, 4, 4), None), 0)
     assert e.value.kind == "TypeNotSupport"
+
+
+# --------------------------------------------------------------- mat_mul ----
+# Neither backend of the reference multiplies bf16 (mat_mul/cuda/mod.rs:73 checks for F16, the CPU backend lists f16, f32,
+# f64): parity unpinned.  The kernels are the f16 kernels compiled on bf16 elements; what is checked is the product in f64
+# within one bf16 step of the result plus the f32 accumulation's share, and -- on operands whose products and sums are
+# exact in f32 -- every bit of the result, beside the f16 build on the same numbers.
+
+def layout_of_view(dtype, view):
+    """Layout of a numpy view over 2-byte elements, with the given element type."""
+    return TensorLayout(dtype, list(view.shape), list(view.strides))
+
+
+def base_ptr(mem, view, buf):
+    return mem.ptr + (view.__array_interface__["data"][0] - buf.__array_interface__["data"][0])
+
+
+def run_mm_bits(gpu, stream, dtype, cv, cbuf, av, abuf, bv, bbuf, alpha, beta, op=None):
+    ad, bd, cd = gpu.from_host(abuf), gpu.from_host(bbuf), gpu.from_host(cbuf)
+    op = op or ophip.MatMul(gpu)
+    args = ophip.MatMulArgs(layout_of_view(dtype, cv), base_ptr(cd, cv, cbuf), beta, layout_of_view(dtype, av), base_ptr(ad, av, abuf),
+                            layout_of_view(dtype, bv), base_ptr(bd, bv, bbuf), alpha)
+    what = op.describe(args)
+    ws = gpu.malloc(max(op.scheme(args, 1 << 40), 16))
+    op.launch(args, ws, stream)
+    out = gpu.to_host(cd, u16, cbuf.size, stream=stream).reshape(cbuf.shape)
+    return out, what
+
+
+def views(bt, m, n, k, ta, tb, tc, rng, scale_b=0.05):
+    a = to_bf16(rng.standard_normal((bt, k, m) if ta else (bt, m, k)).astype(f32) * f32(0.5))
+    b = to_bf16(rng.standard_normal((bt, n, k) if tb else (bt, k, n)).astype(f32) * f32(scale_b))
+    c = to_bf16(rng.standard_normal((bt, n, m) if tc else (bt, m, n)).astype(f32))
+    return (a.transpose(0, 2, 1) if ta else a, a), (b.transpose(0, 2, 1) if tb else b, b), (c.transpose(0, 2, 1) if tc else c, c)
+
+
+def check_bf16_product(out_view, c0, av, bv, alpha, beta, what):
+    alpha_r, beta_r = from_bf16(to_bf16(np.array([alpha, beta], f32))).astype(f64)
+    prod = np.matmul(from_bf16(av).astype(f64), from_bf16(bv).astype(f64))
+    ref = alpha_r * prod + (beta_r * from_bf16(c0).astype(f64) if beta != 0 else 0.0)
+    y = from_bf16(out_view).astype(f64)
+    k = av.shape[-1]
+    # one bf16 step of the result, and the f32 accumulation (k terms of the size of the row's and column's norms)
+    norm = np.sqrt(np.matmul(from_bf16(av).astype(f64) ** 2, from_bf16(bv).astype(f64) ** 2))
+    tol = np.abs(ref) * 2.0 ** -7 + norm * abs(alpha_r) * np.sqrt(k) * 2.0 ** -22 + 1e-30
+    bad = np.abs(y - ref) > tol
+    assert not bad.any(), "%s: %d of %d off, worst %g" % (what, bad.sum(), bad.size, (np.abs(y - ref) / tol).max())
+
+
+@pytest.mark.parametrize("ta", [False, True])
+@pytest.mark.parametrize("tb", [False, True])
+@pytest.mark.parametrize("tc", [False, True])
+@pytest.mark.parametrize("m,n,k,bt", [(16, 256, 512, 3), (40, 136, 72, 2), (3, 5, 7, 2), (130, 70, 33, 1), (256, 512, 96, 2), (128, 384, 64, 1),
+                                      (512, 768, 192, 1), (509, 1536, 1024, 1)])
+def test_mat_mul_bf16_all_layouts(gpu, stream, ta, tb, tc, m, n, k, bt):
+    rng = np.random.default_rng(m + n + k + 4 * ta + 2 * tb + tc)
+    (av, a), (bv, b), (cv, c) = views(bt, m, n, k, ta, tb, tc, rng, scale_b=1.0 / np.sqrt(k))
+    say("mat_mul bf16 ta=%s tb=%s tc=%s %dx%dx%d x%d" % (ta, tb, tc, m, n, k, bt))
+    out, what = run_mm_bits(gpu, stream, dt.BF16, cv, c, av, a, bv, b, 0.75, 0.5)
+    ov = out.transpose(0, 2, 1) if tc else out
+    check_bf16_product(ov, cv, av, bv, 0.75, 0.5, "mat_mul bf16 " + what)
+
+
+@pytest.mark.parametrize("name,bt,m,n,k,tb", [("qkv", 1, 16, 12288, 4096, False), ("qk_t", 32, 16, 2048, 128, True), ("pv", 32, 16, 128, 2048, False),
+                                              ("o_proj", 1, 16, 4096, 4096, False), ("gate_up", 1, 16, 22016, 4096, False),
+                                              ("down", 1, 16, 4096, 11008, False), ("down [N,K]", 1, 16, 4096, 11008, True),
+                                              ("prefill", 1, 512, 4096, 4096, False), ("square", 1, 1024, 1024, 1024, True)])
+def test_mat_mul_bf16_decode_layer_shapes(gpu, stream, name, bt, m, n, k, tb):
+    rng = np.random.default_rng(bt + m + n + k)
+    (av, a), (bv, b), (cv, c) = views(bt, m, n, k, False, tb, False, rng, scale_b=0.02)
+    say("mat_mul bf16 %s" % name)
+    out, what = run_mm_bits(gpu, stream, dt.BF16, cv, c, av, a, bv, b, 1.0, 0.0)
+    say("  " + what)
+    assert "generic" not in what
+    check_bf16_product(out, cv, av, bv, 1.0, 0.0, "mat_mul bf16 %s (%s)" % (name, what))
+
+
+@pytest.mark.parametrize("m,n,k,tb", [(16, 4096, 4096, False), (16, 1024, 4096, True), (48, 512, 2048, False), (256, 256, 4096, False),
+                                      (384, 640, 1024, True), (100, 72, 520, False)])
+def test_mat_mul_bf16_and_f16_builds_give_every_bit_on_exact_sums(gpu, stream, m, n, k, tb):
+    """Operands k / 16 with |k| <= 32 are f16 and bf16 numbers alike, their products and any sum of up to 4096 of them are
+    exact in f32 in any order: both builds must return the correctly rounded exact result in their type."""
+    rng = np.random.default_rng(m + n + k)
+    ai = rng.integers(-32, 33, (1, m, k))
+    bi = rng.integers(-32, 33, (1, n, k) if tb else (1, k, n))
+    exact = np.matmul(ai, bi.transpose(0, 2, 1) if tb else bi).astype(f64) / 256.0
+    assert np.abs(exact).max() * 256 < 2 ** 24
+    for dtype, enc, dec in ((dt.BF16, to_bf16, from_bf16), (dt.F16, lambda x: x.astype(np.float16).view(u16), lambda u: u.view(np.float16).astype(f32))):
+        a, b = enc((ai / 16.0).astype(f32)), enc((bi / 16.0).astype(f32))
+        c = np.zeros((1, m, n), u16)
+        bv = b.transpose(0, 2, 1) if tb else b
+        say("mat_mul exact sums %s %dx%dx%d" % ("bf16" if dtype == dt.BF16 else "f16", m, n, k))
+        out, what = run_mm_bits(gpu, stream, dtype, c, c, a, a, bv, b, 1.0, 0.0)
+        assert "generic" not in what or (k % 8)
+        assert np.array_equal(out, enc(exact.astype(f32))), what
+
+
+def test_mat_mul_bf16_scalars_round_to_bf16_and_beta_zero_never_reads_c(gpu, stream):
+    rng = np.random.default_rng(9)
+    (av, a), (bv, b), (cv, c) = views(1, 16, 256, 512, False, False, False, rng)
+    nan = np.full(c.shape, 0x7FC0, u16)
+    out, _ = run_mm_bits(gpu, stream, dt.BF16, nan, nan, av, a, bv, b, 1.0, 0.0)
+    assert not np.isnan(from_bf16(out)).any()
+    # alpha = 1 + 2^-9 rounds to 1 in bf16 (1 + 2^-8 is the tie, which goes to even: also 1)
+    out1, _ = run_mm_bits(gpu, stream, dt.BF16, cv, c, av, a, bv, b, 1.0, 0.0)
+    out2, _ = run_mm_bits(gpu, stream, dt.BF16, cv, c, av, a, bv, b, 1.0 + 2.0 ** -9, 0.0)
+    assert np.array_equal(out1, out2)

@@ -1218,8 +1218,8 @@ def test_mat_mul_errors(gpu, stream):
                                    L(dt.F16, [3, 7], [14, 2]), None, 1.0), None, stream)
     assert e.value.kind == "ShapeMismatch"
     with pytest.raises(ophip.LaunchError) as e:
-        op.launch(ophip.MatMulArgs(L(dt.BF16, [5, 7], [14, 2]), None, 0.0, L(dt.BF16, [5, 3], [6, 2]), None,
-                                   L(dt.BF16, [3, 7], [14, 2]), None, 1.0), None, stream)
+        op.launch(ophip.MatMulArgs(L(dt.U16, [5, 7], [14, 2]), None, 0.0, L(dt.U16, [5, 3], [6, 2]), None,
+                                   L(dt.U16, [3, 7], [14, 2]), None, 1.0), None, stream)
     assert e.value.kind == "TypeNotSupport"
     with pytest.raises(ophip.LaunchError) as e:
         op.launch(ophip.MatMulArgs(L(dt.F16, [5, None], [14, 2]), None, 0.0, L(dt.F16, [5, 3], [6, 2]), None,
