@@ -444,8 +444,6 @@ def mat_mul_lines(o, gpu, stream, rng, add, launches=0):
               (509, 12288, 4096, False), (4000, 4000, 4096, False), (8192, 8192, 8192, True, dt.BF16)]
     for m, n, k, b_nk, *et in shapes:
         et = et[0] if et else dt.F16
-        if launches and et != dt.F16:
-            continue  # (the bf16 build's kernels carry the f16 build's names: a counter run would mix the two)
         # (bf16: the top halves of f32 normals, which are bf16 normals of the same spread)
         mk = normal_f16 if et == dt.F16 else lambda r, sh, std: np.ascontiguousarray(
             (r.standard_normal(sh, dtype=np.float32) * np.float32(std)).view(np.uint32) >> 16).astype(np.uint16)

@@ -393,20 +393,20 @@ struct ophip_mat_mul {
         ophip_device_retain(d);
         static const int mts[3] = {1, 2, 4};
         for (int e = 0; e < 2; ++e) {
-            const char *gemm = e ? "gemm_bf16" : "gemm", *gemm_tile = e ? "gemm_tile_bf16" : "gemm_tile";
+            const char *gemm = e ? "gemm_bf16" : "gemm", *gemm_tile = e ? "gemm_tile_bf16" : "gemm_tile", *tag = e ? "_bf16" : "";
             for (int i = 0; i < 3; ++i)
                 for (int q = 0; q < 4; ++q)
                     skinny[e][i][q] = d->kernel(
-                        gemm, ("gemm_skinny_m" + std::to_string(mts[i]) + "_q" + (q == 3 ? "0p" : std::to_string(q))).c_str());
+                        gemm, ("gemm_skinny_m" + std::to_string(mts[i]) + "_q" + (q == 3 ? "0p" : std::to_string(q)) + tag).c_str());
             for (int b = 0; b < 3; ++b)
                 for (int r = 0; r < 2; ++r)
                     for (int pk = 0; pk < 2; ++pk)
                         for (int qk = 0; qk < 2; ++qk) {
                             const std::string sz = b == 0 ? "256x256" : b == 1 ? "128x128" : "128x128k32";
                             tile[e][b][r][pk][qk] = d->kernel(gemm_tile, ("gemm_tile_" + sz + (r ? "r" : "") + "_p" + std::to_string(pk) +
-                                                                          "_q" + std::to_string(qk)).c_str());
+                                                                          "_q" + std::to_string(qk) + tag).c_str());
                         }
-            reduce[e] = d->kernel(gemm, "gemm_splitk_reduce");
+            reduce[e] = d->kernel(gemm, (std::string("gemm_splitk_reduce") + tag).c_str());
         }
         fill = d->kernel("gemm", "gemm_fill_u32");
         d->make_current();

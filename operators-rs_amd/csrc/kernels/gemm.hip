@@ -504,14 +504,14 @@ __device__ __forceinline__ void gemm_skinny(const GemmParams &p) {
 }
 
 #define GEMM_SKINNY(MT, QMODE)                                                                   \
-    extern "C" __global__ void __launch_bounds__(256) gemm_skinny_m##MT##_q##QMODE(GemmParams p) { \
+    extern "C" __global__ void __launch_bounds__(256) GEMM_KERNEL(gemm_skinny_m##MT##_q##QMODE)(GemmParams p) { \
         gemm_skinny<MT, QMODE, false>(p);                                                        \
     }
 // `q0p`: K-steps dealt to the waves in pairs.  For a split whose steps come in whole groups of 8 (two per
 // wave) and are many: with an odd number of pairs per wave the longest wave decides, and on short K ranges
 // (split 8 of K = 4096) the plain dealing is 3 % faster.
 #define GEMM_SKINNY_PAIRED(MT)                                                                   \
-    extern "C" __global__ void __launch_bounds__(256) gemm_skinny_m##MT##_q0p(GemmParams p) {    \
+    extern "C" __global__ void __launch_bounds__(256) GEMM_KERNEL(gemm_skinny_m##MT##_q0p)(GemmParams p) {    \
         gemm_skinny<MT, 0, true>(p);                                                             \
     }
 GEMM_SKINNY_PAIRED(1)
@@ -528,7 +528,7 @@ GEMM_SKINNY(2, 2)
 GEMM_SKINNY(4, 2)
 
 // One thread per (batch, row, 8 columns): partial sums in ascending split order.
-extern "C" __global__ void __launch_bounds__(256) gemm_splitk_reduce(GemmParams p) {
+extern "C" __global__ void __launch_bounds__(256) GEMM_KERNEL(gemm_splitk_reduce)(GemmParams p) {
     const uint32_t nvec = p.N / 8;
     const size_t total = (size_t)p.batch * p.M * nvec;
     const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;

@@ -1,6 +1,6 @@
 // Element type of the MFMA GEMM kernels.  gemm.hip and gemm_tile.hip are compiled twice: as they stand, on f16 elements
 // (modules `gemm`, `gemm_tile`), and with -DGEMM_ELEM_BF16 on bf16 elements (modules `gemm_bf16`, `gemm_tile_bf16`,
-// same kernel names).  The kernels move elements as 16-bit words, so the type matters in three places only: the MFMA
+// kernel names with `_bf16` appended, so that a trace tells the two apart).  The kernels move elements as 16-bit words, so the type matters in three places only: the MFMA
 // instruction, and the two conversions of the epilogue (f32 -> element rounds to nearest even in both types).
 #pragma once
 #include <type_traits>
@@ -9,8 +9,10 @@
 
 #ifdef GEMM_ELEM_BF16
 typedef bf16 elem;
+#define GEMM_KERNEL(name) name##_bf16
 #else
 typedef f16 elem;
+#define GEMM_KERNEL(name) name
 #endif
 typedef elem elem8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));

@@ -578,10 +578,10 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
 // (One build with the guards switched by a kernel argument runs the whole-tile shapes 3 - 4 % slower:
 // the guards change the register allocation of the main loop.)
 #define GEMM_TILE(NAME, BM, BN, PK, QK, TK, DEPTH)                                                    \
-    extern "C" __global__ void __launch_bounds__(256) gemm_tile_##NAME##_p##PK##_q##QK(GemmParams p) {    \
+    extern "C" __global__ void __launch_bounds__(256) GEMM_KERNEL(gemm_tile_##NAME##_p##PK##_q##QK)(GemmParams p) {    \
         gemm_tile<BM, BN, PK, QK, TK, DEPTH, false>(p);                                               \
     }                                                                                                 \
-    extern "C" __global__ void __launch_bounds__(256) gemm_tile_##NAME##r_p##PK##_q##QK(GemmParams p) {   \
+    extern "C" __global__ void __launch_bounds__(256) GEMM_KERNEL(gemm_tile_##NAME##r_p##PK##_q##QK)(GemmParams p) {   \
         gemm_tile<BM, BN, PK, QK, TK, DEPTH, true>(p);                                                \
     }
 
