@@ -218,14 +218,14 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p) {
 
     // XCD-aware tile order: ids are dealt round-robin over 8 XCDs; give each XCD a
     // contiguous run of tiles, walked in groups of 8 tile-rows so panels are reused.
+    // (XCD x receives the ids x, x + 8, ...: one more than tiles / 8 of them when x < tiles % 8.)
     const uint32_t tiles_m = RAGGED ? (p.M + BM - 1) / BM : p.M / BM, tiles_n = RAGGED ? (p.N + BN - 1) / BN : p.N / BN;
     const uint32_t tiles = tiles_m * tiles_n;
     uint32_t id = blockIdx.x;
     {
-        const uint32_t per_xcd = (tiles + 7) / 8;
+        const uint32_t q8 = tiles / 8, r8 = tiles % 8;
         const uint32_t xcd = id % 8, local = id / 8;
-        const uint32_t lin = xcd * per_xcd + local;
-        id = (tiles % 8 == 0) ? lin : blockIdx.x;  // only remap when the tiles split evenly
+        id = xcd < r8 ? xcd * (q8 + 1) + local : r8 * (q8 + 1) + (xcd - r8) * q8 + local;
     }
     constexpr uint32_t GROUP = 8;
     const uint32_t group_size = GROUP * tiles_n;
