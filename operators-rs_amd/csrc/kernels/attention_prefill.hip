@@ -1,0 +1,193 @@
+// attention in one pass for prefill shapes (many query rows per head): o = softmax(q . k^T / sqrt(dh), causal) . v
+// with the [nh, seq, att] score matrix never leaving the chip.
+//
+// The reference builds the operator from up to five launches (attention/operator.rs:143-277: q . k^T into a workspace,
+// softmax over it, att . v, copies), and at prefill shapes the score matrix is most of the memory traffic: 268 MB
+// written, read, written and read again for 32 heads of 2048 x 2048.  Here a workgroup of four waves owns 128 query rows
+// of one head, a wave 32 of them, and walks the keys in tiles of 64 with the running maximum and sum of the rows
+// (the usual online softmax):
+//
+//   * K and V tiles (64 keys x dh) go from global memory through registers into LDS, double-buffered; the next tile's
+//     loads are in flight while the current one is multiplied.  One barrier per tile.
+//   * Scores are computed transposed, S^T = K . Q^T with v_mfma_f32_32x32x16_f16: A operands are key rows read from LDS
+//     16 bytes per lane, B operands the wave's 32 query rows, which stay in registers for the whole kernel.  In the
+//     result a lane holds ONE query (lane % 32) and 32 of the tile's 64 keys, so the row maximum and sum are sums over
+//     the lane's own registers plus one exchange with lane ^ 32, and every per-row factor is a per-lane scalar.
+//   * The probabilities (f16) are packed straight from that result layout into B operands of the second product,
+//     O^T = V^T . P^T: which of a lane's keys go to which contraction slot is free as long as V^T uses the same order,
+//     and V^T fragments come from the row-major V tile through the transposing LDS read (ds_read_b64_tr_b16): a lane
+//     gets four consecutive keys of one dh column per read.  No transposition in registers, no LDS round trip for P.
+//   * Causal mask: row i keeps keys <= att - seq + i; tiles beyond the block's last row are never visited.  Blocks are
+//     launched last-block-first (the longest first), heads along grid x so that the blocks of a head meet in one XCD's L2.
+//
+// Results agree with the composite within the f16 bar (scores and probabilities are not rounded to f16 in between;
+// the scale is rounded to f16 as the reference's mat_mul rounds alpha).
+#include "device_util.h"
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int AP_BM = 128, AP_BN = 64;
+
+template <int DH>
+__device__ __forceinline__ void attn_prefill(const AttnPrefillParams &p) {
+    constexpr int KP = DH + 8;        // halves per K row in LDS: an odd number of 16-byte units, so 16-byte reads of consecutive rows spread
+    constexpr int VP = DH + 32;       // halves per V row in LDS: 64 bytes past a multiple of 256, so four consecutive rows cover all banks
+    constexpr int CPR = DH / 8;       // 16-byte chunks per row
+    constexpr int NCH = AP_BN * CPR / 256;  // chunks per thread and tile
+    constexpr int DS = DH / 16, DB = DH / 32;
+    __shared__ __attribute__((aligned(16))) f16 k_lds[2][AP_BN * KP];
+    __shared__ __attribute__((aligned(16))) f16 v_lds[2][AP_BN * VP];
+
+    const uint32_t tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+    const uint32_t n32 = lane % 32, h = lane / 32, s16 = lane % 16, b16 = (lane / 16) % 2;
+    const uint32_t head = blockIdx.x, qblock = p.nblocks - 1 - blockIdx.y;
+    const uint32_t kvh = head / p.group;
+    const uint32_t i0 = qblock * AP_BM;
+    const uint32_t row = i0 + wave * 32 + n32, rowc = min(row, p.seq - 1);
+
+    const f16 *qb = reinterpret_cast<const f16 *>(p.q) + (int64_t)head * p.q_sh;
+    const f16 *kb = reinterpret_cast<const f16 *>(p.k) + (int64_t)kvh * p.k_sh;
+    const f16 *vb = reinterpret_cast<const f16 *>(p.v) + (int64_t)kvh * p.v_sh;
+
+    // the wave's queries as B operands: lane (n32, h) holds query row n32, dh slots 16 ds + 8 h .. + 7
+    Pack8 qf[DS];
+#pragma unroll
+    for (int ds = 0; ds < DS; ++ds) qf[ds].u = ld128(qb + (int64_t)rowc * p.q_ss + 16 * ds + 8 * h);
+
+    // keys this block needs: up to the last row's limit
+    const uint32_t last_row = min(i0 + AP_BM, p.seq) - 1;
+    const uint32_t keys = p.causal ? min(p.att, p.att - p.seq + last_row + 1) : p.att;
+    const uint32_t ntiles = (keys + AP_BN - 1) / AP_BN;
+    // the last key this lane's row keeps
+    const int32_t lim = p.causal ? (int32_t)(p.att - p.seq + rowc) : (int32_t)p.att - 1;
+
+    u32x4 kreg[NCH], vreg[NCH];
+    auto fetch = [&](uint32_t t) {
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const uint32_t c = tid + 256 * i, r = c / CPR, cc = c % CPR;
+            const uint32_t key = min(t * AP_BN + r, p.att - 1);
+            kreg[i] = ld128(kb + (int64_t)key * p.k_ss + 8 * cc);
+            vreg[i] = ld128(vb + (int64_t)key * p.v_ss + 8 * cc);
+        }
+    };
+    auto commit = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const uint32_t c = tid + 256 * i, r = c / CPR, cc = c % CPR;
+            st128(&k_lds[buf][r * KP + 8 * cc], kreg[i]);
+            st128(&v_lds[buf][r * VP + 8 * cc], vreg[i]);
+        }
+    };
+
+    f32x16 oacc[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) oacc[db][e] = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;
+    constexpr float LOG2E = 1.4426950408889634f;
+    const float sc2 = p.scale * LOG2E;  // scores in units of log2
+
+    fetch(0);
+    commit(0);
+    __syncthreads();
+    for (uint32_t t = 0; t < ntiles; ++t) {
+        const int buf = t & 1;
+        if (t + 1 < ntiles) fetch(t + 1);
+
+        // S^T = K . Q^T: sacc[kb][e] is key 32 kb + 8 (e / 4) + 4 h + e % 4 of the tile, query n32
+        f32x16 sacc[2];
+#pragma unroll
+        for (int kb2 = 0; kb2 < 2; ++kb2) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) sacc[kb2][e] = 0.f;
+#pragma unroll
+            for (int ds = 0; ds < DS; ++ds) {
+                Pack8 a;
+                a.u = ld128(&k_lds[buf][(32 * kb2 + n32) * KP + 16 * ds + 8 * h]);
+                sacc[kb2] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a.h, qf[ds].h, sacc[kb2], 0, 0, 0);
+            }
+        }
+        // scale, mask, the tile's maximum for this lane's query
+        float mx = -INFINITY;
+#pragma unroll
+        for (int kb2 = 0; kb2 < 2; ++kb2)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int32_t key = (int32_t)(t * AP_BN) + 32 * kb2 + 8 * (e / 4) + 4 * (int32_t)h + (e % 4);
+                const float s = key <= lim ? sacc[kb2][e] * sc2 : -INFINITY;
+                sacc[kb2][e] = s;
+                mx = fmaxf(mx, s);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+        const float m_new = fmaxf(m_run, mx);
+        const float m_ref = m_new == -INFINITY ? 0.f : m_new;  // (a row with nothing kept so far: every term below is 0)
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
+        m_run = m_new;
+        float psum = 0.f;
+        // probabilities, packed for the second product: MFMA j covers the tile's keys 16 j .. 16 j + 15; the lane's eight
+        // contraction slots 8 h .. 8 h + 7 hold keys 16 j + 4 h + {0..3} and 16 j + 8 + 4 h + {0..3}
+        Pack8 pb[4];
+#pragma unroll
+        for (int kb2 = 0; kb2 < 2; ++kb2)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const float pr = __builtin_amdgcn_exp2f(sacc[kb2][e] - m_ref);
+                psum += pr;
+                pb[2 * kb2 + e / 8].e[e % 8] = f2h(pr);
+            }
+        l_run = l_run * alpha + psum;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) oacc[db][e] *= alpha;
+
+        // O^T += V^T . P^T: the A operand's row is dh column 32 db + lane % 32; a transposing read hands a lane four
+        // consecutive keys of that column (the lanes of a 16-lane group address key s16 / 4, columns 4 (s16 % 4) .. + 3)
+        typedef __attribute__((address_space(3))) s16x4 *lds_s16x4;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const f16 *src = &v_lds[buf][(16 * j + 4 * h + s16 / 4) * VP + 32 * db + 16 * b16 + 4 * (s16 % 4)];
+                union {
+                    s16x4 q[2];
+                    f16x8 hv;
+                } a;
+                a.q[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4)src);
+                a.q[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4)(src + 8 * VP));
+                oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a.hv, pb[j].h, oacc[db], 0, 0, 0);
+            }
+
+        if (t + 1 < ntiles) commit(buf ^ 1);
+        __syncthreads();
+    }
+
+    // o = O^T / l: the lane holds, for its query, columns 32 db + 8 (e / 4) + 4 h + e % 4: four adjacent ones per e / 4
+    const float l_tot = l_run + __shfl_xor(l_run, 32, WAVE);
+    const float inv = 1.0f / l_tot;
+    if (row < p.seq) {
+        f16 *orow = reinterpret_cast<f16 *>(p.o) + (int64_t)head * p.o_sh + (int64_t)row * p.o_ss;
+        f16 *qrow = p.q_out ? reinterpret_cast<f16 *>(p.q_out) + (int64_t)head * p.q_sh + (int64_t)row * p.q_ss : nullptr;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                union {
+                    f16 e[4];
+                    u32x2 u;
+                } o;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) o.e[r] = f2h(oacc[db][4 * g + r] * inv);
+                const uint32_t col = 32 * db + 8 * g + 4 * h;
+                *reinterpret_cast<u32x2 *>(orow + col) = o.u;
+                if (qrow) *reinterpret_cast<u32x2 *>(qrow + col) = o.u;
+            }
+    }
+}
+
+// (two waves per SIMD: two workgroups per CU, one multiplying while the other does its exponentials)
+extern "C" __global__ void __launch_bounds__(256, 2) attn_prefill_d128(AttnPrefillParams p) { attn_prefill<128>(p); }
+extern "C" __global__ void __launch_bounds__(256, 2) attn_prefill_d64(AttnPrefillParams p) { attn_prefill<64>(p); }

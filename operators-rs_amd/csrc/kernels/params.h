@@ -94,6 +94,17 @@ struct AttnDecodeParams {
     float scale;
 };
 
+// attention in one pass for prefill shapes (attention_prefill.hip).  Strides in elements; dh is contiguous everywhere.
+struct AttnPrefillParams {
+    const void *q;
+    void *q_out;  // q again when the reference would overwrite it with the result (its heads and tokens merge), else null
+    void *o;
+    const void *k, *v;
+    int64_t q_sh, q_ss, o_sh, o_ss, k_sh, k_ss, v_sh, v_ss;
+    uint32_t nh, group, seq, att, causal, nblocks;
+    float scale;
+};
+
 struct ProbeParams {  // probe.hip
     void *dst;
     const void *src;

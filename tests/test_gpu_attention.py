@@ -274,3 +274,103 @@ def test_decode_layer_chain_matches_the_oracle_end_to_end(gpu, stream):
     print("decode layer: max err %.3g, median err %.3g, output scale %.3g" % (err.max(), np.median(err), scale), flush=True)
     assert err.max() <= 1e-2 * scale, err.max() / scale
     assert np.median(err) <= 1e-3 * scale, np.median(err) / scale
+
+
+# ------------------------------------------------ one pass, prefill shapes ----
+# From 64 query rows per head on, attention runs on one kernel that keeps the scores on the chip (attention_prefill.hip).
+# Same bar as the composite: the oracle's composite and the f64 formula, within the f16 tolerance.
+
+def run_attention(gpu, stream, q, k, v, mask, op=None):
+    qd, kd, vd = upload(gpu, q), upload(gpu, k), upload(gpu, v)
+    od = gpu.malloc(q.nbytes)
+    gpu.memset(od, 0xFF)
+    op = op or ophip.Attention(gpu)
+    lay = TensorLayout.of
+    args = ophip.AttentionArgs(lay(q), qd, lay(k), kd, lay(v), vd, lay(q), od, mask)
+    op.launch(args, None, stream)
+    return download(gpu, stream, od, q), download(gpu, stream, qd, q)
+
+
+@pytest.mark.parametrize("nh,nkvh,seq,att,dh,mask", [(4, 4, 128, 128, 128, CAUSAL), (2, 1, 64, 64, 128, NONE), (8, 2, 256, 256, 64, CAUSAL),
+                                                     (3, 1, 130, 257, 128, CAUSAL), (3, 3, 65, 64 + 65, 64, CAUSAL),
+                                                     (4, 2, 1000, 1000, 64, CAUSAL), (2, 2, 300, 77, 128, NONE),
+                                                     (32, 32, 512, 512, 128, CAUSAL), (8, 8, 1024, 1536, 128, CAUSAL)])
+def test_attention_one_pass_prefill(gpu, stream, nh, nkvh, seq, att, dh, mask):
+    rng = np.random.default_rng(nh + seq + att + dh)
+    q, k, v = normal_f16(rng, (nh, seq, dh)), normal_f16(rng, (nkvh, att, dh)), normal_f16(rng, (nkvh, att, dh))
+    say("attention one pass nh=%d nkvh=%d seq=%d att=%d dh=%d mask=%d" % (nh, nkvh, seq, att, dh, mask))
+    out, q_after = run_attention(gpu, stream, q, k, v, mask)
+    assert_close_f16(out, attention_f64(q, k, v, mask == CAUSAL), "one pass vs f64")
+    oracle.set_threads(8)
+    try:
+        ref = oracle.attention(q.copy(), k, v, np.zeros_like(q), causal=(mask == CAUSAL))
+    finally:
+        oracle.set_threads(1)
+    assert_close_f16(out, ref, "one pass vs oracle")
+    assert np.array_equal(q_after, out)  # contiguous q: heads and tokens merge, q receives att . v as in the reference
+    again, _ = run_attention(gpu, stream, q, k, v, mask)
+    assert np.array_equal(again, out)  # the same bits on every launch
+
+
+@pytest.mark.parametrize("nh,nkvh,seq,att,dh,mask", [(32, 4, 7, 127, 64, CAUSAL), (5, 5, 1, 9, 64, CAUSAL), (6, 2, 40, 40, 128, NONE),
+                                                     (8, 8, 33, 33, 128, CAUSAL)])
+def test_attention_one_pass_forced_on_few_rows_agrees_with_the_composite(gpu, stream, monkeypatch, nh, nkvh, seq, att, dh, mask):
+    rng = np.random.default_rng(nh + seq + att)
+    q, k, v = normal_f16(rng, (nh, seq, dh)), normal_f16(rng, (nkvh, att, dh)), normal_f16(rng, (nkvh, att, dh))
+    monkeypatch.setenv("OPHIP_ATTN_FUSED", "1")
+    fused = ophip.Attention(gpu)
+    monkeypatch.setenv("OPHIP_ATTN_FUSED", "0")
+    composite = ophip.Attention(gpu)
+    say("attention one pass forced nh=%d seq=%d att=%d" % (nh, seq, att))
+    a, qa = run_attention(gpu, stream, q, k, v, mask, op=fused)
+    b, qb = run_attention(gpu, stream, q, k, v, mask, op=composite)
+    ref = attention_f64(q, k, v, mask == CAUSAL)
+    assert_close_f16(a, ref, "one pass")
+    assert_close_f16(b, ref, "composite")
+    assert np.array_equal(qa, a) and np.array_equal(qb, b)
+
+
+def test_attention_one_pass_on_views_of_a_fused_qkv_buffer(gpu, stream):
+    """q, k, v are column slices of one [seq, 3 * nh * dh] buffer viewed head-major, o is token-major: heads and tokens
+    of q do not merge, so q is left alone (the reference works on a copy of it)."""
+    rng = np.random.default_rng(21)
+    seq, nh, dh = 300, 8, 128
+    qkv = normal_f16(rng, (seq, 3 * nh * dh))
+    obuf = np.zeros((seq, nh * dh), f16)
+    qkv_d, od = upload(gpu, qkv), upload(gpu, obuf)
+    row = 3 * nh * dh * 2
+    lay = lambda: TensorLayout(dt.F16, [nh, seq, dh], [dh * 2, row, 2])
+    o_lay = TensorLayout(dt.F16, [nh, seq, dh], [dh * 2, nh * dh * 2, 2])
+    op = ophip.Attention(gpu)
+    args = ophip.AttentionArgs(lay(), qkv_d.ptr, lay(), qkv_d.ptr + nh * dh * 2, lay(), qkv_d.ptr + 2 * nh * dh * 2, o_lay, od, CAUSAL)
+    say("attention one pass, views of a fused QKV buffer")
+    op.launch(args, None, stream)
+    out = download(gpu, stream, od, obuf).reshape(seq, nh, dh).transpose(1, 0, 2)
+    view = lambda i: qkv[:, i * nh * dh:(i + 1) * nh * dh].reshape(seq, nh, dh).transpose(1, 0, 2)
+    assert_close_f16(out, attention_f64(view(0), view(1), view(2), True), "one pass on views")
+    assert np.array_equal(download(gpu, stream, qkv_d, qkv), qkv)
+
+
+def test_attention_one_pass_with_o_in_place_of_q(gpu, stream):
+    rng = np.random.default_rng(22)
+    nh, seq, dh = 4, 192, 64
+    q, k, v = normal_f16(rng, (nh, seq, dh)), normal_f16(rng, (nh, seq, dh)), normal_f16(rng, (nh, seq, dh))
+    qd, kd, vd = upload(gpu, q), upload(gpu, k), upload(gpu, v)
+    lay = TensorLayout.of
+    op = ophip.Attention(gpu)
+    op.launch(ophip.AttentionArgs(lay(q), qd, lay(k), kd, lay(v), vd, lay(q), qd, CAUSAL), None, stream)
+    assert_close_f16(download(gpu, stream, qd, q), attention_f64(q, k, v, True), "o = q")
+
+
+def test_attention_kv_cached_prefill_goes_through_the_one_pass_kernel(gpu, stream):
+    rng = np.random.default_rng(23)
+    op = ophip.AttnKVCached(gpu)
+    for pos, seq, strided in ((0, 256, False), (100, 200, False), (40, 128, True)):
+        say("attention_kv_cached prefill pos=%d seq=%d strided=%s" % (pos, seq, strided))
+        out, q_after, kc_out, vc_out, (q, k, v, kc, vc) = kv_cached_case(gpu, stream, op, 8, 2, seq, 128, 512, pos, CAUSAL, rng, strided)
+        kc_ref, vc_ref = kc.copy(), vc.copy()
+        ref = oracle.attention_kv_cached(q.copy(), k, v, np.zeros_like(q), kc_ref, vc_ref, pos, causal=True)
+        assert np.array_equal(kc_out, kc_ref) and np.array_equal(vc_out, vc_ref)
+        assert_close_f16(out, ref, "kv cached prefill vs oracle")
+        assert_close_f16(out, attention_f64(q, kc_ref[:, :pos + seq], vc_ref[:, :pos + seq], True), "kv cached prefill vs f64")
+        assert np.array_equal(q_after, q if strided else out)
