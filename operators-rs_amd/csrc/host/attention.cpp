@@ -3,6 +3,7 @@
 // (attention/operator.rs:1-278, attention_kv_cached/operator.rs:1-184).  They own no
 // kernels: they plan workspace, build views and launch the three operators in the
 // reference's order, so the work lands on the queue exactly as the crate would put it.
+#include <algorithm>
 #include <cmath>
 #include <cstdlib>
 
@@ -92,7 +93,9 @@ struct ophip_attention {
     ophip_mat_mul *mat_mul = nullptr;
     ophip_fused_softmax *softmax = nullptr;
     ophip_rearrange *rearrange = nullptr;
-    hipFunction_t prefill[2] = {nullptr, nullptr};  // the one-pass kernel for many query rows: dh 64 / 128
+    // the one-pass kernel for many query rows: [dh 64 / 128][4 waves on all key tiles / 8 waves, even and odd key tiles]
+    hipFunction_t prefill[2][2] = {};
+    int key_split = -1;  // OPHIP_ATTN_KEYSPLIT=0|1 keeps one of the two builds (sweeps); read once, here
     // OPHIP_ATTN_FUSED=0 keeps the composite (tests, comparisons), =1 takes the one-pass kernel wherever it applies;
     // read once, here.  Otherwise the row count decides (attention_launch).
     int fused = -1;
@@ -102,9 +105,12 @@ struct ophip_attention {
             sub(ophip_mat_mul_create(d, &mat_mul));
             sub(ophip_fused_softmax_create(d, &softmax));
             sub(ophip_rearrange_create(d, &rearrange));
-            prefill[0] = d->kernel("attention_prefill", "attn_prefill_d64");
-            prefill[1] = d->kernel("attention_prefill", "attn_prefill_d128");
+            prefill[0][0] = d->kernel("attention_prefill", "attn_prefill_d64");
+            prefill[1][0] = d->kernel("attention_prefill", "attn_prefill_d128");
+            prefill[0][1] = d->kernel("attention_prefill", "attn_prefill_d64_g2");
+            prefill[1][1] = d->kernel("attention_prefill", "attn_prefill_d128_g2");
             if (const char *e = std::getenv("OPHIP_ATTN_FUSED")) fused = std::atoi(e) != 0;
+            if (const char *e = std::getenv("OPHIP_ATTN_KEYSPLIT")) key_split = std::atoi(e) != 0;
         } catch (...) {
             release();
             throw;
@@ -190,6 +196,7 @@ bool attention_one_pass(const ophip_attention *op, const ophip_attention_args &a
         if (!t->base || !aligned16(t->base)) return false;
         const ptrdiff_t s0 = static_of(t->l.strides[0]), s1 = static_of(t->l.strides[1]), s2 = static_of(t->l.strides[2]);
         if (s2 != 2 || s0 < 0 || s1 < 0 || !mult16(s0) || !mult16(s1)) return false;
+        if (s1 >= ((ptrdiff_t)1 << 24)) return false;  // the kernel adds 32-bit byte offsets inside a tile of 64 rows
     }
     // o must not lie over anything the other workgroups still read: apart from q itself in q's own layout
     auto span = [](const View &t) {
@@ -230,7 +237,12 @@ bool attention_one_pass(const ophip_attention *op, const ophip_attention_args &a
     p.scale = round_to_f16(1.0f / std::sqrt((float)dh));  // the reference's mat_mul rounds alpha to the data type
     if (p.nblocks > 65535) return false;
     op->dev->make_current();
-    launch(op->prefill[dh == 64 ? 0 : 1], Dim3{(unsigned)nh, p.nblocks}, Dim3{256}, 0, stream_of(qa), p);
+    // Under a causal mask the block with the most keys decides once there are no more workgroups than places for
+    // them (two per CU): then the eight-wave build, whose workgroups take half as long (32 heads, causal: 2048 x 2048
+    // 67.9 against 73.1 us, 512 x 512 19.5 against 21.3; 4096 x 4096 232 against 203, and without a mask it always loses)
+    const size_t cus = (size_t)op->dev->props.multiProcessorCount;
+    const bool split = op->key_split >= 0 ? op->key_split != 0 : p.causal && nh * (size_t)p.nblocks <= 2 * cus;
+    launch(op->prefill[dh == 64 ? 0 : 1][split], Dim3{(unsigned)nh, p.nblocks}, Dim3{split ? 512u : 256u}, 0, stream_of(qa), p);
     return true;
 }
 

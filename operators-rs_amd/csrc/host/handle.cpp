@@ -256,8 +256,8 @@ int ophip_device_get_info(const ophip_device *dev, ophip_device_info *out) {
     return guard([&] {
         if (!dev || !out) throw args_not_support("null argument");
         std::memset(out, 0, sizeof(*out));
-        std::snprintf(out->name, sizeof(out->name), "%s", dev->props.name);
-        std::snprintf(out->arch, sizeof(out->arch), "%s", dev->props.gcnArchName);
+        std::snprintf(out->name, sizeof(out->name), "%.*s", (int)sizeof(out->name) - 1, dev->props.name);
+        std::snprintf(out->arch, sizeof(out->arch), "%.*s", (int)sizeof(out->arch) - 1, dev->props.gcnArchName);
         out->compute_units = dev->props.multiProcessorCount;
         out->wavefront_size = dev->props.warpSize;
         out->max_threads_per_block = dev->props.maxThreadsPerBlock;

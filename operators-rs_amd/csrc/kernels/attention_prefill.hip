@@ -29,22 +29,31 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int AP_BM = 128, AP_BN = 64;
 
-template <int DH>
+// G = 1: a workgroup of 4 waves walks all key tiles of its 128 rows; two such workgroups share a CU.
+// G = 2: a workgroup of 8 waves, two groups of 4 on the same 128 rows: group 0 takes the even key tiles, group 1 the odd
+// ones, each with its own LDS buffers and its own threads loading them; at the end group 1 hands its maxima, sums and
+// output to group 0 through LDS.  One such workgroup fills a CU.  A workgroup's time halves, which is what a causal
+// mask wants when there are about as many workgroups as places for them: the block with the most keys decides.
+template <int DH, int G>
 __device__ __forceinline__ void attn_prefill(const AttnPrefillParams &p) {
     constexpr int KP = DH + 8;        // halves per K row in LDS: an odd number of 16-byte units, so 16-byte reads of consecutive rows spread
     constexpr int VP = DH + 32;       // halves per V row in LDS: 64 bytes past a multiple of 256, so four consecutive rows cover all banks
     constexpr int CPR = DH / 8;       // 16-byte chunks per row
     constexpr int NCH = AP_BN * CPR / 256;  // chunks per thread and tile
     constexpr int DS = DH / 16, DB = DH / 32;
-    __shared__ __attribute__((aligned(16))) f16 k_lds[2][AP_BN * KP];
-    __shared__ __attribute__((aligned(16))) f16 v_lds[2][AP_BN * VP];
+    constexpr int TILE_HALVES = AP_BN * (KP + VP);
+    __shared__ __attribute__((aligned(16))) f16 lds[G * 2 * TILE_HALVES];
 
-    const uint32_t tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+    const uint32_t grp = G == 1 ? 0 : threadIdx.x / 256;
+    const uint32_t tid = threadIdx.x % 256, wave = tid / WAVE, lane = tid % WAVE;
     const uint32_t n32 = lane % 32, h = lane / 32, s16 = lane % 16, b16 = (lane / 16) % 2;
+    // blocks go out longest first (the last block of rows has the most keys under a causal mask), heads along x
     const uint32_t head = blockIdx.x, qblock = p.nblocks - 1 - blockIdx.y;
     const uint32_t kvh = head / p.group;
     const uint32_t i0 = qblock * AP_BM;
     const uint32_t row = i0 + wave * 32 + n32, rowc = min(row, p.seq - 1);
+    f16 *const k_lds = lds + grp * 2 * TILE_HALVES;          // [2][AP_BN * KP]
+    f16 *const v_lds = k_lds + 2 * AP_BN * KP;               // [2][AP_BN * VP]
 
     const f16 *qb = reinterpret_cast<const f16 *>(p.q) + (int64_t)head * p.q_sh;
     const f16 *kb = reinterpret_cast<const f16 *>(p.k) + (int64_t)kvh * p.k_sh;
@@ -61,23 +70,43 @@ __device__ __forceinline__ void attn_prefill(const AttnPrefillParams &p) {
     const uint32_t ntiles = (keys + AP_BN - 1) / AP_BN;
     // the last key this lane's row keeps
     const int32_t lim = p.causal ? (int32_t)(p.att - p.seq + rowc) : (int32_t)p.att - 1;
+    const int32_t lim_first = __builtin_amdgcn_readfirstlane(lim);  // the wave's smallest: its first row's
 
+    // The thread's chunks of a tile: byte offsets from the tile's first key (32 bits: the host checks that 64 rows of k
+    // and v span less than 2 GiB), so that a load is a uniform base plus a lane offset.  Only a last tile that reaches
+    // past att clamps its rows.
     u32x4 kreg[NCH], vreg[NCH];
-    auto fetch = [&](uint32_t t) {
+    uint32_t koff[NCH], voff[NCH];
 #pragma unroll
-        for (int i = 0; i < NCH; ++i) {
-            const uint32_t c = tid + 256 * i, r = c / CPR, cc = c % CPR;
-            const uint32_t key = min(t * AP_BN + r, p.att - 1);
-            kreg[i] = ld128(kb + (int64_t)key * p.k_ss + 8 * cc);
-            vreg[i] = ld128(vb + (int64_t)key * p.v_ss + 8 * cc);
+    for (int i = 0; i < NCH; ++i) {
+        const uint32_t c = tid + 256 * i, r = c / CPR, cc = c % CPR;
+        koff[i] = (r * (uint32_t)p.k_ss + 8 * cc) * 2;
+        voff[i] = (r * (uint32_t)p.v_ss + 8 * cc) * 2;
+    }
+    auto fetch = [&](uint32_t t) {
+        const char *kt = reinterpret_cast<const char *>(kb + (int64_t)(t * AP_BN) * p.k_ss);
+        const char *vt = reinterpret_cast<const char *>(vb + (int64_t)(t * AP_BN) * p.v_ss);
+        if (t * AP_BN + AP_BN <= p.att) {
+#pragma unroll
+            for (int i = 0; i < NCH; ++i) {
+                kreg[i] = ld128(kt + koff[i]);
+                vreg[i] = ld128(vt + voff[i]);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < NCH; ++i) {
+                const uint32_t c = tid + 256 * i, r = min(c / CPR, p.att - 1 - t * AP_BN), cc = c % CPR;
+                kreg[i] = ld128(kt + (r * (uint32_t)p.k_ss + 8 * cc) * 2);
+                vreg[i] = ld128(vt + (r * (uint32_t)p.v_ss + 8 * cc) * 2);
+            }
         }
     };
     auto commit = [&](int buf) {
 #pragma unroll
         for (int i = 0; i < NCH; ++i) {
             const uint32_t c = tid + 256 * i, r = c / CPR, cc = c % CPR;
-            st128(&k_lds[buf][r * KP + 8 * cc], kreg[i]);
-            st128(&v_lds[buf][r * VP + 8 * cc], vreg[i]);
+            st128(k_lds + buf * (AP_BN * KP) + r * KP + 8 * cc, kreg[i]);
+            st128(v_lds + buf * (AP_BN * VP) + r * VP + 8 * cc, vreg[i]);
         }
     };
 
@@ -88,85 +117,126 @@ __device__ __forceinline__ void attn_prefill(const AttnPrefillParams &p) {
         for (int e = 0; e < 16; ++e) oacc[db][e] = 0.f;
     float m_run = -INFINITY, l_run = 0.f;
     constexpr float LOG2E = 1.4426950408889634f;
-    const float sc2 = p.scale * LOG2E;  // scores in units of log2
+    const float sc2 = p.scale * LOG2E;  // scores in units of log2 (positive: maxima commute with it)
 
-    fetch(0);
-    commit(0);
+    // this group's tiles: grp, grp + G, ...  (a group without tiles still meets every barrier)
+    if (grp < ntiles) {
+        fetch(grp);
+        commit(0);
+    }
     __syncthreads();
-    for (uint32_t t = 0; t < ntiles; ++t) {
-        const int buf = t & 1;
-        if (t + 1 < ntiles) fetch(t + 1);
+    for (uint32_t u = 0; u * G < ntiles; ++u) {
+        const uint32_t t = u * G + grp;
+        const int buf = u & 1;
+        if (t < ntiles) {
+            const bool more = t + G < ntiles;
+            if (more) fetch(t + G);
+            const f16 *kt = k_lds + buf * (AP_BN * KP), *vt = v_lds + buf * (AP_BN * VP);
 
-        // S^T = K . Q^T: sacc[kb][e] is key 32 kb + 8 (e / 4) + 4 h + e % 4 of the tile, query n32
-        f32x16 sacc[2];
+            // S^T = K . Q^T: sacc[kb][e] is key 32 kb + 8 (e / 4) + 4 h + e % 4 of the tile, query n32
+            f32x16 sacc[2];
 #pragma unroll
-        for (int kb2 = 0; kb2 < 2; ++kb2) {
+            for (int kb2 = 0; kb2 < 2; ++kb2) {
 #pragma unroll
-            for (int e = 0; e < 16; ++e) sacc[kb2][e] = 0.f;
+                for (int e = 0; e < 16; ++e) sacc[kb2][e] = 0.f;
 #pragma unroll
-            for (int ds = 0; ds < DS; ++ds) {
-                Pack8 a;
-                a.u = ld128(&k_lds[buf][(32 * kb2 + n32) * KP + 16 * ds + 8 * h]);
-                sacc[kb2] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a.h, qf[ds].h, sacc[kb2], 0, 0, 0);
+                for (int ds = 0; ds < DS; ++ds) {
+                    Pack8 a;
+                    a.u = ld128(kt + (32 * kb2 + n32) * KP + 16 * ds + 8 * h);
+                    sacc[kb2] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a.h, qf[ds].h, sacc[kb2], 0, 0, 0);
+                }
             }
+            // mask (only a tile that reaches past the wave's first limit has anything to mask), the tile's maximum for
+            // this lane's query
+            if ((int32_t)(t * AP_BN) + AP_BN - 1 > lim_first) {
+#pragma unroll
+                for (int kb2 = 0; kb2 < 2; ++kb2)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const int32_t key = (int32_t)(t * AP_BN) + 32 * kb2 + 8 * (e / 4) + 4 * (int32_t)h + (e % 4);
+                        if (key > lim) sacc[kb2][e] = -INFINITY;
+                    }
+            }
+            float mx = -INFINITY;
+#pragma unroll
+            for (int kb2 = 0; kb2 < 2; ++kb2)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sacc[kb2][e]);
+            mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+            const float m_new = fmaxf(m_run, mx * sc2);
+            const float m_ref = m_new == -INFINITY ? 0.f : m_new;  // (a row with nothing kept so far: every term below is 0)
+            // a new maximum in any of the wave's rows: the sums and the output so far shrink by 2^(old - new)
+            if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {
+                const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
+                l_run *= alpha;
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) oacc[db][e] *= alpha;
+                m_run = m_new;
+            }
+            float psum = 0.f;
+            // probabilities, packed for the second product: MFMA j covers the tile's keys 16 j .. 16 j + 15; the lane's eight
+            // contraction slots 8 h .. 8 h + 7 hold keys 16 j + 4 h + {0..3} and 16 j + 8 + 4 h + {0..3}
+            Pack8 pb[4];
+#pragma unroll
+            for (int kb2 = 0; kb2 < 2; ++kb2)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb2][e], sc2, -m_ref));
+                    psum += pr;
+                    pb[2 * kb2 + e / 8].e[e % 8] = f2h(pr);
+                }
+            l_run += psum;
+
+            // O^T += V^T . P^T: the A operand's row is dh column 32 db + lane % 32; a transposing read hands a lane four
+            // consecutive keys of that column (the lanes of a 16-lane group address key s16 / 4, columns 4 (s16 % 4) .. + 3)
+            typedef __attribute__((address_space(3))) s16x4 *lds_s16x4;
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const f16 *src = vt + (16 * j + 4 * h + s16 / 4) * VP + 32 * db + 16 * b16 + 4 * (s16 % 4);
+                    union {
+                        s16x4 q[2];
+                        f16x8 hv;
+                    } a;
+                    a.q[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4)src);
+                    a.q[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4)(src + 8 * VP));
+                    oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a.hv, pb[j].h, oacc[db], 0, 0, 0);
+                }
+
+            if (more) commit(buf ^ 1);
         }
-        // scale, mask, the tile's maximum for this lane's query
-        float mx = -INFINITY;
-#pragma unroll
-        for (int kb2 = 0; kb2 < 2; ++kb2)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int32_t key = (int32_t)(t * AP_BN) + 32 * kb2 + 8 * (e / 4) + 4 * (int32_t)h + (e % 4);
-                const float s = key <= lim ? sacc[kb2][e] * sc2 : -INFINITY;
-                sacc[kb2][e] = s;
-                mx = fmaxf(mx, s);
-            }
-        mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-        const float m_new = fmaxf(m_run, mx);
-        const float m_ref = m_new == -INFINITY ? 0.f : m_new;  // (a row with nothing kept so far: every term below is 0)
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
-        m_run = m_new;
-        float psum = 0.f;
-        // probabilities, packed for the second product: MFMA j covers the tile's keys 16 j .. 16 j + 15; the lane's eight
-        // contraction slots 8 h .. 8 h + 7 hold keys 16 j + 4 h + {0..3} and 16 j + 8 + 4 h + {0..3}
-        Pack8 pb[4];
-#pragma unroll
-        for (int kb2 = 0; kb2 < 2; ++kb2)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const float pr = __builtin_amdgcn_exp2f(sacc[kb2][e] - m_ref);
-                psum += pr;
-                pb[2 * kb2 + e / 8].e[e % 8] = f2h(pr);
-            }
-        l_run = l_run * alpha + psum;
-#pragma unroll
-        for (int db = 0; db < DB; ++db)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) oacc[db][e] *= alpha;
-
-        // O^T += V^T . P^T: the A operand's row is dh column 32 db + lane % 32; a transposing read hands a lane four
-        // consecutive keys of that column (the lanes of a 16-lane group address key s16 / 4, columns 4 (s16 % 4) .. + 3)
-        typedef __attribute__((address_space(3))) s16x4 *lds_s16x4;
-#pragma unroll
-        for (int db = 0; db < DB; ++db)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const f16 *src = &v_lds[buf][(16 * j + 4 * h + s16 / 4) * VP + 32 * db + 16 * b16 + 4 * (s16 % 4)];
-                union {
-                    s16x4 q[2];
-                    f16x8 hv;
-                } a;
-                a.q[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4)src);
-                a.q[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4)(src + 8 * VP));
-                oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a.hv, pb[j].h, oacc[db], 0, 0, 0);
-            }
-
-        if (t + 1 < ntiles) commit(buf ^ 1);
         __syncthreads();
     }
 
+    float l_tot = l_run + __shfl_xor(l_run, 32, WAVE);
+    if constexpr (G == 2) {
+        // group 1 hands over through LDS (the tiles are done with: the loop ended on a barrier): value j of lane l of wave
+        // w at float (w * (2 + 16 DB) + j) * 64 + l
+        float *x = reinterpret_cast<float *>(lds) + wave * (2 + 16 * DB) * WAVE + lane;
+        if (grp == 1) {
+            x[0] = m_run;
+            x[WAVE] = l_tot;
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) x[(2 + 16 * db + e) * WAVE] = oacc[db][e];
+        }
+        __syncthreads();
+        if (grp == 1) return;
+        const float m1 = x[0], l1 = x[WAVE];
+        const float m = fmaxf(m_run, m1);  // finite: group 0 has the first tile, in which every row keeps key 0
+        const float a0 = __builtin_amdgcn_exp2f(m_run - m), a1 = __builtin_amdgcn_exp2f(m1 - m);
+        l_tot = l_tot * a0 + l1 * a1;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) oacc[db][e] = oacc[db][e] * a0 + x[(2 + 16 * db + e) * WAVE] * a1;
+    }
+
     // o = O^T / l: the lane holds, for its query, columns 32 db + 8 (e / 4) + 4 h + e % 4: four adjacent ones per e / 4
-    const float l_tot = l_run + __shfl_xor(l_run, 32, WAVE);
     const float inv = 1.0f / l_tot;
     if (row < p.seq) {
         f16 *orow = reinterpret_cast<f16 *>(p.o) + (int64_t)head * p.o_sh + (int64_t)row * p.o_ss;
@@ -188,6 +258,9 @@ __device__ __forceinline__ void attn_prefill(const AttnPrefillParams &p) {
     }
 }
 
-// (two waves per SIMD: two workgroups per CU, one multiplying while the other does its exponentials)
-extern "C" __global__ void __launch_bounds__(256, 2) attn_prefill_d128(AttnPrefillParams p) { attn_prefill<128>(p); }
-extern "C" __global__ void __launch_bounds__(256, 2) attn_prefill_d64(AttnPrefillParams p) { attn_prefill<64>(p); }
+// (two waves per SIMD: two workgroups of four waves per CU, or one of eight; one wave multiplies while the other does its
+// exponentials)
+extern "C" __global__ void __launch_bounds__(256, 2) attn_prefill_d128(AttnPrefillParams p) { attn_prefill<128, 1>(p); }
+extern "C" __global__ void __launch_bounds__(256, 2) attn_prefill_d64(AttnPrefillParams p) { attn_prefill<64, 1>(p); }
+extern "C" __global__ void __launch_bounds__(512) attn_prefill_d128_g2(AttnPrefillParams p) { attn_prefill<128, 2>(p); }
+extern "C" __global__ void __launch_bounds__(512) attn_prefill_d64_g2(AttnPrefillParams p) { attn_prefill<64, 2>(p); }

@@ -330,6 +330,24 @@ def test_attention_one_pass_forced_on_few_rows_agrees_with_the_composite(gpu, st
     assert np.array_equal(qa, a) and np.array_equal(qb, b)
 
 
+@pytest.mark.parametrize("split", ["0", "1"])
+@pytest.mark.parametrize("nh,nkvh,seq,att,dh,mask", [(4, 2, 384, 384, 128, CAUSAL), (3, 3, 130, 257, 64, CAUSAL), (2, 1, 100, 64, 128, NONE),
+                                                     (2, 2, 128, 1, 64, NONE), (4, 4, 70, 70, 128, CAUSAL)])
+def test_attention_one_pass_both_builds(gpu, stream, monkeypatch, split, nh, nkvh, seq, att, dh, mask):
+    """Four waves on all key tiles, or eight waves of which four take the even and four the odd tiles (one tile only: the
+    second group has nothing to add): the planner picks by shape, OPHIP_ATTN_KEYSPLIT keeps one."""
+    rng = np.random.default_rng(nh + seq + att + dh)
+    q, k, v = normal_f16(rng, (nh, seq, dh)), normal_f16(rng, (nkvh, att, dh)), normal_f16(rng, (nkvh, att, dh))
+    monkeypatch.setenv("OPHIP_ATTN_KEYSPLIT", split)
+    op = ophip.Attention(gpu)
+    say("attention one pass key split=%s nh=%d seq=%d att=%d dh=%d" % (split, nh, seq, att, dh))
+    out, q_after = run_attention(gpu, stream, q, k, v, mask, op=op)
+    assert_close_f16(out, attention_f64(q, k, v, mask == CAUSAL), "one pass, split " + split)
+    assert np.array_equal(q_after, out)
+    again, _ = run_attention(gpu, stream, q, k, v, mask, op=op)
+    assert np.array_equal(again, out)
+
+
 def test_attention_one_pass_on_views_of_a_fused_qkv_buffer(gpu, stream):
     """q, k, v are column slices of one [seq, 3 * nh * dh] buffer viewed head-major, o is token-major: heads and tokens
     of q do not merge, so q is left alone (the reference works on a copy of it)."""
