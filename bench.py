@@ -623,6 +623,19 @@ def standalone_ops(ophip, gpu, stream, rng, reps, ceiling=None):
         note="as above on caches that come from HBM")
     for kb_, vb_ in sets[1:]:
         kb_.free(); vb_.free()
+    # attention at prefill shapes (32 heads, dh 128, causal): one pass with the scores kept on the chip where the crate's
+    # composite writes and reads the [nh, seq, att] score matrix four times.  flops = 4 nh seq att dh / 2 (the half of
+    # the score matrix a causal mask keeps); bytes = q, k, v, o once.
+    at = o.Attention(gpu)
+    for seq in (512, 2048, 4096):
+        q, k, v = (gpu.from_host(normal_f16(rng, (NH, seq, DH), 1.0)) for _ in range(3))
+        od = gpu.malloc(NH * seq * DH * 2)
+        a = o.AttentionArgs(c(NH, seq, DH), q, c(NH, seq, DH), k, c(NH, seq, DH), v, c(NH, seq, DH), od, o.AttnMask.CAUSAL)
+        us = time_launches(gpu, stream, lambda: at.launch(a, None, stream), max(5, reps // 2))
+        add("attention", "nh32 seq%d att%d dh128 causal" % (seq, seq), 4 * NH * seq * DH * 2, us, flops=2 * NH * seq * seq * DH,
+            note="one pass (attention_prefill.hip); flops count the unmasked half of the scores")
+        for m_ in (q, k, v, od):
+            m_.free()
     # the dominant decode GEMM (gate/up) on its own, weights stored [K, N] and [N, K]: two copies of the
     # weights alternate so that no launch finds them in the Infinity Cache
     mm = o.MatMul(gpu)
