@@ -183,9 +183,18 @@ bool attention_one_pass(const ophip_attention *op, const ophip_attention_args &a
     if ((dh != 64 && dh != 128) || nh == 0 || seq == 0 || att == 0 || nh > 0x7fffffffu || seq > 0x7fffffffu || att > 0x7fffffffu) return false;
     if (args.mask != OPHIP_MASK_NONE && args.mask != OPHIP_MASK_CAUSAL) return false;
     if (args.mask == OPHIP_MASK_CAUSAL && att < seq) return false;  // rows that keep no column: the softmax of the composite refuses them
-    // Few rows per head leave the composite's products on the weight-streaming kernel and the score matrix small;
-    // from 64 rows on one pass wins (32 heads x 2048 keys: 64 rows 42 against 58 us, 512 x 512: 14 against 35 us)
-    if (op->fused < 0 && seq < 64) return false;
+    // A workgroup walks its keys tile after tile (two tiles of 64 per 2.7 us in the eight-wave build at dh 128), so with
+    // fewer workgroups than CUs the longest walk is the kernel's time, while the composite pays five launches and
+    // four passes over the score matrix (about 20 us + 1 us per MB of it).  Measured, 32 heads, dh 128, causal, one
+    // pass against composite: 16 rows x 2048 keys 42 / 21 us, 128 x 2048 47 / 41, 64 x 64 7 / 16, 256 x 256 13 / 23,
+    // 512 x 512 19 / 35, 2048 x 2048 68 / 326.
+    const size_t cus = (size_t)op->dev->props.multiProcessorCount;
+    const size_t wgs = nh * ((seq + 127) / 128), tiles = (att + 63) / 64;
+    if (op->fused < 0 && wgs <= cus) {
+        const double walk = 4.0 + (double)((tiles + 1) / 2) * (dh == 128 ? 2.7 : 1.6);
+        const double composite = 20.0 + (double)nh * (double)seq * (double)att * 2.0 / 1e6;
+        if (walk >= composite) return false;
+    }
     struct View {
         const ophip_tensor_layout &l;
         const void *base;
@@ -240,8 +249,8 @@ bool attention_one_pass(const ophip_attention *op, const ophip_attention_args &a
     // Under a causal mask the block with the most keys decides once there are no more workgroups than places for
     // them (two per CU): then the eight-wave build, whose workgroups take half as long (32 heads, causal: 2048 x 2048
     // 67.9 against 73.1 us, 512 x 512 19.5 against 21.3; 4096 x 4096 232 against 203, and without a mask it always loses)
-    const size_t cus = (size_t)op->dev->props.multiProcessorCount;
-    const bool split = op->key_split >= 0 ? op->key_split != 0 : p.causal && nh * (size_t)p.nblocks <= 2 * cus;
+    // (and whenever there are fewer workgroups than CUs: a lone workgroup's walk takes 2.7 us per two tiles against 1.75 us per tile)
+    const bool split = op->key_split >= 0 ? op->key_split != 0 : wgs <= cus || (p.causal && wgs <= 2 * cus);
     launch(op->prefill[dh == 64 ? 0 : 1][split], Dim3{(unsigned)nh, p.nblocks}, Dim3{split ? 512u : 256u}, 0, stream_of(qa), p);
     return true;
 }

@@ -277,8 +277,8 @@ def test_decode_layer_chain_matches_the_oracle_end_to_end(gpu, stream):
 
 
 # ------------------------------------------------ one pass, prefill shapes ----
-# From 64 query rows per head on, attention runs on one kernel that keeps the scores on the chip (attention_prefill.hip).
-# Same bar as the composite: the oracle's composite and the f64 formula, within the f16 tolerance.
+# Where its walk over the keys is shorter than the composite's passes over the score matrix (prefill shapes), attention
+# runs on one kernel that keeps the scores on the chip (attention_prefill.hip).  Same bar as the composite: the oracle's composite and the f64 formula, within the f16 tolerance.
 
 def run_attention(gpu, stream, q, k, v, mask, op=None):
     qd, kd, vd = upload(gpu, q), upload(gpu, k), upload(gpu, v)
@@ -295,7 +295,8 @@ def run_attention(gpu, stream, q, k, v, mask, op=None):
                                                      (3, 1, 130, 257, 128, CAUSAL), (3, 3, 65, 64 + 65, 64, CAUSAL),
                                                      (4, 2, 1000, 1000, 64, CAUSAL), (2, 2, 300, 77, 128, NONE),
                                                      (32, 32, 512, 512, 128, CAUSAL), (8, 8, 1024, 1536, 128, CAUSAL)])
-def test_attention_one_pass_prefill(gpu, stream, nh, nkvh, seq, att, dh, mask):
+def test_attention_one_pass_prefill(gpu, stream, monkeypatch, nh, nkvh, seq, att, dh, mask):
+    monkeypatch.setenv("OPHIP_ATTN_FUSED", "1")  # (the planner would take the composite for some of the small ones)
     rng = np.random.default_rng(nh + seq + att + dh)
     q, k, v = normal_f16(rng, (nh, seq, dh)), normal_f16(rng, (nkvh, att, dh)), normal_f16(rng, (nkvh, att, dh))
     say("attention one pass nh=%d nkvh=%d seq=%d att=%d dh=%d mask=%d" % (nh, nkvh, seq, att, dh, mask))
@@ -339,6 +340,7 @@ def test_attention_one_pass_both_builds(gpu, stream, monkeypatch, split, nh, nkv
     rng = np.random.default_rng(nh + seq + att + dh)
     q, k, v = normal_f16(rng, (nh, seq, dh)), normal_f16(rng, (nkvh, att, dh)), normal_f16(rng, (nkvh, att, dh))
     monkeypatch.setenv("OPHIP_ATTN_KEYSPLIT", split)
+    monkeypatch.setenv("OPHIP_ATTN_FUSED", "1")
     op = ophip.Attention(gpu)
     say("attention one pass key split=%s nh=%d seq=%d att=%d dh=%d" % (split, nh, seq, att, dh))
     out, q_after = run_attention(gpu, stream, q, k, v, mask, op=op)
@@ -348,9 +350,10 @@ def test_attention_one_pass_both_builds(gpu, stream, monkeypatch, split, nh, nkv
     assert np.array_equal(again, out)
 
 
-def test_attention_one_pass_on_views_of_a_fused_qkv_buffer(gpu, stream):
+def test_attention_one_pass_on_views_of_a_fused_qkv_buffer(gpu, stream, monkeypatch):
     """q, k, v are column slices of one [seq, 3 * nh * dh] buffer viewed head-major, o is token-major: heads and tokens
     of q do not merge, so q is left alone (the reference works on a copy of it)."""
+    monkeypatch.setenv("OPHIP_ATTN_FUSED", "1")
     rng = np.random.default_rng(21)
     seq, nh, dh = 300, 8, 128
     qkv = normal_f16(rng, (seq, 3 * nh * dh))
@@ -369,7 +372,8 @@ def test_attention_one_pass_on_views_of_a_fused_qkv_buffer(gpu, stream):
     assert np.array_equal(download(gpu, stream, qkv_d, qkv), qkv)
 
 
-def test_attention_one_pass_with_o_in_place_of_q(gpu, stream):
+def test_attention_one_pass_with_o_in_place_of_q(gpu, stream, monkeypatch):
+    monkeypatch.setenv("OPHIP_ATTN_FUSED", "1")
     rng = np.random.default_rng(22)
     nh, seq, dh = 4, 192, 64
     q, k, v = normal_f16(rng, (nh, seq, dh)), normal_f16(rng, (nh, seq, dh)), normal_f16(rng, (nh, seq, dh))
