@@ -303,3 +303,45 @@ def test_random_mat_mul_ragged_tile_shapes(gpu, stream, monkeypatch, sweep):
             assert err <= 2e-3 + 4e-3 * scale, (err, scale)
     finally:
         oracle.set_threads(1)
+
+
+@SWEEPS
+def test_random_attention_one_pass(gpu, stream, monkeypatch, sweep):
+    """attention on the one-pass kernel (both builds) over random head counts, groupings, row and key counts and row
+    paddings, against the f64 formula; nothing outside o and q (which receives the result too) may change."""
+    rng = np.random.default_rng(800 + 1000 * sweep)
+    monkeypatch.setenv("OPHIP_ATTN_FUSED", "1")
+    ops = {}
+    for split in ("0", "1"):
+        monkeypatch.setenv("OPHIP_ATTN_KEYSPLIT", split)
+        ops[split] = ophip.Attention(gpu)
+    for case in range(16):
+        dh = int(rng.choice([64, 128]))
+        nkvh = int(rng.choice([1, 2, 3, 5]))
+        nh = nkvh * int(rng.choice([1, 2, 4]))
+        seq = int(rng.choice([1, 31, 64, 100, 128, 129, 200, 333]))
+        causal = bool(rng.integers(0, 2))
+        att = seq + int(rng.choice([0, 0, 1, 63, 64, 130])) if causal else int(rng.choice([1, 17, 64, 65, 200, 384]))
+        pq, pk, pv, po = (int(rng.choice([0, 8, 24])) for _ in range(4))
+        Q, K, V = Guarded(gpu, rng, (nh, seq, dh), f16, pq), Guarded(gpu, rng, (nkvh, att, dh), f16, pk), Guarded(gpu, rng, (nkvh, att, dh), f16, pv)
+        O = Guarded(gpu, rng, (nh, seq, dh), f16, po, fill=0)
+        split = "01"[case % 2]
+        say("random attention %d: nh=%d nkvh=%d seq=%d att=%d dh=%d causal=%s pads=%d %d %d %d split=%s" % (
+            case, nh, nkvh, seq, att, dh, causal, pq, pk, pv, po, split))
+        q, k, v = Q.view().copy(), K.view().copy(), V.view().copy()
+        args = ophip.AttentionArgs(Q.layout, Q.ptr, K.layout, K.ptr, V.layout, V.ptr, O.layout, O.ptr,
+                                   ophip.AttnMask.CAUSAL if causal else ophip.AttnMask.NONE)
+        ops[split].launch(args, None, stream)
+        got = O.fetch(stream)
+        g = nh // nkvh
+        kk, vv = np.repeat(k.astype(np.float64), g, axis=0), np.repeat(v.astype(np.float64), g, axis=0)
+        s = np.einsum("hsd,had->hsa", q.astype(np.float64), kk) / np.sqrt(dh)
+        if causal:
+            s = np.where((np.arange(att)[None, :] <= (att - seq + np.arange(seq))[:, None])[None], s, -np.inf)
+        pr = np.exp(s - s.max(-1, keepdims=True))
+        ref = np.einsum("hsa,had->hsd", pr / pr.sum(-1, keepdims=True), vv)
+        assert_close_f16(got, ref, "random attention")
+        assert np.array_equal(K.fetch(stream), k) and np.array_equal(V.fetch(stream), v)
+        # padded rows still follow each other head after head: heads and tokens fold into one dimension, and the reference
+        # then leaves att . v in q
+        assert np.array_equal(Q.fetch(stream), got)
