@@ -93,7 +93,7 @@ __device__ __forceinline__ float wave_max_dpp(float v) {
 // (one float per wave of the block) in a fixed order; all threads must call.
 template <int G>
 __device__ __forceinline__ float group_sum(float v, float *smem) {
-    v = wave_sum(v);
+    v = wave_sum_dpp(v);
     if constexpr (G > WAVE) {
         const int wave = threadIdx.x / WAVE;
         __syncthreads();
@@ -109,7 +109,7 @@ __device__ __forceinline__ float group_sum(float v, float *smem) {
 }
 template <int G>
 __device__ __forceinline__ float group_max(float v, float *smem) {
-    v = wave_max(v);
+    v = wave_max_dpp(v);
     if constexpr (G > WAVE) {
         const int wave = threadIdx.x / WAVE;
         __syncthreads();

@@ -179,8 +179,8 @@ __device__ __forceinline__ void layer_norm_rows(const LayerNormParams &p) {
                 }
             }
         }
-        s1 = wave_sum(s1);
-        s2 = wave_sum(s2);
+        s1 = wave_sum_dpp(s1);
+        s2 = wave_sum_dpp(s2);
         float e, k;
         mean_and_scale(s1, s2, p.d, p.epsilon, e, k);
         char *yr = reinterpret_cast<char *>(p.y) + (int64_t)row * p.nsy;

@@ -209,7 +209,7 @@ __device__ __forceinline__ void rms_norm_rows(const RmsNormParams &p) {
                 }
             }
         }
-        ss = wave_sum(ss);
+        ss = wave_sum_dpp(ss);
         const float k = 1.0f / sqrtf(ss / (float)p.d + p.epsilon);
         char *yr = reinterpret_cast<char *>(p.y) + (int64_t)row * p.nsy;
 #pragma unroll
