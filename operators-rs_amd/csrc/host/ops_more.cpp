@@ -14,6 +14,18 @@ namespace {
 const char *dt_tag(uint64_t dt) {
     return dt == OPHIP_DT_F16 ? "f16" : dt == OPHIP_DT_BF16 ? "bf16" : dt == OPHIP_DT_F32 ? "f32" : dt == OPHIP_DT_F64 ? "f64" : "?";
 }
+bool is_float_dt(uint64_t dt) { return dt == OPHIP_DT_F16 || dt == OPHIP_DT_BF16 || dt == OPHIP_DT_F32 || dt == OPHIP_DT_F64; }
+// integers by width (signed and unsigned sums are the same bits), bool on its own; null for anything else
+const char *int_tag(uint64_t dt) {
+    switch (dt) {
+        case OPHIP_DT_U8: case OPHIP_DT_I8: return "i8";
+        case OPHIP_DT_U16: case OPHIP_DT_I16: return "i16";
+        case OPHIP_DT_U32: case OPHIP_DT_I32: return "i32";
+        case OPHIP_DT_U64: case OPHIP_DT_I64: return "i64";
+        case OPHIP_DT_BOOL: return "bool";
+        default: return nullptr;
+    }
+}
 
 }  // namespace
 
@@ -275,9 +287,9 @@ extern "C" int ophip_add_launch(const ophip_add *op, const ophip_add_args *args,
                                 const ophip_queue_alloc *qa) {
     return guard([&] {
         AddScheme s = add_scheme(*args);
-        // (bf16: no CPU kernel in the reference, but its CUDA backend adds any named type, add/cuda/mod.rs:105-123)
-        if (s.dt != OPHIP_DT_F16 && s.dt != OPHIP_DT_BF16 && s.dt != OPHIP_DT_F32 && s.dt != OPHIP_DT_F64)
-            throw type_not_support("add supports f16, bf16, f32 and f64");
+        // (bf16, integers, bool: no CPU kernel in the reference, but its CUDA backend adds any named type,
+        // add/cuda/mod.rs:105-123)
+        if (!is_float_dt(s.dt) && !int_tag(s.dt)) throw type_not_support("add supports the float, integer and bool types");
         if (s.dims.size() > OPHIP_REARRANGE_MAXD)
             throw rank_not_support("add supports at most " + std::to_string(OPHIP_REARRANGE_MAXD) +
                                    " non-mergeable dimensions");
@@ -295,7 +307,7 @@ extern "C" int ophip_add_launch(const ophip_add *op, const ophip_add_args *args,
         const size_t per = 16 / unit;
         if (!s.dims.empty()) {
             AddDim &in = s.dims.back();
-            vec = s.dt != OPHIP_DT_F64 && in.c == (ptrdiff_t)unit && in.a == (ptrdiff_t)unit && in.b == (ptrdiff_t)unit && in.d % per == 0 &&
+            vec = is_float_dt(s.dt) && s.dt != OPHIP_DT_F64 && in.c == (ptrdiff_t)unit && in.a == (ptrdiff_t)unit && in.b == (ptrdiff_t)unit && in.d % per == 0 &&
                   aligned16(p.c) && aligned16(p.a) && aligned16(p.b);
             for (size_t i = 0; vec && i + 1 < s.dims.size(); ++i)
                 vec = mult16(s.dims[i].c) && mult16(s.dims[i].a) && mult16(s.dims[i].b);
@@ -316,7 +328,7 @@ extern "C" int ophip_add_launch(const ophip_add *op, const ophip_add_args *args,
         }
         // (more output than the caches hold: the build that stores with the non-temporal hint)
         const bool nt = vec && total * 16 >= ((size_t)64 << 20);
-        const std::string name = std::string("add_") + dt_tag(s.dt) + (vec ? (nt ? "_vec_nt" : "_vec") : "_scalar");
+        const std::string name = std::string("add_") + (is_float_dt(s.dt) ? dt_tag(s.dt) : int_tag(s.dt)) + (vec ? (nt ? "_vec_nt" : "_vec") : "_scalar");
         const unsigned blocks = (unsigned)std::min<size_t>(ceil_div(total, 256), 1u << 20);
         if (!p.c || !p.a || !p.b) throw args_not_support("null base address");
         op->dev->make_current();
@@ -384,9 +396,9 @@ extern "C" int ophip_add_rows_launch(const ophip_add_rows *op, const ophip_add_r
                         nsd = static_of(args->dst_layout.strides[2]);
         const ptrdiff_t bsi = static_of(args->idx_layout.strides[0]), msi = static_of(args->idx_layout.strides[1]);
         const ptrdiff_t kss = static_of(args->src_layout.strides[0]), nss = static_of(args->src_layout.strides[1]);
-        // (bf16: no CPU kernel in the reference, but its CUDA backend compiles one for any named type, add_rows/cuda/mod.rs:135-163)
-        if (r.dt != OPHIP_DT_F16 && r.dt != OPHIP_DT_BF16 && r.dt != OPHIP_DT_F32 && r.dt != OPHIP_DT_F64)
-            throw type_not_support("add_rows supports f16, bf16, f32 and f64");
+        // (bf16, integers, bool: no CPU kernel in the reference, but its CUDA backend compiles one for any named type,
+        // add_rows/cuda/mod.rs:135-163)
+        if (!is_float_dt(r.dt) && !int_tag(r.dt)) throw type_not_support("add_rows supports the float, integer and bool types");
         if (r.dt_idx != OPHIP_DT_U32 && r.dt_idx != OPHIP_DT_U64) throw type_not_support("idx must be u32 or u64");
         const ptrdiff_t unit = (ptrdiff_t)ophip_dtype_nbytes(r.dt), iunit = (ptrdiff_t)ophip_dtype_nbytes(r.dt_idx);
         for (ptrdiff_t st : {bsd, msd, nsd, kss, nss})
@@ -412,7 +424,7 @@ extern "C" int ophip_add_rows_launch(const ophip_add_rows *op, const ophip_add_r
         p.idx_is_u64 = r.dt_idx == OPHIP_DT_U64;
         q.nsd = nsd;
         q.nss = nss;
-        const bool vec = unit == 2 && nsd == unit && nss == unit && n % 8 == 0 && aligned16(p.dst) &&
+        const bool vec = (r.dt == OPHIP_DT_F16 || r.dt == OPHIP_DT_BF16) && nsd == unit && nss == unit && n % 8 == 0 && aligned16(p.dst) &&
                          aligned16(p.src) && mult16(bsd) && mult16(msd) && mult16(kss);
         const size_t items = vec ? n / 8 : n;
         const unsigned gx = std::min<unsigned>(ceil_div(items, 256), 65535u);
@@ -423,7 +435,7 @@ extern "C" int ophip_add_rows_launch(const ophip_add_rows *op, const ophip_add_r
             launch(op->dev->kernel("add_rows", r.dt == OPHIP_DT_F16 ? "add_rows_f16_vec" : "add_rows_bf16_vec"), Dim3{gx, gy}, Dim3{256}, 0,
                stream_of(qa), p);
         } else {
-            const std::string name = std::string("add_rows_") + dt_tag(r.dt) + "_scalar";
+            const std::string name = std::string("add_rows_") + (is_float_dt(r.dt) ? dt_tag(r.dt) : int_tag(r.dt)) + "_scalar";
             launch(op->dev->kernel("add_rows", name.c_str()), Dim3{gx, gy}, Dim3{256}, 0, stream_of(qa), q);
         }
     });

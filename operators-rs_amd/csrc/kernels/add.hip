@@ -78,3 +78,21 @@ extern "C" __global__ void __launch_bounds__(256) add_f16_scalar(AddParams p) { 
 extern "C" __global__ void __launch_bounds__(256) add_bf16_scalar(AddParams p) { add_scalar<bf16>(p); }
 extern "C" __global__ void __launch_bounds__(256) add_f32_scalar(AddParams p) { add_scalar<float>(p); }
 extern "C" __global__ void __launch_bounds__(256) add_f64_scalar(AddParams p) { add_scalar<double>(p); }
+
+// Integer and bool elements: the reference's CUDA backend compiles `c[idx] = a[idx] + b[idx]` for any named type
+// (add/cuda/mod.rs:105-123 with handle/cuda/mod.rs:188-210), which for integers is the sum modulo 2^bits (signed and
+// unsigned alike in two's complement: one kernel per width) and for bool "either is set".  Its CPU backend has floats only.
+template <typename U, bool IS_BOOL = false>
+__device__ __forceinline__ void add_int_scalar(const AddParams &p) {
+    for (uint32_t g = blockIdx.x * blockDim.x + threadIdx.x; g < p.total; g += gridDim.x * blockDim.x) {
+        const AddOffsets o = add_decode(p, g);
+        const U a = *reinterpret_cast<const U *>(reinterpret_cast<const char *>(p.a) + o.a);
+        const U b = *reinterpret_cast<const U *>(reinterpret_cast<const char *>(p.b) + o.b);
+        *reinterpret_cast<U *>(reinterpret_cast<char *>(p.c) + o.c) = IS_BOOL ? (U)((a | b) != 0) : (U)(a + b);
+    }
+}
+extern "C" __global__ void __launch_bounds__(256) add_i8_scalar(AddParams p) { add_int_scalar<uint8_t>(p); }
+extern "C" __global__ void __launch_bounds__(256) add_i16_scalar(AddParams p) { add_int_scalar<uint16_t>(p); }
+extern "C" __global__ void __launch_bounds__(256) add_i32_scalar(AddParams p) { add_int_scalar<uint32_t>(p); }
+extern "C" __global__ void __launch_bounds__(256) add_i64_scalar(AddParams p) { add_int_scalar<uint64_t>(p); }
+extern "C" __global__ void __launch_bounds__(256) add_bool_scalar(AddParams p) { add_int_scalar<uint8_t, true>(p); }

@@ -71,3 +71,24 @@ extern "C" __global__ void __launch_bounds__(256) add_rows_f32_scalar(AddRowsSca
 extern "C" __global__ void __launch_bounds__(256) add_rows_f64_scalar(AddRowsScalarParams q) {
     add_rows_scalar<double>(q.p, q.nsd, q.nss);
 }
+
+// Integer and bool rows, as the reference's CUDA backend would compile them (add_rows/cuda/mod.rs:135-163): sums modulo
+// 2^bits, one kernel per width; bool: either is set.
+template <typename U, bool IS_BOOL = false>
+__device__ __forceinline__ void add_rows_int(const AddRowsParams &p, int64_t nsd, int64_t nss) {
+    for (uint32_t bm = blockIdx.y; bm < p.batch * p.m; bm += gridDim.y) {
+        char *dst;
+        const char *src;
+        if (!add_rows_locate(p, bm, dst, src)) continue;
+        for (uint32_t j = blockIdx.x * blockDim.x + threadIdx.x; j < p.n; j += gridDim.x * blockDim.x) {
+            U *d = reinterpret_cast<U *>(dst + (int64_t)j * nsd);
+            const U s = *reinterpret_cast<const U *>(src + (int64_t)j * nss);
+            *d = IS_BOOL ? (U)((*d | s) != 0) : (U)(*d + s);
+        }
+    }
+}
+extern "C" __global__ void __launch_bounds__(256) add_rows_i8_scalar(AddRowsScalarParams q) { add_rows_int<uint8_t>(q.p, q.nsd, q.nss); }
+extern "C" __global__ void __launch_bounds__(256) add_rows_i16_scalar(AddRowsScalarParams q) { add_rows_int<uint16_t>(q.p, q.nsd, q.nss); }
+extern "C" __global__ void __launch_bounds__(256) add_rows_i32_scalar(AddRowsScalarParams q) { add_rows_int<uint32_t>(q.p, q.nsd, q.nss); }
+extern "C" __global__ void __launch_bounds__(256) add_rows_i64_scalar(AddRowsScalarParams q) { add_rows_int<uint64_t>(q.p, q.nsd, q.nss); }
+extern "C" __global__ void __launch_bounds__(256) add_rows_bool_scalar(AddRowsScalarParams q) { add_rows_int<uint8_t, true>(q.p, q.nsd, q.nss); }

@@ -173,6 +173,47 @@ def test_add_contiguous(gpu, stream, dtype, shape):
     assert np.array_equal(out, oracle.add(c, a, b))
 
 
+@pytest.mark.parametrize("dtype", [np.uint8, np.int8, np.uint16, np.int16, np.uint32, np.int32, np.uint64, np.int64])
+def test_add_and_add_rows_integers_wrap_like_the_cuda_kernels(gpu, stream, dtype):
+    """The reference's CUDA backend compiles add and add_rows for any named type (add/cuda/mod.rs:105-123,
+    add_rows/cuda/mod.rs:135-163): integer sums are modulo 2^bits.  Its CPU backend has no integer kernels, so the
+    expected values are numpy's (which wraps the same way)."""
+    rng = np.random.default_rng(np.dtype(dtype).itemsize * 7 + (1 if np.dtype(dtype).kind == "i" else 0))
+    info = np.iinfo(dtype)
+    draw = lambda shape: rng.integers(info.min, info.max, shape, dtype=dtype, endpoint=True)
+    a, b = draw((5, 77)), draw((5, 77))
+    c = np.zeros((5, 77), dtype)
+    say("add %s" % np.dtype(dtype).name)
+    out = run_add(gpu, stream, c, c, a, a, b, b).view(dtype).reshape(5, 77)
+    assert np.array_equal(out, a + b)   # numpy wraps silently on arrays
+    bias = draw((77,))
+    at = a.T.copy()  # a stored column-major, read through its transposed view
+    out = run_add(gpu, stream, c, c, at.T, at, np.lib.stride_tricks.as_strided(bias, (5, 77), (0, bias.itemsize)), bias)
+    assert np.array_equal(out.view(dtype).reshape(5, 77), a + bias[None, :])
+    dst, src = draw((2, 3, 40)), draw((6, 40))
+    idx = rng.integers(0, 6, (2, 3)).astype(np.uint32)
+    dd, sd, idd = gpu.from_host(dst), gpu.from_host(src), gpu.from_host(idx)
+    L = TensorLayout
+    ophip.AddRows(gpu).launch(ophip.AddRowsArgs(L.of(dst), dd, L.of(src), sd, L.of(idx), idd), None, stream)
+    got = gpu.to_host(dd, dtype, dst.size, stream=stream).reshape(dst.shape)
+    assert np.array_equal(got, dst + src[idx])
+
+
+def test_add_and_add_rows_bool(gpu, stream):
+    rng = np.random.default_rng(5)
+    a, b = rng.integers(0, 2, (4, 50)).astype(np.uint8), rng.integers(0, 2, (4, 50)).astype(np.uint8)
+    ad, bd, cd = gpu.from_host(a), gpu.from_host(b), gpu.malloc(a.nbytes)
+    lay = TensorLayout.new_contiguous(dt.BOOL, [4, 50])
+    ophip.Add(gpu).launch(ophip.AddArgs(lay, cd, lay, ad, lay, bd), None, stream)
+    assert np.array_equal(gpu.to_host(cd, np.uint8, a.size, stream=stream).reshape(4, 50), a | b)   # true + true is true
+    idx = rng.integers(0, 4, (1, 4)).astype(np.uint32)
+    dst = rng.integers(0, 2, (1, 4, 50)).astype(np.uint8)
+    dd, idd = gpu.from_host(dst), gpu.from_host(idx)
+    ophip.AddRows(gpu).launch(ophip.AddRowsArgs(TensorLayout.new_contiguous(dt.BOOL, [1, 4, 50]), dd, lay, ad,
+                                                TensorLayout.of(idx), idd), None, stream)
+    assert np.array_equal(gpu.to_host(dd, np.uint8, dst.size, stream=stream).reshape(1, 4, 50), dst | a[idx])
+
+
 def test_add_permuted_and_broadcast_views(gpu, stream):
     rng = np.random.default_rng(10)
     a = normal_f16(rng, (6, 5, 64))
