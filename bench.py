@@ -467,6 +467,26 @@ def mat_mul_lines(o, gpu, stream, rng, add, launches=0):
         A_.free(); B_.free(); C_.free(); ws.free()
 
 
+def attention_lines(o, gpu, stream, rng, add, reps, full=False):
+    """attention at prefill shapes (32 heads, dh 128): one pass with the scores kept on the chip where the crate's
+    composite writes and reads the [nh, seq, att] score matrix four times.  flops = 4 nh seq att dh, half of it under a
+    causal mask (the part of the score matrix the mask keeps); bytes = q, k, v, o once.  `full`: the unmasked shapes too."""
+    L, F16 = o.TensorLayout, o.dt.F16
+    c = lambda *s: L.new_contiguous(F16, list(s))
+    at = o.Attention(gpu)
+    for seq, causal in [(512, True), (2048, True), (4096, True)] + ([(2048, False), (4096, False)] if full else []):
+        q, k, v = (gpu.from_host(normal_f16(rng, (NH, seq, DH), 1.0)) for _ in range(3))
+        od = gpu.malloc(NH * seq * DH * 2)
+        a = o.AttentionArgs(c(NH, seq, DH), q, c(NH, seq, DH), k, c(NH, seq, DH), v, c(NH, seq, DH), od,
+                            o.AttnMask.CAUSAL if causal else o.AttnMask.NONE)
+        us = time_launches(gpu, stream, lambda: at.launch(a, None, stream), reps)
+        add("attention", "nh32 seq%d att%d dh128 %s" % (seq, seq, "causal" if causal else "no mask"), 4 * NH * seq * DH * 2, us,
+            flops=(2 if causal else 4) * NH * seq * seq * DH,
+            note="one pass (attention_prefill.hip)" + ("; flops count the unmasked half of the scores" if causal else ""))
+        for m_ in (q, k, v, od):
+            m_.free()
+
+
 def standalone_ops(ophip, gpu, stream, rng, reps, ceiling=None):
     """Every operator at its benchmark shape plus a scaled shape that does not fit the Infinity Cache."""
     o, L, F16 = ophip, ophip.TensorLayout, ophip.dt.F16
@@ -623,19 +643,7 @@ def standalone_ops(ophip, gpu, stream, rng, reps, ceiling=None):
         note="as above on caches that come from HBM")
     for kb_, vb_ in sets[1:]:
         kb_.free(); vb_.free()
-    # attention at prefill shapes (32 heads, dh 128, causal): one pass with the scores kept on the chip where the crate's
-    # composite writes and reads the [nh, seq, att] score matrix four times.  flops = 4 nh seq att dh / 2 (the half of
-    # the score matrix a causal mask keeps); bytes = q, k, v, o once.
-    at = o.Attention(gpu)
-    for seq in (512, 2048, 4096):
-        q, k, v = (gpu.from_host(normal_f16(rng, (NH, seq, DH), 1.0)) for _ in range(3))
-        od = gpu.malloc(NH * seq * DH * 2)
-        a = o.AttentionArgs(c(NH, seq, DH), q, c(NH, seq, DH), k, c(NH, seq, DH), v, c(NH, seq, DH), od, o.AttnMask.CAUSAL)
-        us = time_launches(gpu, stream, lambda: at.launch(a, None, stream), max(5, reps // 2))
-        add("attention", "nh32 seq%d att%d dh128 causal" % (seq, seq), 4 * NH * seq * DH * 2, us, flops=2 * NH * seq * seq * DH,
-            note="one pass (attention_prefill.hip); flops count the unmasked half of the scores")
-        for m_ in (q, k, v, od):
-            m_.free()
+    attention_lines(o, gpu, stream, rng, add, max(5, reps // 2))
     # the dominant decode GEMM (gate/up) on its own, weights stored [K, N] and [N, K]: two copies of the
     # weights alternate so that no launch finds them in the Infinity Cache
     mm = o.MatMul(gpu)
@@ -738,6 +746,9 @@ def main():
     ap.add_argument("--mat-mul-only", type=int, nargs="?", const=0, default=None, metavar="LAUNCHES",
                     help="only the compute-bound mat_mul shapes (not the benchmark line); with a number, that many "
                          "plain launches per shape, for hardware-counter runs")
+    ap.add_argument("--attention-only", type=int, nargs="?", const=0, default=None, metavar="LAUNCHES",
+                    help="only attention at prefill shapes, causal and unmasked; with a number, that many launches per "
+                         "shape (hardware-counter runs)")
     ap.add_argument("--floors", action="store_true",
                     help="only the decode layer's GEMMs on cold operands, each beside a bare read of the same bytes")
     ap.add_argument("--ceilings", action="store_true",
@@ -760,6 +771,11 @@ def main():
         return
     if args.ceilings:
         print(json.dumps({"ceilings": ceilings(ophip, gpu, stream)}))
+        return
+    if args.attention_only is not None:
+        lines = []
+        attention_lines(ophip, gpu, stream, rng, adder(lines), args.attention_only or 20, full=True)
+        print(json.dumps({"attention": lines}))
         return
     if args.mat_mul_only is not None:
         lines = []
