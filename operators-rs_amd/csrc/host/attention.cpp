@@ -97,7 +97,7 @@ struct ophip_attention {
     hipFunction_t prefill[2][2] = {};
     int key_split = -1;  // OPHIP_ATTN_KEYSPLIT=0|1 keeps one of the two builds (sweeps); read once, here
     // OPHIP_ATTN_FUSED=0 keeps the composite (tests, comparisons), =1 takes the one-pass kernel wherever it applies;
-    // read once, here.  Otherwise the row count decides (attention_launch).
+    // read once, here.  Otherwise an estimate of the two times decides (attention_one_pass).
     int fused = -1;
     explicit ophip_attention(ophip_device *d) : dev(d) {
         ophip_device_retain(d);
