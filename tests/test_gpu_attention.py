@@ -396,3 +396,72 @@ def test_attention_kv_cached_prefill_goes_through_the_one_pass_kernel(gpu, strea
         assert_close_f16(out, ref, "kv cached prefill vs oracle")
         assert_close_f16(out, attention_f64(q, kc_ref[:, :pos + seq], vc_ref[:, :pos + seq], True), "kv cached prefill vs f64")
         assert np.array_equal(q_after, q if strided else out)
+
+
+def test_prefill_layer_chain_matches_the_oracle_end_to_end(gpu, stream):
+    """A prefill step of a small Llama-shaped layer (192 tokens, d 1024, 8 heads of 128, FFN 2752) on the operators a model
+    runs it with -- rms_norm, QKV mat_mul, rope on q and k, attention_kv_cached from an empty cache (the append and the
+    one-pass attention over views of the QKV buffer), O-proj, rms_norm, gate/up, swiglu, down -- and the same chain
+    through the oracle on the same seeded weights."""
+    nt, d, nh, dh, di, buf = 192, 1024, 8, 128, 2752, 256
+    rng = np.random.default_rng(1)
+    L, c = TensorLayout, lambda *s: TensorLayout.new_contiguous(dt.F16, list(s))
+    h = {"x": normal_f16(rng, (nt, d)), "w1": rng.uniform(0.5, 1.5, d).astype(np.float32), "w2": rng.uniform(0.5, 1.5, d).astype(np.float32),
+         "wqkv": (rng.standard_normal((d, 3 * d)) * 0.03).astype(f16), "wo": (rng.standard_normal((d, d)) * 0.03).astype(f16),
+         "wgu": (rng.standard_normal((d, 2 * di)) * 0.03).astype(f16), "wd": (rng.standard_normal((di, d)) * 0.02).astype(f16),
+         "pos": np.arange(nt, dtype=np.uint32)}
+    dev = {k: upload(gpu, v) for k, v in h.items()}
+    xn, qkv, o, y, yn, gu, out = (gpu.malloc(n * 2) for n in (nt * d, nt * 3 * d, nt * d, nt * d, nt * d, nt * 2 * di, nt * d))
+    kc, vc = gpu.malloc(nh * buf * dh * 2), gpu.malloc(nh * buf * dh * 2)
+    gpu.memset(kc, 0); gpu.memset(vc, 0)
+    w32 = lambda n: L(dt.F32, [n], [4])
+    rms, mm, rope, akv, sw = ophip.RmsNorm(gpu), ophip.MatMul(gpu), ophip.Rope(gpu), ophip.AttnKVCached(gpu), ophip.Swiglu(gpu)
+    ws = gpu.malloc(64 << 20)
+    say("prefill layer chain")
+    rms.launch(ophip.RmsNormArgs(c(nt, d), xn, c(nt, d), dev["x"], w32(d), dev["w1"], 1e-5), None, stream)
+    mm.launch(ophip.MatMulArgs(c(nt, 3 * d), qkv, 0.0, c(nt, d), xn, c(d, 3 * d), dev["wqkv"], 1.0), ws, stream)
+    row = 3 * d * 2
+    tok = L(dt.F16, [nt, 2 * nh, dh], [row, dh * 2, 2])  # q and k heads side by side in a QKV row
+    empty = L(dt.F16, [0, dh], [dh * 2, 2])
+    rope.launch(ophip.RopeArgs(tok, qkv, L.of(h["pos"]), dev["pos"], empty, None, empty, None, 1e4), None, stream)
+    head = lambda: L(dt.F16, [nh, nt, dh], [dh * 2, row, 2])
+    args = ophip.AttnKVCachedArgs(head(), qkv.ptr, head(), qkv.ptr + d * 2, head(), qkv.ptr + 2 * d * 2,
+                                  L(dt.F16, [nh, nt, dh], [dh * 2, d * 2, 2]), o, c(nh, buf, dh), kc, c(nh, buf, dh), vc, CAUSAL, 0)
+    akv.launch(args, ws, stream)
+    mm.launch(ophip.MatMulArgs(c(nt, d), y, 0.0, c(nt, d), o, c(d, d), dev["wo"], 1.0), ws, stream)
+    rms.launch(ophip.RmsNormArgs(c(nt, d), yn, c(nt, d), y, w32(d), dev["w2"], 1e-5), None, stream)
+    mm.launch(ophip.MatMulArgs(c(nt, 2 * di), gu, 0.0, c(nt, d), yn, c(d, 2 * di), dev["wgu"], 1.0), ws, stream)
+    half = L(dt.F16, [nt, di], [2 * di * 2, 2])
+    sw.launch(ophip.SwigluArgs(half, gu, half, gu.ptr + di * 2), None, stream)
+    mm.launch(ophip.MatMulArgs(c(nt, d), out, 0.0, half, gu, c(di, d), dev["wd"], 1.0), ws, stream)
+    got = gpu.to_host(out, f16, nt * d, stream=stream).reshape(nt, d)
+    kc_got = gpu.to_host(kc, f16, nh * buf * dh, stream=stream).reshape(nh, buf, dh)
+
+    oracle.set_threads(8)
+    try:
+        r_xn = oracle.rms_norm(np.empty_like(h["x"]), h["x"], h["w1"], 1e-5)
+        r_qkv = oracle.mat_mul(np.zeros((nt, 3 * d), f16), 0.0, r_xn, h["wqkv"], 1.0)
+        oracle.set_threads(1)
+        oracle.rope(r_qkv[:, :2 * d].reshape(nt, 2 * nh, dh), h["pos"], 1e4)
+        oracle.set_threads(8)
+        view = lambda i: r_qkv[:, i * d:(i + 1) * d].reshape(nt, nh, dh).transpose(1, 0, 2)
+        r_o = np.zeros((nt, d), f16)
+        r_kc, r_vc = np.zeros((nh, buf, dh), f16), np.zeros((nh, buf, dh), f16)
+        oracle.attention_kv_cached(view(0), view(1), view(2), r_o.reshape(nt, nh, dh).transpose(1, 0, 2), r_kc, r_vc, 0, causal=True)
+        r_y = oracle.mat_mul(np.zeros((nt, d), f16), 0.0, r_o, h["wo"], 1.0)
+        r_yn = oracle.rms_norm(np.empty_like(r_y), r_y, h["w2"], 1e-5)
+        r_gu = oracle.mat_mul(np.zeros((nt, 2 * di), f16), 0.0, r_yn, h["wgu"], 1.0)
+        oracle.set_threads(1)
+        oracle.swiglu(r_gu[:, :di], r_gu[:, di:])
+        oracle.set_threads(8)
+        ref = oracle.mat_mul(np.zeros((nt, d), f16), 0.0, r_gu[:, :di], h["wd"], 1.0)
+    finally:
+        oracle.set_threads(1)
+    # the appended keys went through rms_norm, a product and rope on both sides: close, not bit-equal
+    assert_close_f16(kc_got[:, :nt], r_kc[:, :nt], "appended keys", abs_tol=8e-3)
+    assert (kc_got[:, nt:] == 0).all()
+    err = np.abs(got.astype(np.float64) - ref.astype(np.float64))
+    scale = float(np.abs(ref.astype(np.float64)).max())
+    say("prefill layer: max err %.3g, median err %.3g, output scale %.3g" % (err.max(), np.median(err), scale))
+    assert err.max() <= 1e-2 * scale, err.max() / scale
+    assert np.median(err) <= 1e-3 * scale, np.median(err) / scale
