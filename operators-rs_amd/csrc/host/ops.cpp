@@ -183,7 +183,7 @@ static RopeMeta rope_meta(const ophip_rope_args &a) {
 }
 
 struct ophip_rope : OpBase {
-    hipFunction_t f16_vec, f16_pairs, f32_pairs, f64_pairs;
+    hipFunction_t f16_vec, f16_pairs, bf16_vec, bf16_pairs, f32_pairs, f64_pairs;
     // theta^(k / (dh/2)) of the last (theta, dh) launched: a model has one such pair
     mutable std::mutex den_mu;
     mutable float den_theta = 0.f;
@@ -201,6 +201,8 @@ struct ophip_rope : OpBase {
     explicit ophip_rope(ophip_device *d) : OpBase(d) {
         f16_vec = d->kernel("rope", "rope_f16_vec");
         f16_pairs = d->kernel("rope", "rope_f16_pairs");
+        bf16_vec = d->kernel("rope", "rope_bf16_vec");
+        bf16_pairs = d->kernel("rope", "rope_bf16_pairs");
         f32_pairs = d->kernel("rope", "rope_f32_pairs");
         f64_pairs = d->kernel("rope", "rope_f64_pairs");
     }
@@ -225,8 +227,9 @@ extern "C" int ophip_rope_launch(const ophip_rope *op, const ophip_rope_args *ar
                                  const ophip_queue_alloc *qa) {
     return guard([&] {
         const RopeMeta m = rope_meta(*args);
-        if (m.dt_t != OPHIP_DT_F16 && m.dt_t != OPHIP_DT_F32 && m.dt_t != OPHIP_DT_F64)
-            throw type_not_support("rope supports f16, f32 and f64 tokens");
+        // (bf16: in neither backend of the reference; the f16 kernels on bf16 elements)
+        if (m.dt_t != OPHIP_DT_F16 && m.dt_t != OPHIP_DT_BF16 && m.dt_t != OPHIP_DT_F32 && m.dt_t != OPHIP_DT_F64)
+            throw type_not_support("rope supports f16, bf16, f32 and f64 tokens");
         if (m.dt_p != OPHIP_DT_U32 && m.dt_p != OPHIP_DT_U64) throw type_not_support("rope supports u32 and u64 positions");
         const size_t nt = static_of(m.nt), nh = static_of(args->t_layout.shape[1]), dh = static_of(m.dh);
         const ptrdiff_t st = static_of(args->t_layout.strides[0]), sh = static_of(args->t_layout.strides[1]),
@@ -254,7 +257,8 @@ extern "C" int ophip_rope_launch(const ophip_rope *op, const ophip_rope_args *ar
         p.has_den = dh / 2 <= 128;
         if (p.has_den) op->denominators(args->theta, dh / 2, p.den);
 
-        const bool vec = m.dt_t == OPHIP_DT_F16 && dh % 8 == 0 && aligned16(p.t) && mult16(st) && mult16(sh);
+        const bool half = m.dt_t == OPHIP_DT_F16 || m.dt_t == OPHIP_DT_BF16;
+        const bool vec = half && dh % 8 == 0 && aligned16(p.t) && mult16(st) && mult16(sh);
         // split a token's heads over blockIdx.y when there are few tokens, keeping >= 256 items per block
         const size_t per_head = vec ? dh / 8 : dh / 2;
         size_t max_by = std::max<size_t>(1, nh * per_head / 256);
@@ -264,7 +268,10 @@ extern "C" int ophip_rope_launch(const ophip_rope *op, const ophip_rope_args *ar
         by = (nh + hpb - 1) / hpb;
         if (by > 65535) throw shape_not_support("too many heads");
         p.heads_per_block = (uint32_t)hpb;
-        hipFunction_t fn = vec ? op->f16_vec : m.dt_t == OPHIP_DT_F16 ? op->f16_pairs : m.dt_t == OPHIP_DT_F32 ? op->f32_pairs : op->f64_pairs;
+        hipFunction_t fn = m.dt_t == OPHIP_DT_F16    ? (vec ? op->f16_vec : op->f16_pairs)
+                           : m.dt_t == OPHIP_DT_BF16 ? (vec ? op->bf16_vec : op->bf16_pairs)
+                           : m.dt_t == OPHIP_DT_F32  ? op->f32_pairs
+                                                     : op->f64_pairs;
         op->dev->make_current();
         launch(fn, Dim3{(unsigned)nt, (unsigned)by}, Dim3{256}, smem, stream_of(qa), p);
     });
@@ -319,18 +326,21 @@ struct SoftmaxVariant {
 };
 
 struct ophip_fused_softmax : OpBase {
-    std::vector<SoftmaxVariant> variants;
-    hipFunction_t stream_fn, stream_f32, stream_f64, rows4[2];  // rows4: four rows per wave, 1 or 2 vectors per lane and row
+    std::vector<SoftmaxVariant> variants[2];  // [f16 / bf16]
+    hipFunction_t stream_fn[2], stream_f32, stream_f64, rows4[2];  // rows4 (f16): four rows per wave, 1 or 2 vectors per lane and row
     explicit ophip_fused_softmax(ophip_device *d) : OpBase(d) {
         static const int table[][3] = {{8, 1, 64},  {8, 2, 64},   {8, 4, 64},   {8, 1, 256},  {8, 2, 256},
                                        {8, 4, 256}, {8, 8, 256},  {8, 4, 1024}, {8, 8, 1024}, {1, 8, 64},
                                        {1, 16, 64}, {1, 8, 256},  {1, 16, 256}, {1, 32, 256}, {1, 16, 1024}};
-        for (auto &t : table) {
-            const std::string name = "softmax_f16_v" + std::to_string(t[0]) + "_p" + std::to_string(t[1]) + "_g" +
-                                     std::to_string(t[2]);
-            variants.push_back({t[0], t[1], t[2], d->kernel("fused_softmax", name.c_str())});
+        for (int e = 0; e < 2; ++e) {
+            const std::string tag = e ? "bf16" : "f16";
+            for (auto &t : table) {
+                const std::string name = "softmax_" + tag + "_v" + std::to_string(t[0]) + "_p" + std::to_string(t[1]) + "_g" +
+                                         std::to_string(t[2]);
+                variants[e].push_back({t[0], t[1], t[2], d->kernel("fused_softmax", name.c_str())});
+            }
+            stream_fn[e] = d->kernel("fused_softmax", ("softmax_" + tag + "_stream").c_str());
         }
-        stream_fn = d->kernel("fused_softmax", "softmax_f16_stream");
         stream_f32 = d->kernel("fused_softmax", "softmax_f32_stream");
         stream_f64 = d->kernel("fused_softmax", "softmax_f64_stream");
         rows4[0] = d->kernel("fused_softmax", "softmax_f16_rows4_p1");
@@ -352,7 +362,8 @@ extern "C" int ophip_fused_softmax_scheme(ophip_fused_softmax *, const ophip_fus
         if (ws) *ws = 0;
         if (args->att_layout.ndim != 3) throw rank_not_support("");
         const uint64_t dt = args->att_layout.dt;
-        if (dt != OPHIP_DT_F16 && dt != OPHIP_DT_F32 && dt != OPHIP_DT_F64) throw type_not_support("fused softmax supports f16, f32 and f64");
+        if (dt != OPHIP_DT_F16 && dt != OPHIP_DT_BF16 && dt != OPHIP_DT_F32 && dt != OPHIP_DT_F64)
+            throw type_not_support("fused softmax supports f16, bf16, f32 and f64");
     });
 }
 
@@ -361,7 +372,9 @@ extern "C" int ophip_fused_softmax_launch(const ophip_fused_softmax *op, const o
     return guard([&] {
         const ophip_tensor_layout &l = args->att_layout;
         if (l.ndim != 3) throw rank_not_support("");
-        if (l.dt != OPHIP_DT_F16 && l.dt != OPHIP_DT_F32 && l.dt != OPHIP_DT_F64) throw type_not_support("fused softmax supports f16, f32 and f64");
+        // (bf16: in neither backend of the reference; the f16 kernels on bf16 elements)
+        if (l.dt != OPHIP_DT_F16 && l.dt != OPHIP_DT_BF16 && l.dt != OPHIP_DT_F32 && l.dt != OPHIP_DT_F64)
+            throw type_not_support("fused softmax supports f16, bf16, f32 and f64");
         const ptrdiff_t unit = (ptrdiff_t)ophip_dtype_nbytes(l.dt);
         if (args->att_mask != OPHIP_MASK_NONE && args->att_mask != OPHIP_MASK_CAUSAL)
             throw args_not_support("unknown attention mask");
@@ -386,7 +399,7 @@ extern "C" int ophip_fused_softmax_launch(const ophip_fused_softmax *op, const o
         p.causal = causal;
 
         if (!p.att) throw args_not_support("null base address");
-        if (l.dt != OPHIP_DT_F16) {
+        if (l.dt != OPHIP_DT_F16 && l.dt != OPHIP_DT_BF16) {
             op->dev->make_current();
             launch(l.dt == OPHIP_DT_F32 ? op->stream_f32 : op->stream_f64, Dim3{(unsigned)rows}, Dim3{1024}, 0, stream_of(qa), p);
             return;
@@ -396,14 +409,15 @@ extern "C" int ophip_fused_softmax_launch(const ophip_fused_softmax *op, const o
         // narrowest group that holds the row in registers; with few rows prefer a
         // whole workgroup per row so more lanes pull on memory
         const SoftmaxVariant *pick = nullptr;
-        for (const auto &v : op->variants) {
+        const int e = l.dt == OPHIP_DT_BF16 ? 1 : 0;
+        for (const auto &v : op->variants[e]) {
             if (v.vec != want_vec) continue;
             if ((size_t)v.vec * v.pt * v.g < att) continue;
             if (rows < 2048 && v.g < 256 && att >= (size_t)256 * v.vec) continue;
             if (!pick || v.g < pick->g || (v.g == pick->g && v.pt < pick->pt)) pick = &v;
         }
         op->dev->make_current();
-        if (vec && att % 8 == 0 && att <= 1024 && rows >= 8192) {
+        if (e == 0 && vec && att % 8 == 0 && att <= 1024 && rows >= 8192) {
             // many short rows: four per wave, their loads in flight together (16384 waves of one 512-column row
             // each cost more in start-up than in traffic: [32, 512, 512] causal 9.6 -> see the kernel's note)
             const size_t waves = nh * ((seq + 3) / 4);
@@ -411,7 +425,7 @@ extern "C" int ophip_fused_softmax_launch(const ophip_fused_softmax *op, const o
             return;
         }
         if (!pick) {
-            launch(op->stream_fn, Dim3{(unsigned)rows}, Dim3{1024}, 0, stream_of(qa), p);
+            launch(op->stream_fn[e], Dim3{(unsigned)rows}, Dim3{1024}, 0, stream_of(qa), p);
             return;
         }
         const unsigned block = pick->g < 256 ? 256 : pick->g, rpb = block / pick->g;
@@ -647,8 +661,11 @@ extern "C" int ophip_rearrange_launch(const ophip_rearrange *op, const ophip_rea
 // Args::meta: swiglu/args.rs:31-50; launch checks: swiglu/cuda/mod.rs:53-98.
 
 struct ophip_swiglu : OpBase {
-    hipFunction_t f16_vec, f16_vec_nt, f16_scalar, f32_scalar, f64_scalar;
+    hipFunction_t f16_vec, f16_vec_nt, f16_scalar, f32_scalar, f64_scalar, bf16_vec, bf16_vec_nt, bf16_scalar;
     explicit ophip_swiglu(ophip_device *d) : OpBase(d) {
+        bf16_vec = d->kernel("swiglu", "swiglu_bf16_vec");
+        bf16_vec_nt = d->kernel("swiglu", "swiglu_bf16_vec_nt");
+        bf16_scalar = d->kernel("swiglu", "swiglu_bf16_scalar");
         f16_vec = d->kernel("swiglu", "swiglu_f16_vec");
         f16_scalar = d->kernel("swiglu", "swiglu_f16_scalar");
         f32_scalar = d->kernel("swiglu", "swiglu_f32_scalar");
@@ -690,7 +707,9 @@ extern "C" int ophip_swiglu_launch(const ophip_swiglu *op, const ophip_swiglu_ar
                                    const ophip_queue_alloc *qa) {
     return guard([&] {
         const SwigluMeta m = swiglu_meta(*args);
-        if (m.dt != OPHIP_DT_F16 && m.dt != OPHIP_DT_F32 && m.dt != OPHIP_DT_F64) throw type_not_support("swiglu supports f16, f32 and f64");
+        // (bf16: in neither backend of the reference; the f16 kernels on bf16 elements)
+        if (m.dt != OPHIP_DT_F16 && m.dt != OPHIP_DT_BF16 && m.dt != OPHIP_DT_F32 && m.dt != OPHIP_DT_F64)
+            throw type_not_support("swiglu supports f16, bf16, f32 and f64");
         const size_t n = static_of(m.n), d = static_of(m.d);
         const ptrdiff_t sgn = static_of(args->gate_layout.strides[0]), sgd = static_of(args->gate_layout.strides[1]);
         const ptrdiff_t sun = static_of(args->up_layout.strides[0]), sud = static_of(args->up_layout.strides[1]);
@@ -706,13 +725,18 @@ extern "C" int ophip_swiglu_launch(const ophip_swiglu *op, const ophip_swiglu_ar
         p.sun = sun;
         p.n = (uint32_t)n;
         p.d = (uint32_t)d;
-        const bool vec = m.dt == OPHIP_DT_F16 && d % 8 == 0 && aligned16(p.gate) && aligned16(p.up) && mult16(sgn) &&
+        const bool bf = m.dt == OPHIP_DT_BF16;
+        const bool vec = (m.dt == OPHIP_DT_F16 || bf) && d % 8 == 0 && aligned16(p.gate) && aligned16(p.up) && mult16(sgn) &&
                          mult16(sun);
         const size_t items = vec ? d / 8 : d;
         const unsigned gx = std::min<unsigned>(ceil_div(items, 256), 65535u);
         const unsigned gy = (unsigned)std::min<size_t>(n, 65535);
         const bool big = n * d * (size_t)unit >= ((size_t)64 << 20);  // more than the caches hold
-        hipFunction_t fn = vec ? (big ? op->f16_vec_nt : op->f16_vec) : m.dt == OPHIP_DT_F16 ? op->f16_scalar : m.dt == OPHIP_DT_F32 ? op->f32_scalar : op->f64_scalar;
+        hipFunction_t fn = vec ? (bf ? (big ? op->bf16_vec_nt : op->bf16_vec) : (big ? op->f16_vec_nt : op->f16_vec))
+                           : m.dt == OPHIP_DT_F16 ? op->f16_scalar
+                           : bf                   ? op->bf16_scalar
+                           : m.dt == OPHIP_DT_F32 ? op->f32_scalar
+                                                  : op->f64_scalar;
         if (!p.gate || !p.up) throw args_not_support("null base address");
         op->dev->make_current();
         launch(fn, Dim3{gx, gy}, Dim3{256}, 0, stream_of(qa), p);

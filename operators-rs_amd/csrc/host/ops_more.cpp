@@ -166,7 +166,8 @@ extern "C" int ophip_gelu_launch(const ophip_gelu *op, const ophip_gelu_args *ar
         const uint64_t dt = args->layout.dt;
         const size_t n = static_of(args->layout.shape[0]), d = static_of(args->layout.shape[1]);
         const ptrdiff_t sn = static_of(args->layout.strides[0]), sd = static_of(args->layout.strides[1]);
-        if (dt != OPHIP_DT_F16 && dt != OPHIP_DT_F32 && dt != OPHIP_DT_F64) throw type_not_support("gelu supports f16, f32 and f64");
+        // (bf16: in neither backend of the reference; the f16 kernels on bf16 elements)
+        if (!is_float_dt(dt)) throw type_not_support("gelu supports f16, bf16, f32 and f64");
         const ptrdiff_t unit = (ptrdiff_t)ophip_dtype_nbytes(dt);
         if (sd != unit) throw strides_not_support("gelu needs a contiguous inner dimension");
         if (sn % unit != 0) throw strides_not_support("misaligned strides");
@@ -177,14 +178,14 @@ extern "C" int ophip_gelu_launch(const ophip_gelu *op, const ophip_gelu_args *ar
         p.sn = sn;
         p.n = (uint32_t)n;
         p.d = (uint32_t)d;
-        const bool vec = dt == OPHIP_DT_F16 && d % 8 == 0 && aligned16(p.base) && mult16(sn);
+        const bool vec = (dt == OPHIP_DT_F16 || dt == OPHIP_DT_BF16) && d % 8 == 0 && aligned16(p.base) && mult16(sn);
         const size_t items = vec ? d / 8 : d;
         const unsigned gx = std::min<unsigned>(ceil_div(items, 256), 65535u);
         const unsigned gy = (unsigned)std::min<size_t>(n, 65535);
-        const char *name = vec ? "gelu_f16_vec" : dt == OPHIP_DT_F16 ? "gelu_f16_scalar" : dt == OPHIP_DT_F32 ? "gelu_f32_scalar" : "gelu_f64_scalar";
+        const std::string name = std::string("gelu_") + dt_tag(dt) + (vec ? "_vec" : "_scalar");
         if (!p.base) throw args_not_support("null base address");
         op->dev->make_current();
-        launch(op->dev->kernel("gelu", name), Dim3{gx, gy}, Dim3{256}, 0, stream_of(qa), p);
+        launch(op->dev->kernel("gelu", name.c_str()), Dim3{gx, gy}, Dim3{256}, 0, stream_of(qa), p);
     });
 }
 

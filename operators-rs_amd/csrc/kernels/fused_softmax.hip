@@ -19,7 +19,9 @@ __device__ __forceinline__ uint32_t kept_columns(const SoftmaxParams &p, uint32_
 // VEC = 8: 16-byte accesses (16-byte aligned rows; the last, partial group of an att_len that is no
 // multiple of 8 goes element by element, so nothing past att_len is read or written); VEC = 1: element-wise.
 // PT = register slots per thread (vectors or elements).
-template <int VEC, int PT, int G>
+// T: f16, or bf16 (which neither backend of the reference has for this operator: the same arithmetic, the stored
+// exponential rounded to bf16 where the f16 path rounds it to f16).
+template <typename T, int VEC, int PT, int G>
 __device__ __forceinline__ void softmax_reg(const SoftmaxParams &p) {
     constexpr int BLOCK = G < 256 ? 256 : G;
     constexpr int RPB = BLOCK / G;
@@ -32,7 +34,7 @@ __device__ __forceinline__ void softmax_reg(const SoftmaxParams &p) {
     if (!live) flat = rows - 1;
     const uint32_t h = flat / p.seq, r = flat % p.seq;
     const uint32_t kept = kept_columns(p, r);
-    f16 *row = reinterpret_cast<f16 *>(reinterpret_cast<char *>(p.att) + (int64_t)h * p.sh + (int64_t)r * p.ss);
+    T *row = reinterpret_cast<T *>(reinterpret_cast<char *>(p.att) + (int64_t)h * p.sh + (int64_t)r * p.ss);
 
     float x[PT][VEC];
     float mx = -INFINITY;
@@ -40,7 +42,7 @@ __device__ __forceinline__ void softmax_reg(const SoftmaxParams &p) {
     for (int i = 0; i < PT; ++i) {
         const uint32_t col0 = (lane + i * G) * VEC;
         if constexpr (VEC == 8) {
-            Pack8 v;
+            PackOf<T> v;
             v.u = u32x4{0, 0, 0, 0};
             if (col0 + 8 <= p.att_len) {
                 if (col0 < kept) v.u = ld128_nt(row + col0);
@@ -51,11 +53,11 @@ __device__ __forceinline__ void softmax_reg(const SoftmaxParams &p) {
             }
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                x[i][e] = col0 + e < kept ? h2f(v.e[e]) : -INFINITY;
+                x[i][e] = col0 + e < kept ? (float)v.e[e] : -INFINITY;
                 mx = fmaxf(mx, x[i][e]);
             }
         } else {
-            x[i][0] = col0 < kept ? h2f(row[col0]) : -INFINITY;
+            x[i][0] = col0 < kept ? (float)row[col0] : -INFINITY;
             mx = fmaxf(mx, x[i][0]);
         }
     }
@@ -70,7 +72,7 @@ __device__ __forceinline__ void softmax_reg(const SoftmaxParams &p) {
             if (col < kept) {
                 const float ex = fast_exp(x[i][e] - mx);
                 sum += ex;
-                x[i][e] = h2f(f2h(ex));  // the reference stores f16(e) and re-reads it
+                x[i][e] = (float)(T)ex;  // the reference stores f16(e) and re-reads it
             } else {
                 x[i][e] = 0.f;
             }
@@ -83,9 +85,9 @@ __device__ __forceinline__ void softmax_reg(const SoftmaxParams &p) {
         const uint32_t col0 = (lane + i * G) * VEC;
         if (col0 < p.att_len && live) {
             if constexpr (VEC == 8) {
-                Pack8 o;
+                PackOf<T> o;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) o.e[e] = col0 + e < kept ? f2h(x[i][e] * inv) : (f16)0.f;
+                for (int e = 0; e < 8; ++e) o.e[e] = col0 + e < kept ? (T)(x[i][e] * inv) : (T)0.f;
                 if (col0 + 8 <= p.att_len) {
                     st128(row + col0, o.u);
                 } else {
@@ -94,7 +96,7 @@ __device__ __forceinline__ void softmax_reg(const SoftmaxParams &p) {
                         if (col0 + e < p.att_len) row[col0 + e] = o.e[e];
                 }
             } else {
-                row[col0] = col0 < kept ? f2h(x[i][0] * inv) : (f16)0.f;
+                row[col0] = col0 < kept ? (T)(x[i][0] * inv) : (T)0.f;
             }
         }
     }
@@ -207,27 +209,30 @@ extern "C" __global__ void __launch_bounds__(256) softmax_f16_rows4_p2(SoftmaxPa
 
 // Any att_len: one 1024-thread workgroup per row, three sweeps (max; exp + sum,
 // storing f16(e); scale), O(1) LDS.
-extern "C" __global__ void __launch_bounds__(1024) softmax_f16_stream(SoftmaxParams p) {
+template <typename T>
+__device__ __forceinline__ void softmax_stream(const SoftmaxParams &p) {  // T: f16 or bf16
     constexpr int G = 1024;
     __shared__ float smem[G / WAVE];
     const uint32_t flat = blockIdx.x;
     const uint32_t h = flat / p.seq, r = flat % p.seq;
     const uint32_t kept = kept_columns(p, r);
-    f16 *row = reinterpret_cast<f16 *>(reinterpret_cast<char *>(p.att) + (int64_t)h * p.sh + (int64_t)r * p.ss);
+    T *row = reinterpret_cast<T *>(reinterpret_cast<char *>(p.att) + (int64_t)h * p.sh + (int64_t)r * p.ss);
     float mx = -INFINITY;
-    for (uint32_t c = threadIdx.x; c < kept; c += G) mx = fmaxf(mx, h2f(row[c]));
+    for (uint32_t c = threadIdx.x; c < kept; c += G) mx = fmaxf(mx, (float)row[c]);
     mx = group_max<G>(mx, smem);
     float sum = 0.f;
     for (uint32_t c = threadIdx.x; c < kept; c += G) {
-        const float ex = fast_exp(h2f(row[c]) - mx);
+        const float ex = fast_exp((float)row[c] - mx);
         sum += ex;
-        row[c] = f2h(ex);
+        row[c] = (T)ex;
     }
     sum = group_sum<G>(sum, smem);
     const float inv = 1.0f / sum;
-    for (uint32_t c = threadIdx.x; c < kept; c += G) row[c] = f2h(h2f(row[c]) * inv);
-    for (uint32_t c = kept + threadIdx.x; c < p.att_len; c += G) row[c] = (f16)0.f;
+    for (uint32_t c = threadIdx.x; c < kept; c += G) row[c] = (T)((float)row[c] * inv);
+    for (uint32_t c = kept + threadIdx.x; c < p.att_len; c += G) row[c] = (T)0.f;
 }
+extern "C" __global__ void __launch_bounds__(1024) softmax_f16_stream(SoftmaxParams p) { softmax_stream<f16>(p); }
+extern "C" __global__ void __launch_bounds__(1024) softmax_bf16_stream(SoftmaxParams p) { softmax_stream<bf16>(p); }
 
 // f32 and f64 rows (fuesd_softmax/common_cpu/mod.rs:147-193): the same three sweeps in the element's own arithmetic, the
 // library's exp; one 1024-thread workgroup per row.  No register-resident variants: the hot path is f16.
@@ -273,7 +278,11 @@ extern "C" __global__ void __launch_bounds__(1024) softmax_f64_stream(SoftmaxPar
 #define SOFTMAX_REG(VEC, PT, G)                                                                  \
     extern "C" __global__ void __launch_bounds__((G) < 256 ? 256 : (G))                          \
         softmax_f16_v##VEC##_p##PT##_g##G(SoftmaxParams p) {                                     \
-        softmax_reg<VEC, PT, G>(p);                                                              \
+        softmax_reg<f16, VEC, PT, G>(p);                                                         \
+    }                                                                                            \
+    extern "C" __global__ void __launch_bounds__((G) < 256 ? 256 : (G))                          \
+        softmax_bf16_v##VEC##_p##PT##_g##G(SoftmaxParams p) {                                    \
+        softmax_reg<bf16, VEC, PT, G>(p);                                                        \
     }
 
 // vector variants: capacity = 8 * PT * G columns

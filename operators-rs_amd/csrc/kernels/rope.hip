@@ -32,7 +32,8 @@ __device__ __forceinline__ void rope_fill_table(const RopeParams &p, uint32_t to
     __syncthreads();
 }
 
-extern "C" __global__ void __launch_bounds__(256) rope_f16_vec(RopeParams p) {
+template <typename T>
+__device__ __forceinline__ void rope_vec(const RopeParams &p) {  // T: f16 or bf16
     const uint32_t token = blockIdx.x;
     const uint32_t cpv = p.dh / 8;  // 16-byte chunks per head
     const uint32_t h0 = blockIdx.y * p.heads_per_block;
@@ -42,26 +43,29 @@ extern "C" __global__ void __launch_bounds__(256) rope_f16_vec(RopeParams p) {
     auto chunk = [&](uint32_t v) { return base + (int64_t)(h0 + v / cpv) * p.sh + (size_t)(v % cpv) * 16; };
     // The thread's first chunk is requested before the table is filled (a load of pos, the transcendentals, a
     // barrier): on a few tokens the kernel is nothing but latency, and this takes one memory latency out of it.
-    Pack8 first;
+    PackOf<T> first;
     first.u = u32x4{0, 0, 0, 0};
     if (threadIdx.x < total) first.u = ld128(chunk(threadIdx.x));
     rope_fill_table(p, token);
     for (uint32_t v = threadIdx.x; v < total; v += blockDim.x) {
         const uint32_t c = v % cpv;
         char *ptr = chunk(v);
-        Pack8 x, o;
+        PackOf<T> x, o;
         if (v == threadIdx.x) x.u = first.u;
         else x.u = ld128(ptr);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const float2 sc = rope_sc[4 * c + i];
-            const float a = h2f(x.e[2 * i]), b = h2f(x.e[2 * i + 1]);
-            o.e[2 * i] = f2h(a * sc.y - b * sc.x);
-            o.e[2 * i + 1] = f2h(a * sc.x + b * sc.y);
+            const float a = (float)x.e[2 * i], b = (float)x.e[2 * i + 1];
+            o.e[2 * i] = (T)(a * sc.y - b * sc.x);
+            o.e[2 * i + 1] = (T)(a * sc.x + b * sc.y);
         }
         st128(ptr, o.u);
     }
 }
+extern "C" __global__ void __launch_bounds__(256) rope_f16_vec(RopeParams p) { rope_vec<f16>(p); }
+// bf16: neither backend of the reference has it for this operator; the f16 kernels on bf16 elements (f32 inside, one rounding)
+extern "C" __global__ void __launch_bounds__(256) rope_bf16_vec(RopeParams p) { rope_vec<bf16>(p); }
 
 template <typename T>
 __device__ __forceinline__ void rope_pairs(const RopeParams &p) {
@@ -83,6 +87,7 @@ __device__ __forceinline__ void rope_pairs(const RopeParams &p) {
 }
 
 extern "C" __global__ void __launch_bounds__(256) rope_f16_pairs(RopeParams p) { rope_pairs<f16>(p); }
+extern "C" __global__ void __launch_bounds__(256) rope_bf16_pairs(RopeParams p) { rope_pairs<bf16>(p); }
 extern "C" __global__ void __launch_bounds__(256) rope_f32_pairs(RopeParams p) { rope_pairs<float>(p); }
 
 // f64 tokens (rope/common_cpu/mod.rs:125-126): position, angle, sine and cosine in f64, as the reference computes them;

@@ -14,25 +14,28 @@ __device__ __forceinline__ float swiglu_f32(float a, float b) {
 
 // NT: more data than the caches hold (the host decides): the result is stored with the non-temporal hint as well.
 // (Separate builds: a flag in the parameters would make the compiler merge the two stores of an if / else and drop the hint.)
-template <bool NT>
-__device__ __forceinline__ void swiglu_vec(const SwigluParams &p) {
+template <typename T, bool NT>
+__device__ __forceinline__ void swiglu_vec(const SwigluParams &p) {  // T: f16 or bf16
     const uint32_t nvec = p.d / 8;
     for (uint32_t row = blockIdx.y; row < p.n; row += gridDim.y) {
         char *g = reinterpret_cast<char *>(p.gate) + (int64_t)row * p.sgn;
         const char *u = reinterpret_cast<const char *>(p.up) + (int64_t)row * p.sun;
         for (uint32_t v = blockIdx.x * blockDim.x + threadIdx.x; v < nvec; v += gridDim.x * blockDim.x) {
-            Pack8 a, b, o;
+            PackOf<T> a, b, o;
             a.u = ld128_nt(g + (size_t)v * 16);
             b.u = ld128_nt(u + (size_t)v * 16);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) o.e[i] = f2h(swiglu_f32(h2f(a.e[i]), h2f(b.e[i])));
+            for (int i = 0; i < 8; ++i) o.e[i] = (T)swiglu_f32((float)a.e[i], (float)b.e[i]);
             if constexpr (NT) st128_nt(g + (size_t)v * 16, o.u);
             else st128(g + (size_t)v * 16, o.u);
         }
     }
 }
-extern "C" __global__ void __launch_bounds__(256) swiglu_f16_vec(SwigluParams p) { swiglu_vec<false>(p); }
-extern "C" __global__ void __launch_bounds__(256) swiglu_f16_vec_nt(SwigluParams p) { swiglu_vec<true>(p); }
+extern "C" __global__ void __launch_bounds__(256) swiglu_f16_vec(SwigluParams p) { swiglu_vec<f16, false>(p); }
+extern "C" __global__ void __launch_bounds__(256) swiglu_f16_vec_nt(SwigluParams p) { swiglu_vec<f16, true>(p); }
+// bf16: neither backend of the reference has it for this operator; the f16 kernels on bf16 elements (f32 inside, one rounding)
+extern "C" __global__ void __launch_bounds__(256) swiglu_bf16_vec(SwigluParams p) { swiglu_vec<bf16, false>(p); }
+extern "C" __global__ void __launch_bounds__(256) swiglu_bf16_vec_nt(SwigluParams p) { swiglu_vec<bf16, true>(p); }
 
 // f64 data is computed in f64, as the reference does (swiglu/common_cpu/mod.rs:74-76): the library's exp, an IEEE division
 __device__ __forceinline__ double swiglu_f64(double a, double b) { return (a * (1.0 / (1.0 + exp(-a)))) * b; }
@@ -50,5 +53,6 @@ __device__ __forceinline__ void swiglu_scalar(const SwigluParams &p) {
 }
 
 extern "C" __global__ void __launch_bounds__(256) swiglu_f16_scalar(SwigluParams p) { swiglu_scalar<f16>(p); }
+extern "C" __global__ void __launch_bounds__(256) swiglu_bf16_scalar(SwigluParams p) { swiglu_scalar<bf16>(p); }
 extern "C" __global__ void __launch_bounds__(256) swiglu_f32_scalar(SwigluParams p) { swiglu_scalar<float>(p); }
 extern "C" __global__ void __launch_bounds__(256) swiglu_f64_scalar(SwigluParams p) { swiglu_scalar<double>(p); }

@@ -1,10 +1,11 @@
-"""bf16 data on rms_norm, layer_norm, add, add_rows and (further down) mat_mul, through the C ABI.
+"""bf16 data on every floating-point operator, through the C ABI.
 
-The reference's CUDA backend compiles these four for any pair of named types, bf16 included (handle/cuda/mod.rs:188-210
-with rms_norm/cuda/mod.rs:146-147, layer_norm/cuda/mod.rs:158-159, add/cuda/mod.rs:105-123, add_rows/cuda/mod.rs:135-163);
-its CPU backend, which the oracle restates, has no bf16 kernel.  PARITY UNPINNED against the reference: what is checked here
-is the arithmetic the kernels document -- the f16 kernels' formulas in f32, one rounding to bf16 (nearest even) at the end --
-against the same formula in f64 (the norms: within one bf16 step, 2^-7 relative) or in numpy f32 (the sums: every bit)."""
+The reference's CUDA backend compiles rms_norm, layer_norm, add and add_rows for any pair of named types, bf16 included
+(handle/cuda/mod.rs:188-210 with rms_norm/cuda/mod.rs:146-147, layer_norm/cuda/mod.rs:158-159, add/cuda/mod.rs:105-123,
+add_rows/cuda/mod.rs:135-163); its CPU backend, which the oracle restates, has no bf16 kernel at all, and for rope,
+softmax, swiglu, gelu and mat_mul neither backend has one.  PARITY UNPINNED against the reference: what is checked here is
+the arithmetic the kernels document -- the f16 kernels' formulas in f32, one rounding to bf16 (nearest even) at the end --
+against the same formula in f64 (within one bf16 step, 2^-7 relative) or in numpy f32 (the sums: every bit)."""
 import numpy as np
 import pytest
 
@@ -163,11 +164,99 @@ def test_add_rows_bf16_every_bit(gpu, stream, b, m, n, k, idt):
     assert np.array_equal(out, to_bf16(from_bf16(dst) + from_bf16(src)[idx.astype(np.int64)]))
 
 
-def test_bf16_still_refused_where_no_backend_of_the_reference_takes_it(gpu, stream):
-    # rope, softmax, swiglu, gelu, mat_mul: the CUDA backend checks for F16 (rope/cuda/mod.rs:94, fuesd_softmax/cuda/mod.rs:75,
-    # swiglu/cuda/mod.rs:69, gelu/cuda/mod.rs, mat_mul/cuda/mod.rs:73) and the CPU backend has no bf16
-    B = dt.BF16
-    c = lambda *s: TensorLayout.new_contiguous(B, list(s))
+# ---------------------------------------- rope, softmax, swiglu, gelu ----
+# Neither backend of the reference has bf16 for these four (rope/cuda/mod.rs:94, fuesd_softmax/cuda/mod.rs:75,
+# swiglu/cuda/mod.rs:69 and gelu's check for F16; the CPU backend lists f16, f32, f64): parity unpinned.  They are the f16
+# kernels on bf16 elements, so that a bf16 model's layer runs end to end; checked against f64 within one bf16 step.
+
+@pytest.mark.parametrize("n,d", [(16, 11008), (3, 1001), (1, 8), (9000, 4096)])
+def test_swiglu_and_gelu_bf16(gpu, stream, n, d):
+    rng = np.random.default_rng(n + d)
+    g, u = to_bf16(rng.standard_normal((n, d)).astype(f32) * f32(2)), to_bf16(rng.standard_normal((n, d)).astype(f32))
+    gd, ud = gpu.from_host(g), gpu.from_host(u)
+    lay = L2(dt.BF16, n, d)
+    say("swiglu bf16 n=%d d=%d" % (n, d))
+    ophip.Swiglu(gpu).launch(ophip.SwigluArgs(lay, gd, lay, ud), None, stream)
+    a, b = from_bf16(g).astype(f64), from_bf16(u).astype(f64)
+    ref = a / (1 + np.exp(-a)) * b
+    y = from_bf16(gpu.to_host(gd, u16, n * d, stream=stream)).reshape(n, d).astype(f64)
+    assert (np.abs(y - ref) <= one_step(ref) + 1e-6).all(), np.abs(y - ref).max()
+    xd = gpu.from_host(g)
+    say("gelu bf16 n=%d d=%d" % (n, d))
+    ophip.Gelu(gpu).launch(ophip.GeluArgs(lay, xd), None, stream)
+    ref = 0.5 * a * (1 + np.tanh(np.sqrt(2 / np.pi) * (a + 0.044715 * a ** 3)))
+    y = from_bf16(gpu.to_host(xd, u16, n * d, stream=stream)).reshape(n, d).astype(f64)
+    assert (np.abs(y - ref) <= one_step(ref) + 1e-6).all(), np.abs(y - ref).max()
+
+
+@pytest.mark.parametrize("pdt", [np.uint32, np.uint64])
+@pytest.mark.parametrize("shape", [(16, 64, 128), (7, 3, 64), (5, 4, 20), (512, 32, 128)])
+def test_rope_bf16(gpu, stream, shape, pdt):
+    import oracle
+    rng = np.random.default_rng(sum(shape))
+    tb = to_bf16(rng.standard_normal(shape).astype(f32))
+    pos = rng.integers(0, 4096, shape[0]).astype(pdt)
+    td, pd = gpu.from_host(tb), gpu.from_host(pos)
+    nt, nh, dh = shape
+    t_lay = TensorLayout(dt.BF16, list(shape), [nh * dh * 2, dh * 2, 2])
+    empty = TensorLayout(dt.BF16, [0, dh], [dh * 2, 2])
+    say("rope bf16 %s %s" % (shape, np.dtype(pdt).name))
+    ophip.Rope(gpu).launch(ophip.RopeArgs(t_lay, td, TensorLayout.of(pos), pd, empty, None, empty, None, 1e4), None, stream)
+    y = from_bf16(gpu.to_host(td, u16, tb.size, stream=stream)).reshape(shape).astype(f64)
+    ref = oracle.rope(from_bf16(tb).copy(), pos, 1e4).astype(f64)   # the oracle's f32 path on the same numbers
+    # |a c - b s| is at most the pair's norm: one bf16 step of that
+    norm = np.sqrt((from_bf16(tb).astype(f64).reshape(nt, nh, dh // 2, 2) ** 2).sum(-1, keepdims=True)).repeat(2, -1).reshape(shape)
+    assert (np.abs(y - ref) <= norm * 2.0 ** -7 + 1e-6).all(), np.abs(y - ref).max()
+
+
+@pytest.mark.parametrize("shape,causal", [((32, 16, 2048), True), ((4, 7, 511), True), ((2, 3, 8), False), ((3, 300, 300), True),
+                                          ((1, 2, 20000), True), ((1, 1, 70000), False)])
+def test_softmax_bf16(gpu, stream, shape, causal):
+    rng = np.random.default_rng(sum(shape))
+    ab = to_bf16(rng.standard_normal(shape).astype(f32) * f32(2))
+    ad = gpu.from_host(ab)
+    nh, seq, al = shape
+    lay = TensorLayout(dt.BF16, list(shape), [seq * al * 2, al * 2, 2])
+    say("softmax bf16 %s causal=%s" % (shape, causal))
+    ophip.FusedSoftmax(gpu).launch(ophip.FusedSoftmaxArgs(ophip.AttnMask.CAUSAL if causal else ophip.AttnMask.NONE, lay, ad), None, stream)
+    y = from_bf16(gpu.to_host(ad, u16, ab.size, stream=stream)).reshape(shape).astype(f64)
+    x = from_bf16(ab).astype(f64)
+    if causal:
+        keep = np.arange(al)[None, :] <= (al - seq + np.arange(seq))[:, None]
+        x = np.where(keep[None], x, -np.inf)
+    e = np.exp(x - x.max(-1, keepdims=True))
+    ref = e / e.sum(-1, keepdims=True)
+    assert (np.abs(y - ref) <= one_step(ref) + 1e-12).all(), (np.abs(y - ref) / one_step(ref)).max()
+    if causal:
+        assert (y[~np.broadcast_to(keep[None], shape)] == 0).all()
+
+
+def test_attention_bf16_runs_on_the_composite(gpu, stream):
+    """mat_mul, softmax and rearrange all take bf16, so the composite of launches does: against f64."""
+    rng = np.random.default_rng(31)
+    nh, nkvh, seq, att, dh = 8, 2, 40, 136, 64
+    q, k, v = (to_bf16(rng.standard_normal(s).astype(f32)) for s in ((nh, seq, dh), (nkvh, att, dh), (nkvh, att, dh)))
+    qd, kd, vd, od = gpu.from_host(q), gpu.from_host(k), gpu.from_host(v), gpu.malloc(q.nbytes)
+    c = lambda *s: TensorLayout.new_contiguous(dt.BF16, list(s))
+    op = ophip.Attention(gpu)
+    args = ophip.AttentionArgs(c(nh, seq, dh), qd, c(nkvh, att, dh), kd, c(nkvh, att, dh), vd, c(nh, seq, dh), od, ophip.AttnMask.CAUSAL)
+    ws = gpu.malloc(max(op.scheme(args, 1 << 30), 16))
+    say("attention bf16 (composite)")
+    op.launch(args, ws, stream)
+    y = from_bf16(gpu.to_host(od, u16, q.size, stream=stream)).reshape(nh, seq, dh).astype(f64)
+    g = nh // nkvh
+    kk, vv = np.repeat(from_bf16(k).astype(f64), g, axis=0), np.repeat(from_bf16(v).astype(f64), g, axis=0)
+    s = np.einsum("hsd,had->hsa", from_bf16(q).astype(f64), kk) / np.sqrt(dh)
+    s = np.where((np.arange(att)[None, :] <= (att - seq + np.arange(seq))[:, None])[None], s, -np.inf)
+    pr = np.exp(s - s.max(-1, keepdims=True))
+    ref = np.einsum("hsa,had->hsd", pr / pr.sum(-1, keepdims=True), vv)
+    # scores and probabilities are rounded to bf16 between the launches: a few steps of the output's scale
+    assert np.abs(y - ref).max() <= 4 * 2.0 ** -7 * np.abs(ref).max(), np.abs(y - ref).max()
+
+
+def test_types_no_kernel_takes_are_refused(gpu, stream):
+    U = dt.U16
+    c = lambda *s: TensorLayout.new_contiguous(U, list(s))
     with pytest.raises(ophip.LaunchError) as e:
         ophip.Swiglu(gpu).launch(ophip.SwigluArgs(c(4, 8), None, c(4, 8), None), None, stream)
     assert e.value.kind == "TypeNotSupport"

@@ -350,7 +350,7 @@ def test_softmax_errors(gpu, stream):
         op.scheme(ophip.FusedSoftmaxArgs(1, L(dt.F16, [4, 4], [8, 2]), None), 0)
     assert e.value.kind == "RankNotSupport"
     with pytest.raises(ophip.SchemeError) as e:
-        op.scheme(ophip.FusedSoftmaxArgs(1, L(dt.BF16, [1, 4, 4], [32, 8, 2]), None), 0)
+        op.scheme(ophip.FusedSoftmaxArgs(1, L(dt.U16, [1, 4, 4], [32, 8, 2]), None), 0)
     assert e.value.kind == "TypeNotSupport"
     with pytest.raises(ophip.LaunchError) as e:
         op.launch(ophip.FusedSoftmaxArgs(1, L(dt.F16, [1, 4, 4], [64, 16, 4]), None), None, stream)
