@@ -471,17 +471,21 @@ def attention_lines(o, gpu, stream, rng, add, reps, full=False):
     """attention at prefill shapes (32 heads, dh 128): one pass with the scores kept on the chip where the crate's
     composite writes and reads the [nh, seq, att] score matrix four times.  flops = 4 nh seq att dh, half of it under a
     causal mask (the part of the score matrix the mask keeps); bytes = q, k, v, o once.  `full`: the unmasked shapes too."""
-    L, F16 = o.TensorLayout, o.dt.F16
-    c = lambda *s: L.new_contiguous(F16, list(s))
+    L = o.TensorLayout
     at = o.Attention(gpu)
-    for seq, causal in [(512, True), (2048, True), (4096, True)] + ([(2048, False), (4096, False)] if full else []):
-        q, k, v = (gpu.from_host(normal_f16(rng, (NH, seq, DH), 1.0)) for _ in range(3))
+    cases = [(512, True, False), (2048, True, False), (2048, True, True), (4096, True, False)]
+    for seq, causal, bf in cases + ([(2048, False, False), (4096, False, False)] if full else []):
+        c = lambda *s: L.new_contiguous(o.dt.BF16 if bf else o.dt.F16, list(s))
+        # (bf16: the top halves of f32 normals, which are bf16 normals of the same spread)
+        mk = (lambda: (rng.standard_normal((NH, seq, DH), dtype=np.float32).view(np.uint32) >> 16).astype(np.uint16)) if bf else \
+            (lambda: normal_f16(rng, (NH, seq, DH), 1.0))
+        q, k, v = (gpu.from_host(mk()) for _ in range(3))
         od = gpu.malloc(NH * seq * DH * 2)
         a = o.AttentionArgs(c(NH, seq, DH), q, c(NH, seq, DH), k, c(NH, seq, DH), v, c(NH, seq, DH), od,
                             o.AttnMask.CAUSAL if causal else o.AttnMask.NONE)
         us = time_launches(gpu, stream, lambda: at.launch(a, None, stream), reps)
-        add("attention", "nh32 seq%d att%d dh128 %s" % (seq, seq, "causal" if causal else "no mask"), 4 * NH * seq * DH * 2, us,
-            flops=(2 if causal else 4) * NH * seq * seq * DH,
+        add("attention", "nh32 seq%d att%d dh128 %s%s" % (seq, seq, "causal" if causal else "no mask", " bf16" if bf else ""),
+            4 * NH * seq * DH * 2, us, flops=(2 if causal else 4) * NH * seq * seq * DH,
             note="one pass (attention_prefill.hip)" + ("; flops count the unmasked half of the scores" if causal else ""))
         for m_ in (q, k, v, od):
             m_.free()

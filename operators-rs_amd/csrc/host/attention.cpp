@@ -93,8 +93,8 @@ struct ophip_attention {
     ophip_mat_mul *mat_mul = nullptr;
     ophip_fused_softmax *softmax = nullptr;
     ophip_rearrange *rearrange = nullptr;
-    // the one-pass kernel for many query rows: [dh 64 / 128][4 waves on all key tiles / 8 waves, even and odd key tiles]
-    hipFunction_t prefill[2][2] = {};
+    // the one-pass kernel for many query rows: [f16 / bf16][dh 64 / 128][4 waves on all key tiles / 8 waves, even and odd key tiles]
+    hipFunction_t prefill[2][2][2] = {};
     int key_split = -1;  // OPHIP_ATTN_KEYSPLIT=0|1 keeps one of the two builds (sweeps); read once, here
     // OPHIP_ATTN_FUSED=0 keeps the composite (tests, comparisons), =1 takes the one-pass kernel wherever it applies;
     // read once, here.  Otherwise an estimate of the two times decides (attention_one_pass).
@@ -105,10 +105,13 @@ struct ophip_attention {
             sub(ophip_mat_mul_create(d, &mat_mul));
             sub(ophip_fused_softmax_create(d, &softmax));
             sub(ophip_rearrange_create(d, &rearrange));
-            prefill[0][0] = d->kernel("attention_prefill", "attn_prefill_d64");
-            prefill[1][0] = d->kernel("attention_prefill", "attn_prefill_d128");
-            prefill[0][1] = d->kernel("attention_prefill", "attn_prefill_d64_g2");
-            prefill[1][1] = d->kernel("attention_prefill", "attn_prefill_d128_g2");
+            for (int e = 0; e < 2; ++e) {
+                const std::string mod = e ? "attention_prefill_bf16" : "attention_prefill", tag = e ? "_bf16" : "";
+                prefill[e][0][0] = d->kernel(mod.c_str(), ("attn_prefill_d64" + tag).c_str());
+                prefill[e][1][0] = d->kernel(mod.c_str(), ("attn_prefill_d128" + tag).c_str());
+                prefill[e][0][1] = d->kernel(mod.c_str(), ("attn_prefill_d64_g2" + tag).c_str());
+                prefill[e][1][1] = d->kernel(mod.c_str(), ("attn_prefill_d128_g2" + tag).c_str());
+            }
             if (const char *e = std::getenv("OPHIP_ATTN_FUSED")) fused = std::atoi(e) != 0;
             if (const char *e = std::getenv("OPHIP_ATTN_KEYSPLIT")) key_split = std::atoi(e) != 0;
         } catch (...) {
@@ -178,7 +181,7 @@ size_t attention_scheme(ophip_attention *op, const ophip_attention_args &args, s
 // `merged`: the reference would use q in place and leave att . v in it.
 bool attention_one_pass(const ophip_attention *op, const ophip_attention_args &args, const AttentionMeta &m, bool merged,
                         const ophip_queue_alloc *qa) {
-    if (op->fused == 0 || m.dt != OPHIP_DT_F16) return false;
+    if (op->fused == 0 || (m.dt != OPHIP_DT_F16 && m.dt != OPHIP_DT_BF16)) return false;
     const size_t nh = static_of(m.nh), nkvh = static_of(m.nkvh), seq = static_of(m.seq), att = static_of(m.att), dh = static_of(m.dh);
     if ((dh != 64 && dh != 128) || nh == 0 || seq == 0 || att == 0 || nh > 0x7fffffffu || seq > 0x7fffffffu || att > 0x7fffffffu) return false;
     if (args.mask != OPHIP_MASK_NONE && args.mask != OPHIP_MASK_CAUSAL) return false;
@@ -243,7 +246,8 @@ bool attention_one_pass(const ophip_attention *op, const ophip_attention_args &a
     p.att = (uint32_t)att;
     p.causal = args.mask == OPHIP_MASK_CAUSAL;
     p.nblocks = (uint32_t)((seq + 127) / 128);
-    p.scale = round_to_f16(1.0f / std::sqrt((float)dh));  // the reference's mat_mul rounds alpha to the data type
+    // the reference's mat_mul rounds alpha to the data type
+    p.scale = m.dt == OPHIP_DT_BF16 ? round_to_bf16(1.0f / std::sqrt((float)dh)) : round_to_f16(1.0f / std::sqrt((float)dh));
     if (p.nblocks > 65535) return false;
     op->dev->make_current();
     // Under a causal mask the block with the most keys decides once there are no more workgroups than places for
@@ -251,7 +255,7 @@ bool attention_one_pass(const ophip_attention *op, const ophip_attention_args &a
     // 67.9 against 73.1 us, 512 x 512 19.5 against 21.3; 4096 x 4096 232 against 203, and without a mask it always loses)
     // (and whenever there are fewer workgroups than CUs: a lone workgroup's walk takes 2.7 us per two tiles against 1.75 us per tile)
     const bool split = op->key_split >= 0 ? op->key_split != 0 : wgs <= cus || (p.causal && wgs <= 2 * cus);
-    launch(op->prefill[dh == 64 ? 0 : 1][split], Dim3{(unsigned)nh, p.nblocks}, Dim3{split ? 512u : 256u}, 0, stream_of(qa), p);
+    launch(op->prefill[m.dt == OPHIP_DT_BF16 ? 1 : 0][dh == 64 ? 0 : 1][split], Dim3{(unsigned)nh, p.nblocks}, Dim3{split ? 512u : 256u}, 0, stream_of(qa), p);
     return true;
 }
 
@@ -329,8 +333,8 @@ struct ophip_attention_kv_cached {
     ophip_device *dev;
     ophip_rearrange *rearrange = nullptr;
     ophip_attention *attention = nullptr;
-    // the one-pass kernels for decode shapes: [16 * {1, 2, 4} query rows per kv head][dh 64 / 128]
-    hipFunction_t decode[3][2][2], combine[3][2];  // decode: [..][..][256 / 128 keys per workgroup]
+    // the one-pass kernels for decode shapes: [f16 / bf16][16 * {1, 2, 4} query rows per kv head][dh 64 / 128]
+    hipFunction_t decode[2][3][2][2], combine[2][3][2];  // decode: [..][..][..][256 / 128 keys per workgroup]
     bool one_pass = true;  // OPHIP_ATTN_ONE_PASS=0 keeps the composite (tests, comparisons); read once, here
     int force_chunk = 0;   // OPHIP_ATTN_CHUNK=256|128 keeps one chunk size (sweeps)
     explicit ophip_attention_kv_cached(ophip_device *d) : dev(d) {
@@ -339,13 +343,15 @@ struct ophip_attention_kv_cached {
             sub(ophip_rearrange_create(d, &rearrange));
             sub(ophip_attention_create(d, &attention));
             static const char *mt_tag[3] = {"m1", "m2", "m4"}, *dh_tag[2] = {"d64", "d128"};
-            for (int i = 0; i < 3; ++i)
-                for (int j = 0; j < 2; ++j) {
-                    const std::string tail = std::string(mt_tag[i]) + "_" + dh_tag[j];
-                    decode[i][j][0] = d->kernel("attention_decode", ("attn_decode_" + tail + "_k64").c_str());
-                    decode[i][j][1] = d->kernel("attention_decode", ("attn_decode_" + tail + "_k32").c_str());
-                    combine[i][j] = d->kernel("attention_decode", ("attn_decode_combine_" + tail).c_str());
-                }
+            for (int e = 0; e < 2; ++e)
+                for (int i = 0; i < 3; ++i)
+                    for (int j = 0; j < 2; ++j) {
+                        const std::string mod = e ? "attention_decode_bf16" : "attention_decode", tag = e ? "_bf16" : "";
+                        const std::string tail = std::string(mt_tag[i]) + "_" + dh_tag[j];
+                        decode[e][i][j][0] = d->kernel(mod.c_str(), ("attn_decode_" + tail + "_k64" + tag).c_str());
+                        decode[e][i][j][1] = d->kernel(mod.c_str(), ("attn_decode_" + tail + "_k32" + tag).c_str());
+                        combine[e][i][j] = d->kernel(mod.c_str(), ("attn_decode_combine_" + tail + tag).c_str());
+                    }
             if (const char *e = std::getenv("OPHIP_ATTN_ONE_PASS")) one_pass = std::atoi(e) != 0;
             if (const char *e = std::getenv("OPHIP_ATTN_CHUNK")) force_chunk = std::atoi(e);
         } catch (...) {
@@ -400,7 +406,7 @@ size_t decode_chunk(size_t nkvh, size_t att, unsigned cus, int force) {
 // Workspace of the one-pass kernel for these sizes, or SIZE_MAX when it does not serve them (the shapes alone
 // decide here; launch also looks at strides and alignment).
 size_t one_pass_workspace(uint64_t dt, size_t nh, size_t nkvh, size_t seq, size_t att, size_t dh, size_t chunk) {
-    if (dt != OPHIP_DT_F16 || (dh != 64 && dh != 128) || nkvh == 0 || nh % nkvh != 0 || seq == 0 || att == 0) return SIZE_MAX;
+    if ((dt != OPHIP_DT_F16 && dt != OPHIP_DT_BF16) || (dh != 64 && dh != 128) || nkvh == 0 || nh % nkvh != 0 || seq == 0 || att == 0) return SIZE_MAX;
     const size_t rows = nh / nkvh * seq;
     if (rows > 64 || att > 0x7fffffffu) return SIZE_MAX;
     const size_t nchunk = (att + chunk - 1) / chunk, rp = rows <= 16 ? 16 : rows <= 32 ? 32 : 64;
@@ -472,14 +478,15 @@ bool kv_cached_one_pass(const ophip_attention_kv_cached *op, const ophip_attenti
     p.nkvh = (uint32_t)nkvh, p.group = (uint32_t)group, p.seq = (uint32_t)seq, p.att = (uint32_t)att, p.pos = (uint32_t)pos;
     p.nchunk = (uint32_t)((att + chunk - 1) / chunk);
     p.causal = args.mask == OPHIP_MASK_CAUSAL;
-    p.scale = round_to_f16(1.0f / std::sqrt((float)dh));  // the reference's mat_mul rounds alpha to the data type
+    // the reference's mat_mul rounds alpha to the data type
+    p.scale = m.dt == OPHIP_DT_BF16 ? round_to_bf16(1.0f / std::sqrt((float)dh)) : round_to_f16(1.0f / std::sqrt((float)dh));
     if (p.nchunk > 65535 || nkvh > 65535) return false;
     Workspace ws(qa, workspace, workspace_len, need);
     p.partial = static_cast<float *>(ws.ptr());
-    const int mi = rows <= 16 ? 0 : rows <= 32 ? 1 : 2, di = dh == 64 ? 0 : 1;
+    const int mi = rows <= 16 ? 0 : rows <= 32 ? 1 : 2, di = dh == 64 ? 0 : 1, ei = m.dt == OPHIP_DT_BF16 ? 1 : 0;
     op->dev->make_current();
-    launch(op->decode[mi][di][chunk == 256 ? 0 : 1], Dim3{p.nchunk, (unsigned)nkvh}, Dim3{256}, 0, stream_of(qa), p);
-    if (p.nchunk > 1) launch(op->combine[mi][di], Dim3{(unsigned)(nkvh * rows)}, Dim3{256}, 0, stream_of(qa), p);
+    launch(op->decode[ei][mi][di][chunk == 256 ? 0 : 1], Dim3{p.nchunk, (unsigned)nkvh}, Dim3{256}, 0, stream_of(qa), p);
+    if (p.nchunk > 1) launch(op->combine[ei][mi][di], Dim3{(unsigned)(nkvh * rows)}, Dim3{256}, 0, stream_of(qa), p);
     return true;
 }
 

@@ -21,7 +21,10 @@
 //   them writes them to the caches bit for bit; no workgroup reads a cache row that another one writes.
 //
 // As in the reference the v-cache is addressed with the k-cache's strides (operator.rs:114, 156).
-#include "device_util.h"
+//
+// Compiled twice, like the MFMA GEMMs (gemm_elem.h): on f16 elements as it stands, and with -DGEMM_ELEM_BF16 on bf16
+// elements (module `attention_decode_bf16`, kernel names with `_bf16` appended).
+#include "gemm_elem.h"
 
 constexpr int AD_WAVES = 4;
 // KPW, keys per wave (64 or 32; a workgroup takes 4 * KPW keys), is a template parameter: few kv heads or a short
@@ -46,7 +49,7 @@ __device__ __forceinline__ void attn_decode(const AttnDecodeParams &p) {
     constexpr int AD_P_PITCH = AD_KPW + 8;       // halves per row of the probability tile (an odd number of 16-byte units)
     __shared__ float red[AD_WAVES][32][WAVE];
     __shared__ float s_max[AD_WAVES][16 * MT], s_sum[AD_WAVES][16 * MT];
-    __shared__ __attribute__((aligned(16))) f16 s_p[AD_WAVES][16 * MT][AD_P_PITCH];
+    __shared__ __attribute__((aligned(16))) elem s_p[AD_WAVES][16 * MT][AD_P_PITCH];
 
     const uint32_t wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
     const uint32_t j16 = lane % 16, g = lane / 16;
@@ -54,11 +57,11 @@ __device__ __forceinline__ void attn_decode(const AttnDecodeParams &p) {
     const uint32_t rows = p.group * p.seq;  // query rows of this kv head: row = head-in-group * seq + token
     const uint32_t key0 = chunk * AD_CHUNK + wave * AD_KPW;
 
-    const f16 *qb = reinterpret_cast<const f16 *>(p.q);
-    const f16 *kn = reinterpret_cast<const f16 *>(p.k_new) + (int64_t)kvh * p.kn_sh;
-    const f16 *vn = reinterpret_cast<const f16 *>(p.v_new) + (int64_t)kvh * p.vn_sh;
-    f16 *kc = reinterpret_cast<f16 *>(p.k_cache) + (int64_t)kvh * p.kc_sh;
-    f16 *vc = reinterpret_cast<f16 *>(p.v_cache) + (int64_t)kvh * p.kc_sh;
+    const elem *qb = reinterpret_cast<const elem *>(p.q);
+    const elem *kn = reinterpret_cast<const elem *>(p.k_new) + (int64_t)kvh * p.kn_sh;
+    const elem *vn = reinterpret_cast<const elem *>(p.v_new) + (int64_t)kvh * p.vn_sh;
+    elem *kc = reinterpret_cast<elem *>(p.k_cache) + (int64_t)kvh * p.kc_sh;
+    elem *vc = reinterpret_cast<elem *>(p.v_cache) + (int64_t)kvh * p.kc_sh;
     auto q_row = [&](uint32_t r) {  // r < rows
         const uint32_t hg = r / p.seq, s = r - hg * p.seq;
         return (int64_t)(kvh * p.group + hg) * p.q_sh + (int64_t)s * p.q_ss;
@@ -68,7 +71,7 @@ __device__ __forceinline__ void attn_decode(const AttnDecodeParams &p) {
     u32x4 qa[MT][KS];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-        const f16 *src = qb + q_row(min((uint32_t)mt * 16 + j16, rows - 1)) + 8 * g;
+        const elem *src = qb + q_row(min((uint32_t)mt * 16 + j16, rows - 1)) + 8 * g;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) qa[mt][ks] = ld128(src + 32 * ks);
     }
@@ -78,11 +81,11 @@ __device__ __forceinline__ void attn_decode(const AttnDecodeParams &p) {
 #pragma unroll
     for (int ct = 0; ct < AD_KPW / 16; ++ct) {
         const uint32_t key = key0 + ct * 16 + j16, keyc = min(key, p.att - 1);
-        const f16 *src = (keyc >= p.pos ? kn + (int64_t)(keyc - p.pos) * p.kn_ss : kc + (int64_t)keyc * p.kc_ss) + 8 * g;
+        const elem *src = (keyc >= p.pos ? kn + (int64_t)(keyc - p.pos) * p.kn_ss : kc + (int64_t)keyc * p.kc_ss) + 8 * g;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) kb[ct][ks] = ld128(src + 32 * ks);
         if (key >= p.pos && key < p.att) {
-            f16 *dst = kc + (int64_t)key * p.kc_ss + 8 * g;
+            elem *dst = kc + (int64_t)key * p.kc_ss + 8 * g;
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) st128(dst + 32 * ks, kb[ct][ks]);
         }
@@ -96,7 +99,7 @@ __device__ __forceinline__ void attn_decode(const AttnDecodeParams &p) {
 #pragma unroll
         for (int r = 0; r < 8; ++r) {
             const uint32_t key = key0 + kk * 32 + 8 * g + r, keyc = min(key, p.att - 1);
-            const f16 *src = (keyc >= p.pos ? vn + (int64_t)(keyc - p.pos) * p.vn_ss : vc + (int64_t)keyc * p.kc_ss) + 8 * cg;
+            const elem *src = (keyc >= p.pos ? vn + (int64_t)(keyc - p.pos) * p.vn_ss : vc + (int64_t)keyc * p.kc_ss) + 8 * cg;
             vw[kk][r] = ld128(src);
             if (key >= p.pos && key < p.att && j16 < NCG) st128(vc + (int64_t)key * p.kc_ss + 8 * cg, vw[kk][r]);
         }
@@ -110,10 +113,10 @@ __device__ __forceinline__ void attn_decode(const AttnDecodeParams &p) {
             f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                Pack8 a, b;
+                PackE a, b;
                 a.u = qa[mt][ks];
                 b.u = kb[ct][ks];
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a.h, b.h, acc, 0, 0, 0);
+                acc = mfma_16x16x32(a.h, b.h, acc);
             }
             sc[mt][ct] = acc;
         }
@@ -154,7 +157,7 @@ __device__ __forceinline__ void attn_decode(const AttnDecodeParams &p) {
             for (int ct = 0; ct < AD_KPW / 16; ++ct) {
                 const float e = __builtin_amdgcn_exp2f(sc[mt][ct][i] - m);
                 l += e;
-                s_p[wave][r][ct * 16 + j16] = f2h(e);
+                s_p[wave][r][ct * 16 + j16] = f2e(e);
             }
 #pragma unroll
             for (int o = 8; o > 0; o >>= 1) l += __shfl_xor(l, o, WAVE);
@@ -172,13 +175,13 @@ __device__ __forceinline__ void attn_decode(const AttnDecodeParams &p) {
         ad_transpose8x8(vw[kk], vb);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-            Pack8 a;
+            PackE a;
             a.u = ld128(&s_p[wave][mt * 16 + j16][kk * 32 + 8 * g]);
 #pragma unroll
             for (int t = 0; t < 8; ++t) {
-                Pack8 b;
+                PackE b;
                 b.u = vb[t];
-                oc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a.h, b.h, oc[mt][t], 0, 0, 0);
+                oc[mt][t] = mfma_16x16x32(a.h, b.h, oc[mt][t]);
             }
         }
     }
@@ -210,13 +213,13 @@ __device__ __forceinline__ void attn_decode(const AttnDecodeParams &p) {
         for (int w = 0; w < AD_WAVES; ++w) l += s_sum[w][r];
         if (p.nchunk == 1) {
             const float inv = 1.0f / l;
-            Pack8 o;
+            PackE o;
 #pragma unroll
-            for (int t = 0; t < 8; ++t) o.e[t] = f2h(out[t] * inv);
+            for (int t = 0; t < 8; ++t) o.e[t] = f2e(out[t] * inv);
             const uint32_t hg = r / p.seq, s = r - hg * p.seq;
             const int64_t h = kvh * p.group + hg;
-            st128(reinterpret_cast<f16 *>(p.o) + h * p.o_sh + (int64_t)s * p.o_ss + 8 * j16, o.u);
-            if (p.q_out) st128(reinterpret_cast<f16 *>(p.q_out) + h * p.q_sh + (int64_t)s * p.q_ss + 8 * j16, o.u);
+            st128(reinterpret_cast<elem *>(p.o) + h * p.o_sh + (int64_t)s * p.o_ss + 8 * j16, o.u);
+            if (p.q_out) st128(reinterpret_cast<elem *>(p.q_out) + h * p.q_sh + (int64_t)s * p.q_ss + 8 * j16, o.u);
         } else {
             // [kv head][chunk]: 16 * MT rows of DH floats, then per row the pair (maximum, sum)
             float *base = p.partial + ((size_t)kvh * p.nchunk + chunk) * (size_t)(16 * MT) * (DH + 2);
@@ -274,23 +277,23 @@ __device__ __forceinline__ void attn_decode_combine(const AttnDecodeParams &p) {
         M = Mn;
     }
     const float inv = 1.0f / L;
-    Pack8 o;
+    PackE o;
 #pragma unroll
-    for (int t = 0; t < 8; ++t) o.e[t] = f2h(acc[t] * inv);
+    for (int t = 0; t < 8; ++t) o.e[t] = f2e(acc[t] * inv);
     const uint32_t hg = r / p.seq, s = r - hg * p.seq;
     const int64_t h = kvh * p.group + hg;
-    st128(reinterpret_cast<f16 *>(p.o) + h * p.o_sh + (int64_t)s * p.o_ss + 8 * cgi, o.u);
-    if (p.q_out) st128(reinterpret_cast<f16 *>(p.q_out) + h * p.q_sh + (int64_t)s * p.q_ss + 8 * cgi, o.u);
+    st128(reinterpret_cast<elem *>(p.o) + h * p.o_sh + (int64_t)s * p.o_ss + 8 * cgi, o.u);
+    if (p.q_out) st128(reinterpret_cast<elem *>(p.q_out) + h * p.q_sh + (int64_t)s * p.q_ss + 8 * cgi, o.u);
 }
 
 #define ATTN_DECODE(MT, DH)                                                                                  \
-    extern "C" __global__ void __launch_bounds__(256) attn_decode_m##MT##_d##DH##_k64(AttnDecodeParams p) {   \
+    extern "C" __global__ void __launch_bounds__(256) GEMM_KERNEL(attn_decode_m##MT##_d##DH##_k64)(AttnDecodeParams p) {   \
         attn_decode<MT, DH, 64>(p);                                                                          \
     }                                                                                                        \
-    extern "C" __global__ void __launch_bounds__(256) attn_decode_m##MT##_d##DH##_k32(AttnDecodeParams p) {   \
+    extern "C" __global__ void __launch_bounds__(256) GEMM_KERNEL(attn_decode_m##MT##_d##DH##_k32)(AttnDecodeParams p) {   \
         attn_decode<MT, DH, 32>(p);                                                                          \
     }                                                                                                        \
-    extern "C" __global__ void __launch_bounds__(256) attn_decode_combine_m##MT##_d##DH(AttnDecodeParams p) { \
+    extern "C" __global__ void __launch_bounds__(256) GEMM_KERNEL(attn_decode_combine_m##MT##_d##DH)(AttnDecodeParams p) { \
         attn_decode_combine<MT, DH>(p);                                                                      \
     }
 ATTN_DECODE(1, 64)

@@ -22,10 +22,13 @@
 //
 // Results agree with the composite within the f16 bar (scores and probabilities are not rounded to f16 in between;
 // the scale is rounded to f16 as the reference's mat_mul rounds alpha).
-#include "device_util.h"
+//
+// Compiled twice, like the MFMA GEMMs (gemm_elem.h): on f16 elements as it stands, and with -DGEMM_ELEM_BF16 on bf16
+// elements (module `attention_prefill_bf16`, kernel names with `_bf16` appended): the element type decides the two MFMA
+// instructions and the rounding of the probabilities and of the output, nothing else.
+#include "gemm_elem.h"
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int AP_BM = 128, AP_BN = 64;
 
@@ -42,7 +45,7 @@ __device__ __forceinline__ void attn_prefill(const AttnPrefillParams &p) {
     constexpr int NCH = AP_BN * CPR / 256;  // chunks per thread and tile
     constexpr int DS = DH / 16, DB = DH / 32;
     constexpr int TILE_HALVES = AP_BN * (KP + VP);
-    __shared__ __attribute__((aligned(16))) f16 lds[G * 2 * TILE_HALVES];
+    __shared__ __attribute__((aligned(16))) elem lds[G * 2 * TILE_HALVES];
 
     const uint32_t grp = G == 1 ? 0 : threadIdx.x / 256;
     const uint32_t tid = threadIdx.x % 256, wave = tid / WAVE, lane = tid % WAVE;
@@ -52,15 +55,15 @@ __device__ __forceinline__ void attn_prefill(const AttnPrefillParams &p) {
     const uint32_t kvh = head / p.group;
     const uint32_t i0 = qblock * AP_BM;
     const uint32_t row = i0 + wave * 32 + n32, rowc = min(row, p.seq - 1);
-    f16 *const k_lds = lds + grp * 2 * TILE_HALVES;          // [2][AP_BN * KP]
-    f16 *const v_lds = k_lds + 2 * AP_BN * KP;               // [2][AP_BN * VP]
+    elem *const k_lds = lds + grp * 2 * TILE_HALVES;          // [2][AP_BN * KP]
+    elem *const v_lds = k_lds + 2 * AP_BN * KP;               // [2][AP_BN * VP]
 
-    const f16 *qb = reinterpret_cast<const f16 *>(p.q) + (int64_t)head * p.q_sh;
-    const f16 *kb = reinterpret_cast<const f16 *>(p.k) + (int64_t)kvh * p.k_sh;
-    const f16 *vb = reinterpret_cast<const f16 *>(p.v) + (int64_t)kvh * p.v_sh;
+    const elem *qb = reinterpret_cast<const elem *>(p.q) + (int64_t)head * p.q_sh;
+    const elem *kb = reinterpret_cast<const elem *>(p.k) + (int64_t)kvh * p.k_sh;
+    const elem *vb = reinterpret_cast<const elem *>(p.v) + (int64_t)kvh * p.v_sh;
 
     // the wave's queries as B operands: lane (n32, h) holds query row n32, dh slots 16 ds + 8 h .. + 7
-    Pack8 qf[DS];
+    PackE qf[DS];
 #pragma unroll
     for (int ds = 0; ds < DS; ++ds) qf[ds].u = ld128(qb + (int64_t)rowc * p.q_ss + 16 * ds + 8 * h);
 
@@ -131,7 +134,7 @@ __device__ __forceinline__ void attn_prefill(const AttnPrefillParams &p) {
         if (t < ntiles) {
             const bool more = t + G < ntiles;
             if (more) fetch(t + G);
-            const f16 *kt = k_lds + buf * (AP_BN * KP), *vt = v_lds + buf * (AP_BN * VP);
+            const elem *kt = k_lds + buf * (AP_BN * KP), *vt = v_lds + buf * (AP_BN * VP);
 
             // S^T = K . Q^T: sacc[kb][e] is key 32 kb + 8 (e / 4) + 4 h + e % 4 of the tile, query n32
             f32x16 sacc[2];
@@ -141,9 +144,9 @@ __device__ __forceinline__ void attn_prefill(const AttnPrefillParams &p) {
                 for (int e = 0; e < 16; ++e) sacc[kb2][e] = 0.f;
 #pragma unroll
                 for (int ds = 0; ds < DS; ++ds) {
-                    Pack8 a;
+                    PackE a;
                     a.u = ld128(kt + (32 * kb2 + n32) * KP + 16 * ds + 8 * h);
-                    sacc[kb2] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a.h, qf[ds].h, sacc[kb2], 0, 0, 0);
+                    sacc[kb2] = mfma_32x32x16(a.h, qf[ds].h, sacc[kb2]);
                 }
             }
             // mask (only a tile that reaches past the wave's first limit has anything to mask), the tile's maximum for
@@ -178,14 +181,14 @@ __device__ __forceinline__ void attn_prefill(const AttnPrefillParams &p) {
             float psum = 0.f;
             // probabilities, packed for the second product: MFMA j covers the tile's keys 16 j .. 16 j + 15; the lane's eight
             // contraction slots 8 h .. 8 h + 7 hold keys 16 j + 4 h + {0..3} and 16 j + 8 + 4 h + {0..3}
-            Pack8 pb[4];
+            PackE pb[4];
 #pragma unroll
             for (int kb2 = 0; kb2 < 2; ++kb2)
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     const float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb2][e], sc2, -m_ref));
                     psum += pr;
-                    pb[2 * kb2 + e / 8].e[e % 8] = f2h(pr);
+                    pb[2 * kb2 + e / 8].e[e % 8] = f2e(pr);
                 }
             l_run += psum;
 
@@ -196,14 +199,14 @@ __device__ __forceinline__ void attn_prefill(const AttnPrefillParams &p) {
             for (int db = 0; db < DB; ++db)
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const f16 *src = vt + (16 * j + 4 * h + s16 / 4) * VP + 32 * db + 16 * b16 + 4 * (s16 % 4);
+                    const elem *src = vt + (16 * j + 4 * h + s16 / 4) * VP + 32 * db + 16 * b16 + 4 * (s16 % 4);
                     union {
                         s16x4 q[2];
-                        f16x8 hv;
+                        elem8 hv;
                     } a;
                     a.q[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4)src);
                     a.q[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4)(src + 8 * VP));
-                    oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a.hv, pb[j].h, oacc[db], 0, 0, 0);
+                    oacc[db] = mfma_32x32x16(a.hv, pb[j].h, oacc[db]);
                 }
 
             if (more) commit(buf ^ 1);
@@ -239,18 +242,18 @@ __device__ __forceinline__ void attn_prefill(const AttnPrefillParams &p) {
     // o = O^T / l: the lane holds, for its query, columns 32 db + 8 (e / 4) + 4 h + e % 4: four adjacent ones per e / 4
     const float inv = 1.0f / l_tot;
     if (row < p.seq) {
-        f16 *orow = reinterpret_cast<f16 *>(p.o) + (int64_t)head * p.o_sh + (int64_t)row * p.o_ss;
-        f16 *qrow = p.q_out ? reinterpret_cast<f16 *>(p.q_out) + (int64_t)head * p.q_sh + (int64_t)row * p.q_ss : nullptr;
+        elem *orow = reinterpret_cast<elem *>(p.o) + (int64_t)head * p.o_sh + (int64_t)row * p.o_ss;
+        elem *qrow = p.q_out ? reinterpret_cast<elem *>(p.q_out) + (int64_t)head * p.q_sh + (int64_t)row * p.q_ss : nullptr;
 #pragma unroll
         for (int db = 0; db < DB; ++db)
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 union {
-                    f16 e[4];
+                    elem e[4];
                     u32x2 u;
                 } o;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) o.e[r] = f2h(oacc[db][4 * g + r] * inv);
+                for (int r = 0; r < 4; ++r) o.e[r] = f2e(oacc[db][4 * g + r] * inv);
                 const uint32_t col = 32 * db + 8 * g + 4 * h;
                 *reinterpret_cast<u32x2 *>(orow + col) = o.u;
                 if (qrow) *reinterpret_cast<u32x2 *>(qrow + col) = o.u;
@@ -260,7 +263,7 @@ __device__ __forceinline__ void attn_prefill(const AttnPrefillParams &p) {
 
 // (two waves per SIMD: two workgroups of four waves per CU, or one of eight; one wave multiplies while the other does its
 // exponentials)
-extern "C" __global__ void __launch_bounds__(256, 2) attn_prefill_d128(AttnPrefillParams p) { attn_prefill<128, 1>(p); }
-extern "C" __global__ void __launch_bounds__(256, 2) attn_prefill_d64(AttnPrefillParams p) { attn_prefill<64, 1>(p); }
-extern "C" __global__ void __launch_bounds__(512) attn_prefill_d128_g2(AttnPrefillParams p) { attn_prefill<128, 2>(p); }
-extern "C" __global__ void __launch_bounds__(512) attn_prefill_d64_g2(AttnPrefillParams p) { attn_prefill<64, 2>(p); }
+extern "C" __global__ void __launch_bounds__(256, 2) GEMM_KERNEL(attn_prefill_d128)(AttnPrefillParams p) { attn_prefill<128, 1>(p); }
+extern "C" __global__ void __launch_bounds__(256, 2) GEMM_KERNEL(attn_prefill_d64)(AttnPrefillParams p) { attn_prefill<64, 1>(p); }
+extern "C" __global__ void __launch_bounds__(512) GEMM_KERNEL(attn_prefill_d128_g2)(AttnPrefillParams p) { attn_prefill<128, 2>(p); }
+extern "C" __global__ void __launch_bounds__(512) GEMM_KERNEL(attn_prefill_d64_g2)(AttnPrefillParams p) { attn_prefill<64, 2>(p); }

@@ -1,4 +1,4 @@
-// Element type of the MFMA GEMM kernels.  gemm.hip and gemm_tile.hip are compiled twice: as they stand, on f16 elements
+// Element type of the MFMA kernels.  gemm.hip and gemm_tile.hip (and attention_prefill.hip, attention_decode.hip) are compiled twice: as they stand, on f16 elements
 // (modules `gemm`, `gemm_tile`), and with -DGEMM_ELEM_BF16 on bf16 elements (modules `gemm_bf16`, `gemm_tile_bf16`,
 // kernel names with `_bf16` appended, so that a trace tells the two apart).  The kernels move elements as 16-bit words, so the type matters in three places only: the MFMA
 // instruction, and the two conversions of the epilogue (f32 -> element rounds to nearest even in both types).

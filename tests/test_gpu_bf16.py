@@ -231,8 +231,24 @@ def test_softmax_bf16(gpu, stream, shape, causal):
         assert (y[~np.broadcast_to(keep[None], shape)] == 0).all()
 
 
-def test_attention_bf16_runs_on_the_composite(gpu, stream):
-    """mat_mul, softmax and rearrange all take bf16, so the composite of launches does: against f64."""
+def attention_f64_bf16(q, k, v, causal):
+    """softmax(q . k^T / sqrt(dh), mask) . v in f64 on bf16 bit patterns; heads of q share kv heads in groups."""
+    nh, seq, dh = q.shape
+    nkvh, att, _ = k.shape
+    g = nh // nkvh
+    kk, vv = np.repeat(from_bf16(k).astype(f64), g, axis=0), np.repeat(from_bf16(v).astype(f64), g, axis=0)
+    s = np.einsum("hsd,had->hsa", from_bf16(q).astype(f64), kk) / np.sqrt(dh)
+    if causal:
+        s = np.where((np.arange(att)[None, :] <= (att - seq + np.arange(seq))[:, None])[None], s, -np.inf)
+    pr = np.exp(s - s.max(-1, keepdims=True))
+    return np.einsum("hsa,had->hsd", pr / pr.sum(-1, keepdims=True), vv)
+
+
+@pytest.mark.parametrize("fused", ["0", "1"])
+def test_attention_bf16_composite_and_one_pass(gpu, stream, monkeypatch, fused):
+    """mat_mul, softmax and rearrange all take bf16, so the composite of launches does (OPHIP_ATTN_FUSED=0); the one-pass
+    kernel is built on bf16 elements as well (=1): both against f64."""
+    monkeypatch.setenv("OPHIP_ATTN_FUSED", fused)
     rng = np.random.default_rng(31)
     nh, nkvh, seq, att, dh = 8, 2, 40, 136, 64
     q, k, v = (to_bf16(rng.standard_normal(s).astype(f32)) for s in ((nh, seq, dh), (nkvh, att, dh), (nkvh, att, dh)))
@@ -241,17 +257,72 @@ def test_attention_bf16_runs_on_the_composite(gpu, stream):
     op = ophip.Attention(gpu)
     args = ophip.AttentionArgs(c(nh, seq, dh), qd, c(nkvh, att, dh), kd, c(nkvh, att, dh), vd, c(nh, seq, dh), od, ophip.AttnMask.CAUSAL)
     ws = gpu.malloc(max(op.scheme(args, 1 << 30), 16))
-    say("attention bf16 (composite)")
+    say("attention bf16 fused=%s" % fused)
     op.launch(args, ws, stream)
     y = from_bf16(gpu.to_host(od, u16, q.size, stream=stream)).reshape(nh, seq, dh).astype(f64)
-    g = nh // nkvh
-    kk, vv = np.repeat(from_bf16(k).astype(f64), g, axis=0), np.repeat(from_bf16(v).astype(f64), g, axis=0)
-    s = np.einsum("hsd,had->hsa", from_bf16(q).astype(f64), kk) / np.sqrt(dh)
-    s = np.where((np.arange(att)[None, :] <= (att - seq + np.arange(seq))[:, None])[None], s, -np.inf)
-    pr = np.exp(s - s.max(-1, keepdims=True))
-    ref = np.einsum("hsa,had->hsd", pr / pr.sum(-1, keepdims=True), vv)
-    # scores and probabilities are rounded to bf16 between the launches: a few steps of the output's scale
-    assert np.abs(y - ref).max() <= 4 * 2.0 ** -7 * np.abs(ref).max(), np.abs(y - ref).max()
+    ref = attention_f64_bf16(q, k, v, True)
+    # the composite rounds scores and probabilities to bf16 between the launches: a few steps of the output's scale;
+    # the one pass keeps them in f32 and rounds the probabilities once, for the second product
+    steps = 4 if fused == "0" else 1.5
+    assert np.abs(y - ref).max() <= steps * 2.0 ** -7 * np.abs(ref).max(), np.abs(y - ref).max()
+
+
+@pytest.mark.parametrize("split", ["0", "1"])
+@pytest.mark.parametrize("nh,nkvh,seq,att,dh,causal", [
+    (32, 32, 512, 512, 128, True),     # a prefill step
+    (8, 2, 300, 700, 64, True),        # grouped heads, a cache before the rows, ragged last block and tile
+    (4, 4, 129, 129, 128, True),       # one row into the second block
+    (6, 3, 100, 333, 64, False),       # no mask
+    (2, 1, 1000, 1000, 128, True),
+])
+def test_attention_bf16_one_pass_shapes(gpu, stream, monkeypatch, split, nh, nkvh, seq, att, dh, causal):
+    """The one-pass kernel's bf16 build, both of its workgroup shapes (OPHIP_ATTN_KEYSPLIT), against f64; q, left in
+    place by the operator when o is another buffer and the heads do not merge with the tokens, is overwritten with the
+    result when they do (contiguous q), as the reference's composite does."""
+    monkeypatch.setenv("OPHIP_ATTN_FUSED", "1")
+    monkeypatch.setenv("OPHIP_ATTN_KEYSPLIT", split)
+    rng = np.random.default_rng(nh * seq + att)
+    q, k, v = (to_bf16(rng.standard_normal(s).astype(f32)) for s in ((nh, seq, dh), (nkvh, att, dh), (nkvh, att, dh)))
+    qd, kd, vd, od = gpu.from_host(q), gpu.from_host(k), gpu.from_host(v), gpu.malloc(q.nbytes)
+    gpu.memset(od, 0)
+    c = lambda *s: TensorLayout.new_contiguous(dt.BF16, list(s))
+    mask = ophip.AttnMask.CAUSAL if causal else ophip.AttnMask.NONE
+    op = ophip.Attention(gpu)
+    args = ophip.AttentionArgs(c(nh, seq, dh), qd, c(nkvh, att, dh), kd, c(nkvh, att, dh), vd, c(nh, seq, dh), od, mask)
+    ws = gpu.malloc(max(op.scheme(args, 1 << 30), 16))
+    say("attention bf16 one pass split=%s nh=%d nkvh=%d seq=%d att=%d dh=%d causal=%s" % (split, nh, nkvh, seq, att, dh, causal))
+    op.launch(args, ws, stream)
+    yb = gpu.to_host(od, u16, q.size, stream=stream).reshape(nh, seq, dh)
+    ref = attention_f64_bf16(q, k, v, causal)
+    y = from_bf16(yb).astype(f64)
+    assert np.abs(y - ref).max() <= 1.5 * 2.0 ** -7 * np.abs(ref).max(), np.abs(y - ref).max()
+    assert np.array_equal(gpu.to_host(qd, u16, q.size, stream=stream).reshape(nh, seq, dh), yb)
+
+
+@pytest.mark.parametrize("nh,nkvh,seq,dh,buf,pos", [(32, 32, 16, 128, 2048, 2032), (32, 8, 1, 128, 4096, 4095), (32, 4, 7, 64, 1500, 1017),
+                                                    (8, 8, 16, 64, 700, 0), (3, 3, 33, 64, 100, 10)])
+def test_attention_kv_cached_bf16_one_pass(gpu, stream, nh, nkvh, seq, dh, buf, pos):
+    """attention_kv_cached on bf16: decode shapes on the one-pass kernel's bf16 build.  o against f64 over the cache's
+    first pos rows and the new ones; the appended cache rows bit for bit, the rest of the caches untouched."""
+    rng = np.random.default_rng(nh + buf + pos)
+    mk = lambda *s: to_bf16(rng.standard_normal(s).astype(f32))
+    q, k, v, kc, vc = mk(nh, seq, dh), mk(nkvh, seq, dh), mk(nkvh, seq, dh), mk(nkvh, buf, dh), mk(nkvh, buf, dh)
+    qd, kd, vd, kcd, vcd = (gpu.from_host(a) for a in (q, k, v, kc, vc))
+    od = gpu.malloc(q.nbytes)
+    c = lambda *s: TensorLayout.new_contiguous(dt.BF16, list(s))
+    op = ophip.AttnKVCached(gpu)
+    args = ophip.AttnKVCachedArgs(c(nh, seq, dh), qd, c(nkvh, seq, dh), kd, c(nkvh, seq, dh), vd, c(nh, seq, dh), od,
+                                  c(nkvh, buf, dh), kcd, c(nkvh, buf, dh), vcd, ophip.AttnMask.CAUSAL, pos)
+    ws = gpu.malloc(max(op.scheme(args, 1 << 30), 16))
+    say("attention_kv_cached bf16 nh=%d nkvh=%d seq=%d dh=%d buf=%d pos=%d" % (nh, nkvh, seq, dh, buf, pos))
+    op.launch(args, ws, stream)
+    kc_ref, vc_ref = kc.copy(), vc.copy()
+    kc_ref[:, pos:pos + seq], vc_ref[:, pos:pos + seq] = k, v
+    assert np.array_equal(gpu.to_host(kcd, u16, kc.size, stream=stream).reshape(kc.shape), kc_ref)
+    assert np.array_equal(gpu.to_host(vcd, u16, vc.size, stream=stream).reshape(vc.shape), vc_ref)
+    y = from_bf16(gpu.to_host(od, u16, q.size, stream=stream)).reshape(nh, seq, dh).astype(f64)
+    ref = attention_f64_bf16(q, kc_ref[:, :pos + seq], vc_ref[:, :pos + seq], True)
+    assert np.abs(y - ref).max() <= 1.5 * 2.0 ** -7 * np.abs(ref).max(), np.abs(y - ref).max()
 
 
 def test_types_no_kernel_takes_are_refused(gpu, stream):
