@@ -731,7 +731,12 @@ extern "C" int ophip_swiglu_launch(const ophip_swiglu *op, const ophip_swiglu_ar
         const size_t items = vec ? d / 8 : d;
         const unsigned gx = std::min<unsigned>(ceil_div(items, 256), 65535u);
         const unsigned gy = (unsigned)std::min<size_t>(n, 65535);
-        const bool big = n * d * (size_t)unit >= ((size_t)64 << 20);  // more than the caches hold
+        // more than the caches hold (and few enough vectors to number them with 32 bits, one per thread)
+        const bool big = n * d * (size_t)unit >= ((size_t)64 << 20) && vec && n * items < ((size_t)1 << 31);
+        if (big) {
+            p.total = (uint32_t)(n * items);
+            p.per_row = make_fastdiv((uint32_t)items);
+        }
         hipFunction_t fn = vec ? (bf ? (big ? op->bf16_vec_nt : op->bf16_vec) : (big ? op->f16_vec_nt : op->f16_vec))
                            : m.dt == OPHIP_DT_F16 ? op->f16_scalar
                            : bf                   ? op->bf16_scalar
@@ -739,6 +744,7 @@ extern "C" int ophip_swiglu_launch(const ophip_swiglu *op, const ophip_swiglu_ar
                                                   : op->f64_scalar;
         if (!p.gate || !p.up) throw args_not_support("null base address");
         op->dev->make_current();
-        launch(fn, Dim3{gx, gy}, Dim3{256}, 0, stream_of(qa), p);
+        if (big) launch(fn, Dim3{(unsigned)ceil_div(n * items, 256)}, Dim3{256}, 0, stream_of(qa), p);
+        else launch(fn, Dim3{gx, gy}, Dim3{256}, 0, stream_of(qa), p);
     });
 }

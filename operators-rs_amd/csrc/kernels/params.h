@@ -26,6 +26,8 @@ struct SwigluParams {
     const void *up;
     int64_t sgn, sun;  // row strides in bytes
     uint32_t n, d;
+    uint32_t total;      // the `_nt` kernels: 16-byte vectors in all, numbered row by row ...
+    FastDivU32 per_row;  // ... this many to a row
 };
 
 struct RopeParams {
