@@ -31,7 +31,7 @@ __device__ __forceinline__ AddOffsets add_decode(const AddParams &p, uint32_t g)
 // in the parameters would make the compiler merge the two stores of an if / else and drop the hint.)
 template <typename T, bool NT>
 __device__ __forceinline__ void add_h_vec_impl(const AddParams &p) {  // T: f16 or bf16
-    for (uint32_t g = blockIdx.x * blockDim.x + threadIdx.x; g < p.total; g += gridDim.x * blockDim.x) {
+    for (uint32_t g = blockIdx.x * WG_THREADS + threadIdx.x; g < p.total; g += gridDim.x * WG_THREADS) {
         const AddOffsets o = add_decode(p, g);
         PackOf<T> a, b, c;
         a.u = ld128_nt(reinterpret_cast<const char *>(p.a) + o.a);
@@ -50,7 +50,7 @@ extern "C" __global__ void __launch_bounds__(256) add_bf16_vec_nt(AddParams p) {
 
 template <bool NT>
 __device__ __forceinline__ void add_f32_vec_impl(const AddParams &p) {
-    for (uint32_t g = blockIdx.x * blockDim.x + threadIdx.x; g < p.total; g += gridDim.x * blockDim.x) {
+    for (uint32_t g = blockIdx.x * WG_THREADS + threadIdx.x; g < p.total; g += gridDim.x * WG_THREADS) {
         const AddOffsets o = add_decode(p, g);
         Pack4f a, b, c;
         a.u = ld128_nt(reinterpret_cast<const char *>(p.a) + o.a);
@@ -65,7 +65,7 @@ extern "C" __global__ void __launch_bounds__(256) add_f32_vec_nt(AddParams p) { 
 
 template <typename T>
 __device__ __forceinline__ void add_scalar(const AddParams &p) {
-    for (uint32_t g = blockIdx.x * blockDim.x + threadIdx.x; g < p.total; g += gridDim.x * blockDim.x) {
+    for (uint32_t g = blockIdx.x * WG_THREADS + threadIdx.x; g < p.total; g += gridDim.x * WG_THREADS) {
         const AddOffsets o = add_decode(p, g);
         using Calc = std::conditional_t<sizeof(T) == 8, double, float>;  // f64 data adds in f64
         const Calc a = (Calc)*reinterpret_cast<const T *>(reinterpret_cast<const char *>(p.a) + o.a);
@@ -84,7 +84,7 @@ extern "C" __global__ void __launch_bounds__(256) add_f64_scalar(AddParams p) { 
 // unsigned alike in two's complement: one kernel per width) and for bool "either is set".  Its CPU backend has floats only.
 template <typename U, bool IS_BOOL = false>
 __device__ __forceinline__ void add_int_scalar(const AddParams &p) {
-    for (uint32_t g = blockIdx.x * blockDim.x + threadIdx.x; g < p.total; g += gridDim.x * blockDim.x) {
+    for (uint32_t g = blockIdx.x * WG_THREADS + threadIdx.x; g < p.total; g += gridDim.x * WG_THREADS) {
         const AddOffsets o = add_decode(p, g);
         const U a = *reinterpret_cast<const U *>(reinterpret_cast<const char *>(p.a) + o.a);
         const U b = *reinterpret_cast<const U *>(reinterpret_cast<const char *>(p.b) + o.b);

@@ -24,7 +24,7 @@ __device__ __forceinline__ void add_rows_h_vec(const AddRowsParams &p) {  // T: 
         char *dst;
         const char *src;
         if (!add_rows_locate(p, bm, dst, src)) continue;
-        for (uint32_t v = blockIdx.x * blockDim.x + threadIdx.x; v < nvec; v += gridDim.x * blockDim.x) {
+        for (uint32_t v = blockIdx.x * WG_THREADS + threadIdx.x; v < nvec; v += gridDim.x * WG_THREADS) {
             PackOf<T> d, s;
             d.u = ld128_nt(dst + (size_t)v * 16);
             s.u = ld128(src + (size_t)v * 16);
@@ -46,7 +46,7 @@ __device__ __forceinline__ void add_rows_scalar(const AddRowsParams &p, int64_t 
         char *dst;
         const char *src;
         if (!add_rows_locate(p, bm, dst, src)) continue;
-        for (uint32_t j = blockIdx.x * blockDim.x + threadIdx.x; j < p.n; j += gridDim.x * blockDim.x) {
+        for (uint32_t j = blockIdx.x * WG_THREADS + threadIdx.x; j < p.n; j += gridDim.x * WG_THREADS) {
             T *d = reinterpret_cast<T *>(dst + (int64_t)j * nsd);
             const T *s = reinterpret_cast<const T *>(src + (int64_t)j * nss);
             using Calc = std::conditional_t<sizeof(T) == 8, double, float>;  // f64 data adds in f64
@@ -80,7 +80,7 @@ __device__ __forceinline__ void add_rows_int(const AddRowsParams &p, int64_t nsd
         char *dst;
         const char *src;
         if (!add_rows_locate(p, bm, dst, src)) continue;
-        for (uint32_t j = blockIdx.x * blockDim.x + threadIdx.x; j < p.n; j += gridDim.x * blockDim.x) {
+        for (uint32_t j = blockIdx.x * WG_THREADS + threadIdx.x; j < p.n; j += gridDim.x * WG_THREADS) {
             U *d = reinterpret_cast<U *>(dst + (int64_t)j * nsd);
             const U s = *reinterpret_cast<const U *>(src + (int64_t)j * nss);
             *d = IS_BOOL ? (U)((*d | s) != 0) : (U)(*d + s);

@@ -125,7 +125,7 @@ __device__ __forceinline__ void softmax_rows4(const SoftmaxParams &p) {
     __syncthreads();
     const uint32_t lane = threadIdx.x % WAVE;
     const uint32_t per_head = (p.seq + ROWS - 1) / ROWS;  // waves per head
-    const uint32_t w = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+    const uint32_t w = blockIdx.x * (WG_THREADS / WAVE) + threadIdx.x / WAVE;
     if (w >= p.nh * per_head) return;  // (no barrier below this line)
     const uint32_t h = w / per_head, j = w - h * per_head;
     const bool paired = p.seq % ROWS == 0;

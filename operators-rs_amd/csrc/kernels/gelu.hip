@@ -16,7 +16,7 @@ __device__ __forceinline__ void gelu_vec(const GeluParams &p) {  // T: f16 or bf
     const uint32_t nvec = p.d / 8;
     for (uint32_t row = blockIdx.y; row < p.n; row += gridDim.y) {
         char *r = reinterpret_cast<char *>(p.base) + (int64_t)row * p.sn;
-        for (uint32_t v = blockIdx.x * blockDim.x + threadIdx.x; v < nvec; v += gridDim.x * blockDim.x) {
+        for (uint32_t v = blockIdx.x * WG_THREADS + threadIdx.x; v < nvec; v += gridDim.x * WG_THREADS) {
             PackOf<T> a, o;
             a.u = ld128_nt(r + (size_t)v * 16);
 #pragma unroll
@@ -39,7 +39,7 @@ template <typename T>
 __device__ __forceinline__ void gelu_scalar(const GeluParams &p) {
     for (uint32_t row = blockIdx.y; row < p.n; row += gridDim.y) {
         T *r = reinterpret_cast<T *>(reinterpret_cast<char *>(p.base) + (int64_t)row * p.sn);
-        for (uint32_t j = blockIdx.x * blockDim.x + threadIdx.x; j < p.d; j += gridDim.x * blockDim.x) {
+        for (uint32_t j = blockIdx.x * WG_THREADS + threadIdx.x; j < p.d; j += gridDim.x * WG_THREADS) {
             if constexpr (sizeof(T) == 8) r[j] = gelu_f64(r[j]);
             else r[j] = (T)gelu_f32((float)r[j]);
         }

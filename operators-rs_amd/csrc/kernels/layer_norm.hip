@@ -135,15 +135,15 @@ template <typename TA, typename TW>
 __device__ __forceinline__ void layer_norm_rows(const LayerNormParams &p) {
     constexpr int CACHE = 8, MAXD = 4096;
     __shared__ float s_scale[MAXD], s_bias[MAXD];
-    for (uint32_t j = threadIdx.x; j < p.d; j += blockDim.x) {
+    for (uint32_t j = threadIdx.x; j < p.d; j += WG_THREADS) {
         s_scale[j] = (float)reinterpret_cast<const TW *>(p.scale)[j];
         s_bias[j] = (float)reinterpret_cast<const TW *>(p.bias)[j];
     }
     __syncthreads();
 
     const uint32_t lane = threadIdx.x % WAVE;
-    const uint32_t waves = gridDim.x * (blockDim.x / WAVE);
-    uint32_t row = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+    const uint32_t waves = gridDim.x * (WG_THREADS / WAVE);
+    uint32_t row = blockIdx.x * (WG_THREADS / WAVE) + threadIdx.x / WAVE;
     const uint32_t nvec = p.d / 8;
     if (row >= p.n) return;
 

@@ -13,8 +13,8 @@
 
 extern "C" __global__ void __launch_bounds__(256) probe_read(ProbeParams p) {
     const u32x4 *w = reinterpret_cast<const u32x4 *>(p.src);
-    const size_t nvec = p.bytes / 16, st = (size_t)gridDim.x * blockDim.x;
-    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t nvec = p.bytes / 16, st = (size_t)gridDim.x * WG_THREADS;
+    size_t i = (size_t)blockIdx.x * WG_THREADS + threadIdx.x;
     u32x4 acc = {0, 0, 0, 0};
     for (; i + 3 * st < nvec; i += 4 * st) {
         const u32x4 a = w[i], b = w[i + st], c = w[i + 2 * st], d = w[i + 3 * st];
@@ -26,8 +26,8 @@ extern "C" __global__ void __launch_bounds__(256) probe_read(ProbeParams p) {
 
 extern "C" __global__ void __launch_bounds__(256) probe_read_nt(ProbeParams p) {
     const u32x4 *w = reinterpret_cast<const u32x4 *>(p.src);
-    const size_t nvec = p.bytes / 16, st = (size_t)gridDim.x * blockDim.x;
-    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t nvec = p.bytes / 16, st = (size_t)gridDim.x * WG_THREADS;
+    size_t i = (size_t)blockIdx.x * WG_THREADS + threadIdx.x;
     u32x4 acc = {0, 0, 0, 0};
     for (; i + 3 * st < nvec; i += 4 * st) {
         const u32x4 a = ld128_nt(w + i), b = ld128_nt(w + i + st), c = ld128_nt(w + i + 2 * st), d = ld128_nt(w + i + 3 * st);
@@ -42,8 +42,8 @@ extern "C" __global__ void __launch_bounds__(256) probe_read_nt(ProbeParams p) {
 template <bool NT>
 __device__ __forceinline__ void probe_read_deep(const ProbeParams &p) {
     const u32x4 *w = reinterpret_cast<const u32x4 *>(p.src);
-    const size_t nvec = p.bytes / 16, st = (size_t)gridDim.x * blockDim.x;
-    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t nvec = p.bytes / 16, st = (size_t)gridDim.x * WG_THREADS;
+    size_t i = (size_t)blockIdx.x * WG_THREADS + threadIdx.x;
     u32x4 acc = {0, 0, 0, 0};
     for (; i + 15 * st < nvec; i += 16 * st) {
         u32x4 v[16];
@@ -88,16 +88,16 @@ extern "C" __global__ void __launch_bounds__(256) probe_strips(ProbeParams p) {
 
 extern "C" __global__ void __launch_bounds__(256) probe_write(ProbeParams p) {
     u32x4 *d = reinterpret_cast<u32x4 *>(p.dst);
-    const size_t nvec = p.bytes / 16, st = (size_t)gridDim.x * blockDim.x;
+    const size_t nvec = p.bytes / 16, st = (size_t)gridDim.x * WG_THREADS;
     const u32x4 v = {p.seed, p.seed, p.seed, p.seed};
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += st) d[i] = v;
+    for (size_t i = (size_t)blockIdx.x * WG_THREADS + threadIdx.x; i < nvec; i += st) d[i] = v;
 }
 
 extern "C" __global__ void __launch_bounds__(256) probe_copy(ProbeParams p) {
     const u32x4 *w = reinterpret_cast<const u32x4 *>(p.src);
     u32x4 *d = reinterpret_cast<u32x4 *>(p.dst);
-    const size_t nvec = p.bytes / 16, st = (size_t)gridDim.x * blockDim.x;
-    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t nvec = p.bytes / 16, st = (size_t)gridDim.x * WG_THREADS;
+    size_t i = (size_t)blockIdx.x * WG_THREADS + threadIdx.x;
     for (; i + 3 * st < nvec; i += 4 * st) {
         const u32x4 a = w[i], b = w[i + st], c = w[i + 2 * st], e = w[i + 3 * st];
         d[i] = a, d[i + st] = b, d[i + 2 * st] = c, d[i + 3 * st] = e;

@@ -39,7 +39,7 @@ __device__ __forceinline__ void rearrange32(const RearrangeParams &p) {
     bool ok[RE_ITEMS];
 #pragma unroll
     for (int it = 0; it < RE_ITEMS; ++it) {
-        const uint32_t g = (blockIdx.x * RE_ITEMS + it) * blockDim.x + threadIdx.x;
+        const uint32_t g = (blockIdx.x * RE_ITEMS + it) * WG_THREADS + threadIdx.x;
         ok[it] = g < total;
         doff[it] = 0;
         if (ok[it]) {
@@ -69,8 +69,8 @@ __device__ __forceinline__ void rearrange32(const RearrangeParams &p) {
 template <int B>
 __device__ __forceinline__ void rearrange64(const RearrangeParams &p) {
     typedef typename Chunk<B>::T T;
-    for (uint64_t g = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; g < p.total;
-         g += (uint64_t)gridDim.x * blockDim.x) {
+    for (uint64_t g = (uint64_t)blockIdx.x * WG_THREADS + threadIdx.x; g < p.total;
+         g += (uint64_t)gridDim.x * WG_THREADS) {
         const uint64_t u = g / p.chunks_per_unit;
         const uint64_t c = g % p.chunks_per_unit;
         uint64_t rem = u;

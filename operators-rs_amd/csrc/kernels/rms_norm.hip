@@ -151,8 +151,8 @@ template <typename TA, typename TW>
 __device__ __forceinline__ void rms_norm_rows(const RmsNormParams &p) {
     constexpr int CACHE = 8;
     const uint32_t lane = threadIdx.x % WAVE;
-    const uint32_t waves = gridDim.x * (blockDim.x / WAVE);
-    uint32_t row = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+    const uint32_t waves = gridDim.x * (WG_THREADS / WAVE);
+    uint32_t row = blockIdx.x * (WG_THREADS / WAVE) + threadIdx.x / WAVE;
     const uint32_t nvec = p.d / 8;
     if (row >= p.n) return;
 

@@ -24,7 +24,7 @@ __device__ __forceinline__ void rope_fill_table(const RopeParams &p, uint32_t to
     // one entry of the table per thread, the sines by the first H threads and the cosines by the next H: the
     // table is the kernel's critical path (everything else waits for it at the barrier)
     float *flat = reinterpret_cast<float *>(rope_sc);
-    for (uint32_t e = threadIdx.x; e < 2 * H; e += blockDim.x) {
+    for (uint32_t e = threadIdx.x; e < 2 * H; e += WG_THREADS) {
         const uint32_t k = e < H ? e : e - H;
         const float ang = pos / (p.has_den ? p.den[k] : powf(p.theta, (float)k / (float)H));
         flat[2 * k + (e < H ? 0 : 1)] = e < H ? sinf(ang) : cosf(ang);
@@ -47,7 +47,7 @@ __device__ __forceinline__ void rope_vec(const RopeParams &p) {  // T: f16 or bf
     first.u = u32x4{0, 0, 0, 0};
     if (threadIdx.x < total) first.u = ld128(chunk(threadIdx.x));
     rope_fill_table(p, token);
-    for (uint32_t v = threadIdx.x; v < total; v += blockDim.x) {
+    for (uint32_t v = threadIdx.x; v < total; v += WG_THREADS) {
         const uint32_t c = v % cpv;
         char *ptr = chunk(v);
         PackOf<T> x, o;
@@ -76,7 +76,7 @@ __device__ __forceinline__ void rope_pairs(const RopeParams &p) {
     const uint32_t h1 = min(h0 + p.heads_per_block, p.nh);
     const uint32_t total = (h1 - h0) * H;
     char *base = reinterpret_cast<char *>(p.t) + (int64_t)token * p.st;
-    for (uint32_t v = threadIdx.x; v < total; v += blockDim.x) {
+    for (uint32_t v = threadIdx.x; v < total; v += WG_THREADS) {
         const uint32_t h = h0 + v / H, k = v % H;
         T *ptr = reinterpret_cast<T *>(base + (int64_t)h * p.sh) + 2 * k;
         const float2 sc = rope_sc[k];
@@ -98,7 +98,7 @@ extern "C" __global__ void __launch_bounds__(256) rope_f64_pairs(RopeParams p) {
     const uint32_t H = p.dh / 2;
     const char *pp = reinterpret_cast<const char *>(p.pos) + (int64_t)token * p.sp;
     const double pos = p.pos_is_u64 ? (double)*reinterpret_cast<const uint64_t *>(pp) : (double)*reinterpret_cast<const uint32_t *>(pp);
-    for (uint32_t k = threadIdx.x; k < H; k += blockDim.x) {
+    for (uint32_t k = threadIdx.x; k < H; k += WG_THREADS) {
         const double ang = pos / pow((double)p.theta, (double)k / (double)H);
         table[k] = double2{sin(ang), cos(ang)};
     }
@@ -107,7 +107,7 @@ extern "C" __global__ void __launch_bounds__(256) rope_f64_pairs(RopeParams p) {
     const uint32_t h1 = min(h0 + p.heads_per_block, p.nh);
     const uint32_t total = (h1 - h0) * H;
     char *base = reinterpret_cast<char *>(p.t) + (int64_t)token * p.st;
-    for (uint32_t v = threadIdx.x; v < total; v += blockDim.x) {
+    for (uint32_t v = threadIdx.x; v < total; v += WG_THREADS) {
         const uint32_t h = h0 + v / H, k = v % H;
         double *ptr = reinterpret_cast<double *>(base + (int64_t)h * p.sh) + 2 * k;
         const double2 sc = table[k];

@@ -19,7 +19,7 @@ __device__ __forceinline__ void swiglu_vec(const SwigluParams &p) {  // T: f16 o
     if constexpr (NT) {
         // one vector per thread over the whole tensor (a row's vectors seldom fill whole workgroups: 11008 columns are
         // 5.4 of them; 16384 rows of them at 76 % of 8 TB/s against 71 % row by row, and two vectors per thread 75 %)
-        const uint32_t g = blockIdx.x * blockDim.x + threadIdx.x;
+        const uint32_t g = blockIdx.x * WG_THREADS + threadIdx.x;
         if (g >= p.total) return;
         const uint32_t row = fastdiv(g, p.per_row), v = g - row * p.per_row.d;
         char *gp = reinterpret_cast<char *>(p.gate) + (int64_t)row * p.sgn + (size_t)v * 16;
@@ -36,7 +36,7 @@ __device__ __forceinline__ void swiglu_vec(const SwigluParams &p) {  // T: f16 o
     for (uint32_t row = blockIdx.y; row < p.n; row += gridDim.y) {
         char *g = reinterpret_cast<char *>(p.gate) + (int64_t)row * p.sgn;
         const char *u = reinterpret_cast<const char *>(p.up) + (int64_t)row * p.sun;
-        for (uint32_t v = blockIdx.x * blockDim.x + threadIdx.x; v < nvec; v += gridDim.x * blockDim.x) {
+        for (uint32_t v = blockIdx.x * WG_THREADS + threadIdx.x; v < nvec; v += gridDim.x * WG_THREADS) {
             PackOf<T> a, b, o;
             a.u = ld128_nt(g + (size_t)v * 16);
             b.u = ld128_nt(u + (size_t)v * 16);
@@ -60,7 +60,7 @@ __device__ __forceinline__ void swiglu_scalar(const SwigluParams &p) {
     for (uint32_t row = blockIdx.y; row < p.n; row += gridDim.y) {
         T *g = reinterpret_cast<T *>(reinterpret_cast<char *>(p.gate) + (int64_t)row * p.sgn);
         const T *u = reinterpret_cast<const T *>(reinterpret_cast<const char *>(p.up) + (int64_t)row * p.sun);
-        for (uint32_t j = blockIdx.x * blockDim.x + threadIdx.x; j < p.d; j += gridDim.x * blockDim.x) {
+        for (uint32_t j = blockIdx.x * WG_THREADS + threadIdx.x; j < p.d; j += gridDim.x * WG_THREADS) {
             if constexpr (sizeof(T) == 8) g[j] = swiglu_f64(g[j], u[j]);
             else g[j] = (T)swiglu_f32((float)g[j], (float)u[j]);
         }
