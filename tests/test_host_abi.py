@@ -302,3 +302,32 @@ def test_every_operator_of_the_rust_side_names_what_the_header_has():
                 literals += 1
     assert len(used) >= 60 and literals >= 11
     assert used <= known, sorted(used - known)
+
+
+# ---- the kernels' workgroup size against the host's launches, as text ---------------------------------------------
+
+def test_kernels_that_stride_by_their_workgroup_size_are_launched_with_it():
+    """The streaming kernels advance by the constant WG_THREADS (device_util.h) instead of blockDim.x (which, read
+    inside a __device__ function, costs a vector load and a wait at the head of every workgroup): no kernel source may
+    read blockDim inside such a function, and the host must launch every kernel of those files with exactly that many
+    threads, or with a size the kernel takes as a template argument."""
+    csrc = os.path.join(ROOT, "operators-rs_amd", "csrc")
+    util = open(os.path.join(csrc, "kernels", "device_util.h")).read()
+    wg = int(re.search(r"constexpr uint32_t WG_THREADS = (\d+);", util).group(1))
+    assert wg == 256
+    users = []
+    for f in sorted(os.listdir(os.path.join(csrc, "kernels"))):
+        if not f.endswith(".hip"):
+            continue
+        text = re.sub(r"//[^\n]*", " ", open(os.path.join(csrc, "kernels", f)).read())
+        if "WG_THREADS" in text:
+            users.append(f[:-4])
+        for m in re.finditer(r"blockDim", text):
+            # allowed only directly in a __global__ function: the nearest function head above it is one
+            head = text.rfind("__global__", 0, m.start()), text.rfind("__device__", 0, m.start())
+            assert head[0] > head[1], (f, text[m.start() - 60:m.start() + 20])
+    assert {"add", "add_rows", "gelu", "swiglu", "rearrange", "rope", "rms_norm", "layer_norm"} <= set(users)
+    # the host's launches of those modules: Dim3{256}, Dim3{block} (a templated group size) or the 1024-thread stream kernels
+    host = "".join(open(os.path.join(csrc, "host", f)).read() for f in ("ops.cpp", "ops_more.cpp", "handle.cpp"))
+    sizes = set(re.findall(r"launch\([^;]*?Dim3\{[^;]*?\},\s*Dim3\{([^}]*)\}", host, re.S))
+    assert sizes <= {"256", "block", "1024", "256u", "1"}, sizes
