@@ -645,6 +645,18 @@ def standalone_ops(ophip, gpu, stream, rng, reps, ceiling=None):
     us = time_launches(gpu, stream, launch_rotating, max(reps, 2 * len(rot)), warm=len(rot))
     add("attention_kv_cached", "nh32 seq16 pos2032 dh128, ten cache sets in rotation", 2 * NH * KV * DH * 2 + 8 * nt * D * 2, us,
         note="as above on caches that come from HBM")
+    # attention itself at the same shape (a caller that keeps its own cache): q from the QKV rows against the full caches
+    att_op = o.Attention(gpu)
+    rot_at = [o.AttentionArgs(head_major(3 * D * 2), qkv.ptr, c(NH, KV, DH), kb_, c(NH, KV, DH), vb_, head_major(D * 2), obuf,
+                              o.AttnMask.CAUSAL) for kb_, vb_ in sets]
+    ws_at = gpu.malloc(max(att_op.scheme(rot_at[0], 1 << 30), 1))
+
+    def launch_rotating_attention():
+        att_op.launch(rot_at[turn[0] % len(rot_at)], ws_at, stream)
+        turn[0] += 1
+    us = time_launches(gpu, stream, launch_rotating_attention, max(reps, 2 * len(rot_at)), warm=len(rot_at))
+    add("attention", "nh32 seq16 att2048 dh128 causal (decode shape), ten cache sets in rotation", 2 * NH * KV * DH * 2 + 2 * nt * D * 2, us,
+        flops=4 * NH * nt * KV * DH, note="the decode kernel of attention_kv_cached with nothing to append (the crate's composite: 5 launches)")
     for kb_, vb_ in sets[1:]:
         kb_.free(); vb_.free()
     attention_lines(o, gpu, stream, rng, add, max(5, reps // 2))

@@ -99,6 +99,11 @@ struct ophip_attention {
     // OPHIP_ATTN_FUSED=0 keeps the composite (tests, comparisons), =1 takes the one-pass kernel wherever it applies;
     // read once, here.  Otherwise an estimate of the two times decides (attention_one_pass).
     int fused = -1;
+    // the one-pass kernels for decode shapes (few query rows per kv head against many keys; attention_kv_cached uses them
+    // through its own attention operator): [f16 / bf16][16 * {1, 2, 4} query rows per kv head][dh 64 / 128]
+    hipFunction_t decode[2][3][2][2], combine[2][3][2];  // decode: [..][..][..][256 / 128 keys per workgroup]
+    bool one_pass = true;  // OPHIP_ATTN_ONE_PASS=0 keeps the composite (tests, comparisons); read once, here
+    int force_chunk = 0;   // OPHIP_ATTN_CHUNK=256|128 keeps one chunk size (sweeps)
     explicit ophip_attention(ophip_device *d) : dev(d) {
         ophip_device_retain(d);
         try {
@@ -112,6 +117,18 @@ struct ophip_attention {
                 prefill[e][0][1] = d->kernel(mod.c_str(), ("attn_prefill_d64_g2" + tag).c_str());
                 prefill[e][1][1] = d->kernel(mod.c_str(), ("attn_prefill_d128_g2" + tag).c_str());
             }
+            static const char *mt_tag[3] = {"m1", "m2", "m4"}, *dh_tag[2] = {"d64", "d128"};
+            for (int e = 0; e < 2; ++e)
+                for (int i = 0; i < 3; ++i)
+                    for (int j = 0; j < 2; ++j) {
+                        const std::string mod = e ? "attention_decode_bf16" : "attention_decode", tag = e ? "_bf16" : "";
+                        const std::string tail = std::string(mt_tag[i]) + "_" + dh_tag[j];
+                        decode[e][i][j][0] = d->kernel(mod.c_str(), ("attn_decode_" + tail + "_k64" + tag).c_str());
+                        decode[e][i][j][1] = d->kernel(mod.c_str(), ("attn_decode_" + tail + "_k32" + tag).c_str());
+                        combine[e][i][j] = d->kernel(mod.c_str(), ("attn_decode_combine_" + tail + tag).c_str());
+                    }
+            if (const char *e = std::getenv("OPHIP_ATTN_ONE_PASS")) one_pass = std::atoi(e) != 0;
+            if (const char *e = std::getenv("OPHIP_ATTN_CHUNK")) force_chunk = std::atoi(e);
             if (const char *e = std::getenv("OPHIP_ATTN_FUSED")) fused = std::atoi(e) != 0;
             if (const char *e = std::getenv("OPHIP_ATTN_KEYSPLIT")) key_split = std::atoi(e) != 0;
         } catch (...) {
@@ -259,6 +276,86 @@ bool attention_one_pass(const ophip_attention *op, const ophip_attention_args &a
     return true;
 }
 
+// Keys per workgroup of the one-pass kernel: 256, or 128 when that leaves CUs without a workgroup (measured: the
+// decode layer, 32 kv heads x 2048 keys, 15.5 us with 256 keys against 17.0; 8 kv heads x 4096 keys 12.3 against 10.7).
+size_t decode_chunk(size_t nkvh, size_t att, unsigned cus, int force) {
+    if (force == 256 || force == 128) return (size_t)force;
+    return (att + 255) / 256 * nkvh < (size_t)cus ? 128 : 256;
+}
+
+// Workspace of the one-pass kernel for these sizes, or SIZE_MAX when it does not serve them (the shapes alone
+// decide here; launch also looks at strides and alignment).
+size_t one_pass_workspace(uint64_t dt, size_t nh, size_t nkvh, size_t seq, size_t att, size_t dh, size_t chunk) {
+    if ((dt != OPHIP_DT_F16 && dt != OPHIP_DT_BF16) || (dh != 64 && dh != 128) || nkvh == 0 || nh % nkvh != 0 || seq == 0 || att == 0) return SIZE_MAX;
+    const size_t rows = nh / nkvh * seq;
+    if (rows > 64 || att > 0x7fffffffu) return SIZE_MAX;
+    const size_t nchunk = (att + chunk - 1) / chunk, rp = rows <= 16 ? 16 : rows <= 32 ? 32 : 64;
+    return nchunk == 1 ? 0 : nkvh * nchunk * rp * (dh + 2) * sizeof(float);
+}
+
+// One call of the one-pass decode kernel (attention_decode.hip): q against the first `pos` rows of the caches followed by
+// the rows of k_new / v_new, which the kernel also appends to the caches at `pos`; att = keys in all.  With pos = att
+// nothing is new and nothing is appended: plain attention over k and v.  As in the reference's attention_kv_cached the
+// v-cache is addressed with the k-cache's strides.
+struct DecodeCall {
+    uint64_t dt;
+    int mask;
+    size_t nh, nkvh, seq, dh, att, pos;
+    const ophip_tensor_layout *q, *o, *k_new, *v_new, *k_cache;
+    void *q_base, *o_base;
+    const void *k_new_base, *v_new_base;
+    void *k_cache_base, *v_cache_base;
+};
+
+// The kernel when it serves this call; false, with nothing done, otherwise.
+bool decode_one_pass(const ophip_attention *op, const DecodeCall &c, void *workspace, size_t workspace_len, const ophip_queue_alloc *qa) {
+    if (!op->one_pass) return false;
+    const size_t nh = c.nh, nkvh = c.nkvh, seq = c.seq, dh = c.dh, att = c.att;
+    const size_t chunk = decode_chunk(nkvh, att, (unsigned)op->dev->props.multiProcessorCount, op->force_chunk);
+    const size_t need = one_pass_workspace(c.dt, nh, nkvh, seq, att, dh, chunk);
+    if (need == SIZE_MAX || (c.mask != OPHIP_MASK_NONE && c.mask != OPHIP_MASK_CAUSAL)) return false;
+    if (c.mask == OPHIP_MASK_CAUSAL && att < seq) return false;  // rows that keep no column: the softmax of the composite refuses them
+    // every tensor: dh contiguous, rows and heads on 16-byte boundaries
+    auto fits = [](const ophip_tensor_layout &l, const void *base) {
+        for (int i = 0; i < 3; ++i)
+            if (is_dyn(l.strides[i])) return false;
+        return l.strides[2] == 2 && mult16(l.strides[0]) && mult16(l.strides[1]) && aligned16(base);
+    };
+    if (!fits(*c.q, c.q_base) || !fits(*c.o, c.o_base) || !fits(*c.k_new, c.k_new_base) || !fits(*c.v_new, c.v_new_base) ||
+        !fits(*c.k_cache, c.k_cache_base) || !aligned16(c.v_cache_base))
+        return false;
+    const size_t group = nh / nkvh, rows = group * seq;
+    AttnDecodeParams p{};
+    p.q = c.q_base;
+    p.o = c.o_base;
+    // the reference overwrites q with the result when q's heads and tokens merge (attention/operator.rs:186-239)
+    const ptrdiff_t nh_sq = c.q->strides[0], seq_sq = c.q->strides[1];
+    const bool merged = nh == 1 || seq == 1 || nh_sq == (ptrdiff_t)seq * seq_sq;
+    p.q_out = merged && c.q_base != c.o_base ? c.q_base : nullptr;
+    p.k_new = c.k_new_base;
+    p.v_new = c.v_new_base;
+    p.k_cache = c.k_cache_base;
+    p.v_cache = c.v_cache_base;
+    p.q_sh = nh_sq / 2, p.q_ss = seq_sq / 2;
+    p.o_sh = c.o->strides[0] / 2, p.o_ss = c.o->strides[1] / 2;
+    p.kn_sh = c.k_new->strides[0] / 2, p.kn_ss = c.k_new->strides[1] / 2;
+    p.vn_sh = c.v_new->strides[0] / 2, p.vn_ss = c.v_new->strides[1] / 2;
+    p.kc_sh = c.k_cache->strides[0] / 2, p.kc_ss = c.k_cache->strides[1] / 2;
+    p.nkvh = (uint32_t)nkvh, p.group = (uint32_t)group, p.seq = (uint32_t)seq, p.att = (uint32_t)att, p.pos = (uint32_t)c.pos;
+    p.nchunk = (uint32_t)((att + chunk - 1) / chunk);
+    p.causal = c.mask == OPHIP_MASK_CAUSAL;
+    // the reference's mat_mul rounds alpha to the data type
+    p.scale = c.dt == OPHIP_DT_BF16 ? round_to_bf16(1.0f / std::sqrt((float)dh)) : round_to_f16(1.0f / std::sqrt((float)dh));
+    if (p.nchunk > 65535 || nkvh > 65535) return false;
+    Workspace ws(qa, workspace, workspace_len, need);
+    p.partial = static_cast<float *>(ws.ptr());
+    const int mi = rows <= 16 ? 0 : rows <= 32 ? 1 : 2, di = dh == 64 ? 0 : 1, ei = c.dt == OPHIP_DT_BF16 ? 1 : 0;
+    op->dev->make_current();
+    launch(op->decode[ei][mi][di][chunk == 256 ? 0 : 1], Dim3{p.nchunk, (unsigned)nkvh}, Dim3{256}, 0, stream_of(qa), p);
+    if (p.nchunk > 1) launch(op->combine[ei][mi][di], Dim3{(unsigned)(nkvh * rows)}, Dim3{256}, 0, stream_of(qa), p);
+    return true;
+}
+
 // Operator::launch (attention/operator.rs:143-277).  q is overwritten with att . v, as in
 // the reference, unless it had to be copied into the workspace first.
 void attention_launch(const ophip_attention *op, const ophip_attention_args &args, void *workspace,
@@ -278,6 +375,21 @@ void attention_launch(const ophip_attention *op, const ophip_attention_args &arg
     // when the head stride is seq * token stride (a dimension of length 1 folds with anything)
     const bool merged = nh == 1 || seq == 1 || nh_sq == (ptrdiff_t)seq * seq_sq;
     const ptrdiff_t row_sq = seq == 1 ? nh_sq : seq_sq;  // stride of the merged [nh * seq] dimension
+    // Few rows per kv head against k and v of one layout: the decode kernel with nothing to append (unless a knob asks
+    // for the composite or for the prefill kernel).
+    if (op->fused == -1 && !is_dyn(args.v_layout.strides[0]) && args.v_layout.strides[0] == args.k_layout.strides[0] &&
+        args.v_layout.strides[1] == args.k_layout.strides[1]) {
+        DecodeCall c{};
+        c.dt = dt, c.mask = args.mask;
+        c.nh = nh, c.nkvh = nkvh, c.seq = seq, c.dh = dh, c.att = att, c.pos = att;
+        c.q = &args.q_layout, c.q_base = args.q_base;
+        c.o = &args.o_layout, c.o_base = args.o_base;
+        c.k_new = &args.k_layout, c.k_new_base = args.k_base;
+        c.v_new = &args.v_layout, c.v_new_base = args.v_base;
+        c.k_cache = &args.k_layout, c.k_cache_base = const_cast<void *>(args.k_base);
+        c.v_cache_base = const_cast<void *>(args.v_base);
+        if (decode_one_pass(op, c, workspace, workspace_len, qa)) return;
+    }
     if (attention_one_pass(op, args, m, merged, qa)) return;
     // k^T: ArrayLayout::transpose(&[2, 1])
     const Lay3 kt{{nkvh, dh, att}, {nkvh_sk, dh_sk, att_sk}};
@@ -333,27 +445,11 @@ struct ophip_attention_kv_cached {
     ophip_device *dev;
     ophip_rearrange *rearrange = nullptr;
     ophip_attention *attention = nullptr;
-    // the one-pass kernels for decode shapes: [f16 / bf16][16 * {1, 2, 4} query rows per kv head][dh 64 / 128]
-    hipFunction_t decode[2][3][2][2], combine[2][3][2];  // decode: [..][..][..][256 / 128 keys per workgroup]
-    bool one_pass = true;  // OPHIP_ATTN_ONE_PASS=0 keeps the composite (tests, comparisons); read once, here
-    int force_chunk = 0;   // OPHIP_ATTN_CHUNK=256|128 keeps one chunk size (sweeps)
     explicit ophip_attention_kv_cached(ophip_device *d) : dev(d) {
         ophip_device_retain(d);
         try {
             sub(ophip_rearrange_create(d, &rearrange));
             sub(ophip_attention_create(d, &attention));
-            static const char *mt_tag[3] = {"m1", "m2", "m4"}, *dh_tag[2] = {"d64", "d128"};
-            for (int e = 0; e < 2; ++e)
-                for (int i = 0; i < 3; ++i)
-                    for (int j = 0; j < 2; ++j) {
-                        const std::string mod = e ? "attention_decode_bf16" : "attention_decode", tag = e ? "_bf16" : "";
-                        const std::string tail = std::string(mt_tag[i]) + "_" + dh_tag[j];
-                        decode[e][i][j][0] = d->kernel(mod.c_str(), ("attn_decode_" + tail + "_k64" + tag).c_str());
-                        decode[e][i][j][1] = d->kernel(mod.c_str(), ("attn_decode_" + tail + "_k32" + tag).c_str());
-                        combine[e][i][j] = d->kernel(mod.c_str(), ("attn_decode_combine_" + tail + tag).c_str());
-                    }
-            if (const char *e = std::getenv("OPHIP_ATTN_ONE_PASS")) one_pass = std::atoi(e) != 0;
-            if (const char *e = std::getenv("OPHIP_ATTN_CHUNK")) force_chunk = std::atoi(e);
         } catch (...) {
             release();
             throw;
@@ -396,23 +492,6 @@ KvCachedMeta kv_cached_meta(const ophip_attention_kv_cached_args &a) {
     return m;
 }
 
-// Keys per workgroup of the one-pass kernel: 256, or 128 when that leaves CUs without a workgroup (measured: the
-// decode layer, 32 kv heads x 2048 keys, 15.5 us with 256 keys against 17.0; 8 kv heads x 4096 keys 12.3 against 10.7).
-size_t decode_chunk(size_t nkvh, size_t att, unsigned cus, int force) {
-    if (force == 256 || force == 128) return (size_t)force;
-    return (att + 255) / 256 * nkvh < (size_t)cus ? 128 : 256;
-}
-
-// Workspace of the one-pass kernel for these sizes, or SIZE_MAX when it does not serve them (the shapes alone
-// decide here; launch also looks at strides and alignment).
-size_t one_pass_workspace(uint64_t dt, size_t nh, size_t nkvh, size_t seq, size_t att, size_t dh, size_t chunk) {
-    if ((dt != OPHIP_DT_F16 && dt != OPHIP_DT_BF16) || (dh != 64 && dh != 128) || nkvh == 0 || nh % nkvh != 0 || seq == 0 || att == 0) return SIZE_MAX;
-    const size_t rows = nh / nkvh * seq;
-    if (rows > 64 || att > 0x7fffffffu) return SIZE_MAX;
-    const size_t nchunk = (att + chunk - 1) / chunk, rp = rows <= 16 ? 16 : rows <= 32 ? 32 : 64;
-    return nchunk == 1 ? 0 : nkvh * nchunk * rp * (dh + 2) * sizeof(float);
-}
-
 // Operator::scheme (attention_kv_cached/operator.rs:42-77)
 size_t kv_cached_scheme(ophip_attention_kv_cached *op, const ophip_attention_kv_cached_args &args, size_t max_ws) {
     const KvCachedMeta m = kv_cached_meta(args);
@@ -433,9 +512,9 @@ size_t kv_cached_scheme(ophip_attention_kv_cached *op, const ophip_attention_kv_
     wc.push_sub(need);
     size_t ans = wc.calculate(max_ws);
     // a launch of these sizes may run on the one-pass kernel instead: a workspace that serves either
-    if (op->one_pass && !is_dyn(m.nh) && !is_dyn(m.nkvh) && !is_dyn(m.dh) && !is_dyn(att)) {
+    if (op->attention->one_pass && !is_dyn(m.nh) && !is_dyn(m.nkvh) && !is_dyn(m.dh) && !is_dyn(att)) {
         const size_t fused = one_pass_workspace(m.dt, m.nh, m.nkvh, m.seq, att, m.dh,
-                                                decode_chunk(m.nkvh, att, (unsigned)op->dev->props.multiProcessorCount, op->force_chunk));
+                                                decode_chunk(m.nkvh, att, (unsigned)op->dev->props.multiProcessorCount, op->attention->force_chunk));
         if (fused != SIZE_MAX && fused <= max_ws) ans = std::max(ans, fused);
     }
     return ans;
@@ -444,50 +523,16 @@ size_t kv_cached_scheme(ophip_attention_kv_cached *op, const ophip_attention_kv_
 // The one-pass kernel (attention_decode.hip) when it serves this call; false, with nothing done, otherwise.
 bool kv_cached_one_pass(const ophip_attention_kv_cached *op, const ophip_attention_kv_cached_args &args, const KvCachedMeta &m,
                         size_t pos, size_t att, void *workspace, size_t workspace_len, const ophip_queue_alloc *qa) {
-    if (!op->one_pass) return false;
-    const size_t nh = static_of(m.nh), nkvh = static_of(m.nkvh), seq = static_of(m.seq), dh = static_of(m.dh);
-    const size_t chunk = decode_chunk(nkvh, att, (unsigned)op->dev->props.multiProcessorCount, op->force_chunk);
-    const size_t need = one_pass_workspace(m.dt, nh, nkvh, seq, att, dh, chunk);
-    if (need == SIZE_MAX || (args.mask != OPHIP_MASK_NONE && args.mask != OPHIP_MASK_CAUSAL)) return false;
-    // every tensor: dh contiguous, rows and heads on 16-byte boundaries
-    auto fits = [](const ophip_tensor_layout &l, const void *base) {
-        for (int i = 0; i < 3; ++i)
-            if (is_dyn(l.strides[i])) return false;
-        return l.strides[2] == 2 && mult16(l.strides[0]) && mult16(l.strides[1]) && aligned16(base);
-    };
-    if (!fits(args.q_layout, args.q_base) || !fits(args.o_layout, args.o_base) || !fits(args.k_layout, args.k_base) ||
-        !fits(args.v_layout, args.v_base) || !fits(args.k_cache_layout, args.k_cache_base) || !aligned16(args.v_cache_base))
-        return false;
-    const size_t group = nh / nkvh, rows = group * seq;
-    AttnDecodeParams p{};
-    p.q = args.q_base;
-    p.o = args.o_base;
-    // the reference overwrites q with the result when q's heads and tokens merge (attention/operator.rs:186-239)
-    const ptrdiff_t nh_sq = args.q_layout.strides[0], seq_sq = args.q_layout.strides[1];
-    const bool merged = nh == 1 || seq == 1 || nh_sq == (ptrdiff_t)seq * seq_sq;
-    p.q_out = merged && args.q_base != args.o_base ? args.q_base : nullptr;
-    p.k_new = args.k_base;
-    p.v_new = args.v_base;
-    p.k_cache = args.k_cache_base;
-    p.v_cache = args.v_cache_base;
-    p.q_sh = nh_sq / 2, p.q_ss = seq_sq / 2;
-    p.o_sh = args.o_layout.strides[0] / 2, p.o_ss = args.o_layout.strides[1] / 2;
-    p.kn_sh = args.k_layout.strides[0] / 2, p.kn_ss = args.k_layout.strides[1] / 2;
-    p.vn_sh = args.v_layout.strides[0] / 2, p.vn_ss = args.v_layout.strides[1] / 2;
-    p.kc_sh = args.k_cache_layout.strides[0] / 2, p.kc_ss = args.k_cache_layout.strides[1] / 2;
-    p.nkvh = (uint32_t)nkvh, p.group = (uint32_t)group, p.seq = (uint32_t)seq, p.att = (uint32_t)att, p.pos = (uint32_t)pos;
-    p.nchunk = (uint32_t)((att + chunk - 1) / chunk);
-    p.causal = args.mask == OPHIP_MASK_CAUSAL;
-    // the reference's mat_mul rounds alpha to the data type
-    p.scale = m.dt == OPHIP_DT_BF16 ? round_to_bf16(1.0f / std::sqrt((float)dh)) : round_to_f16(1.0f / std::sqrt((float)dh));
-    if (p.nchunk > 65535 || nkvh > 65535) return false;
-    Workspace ws(qa, workspace, workspace_len, need);
-    p.partial = static_cast<float *>(ws.ptr());
-    const int mi = rows <= 16 ? 0 : rows <= 32 ? 1 : 2, di = dh == 64 ? 0 : 1, ei = m.dt == OPHIP_DT_BF16 ? 1 : 0;
-    op->dev->make_current();
-    launch(op->decode[ei][mi][di][chunk == 256 ? 0 : 1], Dim3{p.nchunk, (unsigned)nkvh}, Dim3{256}, 0, stream_of(qa), p);
-    if (p.nchunk > 1) launch(op->combine[ei][mi][di], Dim3{(unsigned)(nkvh * rows)}, Dim3{256}, 0, stream_of(qa), p);
-    return true;
+    DecodeCall c{};
+    c.dt = m.dt, c.mask = args.mask;
+    c.nh = static_of(m.nh), c.nkvh = static_of(m.nkvh), c.seq = static_of(m.seq), c.dh = static_of(m.dh), c.att = att, c.pos = pos;
+    c.q = &args.q_layout, c.q_base = args.q_base;
+    c.o = &args.o_layout, c.o_base = args.o_base;
+    c.k_new = &args.k_layout, c.k_new_base = args.k_base;
+    c.v_new = &args.v_layout, c.v_new_base = args.v_base;
+    c.k_cache = &args.k_cache_layout, c.k_cache_base = args.k_cache_base;
+    c.v_cache_base = args.v_cache_base;
+    return decode_one_pass(op->attention, c, workspace, workspace_len, qa);
 }
 
 // Operator::launch (attention_kv_cached/operator.rs:79-183).  As in the reference, the

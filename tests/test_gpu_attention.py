@@ -465,3 +465,67 @@ def test_prefill_layer_chain_matches_the_oracle_end_to_end(gpu, stream):
     say("prefill layer: max err %.3g, median err %.3g, output scale %.3g" % (err.max(), np.median(err), scale))
     assert err.max() <= 1e-2 * scale, err.max() / scale
     assert np.median(err) <= 1e-3 * scale, np.median(err) / scale
+
+
+# ------------------------------------------------ attention at decode shapes ----
+# `attention` with few query rows per kv head against many keys (a runtime that keeps its own cache and calls attention
+# on it) runs on the decode kernel of attention_kv_cached with nothing to append, when k and v have one layout.
+
+@pytest.mark.parametrize("nh,nkvh,seq,att,dh,mask", [
+    (32, 32, 16, 2048, 128, CAUSAL),   # the decode layer's shape: 16 rows per kv head, 8 chunks
+    (32, 8, 1, 4096, 128, CAUSAL),     # one token, grouped heads
+    (32, 4, 7, 127, 64, CAUSAL),       # attention/cuda.rs: 56 rows per kv head, one ragged chunk
+    (12, 4, 5, 257, 128, NONE),        # no mask, a second chunk with one key
+    (3, 3, 33, 100, 64, CAUSAL),       # 33 rows per kv head
+    (8, 8, 64, 64, 128, CAUSAL),       # as many rows as keys
+])
+def test_attention_at_decode_shapes_runs_in_one_pass(gpu, stream, monkeypatch, nh, nkvh, seq, att, dh, mask):
+    """Against f64 and the oracle's composite, and against the composite of launches (OPHIP_ATTN_FUSED=0) for what the
+    reference makes observable besides o: q overwritten with the result (contiguous q: heads and tokens merge), k and v
+    untouched."""
+    rng = np.random.default_rng(nh + seq + att + dh)
+    q, k, v = normal_f16(rng, (nh, seq, dh)), normal_f16(rng, (nkvh, att, dh)), normal_f16(rng, (nkvh, att, dh))
+    say("attention at a decode shape nh=%d nkvh=%d seq=%d att=%d dh=%d mask=%d" % (nh, nkvh, seq, att, dh, mask))
+    qd, kd, vd = upload(gpu, q), upload(gpu, k), upload(gpu, v)
+    od = gpu.malloc(q.nbytes)
+    gpu.memset(od, 0xFF)
+    lay = TensorLayout.of
+    args = ophip.AttentionArgs(lay(q), qd, lay(k), kd, lay(v), vd, lay(q), od, mask)
+    ophip.Attention(gpu).launch(args, None, stream)
+    out, q_after = download(gpu, stream, od, q), download(gpu, stream, qd, q)
+    assert np.array_equal(download(gpu, stream, kd, k), k) and np.array_equal(download(gpu, stream, vd, v), v)
+    assert_close_f16(out, attention_f64(q, k, v, mask == CAUSAL), "decode kernel vs f64")
+    assert_close_f16(out, oracle.attention(q.copy(), k, v, np.zeros_like(q), causal=(mask == CAUSAL)), "decode kernel vs oracle")
+    assert np.array_equal(q_after, out)
+    monkeypatch.setenv("OPHIP_ATTN_FUSED", "0")
+    b, qb = run_attention(gpu, stream, q, k, v, mask)
+    assert_close_f16(b, attention_f64(q, k, v, mask == CAUSAL), "composite vs f64")
+    assert np.array_equal(qb, b)
+    # the two paths differ where the composite rounds scores and probabilities to f16: well inside the bar of either
+    assert np.abs(out.astype(np.float32) - b.astype(np.float32)).max() <= 4e-3
+
+
+def test_attention_at_a_decode_shape_with_strided_views_and_separate_layouts(gpu, stream):
+    """q inside a token-major QKV buffer (heads and tokens do not merge: q stays as it was), k and v as views of caches
+    longer than att; then v with another layout than k, which the decode kernel does not take (the other paths do)."""
+    rng = np.random.default_rng(99)
+    nh, nkvh, seq, att, dh, buf = 8, 2, 4, 300, 128, 512
+    q, kc, vc = normal_f16(rng, (nh, seq, dh)), normal_f16(rng, (nkvh, buf, dh)), normal_f16(rng, (nkvh, buf, dh))
+    row = nh * dh
+    qkv = np.ascontiguousarray(q.transpose(1, 0, 2).reshape(seq, row))
+    qd, kd, vd = upload(gpu, qkv), upload(gpu, kc), upload(gpu, vc)
+    od = gpu.malloc(q.nbytes)
+    q_lay = TensorLayout(dt.F16, [nh, seq, dh], [dh * 2, row * 2, 2])
+    kv_lay = TensorLayout(dt.F16, [nkvh, att, dh], [buf * dh * 2, dh * 2, 2])
+    o_lay = TensorLayout.new_contiguous(dt.F16, [nh, seq, dh])
+    say("attention at a decode shape, strided views")
+    ophip.Attention(gpu).launch(ophip.AttentionArgs(q_lay, qd, kv_lay, kd, kv_lay, vd, o_lay, od, CAUSAL), None, stream)
+    ref = attention_f64(q, kc[:, :att], vc[:, :att], True)
+    assert_close_f16(download(gpu, stream, od, q), ref, "views vs f64")
+    assert np.array_equal(download(gpu, stream, qd, qkv), qkv)  # staged in the reference, left alone here
+    # v stored [att, nkvh, dh]: another layout than k's
+    vt = np.ascontiguousarray(vc[:, :att].transpose(1, 0, 2))
+    vtd = upload(gpu, vt)
+    v_lay = TensorLayout(dt.F16, [nkvh, att, dh], [dh * 2, nkvh * dh * 2, 2])
+    ophip.Attention(gpu).launch(ophip.AttentionArgs(q_lay, qd, kv_lay, kd, v_lay, vtd, o_lay, od, CAUSAL), None, stream)
+    assert_close_f16(download(gpu, stream, od, q), ref, "separate layouts vs f64")
