@@ -443,7 +443,11 @@ OPHIP_API int ophip_mat_mul_describe(const ophip_mat_mul *op, const ophip_mat_mu
  * nh must be a multiple of nkvh.  As in the reference, q is overwritten (it
  * receives att . v before the copy into o) unless its layout forces a staging
  * copy, and launch() needs nh*seq*(dh + att) elements of workspace, taken from
- * the queue allocator when the caller's slice is smaller. */
+ * the queue allocator when the caller's slice is smaller.
+ * f16 / bf16 shapes that one kernel serves (prefill: many query rows per head;
+ * decode: up to 64 rows per kv head with k and v of one layout) run on it instead
+ * of the composite's launches: the same o within the f16 bar, q overwritten or
+ * left alone exactly as the composite would, k and v untouched. */
 typedef struct ophip_attention_args {
     ophip_tensor_layout q_layout;
     void *q_base;
