@@ -505,7 +505,8 @@ def test_swiglu_reference_shape(gpu, stream):
 
 
 @pytest.mark.parametrize("n,d,ld", [(16, 11008, 22016), (3, 1001, 2002), (1, 8, 16), (70000, 16, 40), (8195, 512, 1032),
-                                     (16400, 2048, 4096)])  # the last: > 64 MiB
+                                     (16400, 2048, 4096), (3100, 11008, 22016)])  # the last two: > 64 MiB (one vector per thread
+                                                                                   # over the whole tensor; 1376 vectors a row: workgroups straddle rows)
 def test_swiglu_gate_up_halves(gpu, stream, n, d, ld):
     """gate and up are the two halves of one [n, 2*d] GEMM output (independent row strides)."""
     rng = np.random.default_rng(n + d)
