@@ -293,9 +293,21 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
                 // and when the part of the last tiles that lies outside the matrix costs more than the large tile's
                 // advantage (about 1.4 x per multiply at these sizes)
                 if (b == 256 && !force) {
-                    const size_t t256 = (size_t)((p.M + 255) / 256) * ((p.N + 255) / 256);
-                    const size_t t128 = (size_t)((p.M + 127) / 128) * ((p.N + 127) / 128);
-                    if (t256 * p.batch * 5 < (size_t)cus * 3 || t256 * 4 * 5 > t128 * 7) continue;
+                    const size_t t256 = (size_t)((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batch;
+                    const size_t t128 = (size_t)((p.M + 127) / 128) * ((p.N + 127) / 128) * p.batch;
+                    // A last round of a few tiles costs a whole round.  The 128 tiles (two to a CU) after full rounds:
+                    const size_t tail128 = t128 % (2 * (size_t)cus), tail256 = t256 % (size_t)cus;
+                    const bool bad128 = t128 > 2 * (size_t)cus && tail128 != 0 && tail128 * 4 <= (size_t)cus;
+                    // and the 256 tiles: 640 x 22016 x 4096 is 258 of them, 198 us against 135 on 128 tiles (768 rows: 187 / 167;
+                    // 1024 rows, 344 tiles: 189 / 202)
+                    if (t256 > (size_t)cus && t256 < 3 * (size_t)cus && tail256 != 0 && tail256 * 4 < (size_t)cus) continue;
+                    // too few 256 tiles for the CUs, unless the 128 tiles end on such a round (768 x 12288 x 4096: 144 tiles
+                    // 81 us, 576 tiles of 128 97 us)
+                    if (t256 * 5 < (size_t)cus * 3 && !bad128) continue;
+                    // the part of the last tiles outside the matrix: at a third more area (384 rows) the 128 tiles win by a
+                    // tenth (384 x 32000 x 4096: 128 / 117 us) unless they end on a short round (384 x 22016: 94 / 97)
+                    if (t256 * 4 * 10 >= t128 * 13 && !bad128) continue;
+                    if (t256 * 4 * 5 > t128 * 7) continue;
                 }
                 // (gemm_splitk_reduce works on groups of 8 columns: an orientation whose N is no multiple of 8 cannot split)
                 const bool can_split = split > 1 && p.N % 8 == 0;
