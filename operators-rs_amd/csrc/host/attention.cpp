@@ -149,6 +149,23 @@ struct ophip_attention {
 
 namespace {
 
+// Keys per workgroup of the one-pass kernel: 256, or 128 when that leaves CUs without a workgroup (measured: the
+// decode layer, 32 kv heads x 2048 keys, 15.5 us with 256 keys against 17.0; 8 kv heads x 4096 keys 12.3 against 10.7).
+size_t decode_chunk(size_t nkvh, size_t att, unsigned cus, int force) {
+    if (force == 256 || force == 128) return (size_t)force;
+    return (att + 255) / 256 * nkvh < (size_t)cus ? 128 : 256;
+}
+
+// Workspace of the one-pass kernel for these sizes, or SIZE_MAX when it does not serve them (the shapes alone
+// decide here; launch also looks at strides and alignment).
+size_t one_pass_workspace(uint64_t dt, size_t nh, size_t nkvh, size_t seq, size_t att, size_t dh, size_t chunk) {
+    if ((dt != OPHIP_DT_F16 && dt != OPHIP_DT_BF16) || (dh != 64 && dh != 128) || nkvh == 0 || nh % nkvh != 0 || seq == 0 || att == 0) return SIZE_MAX;
+    const size_t rows = nh / nkvh * seq;
+    if (rows > 64 || att > 0x7fffffffu) return SIZE_MAX;
+    const size_t nchunk = (att + chunk - 1) / chunk, rp = rows <= 16 ? 16 : rows <= 32 ? 32 : 64;
+    return nchunk == 1 ? 0 : nkvh * nchunk * rp * (dh + 2) * sizeof(float);
+}
+
 // Operator::scheme (attention/operator.rs:46-141)
 size_t attention_scheme(ophip_attention *op, const ophip_attention_args &args, size_t max_ws) {
     const AttentionMeta m = attention_meta(args);
@@ -191,7 +208,14 @@ size_t attention_scheme(ophip_attention *op, const ophip_attention_args &args, s
     const ophip_rearrange_args re{args.o_layout, nullptr, args.q_layout, nullptr};
     sub(ophip_rearrange_scheme(op->rearrange, &re, rest, &need));
     wc.push_sub(need);
-    return wc.calculate(max_ws);
+    size_t ans = wc.calculate(max_ws);
+    // a launch of these sizes may run on the decode kernel instead: a workspace that serves either
+    if (op->one_pass && !is_dyn(m.nkvh)) {
+        const size_t fused = one_pass_workspace(m.dt, m.nh, m.nkvh, m.seq, m.att, m.dh,
+                                                decode_chunk(m.nkvh, m.att, (unsigned)op->dev->props.multiProcessorCount, op->force_chunk));
+        if (fused != SIZE_MAX && fused <= max_ws) ans = std::max(ans, fused);
+    }
+    return ans;
 }
 
 // The one-pass kernel (attention_prefill.hip) when it serves this call; false, with nothing done, otherwise.
@@ -205,14 +229,15 @@ bool attention_one_pass(const ophip_attention *op, const ophip_attention_args &a
     if (args.mask == OPHIP_MASK_CAUSAL && att < seq) return false;  // rows that keep no column: the softmax of the composite refuses them
     // A workgroup walks its keys tile after tile (two tiles of 64 per 2.7 us in the eight-wave build at dh 128), so with
     // fewer workgroups than CUs the longest walk is the kernel's time, while the composite pays five launches and
-    // four passes over the score matrix (about 20 us + 1 us per MB of it).  Measured, 32 heads, dh 128, causal, one
+    // four passes over the score matrix (about 24 us + 1.25 us per MB of it: 32 heads of 256 x 4096 108 us, where the
+    // eight-wave build takes 88; 8 heads 40 us against 81).  Measured, 32 heads, dh 128, causal, one
     // pass against composite: 16 rows x 2048 keys 42 / 21 us, 128 x 2048 47 / 41, 64 x 64 7 / 16, 256 x 256 13 / 23,
     // 512 x 512 19 / 35, 2048 x 2048 68 / 326.
     const size_t cus = (size_t)op->dev->props.multiProcessorCount;
     const size_t wgs = nh * ((seq + 127) / 128), tiles = (att + 63) / 64;
     if (op->fused < 0 && wgs <= cus) {
         const double walk = 4.0 + (double)((tiles + 1) / 2) * (dh == 128 ? 2.7 : 1.6);
-        const double composite = 20.0 + (double)nh * (double)seq * (double)att * 2.0 / 1e6;
+        const double composite = 24.0 + 1.25 * (double)nh * (double)seq * (double)att * 2.0 / 1e6;
         if (walk >= composite) return false;
     }
     struct View {
@@ -274,23 +299,6 @@ bool attention_one_pass(const ophip_attention *op, const ophip_attention_args &a
     const bool split = op->key_split >= 0 ? op->key_split != 0 : wgs <= cus || (p.causal && wgs <= 2 * cus);
     launch(op->prefill[m.dt == OPHIP_DT_BF16 ? 1 : 0][dh == 64 ? 0 : 1][split], Dim3{(unsigned)nh, p.nblocks}, Dim3{split ? 512u : 256u}, 0, stream_of(qa), p);
     return true;
-}
-
-// Keys per workgroup of the one-pass kernel: 256, or 128 when that leaves CUs without a workgroup (measured: the
-// decode layer, 32 kv heads x 2048 keys, 15.5 us with 256 keys against 17.0; 8 kv heads x 4096 keys 12.3 against 10.7).
-size_t decode_chunk(size_t nkvh, size_t att, unsigned cus, int force) {
-    if (force == 256 || force == 128) return (size_t)force;
-    return (att + 255) / 256 * nkvh < (size_t)cus ? 128 : 256;
-}
-
-// Workspace of the one-pass kernel for these sizes, or SIZE_MAX when it does not serve them (the shapes alone
-// decide here; launch also looks at strides and alignment).
-size_t one_pass_workspace(uint64_t dt, size_t nh, size_t nkvh, size_t seq, size_t att, size_t dh, size_t chunk) {
-    if ((dt != OPHIP_DT_F16 && dt != OPHIP_DT_BF16) || (dh != 64 && dh != 128) || nkvh == 0 || nh % nkvh != 0 || seq == 0 || att == 0) return SIZE_MAX;
-    const size_t rows = nh / nkvh * seq;
-    if (rows > 64 || att > 0x7fffffffu) return SIZE_MAX;
-    const size_t nchunk = (att + chunk - 1) / chunk, rp = rows <= 16 ? 16 : rows <= 32 ? 32 : 64;
-    return nchunk == 1 ? 0 : nkvh * nchunk * rp * (dh + 2) * sizeof(float);
 }
 
 // One call of the one-pass decode kernel (attention_decode.hip): q against the first `pos` rows of the caches followed by
