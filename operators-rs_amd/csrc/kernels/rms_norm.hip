@@ -147,9 +147,10 @@ __device__ __forceinline__ void rms_norm_scalar(const RmsNormParams &p) {
 // fixed number of waves.  w is converted once and stays in registers for all rows
 // of the wave; the next row's x is already in flight while the current one is reduced
 // and written, so each wave keeps reads and writes streaming.
-template <typename TA, typename TW>
+// CACHE: 16-byte vectors per lane and row: 8 (rows of up to 4096 elements) or 16 (up to 8192: twice the registers, half
+// the waves per CU; two-byte weights only).
+template <typename TA, typename TW, int CACHE = 8>
 __device__ __forceinline__ void rms_norm_rows(const RmsNormParams &p) {
-    constexpr int CACHE = 8;
     const uint32_t lane = threadIdx.x % WAVE;
     const uint32_t waves = gridDim.x * (WG_THREADS / WAVE);
     uint32_t row = blockIdx.x * (WG_THREADS / WAVE) + threadIdx.x / WAVE;
@@ -231,6 +232,8 @@ extern "C" __global__ void __launch_bounds__(256) rms_norm_f16_f16_rows(RmsNormP
 extern "C" __global__ void __launch_bounds__(256) rms_norm_f16_f32_rows(RmsNormParams p) { rms_norm_rows<f16, float>(p); }
 extern "C" __global__ void __launch_bounds__(256) rms_norm_bf16_bf16_rows(RmsNormParams p) { rms_norm_rows<bf16, bf16>(p); }
 extern "C" __global__ void __launch_bounds__(256) rms_norm_bf16_f32_rows(RmsNormParams p) { rms_norm_rows<bf16, float>(p); }
+extern "C" __global__ void __launch_bounds__(256) rms_norm_f16_f16_rows16(RmsNormParams p) { rms_norm_rows<f16, f16, 16>(p); }
+extern "C" __global__ void __launch_bounds__(256) rms_norm_bf16_bf16_rows16(RmsNormParams p) { rms_norm_rows<bf16, bf16, 16>(p); }
 
 #define RMS_VEC(NAME, TA, TW, G)                                                        \
     extern "C" __global__ void __launch_bounds__((G) < 256 ? 256 : (G)) NAME(RmsNormParams p) { \

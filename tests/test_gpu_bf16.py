@@ -48,7 +48,7 @@ def one_step(ref):
 
 
 @pytest.mark.parametrize("wdt", ["bf16", "f32"])
-@pytest.mark.parametrize("n,d", [(64, 4096), (16, 4096), (3, 1001), (5, 24), (300, 512), (2, 16384), (20000, 2048), (1, 8)])
+@pytest.mark.parametrize("n,d", [(64, 4096), (16, 4096), (3, 1001), (5, 24), (300, 512), (2, 16384), (20000, 2048), (1, 8), (8200, 5120)])
 def test_rms_norm_bf16(gpu, stream, n, d, wdt):
     rng = np.random.default_rng(n + d)
     xb = to_bf16(rng.standard_normal((n, d)).astype(f32))
