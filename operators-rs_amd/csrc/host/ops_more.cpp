@@ -131,6 +131,11 @@ extern "C" int ophip_layer_norm_launch(const ophip_layer_norm *op, const ophip_l
             launch(op->dev->kernel("layer_norm", (base + "_rows").c_str()), Dim3{cus * 4}, Dim3{256}, 0, stream_of(qa), p);
             return;
         }
+        if (unit == 2 && d > 4096 && d <= 8192 && n >= (size_t)cus * 32 && n * d * (size_t)unit >= ((size_t)32 << 20)) {
+            // the same for rows of 4097 .. 8192 elements: 16 vectors per lane, 64 KiB of LDS, two workgroups per CU
+            launch(op->dev->kernel("layer_norm", (base + "_rows16").c_str()), Dim3{cus * 2}, Dim3{256}, 0, stream_of(qa), p);
+            return;
+        }
         const unsigned block = G < 256 ? 256 : G, rpb = block / G;
         const std::string name = base + (G == 64 ? "_g64" : G == 256 ? "_g256" : "_g1024");
         launch(op->dev->kernel("layer_norm", name.c_str()), Dim3{ceil_div(n, rpb)}, Dim3{block}, 0, stream_of(qa), p);

@@ -131,9 +131,11 @@ __device__ __forceinline__ void layer_norm_scalar(const LayerNormParams &p) {
 // once into LDS, then each of its waves streams rows (dealt round-robin over all waves of the
 // grid) with the next row's loads in flight while the current one is reduced and written.
 // Per row the only global traffic left is x in and y out.
-template <typename TA, typename TW>
+// CACHE: 16-byte vectors per lane and row: 8 (d <= 4096) or 16 (d <= 8192: 64 KiB of LDS for scale and bias, two
+// workgroups per CU).
+template <typename TA, typename TW, int CACHE = 8>
 __device__ __forceinline__ void layer_norm_rows(const LayerNormParams &p) {
-    constexpr int CACHE = 8, MAXD = 4096;
+    constexpr int MAXD = CACHE * WAVE * 8;
     __shared__ float s_scale[MAXD], s_bias[MAXD];
     for (uint32_t j = threadIdx.x; j < p.d; j += WG_THREADS) {
         s_scale[j] = (float)reinterpret_cast<const TW *>(p.scale)[j];
@@ -204,6 +206,10 @@ extern "C" __global__ void __launch_bounds__(256) layer_norm_f16_f16_rows(LayerN
 extern "C" __global__ void __launch_bounds__(256) layer_norm_f16_f32_rows(LayerNormParams p) { layer_norm_rows<f16, float>(p); }
 extern "C" __global__ void __launch_bounds__(256) layer_norm_bf16_bf16_rows(LayerNormParams p) { layer_norm_rows<bf16, bf16>(p); }
 extern "C" __global__ void __launch_bounds__(256) layer_norm_bf16_f32_rows(LayerNormParams p) { layer_norm_rows<bf16, float>(p); }
+extern "C" __global__ void __launch_bounds__(256) layer_norm_f16_f16_rows16(LayerNormParams p) { layer_norm_rows<f16, f16, 16>(p); }
+extern "C" __global__ void __launch_bounds__(256) layer_norm_f16_f32_rows16(LayerNormParams p) { layer_norm_rows<f16, float, 16>(p); }
+extern "C" __global__ void __launch_bounds__(256) layer_norm_bf16_bf16_rows16(LayerNormParams p) { layer_norm_rows<bf16, bf16, 16>(p); }
+extern "C" __global__ void __launch_bounds__(256) layer_norm_bf16_f32_rows16(LayerNormParams p) { layer_norm_rows<bf16, float, 16>(p); }
 
 #define LAYER_NORM(NAME, TA, TW)                                                                                  \
     extern "C" __global__ void __launch_bounds__(256) layer_norm_##NAME##_g64(LayerNormParams p) {                \

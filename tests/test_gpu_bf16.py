@@ -92,7 +92,7 @@ def test_rms_norm_bf16_strided_rows_and_scalar_path(gpu, stream):
 
 
 @pytest.mark.parametrize("wdt", ["bf16", "f32"])
-@pytest.mark.parametrize("n,d", [(64, 4096), (3, 1001), (300, 512), (2, 16384), (20000, 1024)])
+@pytest.mark.parametrize("n,d", [(64, 4096), (3, 1001), (300, 512), (2, 16384), (20000, 1024), (8200, 5120)])
 def test_layer_norm_bf16(gpu, stream, n, d, wdt):
     rng = np.random.default_rng(n * 7 + d)
     xb = to_bf16(rng.standard_normal((n, d)).astype(f32) * f32(1.5) + f32(0.25))
