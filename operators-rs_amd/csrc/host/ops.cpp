@@ -62,6 +62,7 @@ struct RmsKeyHash {
 struct RmsScheme {  // kernels for one (dt_a, dt_w, d): a vector variant per group width plus the scalar one
     hipFunction_t g64, g256, g1024, scalar;
     hipFunction_t rows;  // f16 and bf16 activations only: one wave per row over many rows
+    hipFunction_t rows_short[3] = {};  // the same, 8 / 4 / 2 rows of up to 512 / 1024 / 2048 elements per wave and trip
     hipFunction_t rows16 = nullptr;  // the same for rows of up to 8192 elements (activations and weights of one two-byte type)
 };
 
@@ -83,6 +84,8 @@ struct ophip_rms_norm : OpBase {
             s.scalar = dev->kernel("rms_norm", (base + "_scalar").c_str());
             s.rows = key.dt_a == OPHIP_DT_F16 || key.dt_a == OPHIP_DT_BF16 ? dev->kernel("rms_norm", (base + "_rows").c_str()) : nullptr;
             if (s.rows && key.dt_w == key.dt_a) s.rows16 = dev->kernel("rms_norm", (base + "_rows16").c_str());
+            if (s.rows)
+                for (int i = 0; i < 3; ++i) s.rows_short[i] = dev->kernel("rms_norm", (base + "_rows_s" + std::to_string(1 << i)).c_str());
             return s;
         });
     }
@@ -151,7 +154,8 @@ extern "C" int ophip_rms_norm_launch(const ophip_rms_norm *op, const ophip_rms_n
             // enough rows for several per wave: as many waves as stay resident (registers allow
             // 16 per CU with two-byte weights, 12 with f32), each streaming rows with w held in registers
             const unsigned per_cu = m.dt_w == OPHIP_DT_F32 ? 3 : 4;
-            launch(s.rows, Dim3{cus * per_cu}, Dim3{256}, 0, stream_of(qa), p);
+            hipFunction_t fn = nvec <= 64 ? s.rows_short[0] : nvec <= 128 ? s.rows_short[1] : nvec <= 256 ? s.rows_short[2] : s.rows;
+            launch(fn, Dim3{cus * per_cu}, Dim3{256}, 0, stream_of(qa), p);
             return;
         }
         // rows of 4097 .. 8192 two-byte elements, many of them: the same with 16 vectors per lane (a workgroup per row

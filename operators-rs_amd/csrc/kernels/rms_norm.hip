@@ -149,11 +149,15 @@ __device__ __forceinline__ void rms_norm_scalar(const RmsNormParams &p) {
 // and written, so each wave keeps reads and writes streaming.
 // CACHE: 16-byte vectors per lane and row: 8 (rows of up to 4096 elements) or 16 (up to 8192: twice the registers, half
 // the waves per CU; two-byte weights only).
-template <typename TA, typename TW, int CACHE = 8>
+// S: vectors per lane one row takes (d <= 512 S elements); a wave takes CACHE / S consecutive rows per trip, all their
+// loads in flight together: a wave on one 1 KB row at a time leaves the memory system idle
+// ([524288, 512]: 52 % of 8 TB/s with one row per trip).
+template <typename TA, typename TW, int CACHE = 8, int S = CACHE>
 __device__ __forceinline__ void rms_norm_rows(const RmsNormParams &p) {
+    constexpr int R = CACHE / S;  // rows per trip
     const uint32_t lane = threadIdx.x % WAVE;
     const uint32_t waves = gridDim.x * (WG_THREADS / WAVE);
-    uint32_t row = blockIdx.x * (WG_THREADS / WAVE) + threadIdx.x / WAVE;
+    uint32_t row = (blockIdx.x * (WG_THREADS / WAVE) + threadIdx.x / WAVE) * R;  // first row of the trip
     const uint32_t nvec = p.d / 8;
     if (row >= p.n) return;
 
@@ -169,9 +173,9 @@ __device__ __forceinline__ void rms_norm_rows(const RmsNormParams &p) {
                 return __uint_as_float(raw[i / 4][i % 4]);
             }
         }
-    } w[CACHE];
+    } w[S];
 #pragma unroll
-    for (int c = 0; c < CACHE; ++c) {
+    for (int c = 0; c < S; ++c) {
         const uint32_t v = lane + c * WAVE;
         if (v < nvec) {
 #pragma unroll
@@ -179,48 +183,49 @@ __device__ __forceinline__ void rms_norm_rows(const RmsNormParams &p) {
                 w[c].raw[q] = ld128(reinterpret_cast<const char *>(p.w) + ((size_t)v * 8 * sizeof(TW)) + 16 * q);
         }
     }
+    // slot c of the trip: row c / S of it, vector lane + (c % S) * 64 of that row
     PackOf<TA> cur[CACHE], nxt[CACHE];
-    {
-        const char *xr = reinterpret_cast<const char *>(p.x) + (int64_t)row * p.nsx;
+    auto request = [&](PackOf<TA>(&buf)[CACHE], uint32_t first) {
 #pragma unroll
         for (int c = 0; c < CACHE; ++c) {
-            const uint32_t v = lane + c * WAVE;
-            if (v < nvec) cur[c].u = ld128_nt(xr + (size_t)v * 16);
+            const uint32_t v = lane + (c % S) * WAVE, r = first + c / S;
+            if (v < nvec && r < p.n) buf[c].u = ld128_nt(reinterpret_cast<const char *>(p.x) + (int64_t)r * p.nsx + (size_t)v * 16);
         }
-    }
-    for (; row < p.n; row += waves) {
-        const uint32_t next = row + waves;
-        if (next < p.n) {
-            const char *xn = reinterpret_cast<const char *>(p.x) + (int64_t)next * p.nsx;
+    };
+    request(cur, row);
+    for (; row < p.n; row += waves * R) {
+        if (row + waves * R < p.n) request(nxt, row + waves * R);
+        float ss[R];
 #pragma unroll
-            for (int c = 0; c < CACHE; ++c) {
-                const uint32_t v = lane + c * WAVE;
-                if (v < nvec) nxt[c].u = ld128_nt(xn + (size_t)v * 16);
-            }
-        }
-        float ss = 0.f;
+        for (int rr = 0; rr < R; ++rr) {
+            ss[rr] = 0.f;
 #pragma unroll
-        for (int c = 0; c < CACHE; ++c) {
-            const uint32_t v = lane + c * WAVE;
-            if (v < nvec) {
+            for (int c = rr * S; c < (rr + 1) * S; ++c) {
+                if (lane + (c % S) * WAVE < nvec) {
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const float f = (float)cur[c].e[i];
-                    ss += f * f;
+                    for (int i = 0; i < 8; ++i) {
+                        const float f = (float)cur[c].e[i];
+                        ss[rr] += f * f;
+                    }
                 }
             }
         }
-        ss = wave_sum_dpp(ss);
-        const float k = 1.0f / sqrtf(ss / (float)p.d + p.epsilon);
-        char *yr = reinterpret_cast<char *>(p.y) + (int64_t)row * p.nsy;
 #pragma unroll
-        for (int c = 0; c < CACHE; ++c) {
-            const uint32_t v = lane + c * WAVE;
-            if (v < nvec) {
-                PackOf<TA> o;
+        for (int rr = 0; rr < R; ++rr) ss[rr] = wave_sum_dpp(ss[rr]);
 #pragma unroll
-                for (int i = 0; i < 8; ++i) o.e[i] = (TA)((k * w[c].get(i)) * (float)cur[c].e[i]);
-                st128_nt(yr + (size_t)v * 16, o.u);
+        for (int rr = 0; rr < R; ++rr) {
+            if (row + rr >= p.n) break;  // wave-uniform
+            const float k = 1.0f / sqrtf(ss[rr] / (float)p.d + p.epsilon);
+            char *yr = reinterpret_cast<char *>(p.y) + (int64_t)(row + rr) * p.nsy;
+#pragma unroll
+            for (int c = rr * S; c < (rr + 1) * S; ++c) {
+                const uint32_t v = lane + (c % S) * WAVE;
+                if (v < nvec) {
+                    PackOf<TA> o;
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) o.e[i] = (TA)((k * w[c % S].get(i)) * (float)cur[c].e[i]);
+                    st128_nt(yr + (size_t)v * 16, o.u);
+                }
             }
         }
 #pragma unroll
@@ -232,6 +237,14 @@ extern "C" __global__ void __launch_bounds__(256) rms_norm_f16_f16_rows(RmsNormP
 extern "C" __global__ void __launch_bounds__(256) rms_norm_f16_f32_rows(RmsNormParams p) { rms_norm_rows<f16, float>(p); }
 extern "C" __global__ void __launch_bounds__(256) rms_norm_bf16_bf16_rows(RmsNormParams p) { rms_norm_rows<bf16, bf16>(p); }
 extern "C" __global__ void __launch_bounds__(256) rms_norm_bf16_f32_rows(RmsNormParams p) { rms_norm_rows<bf16, float>(p); }
+#define RMS_ROWS_SHORT(NAME, TA, TW)                                                                                          \
+    extern "C" __global__ void __launch_bounds__(256) rms_norm_##NAME##_rows_s1(RmsNormParams p) { rms_norm_rows<TA, TW, 8, 1>(p); } \
+    extern "C" __global__ void __launch_bounds__(256) rms_norm_##NAME##_rows_s2(RmsNormParams p) { rms_norm_rows<TA, TW, 8, 2>(p); } \
+    extern "C" __global__ void __launch_bounds__(256) rms_norm_##NAME##_rows_s4(RmsNormParams p) { rms_norm_rows<TA, TW, 8, 4>(p); }
+RMS_ROWS_SHORT(f16_f16, f16, f16)
+RMS_ROWS_SHORT(f16_f32, f16, float)
+RMS_ROWS_SHORT(bf16_bf16, bf16, bf16)
+RMS_ROWS_SHORT(bf16_f32, bf16, float)
 extern "C" __global__ void __launch_bounds__(256) rms_norm_f16_f16_rows16(RmsNormParams p) { rms_norm_rows<f16, f16, 16>(p); }
 extern "C" __global__ void __launch_bounds__(256) rms_norm_bf16_bf16_rows16(RmsNormParams p) { rms_norm_rows<bf16, bf16, 16>(p); }
 

@@ -85,6 +85,7 @@ def test_rms_norm_reference_sweep_f32_weights(gpu, stream, k):
                                           (7, 1000, f16, f16), (9, 4095, f16, f32), (300, 4096, f32, f32),
                                           (2, 130, f32, f32), (1, 8, f16, f16), (33, 2048, f16, f16),
                                           (20001, 1024, f16, f16), (17000, 1024, f16, f32),  # these two: one wave streaming many rows
+                                          (16500, 512, f16, f16), (16499, 768, f16, f32), (16387, 1600, f16, f16), (16390, 2048, f16, f16),  # 8 / 4 / 2 / 2 rows per trip
                                           (8200, 5120, f16, f16), (8193, 8192, f16, f16), (8200, 4104, f16, f16),  # the same, 16 vectors a lane
                                           (8200, 5120, f16, f32),  # (f32 weights: a workgroup per row)
                                           (5, 4096, np.float64, np.float64), (64, 333, np.float64, np.float64)])
