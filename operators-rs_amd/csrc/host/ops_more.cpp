@@ -128,7 +128,9 @@ extern "C" int ophip_layer_norm_launch(const ophip_layer_norm *op, const ophip_l
             n * d * (size_t)unit >= ((size_t)32 << 20)) {
             // many rows and more bytes than the L2s hold: persistent workgroups (four per CU: 32 KiB
             // of LDS each for scale and bias) whose waves stream rows
-            launch(op->dev->kernel("layer_norm", (base + "_rows").c_str()), Dim3{cus * 4}, Dim3{256}, 0, stream_of(qa), p);
+            // (8 / 4 / 2 rows of up to 512 / 1024 / 2048 elements per wave and trip)
+            const char *tail = nvec <= 64 ? "_rows_s1" : nvec <= 128 ? "_rows_s2" : nvec <= 256 ? "_rows_s4" : "_rows";
+            launch(op->dev->kernel("layer_norm", (base + tail).c_str()), Dim3{cus * 4}, Dim3{256}, 0, stream_of(qa), p);
             return;
         }
         if (unit == 2 && d > 4096 && d <= 8192 && n >= (size_t)cus * 32 && n * d * (size_t)unit >= ((size_t)32 << 20)) {

@@ -202,10 +202,94 @@ __device__ __forceinline__ void layer_norm_rows(const LayerNormParams &p) {
     }
 }
 
+// The same for rows of up to 2048 elements.  S: vectors per lane one row takes (d <= 512 S elements); a wave takes
+// CACHE / S consecutive rows per trip, all their loads in flight together ([524288, 512]: 39 % of 8 TB/s with one row
+// per trip, 67 % with eight).  (A build of its own: the general form of the loop made the one-row-per-trip kernel above
+// 14 points slower.)
+template <typename TA, typename TW, int CACHE, int S>
+__device__ __forceinline__ void layer_norm_rows_short(const LayerNormParams &p) {
+    constexpr int MAXD = S * WAVE * 8, R = CACHE / S;
+    __shared__ float s_scale[MAXD], s_bias[MAXD];
+    for (uint32_t j = threadIdx.x; j < p.d; j += WG_THREADS) {
+        s_scale[j] = (float)reinterpret_cast<const TW *>(p.scale)[j];
+        s_bias[j] = (float)reinterpret_cast<const TW *>(p.bias)[j];
+    }
+    __syncthreads();
+
+    const uint32_t lane = threadIdx.x % WAVE;
+    const uint32_t waves = gridDim.x * (WG_THREADS / WAVE);
+    uint32_t row = (blockIdx.x * (WG_THREADS / WAVE) + threadIdx.x / WAVE) * R;  // first row of the trip
+    const uint32_t nvec = p.d / 8;
+    if (row >= p.n) return;
+
+    // slot c of the trip: row c / S of it, vector lane + (c % S) * 64 of that row
+    PackOf<TA> cur[CACHE], nxt[CACHE];
+    auto request = [&](PackOf<TA>(&buf)[CACHE], uint32_t first) {
+#pragma unroll
+        for (int c = 0; c < CACHE; ++c) {
+            const uint32_t v = lane + (c % S) * WAVE, r = first + c / S;
+            if (v < nvec && r < p.n) buf[c].u = ld128_nt(reinterpret_cast<const char *>(p.x) + (int64_t)r * p.nsx + (size_t)v * 16);
+        }
+    };
+    request(cur, row);
+    for (; row < p.n; row += waves * R) {
+        if (row + waves * R < p.n) request(nxt, row + waves * R);
+        float s1[R], s2[R];
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) {
+            s1[rr] = 0.f, s2[rr] = 0.f;
+#pragma unroll
+            for (int c = rr * S; c < (rr + 1) * S; ++c) {
+                if (lane + (c % S) * WAVE < nvec) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        const float f = (float)cur[c].e[i];
+                        s1[rr] += f;
+                        s2[rr] += f * f;
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) {
+            s1[rr] = wave_sum_dpp(s1[rr]);
+            s2[rr] = wave_sum_dpp(s2[rr]);
+        }
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) {
+            if (row + rr >= p.n) break;  // wave-uniform
+            float e, k;
+            mean_and_scale(s1[rr], s2[rr], p.d, p.epsilon, e, k);
+            char *yr = reinterpret_cast<char *>(p.y) + (int64_t)(row + rr) * p.nsy;
+#pragma unroll
+            for (int c = rr * S; c < (rr + 1) * S; ++c) {
+                const uint32_t v = lane + (c % S) * WAVE;
+                if (v < nvec) {
+                    PackOf<TA> o;
+#pragma unroll
+                    for (int i = 0; i < 8; ++i)
+                        o.e[i] = (TA)__builtin_fmaf((float)cur[c].e[i] - e, s_scale[v * 8 + i] * k, s_bias[v * 8 + i]);
+                    st128_nt(yr + (size_t)v * 16, o.u);
+                }
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < CACHE; ++c) cur[c] = nxt[c];
+    }
+}
+
 extern "C" __global__ void __launch_bounds__(256) layer_norm_f16_f16_rows(LayerNormParams p) { layer_norm_rows<f16, f16>(p); }
 extern "C" __global__ void __launch_bounds__(256) layer_norm_f16_f32_rows(LayerNormParams p) { layer_norm_rows<f16, float>(p); }
 extern "C" __global__ void __launch_bounds__(256) layer_norm_bf16_bf16_rows(LayerNormParams p) { layer_norm_rows<bf16, bf16>(p); }
 extern "C" __global__ void __launch_bounds__(256) layer_norm_bf16_f32_rows(LayerNormParams p) { layer_norm_rows<bf16, float>(p); }
+#define LAYER_NORM_ROWS_SHORT(NAME, TA, TW)                                                                                             \
+    extern "C" __global__ void __launch_bounds__(256) layer_norm_##NAME##_rows_s1(LayerNormParams p) { layer_norm_rows_short<TA, TW, 8, 1>(p); } \
+    extern "C" __global__ void __launch_bounds__(256) layer_norm_##NAME##_rows_s2(LayerNormParams p) { layer_norm_rows_short<TA, TW, 8, 2>(p); } \
+    extern "C" __global__ void __launch_bounds__(256) layer_norm_##NAME##_rows_s4(LayerNormParams p) { layer_norm_rows_short<TA, TW, 8, 4>(p); }
+LAYER_NORM_ROWS_SHORT(f16_f16, f16, f16)
+LAYER_NORM_ROWS_SHORT(f16_f32, f16, float)
+LAYER_NORM_ROWS_SHORT(bf16_bf16, bf16, bf16)
+LAYER_NORM_ROWS_SHORT(bf16_f32, bf16, float)
 extern "C" __global__ void __launch_bounds__(256) layer_norm_f16_f16_rows16(LayerNormParams p) { layer_norm_rows<f16, f16, 16>(p); }
 extern "C" __global__ void __launch_bounds__(256) layer_norm_f16_f32_rows16(LayerNormParams p) { layer_norm_rows<f16, float, 16>(p); }
 extern "C" __global__ void __launch_bounds__(256) layer_norm_bf16_bf16_rows16(LayerNormParams p) { layer_norm_rows<bf16, bf16, 16>(p); }

@@ -41,6 +41,7 @@ def view(buf_u8, dtype, shape, strides, offset=0):
 
 @pytest.mark.parametrize("n,d,adt,wdt", [(4, 256, f16, f32), (4, 8192, f16, f32), (64, 4096, f16, f16),
                                          (8200, 5120, f16, f16), (8193, 8192, f16, f32),  # many rows beyond 4096 elements: 16 vectors a lane
+                                         (32772, 512, f16, f16), (22003, 768, f16, f32), (16387, 1600, f16, f16), (16390, 2048, f16, f16),  # 8 / 4 / 2 / 2 rows per trip
                                          (3, 16384, f16, f16), (5, 80000, f16, f32), (7, 1001, f16, f16),
                                          (300, 768, f32, f32), (2, 130, f32, f32), (5000, 1024, f16, f16),
                                          (20001, 1024, f16, f16), (17000, 1024, f16, f32)])  # the last two: rows streamed by persistent waves
