@@ -195,7 +195,7 @@ static RopeMeta rope_meta(const ophip_rope_args &a) {
 }
 
 struct ophip_rope : OpBase {
-    hipFunction_t f16_vec, f16_pairs, bf16_vec, bf16_pairs, f32_pairs, f64_pairs;
+    hipFunction_t f16_vec, f16_pairs, bf16_vec, bf16_pairs, f32_pairs, f64_pairs, f16_vec_multi, bf16_vec_multi;
     // theta^(k / (dh/2)) of the last (theta, dh) launched: a model has one such pair
     mutable std::mutex den_mu;
     mutable float den_theta = 0.f;
@@ -212,6 +212,8 @@ struct ophip_rope : OpBase {
     }
     explicit ophip_rope(ophip_device *d) : OpBase(d) {
         f16_vec = d->kernel("rope", "rope_f16_vec");
+        f16_vec_multi = d->kernel("rope", "rope_f16_vec_multi");
+        bf16_vec_multi = d->kernel("rope", "rope_bf16_vec_multi");
         f16_pairs = d->kernel("rope", "rope_f16_pairs");
         bf16_vec = d->kernel("rope", "rope_bf16_vec");
         bf16_pairs = d->kernel("rope", "rope_bf16_pairs");
@@ -285,6 +287,16 @@ extern "C" int ophip_rope_launch(const ophip_rope *op, const ophip_rope_args *ar
                            : m.dt_t == OPHIP_DT_F32  ? op->f32_pairs
                                                      : op->f64_pairs;
         op->dev->make_current();
+        // many tokens of few vectors each (8 heads of 128, 16 of 64: 128 vectors; twice that up to 64 K tokens): several
+        // consecutive tokens per workgroup, about 1024 vectors.  [204800, 8, 128] 49 -> 70 % of 8 TB/s, [8192, 16, 128]
+        // 71 -> 79 %; tokens of 512 vectors gain nothing, and beyond 64 K tokens those of 256 lose 4 points.
+        const size_t per_token = nh * (dh / 8), tpb = per_token ? std::min<size_t>(8, 1024 / std::max<size_t>(per_token, 1)) : 0;
+        if (vec && by == 1 && nt >= 4096 && (tpb == 8 || (tpb >= 4 && nt < 65536))) {
+            p.tokens_per_block = (uint32_t)tpb;
+            launch(m.dt_t == OPHIP_DT_F16 ? op->f16_vec_multi : op->bf16_vec_multi, Dim3{(unsigned)((nt + tpb - 1) / tpb)}, Dim3{256}, smem * tpb,
+                   stream_of(qa), p);
+            return;
+        }
         launch(fn, Dim3{(unsigned)nt, (unsigned)by}, Dim3{256}, smem, stream_of(qa), p);
     });
 }

@@ -38,6 +38,7 @@ struct RopeParams {
     float theta;
     uint32_t pos_is_u64;
     uint32_t heads_per_block;
+    uint32_t tokens_per_block;  // the `_multi` kernels: consecutive tokens a workgroup takes
     // theta^(k / (dh/2)) for k < dh/2, evaluated by the host's powf (what the reference's CPU backend divides by) when
     // dh <= 256; has_den = 0: the kernel evaluates powf itself
     uint32_t has_den;

@@ -63,6 +63,48 @@ __device__ __forceinline__ void rope_vec(const RopeParams &p) {  // T: f16 or bf
         st128(ptr, o.u);
     }
 }
+// Many tokens: a workgroup takes tokens_per_block consecutive ones (about 1024 vectors), one table per token, every
+// entry's sine and cosine from one evaluation (sincosf: one range reduction for both) spread over all 256 threads; with a
+// token per workgroup half the threads idle through the table and a token of 8 heads gives the other half one vector
+// each.
+template <typename T>
+__device__ __forceinline__ void rope_vec_multi(const RopeParams &p) {  // T: f16 or bf16
+    const uint32_t H = p.dh / 2, cpv = p.dh / 8, per_token = p.nh * cpv;
+    const uint32_t t0 = blockIdx.x * p.tokens_per_block, tokens = min(p.tokens_per_block, p.nt - t0);
+    const uint32_t total = tokens * per_token;
+    auto chunk = [&](uint32_t v) {
+        const uint32_t tt = v / per_token, r = v - tt * per_token;
+        return reinterpret_cast<char *>(p.t) + (int64_t)(t0 + tt) * p.st + (int64_t)(r / cpv) * p.sh + (size_t)(r % cpv) * 16;
+    };
+    PackOf<T> first;
+    first.u = u32x4{0, 0, 0, 0};
+    if (threadIdx.x < total) first.u = ld128(chunk(threadIdx.x));
+    for (uint32_t e = threadIdx.x; e < tokens * H; e += WG_THREADS) {
+        const uint32_t tt = e / H, k = e - tt * H;
+        const float ang = rope_pos(p, t0 + tt) / (p.has_den ? p.den[k] : powf(p.theta, (float)k / (float)H));
+        float sn, cs;
+        sincosf(ang, &sn, &cs);
+        rope_sc[e] = float2{sn, cs};
+    }
+    __syncthreads();
+    for (uint32_t v = threadIdx.x; v < total; v += WG_THREADS) {
+        const uint32_t tt = v / per_token, c = (v - tt * per_token) % cpv;
+        char *ptr = chunk(v);
+        PackOf<T> x, o;
+        if (v == threadIdx.x) x.u = first.u;
+        else x.u = ld128(ptr);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float2 sc = rope_sc[tt * H + 4 * c + i];
+            const float a = (float)x.e[2 * i], b = (float)x.e[2 * i + 1];
+            o.e[2 * i] = (T)(a * sc.y - b * sc.x);
+            o.e[2 * i + 1] = (T)(a * sc.x + b * sc.y);
+        }
+        st128(ptr, o.u);
+    }
+}
+extern "C" __global__ void __launch_bounds__(256) rope_f16_vec_multi(RopeParams p) { rope_vec_multi<f16>(p); }
+extern "C" __global__ void __launch_bounds__(256) rope_bf16_vec_multi(RopeParams p) { rope_vec_multi<bf16>(p); }
 extern "C" __global__ void __launch_bounds__(256) rope_f16_vec(RopeParams p) { rope_vec<f16>(p); }
 // bf16: neither backend of the reference has it for this operator; the f16 kernels on bf16 elements (f32 inside, one rounding)
 extern "C" __global__ void __launch_bounds__(256) rope_bf16_vec(RopeParams p) { rope_vec<bf16>(p); }

@@ -190,7 +190,7 @@ def test_swiglu_and_gelu_bf16(gpu, stream, n, d):
 
 
 @pytest.mark.parametrize("pdt", [np.uint32, np.uint64])
-@pytest.mark.parametrize("shape", [(16, 64, 128), (7, 3, 64), (5, 4, 20), (512, 32, 128)])
+@pytest.mark.parametrize("shape", [(16, 64, 128), (7, 3, 64), (5, 4, 20), (512, 32, 128), (4099, 8, 128)])
 def test_rope_bf16(gpu, stream, shape, pdt):
     import oracle
     rng = np.random.default_rng(sum(shape))

@@ -207,7 +207,8 @@ def test_rope_reference_shape(gpu, stream, pdt):
 
 
 @pytest.mark.parametrize("shape,dtype", [((16, 32, 128), f16), ((3, 5, 20), f16), ((2, 1, 2), f16),
-                                         ((5, 7, 64), f32), ((1, 40, 256), f16), ((100, 8, 96), f16)])
+                                         ((5, 7, 64), f32), ((1, 40, 256), f16), ((100, 8, 96), f16),
+                                         ((4099, 8, 128), f16), ((4101, 16, 128), f16), ((4097, 16, 64), f16)])  # several tokens per workgroup
 def test_rope_shapes(gpu, stream, shape, dtype):
     rng = np.random.default_rng(sum(shape))
     t = rng.standard_normal(shape).astype(f32).astype(dtype)
