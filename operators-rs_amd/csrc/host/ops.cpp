@@ -583,6 +583,21 @@ extern "C" int ophip_rearrange_launch(const ophip_rearrange *op, const ophip_rea
         if (s.unit == 0 || s.count() == 0) return;
         op->dev->make_current();
         if (s.ndim() == 0) {  // one contiguous run: a device-to-device copy (rearrange/cuda/mod.rs:64-70)
+            // beyond the caches, in whole aligned 16-byte chunks: the copy kernel with non-temporal loads and stores
+            // (512 MiB: 79 % of 8 TB/s against the runtime's copy at 67 %)
+            const size_t chunks = s.unit / 16;
+            if (s.unit >= ((size_t)64 << 20) && s.unit % 16 == 0 && chunks <= 0x7fffffffu && aligned16(args->dst_base) &&
+                aligned16(args->src_base)) {
+                RearrangeParams p{};
+                p.dst = args->dst_base;
+                p.src = args->src_base;
+                p.total = chunks;
+                p.ndim = 0;
+                p.chunks_per_unit = (uint32_t)chunks;
+                p.cpu_div = make_fastdiv((uint32_t)chunks);
+                launch(op->k32_nt[0], Dim3{ceil_div(chunks, 256 * 4)}, Dim3{256}, 0, stream_of(qa), p);
+                return;
+            }
             check_hip(hipMemcpyAsync(args->dst_base, args->src_base, s.unit, hipMemcpyDeviceToDevice, stream_of(qa)),
                       "hipMemcpyAsync");
             return;

@@ -1408,3 +1408,20 @@ def test_one_operator_instance_launched_from_several_threads(gpu):
     for t in threads:
         t.join()
     assert not errors, errors
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("nbytes,off", [((64 << 20) + 4096, 0), ((64 << 20) + 16, 32), ((64 << 20) + 24, 0), ((70 << 20), 8)])
+def test_rearrange_large_contiguous_run_is_bit_exact(gpu, stream, nbytes, off):
+    """One contiguous run beyond 64 MiB: the copy kernel when bases and length are whole 16-byte chunks, the runtime's
+    device-to-device copy otherwise; every byte, and nothing outside the run."""
+    rng = np.random.default_rng(nbytes % 1000 + off)
+    src = rng.integers(0, 256, nbytes + 64, dtype=np.uint8)
+    sd, dd = gpu.from_host(src), gpu.malloc(nbytes + 128)
+    gpu.memset(dd, 0xEE)
+    lay = TensorLayout(dt.U8, [nbytes], [1])
+    say("rearrange contiguous %d bytes, offset %d" % (nbytes, off))
+    ophip.Rearrange(gpu).launch(ophip.RearrangeArgs(lay, dd.ptr + off, lay, sd.ptr + off), None, stream)
+    out = gpu.to_host(dd, np.uint8, nbytes + 128, stream=stream)
+    assert np.array_equal(out[off:off + nbytes], src[off:off + nbytes])
+    assert (out[:off] == 0xEE).all() and (out[off + nbytes:] == 0xEE).all()
