@@ -550,6 +550,7 @@ extern "C" int ophip_rearrange_plan(const ophip_rearrange_args *args, ptrdiff_t 
 
 struct ophip_rearrange : OpBase {
     hipFunction_t k32[5], k32_nt[5], k32_one[5], k64[5];  // chunk sizes 16, 8, 4, 2, 1; k32_one: one chunk per thread; k32_nt: non-temporal stores
+    hipFunction_t transpose[3];  // units of 2, 4, 8 bytes turned in LDS tiles
     explicit ophip_rearrange(ophip_device *d) : OpBase(d) {
         static const int sizes[5] = {16, 8, 4, 2, 1};
         for (int i = 0; i < 5; ++i) {
@@ -557,6 +558,7 @@ struct ophip_rearrange : OpBase {
             k32_one[i] = d->kernel("rearrange", ("rearrange1_b" + std::to_string(sizes[i])).c_str());
             k32_nt[i] = d->kernel("rearrange", ("rearrange_nt_b" + std::to_string(sizes[i])).c_str());
             k64[i] = d->kernel("rearrange", ("rearrange64_b" + std::to_string(sizes[i])).c_str());
+            if (i < 3) transpose[i] = d->kernel("rearrange", ("rearrange_transpose_b" + std::to_string(2 << i)).c_str());
         }
     }
 };
@@ -605,6 +607,49 @@ extern "C" int ophip_rearrange_launch(const ophip_rearrange *op, const ophip_rea
         if (s.ndim() > OPHIP_REARRANGE_MAXD)
             throw rank_not_support("rearrange supports at most " + std::to_string(OPHIP_REARRANGE_MAXD) +
                                    " non-mergeable dimensions");
+        // A transposition of small units: the destination contiguous along its innermost dimension A, the source along
+        // another one, B, both at least 32 long: 64 x 64 tiles through LDS.
+        if ((s.unit == 2 || s.unit == 4 || s.unit == 8) && s.ndim() >= 2 && s.dst[s.ndim() - 1] == (ptrdiff_t)s.unit &&
+            reinterpret_cast<uintptr_t>(args->dst_base) % s.unit == 0 && reinterpret_cast<uintptr_t>(args->src_base) % s.unit == 0) {
+            const size_t A = s.ndim() - 1;
+            size_t Bd = A;
+            for (size_t i = 0; i < A; ++i)
+                if (s.src[i] == (ptrdiff_t)s.unit) Bd = i;
+            std::vector<size_t> len(s.ndim());
+            for (size_t i = 0; i < s.ndim(); ++i) len[i] = s.idx[i] / s.idx[i + 1];
+            bool fits = Bd != A && len[A] >= 32 && len[Bd] >= 32 && len[A] <= 0x7fffffffu && len[Bd] <= 0x7fffffffu;
+            for (size_t i = 0; i < s.ndim() && fits; ++i)
+                if (s.dst[i] % (ptrdiff_t)s.unit != 0 || s.src[i] % (ptrdiff_t)s.unit != 0) fits = false;
+            if (fits) {
+                TransposeParams t{};
+                t.dst = args->dst_base;
+                t.src = args->src_base;
+                t.len_a = (uint32_t)len[A];
+                t.len_b = (uint32_t)len[Bd];
+                t.dst_b = s.dst[Bd];
+                t.src_a = s.src[A];
+                t.tiles_a = (uint32_t)((len[A] + 63) / 64);
+                t.tiles_b = (uint32_t)((len[Bd] + 63) / 64);
+                size_t outer = 1;
+                std::vector<size_t> od;
+                for (size_t i = 0; i < s.ndim(); ++i)
+                    if (i != A && i != Bd) od.push_back(i);
+                t.nouter = (uint32_t)od.size();
+                for (size_t q = od.size(); q-- > 0;) {
+                    t.outer_div[q] = make_fastdiv((uint32_t)outer);
+                    t.outer_dst[q] = s.dst[od[q]];
+                    t.outer_src[q] = s.src[od[q]];
+                    outer *= len[od[q]];
+                }
+                const size_t tiles = (size_t)t.tiles_a * t.tiles_b;
+                if (outer <= 0x7fffffffu && tiles <= 0x7fffffffu && outer * tiles <= 0x7fffffffu) {
+                    t.tiles_div = make_fastdiv((uint32_t)tiles);
+                    t.tb_div = make_fastdiv(t.tiles_b);
+                    launch(op->transpose[s.unit == 2 ? 0 : s.unit == 4 ? 1 : 2], Dim3{(unsigned)(outer * tiles)}, Dim3{256}, 0, stream_of(qa), t);
+                    return;
+                }
+            }
+        }
         // widest chunk that divides the unit and keeps every access aligned
         uintptr_t bits = (uintptr_t)s.unit | reinterpret_cast<uintptr_t>(args->dst_base) |
                          reinterpret_cast<uintptr_t>(args->src_base);

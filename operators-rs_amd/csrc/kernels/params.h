@@ -66,6 +66,21 @@ struct RearrangeParams {
     int64_t src_s[OPHIP_REARRANGE_MAXD];     // bytes
 };
 
+// rearrange where the destination is contiguous along one dimension (A) and the source along another (B), unit 2 / 4 / 8
+// bytes: tiles of 64 x 64 units through LDS.  Workgroup ids enumerate (outer index, tile of A, tile of B).
+struct TransposeParams {
+    void *dst;
+    const void *src;
+    uint32_t len_a, len_b;        // units along A and B
+    int64_t dst_b, src_a;         // bytes: destination stride along B, source stride along A (the other two are the unit)
+    uint32_t tiles_a, tiles_b;
+    uint32_t nouter;              // outer dimensions
+    FastDivU32 tiles_div;         // tiles_a * tiles_b
+    FastDivU32 tb_div;            // tiles_b
+    FastDivU32 outer_div[OPHIP_REARRANGE_MAXD];  // units per step of outer dimension q (innermost outer = 1)
+    int64_t outer_dst[OPHIP_REARRANGE_MAXD], outer_src[OPHIP_REARRANGE_MAXD];  // bytes
+};
+
 struct SampleParams {
     void *kv;            // ophip_kv_pair*, one per row
     const void *logits;  // rows x n

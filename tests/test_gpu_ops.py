@@ -1425,3 +1425,28 @@ def test_rearrange_large_contiguous_run_is_bit_exact(gpu, stream, nbytes, off):
     out = gpu.to_host(dd, np.uint8, nbytes + 128, stream=stream)
     assert np.array_equal(out[off:off + nbytes], src[off:off + nbytes])
     assert (out[:off] == 0xEE).all() and (out[off + nbytes:] == 0xEE).all()
+
+
+@pytest.mark.parametrize("shape,perm,dtype", [((8192, 4096), (1, 0), np.uint16), ((1000, 777), (1, 0), np.uint16), ((33, 4099), (1, 0), np.uint32),
+                                              ((5, 300, 200), (0, 2, 1), np.uint16), ((3, 64, 5, 96), (2, 3, 0, 1), np.uint64),
+                                              ((7, 129, 65), (2, 1, 0), np.uint32), ((40, 33, 32), (2, 0, 1), np.uint16)])
+def test_rearrange_transposes_of_small_units_bit_exact(gpu, stream, shape, perm, dtype):
+    """dst = src.transpose(perm), both contiguous, units of 2 / 4 / 8 bytes: the LDS-tiled kernel where the destination's
+    and the source's contiguous dimensions are both at least 32 long, the element-wise one otherwise; every byte against
+    numpy and the oracle."""
+    rng = np.random.default_rng(sum(shape))
+    src = rng.integers(0, np.iinfo(dtype).max, shape, dtype=dtype)
+    want = np.ascontiguousarray(src.transpose(perm))
+    nb = src.dtype.itemsize
+    # the destination seen in the source's index order: contiguous strides of `want`, permuted back
+    dstrides = [0] * len(shape)
+    for k, ax in enumerate(perm):
+        dstrides[ax] = want.strides[k]
+    code = {2: dt.U16, 4: dt.U32, 8: dt.U64}[nb]
+    sd, dd = gpu.from_host(src), gpu.malloc(src.nbytes + 64)
+    gpu.memset(dd, 0xEE)
+    say("rearrange transpose %s perm %s %d-byte units" % (shape, perm, nb))
+    ophip.Rearrange(gpu).launch(ophip.RearrangeArgs(TensorLayout(code, list(shape), dstrides), dd, TensorLayout.of(src), sd), None, stream)
+    out = gpu.to_host(dd, np.uint8, src.nbytes + 64, stream=stream)
+    assert np.array_equal(out[:src.nbytes].view(dtype).reshape(want.shape), want)
+    assert (out[src.nbytes:] == 0xEE).all()
