@@ -42,6 +42,25 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+_PROBE_LIB = None
+
+
+def bench_probe(kind, dst, src, nbytes, iters, seed, blocks, stream):
+    """One launch of a measurement probe (bench_probes/probe.hip, a library of its own beside the operator library)."""
+    global _PROBE_LIB
+    if _PROBE_LIB is None:
+        path = os.path.join(ROOT, "bench_probes", "libbenchprobe.so")
+        if not os.path.exists(path):
+            raise RuntimeError("%s is missing: make -C bench_probes" % path)
+        _PROBE_LIB = ctypes.CDLL(path)
+        _PROBE_LIB.bench_probe.argtypes = [ctypes.c_char_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint,
+                                           ctypes.c_uint, ctypes.c_uint, ctypes.c_void_p]
+        _PROBE_LIB.bench_probe_error.restype = ctypes.c_char_p
+    ptr = lambda m: None if m is None else (m.ptr if hasattr(m, "ptr") else int(m))
+    if _PROBE_LIB.bench_probe(kind.encode(), ptr(dst), ptr(src), nbytes, iters, seed, blocks, stream.handle):
+        raise RuntimeError("bench_probe(%s): %s" % (kind, _PROBE_LIB.bench_probe_error().decode()))
+
+
 def normal_f16(rng, shape, std):
     return (rng.standard_normal(shape, dtype=np.float32) * np.float32(std)).astype(f16)
 
@@ -213,9 +232,7 @@ def ceilings(ophip, gpu, stream):
     a_, b_ = gpu.malloc(nbytes), gpu.malloc(nbytes)
     gpu.memset(a_, 0x3C)
     gpu.memset(b_, 0)
-    probe = lambda kind, blocks, iters=0, seed=1, dst=None: ophip._check(ophip.lib().ophip_probe(
-        gpu.handle, kind.encode(), ctypes.c_void_p((dst or b_).ptr), ctypes.c_void_p(a_.ptr), ctypes.c_size_t(nbytes),
-        ctypes.c_uint(iters), ctypes.c_uint(seed), ctypes.c_uint(blocks), stream.handle))
+    probe = lambda kind, blocks, iters=0, seed=1, dst=None: bench_probe(kind, dst or b_, a_, nbytes, iters, seed, blocks, stream)
     for kind, moved in (("read", nbytes), ("read_nt", nbytes), ("write", nbytes), ("copy", 2 * nbytes)):
         best = None
         for blocks in (1024, 2048, 4096, 8192, 16384, 65536):
@@ -256,6 +273,51 @@ def ceilings(ophip, gpu, stream):
     return out
 
 
+def granule_classes(ophip, gpu, stream):
+    """A walk down one 128-column strip of an N-contiguous f16 weight reads one 256-byte granule per row.  Probe
+    "granules": one workgroup per strip, each noting its own time, on the decode layer's weight shapes and on row lengths
+    of other residues: per class of a strip's first granule (address bits 8..10 of its first byte), the mean time of the
+    strips of that class.  The classes that come out slower are the ones mat_mul's planner cuts into more K ranges."""
+    out = []
+    # (name, rows K, columns N): rows of 172 / 96 / 32 granules (residues 4, 0, 0 modulo 8), then 174 (residue 6), 173 (odd)
+    shapes = [("gate_up", 4096, 22016), ("qkv", 4096, 12288), ("o_proj", 4096, 4096), ("rows of 174 granules", 4096, 22272),
+              ("rows of 173 granules", 4096, 22144)]
+    for name, k, n in shapes:
+        nbytes = k * n * 2
+        ncopy = max(2, (600 << 20) // nbytes + 1)
+        copies = [gpu.malloc(nbytes) for _ in range(ncopy)]
+        for c in copies:
+            gpu.memset(c, 0x3C)
+        strips = (n + 127) // 128
+        ticks = gpu.malloc(4 * (strips + 1))
+        per_class = np.zeros(8)
+        count = np.zeros(8)
+        total = []
+        reps = 20
+        for it in range(reps + 2):
+            w = copies[it % ncopy]
+            bench_probe("granules", ticks, w, nbytes, n, k, 1, stream)
+            t = gpu.to_host(ticks, np.uint32, strips, stream=stream).astype(np.float64) / 100.0  # 100 MHz ticks -> us
+            if it < 2:
+                continue
+            cls = ((w.ptr >> 8) + np.arange(strips)) & 7
+            for c in range(8):
+                per_class[c] += t[cls == c].sum()
+                count[c] += (cls == c).sum()
+            total.append(t.max())
+        row = {"shape": name, "k": k, "n": n, "strips": strips, "granules_per_row": n * 2 // 256,
+               "us_by_class_of_first_granule": [round(float(per_class[c] / max(count[c], 1)), 2) for c in range(8)],
+               "slowest_strip_us": round(float(np.mean(total)), 2)}
+        out.append(row)
+        log("  granules %-22s %d strips, rows of %d granules: us by class %s, slowest strip %.2f" % (
+            name, strips, row["granules_per_row"], " ".join("%d:%.1f" % (c, v) for c, v in enumerate(row["us_by_class_of_first_granule"])),
+            row["slowest_strip_us"]))
+        for c in copies:
+            c.free()
+        ticks.free()
+    return out
+
+
 def gemm_floors(ophip, gpu, stream, rng, reps):
     """The six GEMMs of the decode layer on cold operands (copies of the weight or cache operand rotate through more than
     600 MB), each beside what a bare read of the same bytes takes: the library's read probe (non-temporal loads) over
@@ -267,9 +329,7 @@ def gemm_floors(ophip, gpu, stream, rng, reps):
     mm = layer.ops["mm"]
     out = []
     one = gpu.malloc(4096)
-    probe = lambda kind, dst, src, nbytes, blocks: ophip._check(ophip.lib().ophip_probe(
-        gpu.handle, kind.encode(), ctypes.c_void_p(dst.ptr), ctypes.c_void_p(src.ptr if src else dst.ptr),
-        ctypes.c_size_t(nbytes), ctypes.c_uint(0), ctypes.c_uint(1), ctypes.c_uint(blocks), stream.handle))
+    probe = lambda kind, dst, src, nbytes, blocks: bench_probe(kind, dst, src if src else dst, nbytes, 0, 1, blocks, stream)
     empty_us = time_launches(gpu, stream, lambda: probe("write", one, None, 16, 1), 200, warm=10)
     log("  empty launch (16 bytes written by one workgroup), back to back: %.2f us" % empty_us)
     work = layer_work()
@@ -374,8 +434,7 @@ def gemm_floors(ophip, gpu, stream, rng, reps):
             it = [0]
 
             def run_pattern():
-                ophip._check(ophip.lib().ophip_probe(gpu.handle, b"strips", ctypes.c_void_p(one.ptr), ctypes.c_void_p(copies[it[0] % ncopy].ptr),
-                                                     ctypes.c_size_t(nbytes), ctypes.c_uint(n), ctypes.c_uint(k), ctypes.c_uint(ranges), stream.handle))
+                bench_probe("strips", one, copies[it[0] % ncopy], nbytes, n, k, ranges, stream)
                 it[0] += 1
             row["us_by_k_ranges"][ranges] = round(time_launches(gpu, stream, run_pattern, reps, warm=ncopy), 2)
         pattern.append(row)
@@ -767,6 +826,8 @@ def main():
                          "shape (hardware-counter runs)")
     ap.add_argument("--floors", action="store_true",
                     help="only the decode layer's GEMMs on cold operands, each beside a bare read of the same bytes")
+    ap.add_argument("--granules", action="store_true",
+                    help="only the granule-class probe: how long a walk down each 128-column strip of a weight takes")
     ap.add_argument("--ceilings", action="store_true",
                     help="only the machine's ceilings: stream probes (read, write, copy) and the bare MFMA loop")
     args = ap.parse_args()
@@ -787,6 +848,9 @@ def main():
         return
     if args.ceilings:
         print(json.dumps({"ceilings": ceilings(ophip, gpu, stream)}))
+        return
+    if args.granules:
+        print(json.dumps({"granules": granule_classes(ophip, gpu, stream)}))
         return
     if args.attention_only is not None:
         lines = []

@@ -157,16 +157,6 @@ OPHIP_API int ophip_event_elapsed_ms(ophip_device *dev, ophip_event start, ophip
  * records around it.  An operator that launches several kernels times its first. */
 OPHIP_API int ophip_time_next_launch(ophip_device *dev, ophip_stream stream, ophip_event start, ophip_event stop);
 
-/* Measurement aid, no counterpart in the reference: one launch of a probe kernel, for ceilings measured on the machine
- * at hand.  kind = "read", "read_nt" (non-temporal loads), "read16", "read_nt16" (sixteen instead of four 16-byte loads
- * in flight per thread), "write", "copy": `blocks` workgroups of 256 threads stream
- * `bytes` (a multiple of 16) from `src` and / or into `dst` (16-byte aligned; a read-only probe writes at most 16 bytes
- * to dst).  kind = "strips": the weight-streaming mat_mul's access pattern alone; `src` is a row-major f16 matrix of `seed`
- * rows and `iters` columns (a multiple of 8) inside `bytes`, read in 128-column strips by one workgroup per strip and
- * per each of `blocks` equal row ranges (`seed` a multiple of 32 * blocks).  kind = "mfma": `blocks` workgroups run `iters` trips of 128 v_mfma_f32_32x32x16_f16 per wave on operands made
- * in registers from `seed` (0: all-zero operands) = blocks * 4 * iters * 128 * 32768 flop; dst needs blocks * 1024 bytes. */
-OPHIP_API int ophip_probe(ophip_device *dev, const char *kind, void *dst, const void *src, size_t bytes,
-                          unsigned iters, unsigned seed, unsigned blocks, ophip_stream stream);
 
 /* Launch graphs (no counterpart in the reference's driver crate): a fixed sequence of launch()
  * calls on `stream` between begin and end is recorded instead of run, and replayed by
@@ -178,9 +168,11 @@ OPHIP_API int ophip_probe(ophip_device *dev, const char *kind, void *dst, const 
  * stream it was recorded on.  Hence: replay a graph on the stream it was recorded on (on another stream,
  * while that one also runs split-K products of the same operator, two kernels would share one set of
  * counters and sum wrongly), and destroy a graph before the operators recorded into it (the operator
- * frees its counters).  An operator keeps one 256 KiB counter buffer per stream it is launched on; a
- * stream ended with ophip_stream_destroy (which then waits for the stream's work first) hands its
- * buffer to the next new stream, the rest is freed with the operator. */
+ * frees its counters) and before the stream it was recorded on (the counters a graph names go to the
+ * next new stream once theirs is destroyed).  An operator keeps one 256 KiB counter buffer per stream
+ * it is launched on; a stream ended with ophip_stream_destroy (which waits for the stream's work first,
+ * unless the stream is still recording: then nothing is handed on) hands its buffer to the next new
+ * stream, the rest is freed with the operator. */
 typedef void *ophip_graph; /* hipGraphExec_t */
 OPHIP_API int ophip_stream_begin_capture(ophip_device *dev, ophip_stream stream);
 OPHIP_API int ophip_stream_end_capture(ophip_device *dev, ophip_stream stream, ophip_graph *out);
@@ -431,9 +423,11 @@ OPHIP_API void ophip_mat_mul_destroy(ophip_mat_mul *op);
 OPHIP_API int ophip_mat_mul_launch_static(const ophip_mat_mul *op, const ophip_mat_mul_args *args,
                                           ophip_stream stream);
 /* Diagnostics, no counterpart in the reference: writes the name of the kernel family launch()
- * would pick for these arguments on this device ("skinny rows<=16 qN split_k=8", "skinny rows<=16 qN paired split_k=1",
+ * would pick for these arguments on this device ("stream rows<=16 qN split_k=1 (2 on granule classes 0x22)",
+ * "stream rows<=16 qN split_k=8", "skinny rows<=32 qN paired split_k=1",
  * "skinny rows<=32 qK256 split_k=2", "tile256x64 pK qN split_k=1",
- * "tile128x64 ragged pK qK split_k=1" when M or N is not in whole tiles, "tile128x32 ...", "generic") into out[0..len). */
+ * "tile128x64 ragged pK qK split_k=1" when M or N is not in whole tiles, "tile128x32 ...", "generic") into out[0..len).
+ * `op` may be null: the choice for a device of 256 compute units (needs no device; the CPU tests of the planner use it). */
 OPHIP_API int ophip_mat_mul_describe(const ophip_mat_mul *op, const ophip_mat_mul_args *args, char *out, size_t len);
 
 /* ---- attention: attention/args.rs:10-24, attention/operator.rs:31-277 ------ */

@@ -218,6 +218,24 @@ size_t attention_scheme(ophip_attention *op, const ophip_attention_args &args, s
     return ans;
 }
 
+// The bytes a rank-3 view can touch, as [first, last) addresses (strides in bytes, of either sign; an empty view
+// touches nothing).
+struct ByteSpan {
+    const char *lo, *hi;
+};
+ByteSpan span_of(const void *base, const size_t (&shape)[3], const ptrdiff_t (&strides)[3], size_t ele) {
+    const char *b = static_cast<const char *>(base);
+    if (shape[0] == 0 || shape[1] == 0 || shape[2] == 0) return {b, b};
+    ptrdiff_t lo = 0, hi = 0;
+    for (int i = 0; i < 3; ++i) {
+        const ptrdiff_t reach = (ptrdiff_t)(shape[i] - 1) * strides[i];
+        (reach < 0 ? lo : hi) += reach;
+    }
+    return {b + lo, b + hi + (ptrdiff_t)ele};
+}
+bool spans_apart(const ByteSpan &x, const ByteSpan &y) { return x.lo == x.hi || y.lo == y.hi || x.hi <= y.lo || y.hi <= x.lo; }
+
+
 // The one-pass kernel (attention_prefill.hip) when it serves this call; false, with nothing done, otherwise.
 // `merged`: the reference would use q in place and leave att . v in it.
 bool attention_one_pass(const ophip_attention *op, const ophip_attention_args &args, const AttentionMeta &m, bool merged,
@@ -254,14 +272,10 @@ bool attention_one_pass(const ophip_attention *op, const ophip_attention_args &a
     }
     // o must not lie over anything the other workgroups still read: apart from q itself in q's own layout
     auto span = [](const View &t) {
-        size_t end = 2;
-        for (int i = 0; i < 3; ++i) end += (size_t)(static_of(t.l.shape[i]) - 1) * (size_t)static_of(t.l.strides[i]);
-        return std::pair<const char *, const char *>(static_cast<const char *>(t.base), static_cast<const char *>(t.base) + end);
+        return span_of(t.base, {static_of(t.l.shape[0]), static_of(t.l.shape[1]), static_of(t.l.shape[2])},
+                       {static_of(t.l.strides[0]), static_of(t.l.strides[1]), static_of(t.l.strides[2])}, 2);
     };
-    auto apart = [&](const View &a, const View &b) {
-        const auto x = span(a), y = span(b);
-        return x.second <= y.first || y.second <= x.first;
-    };
+    auto apart = [&](const View &a, const View &b) { return spans_apart(span(a), span(b)); };
     const bool o_is_q = o.base == q.base && static_of(o.l.strides[0]) == static_of(q.l.strides[0]) &&
                         static_of(o.l.strides[1]) == static_of(q.l.strides[1]);
     if (!o_is_q && !apart(o, q)) return false;
@@ -339,6 +353,23 @@ bool decode_one_pass(const ophip_attention *op, const DecodeCall &c, void *works
     // the reference overwrites q with the result when q's heads and tokens merge (attention/operator.rs:186-239)
     const ptrdiff_t nh_sq = c.q->strides[0], seq_sq = c.q->strides[1];
     const bool merged = nh == 1 || seq == 1 || nh_sq == (ptrdiff_t)seq * seq_sq;
+    // A kv head's workgroup writes o (and q, when the reference would) while the workgroups of other kv heads may
+    // still read q, the appended rows and the caches: the composite reads all of them before it writes, so a call
+    // whose o (or overwritten q) lies over any of them is left to it.  o over q itself, in q's own layout, is fine:
+    // a workgroup reads the rows it writes, and no other.
+    {
+        const size_t fresh = att - c.pos;  // rows of k_new / v_new
+        const ByteSpan qs = span_of(c.q_base, {nh, seq, dh}, {c.q->strides[0], c.q->strides[1], 2}, 2);
+        const ByteSpan os = span_of(c.o_base, {nh, seq, dh}, {c.o->strides[0], c.o->strides[1], 2}, 2);
+        const ByteSpan kn = span_of(c.k_new_base, {nkvh, fresh, dh}, {c.k_new->strides[0], c.k_new->strides[1], 2}, 2);
+        const ByteSpan vn = span_of(c.v_new_base, {nkvh, fresh, dh}, {c.v_new->strides[0], c.v_new->strides[1], 2}, 2);
+        const ByteSpan kc = span_of(c.k_cache_base, {nkvh, att, dh}, {c.k_cache->strides[0], c.k_cache->strides[1], 2}, 2);
+        const ByteSpan vc = span_of(c.v_cache_base, {nkvh, att, dh}, {c.k_cache->strides[0], c.k_cache->strides[1], 2}, 2);
+        const bool o_is_q = c.o_base == c.q_base && c.o->strides[0] == c.q->strides[0] && c.o->strides[1] == c.q->strides[1];
+        if (!o_is_q && !spans_apart(os, qs)) return false;
+        for (const ByteSpan *t : {&kn, &vn, &kc, &vc})
+            if (!spans_apart(os, *t) || (merged && !spans_apart(qs, *t))) return false;
+    }
     p.q_out = merged && c.q_base != c.o_base ? c.q_base : nullptr;
     p.k_new = c.k_new_base;
     p.v_new = c.v_new_base;

@@ -338,13 +338,19 @@ int ophip_stream_create(ophip_device *dev, ophip_stream *out) {
 int ophip_stream_destroy(ophip_device *dev, ophip_stream stream) {
     return guard([&] {
         dev->make_current();
-        {
+        // What the hooks hand on to other streams (mat_mul's arrival counters) must be at rest first.  The wait happens
+        // before the lock is taken, so that creating or destroying an operator on this device never waits for this
+        // stream's work.  A stream that is still recording cannot be waited for; its buffers are then not handed on
+        // (the graph being recorded may hold their addresses): the operators that own them free them when they go.
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        const bool recording = hipStreamIsCapturing((hipStream_t)stream, &capturing) == hipSuccess &&
+                               capturing != hipStreamCaptureStatusNone;
+        if (!recording) {
+            check_hip(hipStreamSynchronize((hipStream_t)stream), "hipStreamSynchronize");
             std::lock_guard<std::mutex> lock(dev->hooks_mu);
-            if (!dev->stream_gone.empty()) {
-                // what the hooks hand on to other streams must be at rest first
-                check_hip(hipStreamSynchronize((hipStream_t)stream), "hipStreamSynchronize");
-                for (auto &h : dev->stream_gone) h.second((hipStream_t)stream);
-            }
+            for (auto &h : dev->stream_gone) h.second((hipStream_t)stream);
+        } else {
+            (void)hipGetLastError();
         }
         check_hip(hipStreamDestroy((hipStream_t)stream), "hipStreamDestroy");
     });
@@ -395,30 +401,6 @@ int ophip_time_next_launch(ophip_device *dev, ophip_stream stream, ophip_event s
         g_timed.stream = (hipStream_t)stream;
         g_timed.start = (hipEvent_t)start;
         g_timed.stop = (hipEvent_t)stop;
-    });
-}
-
-// Measurement probes (probe.hip): one launch of the named probe over `bytes` of memory (streams) or with `iters`
-// trips (mfma), `blocks` workgroups of 256 threads.
-int ophip_probe(ophip_device *dev, const char *kind, void *dst, const void *src, size_t bytes, unsigned iters,
-                unsigned seed, unsigned blocks, ophip_stream stream) {
-    return guard([&] {
-        if (!dev || !kind) throw args_not_support("null argument");
-        const std::string k = kind;
-        const bool reads = k == "read" || k == "read_nt" || k == "read16" || k == "read_nt16" || k == "copy", writes = k == "write" || k == "copy";
-        if (!reads && !writes && k != "mfma" && k != "strips") throw args_not_support("unknown probe: " + k);
-        if ((reads && !src) || !dst || blocks == 0) throw args_not_support("probe: null buffer or empty grid");
-        if ((reads || writes) && (bytes % 16 != 0 || !aligned16(dst) || (reads && !aligned16(src))))
-            throw args_not_support("probe: buffers in whole 16-byte vectors");
-        ProbeParams p{dst, src, (uint64_t)bytes, iters, seed};
-        dev->make_current();
-        if (k == "strips") {  // `src`: [seed rows][iters columns] f16, `blocks` row ranges; one workgroup per 128-column strip and range
-            if (!src || !dst || iters < 8 || iters % 8 != 0 || blocks == 0 || seed % (32 * blocks) != 0 || (size_t)iters * seed * 2 > bytes || !aligned16(src))
-                throw args_not_support("probe strips: [seed][iters] f16 inside `bytes`, rows in whole groups of 32 per range");
-            launch(dev->kernel("probe", "probe_strips"), Dim3{(iters + 127) / 128, blocks}, Dim3{256}, 0, (hipStream_t)stream, p);
-            return;
-        }
-        launch(dev->kernel("probe", ("probe_" + k).c_str()), Dim3{blocks}, Dim3{256}, 0, (hipStream_t)stream, p);
     });
 }
 

@@ -97,7 +97,9 @@ ophip_mat_mul_layout mat_mul_layout(const ophip_mat_mul_args &args) {
 struct GemmPlan {
     GemmParams p{};
     enum Kind { Generic, Skinny, Tile } kind = Generic;
-    int mt = 1, qmode = 0;  // Skinny: 16-row blocks, weight layout mode (3: mode 0 with K-steps dealt in pairs)
+    // Skinny: 16-row blocks, weight layout mode (3: mode 0 with K-steps dealt in pairs; 4: gemm_stream, the build of
+    // mode 0 for up to 16 rows and K in whole steps)
+    int mt = 1, qmode = 0;
     int tile = 256, tk = 64, pk = 1, qk = 1;  // Tile: block size, K-step, and whether P / Q are K-contiguous
     bool ragged = false;                      // Tile: M or N not in whole tiles, or K not in whole K-steps
     size_t workspace = 0;
@@ -109,6 +111,8 @@ bool mult8(int64_t v) { return (v & 7) == 0; }
 // (OPHIP_GEMM_SPLITK, OPHIP_GEMM_TILE_SPLITK, OPHIP_GEMM_TILE); 0 = not set.
 struct GemmKnobs {
     int skinny_split = 0, tile_split = 0, tile = 0;
+    bool stream = true;   // OPHIP_GEMM_STREAM=0: keep gemm_skinny where gemm_stream would run
+    int slow_split = -1;  // OPHIP_GEMM_SLOW_SPLIT: K ranges for strips on the slow granule classes (0: cut all strips alike)
     static GemmKnobs from_env() {
         GemmKnobs k;
         auto num = [](const char *name) {
@@ -119,6 +123,8 @@ struct GemmKnobs {
         k.skinny_split = num("OPHIP_GEMM_SPLITK");
         k.tile_split = num("OPHIP_GEMM_TILE_SPLITK");
         k.tile = num("OPHIP_GEMM_TILE");
+        if (const char *e = std::getenv("OPHIP_GEMM_STREAM")) k.stream = std::atoi(e) != 0;
+        if (const char *e = std::getenv("OPHIP_GEMM_SLOW_SPLIT")) k.slow_split = std::max(0, std::atoi(e));
         return k;
     }
 };
@@ -126,6 +132,54 @@ struct GemmKnobs {
 // f16, f32, f64: the CPU backend's types (mat_mul/common_cpu/mod.rs:99-103).  bf16: neither backend of the reference
 // multiplies it (its CUDA backend checks for F16, mat_mul/cuda/mod.rs:73); taken here because the matrix cores do.
 bool mat_mul_takes(uint64_t dt) { return dt == OPHIP_DT_F16 || dt == OPHIP_DT_BF16 || dt == OPHIP_DT_F32 || dt == OPHIP_DT_F64; }
+
+// gemm_stream's uneven cut.  A workgroup that walks down one 128-column strip of an N-contiguous weight reads one
+// 256-byte granule per row.  When the rows are a multiple of 1 KiB apart and start on a granule boundary, all
+// granules of a strip have the same class (address bits 8..10) or alternate between c and c + 4, and HBM serves
+// classes 1 and 5 about a quarter slower under this access pattern than the rest (4096 x 22016, cold weights, one
+// workgroup per strip: the strips of those two classes take 32 us, the others 25; a plain sequential read of the same
+// matrix shows no such difference, since there every request spans all classes).  The launch ends with its slowest
+// strip, so those strips get more K ranges: as many as still leave at most one workgroup per CU.
+// Returns the ranges for the slow strips and sets p.slow_mask / p.split_slow; 0 (and mask 0): all strips alike.
+size_t plan_slow_strips(GemmParams &p, size_t ntiles, size_t cus, const GemmKnobs &knobs) {
+    p.slow_mask = 0;
+    p.split_slow = 0;
+    if (knobs.slow_split == 0) return 0;
+    const int64_t rowb = p.q_sl * 2, batb = p.q_sb * 2;
+    const uintptr_t base = reinterpret_cast<uintptr_t>(p.q);
+    if (base % 256 != 0 || rowb % 1024 != 0 || (p.batch > 1 && batb % 2048 != 0)) return 0;
+    const uint32_t mask = 0x22;  // classes 1 and 5
+    size_t slow = 0;
+    for (size_t t = 0; t < ntiles; ++t) slow += (mask >> (((base >> 8) + t) & 7)) & 1;
+    if (slow == 0) return 0;
+    const size_t steps = p.K / 32, s0 = p.split_k;
+    // Measured so far only for strips that are otherwise whole (4096 x 22016: 35.6 -> 31.3 us with the slow strips in two
+    // ranges); with two ranges everywhere and four on the slow strips 4096 x 12288 stayed where it was (21.0 against
+    // 21.2 us), so such products keep the even cut.
+    if (s0 != 1 && knobs.slow_split < 0) return 0;
+    auto whole = [&](size_t s) {  // a cut into s ranges of ceil(steps / s) steps leaves none of them empty
+        const size_t sps = (steps + s - 1) / s;
+        return (steps + sps - 1) / sps == s;
+    };
+    size_t best = s0;
+    if (knobs.slow_split > 0) {
+        best = std::min<size_t>((size_t)knobs.slow_split, steps);
+        while (!whole(best)) --best;
+    } else {
+        // a slow strip costs 1.28 fast ones per byte: the smallest cut that brings its ranges under a fast strip's
+        double best_cost = 1.28 / (double)s0;
+        for (size_t s1 = s0 + 1; s1 <= 2 * s0 + 1 && s1 <= steps / 4; ++s1) {
+            if (!whole(s1)) continue;
+            if (((ntiles - slow) * s0 + slow * s1) * p.batch > cus) break;
+            const double cost = std::max(1.0 / (double)s0, 1.28 / (double)s1);
+            if (cost < best_cost - 1e-9) best = s1, best_cost = cost;
+        }
+    }
+    if (best == s0) return 0;
+    p.slow_mask = mask;
+    p.split_slow = (uint32_t)best;
+    return best;
+}
 
 GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L, unsigned cus, const GemmKnobs &knobs) {
     const void *a = L.ab_swap ? args.b_base : args.a_base;
@@ -238,8 +292,17 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
                 // waves in pairs and requests both halves of P's cache lines together (same box, cold weights,
                 // 16 / 32 rows: 4096 x 22016 37.0 -> 35.9 / 42.2 -> 39.1 us, 4096 x 12288 split 2 23.4 -> 22.6 / 27.5 -> 26.3;
                 // K = 4096 split 8 and 11008 split 8 lose 2 - 4 %, so they keep the plain dealing)
+                // Up to 16 rows, N-contiguous weight, K in whole steps: gemm_stream (same wave tile, two register buffers
+                // instead of three, no tail code; cold weights, 16 rows: 4096 x 22016 35.7 -> 35.5 us, 4096 x 12288 split 2
+                // 21.9 -> 21.1, 4096 x 4096 split 8 11.5 -> 10.9, 11008 x 4096 split 8 20.1 -> 19.5).  Its lane offsets are 32 bits.
+                size_t split_slow = 0;
+                if (knobs.stream && g.mt == 1 && g.qmode == 0 && p.K % 32 == 0 && p.q_sl < ((int64_t)1 << 24) && p.p_si < ((int64_t)1 << 26)) {
+                    g.qmode = 4;
+                    split_slow = plan_slow_strips(p, ntiles, (size_t)cus, knobs);
+                }
                 if (g.qmode == 0 && p.k_per_split % 256 == 0 && p.k_per_split >= 1024 && p.K % p.k_per_split == 0) g.qmode = 3;
-                g.workspace = split > 1 ? split * p.batch * (size_t)p.M * p.N * sizeof(float) : 0;
+                const size_t ranges = std::max<size_t>(p.split_k, split_slow);
+                g.workspace = ranges > 1 ? ranges * p.batch * (size_t)p.M * p.N * sizeof(float) : 0;
                 return true;
             }
         }
@@ -363,6 +426,7 @@ struct ophip_mat_mul {
     GemmKnobs knobs = GemmKnobs::from_env();
     // the MFMA kernels exist twice, [0] on f16 and [1] on bf16 elements
     hipFunction_t skinny[2][3][4];  // [mt index 1,2,4][qmode; 3 = mode 0 with paired K-steps]
+    hipFunction_t stream[2];        // gemm_stream_m1
     hipFunction_t reduce[2], fill, generic_f16, generic_bf16, generic_f32, generic_f64;
     // [256 x 64 / 128 x 64 / 128 x 32 (K-step)][M or N not in whole tiles][P K-contiguous][Q K-contiguous]
     hipFunction_t tile[2][3][2][2][2];
@@ -418,6 +482,7 @@ struct ophip_mat_mul {
                             tile[e][b][r][pk][qk] = d->kernel(gemm_tile, ("gemm_tile_" + sz + (r ? "r" : "") + "_p" + std::to_string(pk) +
                                                                           "_q" + std::to_string(qk) + tag).c_str());
                         }
+            stream[e] = d->kernel(gemm, (std::string("gemm_stream_m1") + tag).c_str());
             reduce[e] = d->kernel(gemm, (std::string("gemm_splitk_reduce") + tag).c_str());
         }
         fill = d->kernel("gemm", "gemm_fill_u32");
@@ -457,8 +522,8 @@ struct ophip_mat_mul {
 
 // One launch.  `fixed_counters` null: the ordinary entry point (workspace from the caller or the queue allocator,
 // arrival counters owned by the operator).  Otherwise the caller of this function brings every byte of scratch:
-// `workspace` holds the f32 partials, `fixed_counters` the arrival counters (cleared here, by a kernel, as far as
-// this launch uses them), and nothing is allocated.
+// `workspace` holds the f32 partials, `fixed_counters` the arrival counters (all zero between launches: zero when the
+// caller made them, and every kernel leaves the ones it used at zero), and nothing is allocated.
 static void mat_mul_launch_impl(const ophip_mat_mul *op, const ophip_mat_mul_args *args, void *workspace,
                                 size_t workspace_len, const ophip_queue_alloc *qa, void *fixed_counters,
                                 size_t fixed_counter_count, hipStream_t stream) {
@@ -484,17 +549,24 @@ static void mat_mul_launch_impl(const ophip_mat_mul *op, const ophip_mat_mul_arg
         g.p.partial = ws.ptr();
         const size_t tiles = (size_t)((p.N + 127) / 128) * p.batch;
         if (fixed) {
-            g.p.counters = (p.split_k > 1 && tiles <= fixed_counter_count && g.workspace < ((size_t)1 << 32)) ? fixed_counters : nullptr;
-            if (g.p.counters) {  // the static buffer keeps what the last call left: start this launch's counters at zero
-                FillU32Params f{fixed_counters, (uint32_t)tiles, 0u};
-                launch(op->fill, Dim3{(unsigned)((tiles + 255) / 256)}, Dim3{256}, 0, stream, f);
-            }
+            g.p.counters = ((p.split_k > 1 || p.slow_mask) && tiles <= fixed_counter_count && g.workspace < ((size_t)1 << 32)) ? fixed_counters : nullptr;
+            // (the static array is zero when its module is loaded and every kernel hands its counters back at zero: the
+            //  invariant the operator's own counter buffers rely on as well, so nothing is cleared here)
         } else {
             // (the in-kernel reduction addresses the partials with 32-bit offsets)
-            g.p.counters = (p.split_k > 1 && tiles <= SPLITK_COUNTERS && g.workspace < ((size_t)1 << 32)) ? op->counters_for(stream) : nullptr;
+            g.p.counters = ((p.split_k > 1 || p.slow_mask) && tiles <= SPLITK_COUNTERS && g.workspace < ((size_t)1 << 32)) ? op->counters_for(stream) : nullptr;
         }
         const int mi = g.mt == 1 ? 0 : g.mt == 2 ? 1 : 2;
-        launch(op->skinny[e][mi][g.qmode], Dim3{(p.N + 127) / 128, p.split_k, p.batch}, Dim3{256}, 0, stream, g.p);
+        if (g.qmode == 4) {
+            const bool ranges = p.split_k > 1 || p.slow_mask;
+            if (ranges && !g.p.counters) {  // too many strips for the counters: cut every strip alike and sum in a second launch
+                g.p.slow_mask = 0;
+                g.p.split_slow = 0;
+            }
+            launch(op->stream[e], Dim3{gemm_stream_units(&g.p, reinterpret_cast<uint64_t>(g.p.q)), 1, p.batch}, Dim3{256}, 0, stream, g.p);
+        } else {
+            launch(op->skinny[e][mi][g.qmode], Dim3{(p.N + 127) / 128, p.split_k, p.batch}, Dim3{256}, 0, stream, g.p);
+        }
         if (p.split_k > 1 && !g.p.counters) {
             const size_t total = (size_t)p.batch * p.M * (p.N / 8);
             launch(op->reduce[e], Dim3{(unsigned)((total + 255) / 256)}, Dim3{256}, 0, stream, g.p);
@@ -562,14 +634,20 @@ int ophip_mat_mul_scheme(ophip_mat_mul *op, const ophip_mat_mul_args *args, size
 
 int ophip_mat_mul_describe(const ophip_mat_mul *op, const ophip_mat_mul_args *args, char *out, size_t len) {
     return guard([&] {
-        if (!op || !args || !out || len == 0) throw args_not_support("null argument");
+        if (!args || !out || len == 0) throw args_not_support("null argument");
         const ophip_mat_mul_layout L = mat_mul_layout(*args);
         if (!mat_mul_takes(L.dt)) throw type_not_support("mat_mul supports f16, bf16, f32 and f64");
-        const GemmPlan g = make_plan(*args, L, (unsigned)op->dev->props.multiProcessorCount, op->knobs);
+        const GemmPlan g = op ? make_plan(*args, L, (unsigned)op->dev->props.multiProcessorCount, op->knobs)
+                              : make_plan(*args, L, 256u, GemmKnobs::from_env());
         if (g.kind == GemmPlan::Skinny)
-            std::snprintf(out, len, "skinny rows<=%d q%s split_k=%u", 16 * g.mt,
-                          g.qmode == 0 ? "N" : g.qmode == 1 ? "K" : g.qmode == 2 ? "K256" : "N paired",
-                          g.p.split_k);
+            if (g.qmode == 4 && g.p.slow_mask)
+                std::snprintf(out, len, "stream rows<=16 qN split_k=%u (%u on granule classes 0x%02x)", g.p.split_k, g.p.split_slow,
+                              g.p.slow_mask);
+            else if (g.qmode == 4)
+                std::snprintf(out, len, "stream rows<=16 qN split_k=%u", g.p.split_k);
+            else
+                std::snprintf(out, len, "skinny rows<=%d q%s split_k=%u", 16 * g.mt,
+                              g.qmode == 0 ? "N" : g.qmode == 1 ? "K" : g.qmode == 2 ? "K256" : "N paired", g.p.split_k);
         else if (g.kind == GemmPlan::Tile)
             std::snprintf(out, len, "tile%dx%d%s p%s q%s split_k=%u", g.tile, g.tk,
                           g.ragged ? " ragged" : "", g.pk ? "K" : "M", g.qk ? "K" : "N", g.p.split_k);

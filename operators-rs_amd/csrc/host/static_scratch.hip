@@ -7,8 +7,7 @@
 //
 // This file is compiled by hipcc for host and device: the array is a device symbol, its host-side name is
 // only a handle for hipGetSymbolAddress.  The address is resolved once per device (ophip_device_create,
-// with that device current) and kept; everything that touches the array afterwards -- kernel arguments,
-// the clearing kernel -- uses the resolved pointer.
+// with that device current) and kept; everything that touches the array afterwards uses the resolved pointer.
 #include <hip/hip_runtime.h>
 
 #include <mutex>
@@ -22,7 +21,10 @@ namespace {
 constexpr size_t COUNTER_BYTES = ophip::STATIC_COUNTERS * sizeof(uint32_t);
 constexpr size_t SCRATCH_BYTES = ophip::STATIC_PARTIAL_BYTES + COUNTER_BYTES;
 
-// [0, STATIC_PARTIAL_BYTES): f32 partials; then STATIC_COUNTERS u32 arrival counters
+// [0, STATIC_PARTIAL_BYTES): f32 partials; then STATIC_COUNTERS u32 arrival counters.  The array is zero when the
+// module is loaded, and a kernel that counts arrivals sets the counters it used back to zero before it ends: the
+// counters are zero between launches without anyone clearing them (calls that overlap on one GPU, which the entry
+// point's contract rules out, would break that).
 static __device__ __align__(256) unsigned char scratch[SCRATCH_BYTES];
 
 constexpr int MAX_DEVICES = 64;

@@ -14,7 +14,8 @@ constexpr size_t STATIC_PARTIAL_BYTES = (size_t)32 << 20;
 constexpr size_t STATIC_COUNTERS = (size_t)1 << 16;
 
 // Resolves the array's address on device `ordinal`, which must be the current device; called once per
-// device from ophip_device_create.  Throws ExecutionFailed.
+// device from ophip_device_create.  Never throws: when the address cannot be had the reason is kept, the device is
+// created all the same (nothing else needs the array), and ophip_mat_mul_launch_static reports the reason.
 void static_scratch_resolve(int ordinal);
 
 // mat_mul.cpp: one launch whose scratch (partials, counters) is all brought by the caller of this function.

@@ -123,13 +123,6 @@ struct AttnPrefillParams {
     float scale;
 };
 
-struct ProbeParams {  // probe.hip
-    void *dst;
-    const void *src;
-    uint64_t bytes;
-    uint32_t iters, seed;
-};
-
 // Canonical GEMM seen by the kernels:
 //   D[i, j] = alpha * sum_l P[i, l] * Q[l, j] + beta * D[i, j]
 // element strides; exactly one of each operand's two strides is 1.
@@ -147,7 +140,74 @@ struct GemmParams {
     uint32_t read_dst;  // the reference reads C only when beta != 0
     uint32_t split_k;
     uint32_t k_per_split;  // multiple of 32
+    // gemm_stream only: strips whose first 256-byte granule has its class (address bits 8..10) in `slow_mask` are cut
+    // into `split_slow` K ranges of ceil(K / 32 / split_slow) steps, the others into `split_k`; mask 0: all alike
+    uint32_t slow_mask;
+    uint32_t split_slow;
 };
+
+// gemm_stream's work units, numbered the same way by the kernel (blockIdx.x -> unit) and by the host (grid size; a
+// CPU test walks every unit of a launch through this function before any launch does).
+#if defined(__HIPCC__)
+#define OPHIP_HD __host__ __device__
+#else
+#define OPHIP_HD
+#endif
+struct GemmStreamUnit {
+    uint32_t strip;         // 128-column strip
+    uint32_t range;         // which of the strip's K ranges
+    uint32_t ranges;        // how many K ranges the strip has
+    uint32_t kbeg, kend;    // the range: rows [kbeg, kend), in whole steps of 32; empty if kend <= kbeg
+    uint32_t valid;         // 0: the block has no unit (the last group of eight strips is short)
+};
+// K ranges of a strip whose first 256-byte granule has class `cls` (address bits 8..10)
+static inline OPHIP_HD uint32_t gemm_stream_ranges(const struct GemmParams *p, uint32_t cls) {
+    return (p->slow_mask >> (cls & 7)) & 1 ? p->split_slow : p->split_k;
+}
+// Unit of workgroup `block` (blockIdx.x); `q_addr` = address of Q's first element for the batch entry.
+// Mask 0: strip-major inside each K range (block = range * strips + strip), every strip in split_k ranges of
+// k_per_split rows.  Otherwise: groups of eight consecutive strips, inside a group strip by strip, a strip's ranges
+// next to each other; a strip in n ranges has ranges of ceil(K / 32 / n) steps.
+static inline OPHIP_HD struct GemmStreamUnit gemm_stream_unit(const struct GemmParams *p, uint64_t q_addr, uint32_t block) {
+    struct GemmStreamUnit u;
+    const uint32_t nstrips = (p->N + 127) / 128;
+    uint32_t k_per = p->k_per_split;
+    u.valid = 1;
+    if (p->slow_mask == 0) {
+        u.strip = block % nstrips;
+        u.range = block / nstrips;
+        u.ranges = p->split_k;
+    } else {
+        const uint32_t g0 = (uint32_t)(q_addr >> 8);  // class of strip 0's first granule (strips are 256 bytes wide)
+        uint32_t per8 = 0;
+        for (uint32_t c = 0; c < 8; ++c) per8 += gemm_stream_ranges(p, g0 + c);
+        uint32_t r = block % per8;
+        u.strip = block / per8 * 8;
+        u.ranges = 1;
+        for (uint32_t c = 0; c < 8; ++c) {
+            u.ranges = gemm_stream_ranges(p, g0 + c);
+            if (r < u.ranges) break;
+            r -= u.ranges;
+            ++u.strip;
+        }
+        u.range = r;
+        if (u.strip >= nstrips) u.valid = 0;
+        k_per = (p->K / 32 + u.ranges - 1) / u.ranges * 32;
+    }
+    if (u.range >= u.ranges) u.valid = 0;  // (a grid larger than the units)
+    const uint64_t kb = (uint64_t)u.range * k_per;
+    u.kbeg = kb < p->K ? (uint32_t)kb : p->K;
+    u.kend = (uint64_t)u.kbeg + k_per < p->K ? u.kbeg + k_per : p->K;
+    return u;
+}
+// Workgroups per batch entry of a launch
+static inline OPHIP_HD uint32_t gemm_stream_units(const struct GemmParams *p, uint64_t q_addr) {
+    const uint32_t nstrips = (p->N + 127) / 128;
+    if (p->slow_mask == 0) return nstrips * p->split_k;
+    uint32_t per8 = 0;
+    for (uint32_t c = 0; c < 8; ++c) per8 += gemm_stream_ranges(p, (uint32_t)(q_addr >> 8) + c);
+    return (nstrips + 7) / 8 * per8;
+}
 
 // dst[0 .. size) = value, bytes: the first `head` bytes (up to 16-byte alignment) and the last `tail` bytes one at a
 // time, `body` 16-byte units between them

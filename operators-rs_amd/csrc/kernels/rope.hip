@@ -27,7 +27,11 @@ __device__ __forceinline__ void rope_fill_table(const RopeParams &p, uint32_t to
     for (uint32_t e = threadIdx.x; e < 2 * H; e += WG_THREADS) {
         const uint32_t k = e < H ? e : e - H;
         const float ang = pos / (p.has_den ? p.den[k] : powf(p.theta, (float)k / (float)H));
-        flat[2 * k + (e < H ? 0 : 1)] = e < H ? sinf(ang) : cosf(ang);
+        // the same evaluation as in rope_vec_multi (one sincosf, of which this thread keeps one half), so that a token
+        // gets the same bits whichever kernel its call is given
+        float sn, cs;
+        sincosf(ang, &sn, &cs);
+        flat[2 * k + (e < H ? 0 : 1)] = e < H ? sn : cs;
     }
     __syncthreads();
 }

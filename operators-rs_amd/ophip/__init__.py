@@ -204,7 +204,7 @@ EXPORTS = [
     "ophip_malloc", "ophip_free", "ophip_memcpy_h2d", "ophip_memcpy_d2h", "ophip_memcpy_d2d", "ophip_memset",
     "ophip_stream_create", "ophip_stream_destroy", "ophip_stream_synchronize",
     "ophip_event_create", "ophip_event_destroy", "ophip_event_record", "ophip_event_synchronize",
-    "ophip_event_elapsed_ms", "ophip_time_next_launch", "ophip_probe",
+    "ophip_event_elapsed_ms", "ophip_time_next_launch",
     "ophip_stream_begin_capture", "ophip_stream_end_capture", "ophip_graph_launch", "ophip_graph_destroy",
     "ophip_queue_alloc_from_stream", "ophip_mem_pool_create", "ophip_mem_pool_put",
     "ophip_mem_pool_queue_alloc", "ophip_mem_pool_destroy",
@@ -849,6 +849,13 @@ class RandomSample(_Operator):
         out = ctypes.c_void_p()
         _check(lib().ophip_random_sample_build_indices(ctypes.c_size_t(n), _qa(queue_alloc), ctypes.byref(out)))
         return out.value or 0
+
+
+def mat_mul_describe(args):
+    """MatMul.describe without an operator or a device: the kernel choice for a device of 256 compute units."""
+    buf = ctypes.create_string_buffer(96)
+    _check(lib().ophip_mat_mul_describe(None, ctypes.byref(args.c()), buf, ctypes.c_size_t(96)))
+    return buf.value.decode()
 
 
 class MatMul(_Operator):

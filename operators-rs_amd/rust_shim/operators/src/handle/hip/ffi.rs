@@ -331,8 +331,7 @@ extern "C" {
     pub fn ophip_event_synchronize(dev: *mut ophip_device, ev: *mut c_void) -> c_int;
     pub fn ophip_event_elapsed_ms(dev: *mut ophip_device, start: *mut c_void, stop: *mut c_void, ms: *mut f32) -> c_int;
     pub fn ophip_time_next_launch(dev: *mut ophip_device, stream: *mut c_void, start: *mut c_void, stop: *mut c_void) -> c_int;
-    pub fn ophip_probe(dev: *mut ophip_device, kind: *const c_char, dst: *mut c_void, src: *const c_void, bytes: usize,
-        iters: c_uint, seed: c_uint, blocks: c_uint, stream: *mut c_void) -> c_int;
+
     pub fn ophip_stream_begin_capture(dev: *mut ophip_device, stream: *mut c_void) -> c_int;
     pub fn ophip_stream_end_capture(dev: *mut ophip_device, stream: *mut c_void, out: *mut *mut c_void) -> c_int;
     pub fn ophip_graph_launch(dev: *mut ophip_device, graph: *mut c_void, stream: *mut c_void) -> c_int;

@@ -529,3 +529,31 @@ def test_attention_at_a_decode_shape_with_strided_views_and_separate_layouts(gpu
     v_lay = TensorLayout(dt.F16, [nkvh, att, dh], [dh * 2, nkvh * dh * 2, 2])
     ophip.Attention(gpu).launch(ophip.AttentionArgs(q_lay, qd, kv_lay, kd, v_lay, vtd, o_lay, od, CAUSAL), None, stream)
     assert_close_f16(download(gpu, stream, od, q), ref, "separate layouts vs f64")
+
+
+def test_attention_at_a_decode_shape_with_o_over_other_operands(gpu, stream):
+    """The decode kernel's workgroups (one per kv head and chunk of keys) write o while others still read q, k and v;
+    the reference's composite reads everything before it writes o.  A call whose o lies over v, or over q in another
+    layout, must therefore give what the composite gives: attention over the operands as they were."""
+    rng = np.random.default_rng(123)
+    nh, nkvh, seq, att, dh = 8, 2, 4, 100, 64
+    q, k, v = normal_f16(rng, (nh, seq, dh)), normal_f16(rng, (nkvh, att, dh)), normal_f16(rng, (nkvh, att, dh))
+    ref = attention_f64(q, k, v, True)
+    lay = TensorLayout.of
+    # (a) o at the start of v's buffer
+    say("attention at a decode shape, o over v")
+    qd, kd, vd = upload(gpu, q), upload(gpu, k), upload(gpu, v)
+    ophip.Attention(gpu).launch(ophip.AttentionArgs(lay(q), qd, lay(k), kd, lay(v), vd, lay(q), vd, CAUSAL), None, stream)
+    out = gpu.to_host(vd, np.float16, q.size, stream=stream).reshape(q.shape)
+    assert_close_f16(out, ref, "o over v")
+    # (b) q as a view of a token-major buffer (heads and tokens do not merge: the reference stages it), o contiguous
+    # [nh, seq, dh] over the same bytes
+    say("attention at a decode shape, o over q in another layout")
+    row = nh * dh
+    qkv = np.ascontiguousarray(q.transpose(1, 0, 2).reshape(seq, row))
+    bd, kd, vd = upload(gpu, qkv), upload(gpu, k), upload(gpu, v)
+    q_lay = TensorLayout(dt.F16, [nh, seq, dh], [dh * 2, row * 2, 2])
+    o_lay = TensorLayout.new_contiguous(dt.F16, [nh, seq, dh])
+    ophip.Attention(gpu).launch(ophip.AttentionArgs(q_lay, bd, lay(k), kd, lay(v), vd, o_lay, bd, CAUSAL), None, stream)
+    out = gpu.to_host(bd, np.float16, q.size, stream=stream).reshape(q.shape)
+    assert_close_f16(out, ref, "o over q in another layout")

@@ -222,6 +222,22 @@ def test_rope_shapes(gpu, stream, shape, dtype):
         np.testing.assert_allclose(out, ref, rtol=0, atol=5e-3)  # f32 angles near 4096 rad carry ~ang * 2^-23 of error
 
 
+def test_rope_gives_a_token_the_same_bits_whatever_the_call_holds(gpu, stream):
+    """The host picks another kernel from 4096 tokens on (several tokens per workgroup, one sine / cosine table each):
+    the same tokens at the same positions must come out bit for bit the same on either side of that line, or a
+    prefill cut into chunks would differ from one that is not."""
+    rng = np.random.default_rng(77)
+    for nh, dh in ((8, 128), (16, 64)):
+        t = normal_f16(rng, (4200, nh, dh))
+        pos = rng.integers(0, 100000, 4200).astype(np.uint32)
+        say("rope: 4095 / 4096 / 4200 tokens of %d heads x %d" % (nh, dh))
+        outs = [run_rope(gpu, stream, t[:n].copy(), pos[:n].copy()) for n in (4095, 4096, 4200)]
+        single = run_rope(gpu, stream, t[:7].copy(), pos[:7].copy())
+        assert np.array_equal(outs[0].view(np.uint16), outs[1][:4095].view(np.uint16))
+        assert np.array_equal(outs[1].view(np.uint16), outs[2][:4096].view(np.uint16))
+        assert np.array_equal(single.view(np.uint16), outs[2][:7].view(np.uint16))
+
+
 def test_rope_q_and_k_views_inside_qkv(gpu, stream):
     """Decode layer: q and k are [16, 32, 128] views of one [16, 12288] QKV buffer."""
     rng = np.random.default_rng(2)
@@ -923,14 +939,59 @@ def test_mat_mul_decode_layer_shapes(gpu, stream, name, bt, m, n, k, b_transpose
     b = bfull.swapaxes(-1, -2) if b_transposed else bfull
     c = np.zeros(shape(m, n), f16)
     say("mat_mul decode %s" % name)
-    if name in ("qkv", "gate_up", "qkv_32_rows", "gate_up_48_rows"):
+    if name in ("qkv", "gate_up", "qkv_32_rows", "gate_up_48_rows", "o_proj", "down", "pv"):
         args = ophip.MatMulArgs(TensorLayout.of(c), None, 0.0, TensorLayout.of(a), None, TensorLayout.of(b), None, alpha)
         what = ophip.MatMul(gpu).describe(args)
-        assert what.startswith("skinny") and "paired" in what, what
+        if m <= 16:  # up to 16 rows against an N-contiguous weight: the low-register streaming kernel
+            assert what.startswith("stream"), what
+        else:
+            assert what.startswith("skinny") and "paired" in what, what
     oracle.set_threads(8)
     try:
         out = run_mat_mul(gpu, stream, c, a, b, alpha, 0.0)
         check_mat_mul(out, c, a, b, alpha, 0.0, "decode gemm %s" % name)
+    finally:
+        oracle.set_threads(1)
+
+
+STREAM_CASES = [
+    # m, n, k, batch, beta, forced ranges for the strips on slow granule classes (None: the planner's), column offset of B
+    (16, 22016, 4096, 1, 0.0, None, 0),   # gate/up: the planner cuts the slow strips in two
+    (16, 12288, 4096, 1, 0.0, None, 0),   # qkv: 2 ranges, 3 on the slow strips
+    (16, 12288, 4096, 1, 0.5, 4, 128),    # forced 4, strips shifted by one granule
+    (1, 4096, 4096, 1, 0.0, None, 0),
+    (5, 2056, 1024, 1, 1.0, 3, 256),      # N no multiple of 128: the last strip is partial
+    (16, 1024, 64, 1, 0.0, 2, 0),         # two K-steps, one per range
+    (16, 1024, 32, 1, 0.0, None, 0),      # a single K-step: three of the four waves have nothing to do
+    (9, 640, 11008, 1, 0.0, 11, 384),     # 344 K-steps in 11 ranges
+    (16, 512, 2048, 3, 0.0, 2, 0),        # batched
+    (16, 4096, 4096, 1, 0.0, 0, 0),       # every strip cut alike
+]
+
+
+@pytest.mark.parametrize("m,n,k,bt,beta,slow,shift", STREAM_CASES)
+def test_mat_mul_stream_kernel(gpu, stream, monkeypatch, m, n, k, bt, beta, slow, shift):
+    """gemm_stream (up to 16 rows, N-contiguous weight, K in whole steps of 32): its numbering of (strip, K range) units
+    with the strips of the slow granule classes cut finer, for every alignment of the weight's first strip."""
+    rng = np.random.default_rng(m * 7 + n + k + shift)
+    if slow is not None:
+        monkeypatch.setenv("OPHIP_GEMM_SLOW_SPLIT", str(slow))
+    shape = lambda *s: (bt,) + s if bt > 1 else s
+    a = normal_f16(rng, shape(m, k), std=1.0)
+    wide = normal_f16(rng, shape(k, n + 512 + (-n) % 512), std=0.02)  # rows of whole KiB, at least 512 elements wider than B
+    b = wide[..., shift:shift + n]
+    c = normal_f16(rng, shape(m, n), std=1.0)
+    op = ophip.MatMul(gpu)
+    args = ophip.MatMulArgs(TensorLayout.of(c), None, beta, TensorLayout.of(a), None, TensorLayout.of(b), None, 1.0)
+    what = op.describe(args)
+    say("mat_mul stream %dx%dx%d bt=%d shift=%d: %s" % (m, n, k, bt, shift, what))
+    assert what.startswith("stream"), what
+    oracle.set_threads(8)
+    try:
+        out = run_mat_mul(gpu, stream, c, a, b, 1.0, beta, op=op)
+        check_mat_mul(out, c, a, b, 1.0, beta, "mat_mul stream")
+        again = run_mat_mul(gpu, stream, c, a, b, 1.0, beta, op=op)  # the counters are back at zero
+        assert np.array_equal(out.view(np.uint16), again.view(np.uint16))
     finally:
         oracle.set_threads(1)
 

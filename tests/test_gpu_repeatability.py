@@ -37,6 +37,7 @@ def repeat(gpu, stream, launch, out_mem, nbytes, ws, what):
     (32, 16, 128, 2048, False),    # decode PV: the splits of one strip sit on different XCDs
     (1, 16, 1160, 2048, False),    # ragged last strip, splits on different XCDs
     (2, 40, 512, 1024, True),      # 64-row build, weight stored [N, K]
+    (1, 16, 12288, 4096, False),   # low-register streaming kernel: two K ranges per strip, three on the slow granule classes
 ])
 def test_mat_mul_repeats_bit_for_bit(gpu, stream, bt, m, n, k, b_transposed):
     rng = np.random.default_rng(bt + m + n + k)

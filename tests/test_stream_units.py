@@ -1,0 +1,85 @@
+"""The weight-streaming mat_mul kernel for up to 16 rows (gemm_stream) numbers its workgroups' (strip, K range) units
+with one function that the host and the kernel both compile (operators-rs_amd/csrc/kernels/params.h).  Here it is
+compiled for the CPU and every workgroup of a launch is walked through it: for hand-picked cuts, for what the planner
+chooses on a list of shapes (read back through ophip_mat_mul_describe), and for cuts that must be refused."""
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+import ophip
+from ophip import TensorLayout, dt
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def checker(tmp_path_factory):
+    cxx = shutil.which("g++") or shutil.which("c++")
+    if cxx is None:
+        pytest.skip("no C++ compiler")
+    exe = str(tmp_path_factory.mktemp("units") / "stream_units")
+    res = subprocess.run([cxx, "-std=c++17", "-O1", "-Wall", "-Wextra", "-Werror", "-I",
+                          os.path.join(ROOT, "operators-rs_amd", "csrc", "kernels"),
+                          os.path.join(ROOT, "tests", "c_abi", "stream_units.cpp"), "-o", exe], capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr
+
+    def run(n, k, split_k, k_per_split, mask, split_slow):
+        r = subprocess.run([exe] + [str(v) for v in (n, k, split_k, k_per_split, mask, split_slow)], capture_output=True, text=True)
+        return r.returncode, r.stdout.strip()
+    return run
+
+
+def even_cut(k, split):
+    steps = k // 32
+    sps = -(-steps // split)
+    return -(-steps // sps), sps * 32
+
+
+@pytest.mark.parametrize("n,k,split,mask,slow", [
+    (22016, 4096, 1, 0x22, 2), (12288, 4096, 2, 0, 0), (12288, 4096, 2, 0x22, 3), (12288, 4096, 2, 0x22, 4),
+    (4096, 4096, 8, 0, 0), (4096, 11008, 8, 0x22, 11), (2056, 1024, 1, 0x22, 3), (1024, 64, 1, 0x22, 2), (136, 32, 1, 0xAA, 1),
+    (8, 32, 1, 0, 0), (128256, 4096, 1, 0x22, 2), (36864, 1024, 2, 0, 0), (640, 11008, 1, 0xFF, 43)])
+def test_every_unit_once_and_inside_k(checker, n, k, split, mask, slow):
+    split, kps = even_cut(k, split)
+    rc, out = checker(n, k, split, kps, mask, slow)
+    assert rc == 0 and out.startswith("OK"), out
+
+
+def test_a_cut_with_empty_ranges_is_caught(checker):
+    """128 steps in 24 ranges of 6: ranges 22 and 23 would start past K.  The planner never emits such a cut (it rounds
+    the count to ceil(steps / ceil(steps / n))); the kernel treats such a range as empty; this check names it."""
+    rc, out = checker(12288, 4096, 2, 2048, 0x22, 24)
+    assert rc != 0 and "FAIL" in out, out
+    rc, out = checker(12288, 4096, 24, 192, 0, 0)
+    assert rc != 0 and "FAIL" in out, out
+
+
+SHAPES = [(16, 22016, 4096), (16, 12288, 4096), (16, 4096, 4096), (16, 4096, 11008), (1, 32000, 4096), (8, 128256, 4096),
+          (16, 36864, 1024), (16, 40960, 5120), (3, 1000 * 8, 2048), (16, 128, 2048), (16, 1024, 32), (16, 1024, 64),
+          (5, 2056, 1024), (16, 11008, 4096), (16, 14336, 4096), (16, 28672, 4096), (16, 8192, 8192), (16, 57344, 8192)]
+
+
+@pytest.mark.parametrize("slow_knob", [None, "0", "2", "3", "5", "64"])
+def test_what_the_planner_chooses_numbers_its_units_soundly(checker, monkeypatch, slow_knob):
+    if slow_knob is not None:
+        monkeypatch.setenv("OPHIP_GEMM_SLOW_SPLIT", slow_knob)
+    c = lambda *s: TensorLayout.new_contiguous(dt.F16, list(s))
+    streamed = 0
+    for m, n, k in SHAPES:
+        args = ophip.MatMulArgs(c(m, n), None, 0.0, c(m, k), None, c(k, n), None, 1.0)
+        what = ophip.mat_mul_describe(args)  # no operator: the plan for 256 compute units
+        if not what.startswith("stream"):
+            continue
+        streamed += 1
+        g = re.match(r"stream rows<=16 qN split_k=(\d+)(?: \((\d+) on granule classes 0x([0-9a-f]+)\))?$", what)
+        assert g, what
+        split = int(g.group(1))
+        slow, mask = (int(g.group(2)), int(g.group(3), 16)) if g.group(2) else (0, 0)
+        cut, kps = even_cut(k, split)
+        assert cut == split, (what, cut)
+        rc, out = checker(n, k, split, kps, mask, slow)
+        assert rc == 0 and out.startswith("OK"), (m, n, k, what, out)
+    assert streamed >= 10

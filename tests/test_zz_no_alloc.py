@@ -54,7 +54,8 @@ def test_static_scratch_entry_point_matches_the_ordinary_one(gpu, stream):
         (16, 4096, 4096, None, True),
         (512, 4096, 11008, None, False),  # tile kernel, split K
         (256, 512, 4096, None, True),
-        (16, 22016, 4096, None, False),  # no split: no scratch used
+        (16, 22016, 4096, None, False),  # the strips on slow granule classes in two K ranges, the others whole
+        (40, 22016, 4096, None, False),  # no split: no scratch used
         (7, 24, 40, None, False),        # generic kernel
     ]
     kinds = set()
@@ -62,10 +63,10 @@ def test_static_scratch_entry_point_matches_the_ordinary_one(gpu, stream):
         say("static scratch case %d: %s x %s x %s batch %s B[N,K]=%s" % (i, m, n, k, batch, bk))
         plain, static, what = both_ways(gpu, stream, op, m, n, k, batch, bk, seed=i)
         say("  -> %s" % what)
-        kinds.add(what.split()[0] + (" split" if "split_k=1" not in what and "split_k" in what else ""))
+        kinds.add(what.split()[0] + (" split" if "split_k=1" not in what.replace("split_k=1 (", "") and "split_k" in what else ""))
         assert not np.isnan(plain).any()
         assert np.array_equal(plain.view(np.uint16), static.view(np.uint16)), (i, what)
-    assert {"skinny split", "skinny"} <= kinds and any(w.startswith("tile") and w.endswith("split") for w in kinds), kinds
+    assert {"stream split", "stream", "skinny split", "skinny"} <= kinds and any(w.startswith("tile") and w.endswith("split") for w in kinds), kinds
 
 
 def test_static_scratch_entry_point_refuses_what_does_not_fit(gpu, stream, monkeypatch):
@@ -84,3 +85,35 @@ def test_static_scratch_entry_point_refuses_what_does_not_fit(gpu, stream, monke
     with pytest.raises(ophip.LaunchError) as e:
         op.launch_static(args, stream)
     assert e.value.kind == "ArgsNotSupport" and "static" in str(e.value)
+
+
+def test_static_scratch_entry_point_runs_while_a_stream_records(gpu, stream):
+    """What defines the entry point: it allocates nothing.  A stream that is being recorded into a graph refuses
+    allocations, so the split-K products that need scratch (streaming kernel with arrival counters, tile kernel with
+    the separate sum, and a product without scratch) are recorded through the static entry point, replayed twice and
+    compared with the ordinary entry point's bits."""
+    rng = np.random.default_rng(5)
+    op = ophip.MatMul(gpu)
+    cases = [(16, 4096, 4096), (16, 12288, 4096), (512, 4096, 11008), (7, 24, 40)]
+    prepared = []
+    for m, n, k in cases:
+        a, b, c = normal_f16(rng, (m, k)), normal_f16(rng, (k, n), std=0.05), normal_f16(rng, (m, n))
+        ad, bd, cd = gpu.from_host(a), gpu.from_host(b), gpu.from_host(c)
+        args = ophip.MatMulArgs(TensorLayout.of(c), cd, 0.5, TensorLayout.of(a), ad, TensorLayout.of(b), bd, 0.25)
+        op.launch(args, None, stream)  # warms the operator; its result is what the replays must give
+        want = gpu.to_host(cd, f16, c.size, stream=stream).copy()
+        prepared.append((args, cd, c, want, op.describe(args)))
+    say("static scratch under recording: " + "; ".join(p[4] for p in prepared))
+    stream.begin_capture()
+    for args, cd, c, want, what in prepared:
+        op.launch_static(args, stream)
+    graph = stream.end_capture()
+    for rep in range(2):
+        for args, cd, c, want, what in prepared:  # beta = 0.5 reads C: the original C goes back before every replay
+            gpu.upload(cd, c, stream=stream)
+        stream.synchronize()
+        graph.launch(stream)
+        for args, cd, c, want, what in prepared:
+            got = gpu.to_host(cd, f16, c.size, stream=stream)
+            assert np.array_equal(got.view(np.uint16), want.view(np.uint16)), "replay %d: %s" % (rep, what)
+    graph.destroy()
