@@ -117,7 +117,17 @@ class Layer:
         A["down"] = ("mm", o.MatMulArgs(c(NT, D), d["out"], 0.0, half, d["gu"].ptr, c(DI, D), d["w_d"], 1.0))
         self.order = ["rms_norm_1", "qkv", "rope", "qk_t", "softmax", "pv", "o_proj", "rms_norm_2",
                       "gate_up", "swiglu", "down"]
-        for name in self.order:
+        # The same layer as a runtime built on the crate would run it: the three attention launches replaced by the
+        # crate's own composite attention_kv_cached (which also appends the 16 new k / v rows to the caches at
+        # positions KV - NT .. KV, what the scripted chain leaves out).  q, k and v are views of the qkv rows.
+        self.ops["akv"] = o.AttnKVCached(gpu)
+        kv_new = lambda off: d["qkv"].ptr + off * 2
+        A["attention_kv_cached"] = ("akv", o.AttnKVCachedArgs(
+            qb_lay, kv_new(0), qb_lay, kv_new(D), qb_lay, kv_new(2 * D), ob_lay, d["o"],
+            c(NH, KV, DH), d["k_cache"], c(NH, KV, DH), d["v_cache"], o.AttnMask.CAUSAL, KV - NT))
+        self.order_attention_op = ["rms_norm_1", "qkv", "rope", "attention_kv_cached", "o_proj", "rms_norm_2",
+                                   "gate_up", "swiglu", "down"]
+        for name in self.order + ["attention_kv_cached"]:
             kind, a = A[name]
             self.ops[kind].scheme(a, 64 << 20)
 
@@ -125,10 +135,11 @@ class Layer:
         kind, a = self.args[name]
         self.ops[kind].launch(a, self.d["ws"], stream)
 
-    def step(self, stream, around=None, own=None):
+    def step(self, stream, around=None, own=None, order=None):
         """around: {op: (e0, e1)} records the two events before and after the op's launch; own: {op: (e0, e1)} has
-        the op's kernel record its own begin and end into them (ophip_time_next_launch)."""
-        for name in self.order:
+        the op's kernel record its own begin and end into them (ophip_time_next_launch); order: another sequence of
+        launches than the benchmark's eleven (order_attention_op)."""
+        for name in order or self.order:
             if around and name in around:
                 around[name][0].record(stream)
                 self.launch(name, stream)
@@ -155,6 +166,8 @@ def layer_work():
         "gate_up": gemm(NT, 2 * DI, D),
         "swiglu": (3 * NT * DI * 2, 0),
         "down": gemm(NT, D, DI),
+        # q, o, the new k / v rows read and appended, both caches read once
+        "attention_kv_cached": (2 * NT * NH * DH * 2 + 4 * NT * NH * DH * 2 + 2 * NH * KV * DH * 2, 4 * NH * NT * KV * DH),
     }
     return w
 
@@ -187,7 +200,7 @@ def time_sustained(gpu, stream, fn, seconds=0.3):
 def profiled_traffic():
     """HBM bytes per launch of the dominant kernel, measured with FETCH_SIZE / WRITE_SIZE in separate
     counter runs and kept as text under profiles/ (a counter run cannot share a process with the timing)."""
-    path = os.path.join(ROOT, "profiles", "gemm_skinny_gate_up_pmc.txt")
+    path = os.path.join(ROOT, "profiles", "gemm_stream_gate_up_pmc.txt")
     try:
         for line in open(path):
             if line.startswith("traffic_bytes"):
@@ -785,8 +798,9 @@ def cpu_per_op(oracle, threads):
     return out
 
 
-def cpu_layer_step(oracle, h, threads):
-    """The same operations through the CPU oracle (threads on the axes the reference hands to rayon)."""
+def cpu_layer_step(oracle, h, threads, attention_op=False):
+    """The same operations through the CPU oracle (threads on the axes the reference hands to rayon).  attention_op:
+    the crate's attention_kv_cached composite (on copies of the caches) instead of the three scripted launches."""
     oracle.set_threads(threads)
     xn = oracle.rms_norm(np.empty_like(h["x"]), h["x"], h["w_norm1"], 1e-5)
     qkv = oracle.mat_mul(np.zeros((NT, 3 * D), f16), 0.0, xn, h["w_qkv"], 1.0)
@@ -795,10 +809,16 @@ def cpu_layer_step(oracle, h, threads):
     oracle.rope(qkv[:, D:2 * D].reshape(NT, NH, DH), h["pos"], 1e4)
     oracle.set_threads(threads)
     q = qkv[:, :D].reshape(NT, NH, DH).transpose(1, 0, 2)
-    att = oracle.mat_mul(np.zeros((NH, NT, KV), f16), 0.0, q, h["k_cache"].transpose(0, 2, 1), float(1 / np.sqrt(DH)))
-    oracle.fused_softmax(att, causal=True)
     o = np.zeros((NT, D), f16)
-    oracle.mat_mul(o.reshape(NT, NH, DH).transpose(1, 0, 2), 0.0, att, h["v_cache"], 1.0)
+    if attention_op:
+        k_new = qkv[:, D:2 * D].reshape(NT, NH, DH).transpose(1, 0, 2)
+        v_new = qkv[:, 2 * D:].reshape(NT, NH, DH).transpose(1, 0, 2)
+        oracle.attention_kv_cached(q, k_new, v_new, o.reshape(NT, NH, DH).transpose(1, 0, 2), h["k_cache"].copy(),
+                                   h["v_cache"].copy(), KV - NT, causal=True)
+    else:
+        att = oracle.mat_mul(np.zeros((NH, NT, KV), f16), 0.0, q, h["k_cache"].transpose(0, 2, 1), float(1 / np.sqrt(DH)))
+        oracle.fused_softmax(att, causal=True)
+        oracle.mat_mul(o.reshape(NT, NH, DH).transpose(1, 0, 2), 0.0, att, h["v_cache"], 1.0)
     y = oracle.mat_mul(np.zeros((NT, D), f16), 0.0, o, h["w_o"], 1.0)
     yn = oracle.rms_norm(np.empty_like(y), y, h["w_norm2"], 1e-5)
     gu = oracle.mat_mul(np.zeros((NT, 2 * DI), f16), 0.0, yn, h["w_gu"], 1.0)
@@ -867,8 +887,8 @@ def main():
     # step finds its weights in the 256 MiB Infinity Cache
     layers = [Layer(ophip, gpu, rng, host=(i == 0)) for i in range(2)]
     work = layer_work()
-    layer_bytes = sum(b for b, _ in work.values())
-    layer_flops = sum(f for _, f in work.values())
+    layer_bytes = sum(work[n][0] for n in layers[0].order)
+    layer_flops = sum(work[n][1] for n in layers[0].order)
 
     for i in range(args.warmup):
         layers[i % 2].step(stream)
@@ -903,6 +923,18 @@ def main():
     stream.synchronize()
     graph_ms_per_step = (time.perf_counter() - t0g) * 1e3 / (2 * (args.steps // 2)) if args.steps >= 2 else None
     graph.destroy()
+    # The layer with the crate's composite attention_kv_cached in place of QK^T / softmax / PV (nine launches of the
+    # operator API, ten kernels): what a runtime that calls the crate's attention operator sees.  Reported beside the
+    # headline, which stays BASELINE's eleven-launch chain.
+    for i in range(max(2, args.warmup // 2)):
+        layers[i % 2].step(stream, order=layers[i % 2].order_attention_op)
+    stream.synchronize()
+    t0a = time.perf_counter()
+    for i in range(args.steps):
+        layers[i % 2].step(stream, order=layers[i % 2].order_attention_op)
+    stream.synchronize()
+    attn_ms_per_step = (time.perf_counter() - t0a) * 1e3 / args.steps
+    attn_bytes = sum(work[n][0] for n in layers[0].order_attention_op)
     # For comparison, outside the timed region: two separate event records around the same launch, which read
     # longer by most of what an empty pair of records reads.
     pairs = [(gpu.event(), gpu.event()) for _ in range(20)]
@@ -926,7 +958,7 @@ def main():
     # per-op times inside the layer (back-to-back launches of one op; small ops are cache-resident)
     per_layer = []
     log("decode layer, per op:")
-    for name in layers[0].order:
+    for name in layers[0].order + ["attention_kv_cached"]:
         us = time_launches(gpu, stream, lambda: layers[0].launch(name, stream), args.reps)
         b, f = work[name]
         rec = {"op": name, "us": round(us, 3), "bytes": b, "GBps": round(b / us / 1e3, 1),
@@ -980,8 +1012,13 @@ def main():
         "data": "synthetic",
         "config": {"workload": "llama7b_decode_layer_16tok_kv2048 (BASELINE.json configs[4])",
                    "launches_per_step": len(layers[0].order), "algorithmic_bytes_per_step": layer_bytes,
-                   "flops_per_step": layer_flops, "hbm_frac_of_step": round(layer_bytes / (ms_per_step * 1e-3) / HBM_PEAK, 4)},
-        "roofline": {"bound": "hbm", "kernel": "gemm_skinny (gate/up mat_mul 16x4096 . 4096x22016)",
+                   "flops_per_step": layer_flops, "hbm_frac_of_step": round(layer_bytes / (ms_per_step * 1e-3) / HBM_PEAK, 4),
+                   # the same layer through the crate's own attention_kv_cached operator instead of the three scripted
+                   # attention launches (not the headline: BASELINE.json's chain is the eleven launches above)
+                   "ms_per_step_with_attention_op": round(attn_ms_per_step, 5),
+                   "launches_per_step_with_attention_op": len(layers[0].order_attention_op),
+                   "algorithmic_bytes_per_step_with_attention_op": attn_bytes},
+        "roofline": {"bound": "hbm", "kernel": "gemm_stream_m1 (gate/up mat_mul 16x4096 . 4096x22016)",
                      "achieved": round(dom_bytes / (dom_us * 1e-6) / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(dom_bytes / (dom_us * 1e-6) / HBM_PEAK, 4), "traffic": profiled_traffic(),
                      "us": round(dom_us, 3), "samples": len(own), "algorithmic_bytes": dom_bytes,

@@ -276,6 +276,33 @@ def test_decode_layer_chain_matches_the_oracle_end_to_end(gpu, stream):
     assert np.median(err) <= 1e-3 * scale, np.median(err) / scale
 
 
+def test_decode_layer_chain_with_the_attention_operator_matches_the_oracle_end_to_end(gpu, stream):
+    """The same layer with the crate's composite attention_kv_cached in place of the QK^T / softmax / PV launches (the
+    second figure of the benchmark: nine launches of the operator API): against the oracle's composite on the same
+    seeded weights, and the 16 appended rows of both caches bit for bit."""
+    import bench
+
+    rng = np.random.default_rng(0)
+    layer = bench.Layer(ophip, gpu, rng, host=True)
+    print("decode layer chain through attention_kv_cached, 9 launches", flush=True)
+    layer.step(stream, order=layer.order_attention_op)
+    out = gpu.to_host(layer.d["out"], f16, bench.NT * bench.D, stream=stream).reshape(bench.NT, bench.D)
+    ref = bench.cpu_layer_step(oracle, layer.h, min(oracle.max_threads(), 16), attention_op=True)
+    err = np.abs(out.astype(np.float64) - ref.astype(np.float64))
+    scale = float(np.abs(ref.astype(np.float64)).max())
+    print("decode layer with attention op: max err %.3g, median err %.3g, output scale %.3g" % (err.max(), np.median(err), scale), flush=True)
+    assert err.max() <= 1e-2 * scale, err.max() / scale
+    assert np.median(err) <= 1e-3 * scale, np.median(err) / scale
+    # the caches: rows below KV - NT untouched, the appended rows are the k / v columns of the qkv rows the GPU made
+    nt, d, nh, dh, kv = bench.NT, bench.D, bench.NH, bench.DH, bench.KV
+    qkv = gpu.to_host(layer.d["qkv"], f16, nt * 3 * d, stream=stream).reshape(nt, 3 * d)
+    for name, col in (("k_cache", d), ("v_cache", 2 * d)):
+        cache = gpu.to_host(layer.d[name], f16, nh * kv * dh, stream=stream).reshape(nh, kv, dh)
+        assert np.array_equal(cache[:, :kv - nt], layer.h[name][:, :kv - nt]), name
+        new = qkv[:, col:col + d].reshape(nt, nh, dh).transpose(1, 0, 2)
+        assert np.array_equal(cache[:, kv - nt:].view(np.uint16), new.view(np.uint16)), name
+
+
 # ------------------------------------------------ one pass, prefill shapes ----
 # Where its walk over the keys is shorter than the composite's passes over the score matrix (prefill shapes), attention
 # runs on one kernel that keeps the scores on the chip (attention_prefill.hip).  Same bar as the composite: the oracle's composite and the f64 formula, within the f16 tolerance.
