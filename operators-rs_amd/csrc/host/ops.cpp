@@ -40,15 +40,20 @@ static RmsNormMeta rms_norm_meta(const ophip_rms_norm_args &a) {
     return m;
 }
 
+// The pairs with vector kernels: those of the CPU backend (rms_norm/common_cpu/mod.rs:84-90; anything else is `todo!()`
+// there) and bf16 activations with bf16 or f32 weights.
+static bool rms_norm_tuned_pair(uint64_t dt_a, uint64_t dt_w) {
+    return (dt_a == OPHIP_DT_F16 && (dt_w == OPHIP_DT_F16 || dt_w == OPHIP_DT_F32)) ||
+           (dt_a == OPHIP_DT_BF16 && (dt_w == OPHIP_DT_BF16 || dt_w == OPHIP_DT_F32)) ||
+           (dt_a == OPHIP_DT_F32 && dt_w == OPHIP_DT_F32) || (dt_a == OPHIP_DT_F64 && dt_w == OPHIP_DT_F64);
+}
 static void rms_norm_check_types(uint64_t dt_a, uint64_t dt_w) {
-    // the pairs of the CPU backend (rms_norm/common_cpu/mod.rs:84-90; anything else is `todo!()` there), and bf16
-    // activations with bf16 or f32 weights, which the CUDA backend compiles a kernel for like for any other pair of
-    // named types (rms_norm/cuda/mod.rs:146-147)
-    const bool ok = (dt_a == OPHIP_DT_F16 && (dt_w == OPHIP_DT_F16 || dt_w == OPHIP_DT_F32)) ||
-                    (dt_a == OPHIP_DT_BF16 && (dt_w == OPHIP_DT_BF16 || dt_w == OPHIP_DT_F32)) ||
-                    (dt_a == OPHIP_DT_F32 && dt_w == OPHIP_DT_F32) || (dt_a == OPHIP_DT_F64 && dt_w == OPHIP_DT_F64);
-    if (!ok)
-        throw type_not_support("rms_norm supports (a, w) in {(f16, f16), (f16, f32), (bf16, bf16), (bf16, f32), (f32, f32), (f64, f64)}");
+    // The CUDA backend compiles a kernel for any pair of named types (rms_norm/cuda/mod.rs:117-122): every pair of
+    // f16 / bf16 / f32 is taken here (the pairs without a vector kernel on the element-wise one), and (f64, f64); f64
+    // mixed with a narrower type, which CUDA would compute in f32, and non-floating types are refused.
+    auto narrow = [](uint64_t dt) { return dt == OPHIP_DT_F16 || dt == OPHIP_DT_BF16 || dt == OPHIP_DT_F32; };
+    if (!((narrow(dt_a) && narrow(dt_w)) || (dt_a == OPHIP_DT_F64 && dt_w == OPHIP_DT_F64)))
+        throw type_not_support("rms_norm supports activations and weights of f16, bf16 or f32 in any pairing, and (f64, f64)");
 }
 
 struct RmsKey {
@@ -74,7 +79,7 @@ struct ophip_rms_norm : OpBase {
         return schemes.get_or_insert(key, [&] {
             const std::string base = std::string("rms_norm_") + dt_tag(key.dt_a) + "_" + dt_tag(key.dt_w);
             RmsScheme s{};
-            if (key.dt_a == OPHIP_DT_F64) {  // one kernel only
+            if (key.dt_a == OPHIP_DT_F64 || !rms_norm_tuned_pair(key.dt_a, key.dt_w)) {  // one kernel only
                 s.scalar = dev->kernel("rms_norm", (base + "_scalar").c_str());
                 return s;
             }
@@ -137,7 +142,7 @@ extern "C" int ophip_rms_norm_launch(const ophip_rms_norm *op, const ophip_rms_n
         p.epsilon = args->epsilon;
 
         const size_t vec_elems = 16 / (size_t)unit;
-        const bool vec = m.dt_a != OPHIP_DT_F64 && d % vec_elems == 0 && aligned16(p.y) && aligned16(p.x) && aligned16(p.w) && mult16(nsy) &&
+        const bool vec = s.g64 != nullptr && d % vec_elems == 0 && aligned16(p.y) && aligned16(p.x) && aligned16(p.w) && mult16(nsy) &&
                          mult16(nsx);
         op->dev->make_current();
         if (!vec) {

@@ -278,6 +278,13 @@ RMS_SCALAR(rms_norm_bf16_f32_scalar, bf16, float)
 RMS_SCALAR(rms_norm_f16_f16_scalar, f16, f16)
 RMS_SCALAR(rms_norm_f16_f32_scalar, f16, float)
 RMS_SCALAR(rms_norm_f32_f32_scalar, float, float)
+// The remaining pairs of two- and four-byte floating types, which the reference's CUDA backend would compile a kernel
+// for like for any pair of named types (rms_norm/cuda/mod.rs:117-122) and its CPU backend does not have: the
+// element-wise kernel only, same arithmetic (f32 throughout, one rounding to the activations' type).
+RMS_SCALAR(rms_norm_f16_bf16_scalar, f16, bf16)
+RMS_SCALAR(rms_norm_bf16_f16_scalar, bf16, f16)
+RMS_SCALAR(rms_norm_f32_f16_scalar, float, f16)
+RMS_SCALAR(rms_norm_f32_bf16_scalar, float, bf16)
 
 // f64 rows with f64 weights (rms_norm/common_cpu/mod.rs:84-90 lists the pair): all arithmetic in f64, as the
 // reference's, one workgroup per row.  No vector variant: the hot path is f16.

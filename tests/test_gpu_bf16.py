@@ -91,6 +91,40 @@ def test_rms_norm_bf16_strided_rows_and_scalar_path(gpu, stream):
     assert (out[:, :3] == 0).all() and (out[:, 3 + d:] == 0).all()  # nothing outside the view was written
 
 
+@pytest.mark.parametrize("adt,wdt", [("f16", "bf16"), ("bf16", "f16"), ("f32", "f16"), ("f32", "bf16")])
+@pytest.mark.parametrize("n,d", [(16, 4096), (3, 1001), (64, 24)])
+def test_rms_norm_mixed_activation_and_weight_types(gpu, stream, n, d, adt, wdt):
+    """The pairs of f16 / bf16 / f32 that neither has a vector kernel nor exists in the reference's CPU backend (its CUDA
+    backend compiles rms_norm for any pair of named types, rms_norm/cuda/mod.rs:117-122): parity unpinned against the
+    reference; checked against the formula in f64, within one step of the activations' type."""
+    rng = np.random.default_rng(n * 3 + d)
+    enc = {"f16": lambda v: v.astype(np.float16), "bf16": to_bf16, "f32": lambda v: v.astype(f32)}
+    dec = {"f16": lambda v: v.astype(f64), "bf16": lambda v: from_bf16(v).astype(f64), "f32": lambda v: v.astype(f64)}
+    code = {"f16": dt.F16, "bf16": dt.BF16, "f32": dt.F32}
+    xa, wa = enc[adt](rng.standard_normal((n, d)).astype(f32)), enc[wdt](rng.uniform(0.5, 1.5, d).astype(f32))
+    xd, wd, yd = gpu.from_host(xa), gpu.from_host(wa), gpu.malloc(xa.nbytes)
+    op = ophip.RmsNorm(gpu)
+    args = ophip.RmsNormArgs(L2(code[adt], n, d), yd, L2(code[adt], n, d), xd, TensorLayout(code[wdt], [d], [wa.itemsize]), wd, 1e-5)
+    op.scheme(args, 0)
+    say("rms_norm n=%d d=%d activations %s weights %s" % (n, d, adt, wdt))
+    op.launch(args, None, stream)
+    y = dec[adt](gpu.to_host(yd, xa.dtype, n * d, stream=stream).reshape(n, d))
+    x = dec[adt](xa)
+    ref = (1.0 / np.sqrt((x * x).mean(axis=1, keepdims=True) + 1e-5)) * dec[wdt](wa) * x
+    step = {"f16": 2.0 ** -10, "bf16": 2.0 ** -7, "f32": 2.0 ** -22}[adt]
+    assert (np.abs(y - ref) <= np.abs(ref) * step + 1e-30).all(), np.abs(y - ref).max()
+
+
+def test_rms_norm_refuses_the_pairs_it_has_no_kernel_for(gpu):
+    """f64 mixed with a narrower type (the CUDA backend would compute such a pair in f32) and non-floating types."""
+    op = ophip.RmsNorm(gpu)
+    for adt, wdt in ((dt.F64, dt.F32), (dt.F32, dt.F64), (dt.F16, dt.F64), (dt.F64, dt.BF16), (dt.U32, dt.U32), (dt.F16, dt.I32)):
+        args = ophip.RmsNormArgs(L2(adt, 4, 64), None, L2(adt, 4, 64), None, TensorLayout(wdt, [64], [ophip.dtype_nbytes(wdt)]), None, 1e-5)
+        with pytest.raises(ophip.SchemeError) as e:
+            op.scheme(args, 0)
+        assert e.value.kind == "TypeNotSupport", (adt, wdt)
+
+
 @pytest.mark.parametrize("wdt", ["bf16", "f32"])
 @pytest.mark.parametrize("n,d", [(64, 4096), (3, 1001), (300, 512), (2, 16384), (20000, 1024), (8200, 5120)])
 def test_layer_norm_bf16(gpu, stream, n, d, wdt):

@@ -139,9 +139,9 @@ def test_rms_norm_errors(gpu, stream):
     with pytest.raises(ophip.SchemeError) as e:
         op.scheme(mk(good, L(dt.F32, [4, 256], [1024, 4]), L(dt.F16, [256], [2])), 0)
     assert e.value.kind == "TypeMismatch"
-    # pairs of (activation, weight) types outside the CPU backend's list (rms_norm/common_cpu/mod.rs:84-90, where
-    # they are `todo!()`) and the two bf16 pairs (tests/test_gpu_bf16.py): refused by scheme and launch alike
-    for dta, dtw in [(dt.BF16, dt.F16), (dt.F16, dt.BF16), (dt.F16, dt.F64), (dt.F32, dt.F16), (dt.F64, dt.F32), (dt.U32, dt.U32)]:
+    # f64 mixed with a narrower type and non-floating types (every pairing of f16 / bf16 / f32 has a kernel, tests/test_gpu_bf16.py):
+    # refused by scheme and launch alike
+    for dta, dtw in [(dt.F16, dt.F64), (dt.F64, dt.F32), (dt.F64, dt.BF16), (dt.U32, dt.U32), (dt.F16, dt.I32)]:
         na, nw = ophip.dtype_nbytes(dta), ophip.dtype_nbytes(dtw)
         a = mk(L(dta, [4, 256], [256 * na, na]), L(dta, [4, 256], [256 * na, na]), L(dtw, [256], [nw]))
         with pytest.raises(ophip.SchemeError) as e:
