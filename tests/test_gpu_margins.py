@@ -1,0 +1,94 @@
+"""How close each benchmark configuration sits to its bar, as numbers: for every BASELINE configuration the largest
+absolute error against the oracle, the largest relative error (among elements off by more than f16 eps) and the number
+of outliers by the reference's ErrorCollector rule (common/mod.rs:69-117), printed as one table, written to
+gpurun_out/parity_margins.json when that folder exists, and asserted against the bar (max-abs 2e-3 or rel 1e-2 for f16
+outputs; rel 1e-2 at K = 4096 for f32-accumulated mat_mul, measured against the magnitude a row of the product reaches)."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import ophip
+import oracle
+from helpers import margins_f16, normal_f16
+from test_gpu_ops import run_mat_mul, run_rms_norm, run_rope, run_softmax
+
+pytestmark = pytest.mark.gpu
+f16, f32 = np.float16, np.float32
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_parity_margins_at_the_benchmark_configurations(gpu, stream):
+    import bench
+
+    rows = []
+
+    def note(name, out, ref, mat_mul=False):
+        m = margins_f16(out, ref)
+        if mat_mul:  # relative to the magnitude a row of the product reaches, as check_mat_mul measures it
+            r = np.asarray(ref, np.float64)
+            scale = np.maximum(np.abs(r), np.abs(r).mean() + 1e-6)
+            m["max_rel"] = float((np.abs(np.asarray(out, np.float64) - r) / scale).max())
+        m["config"] = name
+        rows.append(m)
+        print("%-34s max abs %.3g  max rel %.3g  outliers %d / %d" % (name, m["max_abs"], m["max_rel"], m["outliers"], m["elements"]), flush=True)
+        return m
+
+    oracle.set_threads(8)
+    try:
+        rng = np.random.default_rng(0)
+        x = rng.standard_normal((64, 4096)).astype(f32).astype(f16)
+        w = rng.uniform(0.5, 1.5, 4096).astype(f32).astype(f16)
+        note("1 rms_norm [64,4096]", run_rms_norm(gpu, stream, x, w, 1e-5), oracle.rms_norm(np.empty_like(x), x, w, 1e-5))
+
+        rng = np.random.default_rng(0)
+        t = normal_f16(rng, (512, 32, 128))
+        pos = np.arange(512, dtype=np.uint32)
+        note("2a rope [512,32,128]", run_rope(gpu, stream, t, pos), oracle.rope(t.copy(), pos, 1e4))
+
+        for name, shape in (("3p softmax [32,512,512]", (32, 512, 512)), ("3d softmax [32,1,2048]", (32, 1, 2048)),
+                            ("5 softmax [32,16,2048]", (32, 16, 2048))):
+            rng = np.random.default_rng(0)
+            att = normal_f16(rng, shape, std=2.0)
+            note(name, run_softmax(gpu, stream, att), oracle.fused_softmax(att.copy(), causal=True))
+
+        gemms = [("5 qkv 16x4096.4096x12288", 1, 16, 12288, 4096, False, 1.0), ("5 o_proj 16x4096.4096x4096", 1, 16, 4096, 4096, False, 1.0),
+                 ("5 gate_up 16x4096.4096x22016", 1, 16, 22016, 4096, False, 1.0), ("5 down 16x11008.11008x4096", 1, 16, 4096, 11008, False, 1.0),
+                 ("5 qk_t 32x(16x128.128x2048)", 32, 16, 2048, 128, True, float(1.0 / np.sqrt(128.0))),
+                 ("5 pv 32x(16x2048.2048x128)", 32, 16, 128, 2048, False, 1.0)]
+        for name, bt, m, n, k, b_transposed, alpha in gemms:
+            rng = np.random.default_rng(len(name) + n)
+            shape = lambda *s: (bt,) + s if bt > 1 else s
+            if bt > 1:
+                a = normal_f16(rng, shape(m, k), std=1.0 if b_transposed else 0.05)
+                bfull = normal_f16(rng, shape(n, k) if b_transposed else shape(k, n), std=1.0)
+            else:
+                a = normal_f16(rng, shape(m, k), std=1.0)
+                bfull = normal_f16(rng, shape(k, n), std=0.02)
+            b = bfull.swapaxes(-1, -2) if b_transposed else bfull
+            c = np.zeros(shape(m, n), f16)
+            out = run_mat_mul(gpu, stream, c, a, b, alpha, 0.0)
+            ref = oracle.mat_mul(c.copy(), 0.0, a, b, alpha)
+            m_ = note(name, out, ref, mat_mul=True)
+            assert m_["max_rel"] <= 1e-2, (name, m_)
+
+        rng = np.random.default_rng(0)
+        layer = bench.Layer(ophip, gpu, rng, host=True)
+        layer.step(stream)
+        out = gpu.to_host(layer.d["out"], f16, bench.NT * bench.D, stream=stream).reshape(bench.NT, bench.D)
+        ref = bench.cpu_layer_step(oracle, layer.h, 8)
+        e2e = note("5 decode layer, 11 launches", out, ref)
+        scale = float(np.abs(ref.astype(np.float64)).max())
+        e2e["max_abs_over_output_scale"] = e2e["max_abs"] / scale
+        assert e2e["max_abs"] <= 1e-2 * scale
+    finally:
+        oracle.set_threads(1)
+
+    for m in rows[:5]:  # the f16 operators: the bar itself
+        assert m["max_abs"] <= 2e-3 or m["max_rel"] <= 1e-2, m
+        assert m["outliers"] * 1000 <= m["elements"], m
+    out_dir = os.path.join(ROOT, "gpurun_out")
+    if os.path.isdir(out_dir):
+        with open(os.path.join(out_dir, "parity_margins.json"), "w") as f:
+            json.dump(rows, f, indent=1)
