@@ -83,3 +83,28 @@ def test_what_the_planner_chooses_numbers_its_units_soundly(checker, monkeypatch
         rc, out = checker(n, k, split, kps, mask, slow)
         assert rc == 0 and out.startswith("OK"), (m, n, k, what, out)
     assert streamed >= 10
+
+
+def test_the_planner_on_the_decode_layers_products():
+    """What launch() picks for the six GEMMs of the benchmark's decode layer (16 tokens, Llama-7B shapes) and their
+    32- / 48-row siblings, on a device of 256 compute units: the 16-row products against N-contiguous weights on the
+    low-register streaming kernel, about one workgroup per CU, gate/up with its slow strips in two K ranges."""
+    import numpy as np
+
+    f16 = np.float16
+    want = {("qkv", 1, 16, 12288, 4096, False): "stream rows<=16 qN split_k=2",
+            ("o_proj", 1, 16, 4096, 4096, False): "stream rows<=16 qN split_k=8",
+            ("gate_up", 1, 16, 22016, 4096, False): "stream rows<=16 qN split_k=1 (2 on granule classes 0x22)",
+            ("down", 1, 16, 4096, 11008, False): "stream rows<=16 qN split_k=8",
+            ("qk_t", 32, 16, 2048, 128, True): "skinny rows<=16 qK split_k=1",
+            ("pv", 32, 16, 128, 2048, False): "stream rows<=16 qN split_k=4",
+            ("qkv_32_rows", 1, 32, 12288, 4096, False): "skinny rows<=32 qN paired split_k=2",
+            ("gate_up_48_rows", 1, 48, 22016, 4096, False): "skinny rows<=64 qN paired split_k=1",
+            ("ragged_k", 1, 7, 24, 40, False): "skinny rows<=16 qN split_k=1"}
+    for (name, bt, m, n, k, b_transposed), text in want.items():
+        shape = lambda *s: (bt,) + s if bt > 1 else s
+        a, c = np.zeros(shape(m, k), f16), np.zeros(shape(m, n), f16)
+        bfull = np.zeros(shape(n, k) if b_transposed else shape(k, n), f16)
+        b = bfull.swapaxes(-1, -2) if b_transposed else bfull
+        args = ophip.MatMulArgs(TensorLayout.of(c), None, 0.0, TensorLayout.of(a), None, TensorLayout.of(b), None, 1.0)
+        assert ophip.mat_mul_describe(args) == text, (name, ophip.mat_mul_describe(args))

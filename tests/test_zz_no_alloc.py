@@ -56,6 +56,7 @@ def test_static_scratch_entry_point_matches_the_ordinary_one(gpu, stream):
         (256, 512, 4096, None, True),
         (16, 22016, 4096, None, False),  # the strips on slow granule classes in two K ranges, the others whole
         (40, 22016, 4096, None, False),  # no split: no scratch used
+        (16, 49152, 1024, None, False),  # more strips than CUs: the streaming kernel for 16 rows without any cut
         (7, 24, 40, None, False),        # generic kernel
     ]
     kinds = set()
