@@ -296,7 +296,8 @@ GemmPlan make_plan(const ophip_mat_mul_args &args, const ophip_mat_mul_layout &L
                 // instead of three, no tail code; cold weights, 16 rows: 4096 x 22016 35.7 -> 35.5 us, 4096 x 12288 split 2
                 // 21.9 -> 21.1, 4096 x 4096 split 8 11.5 -> 10.9, 11008 x 4096 split 8 20.1 -> 19.5).  Its lane offsets are 32 bits.
                 size_t split_slow = 0;
-                if (knobs.stream && g.mt == 1 && g.qmode == 0 && p.K % 32 == 0 && p.q_sl < ((int64_t)1 << 24) && p.p_si < ((int64_t)1 << 26)) {
+                if (knobs.stream && g.mt == 1 && g.qmode == 0 && p.K % 32 == 0 && p.q_sl > 0 && p.q_sl < ((int64_t)1 << 24) && p.p_si >= 0 &&
+                    p.p_si < ((int64_t)1 << 26)) {  // (unsigned lane offsets: rows of either operand ascend in memory)
                     g.qmode = 4;
                     split_slow = plan_slow_strips(p, ntiles, (size_t)cus, knobs);
                 }
