@@ -108,3 +108,26 @@ def test_the_planner_on_the_decode_layers_products():
         b = bfull.swapaxes(-1, -2) if b_transposed else bfull
         args = ophip.MatMulArgs(TensorLayout.of(c), None, 0.0, TensorLayout.of(a), None, TensorLayout.of(b), None, 1.0)
         assert ophip.mat_mul_describe(args) == text, (name, ophip.mat_mul_describe(args))
+
+
+def test_the_uneven_cut_needs_strips_that_stay_in_their_granule_class():
+    """The slow strips are cut finer only where a strip does stay in one class (or alternates c, c + 4): a weight whose
+    first strip starts on a 256-byte boundary and whose rows are whole KiB apart.  Anything else gets the even cut."""
+    import numpy as np
+
+    f16 = np.float16
+    m, n, k = 16, 22016, 4096
+
+    def what(b_base, row_elems):
+        c, a = np.zeros((m, n), f16), np.zeros((m, k), f16)
+        b_layout = TensorLayout(dt.F16, [k, n], [row_elems * 2, 2])
+        return ophip.mat_mul_describe(ophip.MatMulArgs(TensorLayout.of(c), None, 0.0, TensorLayout.of(a), None, b_layout, b_base, 1.0))
+
+    cut = "stream rows<=16 qN split_k=1 (2 on granule classes 0x22)"
+    even = "stream rows<=16 qN split_k=1"
+    assert what(0x7f0000000000, n) == cut
+    assert what(0x7f0000000000 + 5 * 256, n) == cut          # any granule, as long as it is a whole one
+    assert what(0x7f0000000000 + 128, n) == even             # strips straddle two granules: one odd, one even, always
+    assert what(0x7f0000000000, n + 128) == even             # rows of 172.5 KiB quarters: classes rotate from row to row
+    assert what(0x7f0000000000, n + 512) == cut              # rows of 44 KiB
+    assert what(0x7f0000000000, n + 8) == even
