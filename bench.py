@@ -968,6 +968,9 @@ def main():
             rec["TFLOPs"] = round(f / us / 1e6, 2)
         if b < (256 << 20):
             rec["cache_resident"] = True
+        kind, a = layers[0].args[name]
+        if kind == "mm":
+            rec["kernel"] = layers[0].ops["mm"].describe(a)  # which kernel family and K cut the planner chose
         per_layer.append(rec)
         log("  %-12s %9.2f us %9.1f GB/s %5.1f%% HBM" % (name, us, rec["GBps"], 100 * rec["hbm_frac"]))
 
