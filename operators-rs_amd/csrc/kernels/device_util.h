@@ -18,6 +18,15 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 #define WAVE 64
 
+// Waits until every vector-memory operation the wave has issued is acknowledged (stores included).  Written out where a
+// kernel publishes data to other workgroups: a workgroup-scope fence compiles to no such wait on gfx950.  (A build of
+// the kernels for the host, which the CPU tests run work-item by work-item, has no such instruction: a fence there.)
+#ifdef OPHIP_CPU_SIM
+#define OPHIP_WAIT_VMEM() std::atomic_thread_fence(std::memory_order_seq_cst)
+#else
+#define OPHIP_WAIT_VMEM() asm volatile("s_waitcnt vmcnt(0)" ::: "memory")
+#endif
+
 // Threads per workgroup of every kernel that strides by its workgroup size (the host launches them with exactly this
 // many).  A constant rather than blockDim.x: inside a __device__ function the compiler fetches blockDim.x with a vector
 // load from the implicit arguments and waits for it before the first address is known, which costs a streaming kernel of

@@ -473,7 +473,7 @@ __device__ __forceinline__ void gemm_skinny(const GemmParams &p) {
         // the explicit wait it can overtake them, and a workgroup that arrives last right then sums
         // whatever the buffer held before.
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        OPHIP_WAIT_VMEM();
         __syncthreads();
         uint32_t *counter = reinterpret_cast<uint32_t *>(p.counters) + (size_t)bat * gridDim.x + blockIdx.x;
         if (threadIdx.x == 0) s_last = atomicAdd(counter, 1u) == p.split_k - 1 ? 1u : 0u;
@@ -646,7 +646,7 @@ __device__ __forceinline__ void gemm_stream(const GemmParams &p) {
         partial_store4(r, (uint32_t)(first * 4 + 16), sum[4], sum[5], sum[6], sum[7]);
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    OPHIP_WAIT_VMEM();
     __syncthreads();
     uint32_t *counter = reinterpret_cast<uint32_t *>(p.counters) + (size_t)bat * nstrips + strip;
     if (threadIdx.x == 0) s_last = atomicAdd(counter, 1u) == nsplit - 1 ? 1u : 0u;
