@@ -27,6 +27,16 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 #define OPHIP_WAIT_VMEM() asm volatile("s_waitcnt vmcnt(0)" ::: "memory")
 #endif
 
+// Where a wave reads from LDS what other lanes of the same wave have just stored there, with no workgroup barrier in
+// between: nothing on the GPU, where the LDS operations of a wave complete in the order they were issued for all of
+// its lanes; a meeting point of the wave's lanes in the build of the kernels for the host, which runs the lanes one
+// after another.
+#ifdef OPHIP_CPU_SIM
+#define OPHIP_WAVE_LOCKSTEP() cpusim_wave_sync()
+#else
+#define OPHIP_WAVE_LOCKSTEP() ((void)0)
+#endif
+
 // Threads per workgroup of every kernel that strides by its workgroup size (the host launches them with exactly this
 // many).  A constant rather than blockDim.x: inside a __device__ function the compiler fetches blockDim.x with a vector
 // load from the implicit arguments and waits for it before the first address is known, which costs a streaming kernel of

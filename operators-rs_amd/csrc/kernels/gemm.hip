@@ -215,6 +215,7 @@ __device__ __forceinline__ void gemm_skinny(const GemmParams &p) {
             constexpr int u = decltype(U)::value;
 #pragma unroll
             for (int t = 0; t < 8; ++t) st128(tr + wr_off[t], wbuf[u][t]);
+            OPHIP_WAVE_LOCKSTEP();
 #pragma unroll
             for (int cb = 0; cb < 2; ++cb)
 #pragma unroll

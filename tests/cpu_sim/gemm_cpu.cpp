@@ -12,6 +12,7 @@
 #include "../../operators-rs_amd/csrc/kernels/gemm.hip"
 
 #include <string>
+#include <vector>
 
 static uint16_t to_half_bits(float f) {
     const _Float16 h = (_Float16)f;
@@ -81,9 +82,9 @@ int main(int argc, char **argv) {
 
     if (kernel == "stream") {
         const uint32_t grid = gemm_stream_units(&p, reinterpret_cast<uint64_t>(p.q));
-        cpusim::launch({grid, 1, batch}, {256, 1, 1}, [&] { gemm_stream_m1(p); });
+        cpusim::launch({grid, 1, batch}, {256, 1, 1}, 0, [&] { gemm_stream_m1(p); });
     } else if (kernel == "skinny") {
-        cpusim::launch({nstrips, split_k, batch}, {256, 1, 1}, [&] { gemm_skinny_m1_q0(p); });
+        cpusim::launch({nstrips, split_k, batch}, {256, 1, 1}, 0, [&] { gemm_skinny_m1_q0(p); });
     } else {
         std::printf("unknown kernel\n");
         return 2;
@@ -104,7 +105,7 @@ int main(int argc, char **argv) {
             }
     size_t dirty = 0;
     for (uint32_t c : counters) dirty += c != 0;
-    const uint64_t oor = cpusim::out_of_range_loads().load() + cpusim::out_of_range_stores().load();
+    const uint64_t oor = cpusim::worker().out_of_range_loads + cpusim::worker().out_of_range_stores;
     std::printf("%s M=%u N=%u K=%u batch=%u split=%u mask=%#x slow=%u granule=%u: max err %.3g, %zu bad, %zu counters not back at zero, %llu accesses past a resource's records\n",
                 kernel.c_str(), M, N, K, batch, split_k, mask, split_slow, granule, worst, bad, dirty, (unsigned long long)oor);
     std::free(q_block);

@@ -1,6 +1,6 @@
 """The weight-streaming mat_mul kernels, as they are written, on the CPU.
 
-tests/cpu_sim/hip/hip_runtime.h stands in for the HIP headers: one OS thread per work-item, workgroups one after
+tests/cpu_sim/hip/hip_runtime.h stands in for the HIP headers: every work-item a fiber, workgroups one after
 another, MFMA / shuffles / buffer resources emulated.  tests/cpu_sim/gemm_cpu.cpp compiles
 operators-rs_amd/csrc/kernels/gemm.hip with it for the host, under AddressSanitizer and UndefinedBehaviorSanitizer,
 gives every operand a heap block of exactly its size, launches gemm_stream_m1 (grid from the function the library's
