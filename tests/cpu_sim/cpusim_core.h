@@ -1,12 +1,13 @@
 // The core of the CPU stand-in for the GPU (tests only): runs a kernel launch work-item by work-item.
 //
-// Every work-item of a workgroup is a fiber (its own stack, switched by hand: x86-64 only) of the calling OS thread; workgroups run
-// one after another, in the order x fastest, then y, then z (so the workgroup that is numbered last is the one that
-// "arrives last" at a counter).  A work-item runs until it has to wait for others: at a workgroup barrier or at an
-// operation that crosses the lanes of its wave (a shuffle, an MFMA).  When no work-item can run, the waiting ones are
-// let go: first all that wait at a wave operation (every lane that took part has arrived, since all ran until they
-// had to wait: the lanes that did not arrive are masked out, as the hardware's EXEC mask would have them), otherwise
-// all that wait at the barrier.  A work-item that returns takes part in nothing afterwards.
+// Every work-item of a workgroup is a fiber (its own stack, switched by hand: x86-64 only) of the calling OS thread;
+// workgroups run one after another, by default in the order x fastest, then y, then z (so the workgroup that is
+// numbered last is the one that "arrives last" at a counter; CPUSIM_SCHEDULE chooses other orders of workgroups and
+// of work-items).  A work-item runs until it has to wait for others: at a workgroup barrier or at an operation that
+// crosses the lanes of its wave (a shuffle, an MFMA).  When no work-item can run, the waiting ones are let go: first
+// all that wait at a wave operation (every lane that took part has arrived, since all ran until they had to wait: the
+// lanes that did not arrive are masked out, as the hardware's EXEC mask would have them), otherwise all that wait at
+// the barrier.  A work-item that returns takes part in nothing afterwards.
 //
 // Data crosses lanes through per-wave slots: a lane deposits its operands, waits, reads what the others deposited.
 // Two sets of slots alternate between consecutive operations of a wave, so a lane that is already at the next
@@ -95,6 +96,25 @@ struct Worker {
     }
 };
 
+struct Schedule {
+    enum Kind { Forward, Reverse, Shuffle } kind = Forward;
+    uint64_t seed = 0;
+};
+inline const Schedule &schedule() {
+    static const Schedule s = [] {
+        Schedule out;
+        const char *e = std::getenv("CPUSIM_SCHEDULE");
+        if (e && std::strcmp(e, "reverse") == 0) out.kind = Schedule::Reverse;
+        else if (e && std::strncmp(e, "shuffle", 7) == 0) out.kind = Schedule::Shuffle, out.seed = e[7] == ':' ? std::strtoull(e + 8, nullptr, 0) : 1;
+        else if (e && *e && std::strcmp(e, "forward") != 0) {
+            std::fprintf(stderr, "cpusim: CPUSIM_SCHEDULE=%s is none of forward, reverse, shuffle[:seed]\n", e);
+            std::abort();
+        }
+        return out;
+    }();
+    return s;
+}
+
 inline Worker &worker() {
     static thread_local Worker w;
     return w;
@@ -160,8 +180,27 @@ inline void run_workgroup(Worker &w, uint32_t threads) {
         it->sp = prepare_stack(it->stack, STACK_BYTES, item_entry);
     }
     for (auto &ws : w.waves) ws.generation = 0;
+    const Schedule &sch = schedule();
+    uint64_t rnd = sch.seed * 0x9E3779B97F4A7C15ull + w.workgroups;
     for (;;) {
-        for (uint32_t t = 0; t < threads; ++t) {
+        // The order in which the runnable work-items get their turn: a correct kernel gives the same result for every
+        // order (between barriers the hardware interleaves waves as it likes).  CPUSIM_SCHEDULE=reverse or
+        // shuffle:<seed> (a new order of the waves, and a rotation of the lanes inside them, on every pass) tests that.
+        uint32_t wave_xor = 0, lane_rot = 0;
+        bool backwards = sch.kind == Schedule::Reverse;
+        if (sch.kind == Schedule::Shuffle) {
+            rnd = rnd * 6364136223846793005ull + 1442695040888963407ull;
+            wave_xor = (uint32_t)(rnd >> 33), lane_rot = (uint32_t)(rnd >> 40) % WAVE_LANES, backwards = (rnd >> 60) & 1;
+        }
+        const uint32_t nwaves = threads / WAVE_LANES;
+        uint32_t wave_mask = 1;
+        while (wave_mask < nwaves) wave_mask <<= 1;
+        wave_mask -= 1;
+        for (uint32_t n = 0; n < (wave_mask + 1) * WAVE_LANES; ++n) {
+            const uint32_t m = backwards ? (wave_mask + 1) * WAVE_LANES - 1 - n : n;
+            const uint32_t wv = (m / WAVE_LANES) ^ (wave_xor & wave_mask);
+            if (wv >= nwaves) continue;
+            const uint32_t t = wv * WAVE_LANES + (m % WAVE_LANES + lane_rot) % WAVE_LANES;
             Item *it = w.items[t];
             if (it->state != ItemState::Runnable) continue;
             w.cur = it;
@@ -229,13 +268,29 @@ inline void launch(Dim3u grid, Dim3u block, size_t dynamic_lds_bytes, const std:
     w.body = &body;
     (void)dynamic_lds_bytes;  // dynamic LDS is a thread-local array of the module, of the largest size a launch may ask for
     w.launches++;
-    for (uint32_t bz = 0; bz < grid.z; ++bz)
-        for (uint32_t by = 0; by < grid.y; ++by)
-            for (uint32_t bx = 0; bx < grid.x; ++bx) {
-                w.block_idx = Dim3u{bx, by, bz};
-                w.workgroups++;
-                run_workgroup(w, threads);
+    // Workgroups in ascending order (x fastest); backwards under CPUSIM_SCHEDULE=reverse, in a pseudo-random order under
+    // shuffle: a kernel must not depend on which workgroup runs first or last.
+    const Schedule &sch = schedule();
+    const uint64_t total = (uint64_t)grid.x * grid.y * grid.z;
+    uint64_t mul = 1, add = 0;
+    if (sch.kind == Schedule::Shuffle && total > 2) {
+        auto gcd = [](uint64_t a, uint64_t b) {
+            while (b) {
+                const uint64_t t = a % b;
+                a = b, b = t;
             }
+            return a;
+        };
+        mul = (sch.seed * 2654435761ull + w.launches * 40503ull) % total;
+        while (mul < 2 || gcd(mul, total) != 1) mul = (mul + 1) % total;
+        add = (sch.seed + 7 * w.launches) % total;
+    }
+    for (uint64_t n = 0; n < total; ++n) {
+        uint64_t b = sch.kind == Schedule::Reverse ? total - 1 - n : (uint64_t)((unsigned __int128)n * mul % total + add) % total;
+        w.block_idx = Dim3u{(uint32_t)(b % grid.x), (uint32_t)(b / grid.x % grid.y), (uint32_t)(b / ((uint64_t)grid.x * grid.y))};
+        w.workgroups++;
+        run_workgroup(w, threads);
+    }
     w.body = nullptr;
 }
 

@@ -54,3 +54,32 @@ def test_gpu_tests_against_the_host_build(sim_library, test_file):
     tail = (r.stdout + r.stderr)[-6000:]
     assert r.returncode == 0, tail
     assert ("%d passed" % len(ids)) in tail, tail  # none skipped, none deselected
+
+
+def hand_over_tests():
+    """The selected tests of kernels in which workgroups or waves hand data to each other (K ranges of a product, key
+    ranges of attention, the passes of sampling, rows spread over waves)."""
+    words = ("split_k", "stream", "decode", "kv_cached", "one_pass", "sample", "softmax")
+    return [t for ids in selection().values() for t in ids if any(w in t for w in words)]
+
+
+@pytest.mark.parametrize("schedule", ["shuffle:5"])  # ("reverse" is the other order the stand-in knows)
+def test_results_do_not_depend_on_the_order_of_workgroups_and_waves(sim_library, schedule):
+    """Between barriers the hardware runs workgroups and waves in any order it likes.  The stand-in runs them in a fixed
+    one by default; here backwards, and in a pseudo-random order that changes at every point where work-items wait for
+    each other.  The same tests must pass (several of them compare bit for bit)."""
+    ids = hand_over_tests()
+    assert len(ids) > 50
+    env = dict(os.environ, OPHIP_CPU_SIM_LIBRARY=sim_library, CPUSIM_SCHEDULE=schedule)
+    cmd = [sys.executable, "-m", "pytest", "-m", "gpu", "-q", "-p", "no:cacheprovider", "--timeout", "300", "-n", "4"] + ids
+    r = subprocess.run(cmd, cwd=ROOT, env=env, capture_output=True, text=True, timeout=1500)
+    tail = (r.stdout + r.stderr)[-6000:]
+    assert r.returncode == 0 and ("%d passed" % len(ids)) in tail, tail
+
+
+def test_smoke_against_the_host_build(sim_library):
+    """__graft_entry__.smoke(), the check that runs on the GPU box before the benchmark, line by line on the stand-in."""
+    code = ("import sys; sys.path[:0] = [%r, %r]; import ophip; ophip.LIB_PATH = %r; import __graft_entry__; __graft_entry__.smoke()"
+            % (ROOT, os.path.join(ROOT, "operators-rs_amd"), sim_library))
+    r = subprocess.run([sys.executable, "-c", code], cwd=ROOT, capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0 and "smoke ok" in r.stdout, r.stdout + r.stderr
