@@ -7,7 +7,10 @@ For each code object of the library's Makefile (KERNELS) one translation unit is
 source inside a namespace of the module and registers every `extern "C" __global__` function it defines (found by
 preprocessing the source with __global__ defined to a marker).  Objects are rebuilt when the text they are made from changes.
 
-    python tests/cpu_sim/build_sim.py [out_dir]      (default tests/cpu_sim/_build)
+    python tests/cpu_sim/build_sim.py [out_dir [sanitizers]]      (default tests/cpu_sim/_build, none)
+
+With sanitizers (e.g. `undefined`: UndefinedBehaviorSanitizer needs no preloading, so python can load the result) the
+host sources are compiled here as well, with the same checks, instead of taking the Makefile's objects.
 """
 import concurrent.futures
 import hashlib
@@ -73,8 +76,12 @@ def compile_if_stale(cxx, flags, src, obj, preprocessed_text):
     return True
 
 
-def build_module(cxx, out_dir, name, source, defines):
-    flags = DEVICE_FLAGS + defines
+def sanitizer_flags(sanitize):
+    return ["-g", "-fsanitize=" + sanitize, "-fno-sanitize-recover=all", "-shared-libsan"] if sanitize else []
+
+
+def build_module(cxx, out_dir, name, source, defines, sanitize=None):
+    flags = DEVICE_FLAGS + defines + sanitizer_flags(sanitize)
     marked = run([cxx] + flags + ["-D__global__=CPUSIM_GLOBAL_MARK", "-E", "-P", source])
     kernels = re.findall(r"CPUSIM_GLOBAL_MARK\s+void\s+(\w+)\s*\(", marked)
     if not kernels:
@@ -95,7 +102,7 @@ def build_module(cxx, out_dir, name, source, defines):
     return obj, compile_if_stale(cxx, flags, tu, obj, marked + text), len(kernels)
 
 
-def build(out_dir=None, jobs=8, verbose=False):
+def build(out_dir=None, jobs=8, verbose=False, sanitize=None):
     out_dir = out_dir or os.path.join(HERE, "_build")
     os.makedirs(out_dir, exist_ok=True)
     cxx = compiler()
@@ -104,10 +111,20 @@ def build(out_dir=None, jobs=8, verbose=False):
     # the library's host objects, as its own Makefile builds them
     run(["make", "-C", CSRC, "-j%d" % jobs])
     host = [os.path.join(CSRC, "build", n + ".o") for n in HOST_OBJECTS]
+    if sanitize:  # the host sources too, from source (static_scratch.hip as plain C++: its device array becomes a host array)
+        flags = (["-std=c++17", "-O1", "-fPIC", "-D__HIP_PLATFORM_AMD__", "-I", os.path.join(ROOT, "include"), "-I", os.path.join(ROCM, "include")]
+                 + sanitizer_flags(sanitize))
+        host = []
+        for n in HOST_OBJECTS:
+            src = os.path.join(CSRC, "host", n + (".hip" if n == "static_scratch" else ".cpp"))
+            extra = ["-x", "c++", "-include", os.path.join(HERE, "static_scratch_host.h")] if n == "static_scratch" else []
+            obj = os.path.join(out_dir, "host_%s.o" % n)
+            compile_if_stale(cxx, flags + extra, src, obj, run([cxx] + flags + extra + ["-E", "-P", src]))
+            host.append(obj)
     mods = modules()
     objs = []
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
-        futures = [pool.submit(build_module, cxx, out_dir, *m) for m in mods]
+        futures = [pool.submit(build_module, cxx, out_dir, *m, sanitize) for m in mods]
         for (name, _, _), f in zip(mods, futures):
             obj, rebuilt, count = f.result()
             if verbose:
@@ -120,15 +137,21 @@ def build(out_dir=None, jobs=8, verbose=False):
             + "};\nextern const unsigned ophip_embedded_module_count = %d;\n}\n" % len(mods))
     if not os.path.exists(table) or open(table).read() != text:
         open(table, "w").write(text)
-    host_flags = ["-std=c++20", "-O1", "-g", "-fPIC", "-D__HIP_PLATFORM_AMD__", "-I", os.path.join(ROCM, "include"), "-I", HERE]
+    host_flags = ["-std=c++20", "-O1", "-g", "-fPIC", "-D__HIP_PLATFORM_AMD__", "-I", os.path.join(ROCM, "include"), "-I", HERE] + sanitizer_flags(sanitize)
     runtime_src = os.path.join(HERE, "sim_runtime.cpp")
     runtime_text = open(runtime_src).read() + open(os.path.join(HERE, "cpusim_core.h")).read()
     compile_if_stale(cxx, host_flags, runtime_src, os.path.join(out_dir, "sim_runtime.o"), runtime_text)
     compile_if_stale(cxx, host_flags, table, os.path.join(out_dir, "sim_modules.o"), text)
     lib = os.path.join(out_dir, "libophip_cpusim.so")
-    run([cxx, "-shared", "-o", lib] + host + objs + [os.path.join(out_dir, "sim_runtime.o"), os.path.join(out_dir, "sim_modules.o"), "-lpthread"])
+    rpath = []
+    if sanitize:  # where the sanitizer's shared runtime lives
+        probe = run([cxx, "-print-file-name=libclang_rt.ubsan_standalone-x86_64.so"]).strip()
+        if os.path.isabs(probe):
+            rpath = ["-Wl,-rpath," + os.path.dirname(os.path.realpath(probe))]
+    run([cxx, "-shared", "-o", lib] + sanitizer_flags(sanitize) + rpath + host + objs
+        + [os.path.join(out_dir, "sim_runtime.o"), os.path.join(out_dir, "sim_modules.o"), "-lpthread"])
     return lib
 
 
 if __name__ == "__main__":
-    print(build(sys.argv[1] if len(sys.argv) > 1 else None, verbose=True))
+    print(build(sys.argv[1] if len(sys.argv) > 1 else None, verbose=True, sanitize=sys.argv[2] if len(sys.argv) > 2 else None))

@@ -231,7 +231,12 @@ void __hipRegisterFunction(void **, const void *, char *, const char *, unsigned
 hipError_t hipGetSymbolAddress(void **ptr, const void *symbol) {
     std::lock_guard<std::recursive_mutex> lock(g_mu);
     auto it = g_symbols.find(symbol);
-    if (it == g_symbols.end() || !ptr) return hipErrorInvalidSymbol;
+    if (!ptr || !symbol) return hipErrorInvalidSymbol;
+    if (it == g_symbols.end()) {
+        // nobody registered it: the file that owns the array was compiled as plain C++ (the sanitizer build), the array is a host array
+        *ptr = const_cast<void *>(symbol);
+        return hipSuccess;
+    }
     if (!it->second.storage) {
         if (sim_malloc(&it->second.storage, it->second.size) != hipSuccess) return hipErrorOutOfMemory;
         std::memset(it->second.storage, 0, it->second.size);  // a device array without an initializer is zero when its module is loaded

@@ -15,6 +15,7 @@ selection.txt lists test ids that take a few seconds at most here (the large sha
 by running every GPU test this way once and keeping the fast ones (tests/cpu_sim/select_tests.py).
 """
 import os
+import shutil
 import subprocess
 import sys
 
@@ -83,3 +84,18 @@ def test_smoke_against_the_host_build(sim_library):
             % (ROOT, os.path.join(ROOT, "operators-rs_amd"), sim_library))
     r = subprocess.run([sys.executable, "-c", code], cwd=ROOT, capture_output=True, text=True, timeout=600)
     assert r.returncode == 0 and "smoke ok" in r.stdout, r.stdout + r.stderr
+
+
+def test_c_consumer_against_the_host_build(sim_library, tmp_path):
+    """tests/c_abi/consumer.c (the ABI used from C11 as a binding of another language would use it: create, scheme,
+    launch, compare with plain C) linked against the host build instead of libophip.so."""
+    cc = shutil.which("gcc") or shutil.which("cc")
+    if cc is None:
+        pytest.skip("no C compiler")
+    exe, libdir = str(tmp_path / "consumer"), os.path.dirname(sim_library)
+    cmd = [cc, "-std=c11", "-O1", "-Wall", "-Wextra", "-Werror", "-pedantic", "-I", os.path.join(ROOT, "include"),
+           os.path.join(ROOT, "tests", "c_abi", "consumer.c"), "-o", exe, "-L", libdir, "-lophip_cpusim", "-lm", "-Wl,-rpath," + libdir]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr
+    res = subprocess.run([exe], capture_output=True, text=True, timeout=600)
+    assert res.returncode == 0 and res.stdout.strip().endswith("ok"), (res.returncode, res.stdout, res.stderr)
