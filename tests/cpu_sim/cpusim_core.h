@@ -31,6 +31,13 @@ extern "C" void __sanitizer_start_switch_fiber(void **fake_stack_save, const voi
 extern "C" void __sanitizer_finish_switch_fiber(void *fake_stack_save, const void **bottom_old, size_t *size_old);
 extern "C" void __asan_unpoison_memory_region(void const volatile *addr, size_t size);
 #endif
+#if __has_feature(thread_sanitizer)
+#define CPUSIM_TSAN 1
+extern "C" void *__tsan_get_current_fiber(void);
+extern "C" void *__tsan_create_fiber(unsigned flags);
+extern "C" void __tsan_destroy_fiber(void *fiber);
+extern "C" void __tsan_switch_to_fiber(void *fiber, unsigned flags);
+#endif
 #endif
 
 namespace cpusim {
@@ -74,6 +81,7 @@ struct Item {
     ItemState state = ItemState::Done;
     char *stack = nullptr;
     void *asan_fake = nullptr;
+    void *tsan_fiber = nullptr;
 };
 
 struct Worker {
@@ -81,6 +89,7 @@ struct Worker {
     std::vector<WaveSlots> waves;
     void *sched_sp = nullptr;
     void *asan_fake = nullptr;
+    void *tsan_sched = nullptr;
     const void *sched_stack = nullptr;
     size_t sched_stack_size = 0;
     Item *cur = nullptr;
@@ -125,6 +134,9 @@ inline void to_scheduler() {
     Item *it = w.cur;
 #ifdef CPUSIM_ASAN
     __sanitizer_start_switch_fiber(it->state == ItemState::Done ? nullptr : &it->asan_fake, w.sched_stack, w.sched_stack_size);
+#endif
+#ifdef CPUSIM_TSAN
+    __tsan_switch_to_fiber(w.tsan_sched, 0);
 #endif
     switch_stack(&it->sp, w.sched_sp);
 #ifdef CPUSIM_ASAN
@@ -178,8 +190,15 @@ inline void run_workgroup(Worker &w, uint32_t threads) {
         __asan_unpoison_memory_region(it->stack, STACK_BYTES);  // what the stack's last user left poisoned
 #endif
         it->sp = prepare_stack(it->stack, STACK_BYTES, item_entry);
+#ifdef CPUSIM_TSAN
+        if (it->tsan_fiber) __tsan_destroy_fiber(it->tsan_fiber);
+        it->tsan_fiber = __tsan_create_fiber(0);
+#endif
     }
     for (auto &ws : w.waves) ws.generation = 0;
+#ifdef CPUSIM_TSAN
+    w.tsan_sched = __tsan_get_current_fiber();
+#endif
     const Schedule &sch = schedule();
     uint64_t rnd = sch.seed * 0x9E3779B97F4A7C15ull + w.workgroups;
     for (;;) {
@@ -206,6 +225,9 @@ inline void run_workgroup(Worker &w, uint32_t threads) {
             w.cur = it;
 #ifdef CPUSIM_ASAN
             __sanitizer_start_switch_fiber(&w.asan_fake, it->stack, STACK_BYTES);
+#endif
+#ifdef CPUSIM_TSAN
+            __tsan_switch_to_fiber(it->tsan_fiber, 0);
 #endif
             switch_stack(&w.sched_sp, it->sp);
 #ifdef CPUSIM_ASAN

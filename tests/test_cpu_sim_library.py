@@ -99,3 +99,48 @@ def test_c_consumer_against_the_host_build(sim_library, tmp_path):
     assert res.returncode == 0, res.stderr
     res = subprocess.run([exe], capture_output=True, text=True, timeout=600)
     assert res.returncode == 0 and res.stdout.strip().endswith("ok"), (res.returncode, res.stdout, res.stderr)
+
+
+def build_threads_driver(library, exe, extra=()):
+    sys.path.insert(0, SIM)
+    try:
+        import build_sim
+    finally:
+        sys.path.remove(SIM)
+    libdir = os.path.dirname(library)
+    cmd = [build_sim.compiler(), "-std=c++17", "-O1", "-g", "-pthread", "-I", os.path.join(ROOT, "include"), os.path.join(SIM, "threads_driver.cpp"),
+           "-o", exe, "-L", libdir, "-lophip_cpusim", "-Wl,-rpath," + libdir] + list(extra)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr
+
+
+def test_one_device_and_its_operators_shared_by_several_threads(sim_library, tmp_path):
+    """tests/cpu_sim/threads_driver.cpp: four threads launch through one device, one rms_norm and one mat_mul operator,
+    each on a stream of its own, while operators and streams come and go; every result equals the single-threaded one."""
+    exe = str(tmp_path / "threads_driver")
+    build_threads_driver(sim_library, exe)
+    res = subprocess.run([exe, "4", "8"], capture_output=True, text=True, timeout=600)
+    assert res.returncode == 0 and res.stdout.strip().endswith("ok"), (res.returncode, res.stdout, res.stderr)
+
+
+@pytest.mark.skipif(not os.environ.get("OPHIP_TEST_SANITIZERS"), reason="a second and third build of the stand-in, minutes each: set OPHIP_TEST_SANITIZERS=1")
+def test_under_thread_and_undefined_behaviour_sanitizers(tmp_path):
+    """The same threaded program against a ThreadSanitizer build of the stand-in and of the library's host sources (a
+    data race in the host side ends the run), and the smoke check against an UndefinedBehaviorSanitizer build (which
+    python can load: it needs no preloading).  Both builds are kept under tests/cpu_sim/_build_*."""
+    sys.path.insert(0, SIM)
+    try:
+        import build_sim
+    finally:
+        sys.path.remove(SIM)
+    tsan = build_sim.build(os.path.join(SIM, "_build_thread"), sanitize="thread")
+    exe = str(tmp_path / "threads_driver_tsan")
+    runtime = os.path.dirname(subprocess.run([build_sim.compiler(), "-print-file-name=libclang_rt.tsan-x86_64.so"], capture_output=True, text=True).stdout.strip())
+    build_threads_driver(tsan, exe, ["-fsanitize=thread", "-shared-libsan", "-Wl,-rpath," + runtime])
+    res = subprocess.run([exe, "6", "8"], capture_output=True, text=True, timeout=1200)
+    assert res.returncode == 0 and res.stdout.strip().endswith("ok") and "ThreadSanitizer" not in res.stderr, (res.returncode, res.stdout, res.stderr[-4000:])
+    ubsan = build_sim.build(os.path.join(SIM, "_build_undefined"), sanitize="undefined")
+    code = ("import sys; sys.path[:0] = [%r, %r]; import ophip; ophip.LIB_PATH = %r; import __graft_entry__; __graft_entry__.smoke()"
+            % (ROOT, os.path.join(ROOT, "operators-rs_amd"), ubsan))
+    r = subprocess.run([sys.executable, "-c", code], cwd=ROOT, capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0 and "smoke ok" in r.stdout, r.stdout + r.stderr
