@@ -78,10 +78,17 @@ def test_parity_margins_at_the_benchmark_configurations(gpu, stream):
         layer.step(stream)
         out = gpu.to_host(layer.d["out"], f16, bench.NT * bench.D, stream=stream).reshape(bench.NT, bench.D)
         ref = bench.cpu_layer_step(oracle, layer.h, 8)
+        # Eleven f16 roundings in a row, the GEMMs summing in another order than the oracle: element by element the two
+        # chains drift apart by a few f16 steps of the largest outputs, so the per-operator outlier rule says nothing
+        # here.  What is asserted: the largest error against the largest output, and the rms error against the rms output.
         e2e = note("5 decode layer, 11 launches", out, ref)
-        scale = float(np.abs(ref.astype(np.float64)).max())
+        r64, o64 = ref.astype(np.float64), out.astype(np.float64)
+        scale = float(np.abs(r64).max())
         e2e["max_abs_over_output_scale"] = e2e["max_abs"] / scale
+        e2e["rms_error_over_rms_output"] = float(np.sqrt(np.mean((o64 - r64) ** 2)) / np.sqrt(np.mean(r64 ** 2)))
+        print("%-34s max abs / largest output %.3g  rms error / rms output %.3g" % ("", e2e["max_abs_over_output_scale"], e2e["rms_error_over_rms_output"]), flush=True)
         assert e2e["max_abs"] <= 1e-2 * scale
+        assert e2e["rms_error_over_rms_output"] <= 1e-2
     finally:
         oracle.set_threads(1)
 
