@@ -98,7 +98,12 @@ hipError_t sim_malloc(void **ptr, size_t size) {
     install_fault_handler();
     const size_t user_len = (std::max<size_t>(size, 1) + 255) / 256 * 256;
     const size_t body = (user_len + 4095) / 4096 * 4096, map_len = body + 2 * 4096;
-    if (g_live_bytes + body > ((size_t)24 << 30)) return hipErrorOutOfMemory;  // keep a runaway test from taking the machine's memory
+    // keep a runaway test from taking the machine's memory: 24 GiB of live allocations, or CPUSIM_MEMORY_GIB
+    static const size_t cap = [] {
+        const char *e = std::getenv("CPUSIM_MEMORY_GIB");
+        return (size_t)(e && std::atoi(e) > 0 ? std::atoi(e) : 24) << 30;
+    }();
+    if (g_live_bytes + body > cap) return hipErrorOutOfMemory;
     char *m = static_cast<char *>(mmap(nullptr, map_len, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS, -1, 0));
     if (m == MAP_FAILED) return hipErrorOutOfMemory;
     mprotect(m, 4096, PROT_NONE);

@@ -1,0 +1,210 @@
+"""The streaming operators on tensors larger than 2^32 bytes (and 2^31 elements): what a card with 288 GB invites.
+
+An offset kept in 32 bits, or an element index in a signed int, works at every benchmark shape and wraps here.  Each
+tensor is a [n, d] f16 matrix of about 4.6 GiB whose rows all differ from the rows an address that wrapped by 2^31 or
+2^32 bytes or elements would hit instead (row r is row r mod 8191 of a random base block, with a sign and a scale that
+depend on r), filled on the device in 64 MiB pieces; the operator runs once over the whole tensor; rows are read back
+around every such boundary, at both ends and at random places, and compared with the oracle on the same rows.
+"""
+import numpy as np
+import pytest
+
+import ophip
+import oracle
+from helpers import assert_close_f16
+from ophip import TensorLayout, dt
+
+pytestmark = pytest.mark.gpu
+f16, f32 = np.float16, np.float32
+PERIOD = 8191  # rows of the base block: prime, so no power-of-two distance maps a row onto an equal one
+
+
+def say(msg):
+    print(msg, flush=True)
+
+
+class Big:
+    """An [n, d] f16 tensor on the device whose rows can be regenerated on the host one by one."""
+
+    def __init__(self, gpu, n, d, seed, fill=True):
+        self.gpu, self.n, self.d = gpu, n, d
+        rng = np.random.default_rng(seed)
+        self.base = rng.standard_normal((PERIOD, d)).astype(f32).astype(f16)
+        self.mem = gpu.malloc(n * d * 2)
+        if fill:
+            step = PERIOD * max(1, (64 << 20) // (PERIOD * d * 2))  # pieces of about 64 MiB
+            for r0 in range(0, n, step):
+                gpu.upload(self.mem, self.rows(np.arange(r0, min(n, r0 + step))), offset=r0 * d * 2)
+
+    def rows(self, idx):
+        idx = np.asarray(idx, dtype=np.int64)
+        factor = np.where((idx // PERIOD) % 2 == 0, 1.0, -1.0) * (1.0 + ((idx // (2 * PERIOD)) % 4) * 0.25)
+        return (self.base[idx % PERIOD] * factor[:, None].astype(f16)).astype(f16)
+
+    def fetch(self, stream, idx):
+        return np.stack([self.gpu.to_host(self.mem, f16, self.d, offset=int(r) * self.d * 2, stream=stream) for r in idx])
+
+    def layout(self):
+        return TensorLayout.new_contiguous(dt.F16, [self.n, self.d])
+
+
+def sample_rows(n, d, seed=0):
+    rows = {0, 1, 2, n - 1, n - 2, n // 2}
+    for boundary in (2 ** 31, 2 ** 32, 2 ** 33):  # bytes, then elements
+        for per_row in (d * 2, d):
+            r = boundary // per_row
+            rows.update(x for x in (r - 2, r - 1, r, r + 1) if 0 <= x < n)
+    rows.update(int(x) for x in np.random.default_rng(seed).integers(0, n, 24))
+    return np.array(sorted(rows))
+
+
+SHAPES = {"wide rows": (600000, 4096), "narrow rows": (1200000, 2048)}  # 4.58 GiB either way
+
+
+@pytest.mark.parametrize("shape", sorted(SHAPES))
+def test_rms_norm_and_layer_norm_past_4_gib(gpu, stream, shape):
+    n, d = SHAPES[shape]
+    say("rms_norm, layer_norm [%d, %d] f16" % (n, d))
+    x, y = Big(gpu, n, d, 1), Big(gpu, n, d, 2, fill=False)
+    rng = np.random.default_rng(3)
+    w, b = rng.uniform(0.5, 1.5, d).astype(f32).astype(f16), rng.uniform(-0.5, 0.5, d).astype(f32).astype(f16)
+    wd, bd = gpu.from_host(w), gpu.from_host(b)
+    vec = TensorLayout.new_contiguous(dt.F16, [d])
+    idx = sample_rows(n, d)
+    xs = x.rows(idx)
+    ophip.RmsNorm(gpu).launch(ophip.RmsNormArgs(y.layout(), y.mem, x.layout(), x.mem, vec, wd, 1e-5), None, stream)
+    assert_close_f16(y.fetch(stream, idx), oracle.rms_norm(np.empty_like(xs), xs, w, 1e-5), "rms_norm past 4 GiB")
+    ophip.LayerNorm(gpu).launch(ophip.LayerNormArgs(y.layout(), y.mem, x.layout(), x.mem, vec, wd, vec, bd, 1e-5), None, stream)
+    assert_close_f16(y.fetch(stream, idx), oracle.layer_norm(np.empty_like(xs), xs, w, b, 1e-5), "layer_norm past 4 GiB")
+
+
+def test_swiglu_gelu_and_add_past_4_gib(gpu, stream):
+    n, d = SHAPES["narrow rows"]
+    say("swiglu, gelu, add [%d, %d] f16" % (n, d))
+    gate, up, out = Big(gpu, n, d, 4), Big(gpu, n, d, 5), Big(gpu, n, d, 6, fill=False)
+    idx = sample_rows(n, d)
+    gs, us = gate.rows(idx), up.rows(idx)
+    ophip.Add(gpu).launch(ophip.AddArgs(out.layout(), out.mem, gate.layout(), gate.mem, up.layout(), up.mem), None, stream)
+    assert np.array_equal(out.fetch(stream, idx).view(np.uint16), (gs + us).view(np.uint16)), "add past 4 GiB"
+    ophip.Swiglu(gpu).launch(ophip.SwigluArgs(gate.layout(), gate.mem, up.layout(), up.mem), None, stream)
+    assert_close_f16(gate.fetch(stream, idx), oracle.swiglu(gs.copy(), us), "swiglu past 4 GiB")
+    ophip.Gelu(gpu).launch(ophip.GeluArgs(up.layout(), up.mem), None, stream)
+    assert_close_f16(up.fetch(stream, idx), oracle.gelu(us.copy()), "gelu past 4 GiB")
+
+
+def test_rope_and_softmax_past_4_gib(gpu, stream):
+    n, d = SHAPES["wide rows"]
+    nh, dh = d // 128, 128
+    say("rope [%d, %d, %d], softmax [%d, 8, %d] f16" % (n, nh, dh, n // 8, d))
+    t = Big(gpu, n, d, 7)
+    pos = (np.arange(n, dtype=np.uint64) * 7 % 4099).astype(np.uint32)
+    pd = gpu.from_host(pos)
+    idx = sample_rows(n, d)
+    ts = t.rows(idx)
+    empty = TensorLayout(dt.F16, [0, dh], [2 * dh, 2])
+    ophip.Rope(gpu).launch(ophip.RopeArgs(TensorLayout.new_contiguous(dt.F16, [n, nh, dh]), t.mem, TensorLayout.new_contiguous(dt.U32, [n]), pd,
+                                          empty, None, empty, None, 1e4), None, stream)
+    ref = oracle.rope(ts.reshape(len(idx), nh, dh).copy(), pos[idx], 1e4).reshape(len(idx), d)
+    assert_close_f16(t.fetch(stream, idx), ref, "rope past 4 GiB")
+    # the same memory as n rows of d scores (what rope left there: the reference result, up to the bar)
+    before = t.fetch(stream, idx)
+    ophip.FusedSoftmax(gpu).launch(ophip.FusedSoftmaxArgs(ophip.AttnMask.NONE, TensorLayout.new_contiguous(dt.F16, [n // 8, 8, d]), t.mem), None, stream)
+    ref = oracle.fused_softmax(before.copy().reshape(len(idx), 1, d), causal=False).reshape(len(idx), d)
+    assert_close_f16(t.fetch(stream, idx), ref, "softmax past 4 GiB")
+
+
+def test_rearrange_past_4_gib(gpu, stream):
+    """[n / 16, 16, d] -> [16, n / 16, d]: whole rows move across the 4 GiB line in both directions."""
+    n, d = SHAPES["narrow rows"]
+    say("rearrange [%d, 16, %d] -> [16, %d, %d] f16" % (n // 16, d, n // 16, d))
+    src, dst = Big(gpu, n, d, 8), Big(gpu, n, d, 9, fill=False)
+    s0 = n // 16
+    ophip.Rearrange(gpu).launch(ophip.RearrangeArgs(TensorLayout(dt.F16, [s0, 16, d], [d * 2, s0 * d * 2, 2]), dst.mem,
+                                                    TensorLayout.new_contiguous(dt.F16, [s0, 16, d]), src.mem), None, stream)
+    idx = sample_rows(n, d)  # rows of the destination: row j * s0 + i holds the source's row i * 16 + j
+    assert np.array_equal(dst.fetch(stream, idx).view(np.uint16), src.rows((idx % s0) * 16 + idx // s0).view(np.uint16)), "rearrange past 4 GiB"
+
+
+def rel_error(got, ref):
+    """against the magnitude a row of the product reaches, as the mat_mul parity tests measure it"""
+    err = np.abs(got - ref)
+    return float((err / np.maximum(np.abs(ref), np.abs(ref).mean())).max())
+
+
+def test_mat_mul_weight_past_4_gib(gpu, stream):
+    """c[16, N] = a[16, K] . W[K, N] with a 4.5 GiB weight (the decode-shaped product of a very wide layer):
+    W[k, j] = T[(7 k + 13 j) mod L] for a random table T, so that any (k, j) the kernel might read instead differs."""
+    m, k, n, L = 16, 16384, 147456, 1000003
+    say("mat_mul 16 x %d . %d x %d f16" % (k, k, n))
+    rng = np.random.default_rng(10)
+    table = (rng.standard_normal(L).astype(f32) * f32(0.05)).astype(f16)
+    w = gpu.malloc(k * n * 2)
+    jj = np.arange(n, dtype=np.int64) * 13
+    for k0 in range(0, k, 256):
+        kk = np.arange(k0, min(k, k0 + 256), dtype=np.int64) * 7
+        gpu.upload(w, table[(kk[:, None] + jj[None, :]) % L], offset=k0 * n * 2)
+    a = rng.standard_normal((m, k)).astype(f32).astype(f16)
+    ad, cd = gpu.from_host(a), gpu.malloc(m * n * 2)
+    lay = lambda r, c: TensorLayout.new_contiguous(dt.F16, [1, r, c])
+    op = ophip.MatMul(gpu)
+    args = ophip.MatMulArgs(lay(m, n), cd, 0.0, lay(m, k), ad, lay(k, n), w, 1.0)
+    say("  kernel: " + op.describe(args))
+    op.launch(args, None, stream)
+    got = gpu.to_host(cd, f16, m * n, stream=stream).reshape(m, n)
+    cols = np.array(sorted({0, 1, n - 2, n - 1} | {int(x) for x in rng.integers(0, n, 96)}
+                           | {(b // 2) % n + o for b in (2 ** 31, 2 ** 32, 2 ** 33) for o in (-1, 0, 1)}), dtype=np.int64)
+    cols = cols[(cols >= 0) & (cols < n)]
+    wc = table[(np.arange(k, dtype=np.int64)[:, None] * 7 + cols[None, :] * 13) % L].astype(np.float64)
+    assert rel_error(got[:, cols].astype(np.float64), a.astype(np.float64) @ wc) <= 1e-2
+
+
+def test_mat_mul_rows_past_4_gib(gpu, stream):
+    """C[M, 128] = A[M, 2048] . B[2048, 128] with a 4.6 GiB A (a long prefill batch through a narrow projection)."""
+    m, k, n = 1200000, 2048, 128
+    say("mat_mul %d x %d . %d x %d f16" % (m, k, k, n))
+    a = Big(gpu, m, k, 11)
+    rng = np.random.default_rng(12)
+    b = (rng.standard_normal((k, n)).astype(f32) * f32(0.05)).astype(f16)
+    bd, cd = gpu.from_host(b), gpu.malloc(m * n * 2)
+    lay = lambda r, c: TensorLayout.new_contiguous(dt.F16, [1, r, c])
+    op = ophip.MatMul(gpu)
+    args = ophip.MatMulArgs(lay(m, n), cd, 0.0, lay(m, k), a.mem, lay(k, n), bd, 1.0)
+    say("  kernel: " + op.describe(args))
+    op.launch(args, None, stream)
+    idx = sample_rows(m, k)
+    got = np.stack([gpu.to_host(cd, f16, n, offset=int(r) * n * 2, stream=stream) for r in idx]).astype(np.float64)
+    assert rel_error(got, a.rows(idx).astype(np.float64) @ b.astype(np.float64)) <= 1e-2
+
+
+def test_attention_kv_cached_caches_past_4_gib(gpu, stream):
+    """40 heads of 480000 cached tokens of 128 (4.6 GiB for either cache), ten new tokens appended at the end: the
+    appended rows are read back, and every head's result is compared with softmax(q k^T / sqrt(dh)) v in f64."""
+    nh = nkvh = 40
+    seq, dh, buf = 10, 128, 480000
+    pos = buf - seq
+    say("attention_kv_cached nh=%d seq=%d dh=%d buf=%d pos=%d" % (nh, seq, dh, buf, pos))
+    kc, vc = Big(gpu, nkvh * buf, dh, 13), Big(gpu, nkvh * buf, dh, 14)
+    rng = np.random.default_rng(15)
+    q, k, v = (rng.standard_normal(s).astype(f32).astype(f16) for s in ((nh, seq, dh), (nkvh, seq, dh), (nkvh, seq, dh)))
+    qd, kd, vd, od = gpu.from_host(q), gpu.from_host(k), gpu.from_host(v), gpu.malloc(q.nbytes)
+    c = lambda *shape: TensorLayout.new_contiguous(dt.F16, list(shape))
+    op = ophip.AttnKVCached(gpu)
+    args = ophip.AttnKVCachedArgs(c(nh, seq, dh), qd, c(nkvh, seq, dh), kd, c(nkvh, seq, dh), vd, c(nh, seq, dh), od,
+                                  c(nkvh, buf, dh), kc.mem, c(nkvh, buf, dh), vc.mem, ophip.AttnMask.CAUSAL, pos)
+    op.scheme(args, 2 ** 40)
+    op.launch(args, None, stream)
+    out = gpu.to_host(od, f16, q.size, stream=stream).reshape(q.shape)
+    for h in (0, nkvh // 2, nkvh - 1):  # the appended rows, where the caches start, cross 4 GiB and end
+        rows = np.arange(h * buf + pos, h * buf + pos + seq)
+        assert np.array_equal(kc.fetch(stream, rows), k[h]) and np.array_equal(vc.fetch(stream, rows), v[h])
+        before = np.arange(h * buf + pos - 2, h * buf + pos)
+        assert np.array_equal(kc.fetch(stream, before), kc.rows(before)) and np.array_equal(vc.fetch(stream, before), vc.rows(before))
+    for h in range(nh):
+        rows = np.arange(h * buf, h * buf + pos)
+        keys = np.concatenate([kc.rows(rows), k[h]]).astype(np.float64)
+        vals = np.concatenate([vc.rows(rows), v[h]]).astype(np.float64)
+        scores = q[h].astype(np.float64) @ keys.T / np.sqrt(dh)
+        for i in range(seq):
+            scores[i, pos + i + 1:] = -np.inf
+        p = np.exp(scores - scores.max(axis=1, keepdims=True))
+        assert_close_f16(out[h], (p / p.sum(axis=1, keepdims=True)) @ vals, "attention_kv_cached past 4 GiB, head %d" % h)
