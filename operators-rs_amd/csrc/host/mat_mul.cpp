@@ -525,6 +525,8 @@ struct ophip_mat_mul {
 // arrival counters owned by the operator).  Otherwise the caller of this function brings every byte of scratch:
 // `workspace` holds the f32 partials, `fixed_counters` the arrival counters (all zero between launches: zero when the
 // caller made them, and every kernel leaves the ones it used at zero), and nothing is allocated.
+constexpr size_t GRID_Z_MAX = 65535;
+
 static void mat_mul_launch_impl(const ophip_mat_mul *op, const ophip_mat_mul_args *args, void *workspace,
                                 size_t workspace_len, const ophip_queue_alloc *qa, void *fixed_counters,
                                 size_t fixed_counter_count, hipStream_t stream) {
@@ -533,8 +535,28 @@ static void mat_mul_launch_impl(const ophip_mat_mul *op, const ophip_mat_mul_arg
     if (!mat_mul_takes(L.dt)) throw type_not_support("mat_mul supports f16, bf16, f32 and f64");
     if (is_dyn(args->alpha) || is_dyn(args->beta)) throw dyn_not_support("");
     if (L.m == 0 || L.n == 0 || L.batch == 0) return;
-    if (L.m > 0x7fffffffu || L.n > 0x7fffffffu || L.k > 0x7fffffffu || L.batch > 65535)
-        throw shape_not_support("mat_mul dimension too large");
+    if (L.m > 0x7fffffffu || L.n > 0x7fffffffu || L.k > 0x7fffffffu) throw shape_not_support("mat_mul dimension too large");
+    if (L.batch > GRID_Z_MAX) {
+        // The batch rides on the grid's z extent, which ends at 65535 (cuBLAS, which the reference calls, takes any
+        // count): the same product in as many launches as that needs, each on its share of the batches.
+        for (size_t b0 = 0; b0 < L.batch; b0 += GRID_Z_MAX) {
+            const size_t nb = std::min<size_t>(GRID_Z_MAX, L.batch - b0);
+            ophip_mat_mul_args sub = *args;
+            size_t shapes[3][3];
+            auto cut = [&](ophip_tensor_layout &lay, size_t (&shape)[3]) -> ptrdiff_t {
+                if (lay.ndim != 3 || lay.shape[0] == 1) return 0;  // one matrix shared by every batch
+                std::copy(lay.shape, lay.shape + 3, shape);
+                shape[0] = nb;
+                lay.shape = shape;
+                return (ptrdiff_t)b0 * lay.strides[0];
+            };
+            sub.c_base = static_cast<char *>(args->c_base) + cut(sub.c_layout, shapes[0]);
+            sub.a_base = static_cast<const char *>(args->a_base) + cut(sub.a_layout, shapes[1]);
+            sub.b_base = static_cast<const char *>(args->b_base) + cut(sub.b_layout, shapes[2]);
+            mat_mul_launch_impl(op, &sub, workspace, workspace_len, qa, fixed_counters, fixed_counter_count, stream);
+        }
+        return;
+    }
     GemmPlan g = make_plan(*args, L, (unsigned)op->dev->props.multiProcessorCount, op->knobs);
     const GemmParams &p = g.p;
     const bool fixed = fixed_counters != nullptr;

@@ -910,6 +910,22 @@ def test_mat_mul_reference_shapes(gpu, stream, m):
         oracle.set_threads(1)
 
 
+@pytest.mark.parametrize("shared_b", [False, True])
+def test_mat_mul_more_batches_than_a_grid_holds(gpu, stream, shared_b):
+    """65538 small products in one call (cuBLAS, which the reference calls at mat_mul/cuda/mod.rs:96-126, takes any batch
+    count; a grid's z extent ends at 65535): the call goes out in two launches, the second on the last three batches."""
+    rng = np.random.default_rng(7)
+    bt, m, n, k = 65538, 3, 8, 16
+    a = normal_f16(rng, (bt, m, k))
+    b = normal_f16(rng, (1 if shared_b else bt, k, n))
+    c = normal_f16(rng, (bt, m, n))
+    say("mat_mul batch %d of %dx%dx%d, b %s" % (bt, m, n, k, "shared" if shared_b else "per batch"))
+    out = run_mat_mul(gpu, stream, c, a, b, 0.5, 1.0)
+    ref = (0.5 * a.astype(np.float64) @ b.astype(np.float64) + c.astype(np.float64))
+    assert_close_f16(out, ref.astype(f16), "mat_mul 65538 batches")
+    assert_close_f16(out[-3:], ref[-3:].astype(f16), "the batches of the second launch")
+
+
 DECODE_GEMMS = [
     ("qkv", 1, 16, 12288, 4096, False),
     ("o_proj", 1, 16, 4096, 4096, False),
