@@ -497,7 +497,9 @@ OPHIP_API void ophip_attention_kv_cached_destroy(ophip_attention_kv_cached *op);
 
 /* ---- layer_norm: layer_norm/args.rs:7-55 ----------------------------------- */
 /* y[n,d] = (x - mean) * scale / (std + epsilon) + bias, std = sqrt(mean(x^2) - mean^2)
- * (layer_norm/common_cpu/mod.rs:127-147).  (scale/bias, x/y) in {(f16,f16), (f32,f16), (f32,f32)}. */
+ * (layer_norm/common_cpu/mod.rs:127-147).  (scale/bias, x/y): any pairing of f16, bf16 and f32, and (f64, f64)
+ * (the CPU backend lists (f16,f16), (f32,f16), (f32,f32), (f64,f64); layer_norm/cuda/mod.rs:158-159 takes any pair of
+ * named types). */
 typedef struct ophip_layer_norm_args {
     ophip_tensor_layout y_layout;
     void *y_base;

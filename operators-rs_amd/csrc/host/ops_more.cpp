@@ -83,13 +83,16 @@ extern "C" int ophip_layer_norm_launch(const ophip_layer_norm *op, const ophip_l
         const ptrdiff_t nsx = static_of(args->x_layout.strides[0]), dsx = static_of(args->x_layout.strides[1]);
         const ptrdiff_t dss = static_of(args->scale_layout.strides[0]), dsb = static_of(args->bias_layout.strides[0]);
         const bool f64 = m.dt_a == OPHIP_DT_F64 && m.dt_w == OPHIP_DT_F64;
-        // the CPU backend's pairs (layer_norm/common_cpu/mod.rs:94-97), and bf16 rows with bf16 or f32 parameters, which
-        // the CUDA backend compiles a kernel for like for any other named types (layer_norm/cuda/mod.rs:158-159)
-        const bool ok = (m.dt_a == OPHIP_DT_F16 && (m.dt_w == OPHIP_DT_F16 || m.dt_w == OPHIP_DT_F32)) ||
-                        (m.dt_a == OPHIP_DT_BF16 && (m.dt_w == OPHIP_DT_BF16 || m.dt_w == OPHIP_DT_F32)) ||
-                        (m.dt_a == OPHIP_DT_F32 && m.dt_w == OPHIP_DT_F32) || f64;
-        if (!ok)
-            throw type_not_support("layer_norm supports (scale, x) in (f16,f16), (f32,f16), (bf16,bf16), (f32,bf16), (f32,f32), (f64,f64)");
+        // The pairs with vector kernels: the CPU backend's (layer_norm/common_cpu/mod.rs:94-97), and bf16 rows with bf16
+        // or f32 parameters.  The CUDA backend compiles a kernel for any pair of named types
+        // (layer_norm/cuda/mod.rs:158-159): every other pairing of f16 / bf16 / f32 runs on the element-wise kernel;
+        // f64 mixed with a narrower type and non-floating types are refused.
+        const bool tuned = (m.dt_a == OPHIP_DT_F16 && (m.dt_w == OPHIP_DT_F16 || m.dt_w == OPHIP_DT_F32)) ||
+                           (m.dt_a == OPHIP_DT_BF16 && (m.dt_w == OPHIP_DT_BF16 || m.dt_w == OPHIP_DT_F32)) ||
+                           (m.dt_a == OPHIP_DT_F32 && m.dt_w == OPHIP_DT_F32);
+        auto narrow = [](uint64_t dt) { return dt == OPHIP_DT_F16 || dt == OPHIP_DT_BF16 || dt == OPHIP_DT_F32; };
+        if (!((narrow(m.dt_a) && narrow(m.dt_w)) || f64))
+            throw type_not_support("layer_norm supports rows and parameters of f16, bf16 or f32 in any pairing, and (f64, f64)");
         const ptrdiff_t unit = (ptrdiff_t)ophip_dtype_nbytes(m.dt_a), wunit = (ptrdiff_t)ophip_dtype_nbytes(m.dt_w);
         if (dsy != unit || dsx != unit || dss != wunit || dsb != wunit)
             throw strides_not_support("layer_norm needs contiguous inner dimensions");
@@ -109,7 +112,7 @@ extern "C" int ophip_layer_norm_launch(const ophip_layer_norm *op, const ophip_l
         p.epsilon = args->epsilon;
         const std::string base = std::string("layer_norm_") + dt_tag(m.dt_a) + "_" + dt_tag(m.dt_w);
         const size_t vec_elems = 16 / (size_t)unit;
-        const bool vec = !f64 && d % vec_elems == 0 && aligned16(p.y) && aligned16(p.x) && aligned16(p.scale) &&
+        const bool vec = tuned && d % vec_elems == 0 && aligned16(p.y) && aligned16(p.x) && aligned16(p.scale) &&
                          aligned16(p.bias) && mult16(nsy) && mult16(nsx);
         if (!p.y || !p.x || !p.scale || !p.bias) throw args_not_support("null base address");
         op->dev->make_current();

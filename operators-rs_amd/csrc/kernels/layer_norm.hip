@@ -316,6 +316,14 @@ LAYER_NORM(f32_f32, float, float)
 LAYER_NORM(bf16_bf16, bf16, bf16)
 LAYER_NORM(bf16_f32, bf16, float)
 
+// The remaining pairs of two- and four-byte floating types, which the reference's CUDA backend would compile a kernel
+// for like for any pair of named types (layer_norm/cuda/mod.rs:158-159) and its CPU backend does not have: the
+// element-wise kernel only, same arithmetic (f32 throughout, one rounding to the rows' type).
+extern "C" __global__ void __launch_bounds__(256) layer_norm_f16_bf16_scalar(LayerNormParams p) { layer_norm_scalar<f16, bf16>(p); }
+extern "C" __global__ void __launch_bounds__(256) layer_norm_bf16_f16_scalar(LayerNormParams p) { layer_norm_scalar<bf16, f16>(p); }
+extern "C" __global__ void __launch_bounds__(256) layer_norm_f32_f16_scalar(LayerNormParams p) { layer_norm_scalar<float, f16>(p); }
+extern "C" __global__ void __launch_bounds__(256) layer_norm_f32_bf16_scalar(LayerNormParams p) { layer_norm_scalar<float, bf16>(p); }
+
 // f64 rows with f64 scale and bias (layer_norm/common_cpu/mod.rs:97 lists the pair): all arithmetic in f64, as the
 // reference's, one workgroup per row.  No vector variant: the hot path is f16.
 extern "C" __global__ void __launch_bounds__(256) layer_norm_f64_f64_scalar(LayerNormParams p) {

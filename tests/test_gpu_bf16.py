@@ -156,6 +156,46 @@ def test_layer_norm_bf16(gpu, stream, n, d, wdt):
     assert (np.abs(y - ref) <= one_step(ref) + slack).all(), (np.abs(y - ref) - one_step(ref) - slack).max()
 
 
+@pytest.mark.parametrize("adt,wdt", [("f16", "bf16"), ("bf16", "f16"), ("f32", "f16"), ("f32", "bf16")])
+@pytest.mark.parametrize("n,d", [(16, 4096), (3, 1001), (64, 24)])
+def test_layer_norm_mixed_row_and_parameter_types(gpu, stream, n, d, adt, wdt):
+    """The pairs of f16 / bf16 / f32 that have no vector kernel and do not exist in the reference's CPU backend (its CUDA
+    backend compiles layer_norm for any pair of named types, layer_norm/cuda/mod.rs:158-159): parity unpinned against
+    the reference; checked against the formula in f64 (the reference's: the standard deviation plus epsilon)."""
+    rng = np.random.default_rng(n * 5 + d)
+    enc = {"f16": lambda v: v.astype(np.float16), "bf16": to_bf16, "f32": lambda v: v.astype(f32)}
+    dec = {"f16": lambda v: v.astype(f64), "bf16": lambda v: from_bf16(v).astype(f64), "f32": lambda v: v.astype(f64)}
+    code = {"f16": dt.F16, "bf16": dt.BF16, "f32": dt.F32}
+    xa = enc[adt](rng.standard_normal((n, d)).astype(f32) * f32(1.5) + f32(0.25))
+    sa, ba = enc[wdt](rng.uniform(0.5, 1.5, d).astype(f32)), enc[wdt](rng.uniform(-1, 1, d).astype(f32))
+    xd, sd, bd, yd = gpu.from_host(xa), gpu.from_host(sa), gpu.from_host(ba), gpu.malloc(xa.nbytes)
+    wl = TensorLayout(code[wdt], [d], [sa.itemsize])
+    op = ophip.LayerNorm(gpu)
+    args = ophip.LayerNormArgs(L2(code[adt], n, d), yd, L2(code[adt], n, d), xd, wl, sd, wl, bd, 1e-5)
+    op.scheme(args, 0)
+    say("layer_norm n=%d d=%d rows %s parameters %s" % (n, d, adt, wdt))
+    op.launch(args, None, stream)
+    y = dec[adt](gpu.to_host(yd, xa.dtype, n * d, stream=stream).reshape(n, d))
+    x, s, b = dec[adt](xa), dec[wdt](sa), dec[wdt](ba)
+    e = x.mean(axis=1, keepdims=True)
+    k = 1.0 / (np.sqrt((x * x).mean(axis=1, keepdims=True) - e * e) + 1e-5)
+    ref = (x - e) * (s * k) + b
+    step = {"f16": 2.0 ** -10, "bf16": 2.0 ** -7, "f32": 2.0 ** -18}[adt]
+    slack = (np.abs(x - e) * np.abs(s) * k + np.abs(b)) * 2.0 ** -18 + (2.0 ** -24 if adt == "f16" else 1e-30)
+    assert (np.abs(y - ref) <= np.abs(ref) * step + slack).all(), (np.abs(y - ref) - np.abs(ref) * step - slack).max()
+
+
+def test_layer_norm_refuses_the_pairs_it_has_no_kernel_for(gpu, stream):
+    """f64 mixed with a narrower type and non-floating types."""
+    op = ophip.LayerNorm(gpu)
+    for adt, wdt in ((dt.F64, dt.F32), (dt.F32, dt.F64), (dt.F16, dt.F64), (dt.U32, dt.U32), (dt.F16, dt.I32)):
+        wl = TensorLayout(wdt, [64], [ophip.dtype_nbytes(wdt)])
+        args = ophip.LayerNormArgs(L2(adt, 4, 64), None, L2(adt, 4, 64), None, wl, None, wl, None, 1e-5)
+        with pytest.raises(ophip.LaunchError) as e:
+            op.launch(args, None, stream)
+        assert e.value.kind == "TypeNotSupport", (adt, wdt)
+
+
 @pytest.mark.parametrize("shape", [(16, 4096), (3, 5, 7), (1,), (2, 1000, 33), (4100, 8192)])
 def test_add_bf16_every_bit(gpu, stream, shape):
     rng = np.random.default_rng(sum(shape))

@@ -101,7 +101,7 @@ def test_layer_norm_errors(gpu, stream):
         op.scheme(ophip.LayerNormArgs(c(F, 4, 8), None, c(F, 8), None, c(W, 8), None, c(W, 8), None, 1e-5), 0)
     assert e.value.kind == "RankNotSupport"
     with pytest.raises(ophip.LaunchError) as e:
-        op.launch(ophip.LayerNormArgs(c(W, 4, 8), None, c(W, 4, 8), None, c(F, 8), None, c(F, 8), None, 1e-5), None,
+        op.launch(ophip.LayerNormArgs(c(dt.F64, 4, 8), None, c(dt.F64, 4, 8), None, c(F, 8), None, c(F, 8), None, 1e-5), None,
                   stream)
     assert e.value.kind == "TypeNotSupport"
 
