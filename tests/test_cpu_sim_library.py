@@ -123,11 +123,12 @@ def test_one_device_and_its_operators_shared_by_several_threads(sim_library, tmp
     assert res.returncode == 0 and res.stdout.strip().endswith("ok"), (res.returncode, res.stdout, res.stderr)
 
 
-@pytest.mark.skipif(not os.environ.get("OPHIP_TEST_SANITIZERS"), reason="a second and third build of the stand-in, minutes each: set OPHIP_TEST_SANITIZERS=1")
-def test_under_thread_and_undefined_behaviour_sanitizers(tmp_path):
+@pytest.mark.skipif(not os.environ.get("OPHIP_TEST_SANITIZERS"), reason="three more builds of the stand-in, minutes each: set OPHIP_TEST_SANITIZERS=1")
+def test_under_thread_address_and_undefined_behaviour_sanitizers(tmp_path):
     """The same threaded program against a ThreadSanitizer build of the stand-in and of the library's host sources (a
-    data race in the host side ends the run), and the smoke check against an UndefinedBehaviorSanitizer build (which
-    python can load: it needs no preloading).  Both builds are kept under tests/cpu_sim/_build_*."""
+    data race in the host side ends the run), against an AddressSanitizer build with leak detection, and the smoke check
+    against an UndefinedBehaviorSanitizer build (which python can load: it needs no preloading).  The builds are kept
+    under tests/cpu_sim/_build_*."""
     sys.path.insert(0, SIM)
     try:
         import build_sim
@@ -139,6 +140,13 @@ def test_under_thread_and_undefined_behaviour_sanitizers(tmp_path):
     build_threads_driver(tsan, exe, ["-fsanitize=thread", "-shared-libsan", "-Wl,-rpath," + runtime])
     res = subprocess.run([exe, "6", "8"], capture_output=True, text=True, timeout=1200)
     assert res.returncode == 0 and res.stdout.strip().endswith("ok") and "ThreadSanitizer" not in res.stderr, (res.returncode, res.stdout, res.stderr[-4000:])
+    # the same program under AddressSanitizer with leak detection: heap errors in the host side, and operators, streams
+    # and devices that do not give back what they took
+    asan = build_sim.build(os.path.join(SIM, "_build_address"), sanitize="address")
+    exe = str(tmp_path / "threads_driver_asan")
+    build_threads_driver(asan, exe, ["-fsanitize=address", "-shared-libsan", "-Wl,-rpath," + runtime])
+    res = subprocess.run([exe, "3", "4"], capture_output=True, text=True, timeout=1200, env=dict(os.environ, ASAN_OPTIONS="detect_leaks=1"))
+    assert res.returncode == 0 and res.stdout.strip().endswith("ok") and "AddressSanitizer" not in res.stderr, (res.returncode, res.stdout, res.stderr[-4000:])
     ubsan = build_sim.build(os.path.join(SIM, "_build_undefined"), sanitize="undefined")
     code = ("import sys; sys.path[:0] = [%r, %r]; import ophip; ophip.LIB_PATH = %r; import __graft_entry__; __graft_entry__.smoke()"
             % (ROOT, os.path.join(ROOT, "operators-rs_amd"), ubsan))
