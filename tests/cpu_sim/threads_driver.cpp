@@ -7,7 +7,9 @@
 // buffers, and repeats: rms_norm [16, 1024], mat_mul [16, 1024] x [1024, 512] on a split K (workspace from the queue
 // allocator, arrival counters from the operator), copy back, compare with what thread 0 computed on the host.  Every
 // few rounds a thread also creates and destroys an operator and a stream of its own, which adds and removes hooks while
-// the others launch.  Exit status 0 when every result agreed; a data race ends the run through the sanitizer.
+// the others launch.  Before the threads start, every other operator of the library is created, planned, launched on
+// small zero-filled operands and destroyed once (so that an AddressSanitizer build with leak detection sees the whole
+// life of each).  Exit status 0 when every result agreed; a data race ends the run through the sanitizer.
 //
 //   threads_driver [threads = 4] [rounds = 12]
 #include <atomic>
@@ -111,6 +113,145 @@ void worker(const Shared &sh, int id, int rounds) {
     CHECK(ophip_stream_destroy(sh.dev, stream));
 }
 
+// Every other operator once, on one thread, small shapes, zero-filled operands (what they compute is the parity tests'
+// business): created, planned, launched, destroyed, so that a sanitizer build sees the whole life of each.
+int every_operator_once(ophip_device *dev) {
+#define TRY(call)                                                                     \
+    do {                                                                              \
+        const int rc_ = (call);                                                       \
+        if (rc_ != OPHIP_OK) {                                                        \
+            std::fprintf(stderr, "%s -> %d (%s)\n", #call, rc_, ophip_last_error()); \
+            return 1;                                                                 \
+        }                                                                             \
+    } while (0)
+    ophip_stream stream = nullptr;
+    TRY(ophip_stream_create(dev, &stream));
+    ophip_queue_alloc qa;
+    TRY(ophip_queue_alloc_from_stream(dev, stream, &qa));
+    std::vector<void *> held;
+    auto zeros = [&](size_t bytes) {
+        void *p = nullptr;
+        if (ophip_malloc(dev, bytes, &p) != OPHIP_OK || ophip_memset(dev, p, 0, bytes, stream) != OPHIP_OK) std::abort();
+        held.push_back(p);
+        return p;
+    };
+    size_t ws = 0;
+    const size_t nt = 6, nh = 4, nkvh = 2, dh = 64, buf = 32, d = nh * dh;
+    const size_t s3[3] = {nt, nh, dh}, s3t[3] = {nh, nt, dh}, skv[3] = {nkvh, nt, dh}, sc[3] = {nkvh, buf, dh}, s1[1] = {nt}, s2[2] = {nt, d}, sd[1] = {d};
+    const ptrdiff_t t3[3] = {(ptrdiff_t)(d * 2), (ptrdiff_t)(dh * 2), 2}, t3t[3] = {(ptrdiff_t)(nt * dh * 2), (ptrdiff_t)(dh * 2), 2};
+    const ptrdiff_t tkv[3] = {(ptrdiff_t)(nt * dh * 2), (ptrdiff_t)(dh * 2), 2}, tc[3] = {(ptrdiff_t)(buf * dh * 2), (ptrdiff_t)(dh * 2), 2};
+    const ptrdiff_t t1[1] = {4}, t2[2] = {(ptrdiff_t)(d * 2), 2}, td[1] = {2};
+    const ophip_tensor_layout tok{OPHIP_DT_F16, 3, s3, t3}, heads{OPHIP_DT_F16, 3, s3t, t3t}, kv{OPHIP_DT_F16, 3, skv, tkv}, cache{OPHIP_DT_F16, 3, sc, tc};
+    const ophip_tensor_layout pos{OPHIP_DT_U32, 1, s1, t1}, mat{OPHIP_DT_F16, 2, s2, t2}, vec{OPHIP_DT_F16, 1, sd, td};
+    {
+        ophip_rope *op = nullptr;
+        TRY(ophip_rope_create(dev, &op));
+        const size_t se[2] = {0, dh};
+        const ptrdiff_t te[2] = {(ptrdiff_t)(dh * 2), 2};
+        ophip_rope_args a{};
+        a.t_layout = tok, a.t_base = zeros(nt * d * 2), a.p_layout = pos, a.p_base = zeros(nt * 4);
+        a.sin_layout = a.cos_layout = ophip_tensor_layout{OPHIP_DT_F16, 2, se, te};
+        a.theta = 1e4f;
+        TRY(ophip_rope_scheme(op, &a, 0, &ws));
+        TRY(ophip_rope_launch(op, &a, nullptr, 0, &qa));
+        ophip_rope_destroy(op);
+    }
+    {
+        ophip_fused_softmax *op = nullptr;
+        TRY(ophip_fused_softmax_create(dev, &op));
+        const size_t sa[3] = {nh, nt, buf};
+        const ptrdiff_t ta[3] = {(ptrdiff_t)(nt * buf * 2), (ptrdiff_t)(buf * 2), 2};
+        ophip_fused_softmax_args a{};
+        a.att_mask = 1, a.att_layout = ophip_tensor_layout{OPHIP_DT_F16, 3, sa, ta}, a.att_base = zeros(nh * nt * buf * 2);
+        TRY(ophip_fused_softmax_scheme(op, &a, 0, &ws));
+        TRY(ophip_fused_softmax_launch(op, &a, nullptr, 0, &qa));
+        ophip_fused_softmax_destroy(op);
+    }
+    {
+        ophip_rearrange *op = nullptr;
+        TRY(ophip_rearrange_create(dev, &op));
+        const ptrdiff_t as_heads[3] = {(ptrdiff_t)(dh * 2), (ptrdiff_t)(nt * dh * 2), 2};  // token-major indices over head-major memory
+        ophip_rearrange_args a{};
+        a.dst_layout = ophip_tensor_layout{OPHIP_DT_F16, 3, s3, as_heads}, a.dst_base = zeros(nt * d * 2), a.src_layout = tok, a.src_base = zeros(nt * d * 2);
+        TRY(ophip_rearrange_scheme(op, &a, 0, &ws));
+        TRY(ophip_rearrange_launch(op, &a, nullptr, 0, &qa));
+        ophip_rearrange_destroy(op);
+    }
+    {
+        ophip_swiglu *op = nullptr;
+        TRY(ophip_swiglu_create(dev, &op));
+        ophip_swiglu_args a{};
+        a.gate_layout = a.up_layout = mat, a.gate_base = zeros(nt * d * 2), a.up_base = zeros(nt * d * 2);
+        TRY(ophip_swiglu_scheme(op, &a, 0, &ws));
+        TRY(ophip_swiglu_launch(op, &a, nullptr, 0, &qa));
+        ophip_swiglu_destroy(op);
+        ophip_gelu *g = nullptr;
+        TRY(ophip_gelu_create(dev, &g));
+        ophip_gelu_args ga{};
+        ga.layout = mat, ga.base = zeros(nt * d * 2);
+        TRY(ophip_gelu_scheme(g, &ga, 0, &ws));
+        TRY(ophip_gelu_launch(g, &ga, nullptr, 0, &qa));
+        ophip_gelu_destroy(g);
+        ophip_add *ad = nullptr;
+        TRY(ophip_add_create(dev, &ad));
+        ophip_add_args aa{};
+        aa.c_layout = aa.a_layout = aa.b_layout = mat, aa.c_base = zeros(nt * d * 2), aa.a_base = zeros(nt * d * 2), aa.b_base = zeros(nt * d * 2);
+        TRY(ophip_add_scheme(ad, &aa, 0, &ws));
+        TRY(ophip_add_launch(ad, &aa, nullptr, 0, &qa));
+        ophip_add_destroy(ad);
+        ophip_layer_norm *ln = nullptr;
+        TRY(ophip_layer_norm_create(dev, &ln));
+        ophip_layer_norm_args la{};
+        la.y_layout = la.x_layout = mat, la.scale_layout = la.bias_layout = vec, la.epsilon = 1e-5f;
+        la.y_base = zeros(nt * d * 2), la.x_base = zeros(nt * d * 2), la.scale_base = zeros(d * 2), la.bias_base = zeros(d * 2);
+        TRY(ophip_layer_norm_scheme(ln, &la, 0, &ws));
+        TRY(ophip_layer_norm_launch(ln, &la, nullptr, 0, &qa));
+        ophip_layer_norm_destroy(ln);
+    }
+    {
+        ophip_random_sample *op = nullptr;
+        TRY(ophip_random_sample_create(dev, &op));
+        const size_t n = 5000, sn[1] = {n};
+        const ptrdiff_t tl[1] = {2}, ti[1] = {4};
+        ophip_random_sample_args a{};
+        a.kv_pair = ophip_tensor_layout{OPHIP_DT_KVPAIR, 0, nullptr, nullptr}, a.kv_pair_base = zeros(8);
+        a.logits = ophip_tensor_layout{OPHIP_DT_F16, 1, sn, tl}, a.logits_base = zeros(n * 2);
+        a.indices = ophip_tensor_layout{OPHIP_DT_U32, 1, sn, ti};
+        a.config = ophip_sample_args_argmax();
+        TRY(ophip_random_sample_scheme(op, &a, (size_t)1 << 30, &ws));
+        TRY(ophip_random_sample_launch(op, &a, nullptr, 0, &qa));
+        if (ophip_sample_args_new(0.8f, 0.9f, 200, &a.config) != 0) return 1;
+        a.seed = 0.37f;
+        TRY(ophip_random_sample_scheme(op, &a, (size_t)1 << 30, &ws));
+        TRY(ophip_random_sample_launch(op, &a, nullptr, 0, &qa));  // its workspace from the queue allocator
+        ophip_random_sample_destroy(op);
+    }
+    {
+        ophip_attention *op = nullptr;
+        TRY(ophip_attention_create(dev, &op));
+        ophip_attention_args a{};
+        a.q_layout = a.o_layout = heads, a.k_layout = a.v_layout = kv, a.mask = 1;
+        a.q_base = zeros(nt * d * 2), a.o_base = zeros(nt * d * 2), a.k_base = zeros(nkvh * nt * dh * 2), a.v_base = zeros(nkvh * nt * dh * 2);
+        TRY(ophip_attention_scheme(op, &a, (size_t)1 << 30, &ws));
+        TRY(ophip_attention_launch(op, &a, nullptr, 0, &qa));
+        ophip_attention_destroy(op);
+        ophip_attention_kv_cached *kc = nullptr;
+        TRY(ophip_attention_kv_cached_create(dev, &kc));
+        ophip_attention_kv_cached_args c{};
+        c.q_layout = c.o_layout = heads, c.k_layout = c.v_layout = kv, c.k_cache_layout = c.v_cache_layout = cache, c.mask = 1, c.pos = 9;
+        c.q_base = zeros(nt * d * 2), c.o_base = zeros(nt * d * 2), c.k_base = a.k_base, c.v_base = a.v_base;
+        c.k_cache_base = zeros(nkvh * buf * dh * 2), c.v_cache_base = zeros(nkvh * buf * dh * 2);
+        TRY(ophip_attention_kv_cached_scheme(kc, &c, (size_t)1 << 30, &ws));
+        TRY(ophip_attention_kv_cached_launch(kc, &c, nullptr, 0, &qa));
+        ophip_attention_kv_cached_destroy(kc);
+    }
+    TRY(ophip_stream_synchronize(dev, stream));
+    for (void *p : held) TRY(ophip_free(dev, p));
+    TRY(ophip_stream_destroy(dev, stream));
+    return 0;
+#undef TRY
+}
+
 }  // namespace
 
 int main(int argc, char **argv) {
@@ -200,6 +341,7 @@ int main(int argc, char **argv) {
             return 3;
         }
     }
+    if (every_operator_once(sh.dev) != 0) return 4;
     std::vector<std::thread> pool;
     for (int t = 0; t < threads; ++t) pool.emplace_back(worker, std::cref(sh), t, rounds);
     for (auto &t : pool) t.join();
