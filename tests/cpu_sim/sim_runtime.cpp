@@ -121,7 +121,11 @@ hipError_t sim_free(void *ptr) {
     if (!ptr) return hipSuccess;
     std::lock_guard<std::recursive_mutex> lock(g_mu);
     auto it = g_blocks.find(reinterpret_cast<uintptr_t>(ptr));
-    if (it == g_blocks.end()) return hipErrorInvalidValue;
+    if (it == g_blocks.end()) {
+        // the library gives back exactly what it took, once: anything else is a bug worth stopping for
+        std::fprintf(stderr, "cpusim: hipFree(%p): %s\n", ptr, g_freed.count(reinterpret_cast<uintptr_t>(ptr)) ? "freed before" : "no device allocation starts there");
+        std::abort();
+    }
     g_live_bytes -= it->second.map_len - 2 * 4096;
     // the pages stay reserved and inaccessible: a later access faults instead of landing in a newer allocation
     mmap(it->second.map, it->second.map_len, PROT_NONE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_FIXED | MAP_NORESERVE, -1, 0);
