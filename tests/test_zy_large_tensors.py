@@ -212,3 +212,34 @@ def test_attention_kv_cached_caches_past_4_gib(gpu, stream):
         ref = (p / p.sum(axis=1, keepdims=True)) @ vals
         assert np.abs(ref).max() > 0.25  # (the comparison below means something)
         assert_close_f16(out[h], ref, "attention_kv_cached past 4 GiB, head %d" % h)
+
+
+def test_batched_mat_mul_whose_batches_lie_past_4_gib(gpu, stream):
+    """q . K^T through mat_mul over a 4.6 GiB K cache (40 heads of 480000 keys of 128, K-contiguous): the batch stride
+    carries the later heads past 2^32 bytes.  K[h, j, :] = T[(131 h + 7 j + 13 t) mod L] for a random table T."""
+    nh, seq, dh, buf, L = 40, 16, 128, 480000, 1000003
+    say("mat_mul %d x (%d x %d . %d x %d), B stored [N, K]" % (nh, seq, dh, dh, buf))
+    rng = np.random.default_rng(16)
+    table = rng.standard_normal(L).astype(f32).astype(f16)
+
+    def keys(h, j):
+        j = np.asarray(j, dtype=np.int64)
+        return table[(h * 131 + j[:, None] * 7 + np.arange(dh, dtype=np.int64)[None, :] * 13) % L]
+
+    kc = gpu.malloc(nh * buf * dh * 2)
+    for h in range(nh):
+        for j0 in range(0, buf, 120000):
+            gpu.upload(kc, keys(h, np.arange(j0, min(buf, j0 + 120000))), offset=(h * buf + j0) * dh * 2)
+    q = rng.standard_normal((nh, seq, dh)).astype(f32).astype(f16)
+    qd, cd = gpu.from_host(q), gpu.malloc(nh * seq * buf * 2)
+    op = ophip.MatMul(gpu)
+    args = ophip.MatMulArgs(TensorLayout.new_contiguous(dt.F16, [nh, seq, buf]), cd, 0.0, TensorLayout.new_contiguous(dt.F16, [nh, seq, dh]), qd,
+                            TensorLayout(dt.F16, [nh, dh, buf], [buf * dh * 2, 2, dh * 2]), kc, 0.125)
+    say("  kernel: " + op.describe(args))
+    op.launch(args, None, stream)
+    stream.synchronize()
+    for h in (0, 1, 17, 18, 19, 38, 39):  # the 4 GiB line runs through head 17's keys
+        js = sorted({0, 1, buf - 2, buf - 1} | {int(x) for x in rng.integers(0, buf, 40)})
+        ref = 0.125 * q[h].astype(np.float64) @ keys(h, js).astype(np.float64).T
+        got = np.array([[gpu.to_host(cd, f16, 1, offset=((h * seq + i) * buf + j) * 2, stream=stream)[0] for j in js] for i in range(seq)])
+        assert rel_error(got.astype(np.float64), ref) <= 1e-2, h
