@@ -80,6 +80,7 @@ struct Item {
     uint32_t flat = 0;
     ItemState state = ItemState::Done;
     char *stack = nullptr;
+    uint32_t site = 0;  // where in the source the wave operation it waits at was written
     void *asan_fake = nullptr;
     void *tsan_fiber = nullptr;
 };
@@ -165,9 +166,10 @@ struct WaveView {
     const unsigned char (*a)[SLOT_BYTES];
     const unsigned char (*b)[SLOT_BYTES];
 };
-inline WaveView wave_exchange(const void *op_a, size_t bytes_a, const void *op_b = nullptr, size_t bytes_b = 0) {
+inline WaveView wave_exchange(uint32_t site, const void *op_a, size_t bytes_a, const void *op_b = nullptr, size_t bytes_b = 0) {
     Worker &w = worker();
     Item *it = w.cur;
+    it->site = site;
     WaveSlots &ws = w.waves[it->flat / WAVE_LANES];
     const uint32_t set = ws.generation & 1, lane = it->flat % WAVE_LANES;
     if (bytes_a > SLOT_BYTES || bytes_b > SLOT_BYTES) std::abort();
@@ -246,7 +248,20 @@ inline void run_workgroup(Worker &w, uint32_t threads) {
             // (a wave none of whose lanes waited did no operation: its generation stays)
             for (uint32_t v = 0; v < threads / WAVE_LANES; ++v) {
                 bool woke = false;
-                for (uint32_t l = 0; l < WAVE_LANES; ++l) woke |= w.items[v * WAVE_LANES + l]->state == ItemState::Runnable;
+                uint32_t site = 0;
+                for (uint32_t l = 0; l < WAVE_LANES; ++l) {
+                    const Item *it = w.items[v * WAVE_LANES + l];
+                    if (it->state != ItemState::Runnable) continue;
+                    // The lanes that meet must be at one and the same operation of the source: lanes of a wave that
+                    // took different branches would execute their operations one after the other on the hardware,
+                    // each under its own mask, and pairing them here would hand them each other's operands.
+                    if (woke && it->site != site) {
+                        std::fprintf(stderr, "cpusim: lanes of wave %u of workgroup (%u, %u, %u) met at different wave operations (source lines %u and %u)\n",
+                                     v, w.block_idx.x, w.block_idx.y, w.block_idx.z, site, it->site);
+                        std::abort();
+                    }
+                    woke = true, site = it->site;
+                }
                 if (woke) w.waves[v].generation++;
             }
             continue;

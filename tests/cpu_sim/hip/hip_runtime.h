@@ -43,7 +43,7 @@ using std::min;
 
 inline void __syncthreads() { cpusim::barrier(); }
 // the lanes of the caller's wave meet (the kernels mark the places where they rely on a wave running in lockstep)
-inline void cpusim_wave_sync() { cpusim::wave_exchange(nullptr, 0); }
+inline void cpusim_wave_sync(int line = __builtin_LINE()) { cpusim::wave_exchange((uint32_t)line, nullptr, 0); }
 
 // ---- vector types
 struct float2 {
@@ -157,38 +157,40 @@ inline void cpusim_buffer_store_b128(cpusim_u32x4 v, __amdgpu_buffer_rsrc_t r, u
 // ---- cross-lane
 // value of `v` held by lane `src` of the caller's wave
 template <class T>
-inline T cpusim_read_lane(T v, uint32_t src) {
+inline T cpusim_read_lane(int line, T v, uint32_t src) {
     static_assert(sizeof(T) <= cpusim::SLOT_BYTES, "operand too wide");
-    const cpusim::WaveView w = cpusim::wave_exchange(&v, sizeof(T));
+    const cpusim::WaveView w = cpusim::wave_exchange((uint32_t)line, &v, sizeof(T));
     T out;
     std::memcpy(&out, w.a[src % cpusim::WAVE_LANES], sizeof(T));
     return out;
 }
+// (the last parameter of each: the line of the call, by which the scheduler checks that the lanes that meet are at the
+// same operation)
 template <class T>
-inline T __shfl_xor(T v, int mask, int = 64) {
-    return cpusim_read_lane(v, cpusim::lane_id() ^ (uint32_t)mask);
+inline T __shfl_xor(T v, int mask, int = 64, int line = __builtin_LINE()) {
+    return cpusim_read_lane(line, v, cpusim::lane_id() ^ (uint32_t)mask);
 }
 template <class T>
-inline T __shfl(T v, int src, int = 64) {
-    return cpusim_read_lane(v, (uint32_t)src);
+inline T __shfl(T v, int src, int = 64, int line = __builtin_LINE()) {
+    return cpusim_read_lane(line, v, (uint32_t)src);
 }
 template <class T>
-inline T __shfl_up(T v, unsigned delta, int = 64) {
+inline T __shfl_up(T v, unsigned delta, int = 64, int line = __builtin_LINE()) {
     const uint32_t lane = cpusim::lane_id();
-    return cpusim_read_lane(v, lane >= delta ? lane - delta : lane);
+    return cpusim_read_lane(line, v, lane >= delta ? lane - delta : lane);
 }
 template <class T>
-inline T __shfl_down(T v, unsigned delta, int = 64) {
+inline T __shfl_down(T v, unsigned delta, int = 64, int line = __builtin_LINE()) {
     const uint32_t lane = cpusim::lane_id();
-    return cpusim_read_lane(v, lane + delta < cpusim::WAVE_LANES ? lane + delta : lane);
+    return cpusim_read_lane(line, v, lane + delta < cpusim::WAVE_LANES ? lane + delta : lane);
 }
 // A lane that is not at the ballot (masked out, or returned) counts as 0: a slot it left from an earlier operation
 // must not be read, so every lane deposits a marker that carries the wave's operation number.
-inline uint64_t __ballot(int pred) {
+inline uint64_t __ballot(int pred, int line = __builtin_LINE()) {
     cpusim::Worker &wk = cpusim::worker();
     const uint32_t gen = wk.waves[wk.cur->flat / cpusim::WAVE_LANES].generation;
     const uint32_t mine[2] = {gen, pred ? 1u : 0u};
-    const cpusim::WaveView w = cpusim::wave_exchange(mine, sizeof(mine));
+    const cpusim::WaveView w = cpusim::wave_exchange((uint32_t)line, mine, sizeof(mine));
     uint64_t out = 0;
     for (uint32_t l = 0; l < cpusim::WAVE_LANES; ++l) {
         uint32_t theirs[2];
@@ -197,9 +199,9 @@ inline uint64_t __ballot(int pred) {
     }
     return out;
 }
-#define __builtin_amdgcn_ballot_w64(p) __ballot(p)
+#define __builtin_amdgcn_ballot_w64(p) __ballot(p, __LINE__)
 // DPP moves: quad permutes (ctrl < 0x100), row_mirror (0x140), row_half_mirror (0x141); full masks, bound_ctrl set
-inline int cpusim_update_dpp(int, int src, int ctrl, int row_mask, int bank_mask, bool) {
+inline int cpusim_update_dpp(int line, int, int src, int ctrl, int row_mask, int bank_mask, bool) {
     const uint32_t lane = cpusim::lane_id();
     uint32_t from;
     if (ctrl < 0x100) from = (lane & ~3u) | ((uint32_t)(ctrl >> (2 * (lane & 3))) & 3u);
@@ -213,16 +215,16 @@ inline int cpusim_update_dpp(int, int src, int ctrl, int row_mask, int bank_mask
         std::fprintf(stderr, "cpusim: partial DPP masks are not emulated\n");
         std::abort();
     }
-    return cpusim_read_lane(src, from);
+    return cpusim_read_lane(line, src, from);
 }
-#define __builtin_amdgcn_update_dpp(old, src, ctrl, row_mask, bank_mask, bound) cpusim_update_dpp(old, src, ctrl, row_mask, bank_mask, bound)
+#define __builtin_amdgcn_update_dpp(old, src, ctrl, row_mask, bank_mask, bound) cpusim_update_dpp(__LINE__, old, src, ctrl, row_mask, bank_mask, bound)
 
 // ds_read_b64_tr_b16: the 16 lanes of a group each address four 16-bit elements; seen as a [4 rows][16 columns] matrix
 // (lane 4 r + m of the group addresses row r, columns 4 m .. 4 m + 3), lane c of the group receives column c, rows 0 .. 3.
-inline cpusim_s16x4 cpusim_ds_read_tr16_b64(const void *p) {
+inline cpusim_s16x4 cpusim_ds_read_tr16_b64(int line, const void *p) {
     unsigned char mine[8];
     std::memcpy(mine, p, 8);
-    const cpusim::WaveView w = cpusim::wave_exchange(mine, 8);
+    const cpusim::WaveView w = cpusim::wave_exchange((uint32_t)line, mine, 8);
     const uint32_t lane = cpusim::lane_id(), group = lane & ~15u, c = lane & 15u;
     cpusim_s16x4 out;
     for (uint32_t r = 0; r < 4; ++r) {
@@ -232,15 +234,15 @@ inline cpusim_s16x4 cpusim_ds_read_tr16_b64(const void *p) {
     }
     return out;
 }
-#define __builtin_amdgcn_ds_read_tr16_b64_v4i16(p) cpusim_ds_read_tr16_b64((const void *)(p))
+#define __builtin_amdgcn_ds_read_tr16_b64_v4i16(p) cpusim_ds_read_tr16_b64(__LINE__, (const void *)(p))
 
 // ---- MFMA.  v_mfma_f32_16x16x32_{f16,bf16}: D[16 x 16] = A[16 x 32] . B[32 x 16] + C.  Lane l holds A[l % 16][8 (l / 16) ..+8],
 // B[8 (l / 16) ..+8][l % 16] and D[4 (l / 16) + q][l % 16], q = 0 .. 3.
 template <class V>
-inline cpusim_f32x4 cpusim_mfma_16x16x32(V a, V b, cpusim_f32x4 c) {
+inline cpusim_f32x4 cpusim_mfma_16x16x32(int line, V a, V b, cpusim_f32x4 c) {
     float af[8], bf[8];
     for (int k = 0; k < 8; ++k) af[k] = (float)a[k], bf[k] = (float)b[k];
-    const cpusim::WaveView w = cpusim::wave_exchange(af, 32, bf, 32);
+    const cpusim::WaveView w = cpusim::wave_exchange((uint32_t)line, af, 32, bf, 32);
     const uint32_t lane = cpusim::lane_id(), j = lane % 16, i0 = 4 * (lane / 16);
     for (int q = 0; q < 4; ++q) {
         float acc = c[q];
@@ -253,15 +255,15 @@ inline cpusim_f32x4 cpusim_mfma_16x16x32(V a, V b, cpusim_f32x4 c) {
     }
     return c;
 }
-#define __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, x, y, z) cpusim_mfma_16x16x32<cpusim_f16x8>(a, b, c)
-#define __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, x, y, z) cpusim_mfma_16x16x32<cpusim_bf16x8>(a, b, c)
+#define __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, x, y, z) cpusim_mfma_16x16x32<cpusim_f16x8>(__LINE__, a, b, c)
+#define __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, x, y, z) cpusim_mfma_16x16x32<cpusim_bf16x8>(__LINE__, a, b, c)
 // v_mfma_f32_32x32x16_{f16,bf16}: D[32 x 32] = A[32 x 16] . B[16 x 32] + C.  Lane l holds A[l % 32][8 (l / 32) ..+8],
 // B[8 (l / 32) ..+8][l % 32] and D[8 (r / 4) + 4 (l / 32) + r % 4][l % 32], r = 0 .. 15.
 template <class V>
-inline cpusim_f32x16 cpusim_mfma_32x32x16(V a, V b, cpusim_f32x16 c) {
+inline cpusim_f32x16 cpusim_mfma_32x32x16(int line, V a, V b, cpusim_f32x16 c) {
     float af[8], bf[8];
     for (int k = 0; k < 8; ++k) af[k] = (float)a[k], bf[k] = (float)b[k];
-    const cpusim::WaveView w = cpusim::wave_exchange(af, 32, bf, 32);
+    const cpusim::WaveView w = cpusim::wave_exchange((uint32_t)line, af, 32, bf, 32);
     const uint32_t lane = cpusim::lane_id(), j = lane % 32, h = lane / 32;
     for (int r = 0; r < 16; ++r) {
         const uint32_t i = 8 * (r / 4) + 4 * h + r % 4;
@@ -275,8 +277,8 @@ inline cpusim_f32x16 cpusim_mfma_32x32x16(V a, V b, cpusim_f32x16 c) {
     }
     return c;
 }
-#define __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, x, y, z) cpusim_mfma_32x32x16<cpusim_f16x8>(a, b, c)
-#define __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, x, y, z) cpusim_mfma_32x32x16<cpusim_bf16x8>(a, b, c)
+#define __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, x, y, z) cpusim_mfma_32x32x16<cpusim_f16x8>(__LINE__, a, b, c)
+#define __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, x, y, z) cpusim_mfma_32x32x16<cpusim_bf16x8>(__LINE__, a, b, c)
 
 // ---- registration of a module's kernels (the generated file of each module lists them after including the source)
 #define CPUSIM_REGISTER(module_name, kernel)                                                                       \
