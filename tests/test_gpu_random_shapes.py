@@ -345,3 +345,66 @@ def test_random_attention_one_pass(gpu, stream, monkeypatch, sweep):
         # padded rows still follow each other head after head: heads and tokens fold into one dimension, and the reference
         # then leaves att . v in q
         assert np.array_equal(Q.fetch(stream), got)
+
+
+def random_view(rng, base):
+    """A view of `base` reached by slicing with steps (negative ones too), dropping and permuting axes: every address
+    inside `base`, no two elements at one address."""
+    idx = []
+    for n in base.shape:
+        kind = rng.integers(0, 4)
+        if kind == 0 or n == 1:
+            idx.append(slice(None))
+        else:
+            a, b = sorted(int(x) for x in rng.integers(0, n + 1, 2))
+            if a == b:
+                a, b = 0, n
+            step = int(rng.choice([1, 1, 2, 3]))
+            idx.append(slice(a, b, step) if kind != 3 else slice(b - 1, a - 1 if a > 0 else None, -step))
+    v = base[tuple(idx)]
+    return v.transpose(list(rng.permutation(v.ndim)))
+
+
+@SWEEPS
+def test_random_rearrange_between_arbitrary_views(gpu, stream, sweep):
+    """rearrange between views that numpy can describe and the structured tests do not reach: elements of 1, 2, 4 and 8
+    bytes, steps, negative strides, a source broadcast along an axis, bases that are only element-aligned.  numpy's
+    own assignment between the same two views is the expected result; everything outside the destination view must
+    keep its bytes."""
+    rng = np.random.default_rng(211 + 1000 * sweep)
+    op = ophip.Rearrange(gpu)
+    types = {1: (np.uint8, dt.U8), 2: (np.uint16, dt.U16), 4: (np.uint32, dt.U32), 8: (np.uint64, dt.U64)}
+    done = 0
+    for case in range(60):
+        size = int(rng.choice([1, 2, 2, 4, 8]))
+        ntype, code = types[size]
+        nd = int(rng.integers(1, 5))
+        dst_base = rng.integers(0, 256, [int(rng.integers(1, 10)) for _ in range(nd)] + [size], dtype=np.uint8).view(ntype)[..., 0]
+        dst_view = random_view(rng, dst_base)
+        # a source of the destination view's shape: a view of another base, some axes broadcast (stride 0)
+        src_shape = [1 if (n > 1 and rng.integers(0, 5) == 0) else n for n in dst_view.shape]
+        pad = [int(rng.integers(0, 3)) for _ in src_shape]
+        src_base = rng.integers(0, 256, [n + p for n, p in zip(src_shape, pad)] + [size], dtype=np.uint8).view(ntype)[..., 0]
+        src_view = src_base[tuple(slice(int(rng.integers(0, p + 1)), None) for p in pad)]
+        src_view = src_view[tuple(slice(0, n) for n in src_shape)]
+        if rng.integers(0, 3) == 0 and src_view.ndim:
+            ax = int(rng.integers(0, src_view.ndim))
+            src_view = np.flip(src_view, ax)
+        src_view = np.broadcast_to(src_view, dst_view.shape)
+        if dst_view.size == 0:
+            continue
+        dd, sd = gpu.from_host(dst_base), gpu.from_host(src_base)
+        d_off = dst_view.__array_interface__["data"][0] - dst_base.__array_interface__["data"][0]
+        s_off = src_view.__array_interface__["data"][0] - src_base.__array_interface__["data"][0]
+        say("random views %d: %d-byte elements, shape %s, dst strides %s, src strides %s" % (case, size, dst_view.shape, dst_view.strides, src_view.strides))
+        op.launch(ophip.RearrangeArgs(TensorLayout(code, list(dst_view.shape), list(dst_view.strides)), dd.ptr + d_off,
+                                      TensorLayout(code, list(src_view.shape), list(src_view.strides)), sd.ptr + s_off), None, stream)
+        want = dst_base.copy()
+        want_view = np.lib.stride_tricks.as_strided(want.reshape(-1)[d_off // size:], dst_view.shape, dst_view.strides) if all(s >= 0 for s in dst_view.strides) else None
+        if want_view is None:  # negative strides: the same view of the copy, by the same recipe relative to its own base
+            want_view = np.ndarray(dst_view.shape, ntype, want.data, d_off, dst_view.strides)
+        want_view[...] = src_view
+        got = gpu.to_host(dd, ntype, dst_base.size, stream=stream).reshape(dst_base.shape)
+        assert np.array_equal(got, want), case
+        done += 1
+    assert done > 40
