@@ -408,3 +408,56 @@ def test_random_rearrange_between_arbitrary_views(gpu, stream, sweep):
         assert np.array_equal(got, want), case
         done += 1
     assert done > 40
+
+
+def random_source(rng, shape, ntype, make):
+    """A view of the given shape over a base of its own: padded, offset, some axes broadcast, one possibly flipped."""
+    src_shape = [1 if (n > 1 and rng.integers(0, 5) == 0) else n for n in shape]
+    pad = [int(rng.integers(0, 3)) for _ in src_shape]
+    base = make([n + p for n, p in zip(src_shape, pad)])
+    view = base[tuple(slice(int(rng.integers(0, p + 1)), None) for p in pad)]
+    view = view[tuple(slice(0, n) for n in src_shape)]
+    if rng.integers(0, 3) == 0 and view.ndim:
+        view = np.flip(view, int(rng.integers(0, view.ndim)))
+    return base, np.broadcast_to(view, shape)
+
+
+@SWEEPS
+def test_random_add_between_arbitrary_views(gpu, stream, sweep):
+    """add with the three operands as unrelated views (steps, negative strides, broadcast a and b, element-aligned
+    bases) in f16, f32, i32 and u8; numpy's sum of the same views is the expected result (f16: the f32 sum rounded
+    once; integers wrap), and nothing outside c's view may change."""
+    rng = np.random.default_rng(223 + 1000 * sweep)
+    op = ophip.Add(gpu)
+    kinds = [(f16, dt.F16), (f32, dt.F32), (np.int32, dt.I32), (np.uint8, dt.U8)]
+    done = 0
+    for case in range(48):
+        ntype, code = kinds[int(rng.integers(0, len(kinds)))]
+        if np.issubdtype(ntype, np.floating):
+            make = lambda s: rng.standard_normal(s).astype(f32).astype(ntype)
+        else:
+            info = np.iinfo(ntype)
+            make = lambda s: rng.integers(info.min, info.max, s, dtype=ntype, endpoint=True)
+        nd = int(rng.integers(1, 5))
+        c_base = make([int(rng.integers(1, 10)) for _ in range(nd)])
+        c_view = random_view(rng, c_base)
+        if c_view.size == 0:
+            continue
+        a_base, a_view = random_source(rng, c_view.shape, ntype, make)
+        b_base, b_view = random_source(rng, c_view.shape, ntype, make)
+        off = lambda v, b: v.__array_interface__["data"][0] - b.__array_interface__["data"][0]
+        cd, ad, bd = gpu.from_host(c_base), gpu.from_host(a_base), gpu.from_host(b_base)
+        lay = lambda v: TensorLayout(code, list(v.shape), list(v.strides))
+        say("random add views %d: %s shape %s, c strides %s, a strides %s, b strides %s" % (case, ntype.__name__, c_view.shape, c_view.strides, a_view.strides, b_view.strides))
+        op.launch(ophip.AddArgs(lay(c_view), cd.ptr + off(c_view, c_base), lay(a_view), ad.ptr + off(a_view, a_base), lay(b_view), bd.ptr + off(b_view, b_base)), None, stream)
+        want = c_base.copy()
+        want_view = np.ndarray(c_view.shape, ntype, want.data, off(c_view, c_base), c_view.strides)
+        if ntype is f16:
+            want_view[...] = (a_view.astype(f32) + b_view.astype(f32)).astype(f16)
+        else:
+            with np.errstate(over="ignore"):
+                want_view[...] = a_view + b_view
+        got = gpu.to_host(cd, ntype, c_base.size, stream=stream).reshape(c_base.shape)
+        assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), case
+        done += 1
+    assert done > 30
