@@ -461,3 +461,48 @@ def test_random_add_between_arbitrary_views(gpu, stream, sweep):
         assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), case
         done += 1
     assert done > 30
+
+
+@SWEEPS
+def test_random_add_rows_between_arbitrary_views(gpu, stream, sweep):
+    """add_rows (dst[b, i, :] += src[idx[b, i], :]) with dst, src and idx as unrelated views: steps and negative strides
+    in every dimension, the last one included; u32 and u64 indices; f16, f32 and i32 elements.  Expected: numpy on the
+    same views, row by row, the sum formed as the operator's type forms it."""
+    rng = np.random.default_rng(227 + 1000 * sweep)
+    op = ophip.AddRows(gpu)
+    kinds = [(f16, dt.F16), (f32, dt.F32), (np.int32, dt.I32)]
+    for case in range(32):
+        ntype, code = kinds[int(rng.integers(0, len(kinds)))]
+        itype, icode = [(np.uint32, dt.U32), (np.uint64, dt.U64)][int(rng.integers(0, 2))]
+        if np.issubdtype(ntype, np.floating):
+            make = lambda s: rng.standard_normal(s).astype(f32).astype(ntype)
+        else:
+            make = lambda s: rng.integers(-2 ** 31, 2 ** 31 - 1, s, dtype=ntype, endpoint=True)
+        batch, m, n, k = (int(rng.integers(1, 5)), int(rng.integers(1, 7)), int(rng.choice([1, 3, 8, 24, 40])), int(rng.integers(1, 9)))
+
+        def strided(shape, make_):
+            """a view of `shape` inside a larger base: a random step and direction per axis"""
+            steps = [int(rng.choice([1, 1, 2, 3])) * int(rng.choice([1, 1, -1])) for _ in shape]
+            base = make_([abs(s) * d + int(rng.integers(0, 3)) for s, d in zip(steps, shape)])
+            return base, base[tuple(slice(None, None, s) for s in steps)][tuple(slice(0, d) for d in shape)]
+
+        dst_base, dst_view = strided((batch, m, n), make)
+        src_base, src_view = strided((k, n), make)
+        idx_base, idx_view = strided((batch, m), lambda s: rng.integers(0, k, s).astype(itype))
+        off = lambda v, b: v.__array_interface__["data"][0] - b.__array_interface__["data"][0]
+        dd, sd, idd = gpu.from_host(dst_base), gpu.from_host(src_base), gpu.from_host(idx_base)
+        say("random add_rows views %d: %s / %s, dst %s strides %s, src strides %s, idx strides %s"
+            % (case, ntype.__name__, itype.__name__, dst_view.shape, dst_view.strides, src_view.strides, idx_view.strides))
+        op.launch(ophip.AddRowsArgs(TensorLayout(code, list(dst_view.shape), list(dst_view.strides)), dd.ptr + off(dst_view, dst_base),
+                                    TensorLayout(code, list(src_view.shape), list(src_view.strides)), sd.ptr + off(src_view, src_base),
+                                    TensorLayout(icode, list(idx_view.shape), list(idx_view.strides)), idd.ptr + off(idx_view, idx_base)), None, stream)
+        want = dst_base.copy()
+        want_view = np.ndarray(dst_view.shape, ntype, want.data, off(dst_view, dst_base), dst_view.strides)
+        rows = src_view[idx_view.astype(np.int64)]  # [batch, m, n]
+        if ntype is f16:
+            want_view[...] = (dst_view.astype(f32) + rows.astype(f32)).astype(f16)
+        else:
+            with np.errstate(over="ignore"):
+                want_view[...] = dst_view + rows
+        got = gpu.to_host(dd, ntype, dst_base.size, stream=stream).reshape(dst_base.shape)
+        assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), case
