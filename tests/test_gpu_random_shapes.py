@@ -9,7 +9,7 @@ import pytest
 
 import ophip
 import oracle
-from helpers import assert_close_f16
+from helpers import assert_close_f16, normal_f16
 from ophip import TensorLayout, dt
 
 pytestmark = pytest.mark.gpu
@@ -506,3 +506,84 @@ def test_random_add_rows_between_arbitrary_views(gpu, stream, sweep):
                 want_view[...] = dst_view + rows
         got = gpu.to_host(dd, ntype, dst_base.size, stream=stream).reshape(dst_base.shape)
         assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), case
+
+
+def outer_strided(rng, shape, make):
+    """A view of `shape` whose last axis is contiguous and whose other axes run with a random step and direction
+    through a larger base."""
+    steps = [int(rng.choice([1, 1, 2, 3])) * int(rng.choice([1, 1, -1])) for _ in shape[:-1]] + [1]
+    base = make([abs(s) * d + int(rng.integers(0, 2)) for s, d in zip(steps, shape)])
+    return base, base[tuple(slice(None, None, s) for s in steps)][tuple(slice(0, d) for d in shape)]
+
+
+def byte_offset(view, base):
+    return view.__array_interface__["data"][0] - base.__array_interface__["data"][0]
+
+
+def view_layout(view, code=None):
+    return TensorLayout(code if code is not None else ophip.NP_DT[view.dtype], list(view.shape), list(view.strides))
+
+
+@SWEEPS
+def test_random_row_operators_on_views_that_step_backwards(gpu, stream, sweep):
+    """rms_norm, layer_norm, swiglu, gelu, fused softmax and rope on tensors whose rows (heads, tokens) lie at a step, or
+    in descending order, inside a larger buffer: the oracle runs on contiguous copies of the same views; whatever lies
+    between the rows must keep its bytes."""
+    rng = np.random.default_rng(229 + 1000 * sweep)
+    make = lambda s: normal_f16(rng, s)
+
+    def settle(base, view, mem, new_rows, what):
+        """device buffer against: the base with `new_rows` in the view's place (within the f16 bar there, equal elsewhere)"""
+        got = gpu.to_host(mem, f16, base.size, stream=stream).reshape(base.shape)
+        got_view = np.ndarray(view.shape, f16, got.data, byte_offset(view, base), view.strides)
+        assert_close_f16(got_view, new_rows, what)
+        keep = np.ones(base.shape, bool)
+        np.ndarray(view.shape, bool, keep.data, byte_offset(view, base) // 2, tuple(s // 2 for s in view.strides))[...] = False
+        assert np.array_equal(got[keep].view(np.uint16), base[keep].view(np.uint16)), what + ": bytes between the rows changed"
+
+    for case in range(10):
+        n, d = int(rng.integers(1, 40)), int(rng.choice([8, 24, 256, 1000, 1024, 4096]))
+        w, b = rng.uniform(0.5, 1.5, d).astype(f32).astype(f16), rng.uniform(-1, 1, d).astype(f32).astype(f16)
+        wd, bd = gpu.from_host(w), gpu.from_host(b)
+        xb, xv = outer_strided(rng, (n, d), make)
+        yb, yv = outer_strided(rng, (n, d), make)
+        xd, yd = gpu.from_host(xb), gpu.from_host(yb)
+        say("views %d: rms_norm / layer_norm [%d, %d], x strides %s, y strides %s" % (case, n, d, xv.strides, yv.strides))
+        xc = np.ascontiguousarray(xv)
+        ophip.RmsNorm(gpu).launch(ophip.RmsNormArgs(view_layout(yv), yd.ptr + byte_offset(yv, yb), view_layout(xv), xd.ptr + byte_offset(xv, xb),
+                                                    TensorLayout.of(w), wd, 1e-5), None, stream)
+        settle(yb, yv, yd, oracle.rms_norm(np.empty_like(xc), xc, w, 1e-5), "rms_norm on views")
+        ophip.LayerNorm(gpu).launch(ophip.LayerNormArgs(view_layout(yv), yd.ptr + byte_offset(yv, yb), view_layout(xv), xd.ptr + byte_offset(xv, xb),
+                                                        TensorLayout.of(w), wd, TensorLayout.of(b), bd, 1e-5), None, stream)
+        settle(yb, yv, yd, oracle.layer_norm(np.empty_like(xc), xc, w, b, 1e-5), "layer_norm on views")
+
+        gb, gv = outer_strided(rng, (n, d), make)
+        gd = gpu.from_host(gb)
+        say("views %d: swiglu, gelu [%d, %d], gate strides %s, up strides %s" % (case, n, d, gv.strides, xv.strides))
+        ophip.Swiglu(gpu).launch(ophip.SwigluArgs(view_layout(gv), gd.ptr + byte_offset(gv, gb), view_layout(xv), xd.ptr + byte_offset(xv, xb)), None, stream)
+        after = oracle.swiglu(np.ascontiguousarray(gv), xc)
+        settle(gb, gv, gd, after, "swiglu on views")
+        got = gpu.to_host(gd, f16, gb.size, stream=stream).reshape(gb.shape)
+        gb2 = got  # what the device holds now is gelu's input
+        gv2 = np.ndarray(gv.shape, f16, gb2.data, byte_offset(gv, gb), gv.strides)
+        ophip.Gelu(gpu).launch(ophip.GeluArgs(view_layout(gv), gd.ptr + byte_offset(gv, gb)), None, stream)
+        settle(gb2, gv2, gd, oracle.gelu(np.ascontiguousarray(gv2)), "gelu on views")
+
+        nh, seq = int(rng.integers(1, 5)), int(rng.integers(1, 9))
+        att = seq + int(rng.integers(0, 600))
+        ab, av = outer_strided(rng, (nh, seq, att), lambda s: normal_f16(rng, s, std=2.0))
+        ad = gpu.from_host(ab)
+        say("views %d: softmax [%d, %d, %d] strides %s" % (case, nh, seq, att, av.strides))
+        ophip.FusedSoftmax(gpu).launch(ophip.FusedSoftmaxArgs(ophip.AttnMask.CAUSAL, view_layout(av), ad.ptr + byte_offset(av, ab)), None, stream)
+        settle(ab, av, ad, oracle.fused_softmax(np.ascontiguousarray(av), causal=True), "softmax on views")
+
+        nt, nh, dh = int(rng.integers(1, 20)), int(rng.integers(1, 6)), int(rng.choice([16, 64, 128]))
+        tb, tv = outer_strided(rng, (nt, nh, dh), make)
+        pb, pv = outer_strided(rng, (nt, 1), lambda s: rng.integers(0, 5000, s).astype(np.uint32))
+        pv = pv[:, 0]
+        td, pd = gpu.from_host(tb), gpu.from_host(pb)
+        say("views %d: rope [%d, %d, %d] strides %s, pos stride %s" % (case, nt, nh, dh, tv.strides, pv.strides))
+        empty = TensorLayout(dt.F16, [0, dh], [2 * dh, 2])
+        ophip.Rope(gpu).launch(ophip.RopeArgs(view_layout(tv), td.ptr + byte_offset(tv, tb), view_layout(pv), pd.ptr + byte_offset(pv, pb),
+                                              empty, None, empty, None, 1e4), None, stream)
+        settle(tb, tv, td, oracle.rope(np.ascontiguousarray(tv), np.ascontiguousarray(pv), 1e4), "rope on views")
