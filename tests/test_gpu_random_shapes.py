@@ -587,3 +587,48 @@ def test_random_row_operators_on_views_that_step_backwards(gpu, stream, sweep):
         ophip.Rope(gpu).launch(ophip.RopeArgs(view_layout(tv), td.ptr + byte_offset(tv, tb), view_layout(pv), pd.ptr + byte_offset(pv, pb),
                                               empty, None, empty, None, 1e4), None, stream)
         settle(tb, tv, td, oracle.rope(np.ascontiguousarray(tv), np.ascontiguousarray(pv), 1e4), "rope on views")
+
+
+@SWEEPS
+def test_random_mat_mul_on_views(gpu, stream, sweep):
+    """mat_mul whose three operands are unrelated views: each row- or column-major at random (one unit stride, as the
+    reference requires, mat_mul/args.rs:160-176), the other axis and the batch axis at a step or in descending order,
+    a and b possibly one matrix for every batch.  A layout the library refuses must be refused as StridesNotSupport;
+    one it takes must give numpy's product, and leave alone what lies between c's elements."""
+    rng = np.random.default_rng(233 + 1000 * sweep)
+    op = ophip.MatMul(gpu)
+    taken = 0
+    for case in range(24):
+        bt, m, n, k = int(rng.integers(1, 4)), int(rng.choice([1, 5, 16, 33, 70])), int(rng.choice([8, 24, 130, 256])), int(rng.choice([16, 32, 100, 512]))
+
+        def matrix(batches, rows, cols, std):
+            """[batches, rows, cols] with rows or columns contiguous and everything else at a step, maybe backwards"""
+            col_major = bool(rng.integers(0, 2))
+            inner, outer = (rows, cols) if col_major else (cols, rows)
+            base, view = outer_strided(rng, (batches, outer, inner), lambda s: normal_f16(rng, s, std=std))
+            return base, (view.transpose(0, 2, 1) if col_major else view)
+
+        cb, cv = matrix(bt, m, n, 1.0)
+        ab, av = matrix(bt if rng.integers(0, 4) else 1, m, k, 1.0)
+        bb, bv = matrix(bt if rng.integers(0, 4) else 1, k, n, 0.1)
+        alpha, beta = float(rng.choice([1.0, 0.5])), float(rng.choice([0.0, 1.0, 0.25]))
+        cd, ad, bd = gpu.from_host(cb), gpu.from_host(ab), gpu.from_host(bb)
+        args = ophip.MatMulArgs(view_layout(cv), cd.ptr + byte_offset(cv, cb), beta, view_layout(av), ad.ptr + byte_offset(av, ab),
+                                view_layout(bv), bd.ptr + byte_offset(bv, bb), alpha)
+        say("mat_mul views %d: %dx(%dx%dx%d), c strides %s, a %s strides %s, b %s strides %s, alpha %g beta %g"
+            % (case, bt, m, n, k, cv.strides, av.shape, av.strides, bv.shape, bv.strides, alpha, beta))
+        try:
+            op.launch(args, None, stream)
+        except ophip.LaunchError as e:
+            assert e.kind == "StridesNotSupport", e
+            continue
+        taken += 1
+        got = gpu.to_host(cd, f16, cb.size, stream=stream).reshape(cb.shape)
+        got_view = np.ndarray(cv.shape, f16, got.data, byte_offset(cv, cb), cv.strides)
+        ref = alpha * np.matmul(av.astype(np.float64), bv.astype(np.float64)) + (beta * cv.astype(np.float64) if beta != 0 else 0.0)
+        err = np.abs(got_view.astype(np.float64) - ref)
+        assert (err <= 4e-3 + 1e-2 * np.maximum(np.abs(ref), np.abs(ref).mean())).all(), (case, err.max())
+        keep = np.ones(cb.shape, bool)
+        np.ndarray(cv.shape, bool, keep.data, byte_offset(cv, cb) // 2, tuple(s // 2 for s in cv.strides))[...] = False
+        assert np.array_equal(got[keep].view(np.uint16), cb[keep].view(np.uint16)), "bytes between c's elements changed"
+    assert taken >= 6
