@@ -632,3 +632,69 @@ def test_random_mat_mul_on_views(gpu, stream, sweep):
         np.ndarray(cv.shape, bool, keep.data, byte_offset(cv, cb) // 2, tuple(s // 2 for s in cv.strides))[...] = False
         assert np.array_equal(got[keep].view(np.uint16), cb[keep].view(np.uint16)), "bytes between c's elements changed"
     assert taken >= 6
+
+
+def attention_in_f64(q, k, v, causal):
+    nh, seq, dh = q.shape
+    nkvh, att, _ = k.shape
+    kk, vv = np.repeat(k.astype(np.float64), nh // nkvh, axis=0), np.repeat(v.astype(np.float64), nh // nkvh, axis=0)
+    s = np.einsum("hsd,had->hsa", q.astype(np.float64), kk) / np.sqrt(dh)
+    if causal:
+        s = np.where((np.arange(att)[None, :] <= (att - seq + np.arange(seq))[:, None])[None], s, -np.inf)
+    p = np.exp(s - s.max(-1, keepdims=True))
+    return np.einsum("hsa,had->hsd", p / p.sum(-1, keepdims=True), vv)
+
+
+@SWEEPS
+def test_random_attention_kv_cached_on_views(gpu, stream, sweep):
+    """attention_kv_cached with q, k, v, o and both caches as unrelated views: head-major or token-major at random,
+    heads and tokens at a step or in descending order (the head dimension contiguous, as every backend requires).
+    Whatever path the library picks (one pass or the composite of launches): o against the formula in f64, the
+    appended cache rows exact, every other byte of the caches and everything between o's elements unchanged."""
+    rng = np.random.default_rng(239 + 1000 * sweep)
+    op = ophip.AttnKVCached(gpu)
+    for case in range(8):
+        nkvh = int(rng.choice([1, 2, 4]))
+        nh = nkvh * int(rng.choice([1, 2, 4]))
+        seq, dh = int(rng.choice([1, 3, 16, 40])), int(rng.choice([64, 128]))
+        pos = int(rng.integers(0, 300))
+        buf = pos + seq + int(rng.integers(0, 9))
+        causal = bool(rng.integers(0, 4))
+
+        def heads(nheads, ntok):
+            """[nheads, ntok, dh], stored head-major or token-major, outer axes at a step or backwards"""
+            token_major = bool(rng.integers(0, 2))
+            base, view = outer_strided(rng, (ntok, nheads, dh) if token_major else (nheads, ntok, dh), lambda s: normal_f16(rng, s))
+            return base, (view.transpose(1, 0, 2) if token_major else view)
+
+        (qb, qv), (kb, kv), (vb, vv), (ob, ov) = heads(nh, seq), heads(nkvh, seq), heads(nkvh, seq), heads(nh, seq)
+        (kcb, kcv), (vcb, vcv) = heads(nkvh, buf), heads(nkvh, buf)
+        dev = {name: gpu.from_host(b) for name, b in (("q", qb), ("k", kb), ("v", vb), ("o", ob), ("kc", kcb), ("vc", vcb))}
+        at = lambda name, view, base: dev[name].ptr + byte_offset(view, base)
+        args = ophip.AttnKVCachedArgs(view_layout(qv), at("q", qv, qb), view_layout(kv), at("k", kv, kb), view_layout(vv), at("v", vv, vb),
+                                      view_layout(ov), at("o", ov, ob), view_layout(kcv), at("kc", kcv, kcb), view_layout(vcv), at("vc", vcv, vcb),
+                                      ophip.AttnMask.CAUSAL if causal else ophip.AttnMask.NONE, pos)
+        say("attention_kv_cached views %d: nh=%d nkvh=%d seq=%d dh=%d pos=%d buf=%d causal=%s q %s k %s o %s caches %s / %s"
+            % (case, nh, nkvh, seq, dh, pos, buf, causal, qv.strides, kv.strides, ov.strides, kcv.strides, vcv.strides))
+        if kcv.strides != vcv.strides:
+            # the reference addresses the v cache with the k cache's strides (attention_kv_cached/operator.rs:114,156):
+            # give both caches one layout, as every caller of the reference has to
+            vcb = normal_f16(rng, kcb.shape)
+            vcv = np.ndarray(kcv.shape, f16, vcb.data, byte_offset(kcv, kcb), kcv.strides)
+            dev["vc"] = gpu.from_host(vcb)
+            args.v_cache_layout, args.v_cache_base = view_layout(vcv), dev["vc"].ptr + byte_offset(vcv, vcb)
+        op.scheme(args, 2 ** 40)
+        op.launch(args, None, stream)
+        keys = np.concatenate([kcv[:, :pos], kv], axis=1)
+        vals = np.concatenate([vcv[:, :pos], vv], axis=1)
+        got_o = gpu.to_host(dev["o"], f16, ob.size, stream=stream).reshape(ob.shape)
+        got_view = np.ndarray(ov.shape, f16, got_o.data, byte_offset(ov, ob), ov.strides)
+        assert_close_f16(got_view, attention_in_f64(qv, keys, vals, causal), "attention_kv_cached on views, case %d" % case)
+        keep = np.ones(ob.shape, bool)
+        np.ndarray(ov.shape, bool, keep.data, byte_offset(ov, ob) // 2, tuple(s // 2 for s in ov.strides))[...] = False
+        assert np.array_equal(got_o[keep].view(np.uint16), ob[keep].view(np.uint16)), "bytes between o's elements changed"
+        for name, base, view, new in (("kc", kcb, kcv, kv), ("vc", vcb, vcv, vv)):
+            want = base.copy()
+            np.ndarray(view.shape, f16, want.data, byte_offset(view, base), view.strides)[:, pos:pos + seq] = new
+            got = gpu.to_host(dev[name], f16, base.size, stream=stream).reshape(base.shape)
+            assert np.array_equal(got.view(np.uint16), want.view(np.uint16)), name
