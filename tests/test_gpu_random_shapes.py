@@ -645,6 +645,18 @@ def attention_in_f64(q, k, v, causal):
     return np.einsum("hsa,had->hsd", p / p.sum(-1, keepdims=True), vv)
 
 
+def assert_attention_close(got, ref, what):
+    """Against the formula in f64: every element within abs 2e-3 or rel 1e-2.  The reference's ErrorCollector outliers
+    (abs > f16 eps and rel > 1e-3) are held to one per hundred elements here, not one per thousand: on these small
+    tensors the composite of launches rounds scores and probabilities to f16 on the way (as the reference does, and
+    as the oracle's composite does in the parity tests), which moves a few elements by a step of f16."""
+    a, r = np.asarray(got, np.float64), np.asarray(ref, np.float64)
+    err = np.abs(a - r)
+    assert ((err <= 2e-3) | (err <= 1e-2 * np.abs(r))).all(), "%s: max abs %g" % (what, err.max())
+    outliers = int(((err > 9.765625e-4) & (err / (np.abs(a) + np.abs(r) + 2.2e-16) > 1e-3)).sum())
+    assert outliers <= max(2, a.size // 100), "%s: %d / %d outliers" % (what, outliers, a.size)
+
+
 @SWEEPS
 def test_random_attention_kv_cached_on_views(gpu, stream, sweep):
     """attention_kv_cached with q, k, v, o and both caches as unrelated views: head-major or token-major at random,
@@ -689,7 +701,7 @@ def test_random_attention_kv_cached_on_views(gpu, stream, sweep):
         vals = np.concatenate([vcv[:, :pos], vv], axis=1)
         got_o = gpu.to_host(dev["o"], f16, ob.size, stream=stream).reshape(ob.shape)
         got_view = np.ndarray(ov.shape, f16, got_o.data, byte_offset(ov, ob), ov.strides)
-        assert_close_f16(got_view, attention_in_f64(qv, keys, vals, causal), "attention_kv_cached on views, case %d" % case)
+        assert_attention_close(got_view, attention_in_f64(qv, keys, vals, causal), "attention_kv_cached on views, case %d" % case)
         keep = np.ones(ob.shape, bool)
         np.ndarray(ov.shape, bool, keep.data, byte_offset(ov, ob) // 2, tuple(s // 2 for s in ov.strides))[...] = False
         assert np.array_equal(got_o[keep].view(np.uint16), ob[keep].view(np.uint16)), "bytes between o's elements changed"
@@ -698,3 +710,41 @@ def test_random_attention_kv_cached_on_views(gpu, stream, sweep):
             np.ndarray(view.shape, f16, want.data, byte_offset(view, base), view.strides)[:, pos:pos + seq] = new
             got = gpu.to_host(dev[name], f16, base.size, stream=stream).reshape(base.shape)
             assert np.array_equal(got.view(np.uint16), want.view(np.uint16)), name
+
+
+@SWEEPS
+def test_random_attention_on_views(gpu, stream, sweep):
+    """attention with q, k, v and o as unrelated views (head-major or token-major, heads and tokens at a step or in
+    descending order), grouped heads, with and without the causal mask, from a handful of query rows to several
+    128-row blocks: o against the formula in f64, everything between o's elements unchanged, k and v untouched."""
+    rng = np.random.default_rng(241 + 1000 * sweep)
+    op = ophip.Attention(gpu)
+    for case in range(8):
+        nkvh = int(rng.choice([1, 2, 4]))
+        nh = nkvh * int(rng.choice([1, 2, 4]))
+        seq, dh = int(rng.choice([1, 5, 16, 70, 200])), int(rng.choice([64, 128]))
+        att = seq + int(rng.choice([0, 0, 3, 130]))
+        causal = bool(rng.integers(0, 4))
+
+        def heads(nheads, ntok):
+            token_major = bool(rng.integers(0, 2))
+            base, view = outer_strided(rng, (ntok, nheads, dh) if token_major else (nheads, ntok, dh), lambda s: normal_f16(rng, s))
+            return base, (view.transpose(1, 0, 2) if token_major else view)
+
+        (qb, qv), (kb, kv), (vb, vv), (ob, ov) = heads(nh, seq), heads(nkvh, att), heads(nkvh, att), heads(nh, seq)
+        dev = {name: gpu.from_host(b) for name, b in (("q", qb), ("k", kb), ("v", vb), ("o", ob))}
+        at = lambda name, view, base: dev[name].ptr + byte_offset(view, base)
+        args = ophip.AttentionArgs(view_layout(qv), at("q", qv, qb), view_layout(kv), at("k", kv, kb), view_layout(vv), at("v", vv, vb),
+                                   view_layout(ov), at("o", ov, ob), ophip.AttnMask.CAUSAL if causal else ophip.AttnMask.NONE)
+        say("attention views %d: nh=%d nkvh=%d seq=%d att=%d dh=%d causal=%s q %s k %s v %s o %s"
+            % (case, nh, nkvh, seq, att, dh, causal, qv.strides, kv.strides, vv.strides, ov.strides))
+        op.scheme(args, 2 ** 40)
+        op.launch(args, None, stream)
+        got_o = gpu.to_host(dev["o"], f16, ob.size, stream=stream).reshape(ob.shape)
+        got_view = np.ndarray(ov.shape, f16, got_o.data, byte_offset(ov, ob), ov.strides)
+        assert_attention_close(got_view, attention_in_f64(qv, kv, vv, causal), "attention on views, case %d" % case)
+        keep = np.ones(ob.shape, bool)
+        np.ndarray(ov.shape, bool, keep.data, byte_offset(ov, ob) // 2, tuple(s // 2 for s in ov.strides))[...] = False
+        assert np.array_equal(got_o[keep].view(np.uint16), ob[keep].view(np.uint16)), "bytes between o's elements changed"
+        for name, base in (("k", kb), ("v", vb)):
+            assert np.array_equal(gpu.to_host(dev[name], f16, base.size, stream=stream).reshape(base.shape).view(np.uint16), base.view(np.uint16)), name
