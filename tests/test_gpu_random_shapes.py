@@ -748,3 +748,55 @@ def test_random_attention_on_views(gpu, stream, sweep):
         assert np.array_equal(got_o[keep].view(np.uint16), ob[keep].view(np.uint16)), "bytes between o's elements changed"
         for name, base in (("k", kb), ("v", vb)):
             assert np.array_equal(gpu.to_host(dev[name], f16, base.size, stream=stream).reshape(base.shape).view(np.uint16), base.view(np.uint16)), name
+
+
+@SWEEPS
+def test_random_launches_need_no_more_workspace_than_scheme_reports(gpu, stream, sweep):
+    """mat_mul (split K), attention and random_sample launched with a workspace of exactly the size scheme() answered
+    and a queue allocator that has nothing to give (an empty StreamMemPool): the launch must not ask for more, and
+    must not reach past the workspace (against the host build of the library its end lies against a guard page)."""
+    rng = np.random.default_rng(251 + 1000 * sweep)
+    pool = ophip.StreamMemPool(gpu, stream)  # no slab was put: every allocation fails
+    mm, at, rs = ophip.MatMul(gpu), ophip.Attention(gpu), ophip.RandomSample(gpu)
+    lay = TensorLayout.of
+    with_workspace = 0
+    for case in range(18):
+        if case % 3 == 0:
+            bt, m = int(rng.choice([1, 1, 4, 32])), int(rng.choice([1, 16, 40, 64, 200]))
+            n, k = int(rng.choice([128, 256, 1024])), int(rng.choice([128, 512, 2048, 4096]))
+            a, b, c = normal_f16(rng, (bt, m, k)), normal_f16(rng, (bt, k, n), std=0.05), np.zeros((bt, m, n), f16)
+            ad, bd, cd = gpu.from_host(a), gpu.from_host(b), gpu.from_host(c)
+            args = ophip.MatMulArgs(lay(c), cd, 0.0, lay(a), ad, lay(b), bd, 1.0)
+            need = mm.scheme(args, 2 ** 40)
+            say("workspace %d: mat_mul %dx(%dx%dx%d), %s, %d bytes" % (case, bt, m, n, k, mm.describe(args), need))
+            mm.launch(args, gpu.malloc(need) if need else None, pool)
+            got = gpu.to_host(cd, f16, c.size, stream=stream).reshape(c.shape).astype(np.float64)
+            ref = a.astype(np.float64) @ b.astype(np.float64)
+            assert (np.abs(got - ref) / np.maximum(np.abs(ref), np.abs(ref).mean())).max() <= 1e-2
+        elif case % 3 == 1:
+            nkvh = int(rng.choice([1, 2, 8]))
+            nh, seq, dh = nkvh * int(rng.choice([1, 4])), int(rng.choice([1, 16, 100, 300])), int(rng.choice([64, 128]))
+            att = seq + int(rng.choice([0, 50, 700]))
+            q, k, v = normal_f16(rng, (nh, seq, dh)), normal_f16(rng, (nkvh, att, dh)), normal_f16(rng, (nkvh, att, dh))
+            qd, kd, vd, od = gpu.from_host(q), gpu.from_host(k), gpu.from_host(v), gpu.malloc(q.nbytes)
+            args = ophip.AttentionArgs(lay(q), qd, lay(k), kd, lay(v), vd, lay(q), od, ophip.AttnMask.CAUSAL)
+            need = at.scheme(args, 2 ** 40)
+            say("workspace %d: attention nh=%d nkvh=%d seq=%d att=%d dh=%d, %d bytes" % (case, nh, nkvh, seq, att, dh, need))
+            at.launch(args, gpu.malloc(need) if need else None, pool)
+            got = gpu.to_host(od, f16, q.size, stream=stream).reshape(q.shape)
+            assert_attention_close(got, attention_in_f64(q, k, v, True), "attention with an exact workspace")
+        else:
+            n = int(rng.choice([1000, 32000, 50257, 128256]))
+            logits = normal_f16(rng, (n,), std=3.0)
+            ld, kvd = gpu.from_host(logits), gpu.malloc(8)
+            args = ophip.RandomSampleArgs.layout(dt.F16, n)
+            args.kv_pair_base, args.logits_base = kvd, ld
+            args.config = ophip.SampleArgs(float(rng.choice([0.7, 1.0])), float(rng.choice([0.5, 0.9, 1.0])), int(rng.choice([1, 50, 300, 5000, 2 ** 62])))
+            args.seed = float(rng.random())
+            need = rs.scheme(args, 2 ** 40)
+            say("workspace %d: random_sample n=%d, %d bytes" % (case, n, need))
+            rs.launch(args, gpu.malloc(need) if need else None, pool)
+            kv = gpu.to_host(kvd, np.uint32, 2, stream=stream)
+            assert int(kv[0]) < n
+        with_workspace += need > 0
+    assert with_workspace >= 8
