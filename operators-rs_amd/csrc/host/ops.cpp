@@ -588,6 +588,7 @@ extern "C" int ophip_rearrange_launch(const ophip_rearrange *op, const ophip_rea
     return guard([&] {
         const RScheme s = rearrange_scheme(*args);
         if (s.unit == 0 || s.count() == 0) return;
+        if (!args->dst_base || !args->src_base) throw args_not_support("null base address");
         op->dev->make_current();
         if (s.ndim() == 0) {  // one contiguous run: a device-to-device copy (rearrange/cuda/mod.rs:64-70)
             // beyond the caches, in whole aligned 16-byte chunks: the copy kernel with non-temporal loads and stores

@@ -505,6 +505,15 @@ def test_rearrange_errors(gpu, stream):
         op.launch(ophip.RearrangeArgs(L(dt.F16, [2, None], [6, 2]), None, L(dt.F16, [2, None], [6, 2]), None), None,
                   stream)
     assert e.value.kind == "DynamicNotSupport"
+    # null bases with something to copy are refused before anything is launched: a scalar (one contiguous run), a
+    # contiguous matrix, a transposition; with nothing to copy they are not looked at
+    buf = gpu.malloc(64)
+    for shape, dst_strides, src_strides in (([], [], []), ([2, 3], [6, 2], [6, 2]), ([64, 64], [2, 128], [128, 2])):
+        for dst, src in ((None, buf), (buf, None), (None, None)):
+            with pytest.raises(ophip.LaunchError) as e:
+                op.launch(ophip.RearrangeArgs(L(dt.F16, shape, dst_strides), dst, L(dt.F16, shape, src_strides), src), None, stream)
+            assert e.value.kind == "ArgsNotSupport", (shape, dst, src)
+    op.launch(ophip.RearrangeArgs(L(dt.F16, [0, 3], [6, 2]), None, L(dt.F16, [0, 3], [6, 2]), None), None, stream)
 
 
 # --------------------------------------------------------------- swiglu ----
