@@ -109,6 +109,8 @@ static void sample_launch(const ophip_random_sample *op, const ophip_random_samp
     if (rows == 0) return;
     if (rows > 0x7fffffffu) throw shape_not_support("too many rows");
     if (row_stride % sp != 0) throw strides_not_support("row stride must be a multiple of the element size");
+    // (Args::layout, random_sample/args.rs:34-49, makes arguments with null bases for scheme(): they must not reach a kernel)
+    if (!args->kv_pair_base || !args->logits_base) throw args_not_support("null base address");
 
     const int ti = m.dt == OPHIP_DT_F16 ? 0 : 1;
     const ophip_sample_args &cfg = args->config;

@@ -849,6 +849,13 @@ def test_random_sample_errors_and_build_indices(gpu, stream):
     with pytest.raises(ophip.LaunchError) as e:
         op.launch(a, None, stream)
     assert e.value.kind == "StridesNotSupport"
+    # Args::layout (random_sample/args.rs:34-49) has null bases, for scheme(): launch refuses them, argmax or not
+    for cfg in (ophip.SampleArgs.argmax(), ophip.SampleArgs(0.8, 0.9, 50)):
+        a = ophip.RandomSampleArgs.layout(dt.F16, 100)
+        a.config = cfg
+        with pytest.raises(ophip.LaunchError) as e:
+            op.launch(a, None, stream)
+        assert e.value.kind == "ArgsNotSupport"
     a = ophip.RandomSampleArgs.layout(dt.F16, None)
     assert op.scheme(a, 0) == 0
     with pytest.raises(ophip.LaunchError) as e:
