@@ -409,6 +409,8 @@ void attention_launch(const ophip_attention *op, const ophip_attention_args &arg
     const ptrdiff_t nkvh_sk = static_of(args.k_layout.strides[0]), att_sk = static_of(args.k_layout.strides[1]),
                     dh_sk = static_of(args.k_layout.strides[2]);
     if (nkvh == 0 || nh % nkvh != 0) throw shape_mismatch("nh must be a multiple of nkvh");
+    if (nh != 0 && seq != 0 && dh != 0 && att != 0 && (!args.q_base || !args.k_base || !args.v_base || !args.o_base))
+        throw args_not_support("null base address");  // (the one-pass kernels would take them as they are)
 
     // ArrayLayout::merge_be(0, 2) of ndarray-layout: heads and tokens fold into one dimension
     // when the head stride is seq * token stride (a dimension of length 1 folds with anything)
@@ -592,6 +594,9 @@ void kv_cached_launch(const ophip_attention_kv_cached *op, const ophip_attention
     // cache capacity
     const size_t att = pos + seq;
     if (buf_k < att || buf_v < att) throw shape_mismatch("Out of cache buffer");
+    if (nkvh != 0 && seq != 0 && dh != 0 && static_of(m.nh) != 0 &&
+        (!args.q_base || !args.k_base || !args.v_base || !args.o_base || !args.k_cache_base || !args.v_cache_base))
+        throw args_not_support("null base address");  // (the one-pass kernel would take them as they are)
     if (kv_cached_one_pass(op, args, m, pos, att, workspace, workspace_len, qa)) return;
     // concatenate the new rows onto the caches: slice(1, pos, 1, seq)
     const Lay3 k_cat{{nkvh, seq, dh}, {nkvh_skc, buf_skc, dh_skc}};

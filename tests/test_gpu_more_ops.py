@@ -308,3 +308,49 @@ def test_add_rows_strided_out_of_range_and_errors(gpu, stream):
     with pytest.raises(ophip.SchemeError) as e:
         op.scheme(ophip.AddRowsArgs(c(dt.F16, 3, 8), None, c(dt.F16, 5, 8), None, c(dt.U32, 2, 3), None), 0)
     assert e.value.kind == "RankNotSupport"
+
+
+def test_one_null_base_is_refused_by_every_launch(gpu, stream):
+    """Arguments with null bases are what every `Args::layout` of the reference makes for scheme(); a launch must refuse
+    them (ArgsNotSupport) before any kernel sees them, whichever single base is missing and whichever kernel the
+    shapes would have gone to (one-pass attention at decode and prefill shapes included)."""
+    c = lambda *s: TensorLayout.new_contiguous(dt.F16, list(s))
+    u32 = lambda *s: TensorLayout.new_contiguous(dt.U32, list(s))
+    mem = lambda: gpu.from_host(np.zeros(1 << 16, f16))
+    empty = TensorLayout(dt.F16, [0, 64], [128, 2])
+    cases = [
+        ("rms_norm", ophip.RmsNorm, lambda b: ophip.RmsNormArgs(c(16, 256), b[0], c(16, 256), b[1], c(256), b[2], 1e-5), 3),
+        ("layer_norm", ophip.LayerNorm, lambda b: ophip.LayerNormArgs(c(16, 256), b[0], c(16, 256), b[1], c(256), b[2], c(256), b[3], 1e-5), 4),
+        ("rope", ophip.Rope, lambda b: ophip.RopeArgs(c(8, 4, 64), b[0], u32(8), b[1], empty, None, empty, None, 1e4), 2),
+        ("fused_softmax", ophip.FusedSoftmax, lambda b: ophip.FusedSoftmaxArgs(ophip.AttnMask.CAUSAL, c(4, 8, 64), b[0]), 1),
+        ("rearrange", ophip.Rearrange, lambda b: ophip.RearrangeArgs(TensorLayout(dt.F16, [8, 64], [2, 16]), b[0], c(8, 64), b[1]), 2),
+        ("swiglu", ophip.Swiglu, lambda b: ophip.SwigluArgs(c(16, 256), b[0], c(16, 256), b[1]), 2),
+        ("gelu", ophip.Gelu, lambda b: ophip.GeluArgs(c(16, 256), b[0]), 1),
+        ("add", ophip.Add, lambda b: ophip.AddArgs(c(16, 256), b[0], c(16, 256), b[1], c(16, 256), b[2]), 3),
+        ("add_rows", ophip.AddRows, lambda b: ophip.AddRowsArgs(c(2, 4, 64), b[0], c(8, 64), b[1], u32(2, 4), b[2]), 3),
+        ("mat_mul, few rows", ophip.MatMul, lambda b: ophip.MatMulArgs(c(1, 16, 256), b[0], 0.0, c(1, 16, 128), b[1], c(1, 128, 256), b[2], 1.0), 3),
+        ("mat_mul, tiles", ophip.MatMul, lambda b: ophip.MatMulArgs(c(1, 128, 128), b[0], 0.0, c(1, 128, 64), b[1], c(1, 64, 128), b[2], 1.0), 3),
+        ("attention, decode shape", ophip.Attention, lambda b: ophip.AttentionArgs(c(4, 16, 64), b[0], c(4, 16, 64), b[1], c(4, 16, 64), b[2], c(4, 16, 64), b[3], 1), 4),
+        ("attention, prefill shape", ophip.Attention, lambda b: ophip.AttentionArgs(c(4, 128, 64), b[0], c(4, 128, 64), b[1], c(4, 128, 64), b[2], c(4, 128, 64), b[3], 1), 4),
+        ("attention_kv_cached", ophip.AttnKVCached, lambda b: ophip.AttnKVCachedArgs(c(4, 16, 64), b[0], c(4, 16, 64), b[1], c(4, 16, 64), b[2], c(4, 16, 64), b[3],
+                                                                                     c(4, 64, 64), b[4], c(4, 64, 64), b[5], 1, 5), 6),
+    ]
+    for name, cls, make, nbases in cases:
+        op = cls(gpu)
+        for missing in range(nbases):
+            bases = [mem() for _ in range(nbases)]
+            bases[missing] = None
+            say("%s, base %d null" % (name, missing))
+            with pytest.raises(ophip.LaunchError) as e:
+                op.launch(make(bases), None, stream)
+            assert e.value.kind == "ArgsNotSupport", (name, missing, e.value.kind)
+    rs = ophip.RandomSample(gpu)
+    for missing in ("kv_pair_base", "logits_base"):
+        a = ophip.RandomSampleArgs.layout(dt.F16, 1000)
+        a.kv_pair_base, a.logits_base = mem(), mem()
+        setattr(a, missing, None)
+        a.config = ophip.SampleArgs(0.8, 0.9, 50)
+        with pytest.raises(ophip.LaunchError) as e:
+            rs.launch(a, None, stream)
+        assert e.value.kind == "ArgsNotSupport", missing
+    stream.synchronize()
