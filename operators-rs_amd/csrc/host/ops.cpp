@@ -106,6 +106,7 @@ extern "C" void ophip_rms_norm_destroy(ophip_rms_norm *op) { delete op; }
 
 extern "C" int ophip_rms_norm_scheme(ophip_rms_norm *op, const ophip_rms_norm_args *args, size_t, size_t *ws) {
     return guard([&] {
+        if (!op || !args) throw args_not_support("null argument");
         if (ws) *ws = 0;
         const RmsNormMeta m = rms_norm_meta(*args);
         const size_t d = static_of(m.d);  // rms_norm/cuda/mod.rs:38-39
@@ -117,6 +118,7 @@ extern "C" int ophip_rms_norm_scheme(ophip_rms_norm *op, const ophip_rms_norm_ar
 extern "C" int ophip_rms_norm_launch(const ophip_rms_norm *op, const ophip_rms_norm_args *args, void *, size_t,
                                      const ophip_queue_alloc *qa) {
     return guard([&] {
+        if (!op || !args) throw args_not_support("null argument");
         const RmsNormMeta m = rms_norm_meta(*args);
         const size_t n = static_of(m.n), d = static_of(m.d);
         const ptrdiff_t nsy = static_of(args->y_layout.strides[0]), dsy = static_of(args->y_layout.strides[1]);
@@ -237,6 +239,7 @@ extern "C" void ophip_rope_destroy(ophip_rope *op) { delete op; }
 
 extern "C" int ophip_rope_scheme(ophip_rope *, const ophip_rope_args *args, size_t, size_t *ws) {
     return guard([&] {
+        if (!args) throw args_not_support("null argument");
         if (ws) *ws = 0;
         (void)rope_meta(*args);
     });
@@ -245,6 +248,7 @@ extern "C" int ophip_rope_scheme(ophip_rope *, const ophip_rope_args *args, size
 extern "C" int ophip_rope_launch(const ophip_rope *op, const ophip_rope_args *args, void *, size_t,
                                  const ophip_queue_alloc *qa) {
     return guard([&] {
+        if (!op || !args) throw args_not_support("null argument");
         const RopeMeta m = rope_meta(*args);
         // (bf16: in neither backend of the reference; the f16 kernels on bf16 elements)
         if (m.dt_t != OPHIP_DT_F16 && m.dt_t != OPHIP_DT_BF16 && m.dt_t != OPHIP_DT_F32 && m.dt_t != OPHIP_DT_F64)
@@ -388,6 +392,7 @@ extern "C" void ophip_fused_softmax_destroy(ophip_fused_softmax *op) { delete op
 extern "C" int ophip_fused_softmax_scheme(ophip_fused_softmax *, const ophip_fused_softmax_args *args, size_t,
                                           size_t *ws) {
     return guard([&] {
+        if (!args) throw args_not_support("null argument");
         if (ws) *ws = 0;
         if (args->att_layout.ndim != 3) throw rank_not_support("");
         const uint64_t dt = args->att_layout.dt;
@@ -399,6 +404,7 @@ extern "C" int ophip_fused_softmax_scheme(ophip_fused_softmax *, const ophip_fus
 extern "C" int ophip_fused_softmax_launch(const ophip_fused_softmax *op, const ophip_fused_softmax_args *args, void *,
                                           size_t, const ophip_queue_alloc *qa) {
     return guard([&] {
+        if (!op || !args) throw args_not_support("null argument");
         const ophip_tensor_layout &l = args->att_layout;
         if (l.ndim != 3) throw rank_not_support("");
         // (bf16: in neither backend of the reference; the f16 kernels on bf16 elements)
@@ -586,6 +592,7 @@ extern "C" int ophip_rearrange_scheme(ophip_rearrange *, const ophip_rearrange_a
 extern "C" int ophip_rearrange_launch(const ophip_rearrange *op, const ophip_rearrange_args *args, void *, size_t,
                                       const ophip_queue_alloc *qa) {
     return guard([&] {
+        if (!op || !args) throw args_not_support("null argument");
         const RScheme s = rearrange_scheme(*args);
         if (s.unit == 0 || s.count() == 0) return;
         if (!args->dst_base || !args->src_base) throw args_not_support("null base address");
@@ -788,6 +795,7 @@ extern "C" void ophip_swiglu_destroy(ophip_swiglu *op) { delete op; }
 
 extern "C" int ophip_swiglu_scheme(ophip_swiglu *, const ophip_swiglu_args *args, size_t, size_t *ws) {
     return guard([&] {
+        if (!args) throw args_not_support("null argument");
         if (ws) *ws = 0;
         (void)swiglu_meta(*args);
     });
@@ -796,6 +804,7 @@ extern "C" int ophip_swiglu_scheme(ophip_swiglu *, const ophip_swiglu_args *args
 extern "C" int ophip_swiglu_launch(const ophip_swiglu *op, const ophip_swiglu_args *args, void *, size_t,
                                    const ophip_queue_alloc *qa) {
     return guard([&] {
+        if (!op || !args) throw args_not_support("null argument");
         const SwigluMeta m = swiglu_meta(*args);
         // (bf16: in neither backend of the reference; the f16 kernels on bf16 elements)
         if (m.dt != OPHIP_DT_F16 && m.dt != OPHIP_DT_BF16 && m.dt != OPHIP_DT_F32 && m.dt != OPHIP_DT_F64)

@@ -69,6 +69,7 @@ extern "C" void ophip_layer_norm_destroy(ophip_layer_norm *op) { delete op; }
 
 extern "C" int ophip_layer_norm_scheme(ophip_layer_norm *, const ophip_layer_norm_args *args, size_t, size_t *ws) {
     return guard([&] {
+        if (!args) throw args_not_support("null argument");
         if (ws) *ws = 0;
         (void)layer_norm_meta(*args);
     });
@@ -77,6 +78,7 @@ extern "C" int ophip_layer_norm_scheme(ophip_layer_norm *, const ophip_layer_nor
 extern "C" int ophip_layer_norm_launch(const ophip_layer_norm *op, const ophip_layer_norm_args *args, void *, size_t,
                                        const ophip_queue_alloc *qa) {
     return guard([&] {
+        if (!op || !args) throw args_not_support("null argument");
         const LayerNormMeta m = layer_norm_meta(*args);
         const size_t n = static_of(m.n), d = static_of(m.d);
         const ptrdiff_t nsy = static_of(args->y_layout.strides[0]), dsy = static_of(args->y_layout.strides[1]);
@@ -164,6 +166,7 @@ extern "C" void ophip_gelu_destroy(ophip_gelu *op) { delete op; }
 
 extern "C" int ophip_gelu_scheme(ophip_gelu *, const ophip_gelu_args *args, size_t, size_t *ws) {
     return guard([&] {
+        if (!args) throw args_not_support("null argument");
         if (ws) *ws = 0;
         expect_rank(args->layout, "layout", 2);
     });
@@ -172,6 +175,7 @@ extern "C" int ophip_gelu_scheme(ophip_gelu *, const ophip_gelu_args *args, size
 extern "C" int ophip_gelu_launch(const ophip_gelu *op, const ophip_gelu_args *args, void *, size_t,
                                  const ophip_queue_alloc *qa) {
     return guard([&] {
+        if (!op || !args) throw args_not_support("null argument");
         expect_rank(args->layout, "layout", 2);
         const uint64_t dt = args->layout.dt;
         const size_t n = static_of(args->layout.shape[0]), d = static_of(args->layout.shape[1]);
@@ -279,6 +283,7 @@ extern "C" void ophip_add_destroy(ophip_add *op) { delete op; }
 // add/cuda/mod.rs:36-47: only the data types are looked at
 extern "C" int ophip_add_scheme(ophip_add *, const ophip_add_args *args, size_t, size_t *ws) {
     return guard([&] {
+        if (!args) throw args_not_support("null argument");
         if (ws) *ws = 0;
         (void)type_distinct({args->c_layout.dt, args->a_layout.dt, args->b_layout.dt});
     });
@@ -303,6 +308,7 @@ extern "C" int ophip_add_plan(const ophip_add_args *args, ptrdiff_t *out, size_t
 extern "C" int ophip_add_launch(const ophip_add *op, const ophip_add_args *args, void *, size_t,
                                 const ophip_queue_alloc *qa) {
     return guard([&] {
+        if (!op || !args) throw args_not_support("null argument");
         AddScheme s = add_scheme(*args);
         // (bf16, integers, bool: no CPU kernel in the reference, but its CUDA backend adds any named type,
         // add/cuda/mod.rs:105-123)
@@ -399,6 +405,7 @@ extern "C" void ophip_add_rows_destroy(ophip_add_rows *op) { delete op; }
 
 extern "C" int ophip_add_rows_scheme(ophip_add_rows *, const ophip_add_rows_args *args, size_t, size_t *ws) {
     return guard([&] {
+        if (!args) throw args_not_support("null argument");
         if (ws) *ws = 0;
         (void)add_rows_meta(*args);
     });
@@ -407,6 +414,7 @@ extern "C" int ophip_add_rows_scheme(ophip_add_rows *, const ophip_add_rows_args
 extern "C" int ophip_add_rows_launch(const ophip_add_rows *op, const ophip_add_rows_args *args, void *, size_t,
                                      const ophip_queue_alloc *qa) {
     return guard([&] {
+        if (!op || !args) throw args_not_support("null argument");
         const AddRowsMeta r = add_rows_meta(*args);
         const size_t batch = static_of(r.batch), m = static_of(r.m), n = static_of(r.n), k = static_of(r.k);
         const ptrdiff_t bsd = static_of(args->dst_layout.strides[0]), msd = static_of(args->dst_layout.strides[1]),

@@ -61,6 +61,7 @@ struct ophip_random_sample {
 extern "C" {
 
 int ophip_sample_args_new(float temperature, float top_p, size_t top_k, ophip_sample_args *out) {
+    if (!out) return OPHIP_ARGS_NOT_SUPPORT;
     if (temperature < 0.f) return 1;           // NegativeTemperature
     if (top_k == 0 || top_p <= 0.f) return 2;  // NonPositiveTop
     out->temperature = temperature;
@@ -84,6 +85,7 @@ void ophip_random_sample_destroy(ophip_random_sample *op) { delete op; }
 int ophip_random_sample_scheme(ophip_random_sample *, const ophip_random_sample_args *args, size_t max_ws,
                                size_t *ws) {
     return guard([&] {
+        if (!args) throw args_not_support("null argument");
         if (ws) *ws = 0;
         const SampleMeta m = sample_meta(*args);
         if (m.dt != OPHIP_DT_F16 && m.dt != OPHIP_DT_F32) throw type_not_support("logits must be f16 or f32");
@@ -96,6 +98,7 @@ int ophip_random_sample_scheme(ophip_random_sample *, const ophip_random_sample_
 static void sample_launch(const ophip_random_sample *op, const ophip_random_sample_args *args, size_t rows,
                           ptrdiff_t row_stride, const float *seeds, void *workspace, size_t workspace_len,
                           const ophip_queue_alloc *qa) {
+    if (!op || !args) throw args_not_support("null argument");
     const SampleMeta m = sample_meta(*args);
     if (args->kv_pair.ndim != 0) throw rank_error("kv_pair", 0, args->kv_pair.ndim);
     const size_t n = static_of(m.n);

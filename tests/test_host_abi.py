@@ -331,3 +331,22 @@ def test_kernels_that_stride_by_their_workgroup_size_are_launched_with_it():
     host = "".join(open(os.path.join(csrc, "host", f)).read() for f in ("ops.cpp", "ops_more.cpp", "handle.cpp"))
     sizes = set(re.findall(r"launch\([^;]*?Dim3\{[^;]*?\},\s*Dim3\{([^}]*)\}", host, re.S))
     assert sizes <= {"256", "block", "1024", "256u", "1"}, sizes
+
+
+def test_null_operators_and_arguments_come_back_as_status_codes():
+    """A binding that passes a null operator, null arguments or no queue allocator gets ArgsNotSupport from every
+    launch (and a status code, not a crash, from every scheme and create): no device is needed to be refused."""
+    import ctypes
+
+    L = ophip.lib()
+    names = ["rms_norm", "rope", "fused_softmax", "rearrange", "swiglu", "random_sample", "mat_mul", "attention",
+             "attention_kv_cached", "layer_norm", "gelu", "add", "add_rows", "conv"]
+    ws = ctypes.c_size_t(0)
+    for n in names:
+        assert getattr(L, "ophip_%s_create" % n)(None, None) == 8, n
+        assert getattr(L, "ophip_%s_launch" % n)(None, None, None, ctypes.c_size_t(0), None) == 8, n
+        assert getattr(L, "ophip_%s_scheme" % n)(None, None, ctypes.c_size_t(0), ctypes.byref(ws)) in (0, 8), n
+        getattr(L, "ophip_%s_destroy" % n)(None)
+    assert L.ophip_random_sample_launch_batch(None, None, ctypes.c_size_t(1), ctypes.c_ssize_t(0), None, None, ctypes.c_size_t(0), None) == 8
+    assert L.ophip_mat_mul_launch_static(None, None, None) == 8
+    assert L.ophip_sample_args_new(ctypes.c_float(1.0), ctypes.c_float(1.0), ctypes.c_size_t(1), None) == 8
