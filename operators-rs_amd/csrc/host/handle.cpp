@@ -184,6 +184,17 @@ ophip_device::~ophip_device() {
     for (auto &m : modules) (void)hipModuleUnload(m.second);
 }
 
+// A null device (or a null place for the result) from a binding comes back as a status, like every other bad argument.
+static ophip_device *need(ophip_device *dev) {
+    if (!dev) throw args_not_support("null device");
+    return dev;
+}
+template <typename T>
+static T *need_out(T *out) {
+    if (!out) throw args_not_support("null argument");
+    return out;
+}
+
 extern "C" {
 
 const char *ophip_last_error(void) { return g_last_error.c_str(); }
@@ -269,21 +280,22 @@ int ophip_device_get_info(const ophip_device *dev, ophip_device_info *out) {
 
 int ophip_malloc(ophip_device *dev, size_t size, void **out) {
     return guard([&] {
-        dev->make_current();
-        *out = nullptr;
+        need(dev)->make_current();
+        *need_out(out) = nullptr;
         if (size) check_hip(hipMalloc(out, size), "hipMalloc");
     });
 }
 int ophip_free(ophip_device *dev, void *ptr) {
     return guard([&] {
-        dev->make_current();
+        need(dev)->make_current();
         if (ptr) check_hip(hipFree(ptr), "hipFree");
     });
 }
 static int copy(ophip_device *dev, void *dst, const void *src, size_t size, ophip_stream stream, hipMemcpyKind kind) {
     return guard([&] {
-        dev->make_current();
+        need(dev)->make_current();
         if (!size) return;
+        if (!dst || !src) throw args_not_support("null pointer");
         // hipMemcpyAsync on the caller's stream; a null stream makes the call synchronous: the data is in
         // place when it returns.  HIP does not promise that a copy between device buffers or a fill has
         // finished when hipMemcpy / hipMemset return, and work on the caller's own (non-blocking) streams
@@ -307,8 +319,9 @@ int ophip_memcpy_d2d(ophip_device *dev, void *dst, const void *src, size_t size,
 }
 int ophip_memset(ophip_device *dev, void *dst, int value, size_t size, ophip_stream stream) {
     return guard([&] {
-        dev->make_current();
+        need(dev)->make_current();
         if (!size) return;
+        if (!dst) throw args_not_support("null pointer");
         if (stream) {
             // a kernel, not hipMemsetAsync: callers record their streams into graphs, and a fill that is an
             // ordinary kernel node replays like every other launch
@@ -329,15 +342,16 @@ int ophip_memset(ophip_device *dev, void *dst, int value, size_t size, ophip_str
 }
 int ophip_stream_create(ophip_device *dev, ophip_stream *out) {
     return guard([&] {
-        dev->make_current();
+        need(dev)->make_current();
         hipStream_t s;
+        need_out(out);
         check_hip(hipStreamCreateWithFlags(&s, hipStreamNonBlocking), "hipStreamCreate");
         *out = s;
     });
 }
 int ophip_stream_destroy(ophip_device *dev, ophip_stream stream) {
     return guard([&] {
-        dev->make_current();
+        need(dev)->make_current();
         // What the hooks hand on to other streams (mat_mul's arrival counters) must be at rest first.  The wait happens
         // before the lock is taken, so that creating or destroying an operator on this device never waits for this
         // stream's work.  A stream that is still recording cannot be waited for; its buffers are then not handed on
@@ -357,40 +371,44 @@ int ophip_stream_destroy(ophip_device *dev, ophip_stream stream) {
 }
 int ophip_stream_synchronize(ophip_device *dev, ophip_stream stream) {
     return guard([&] {
-        dev->make_current();
+        need(dev)->make_current();
         check_hip(hipStreamSynchronize((hipStream_t)stream), "hipStreamSynchronize");
     });
 }
 int ophip_event_create(ophip_device *dev, ophip_event *out) {
     return guard([&] {
-        dev->make_current();
+        need(dev)->make_current();
         hipEvent_t e;
+        need_out(out);
         check_hip(hipEventCreate(&e), "hipEventCreate");
         *out = e;
     });
 }
 int ophip_event_destroy(ophip_device *dev, ophip_event ev) {
     return guard([&] {
-        dev->make_current();
-        check_hip(hipEventDestroy((hipEvent_t)ev), "hipEventDestroy");
+        need(dev)->make_current();
+        if (ev) check_hip(hipEventDestroy((hipEvent_t)ev), "hipEventDestroy");
     });
 }
 int ophip_event_record(ophip_device *dev, ophip_event ev, ophip_stream stream) {
     return guard([&] {
-        dev->make_current();
+        need(dev)->make_current();
+        if (!ev) throw args_not_support("null event");
         check_hip(hipEventRecord((hipEvent_t)ev, (hipStream_t)stream), "hipEventRecord");
     });
 }
 int ophip_event_synchronize(ophip_device *dev, ophip_event ev) {
     return guard([&] {
-        dev->make_current();
+        need(dev)->make_current();
+        if (!ev) throw args_not_support("null event");
         check_hip(hipEventSynchronize((hipEvent_t)ev), "hipEventSynchronize");
     });
 }
 int ophip_event_elapsed_ms(ophip_device *dev, ophip_event start, ophip_event stop, float *ms) {
     return guard([&] {
-        dev->make_current();
-        check_hip(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop), "hipEventElapsedTime");
+        need(dev)->make_current();
+        if (!start || !stop) throw args_not_support("null event");
+        check_hip(hipEventElapsedTime(need_out(ms), (hipEvent_t)start, (hipEvent_t)stop), "hipEventElapsedTime");
     });
 }
 
@@ -409,14 +427,15 @@ int ophip_time_next_launch(ophip_device *dev, ophip_stream stream, ophip_event s
 // the caller's stream, so a fixed sequence of them can be recorded once and replayed.
 int ophip_stream_begin_capture(ophip_device *dev, ophip_stream stream) {
     return guard([&] {
-        dev->make_current();
+        need(dev)->make_current();
         check_hip(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture");
     });
 }
 int ophip_stream_end_capture(ophip_device *dev, ophip_stream stream, ophip_graph *out) {
     return guard([&] {
-        dev->make_current();
+        need(dev)->make_current();
         hipGraph_t graph = nullptr;
+        need_out(out);
         check_hip(hipStreamEndCapture((hipStream_t)stream, &graph), "hipStreamEndCapture");
         hipGraphExec_t exec = nullptr;
         const hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
@@ -427,14 +446,15 @@ int ophip_stream_end_capture(ophip_device *dev, ophip_stream stream, ophip_graph
 }
 int ophip_graph_launch(ophip_device *dev, ophip_graph graph, ophip_stream stream) {
     return guard([&] {
-        dev->make_current();
+        need(dev)->make_current();
+        if (!graph) throw args_not_support("null graph");
         check_hip(hipGraphLaunch((hipGraphExec_t)graph, (hipStream_t)stream), "hipGraphLaunch");
     });
 }
 int ophip_graph_destroy(ophip_device *dev, ophip_graph graph) {
     return guard([&] {
-        dev->make_current();
-        check_hip(hipGraphExecDestroy((hipGraphExec_t)graph), "hipGraphExecDestroy");
+        need(dev)->make_current();
+        if (graph) check_hip(hipGraphExecDestroy((hipGraphExec_t)graph), "hipGraphExecDestroy");
     });
 }
 
@@ -549,9 +569,11 @@ ophip_offset_calculator *ophip_offset_calculator_create(size_t alignment) {
     return c;
 }
 void ophip_offset_calculator_destroy(ophip_offset_calculator *c) { delete c; }
-void ophip_offset_calculator_put(ophip_offset_calculator *c, size_t start, size_t end) { c->put(start, end); }
+void ophip_offset_calculator_put(ophip_offset_calculator *c, size_t start, size_t end) {
+    if (c) c->put(start, end);
+}
 int ophip_offset_calculator_take(ophip_offset_calculator *c, size_t size, size_t *start, size_t *end) {
-    return c->take(size, start, end) ? 1 : 0;
+    return c && start && end && c->take(size, start, end) ? 1 : 0;
 }
 
 int ophip_mem_pool_create(ophip_device *dev, ophip_stream stream, ophip_mem_pool **out) {
@@ -567,6 +589,7 @@ int ophip_mem_pool_create(ophip_device *dev, ophip_stream stream, ophip_mem_pool
 }
 int ophip_mem_pool_put(ophip_mem_pool *pool, size_t size) {
     return guard([&] {
+        if (!pool) throw args_not_support("null argument");
         pool->dev->make_current();
         void *p = nullptr;
         check_hip(hipMalloc(&p, size), "hipMalloc");

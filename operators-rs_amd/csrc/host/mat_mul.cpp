@@ -625,7 +625,10 @@ const ophip_device *mat_mul_device(const ophip_mat_mul *op) { return op->dev; }
 extern "C" {
 
 int ophip_mat_mul_plan(const ophip_mat_mul_args *args, ophip_mat_mul_layout *out) {
-    return guard([&] { *out = mat_mul_layout(*args); });
+    return guard([&] {
+        if (!args || !out) throw args_not_support("null argument");
+        *out = mat_mul_layout(*args);
+    });
 }
 
 int ophip_mat_mul_create(ophip_device *dev, ophip_mat_mul **out) {

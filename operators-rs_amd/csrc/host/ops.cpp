@@ -547,6 +547,7 @@ RScheme rearrange_scheme(const ophip_rearrange_args &a) {
 
 extern "C" int ophip_rearrange_plan(const ophip_rearrange_args *args, ptrdiff_t *out, size_t *ndim_out) {
     return guard([&] {
+        if (!args || !out) throw args_not_support("null argument");
         const RScheme s = rearrange_scheme(*args);
         const size_t nd = s.ndim();
         out[0] = (ptrdiff_t)s.unit;

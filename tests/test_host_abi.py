@@ -350,3 +350,28 @@ def test_null_operators_and_arguments_come_back_as_status_codes():
     assert L.ophip_random_sample_launch_batch(None, None, ctypes.c_size_t(1), ctypes.c_ssize_t(0), None, None, ctypes.c_size_t(0), None) == 8
     assert L.ophip_mat_mul_launch_static(None, None, None) == 8
     assert L.ophip_sample_args_new(ctypes.c_float(1.0), ctypes.c_float(1.0), ctypes.c_size_t(1), None) == 8
+    # the handle: a null device, or nowhere to put the result
+    Z = ctypes.c_size_t(0)
+    handle_calls = {
+        "device_get_info": lambda: L.ophip_device_get_info(None, None), "malloc": lambda: L.ophip_malloc(None, Z, None),
+        "free": lambda: L.ophip_free(None, None), "memcpy_h2d": lambda: L.ophip_memcpy_h2d(None, None, None, Z, None),
+        "memcpy_d2h": lambda: L.ophip_memcpy_d2h(None, None, None, Z, None), "memcpy_d2d": lambda: L.ophip_memcpy_d2d(None, None, None, Z, None),
+        "memset": lambda: L.ophip_memset(None, None, 0, Z, None), "stream_create": lambda: L.ophip_stream_create(None, None),
+        "stream_destroy": lambda: L.ophip_stream_destroy(None, None), "stream_synchronize": lambda: L.ophip_stream_synchronize(None, None),
+        "event_create": lambda: L.ophip_event_create(None, None), "event_record": lambda: L.ophip_event_record(None, None, None),
+        "event_synchronize": lambda: L.ophip_event_synchronize(None, None), "event_elapsed_ms": lambda: L.ophip_event_elapsed_ms(None, None, None, None),
+        "event_destroy": lambda: L.ophip_event_destroy(None, None), "time_next_launch": lambda: L.ophip_time_next_launch(None, None, None, None),
+        "stream_begin_capture": lambda: L.ophip_stream_begin_capture(None, None), "stream_end_capture": lambda: L.ophip_stream_end_capture(None, None, None),
+        "graph_launch": lambda: L.ophip_graph_launch(None, None, None), "graph_destroy": lambda: L.ophip_graph_destroy(None, None),
+        "queue_alloc_from_stream": lambda: L.ophip_queue_alloc_from_stream(None, None, None), "mem_pool_create": lambda: L.ophip_mem_pool_create(None, None, None),
+        "mem_pool_put": lambda: L.ophip_mem_pool_put(None, Z), "mem_pool_queue_alloc": lambda: L.ophip_mem_pool_queue_alloc(None, None),
+        "rope_build_pos": lambda: L.ophip_rope_build_pos(ctypes.c_uint64(0), Z, None, Z, None, None), "rearrange_plan": lambda: L.ophip_rearrange_plan(None, None, None),
+        "random_sample_build_indices": lambda: L.ophip_random_sample_build_indices(Z, None, None), "mat_mul_plan": lambda: L.ophip_mat_mul_plan(None, None),
+        "mat_mul_describe": lambda: L.ophip_mat_mul_describe(None, None, None, Z), "add_plan": lambda: L.ophip_add_plan(None, None, None),
+        "device_create": lambda: L.ophip_device_create(0, None, None),
+    }
+    for name, call in handle_calls.items():
+        assert call() == 8, name
+    L.ophip_mem_pool_destroy(None), L.ophip_device_release(None), L.ophip_device_retain(None)
+    L.ophip_offset_calculator_put(None, Z, Z)
+    assert L.ophip_offset_calculator_take(None, Z, None, None) == 0
