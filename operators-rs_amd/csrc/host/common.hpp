@@ -95,8 +95,13 @@ inline Error rank_error(const char *arg, size_t expected, size_t actual) {
                             std::to_string(expected) + " expected");
 }
 
+// A layout of non-zero rank has to bring its shape and strides (a binding that leaves the pointers null gets a status).
+inline void expect_arrays(const ophip_tensor_layout &l) {
+    if (l.ndim != 0 && (!l.shape || !l.strides)) throw args_not_support("a layout without shape or strides");
+}
 inline void expect_rank(const ophip_tensor_layout &l, const char *name, size_t rank) {
     if (l.ndim != rank) throw rank_error(name, rank, l.ndim);
+    expect_arrays(l);
 }
 
 inline bool is_float_dtype(uint64_t dt) {

@@ -24,6 +24,7 @@ struct Matrix {  // mat_mul/args.rs:124-192, strides in elements
     ptrdiff_t rs, cs;
 
     static Matrix from(const ophip_tensor_layout &t) {
+        expect_arrays(t);
         for (size_t i = 0; i < t.ndim; ++i)
             if (is_dyn(t.shape[i]) || is_dyn(t.strides[i])) throw dyn_not_support("");
         if (t.ndim < 2) throw rank_not_support("Matrix must have rank 2 or more");

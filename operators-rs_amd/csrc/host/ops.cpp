@@ -395,6 +395,7 @@ extern "C" int ophip_fused_softmax_scheme(ophip_fused_softmax *, const ophip_fus
         if (!args) throw args_not_support("null argument");
         if (ws) *ws = 0;
         if (args->att_layout.ndim != 3) throw rank_not_support("");
+        expect_arrays(args->att_layout);
         const uint64_t dt = args->att_layout.dt;
         if (dt != OPHIP_DT_F16 && dt != OPHIP_DT_BF16 && dt != OPHIP_DT_F32 && dt != OPHIP_DT_F64)
             throw type_not_support("fused softmax supports f16, bf16, f32 and f64");
@@ -407,6 +408,7 @@ extern "C" int ophip_fused_softmax_launch(const ophip_fused_softmax *op, const o
         if (!op || !args) throw args_not_support("null argument");
         const ophip_tensor_layout &l = args->att_layout;
         if (l.ndim != 3) throw rank_not_support("");
+        expect_arrays(l);
         // (bf16: in neither backend of the reference; the f16 kernels on bf16 elements)
         if (l.dt != OPHIP_DT_F16 && l.dt != OPHIP_DT_BF16 && l.dt != OPHIP_DT_F32 && l.dt != OPHIP_DT_F64)
             throw type_not_support("fused softmax supports f16, bf16, f32 and f64");
@@ -489,6 +491,8 @@ ptrdiff_t iabs(ptrdiff_t v) { return v < 0 ? -v : v; }
 RScheme rearrange_scheme(const ophip_rearrange_args &a) {
     const ophip_tensor_layout &D = a.dst_layout, &S = a.src_layout;
     (void)type_distinct({D.dt, S.dt});
+    expect_arrays(D);
+    expect_arrays(S);
     if (D.ndim != S.ndim)
         throw rank_mismatch("dst.ndim = " + std::to_string(D.ndim) + ", src.ndim = " + std::to_string(S.ndim));
     std::vector<RDim> dims;

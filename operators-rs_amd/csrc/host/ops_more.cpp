@@ -238,6 +238,9 @@ AddScheme add_scheme(const ophip_add_args &args) {
     AddScheme s;
     s.dt = type_distinct({c.dt, a.dt, b.dt});
     const size_t ndim = c.ndim;
+    expect_arrays(c);
+    expect_arrays(a);
+    expect_arrays(b);
     if (a.ndim != ndim || b.ndim != ndim)
         throw rank_mismatch("c.ndim = " + std::to_string(c.ndim) + ", a.ndim = " + std::to_string(a.ndim) +
                             ", b.ndim = " + std::to_string(b.ndim));

@@ -350,6 +350,28 @@ def test_null_operators_and_arguments_come_back_as_status_codes():
     assert L.ophip_random_sample_launch_batch(None, None, ctypes.c_size_t(1), ctypes.c_ssize_t(0), None, None, ctypes.c_size_t(0), None) == 8
     assert L.ophip_mat_mul_launch_static(None, None, None) == 8
     assert L.ophip_sample_args_new(ctypes.c_float(1.0), ctypes.c_float(1.0), ctypes.c_size_t(1), None) == 8
+    # layouts of non-zero rank that bring no shape or strides
+    empty = ophip._Layout(ctypes.c_uint64(int(dt.F16)), ctypes.c_uint64(3), None, None)
+
+    class NoArrays:
+        def c(self):
+            return empty
+
+    b = NoArrays()
+    makers = {"rms_norm": lambda: ophip.RmsNormArgs(b, None, b, None, b, None, 1e-5), "rope": lambda: ophip.RopeArgs(b, None, b, None, b, None, b, None, 1e4),
+              "fused_softmax": lambda: ophip.FusedSoftmaxArgs(1, b, None), "swiglu": lambda: ophip.SwigluArgs(b, None, b, None),
+              "attention": lambda: ophip.AttentionArgs(b, None, b, None, b, None, b, None, 1),
+              "attention_kv_cached": lambda: ophip.AttnKVCachedArgs(b, None, b, None, b, None, b, None, b, None, b, None, 1, 0),
+              "layer_norm": lambda: ophip.LayerNormArgs(b, None, b, None, b, None, b, None, 1e-5), "gelu": lambda: ophip.GeluArgs(b, None),
+              "add_rows": lambda: ophip.AddRowsArgs(b, None, b, None, b, None)}
+    for rank in (1, 2, 3):
+        empty.ndim = rank
+        for n, make in makers.items():
+            args = make().c()
+            assert getattr(L, "ophip_%s_scheme" % n)(None, ctypes.byref(args), ctypes.c_size_t(0), ctypes.byref(ws)) != 0, (n, rank)
+        for plan, make in (("ophip_mat_mul_plan", lambda: ophip.MatMulArgs(b, None, 0.0, b, None, b, None, 1.0)),):
+            out = ophip.MatMulLayout()
+            assert getattr(L, plan)(ctypes.byref(make().c()), ctypes.byref(out)) != 0, rank
     # the handle: a null device, or nowhere to put the result
     Z = ctypes.c_size_t(0)
     handle_calls = {
