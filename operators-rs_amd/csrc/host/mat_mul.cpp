@@ -652,6 +652,7 @@ int ophip_mat_mul_scheme(ophip_mat_mul *op, const ophip_mat_mul_args *args, size
         try {
             const ophip_mat_mul_layout L = mat_mul_layout(*args);
             if (!mat_mul_takes(L.dt)) return;
+            if (L.m == 0 || L.n == 0 || L.batch == 0) return;  // nothing to compute, nothing to plan (launch returns at once)
             const GemmPlan g = make_plan(*args, L, (unsigned)op->dev->props.multiProcessorCount, op->knobs);
             if (ws && g.workspace <= max_ws) *ws = g.workspace;
         } catch (const Error &) {
@@ -664,6 +665,10 @@ int ophip_mat_mul_describe(const ophip_mat_mul *op, const ophip_mat_mul_args *ar
         if (!args || !out || len == 0) throw args_not_support("null argument");
         const ophip_mat_mul_layout L = mat_mul_layout(*args);
         if (!mat_mul_takes(L.dt)) throw type_not_support("mat_mul supports f16, bf16, f32 and f64");
+        if (L.m == 0 || L.n == 0 || L.batch == 0) {
+            std::snprintf(out, len, "empty");
+            return;
+        }
         const GemmPlan g = op ? make_plan(*args, L, (unsigned)op->dev->props.multiProcessorCount, op->knobs)
                               : make_plan(*args, L, 256u, GemmKnobs::from_env());
         if (g.kind == GemmPlan::Skinny)

@@ -354,3 +354,26 @@ def test_one_null_base_is_refused_by_every_launch(gpu, stream):
             rs.launch(a, None, stream)
         assert e.value.kind == "ArgsNotSupport", missing
     stream.synchronize()
+
+
+def test_mat_mul_with_nothing_to_multiply(gpu, stream):
+    """Empty products: zero rows, columns or batches plan nothing and launch nothing (scheme once divided by the number
+    of column strips, which was zero); K = 0 leaves c = beta * c."""
+    c = lambda *s: TensorLayout.new_contiguous(dt.F16, list(s))
+    op = ophip.MatMul(gpu)
+    for bt, m, n, k in ((1, 0, 128, 64), (1, 16, 0, 64), (0, 16, 128, 64), (3, 0, 0, 0)):
+        a, b, cc = gpu.malloc(max(1, bt * m * k * 2)), gpu.malloc(max(1, bt * k * n * 2)), gpu.malloc(max(1, bt * m * n * 2))
+        args = ophip.MatMulArgs(c(bt, m, n), cc, 0.5, c(bt, m, k), a, c(bt, k, n), b, 1.0)
+        say("mat_mul %dx(%dx%dx%d)" % (bt, m, n, k))
+        assert op.scheme(args, 2 ** 40) == 0
+        assert op.describe(args) == "empty"
+        op.launch(args, None, stream)
+    for bt, m, n in ((1, 16, 128), (2, 300, 300)):
+        c0 = normal_f16(np.random.default_rng(m), (bt, m, n))
+        cd, a, b = gpu.from_host(c0), gpu.malloc(16), gpu.malloc(16)
+        args = ophip.MatMulArgs(c(bt, m, n), cd, 0.5, c(bt, m, 0), a, c(bt, 0, n), b, 1.0)
+        say("mat_mul %dx(%dx%dx0)" % (bt, m, n))
+        op.scheme(args, 2 ** 40)
+        op.launch(args, None, stream)
+        got = gpu.to_host(cd, f16, c0.size, stream=stream).reshape(c0.shape)
+        assert np.array_equal(got, (c0.astype(f32) * f32(0.5)).astype(f16))
