@@ -800,3 +800,64 @@ def test_random_launches_need_no_more_workspace_than_scheme_reports(gpu, stream,
             assert int(kv[0]) < n
         with_workspace += need > 0
     assert with_workspace >= 8
+
+
+@SWEEPS
+def test_random_and_mostly_invalid_arguments_come_back_as_status_codes(gpu, stream, sweep):
+    """Layouts drawn at random (ranks, types, zero, huge and dynamic extents, zero, negative, misaligned and dynamic
+    strides; every so often a plausible contiguous tensor with one entry disturbed) into scheme and launch of every
+    operator, all bases null: each call ends in a status code (a launch in ArgsNotSupport at the latest), never in a
+    kernel and never in a crash of the host side."""
+    rng = np.random.default_rng(257 + 1000 * sweep)
+    types = [dt.F16, dt.F32, dt.F64, dt.BF16, dt.U8, dt.U32, dt.U64, dt.I32, dt.BOOL, dt.KVPAIR]
+    extents = [0, 1, 2, 3, 7, 8, 16, 64, 128, 4096, 2 ** 31, 2 ** 40, None]
+    steps = [0, 1, 2, 4, 8, -2, -8, 6, 256, 8192, 2 ** 33, -(2 ** 33), None]
+    small = [1, 2, 3, 8, 16, 64]
+
+    def lay(rank, typ=dt.F16):
+        nd = rank if rng.integers(0, 8) else int(rng.integers(0, 5))
+        typ = types[int(rng.integers(0, len(types)))] if rng.integers(0, 6) == 0 else typ
+        if rng.integers(0, 2):  # contiguous, one entry disturbed now and then
+            shape = [int(rng.choice(small)) for _ in range(nd)]
+            strides, m = [], ophip.dtype_nbytes(typ)
+            for n in reversed(shape):
+                strides.insert(0, m)
+                m *= n
+            if nd and rng.integers(0, 2):
+                i = int(rng.integers(0, nd))
+                if rng.integers(0, 2):
+                    shape[i] = extents[int(rng.integers(0, len(extents)))]
+                else:
+                    strides[i] = steps[int(rng.integers(0, len(steps)))]
+            return TensorLayout(typ, shape, strides)
+        return TensorLayout(typ, [extents[int(rng.integers(0, len(extents)))] for _ in range(nd)], [steps[int(rng.integers(0, len(steps)))] for _ in range(nd)])
+
+    same = lambda make: make(int(rng.integers(0, 5)))
+    ops = [
+        (ophip.RmsNorm(gpu), lambda: ophip.RmsNormArgs(lay(2), None, lay(2), None, lay(1), None, 1e-5)),
+        (ophip.Rope(gpu), lambda: ophip.RopeArgs(lay(3), None, lay(1, dt.U32), None, lay(2), None, lay(2), None, 1e4)),
+        (ophip.FusedSoftmax(gpu), lambda: ophip.FusedSoftmaxArgs(int(rng.integers(0, 4)), lay(3), None)),
+        (ophip.Rearrange(gpu), lambda: same(lambda n: ophip.RearrangeArgs(lay(n), None, lay(n), None))),
+        (ophip.Swiglu(gpu), lambda: ophip.SwigluArgs(lay(2), None, lay(2), None)),
+        (ophip.MatMul(gpu), lambda: same(lambda n: ophip.MatMulArgs(lay(2 + n % 2), None, 0.5, lay(2 + n % 2), None, lay(2 + n % 2), None, 1.0))),
+        (ophip.Attention(gpu), lambda: ophip.AttentionArgs(lay(3), None, lay(3), None, lay(3), None, lay(3), None, int(rng.integers(0, 3)))),
+        (ophip.AttnKVCached(gpu), lambda: ophip.AttnKVCachedArgs(lay(3), None, lay(3), None, lay(3), None, lay(3), None, lay(3), None, lay(3), None,
+                                                                 int(rng.integers(0, 3)), [0, 5, 2 ** 40, None][int(rng.integers(0, 4))])),
+        (ophip.LayerNorm(gpu), lambda: ophip.LayerNormArgs(lay(2), None, lay(2), None, lay(1), None, lay(1), None, 1e-5)),
+        (ophip.Gelu(gpu), lambda: ophip.GeluArgs(lay(2), None)),
+        (ophip.Add(gpu), lambda: same(lambda n: ophip.AddArgs(lay(n), None, lay(n), None, lay(n), None))),
+        (ophip.AddRows(gpu), lambda: ophip.AddRowsArgs(lay(3), None, lay(2), None, lay(2, dt.U32), None)),
+    ]
+    outcomes = set()
+    for it in range(1800):
+        op, make = ops[it % len(ops)]
+        small[:] = [int(rng.choice([1, 2, 8, 16, 64]))] if rng.integers(0, 4) else [1, 2, 3, 8, 16, 64]
+        args = make()
+        for verb in ("scheme", "launch"):
+            try:
+                op.scheme(args, [0, 1 << 20, 2 ** 40][int(rng.integers(0, 3))]) if verb == "scheme" else op.launch(args, None, stream)
+                outcomes.add("ok")
+            except (ophip.SchemeError, ophip.LaunchError) as e:
+                outcomes.add(e.kind)
+    stream.synchronize()
+    assert len(outcomes) >= 6, outcomes  # the draws reach well past the first check
