@@ -3,7 +3,7 @@
 // against this file instead of libamdhip64 and run unchanged.
 //
 //   * device memory is host memory, every allocation between two inaccessible pages with its end against the upper one
-//     (rounded up to 256 bytes), filled with 0xFE (a NaN in every floating-point type the kernels use): an access past
+//     (rounded up to 256 bytes, or to what CPUSIM_ALIGN says), filled with 0xFE (a NaN in every floating-point type the kernels use): an access past
 //     an allocation, before it or after hipFree stops the process with the address and the nearest allocation;
 //   * streams run in order at once: a launch returns when the kernel has run (cpusim_core.h runs it);
 //   * a stream that records keeps the launches and copies; a graph replays them;
@@ -96,7 +96,15 @@ hipError_t sim_malloc(void **ptr, size_t size) {
     if (!ptr) return hipErrorInvalidValue;
     std::lock_guard<std::recursive_mutex> lock(g_mu);
     install_fault_handler();
-    const size_t user_len = (std::max<size_t>(size, 1) + 255) / 256 * 256;
+    // hipMalloc hands out addresses on 256-byte boundaries; CPUSIM_ALIGN=16 (or another power of two) gives up that
+    // much of it and moves the end of an allocation to within 15 bytes of the guard page: what reads past an
+    // operand by a vector or two then shows
+    static const size_t align = [] {
+        const char *e = std::getenv("CPUSIM_ALIGN");
+        const size_t a = e ? (size_t)std::atoi(e) : 256;
+        return a >= 16 && a <= 4096 && (a & (a - 1)) == 0 ? a : 256;
+    }();
+    const size_t user_len = (std::max<size_t>(size, 1) + align - 1) / align * align;
     const size_t body = (user_len + 4095) / 4096 * 4096, map_len = body + 2 * 4096;
     // keep a runaway test from taking the machine's memory: 24 GiB of live allocations, or CPUSIM_MEMORY_GIB
     static const size_t cap = [] {
