@@ -11,7 +11,7 @@
 // small zero-filled operands and destroyed once (so that an AddressSanitizer build with leak detection sees the whole
 // life of each).  Exit status 0 when every result agreed; a data race ends the run through the sanitizer.
 //
-//   threads_driver [threads = 4] [rounds = 12]
+//   threads_driver [threads = 4] [rounds = 12] [large: any third argument adds a 4096 x 4096 x 64 product, for the 256 x 256 tile]
 #include <atomic>
 #include <cmath>
 #include <cstdio>
@@ -115,7 +115,7 @@ void worker(const Shared &sh, int id, int rounds) {
 
 // Every other operator once, on one thread, small shapes, zero-filled operands (what they compute is the parity tests'
 // business): created, planned, launched, destroyed, so that a sanitizer build sees the whole life of each.
-int every_operator_once(ophip_device *dev) {
+int every_operator_once(ophip_device *dev, bool large) {
 #define TRY(call)                                                                     \
     do {                                                                              \
         const int rc_ = (call);                                                       \
@@ -245,6 +245,132 @@ int every_operator_once(ophip_device *dev) {
         TRY(ophip_attention_kv_cached_launch(kc, &c, nullptr, 0, &qa));
         ophip_attention_kv_cached_destroy(kc);
     }
+    {
+        // More shapes of the row operators, attention and sampling, for the kernel variants the small ones above do not
+        // reach (wide rows on 256 and 1024 work-items, rows streamed in sweeps, many short rows, prefill blocks of 128
+        // query rows at both head dimensions, decode over several chunks of keys, long candidate lists, the full sort);
+        // operands are zeros: what is watched here is where the kernels read and write
+        const size_t rows_shapes[][2] = {{4, 4096}, {2, 16384}, {1, 70000}, {300, 24}, {9000, 256}};
+        for (const auto &rs : rows_shapes) {
+            const size_t n = rs[0], dd = rs[1];
+            const size_t s2r[2] = {n, dd}, s1r[1] = {dd};
+            const ptrdiff_t t2r[2] = {(ptrdiff_t)(dd * 2), 2}, t1r[1] = {2};
+            const ophip_tensor_layout m2{OPHIP_DT_F16, 2, s2r, t2r}, v1{OPHIP_DT_F16, 1, s1r, t1r};
+            void *x = zeros(n * dd * 2), *y = zeros(n * dd * 2), *w = zeros(dd * 2);
+            ophip_rms_norm *rn = nullptr;
+            TRY(ophip_rms_norm_create(dev, &rn));
+            ophip_rms_norm_args ra{};
+            ra.y_layout = ra.x_layout = m2, ra.w_layout = v1, ra.y_base = y, ra.x_base = x, ra.w_base = w, ra.epsilon = 1e-5f;
+            TRY(ophip_rms_norm_launch(rn, &ra, nullptr, 0, &qa));
+            ophip_rms_norm_destroy(rn);
+            ophip_layer_norm *ln = nullptr;
+            TRY(ophip_layer_norm_create(dev, &ln));
+            ophip_layer_norm_args la{};
+            la.y_layout = la.x_layout = m2, la.scale_layout = la.bias_layout = v1, la.y_base = y, la.x_base = x, la.scale_base = w, la.bias_base = w, la.epsilon = 1e-5f;
+            TRY(ophip_layer_norm_launch(ln, &la, nullptr, 0, &qa));
+            ophip_layer_norm_destroy(ln);
+            ophip_fused_softmax *sm = nullptr;
+            TRY(ophip_fused_softmax_create(dev, &sm));
+            const size_t s3r[3] = {1, n, dd};
+            const ptrdiff_t t3r[3] = {(ptrdiff_t)(n * dd * 2), (ptrdiff_t)(dd * 2), 2};
+            ophip_fused_softmax_args sa2{};
+            sa2.att_mask = n <= dd ? 1 : 0, sa2.att_layout = ophip_tensor_layout{OPHIP_DT_F16, 3, s3r, t3r}, sa2.att_base = x;
+            TRY(ophip_fused_softmax_launch(sm, &sa2, nullptr, 0, &qa));
+            ophip_fused_softmax_destroy(sm);
+        }
+        const size_t attn_shapes[][5] = {{4, 2, 128, 128, 64}, {2, 2, 200, 330, 128}, {8, 2, 16, 700, 128}, {4, 4, 1, 2000, 64}};  // nh, nkvh, seq, att, dh
+        for (const auto &as : attn_shapes) {
+            const size_t h = as[0], kvh = as[1], sq = as[2], at = as[3], hd = as[4];
+            const size_t sq3[3] = {h, sq, hd}, sk3[3] = {kvh, at, hd};
+            const ptrdiff_t tq3[3] = {(ptrdiff_t)(sq * hd * 2), (ptrdiff_t)(hd * 2), 2}, tk3[3] = {(ptrdiff_t)(at * hd * 2), (ptrdiff_t)(hd * 2), 2};
+            ophip_attention *op = nullptr;
+            TRY(ophip_attention_create(dev, &op));
+            ophip_attention_args a{};
+            a.q_layout = a.o_layout = ophip_tensor_layout{OPHIP_DT_F16, 3, sq3, tq3}, a.k_layout = a.v_layout = ophip_tensor_layout{OPHIP_DT_F16, 3, sk3, tk3}, a.mask = 1;
+            a.q_base = zeros(h * sq * hd * 2), a.o_base = zeros(h * sq * hd * 2), a.k_base = zeros(kvh * at * hd * 2), a.v_base = zeros(kvh * at * hd * 2);
+            TRY(ophip_attention_launch(op, &a, nullptr, 0, &qa));
+            ophip_attention_destroy(op);
+        }
+        const size_t sample_shapes[][2] = {{50000, 300}, {128256, 5000}, {40000, (size_t)-1}};  // logits, top_k
+        for (const auto &ss : sample_shapes) {
+            ophip_random_sample *op = nullptr;
+            TRY(ophip_random_sample_create(dev, &op));
+            const size_t n = ss[0], sn[1] = {n};
+            const ptrdiff_t tl[1] = {2}, ti[1] = {4};
+            ophip_random_sample_args a{};
+            a.kv_pair = ophip_tensor_layout{OPHIP_DT_KVPAIR, 0, nullptr, nullptr}, a.kv_pair_base = zeros(8);
+            a.logits = ophip_tensor_layout{OPHIP_DT_F16, 1, sn, tl}, a.logits_base = zeros(n * 2);
+            a.indices = ophip_tensor_layout{OPHIP_DT_U32, 1, sn, ti};
+            if (ophip_sample_args_new(1.0f, 0.95f, ss[1], &a.config) != 0) return 1;
+            a.seed = 0.61f;
+            TRY(ophip_random_sample_launch(op, &a, nullptr, 0, &qa));
+            ophip_random_sample_destroy(op);
+        }
+        TRY(ophip_stream_synchronize(dev, stream));
+    }
+    {
+        // mat_mul over the shapes that take it to each kernel family (few rows on an N-contiguous and on a K-contiguous
+        // weight, 17 to 64 rows, tiles of 128 and 256, ragged tiles, a cut K, batches, odd strides), checked against a
+        // plain product
+        struct Shape {
+            size_t bt, m, n, k;
+            bool b_stored_n_by_k;
+            size_t pad;  // extra elements between rows of every operand (odd: the element-wise kernel)
+        };
+        const Shape shapes[] = {{1, 16, 256, 128, false, 0}, {1, 5, 1160, 4096, false, 0}, {1, 16, 256, 256, true, 0}, {1, 16, 128, 2048, true, 0},
+                                {1, 40, 256, 100, false, 0}, {2, 64, 136, 72, false, 0}, {1, 128, 128, 64, false, 0}, {1, 256, 256, 64, false, 0},
+                                {1, 256, 256, 64, true, 0},  {1, 200, 130, 72, false, 0}, {1, 130, 128, 1024, false, 0}, {3, 16, 128, 64, false, 0},
+                                {1, 33, 70, 50, false, 3},   {32, 16, 128, 256, false, 0}};
+        ophip_mat_mul *op = nullptr;
+        TRY(ophip_mat_mul_create(dev, &op));
+        uint32_t seed = 7;
+        auto uniform = [&] {
+            seed = seed * 1664525u + 1013904223u;
+            return (float)(seed >> 8) / 16777216.0f * 2.0f - 1.0f;
+        };
+        std::vector<Shape> todo(std::begin(shapes), std::end(shapes));
+        if (large) todo.push_back({1, 4096, 4096, 64, false, 0});  // enough tiles for the 256 x 256 one (minutes under a sanitizer)
+        for (const Shape &sh : todo) {
+            const size_t lda = sh.k + sh.pad, ldb = (sh.b_stored_n_by_k ? sh.k : sh.n) + sh.pad, ldc = sh.n + sh.pad;
+            const size_t brows = sh.b_stored_n_by_k ? sh.n : sh.k;
+            std::vector<f16> a(sh.bt * sh.m * lda), b(sh.bt * brows * ldb), c(sh.bt * sh.m * ldc, (f16)0);
+            for (auto &v : a) v = (f16)uniform();
+            for (auto &v : b) v = (f16)(0.25f * uniform());
+            void *ad = zeros(a.size() * 2), *bd = zeros(b.size() * 2), *cd = zeros(c.size() * 2);
+            TRY(ophip_memcpy_h2d(dev, ad, a.data(), a.size() * 2, stream));
+            TRY(ophip_memcpy_h2d(dev, bd, b.data(), b.size() * 2, stream));
+            const size_t sa[3] = {sh.bt, sh.m, sh.k}, sb[3] = {sh.bt, sh.k, sh.n}, sc2[3] = {sh.bt, sh.m, sh.n};
+            const ptrdiff_t ta[3] = {(ptrdiff_t)(sh.m * lda * 2), (ptrdiff_t)(lda * 2), 2}, tc2[3] = {(ptrdiff_t)(sh.m * ldc * 2), (ptrdiff_t)(ldc * 2), 2};
+            const ptrdiff_t tb_kn[3] = {(ptrdiff_t)(brows * ldb * 2), (ptrdiff_t)(ldb * 2), 2}, tb_nk[3] = {(ptrdiff_t)(brows * ldb * 2), 2, (ptrdiff_t)(ldb * 2)};
+            ophip_mat_mul_args ma{};
+            ma.c_layout = ophip_tensor_layout{OPHIP_DT_F16, 3, sc2, tc2};
+            ma.a_layout = ophip_tensor_layout{OPHIP_DT_F16, 3, sa, ta};
+            ma.b_layout = ophip_tensor_layout{OPHIP_DT_F16, 3, sb, sh.b_stored_n_by_k ? tb_nk : tb_kn};
+            ma.c_base = cd, ma.a_base = ad, ma.b_base = bd, ma.alpha = 1.0f, ma.beta = 0.0f;
+            char which[128];
+            TRY(ophip_mat_mul_describe(op, &ma, which, sizeof which));
+            TRY(ophip_mat_mul_scheme(op, &ma, (size_t)1 << 30, &ws));
+            TRY(ophip_mat_mul_launch(op, &ma, nullptr, 0, &qa));
+            TRY(ophip_memcpy_d2h(dev, c.data(), cd, c.size() * 2, stream));
+            TRY(ophip_stream_synchronize(dev, stream));
+            size_t off = 0;
+            for (size_t t = 0; t < sh.bt; ++t)
+                for (size_t i = 0; i < sh.m; ++i)
+                    for (size_t j = 0; j < sh.n; ++j) {
+                        float ref = 0.f, mag = 0.f;
+                        for (size_t l = 0; l < sh.k; ++l) {
+                            const float x = (float)a[(t * sh.m + i) * lda + l];
+                            const float y = sh.b_stored_n_by_k ? (float)b[(t * brows + j) * ldb + l] : (float)b[(t * brows + l) * ldb + j];
+                            ref += x * y, mag += std::fabs(x * y);
+                        }
+                        const float got = (float)c[(t * sh.m + i) * ldc + j];
+                        if (std::fabs(got - ref) > 2e-3f + 2e-3f * mag) off++;
+                    }
+            std::printf("mat_mul %zux(%zux%zux%zu)%s: %s, %zu elements off\n", sh.bt, sh.m, sh.n, sh.k, sh.b_stored_n_by_k ? " B stored [N, K]" : "", which, off);
+            if (off) return 1;
+        }
+        ophip_mat_mul_destroy(op);
+    }
     TRY(ophip_stream_synchronize(dev, stream));
     for (void *p : held) TRY(ophip_free(dev, p));
     TRY(ophip_stream_destroy(dev, stream));
@@ -341,7 +467,7 @@ int main(int argc, char **argv) {
             return 3;
         }
     }
-    if (every_operator_once(sh.dev) != 0) return 4;
+    if (every_operator_once(sh.dev, argc > 3) != 0) return 4;
     std::vector<std::thread> pool;
     for (int t = 0; t < threads; ++t) pool.emplace_back(worker, std::cref(sh), t, rounds);
     for (auto &t : pool) t.join();

@@ -145,7 +145,8 @@ def test_under_thread_address_and_undefined_behaviour_sanitizers(tmp_path):
     asan = build_sim.build(os.path.join(SIM, "_build_address"), sanitize="address")
     exe = str(tmp_path / "threads_driver_asan")
     build_threads_driver(asan, exe, ["-fsanitize=address", "-shared-libsan", "-Wl,-rpath," + runtime])
-    res = subprocess.run([exe, "3", "4"], capture_output=True, text=True, timeout=1200, env=dict(os.environ, ASAN_OPTIONS="detect_leaks=1"))
+    # ("large": the driver's sweep over mat_mul's kernel families then reaches the 256 x 256 tile as well)
+    res = subprocess.run([exe, "3", "4", "large"], capture_output=True, text=True, timeout=2400, env=dict(os.environ, ASAN_OPTIONS="detect_leaks=1"))
     assert res.returncode == 0 and res.stdout.strip().endswith("ok") and "AddressSanitizer" not in res.stderr, (res.returncode, res.stdout, res.stderr[-4000:])
     ubsan = build_sim.build(os.path.join(SIM, "_build_undefined"), sanitize="undefined")
     code = ("import sys; sys.path[:0] = [%r, %r]; import ophip; ophip.LIB_PATH = %r; import __graft_entry__; __graft_entry__.smoke()"
