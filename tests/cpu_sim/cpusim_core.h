@@ -98,6 +98,8 @@ struct Worker {
     const std::function<void()> *body = nullptr;
     // statistics of the launches so far
     uint64_t launches = 0, workgroups = 0, out_of_range_loads = 0, out_of_range_stores = 0;
+    // bytes moved by buffer accesses inside their resources, by cache policy: [0] plain, [1] non-temporal, [2] sc1
+    uint64_t buffer_load_bytes[3] = {0, 0, 0}, buffer_store_bytes[3] = {0, 0, 0};
     ~Worker() {
         for (Item *it : items) {
             munmap(it->stack - 4096, STACK_BYTES + 4096);

@@ -133,7 +133,8 @@ inline __amdgpu_buffer_rsrc_t cpusim_make_rsrc(const void *base, int stride, uin
     return {const_cast<char *>(static_cast<const char *>(base)), records};
 }
 #define __builtin_amdgcn_make_buffer_rsrc(base, stride, records, flags) cpusim_make_rsrc(base, stride, records, flags)
-inline cpusim_u32x4 cpusim_buffer_load_b128(__amdgpu_buffer_rsrc_t r, uint32_t voffset, uint32_t soffset, int) {
+inline int cpusim_cache_policy(int aux) { return (aux & 16) ? 2 : (aux & 2) ? 1 : 0; }  // sc1, nt, neither
+inline cpusim_u32x4 cpusim_buffer_load_b128(__amdgpu_buffer_rsrc_t r, uint32_t voffset, uint32_t soffset, int aux) {
     cpusim_u32x4 v = {0, 0, 0, 0};
     const uint64_t off = (uint64_t)voffset + soffset;
     if (off + 16 > r.records) {
@@ -141,15 +142,17 @@ inline cpusim_u32x4 cpusim_buffer_load_b128(__amdgpu_buffer_rsrc_t r, uint32_t v
         return v;
     }
     std::memcpy(&v, r.base + off, 16);
+    cpusim::worker().buffer_load_bytes[cpusim_cache_policy(aux)] += 16;
     return v;
 }
-inline void cpusim_buffer_store_b128(cpusim_u32x4 v, __amdgpu_buffer_rsrc_t r, uint32_t voffset, uint32_t soffset, int) {
+inline void cpusim_buffer_store_b128(cpusim_u32x4 v, __amdgpu_buffer_rsrc_t r, uint32_t voffset, uint32_t soffset, int aux) {
     const uint64_t off = (uint64_t)voffset + soffset;
     if (off + 16 > r.records) {
         cpusim::worker().out_of_range_stores++;
         return;
     }
     std::memcpy(r.base + off, &v, 16);
+    cpusim::worker().buffer_store_bytes[cpusim_cache_policy(aux)] += 16;
 }
 #define __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, aux) cpusim_buffer_load_b128(r, voff, soff, aux)
 #define __builtin_amdgcn_raw_buffer_store_b128(v, r, voff, soff, aux) cpusim_buffer_store_b128(v, r, voff, soff, aux)

@@ -418,10 +418,13 @@ hipError_t hipExtModuleLaunchKernel(hipFunction_t f, uint32_t wx, uint32_t wy, u
 }
 
 // ---- for the tests: counters of the stand-in itself
-//   [0] launches run, [1] workgroups run, [2] buffer loads past a resource's records, [3] buffer stores past them, [4] bytes of live device allocations
-void cpusim_counters(uint64_t out[5]) {
+//   [0] launches run, [1] workgroups run, [2] buffer loads past a resource's records, [3] buffer stores past them, [4] bytes of live device allocations,
+//   [5..7] bytes loaded through buffer resources with the plain, non-temporal and sc1 cache policy, [8..10] bytes stored likewise
+//   (of the calling thread's launches: a launch runs on the thread that makes it)
+void cpusim_counters(uint64_t out[11]) {
     cpusim::Worker &w = cpusim::worker();
     out[0] = w.launches, out[1] = w.workgroups, out[2] = w.out_of_range_loads, out[3] = w.out_of_range_stores, out[4] = g_live_bytes;
+    for (int i = 0; i < 3; ++i) out[5 + i] = w.buffer_load_bytes[i], out[8 + i] = w.buffer_store_bytes[i];
 }
 
 }  // extern "C"

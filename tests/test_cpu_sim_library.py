@@ -86,6 +86,52 @@ def test_smoke_against_the_host_build(sim_library):
     assert r.returncode == 0 and "smoke ok" in r.stdout, r.stdout + r.stderr
 
 
+WEIGHT_TRAFFIC = """
+import ctypes, sys
+sys.path[:0] = [%r, %r]
+import numpy as np
+import ophip
+ophip.LIB_PATH = %r
+from ophip import TensorLayout, dt
+gpu = ophip.Gpu(0)
+stream = gpu.stream()
+def counters():
+    out = (ctypes.c_uint64 * 11)()
+    ophip.lib().cpusim_counters(out)
+    return np.array(list(out), dtype=np.int64)
+for m, n, k in ((16, 4096, 4096), (16, 22016, 4096), (16, 4096, 11008), (7, 12288, 4096)):
+    ad, bd, cd = gpu.malloc(m * k * 2), gpu.malloc(k * n * 2), gpu.malloc(m * n * 2)
+    lay = lambda r, c: TensorLayout.new_contiguous(dt.F16, [1, r, c])
+    op = ophip.MatMul(gpu)
+    args = ophip.MatMulArgs(lay(m, n), cd, 0.0, lay(m, k), ad, lay(k, n), bd, 1.0)
+    kernel = op.describe(args)
+    before = counters()
+    op.launch(args, None, stream)
+    stream.synchronize()
+    d = counters() - before
+    print(m, n, k, kernel, "workgroups", d[1], "loads plain / nt / sc1", d[5:8], "stores", d[8:11], flush=True)
+    assert kernel.startswith("stream"), kernel
+    assert d[0] == 1 and d[2] == 0 and d[3] == 0                  # one launch, nothing past a resource
+    assert d[6] == k * n * 2, (d[6], k * n * 2)                   # the weight, through the non-temporal loads: once
+    strips = -(-n // 128)
+    assert d[5] == strips * 16 * k * 2, (d[5], strips)            # a (16 rows, the ones past m read as zeros) once per strip
+    assert d[7] == d[10] and d[8] == 0 and d[9] == 0              # what crosses workgroups is stored once and loaded once
+    assert d[10] <= 2 * 16 * n * 4 * 8                            # ... and is small beside the weight
+print("ok")
+"""
+
+
+def test_streaming_product_asks_for_every_weight_byte_once(sim_library):
+    """The stand-in counts the bytes that kernels move through buffer resources, by cache policy.  For the decode layer's
+    weight products on gemm_stream_m1 with the planner's cut (even and uneven): the weight goes through the non-temporal
+    loads, each byte exactly once per launch; the activations once per strip of 128 columns (from the caches); the
+    partial sums that cross workgroups are written once and read once.  No counter of the machine, but what the kernel
+    asks of it: a re-read of the weight would have to come from here."""
+    code = WEIGHT_TRAFFIC % (ROOT, os.path.join(ROOT, "operators-rs_amd"), sim_library)
+    r = subprocess.run([sys.executable, "-c", code], cwd=ROOT, capture_output=True, text=True, timeout=900)
+    assert r.returncode == 0 and r.stdout.strip().endswith("ok"), r.stdout + r.stderr[-3000:]
+
+
 def test_c_consumer_against_the_host_build(sim_library, tmp_path):
     """tests/c_abi/consumer.c (the ABI used from C11 as a binding of another language would use it: create, scheme,
     launch, compare with plain C) linked against the host build instead of libophip.so."""

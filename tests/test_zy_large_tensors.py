@@ -3,7 +3,7 @@
 An offset kept in 32 bits, or an element index in a signed int, works at every benchmark shape and wraps here.  Each
 tensor is a [n, d] f16 matrix of about 4.6 GiB whose rows all differ from the rows an address that wrapped by 2^31 or
 2^32 bytes or elements would hit instead (row r is row r mod 8191 of a random base block, with a sign and a scale that
-depend on r), filled on the device in 64 MiB pieces; the operator runs once over the whole tensor; rows are read back
+depend on r), uploaded a block of 8191 rows at a time; the operator runs once over the whole tensor; rows are read back
 around every such boundary, at both ends and at random places, and compared with the oracle on the same rows.
 """
 import numpy as np
@@ -31,10 +31,10 @@ class Big:
         rng = np.random.default_rng(seed)
         self.base = rng.standard_normal((PERIOD, d)).astype(f32).astype(f16)
         self.mem = gpu.malloc(n * d * 2)
-        if fill:
-            step = PERIOD * max(1, (64 << 20) // (PERIOD * d * 2))  # pieces of about 64 MiB
-            for r0 in range(0, n, step):
-                gpu.upload(self.mem, self.rows(np.arange(r0, min(n, r0 + step))), offset=r0 * d * 2)
+        if fill:  # the factor of a row repeats every 8 blocks of PERIOD rows: eight blocks made once, then copies
+            blocks = [self.rows(np.arange(v * PERIOD, (v + 1) * PERIOD)) for v in range(8)]
+            for b in range((n + PERIOD - 1) // PERIOD):
+                gpu.upload(self.mem, blocks[b % 8][:min(PERIOD, n - b * PERIOD)], offset=b * PERIOD * d * 2)
 
     def rows(self, idx):
         idx = np.asarray(idx, dtype=np.int64)
@@ -133,16 +133,17 @@ def rel_error(got, ref):
 
 def test_mat_mul_weight_past_4_gib(gpu, stream):
     """c[16, N] = a[16, K] . W[K, N] with a 4.5 GiB weight (the decode-shaped product of a very wide layer):
-    W[k, j] = T[(7 k + 13 j) mod L] for a random table T, so that any (k, j) the kernel might read instead differs."""
-    m, k, n, L = 16, 16384, 147456, 1000003
+    W[k, j] = T[(7919 k + j) mod L] for a random table T (a row is a run of the table, so filling is copying), and no
+    element 2^31, 2^32 or 2^33 bytes or elements further on holds the same place of the table."""
+    m, k, n, L, P = 16, 16384, 147456, 1000003, 7919
     say("mat_mul 16 x %d . %d x %d f16" % (k, k, n))
+    assert all((b // n * P + b % n) % L for b in (2 ** 30, 2 ** 31, 2 ** 32, 2 ** 33))
     rng = np.random.default_rng(10)
     table = (rng.standard_normal(L).astype(f32) * f32(0.05)).astype(f16)
     w = gpu.malloc(k * n * 2)
-    jj = np.arange(n, dtype=np.int64) * 13
+    twice = np.concatenate([table, table])
     for k0 in range(0, k, 256):
-        kk = np.arange(k0, min(k, k0 + 256), dtype=np.int64) * 7
-        gpu.upload(w, table[(kk[:, None] + jj[None, :]) % L], offset=k0 * n * 2)
+        gpu.upload(w, np.stack([twice[kk * P % L:kk * P % L + n] for kk in range(k0, min(k, k0 + 256))]), offset=k0 * n * 2)
     a = rng.standard_normal((m, k)).astype(f32).astype(f16)
     ad, cd = gpu.from_host(a), gpu.malloc(m * n * 2)
     lay = lambda r, c: TensorLayout.new_contiguous(dt.F16, [1, r, c])
@@ -154,7 +155,7 @@ def test_mat_mul_weight_past_4_gib(gpu, stream):
     cols = np.array(sorted({0, 1, n - 2, n - 1} | {int(x) for x in rng.integers(0, n, 96)}
                            | {(b // 2) % n + o for b in (2 ** 31, 2 ** 32, 2 ** 33) for o in (-1, 0, 1)}), dtype=np.int64)
     cols = cols[(cols >= 0) & (cols < n)]
-    wc = table[(np.arange(k, dtype=np.int64)[:, None] * 7 + cols[None, :] * 13) % L].astype(np.float64)
+    wc = table[(np.arange(k, dtype=np.int64)[:, None] * P + cols[None, :]) % L].astype(np.float64)
     assert rel_error(got[:, cols].astype(np.float64), a.astype(np.float64) @ wc) <= 1e-2
 
 
@@ -178,7 +179,7 @@ def test_mat_mul_rows_past_4_gib(gpu, stream):
 
 def test_attention_kv_cached_caches_past_4_gib(gpu, stream):
     """40 heads of 480000 cached tokens of 128 (4.6 GiB for either cache), ten new tokens appended at the end: the
-    appended rows are read back, and every head's result is compared with softmax(q k^T / sqrt(dh)) v in f64."""
+    appended rows are read back, and the results of the heads at the caches' ends and around 2 and 4 GiB are compared with softmax(q k^T / sqrt(dh)) v in f64."""
     nh = nkvh = 40
     seq, dh, buf = 10, 128, 480000
     pos = buf - seq
@@ -201,7 +202,7 @@ def test_attention_kv_cached_caches_past_4_gib(gpu, stream):
         assert np.array_equal(kc.fetch(stream, rows), k[h]) and np.array_equal(vc.fetch(stream, rows), v[h])
         before = np.arange(h * buf + pos - 2, h * buf + pos)
         assert np.array_equal(kc.fetch(stream, before), kc.rows(before)) and np.array_equal(vc.fetch(stream, before), vc.rows(before))
-    for h in range(nh):
+    for h in (0, 1, 17, 18, 34, 35, nh - 1):  # the 2 GiB and 4 GiB lines run through the caches of heads 17 and 34
         rows = np.arange(h * buf, h * buf + pos)
         keys = np.concatenate([kc.rows(rows), k[h]]).astype(np.float64)
         vals = np.concatenate([vc.rows(rows), v[h]]).astype(np.float64)
@@ -227,9 +228,12 @@ def test_batched_mat_mul_whose_batches_lie_past_4_gib(gpu, stream):
         return table[(h * 131 + j[:, None] * 7 + np.arange(dh, dtype=np.int64)[None, :] * 13) % L]
 
     kc = gpu.malloc(nh * buf * dh * 2)
+    piece = 120000  # keys per upload; a piece's places in the table are one piece's moved on by 131 h + 7 j0
+    twice = np.concatenate([table, table])
+    first = (np.arange(piece, dtype=np.int64)[:, None] * 7 + np.arange(dh, dtype=np.int64)[None, :] * 13) % L
     for h in range(nh):
-        for j0 in range(0, buf, 120000):
-            gpu.upload(kc, keys(h, np.arange(j0, min(buf, j0 + 120000))), offset=(h * buf + j0) * dh * 2)
+        for j0 in range(0, buf, piece):
+            gpu.upload(kc, twice[first + (h * 131 + j0 * 7) % L], offset=(h * buf + j0) * dh * 2)
     q = rng.standard_normal((nh, seq, dh)).astype(f32).astype(f16)
     qd, cd = gpu.from_host(q), gpu.malloc(nh * seq * buf * 2)
     op = ophip.MatMul(gpu)
