@@ -50,6 +50,7 @@ std::map<uintptr_t, size_t> &freed() {  // user address -> size, of blocks given
 #define g_blocks blocks()
 #define g_freed freed()
 size_t g_live_bytes = 0;
+uint64_t g_allocations = 0, g_frees = 0;  // calls that reached the allocator, over the life of the process
 
 void on_fault(int sig, siginfo_t *info, void *) {
     const uintptr_t a = reinterpret_cast<uintptr_t>(info->si_addr);
@@ -121,6 +122,7 @@ hipError_t sim_malloc(void **ptr, size_t size) {
     g_blocks[reinterpret_cast<uintptr_t>(user)] = Block{m, map_len, size};
     g_freed.erase(reinterpret_cast<uintptr_t>(user));
     g_live_bytes += body;
+    ++g_allocations;
     *ptr = user;
     return hipSuccess;
 }
@@ -135,6 +137,7 @@ hipError_t sim_free(void *ptr) {
         std::abort();
     }
     g_live_bytes -= it->second.map_len - 2 * 4096;
+    ++g_frees;
     // the pages stay reserved and inaccessible: a later access faults instead of landing in a newer allocation
     mmap(it->second.map, it->second.map_len, PROT_NONE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_FIXED | MAP_NORESERVE, -1, 0);
     g_freed[it->first] = it->second.size;
@@ -420,11 +423,13 @@ hipError_t hipExtModuleLaunchKernel(hipFunction_t f, uint32_t wx, uint32_t wy, u
 // ---- for the tests: counters of the stand-in itself
 //   [0] launches run, [1] workgroups run, [2] buffer loads past a resource's records, [3] buffer stores past them, [4] bytes of live device allocations,
 //   [5..7] bytes loaded through buffer resources with the plain, non-temporal and sc1 cache policy, [8..10] bytes stored likewise
-//   (of the calling thread's launches: a launch runs on the thread that makes it)
-void cpusim_counters(uint64_t out[11]) {
+//   (of the calling thread's launches: a launch runs on the thread that makes it), [11] device and pinned allocations made, [12] freed (by any thread)
+void cpusim_counters(uint64_t out[13]) {
     cpusim::Worker &w = cpusim::worker();
     out[0] = w.launches, out[1] = w.workgroups, out[2] = w.out_of_range_loads, out[3] = w.out_of_range_stores, out[4] = g_live_bytes;
     for (int i = 0; i < 3; ++i) out[5 + i] = w.buffer_load_bytes[i], out[8 + i] = w.buffer_store_bytes[i];
+    std::lock_guard<std::recursive_mutex> lock(g_mu);
+    out[11] = g_allocations, out[12] = g_frees;
 }
 
 }  // extern "C"

@@ -96,7 +96,7 @@ from ophip import TensorLayout, dt
 gpu = ophip.Gpu(0)
 stream = gpu.stream()
 def counters():
-    out = (ctypes.c_uint64 * 11)()
+    out = (ctypes.c_uint64 * 13)()
     ophip.lib().cpusim_counters(out)
     return np.array(list(out), dtype=np.int64)
 for m, n, k in ((16, 4096, 4096), (16, 22016, 4096), (16, 4096, 11008), (7, 12288, 4096)):
@@ -128,6 +128,66 @@ def test_streaming_product_asks_for_every_weight_byte_once(sim_library):
     partial sums that cross workgroups are written once and read once.  No counter of the machine, but what the kernel
     asks of it: a re-read of the weight would have to come from here."""
     code = WEIGHT_TRAFFIC % (ROOT, os.path.join(ROOT, "operators-rs_amd"), sim_library)
+    r = subprocess.run([sys.executable, "-c", code], cwd=ROOT, capture_output=True, text=True, timeout=900)
+    assert r.returncode == 0 and r.stdout.strip().endswith("ok"), r.stdout + r.stderr[-3000:]
+
+
+NO_ALLOCATION = """
+import ctypes, sys
+sys.path[:0] = [%r, %r, %r]
+import numpy as np
+import ophip
+ophip.LIB_PATH = %r
+from ophip import TensorLayout
+from helpers import normal_f16
+gpu = ophip.Gpu(0)
+stream = gpu.stream()
+def counters():
+    out = (ctypes.c_uint64 * 13)()
+    ophip.lib().cpusim_counters(out)
+    return np.array(list(out), dtype=np.int64)
+before = counters()
+probe = gpu.malloc(64)
+assert counters()[11] == before[11] + 1  # (the counters are alive)
+probe.free()
+assert counters()[12] == before[12] + 1
+op = ophip.MatMul(gpu)
+rng = np.random.default_rng(0)
+kinds = set()
+# split K in the streaming kernel (counters and partial sums), in a skinny kernel ([N, K] operand), in the tile kernel
+# (partial tiles and a reduce kernel), batched with counters per batch; two products that use no scratch
+for m, n, k, batch, b_nk in ((16, 4096, 4096, None, False), (16, 1024, 4096, None, True), (256, 512, 4096, None, True),
+                             (16, 128, 2048, 8, False), (40, 2048, 512, None, False), (7, 24, 40, None, False)):
+    lead = () if batch is None else (batch,)
+    a, c = normal_f16(rng, lead + (m, k)), normal_f16(rng, lead + (m, n))
+    b = normal_f16(rng, lead + ((n, k) if b_nk else (k, n)), std=0.05)
+    b_view = np.swapaxes(b, -1, -2) if b_nk else b
+    ad, bd, c1, c2 = gpu.from_host(a), gpu.from_host(b), gpu.from_host(c), gpu.from_host(c)
+    args = lambda cd: ophip.MatMulArgs(TensorLayout.of(c), cd, 0.5, TensorLayout.of(a), ad, TensorLayout.of(b_view), bd, 0.25)
+    static_args, kind = args(c2), op.describe(args(c2))
+    op.launch(args(c1), None, stream)
+    stream.synchronize()
+    before = counters()
+    op.launch_static(static_args, stream)
+    op.launch_static(static_args, stream)
+    stream.synchronize()
+    d = counters() - before
+    print(m, n, k, batch, kind, "launches", d[0], "allocations", d[11], "frees", d[12], flush=True)
+    assert d[0] >= 2 and d[11] == 0 and d[12] == 0 and d[4] == 0, d
+    kinds.add(kind.split()[0] + (" split" if "split_k=1" not in kind else ""))
+    op.launch_static(args(c1), stream)  # (c1 holds one product already: beta = 0.5 makes this the second for both)
+    one, two = (gpu.to_host(x, np.float16, c.size, stream=stream).view(np.uint16) for x in (c1, c2))
+    assert np.array_equal(one, two), kind
+assert {"stream split", "skinny split", "tile128x64 split", "skinny", "tile128x64"} <= kinds, kinds
+print("ok")
+"""
+
+
+def test_static_entry_point_reaches_no_allocator(sim_library):
+    """ophip_mat_mul_launch_static on the stand-in, whose allocator counts its calls: between the first and the last of
+    its launches, for products that split K in each kernel family and for products that do not, no allocation is made
+    and none is freed (the ordinary entry point, on a fresh operator and stream, makes several)."""
+    code = NO_ALLOCATION % (ROOT, os.path.join(ROOT, "operators-rs_amd"), os.path.join(ROOT, "tests"), sim_library)
     r = subprocess.run([sys.executable, "-c", code], cwd=ROOT, capture_output=True, text=True, timeout=900)
     assert r.returncode == 0 and r.stdout.strip().endswith("ok"), r.stdout + r.stderr[-3000:]
 
