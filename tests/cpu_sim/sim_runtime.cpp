@@ -258,7 +258,10 @@ hipError_t hipGetSymbolAddress(void **ptr, const void *symbol) {
         return hipSuccess;
     }
     if (!it->second.storage) {
+        // (module memory, not an allocation of the program: it stays out of the allocator's books)
+        const size_t live = g_live_bytes;
         if (sim_malloc(&it->second.storage, it->second.size) != hipSuccess) return hipErrorOutOfMemory;
+        g_live_bytes = live, --g_allocations;
         std::memset(it->second.storage, 0, it->second.size);  // a device array without an initializer is zero when its module is loaded
     }
     *ptr = it->second.storage;

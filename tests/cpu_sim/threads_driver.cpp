@@ -22,6 +22,8 @@
 
 #include "ophip.h"
 
+extern "C" void cpusim_counters(uint64_t out[13]);  // of the stand-in (sim_runtime.cpp)
+
 namespace {
 
 typedef _Float16 f16;
@@ -474,7 +476,15 @@ int main(int argc, char **argv) {
     ophip_mat_mul_destroy(sh.mm);
     ophip_rms_norm_destroy(sh.rms);
     ophip_device_release(sh.dev);
-    std::printf("%d threads x %d rounds: %d failures\n", threads, rounds, g_failures.load());
+    // with the device gone the library holds no device memory any more (the stand-in's allocator keeps the books)
+    uint64_t counters[13];
+    cpusim_counters(counters);
+    if (counters[4] != 0 || counters[11] != counters[12]) {
+        std::fprintf(stderr, "%llu bytes of device memory still allocated after the device was released (%llu allocations, %llu freed)\n",
+                     (unsigned long long)counters[4], (unsigned long long)counters[11], (unsigned long long)counters[12]);
+        g_failures++;
+    }
+    std::printf("%d threads x %d rounds: %d failures (%llu device allocations, all returned)\n", threads, rounds, g_failures.load(), (unsigned long long)counters[11]);
     if (!g_failures) std::printf("ok\n");
     return g_failures ? 1 : 0;
 }
